@@ -1,0 +1,254 @@
+"""ctypes driver for the CPU checkers (TEST INFRASTRUCTURE ONLY).
+
+`CpuPath("oracle")` drives oracle/libscn_oracle.so, this repository's own CPU
+restatement of the reference algorithm; `CpuPath("ref")` drives
+oracle/_ref/libscn_ref.so, the reference's CPU sources compiled behind
+oracle/ref_harness.cpp (present only where oracle/Makefile could build it).
+Both expose the same entry points, so one class serves both.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import
+this module; the shipped package never does.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_PATHS = {"oracle": os.path.join(_HERE, "libscn_oracle.so"),
+          "ref": os.path.join(_HERE, "_ref", "libscn_ref.so")}
+_PREFIX = {"oracle": "orc_", "ref": "ref_"}
+_libs = {}
+
+_i64p = C.POINTER(C.c_int64)
+_i32p = C.POINTER(C.c_int32)
+_f32p = C.POINTER(C.c_float)
+
+
+def available(flavour):
+    return os.path.exists(_PATHS[flavour])
+
+
+def _load(flavour):
+    if flavour in _libs:
+        return _libs[flavour]
+    if flavour == "ref":
+        import torch  # noqa: F401  (libscn_ref.so links libtorch_cpu)
+    lib = C.CDLL(_PATHS[flavour])
+    p = _PREFIX[flavour]
+    sig = {
+        "md_create": (C.c_void_p, [C.c_int]),
+        "md_destroy": (None, [C.c_void_p]),
+        "input_layer": (C.c_int, [C.c_void_p, _i64p, _i64p, C.c_int, C.c_int, C.c_int, C.c_int]),
+        "input_rules_header": (None, [C.c_void_p, _i32p]),
+        "input_rules": (None, [C.c_void_p, _i32p]),
+        "nactive": (C.c_int, [C.c_void_p, _i64p]),
+        "batch_size": (C.c_int, [C.c_void_p, _i64p]),
+        "spatial_locations": (None, [C.c_void_p, _i64p, _i64p]),
+        "rb_noffsets": (C.c_int, [C.c_void_p, C.c_int, _i64p, _i64p, _i64p, _i64p]),
+        "rb_counts": (None, [C.c_void_p, C.c_int, _i64p, _i64p, _i64p, _i64p, _i64p]),
+        "rb_copy": (None, [C.c_void_p, C.c_int, _i64p, _i64p, _i64p, _i64p, C.c_int, _i32p]),
+        "subm_conv": (C.c_double, [C.c_void_p, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p,
+                                   C.c_int, C.c_int, C.c_int]),
+        "conv": (C.c_double, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p,
+                              C.c_int, C.c_int, C.c_int]),
+        "deconv": (C.c_double, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, _f32p, _f32p,
+                                _f32p, C.c_int, C.c_int, C.c_int]),
+        "maxpool": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p,
+                           C.c_int, C.c_int]),
+        "bn_eval": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p, _f32p,
+                           _f32p, C.c_float, C.c_float]),
+        "input_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "output_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "s2d": (None, [C.c_void_p, _i64p, _f32p, _f32p, C.c_int]),
+    }
+    fns = {}
+    for name, (res, args) in sig.items():
+        f = getattr(lib, p + name)
+        f.restype = res
+        f.argtypes = args
+        fns[name] = f
+    _libs[flavour] = fns
+    return fns
+
+
+def _sz(dim, x):
+    a = np.ascontiguousarray(np.broadcast_to(np.asarray(x, dtype=np.int64), (dim,)))
+    return a
+
+
+def _p64(a):
+    return a.ctypes.data_as(_i64p) if a is not None else None
+
+
+def _pf(a):
+    return a.ctypes.data_as(_f32p) if a is not None else None
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
+
+
+class CpuPath:
+    """One Metadata object of the CPU path plus the forward ops that use it."""
+
+    def __init__(self, dim, flavour="oracle"):
+        self.f = _load(flavour)
+        self.dim = dim
+        self.h = self.f["md_create"](dim)
+        if not self.h:
+            raise ValueError("unsupported dimension %d" % dim)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.f["md_destroy"](self.h)
+            self.h = None
+
+    # -- metadata ---------------------------------------------------------
+    def input_layer(self, spatial, coords, batch_size=0, mode=3):
+        coords = np.ascontiguousarray(coords, dtype=np.int64)
+        s = _sz(self.dim, spatial)
+        self.input_spatial = s
+        return self.f["input_layer"](self.h, _p64(s), _p64(coords), coords.shape[0],
+                                     coords.shape[1], batch_size, mode)
+
+    def input_rules(self):
+        hdr = np.zeros(4, np.int32)
+        self.f["input_rules_header"](self.h, hdr.ctypes.data_as(_i32p))
+        mode, max_active, n_in, n_out = [int(v) for v in hdr]
+        rows = np.zeros((n_out, 1 + max_active), np.int32)
+        if mode != 0 and n_out:
+            self.f["input_rules"](self.h, rows.ctypes.data_as(_i32p))
+        return hdr, rows
+
+    def nactive(self, spatial):
+        return self.f["nactive"](self.h, _p64(_sz(self.dim, spatial)))
+
+    def batch_size(self, spatial):
+        return self.f["batch_size"](self.h, _p64(_sz(self.dim, spatial)))
+
+    def spatial_locations(self, spatial):
+        n = self.nactive(spatial)
+        out = np.zeros((n, self.dim + 1), np.int64)
+        if n:
+            self.f["spatial_locations"](self.h, _p64(_sz(self.dim, spatial)), _p64(out))
+        return out
+
+    def _rules(self, kind, a, b=None, c=None, d=None):
+        args = [_p64(_sz(self.dim, v)) if v is not None else None for v in (a, b, c, d)]
+        keep = [_sz(self.dim, v) if v is not None else None for v in (a, b, c, d)]
+        args = [_p64(v) for v in keep]
+        k = self.f["rb_noffsets"](self.h, kind, *args)
+        counts = np.zeros(k, np.int64)
+        self.f["rb_counts"](self.h, kind, *args, _p64(counts))
+        out = []
+        for i in range(k):
+            pairs = np.zeros((int(counts[i]), 2), np.int32)
+            if counts[i]:
+                self.f["rb_copy"](self.h, kind, *args, i, pairs.ctypes.data_as(_i32p))
+            out.append(pairs)
+        return out
+
+    def submanifold_rules(self, spatial, filter_size):
+        """List over filter offsets of int32 [n_k, 2] arrays of (in row, out row)."""
+        return self._rules(0, spatial, filter_size)
+
+    def strided_rules(self, in_size, out_size, filter_size, stride):
+        """As above for a strided convolution; creates the out_size level."""
+        return self._rules(1, in_size, out_size, filter_size, stride)
+
+    def s2d_rules(self, spatial):
+        """List over samples of int32 [n_b, 2] arrays of (row, dense offset)."""
+        return self._rules(2, spatial)
+
+    # -- forward ops ------------------------------------------------------
+    def _conv(self, name, sizes, n_out_rows, x, w, bias, groups):
+        x = _f32(x)
+        w = _f32(w)
+        bias = _f32(bias)
+        n_in, n_out = w.shape[2] * w.shape[1], w.shape[3] * w.shape[1]
+        out = np.zeros((n_out_rows, n_out), np.float32)
+        macs = self.f[name](self.h, *[_p64(s) for s in sizes], _pf(x), _pf(out), _pf(w), _pf(bias),
+                            n_in, n_out, groups)
+        return out, macs
+
+    def subm_conv(self, spatial, filter_size, x, w, bias=None):
+        """w: [K, groups, nIn/groups, nOut/groups]."""
+        s, f = _sz(self.dim, spatial), _sz(self.dim, filter_size)
+        self.submanifold_rules(spatial, filter_size)
+        return self._conv("subm_conv", (s, f), self.nactive(spatial), x, w, bias, w.shape[1])
+
+    def conv(self, in_size, out_size, filter_size, stride, x, w, bias=None):
+        self.strided_rules(in_size, out_size, filter_size, stride)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, filter_size, stride)]
+        return self._conv("conv", sizes, self.nactive(out_size), x, w, bias, w.shape[1])
+
+    def deconv(self, in_size, out_size, filter_size, stride, x, w, bias=None):
+        self.strided_rules(out_size, in_size, filter_size, stride)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, filter_size, stride)]
+        return self._conv("deconv", sizes, self.nactive(out_size), x, w, bias, w.shape[1])
+
+    def maxpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
+        x = _f32(x)
+        self.strided_rules(in_size, out_size, size, stride)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, size, stride)]
+        planes = x.shape[1] - n_features_to_drop
+        out = np.zeros((self.nactive(out_size), planes), np.float32)
+        self.f["maxpool"](self.h, *[_p64(s) for s in sizes], _pf(x), x.shape[1], _pf(out), planes,
+                          n_features_to_drop)
+        return out
+
+    def bn_eval(self, x, mean, var, weight=None, bias=None, eps=1e-4, leakiness=1.0):
+        x = _f32(x)
+        out = np.zeros_like(x)
+        mean, var, weight, bias = _f32(mean), _f32(var), _f32(weight), _f32(bias)
+        self.f["bn_eval"](_pf(x), _pf(out), x.shape[0], x.shape[1], x.shape[1], x.shape[1],
+                          _pf(mean), _pf(var), _pf(weight), _pf(bias), eps, leakiness)
+        return out
+
+    def input_fwd(self, x):
+        x = _f32(x)
+        hdr, _ = self.input_rules()
+        out = np.zeros((int(hdr[3]), x.shape[1]), np.float32)
+        self.f["input_fwd"](self.h, _pf(x), _pf(out), x.shape[1])
+        return out
+
+    def output_fwd(self, x):
+        x = _f32(x)
+        hdr, _ = self.input_rules()
+        out = np.zeros((int(hdr[2]), x.shape[1]), np.float32)
+        self.f["output_fwd"](self.h, _pf(x), _pf(out), x.shape[1])
+        return out
+
+    def s2d(self, spatial, x):
+        x = _f32(x)
+        s = _sz(self.dim, spatial)
+        out = np.zeros((self.batch_size(spatial), x.shape[1]) + tuple(int(v) for v in s),
+                       np.float32)
+        self.f["s2d"](self.h, _p64(s), _pf(x), _pf(out), x.shape[1])
+        return out
+
+
+def canon_rules(rules, loc_in, loc_out):
+    """Canonical form of a rulebook: a sorted int64 array of rows
+    (offset, in-site coords+batch, out-site coords+batch), independent of how
+    either side numbers its rows."""
+    rows = []
+    for k, pairs in enumerate(rules):
+        if len(pairs) == 0:
+            continue
+        a = loc_in[pairs[:, 0]]
+        b = loc_out[pairs[:, 1]]
+        rows.append(np.concatenate([np.full((len(pairs), 1), k, np.int64), a, b], axis=1))
+    if not rows:
+        return np.zeros((0, 1 + loc_in.shape[1] + loc_out.shape[1]), np.int64)
+    allr = np.concatenate(rows, axis=0)
+    order = np.lexsort(allr.T[::-1])
+    return allr[order]
+
+
+def canon_rows(loc):
+    """Permutation that sorts sites by (batch, coords): use it to compare feature
+    matrices of two implementations that number rows differently."""
+    key = np.concatenate([loc[:, -1:], loc[:, :-1]], axis=1)
+    return np.lexsort(key.T[::-1])

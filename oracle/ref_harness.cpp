@@ -1,0 +1,219 @@
+// C-ABI harness around the reference's own CPU sources, compiled where they
+// lie (never copied): the two #includes below pull in
+// <reference>/sparseconvnet/SCN/Metadata/Metadata.cpp and the CPU/*.cpp files
+// through the -I path given by oracle/Makefile.
+//
+// TEST INFRASTRUCTURE ONLY.  The resulting oracle/_ref/libscn_ref.so is used to
+// validate oracle/scn_oracle.cpp, to write the golden fixtures under
+// tests/golden/, and as the "reference" flavour of the CPU baseline.  The
+// entry points mirror oracle/scn_oracle.cpp's (prefix ref_ instead of orc_) so
+// one Python wrapper drives both.
+
+#include <torch/torch.h>
+
+#define ENABLE_OPENMP YES
+#include <omp.h>
+
+#include "Metadata/Metadata.cpp"
+template class Metadata<1>;
+template class Metadata<2>;
+template class Metadata<3>;
+template class Metadata<4>;
+
+#include "CPU/BatchNormalization.cpp"
+#include "CPU/Convolution.cpp"
+#include "CPU/Deconvolution.cpp"
+#include "CPU/IOLayers.cpp"
+#include "CPU/MaxPooling.cpp"
+#include "CPU/SparseToDense.cpp"
+
+#include <cstring>
+
+namespace {
+
+struct Handle {
+  int dim;
+  void *m;
+};
+
+at::Tensor lt(const int64_t *p, int n) {
+  return torch::from_blob((void *)p, {n}, at::kLong).clone();
+}
+at::Tensor ft(const float *p, std::vector<int64_t> shape) {
+  if (!p) return torch::empty({0}, at::kFloat);
+  return torch::from_blob((void *)p, shape, at::kFloat);
+}
+void copy_out(const at::Tensor &t, float *out) {
+  auto c = t.contiguous();
+  std::memcpy(out, c.data_ptr<float>(), sizeof(float) * c.numel());
+}
+
+template <Int D>
+RuleBook &rb_get(Metadata<D> &m, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                 const int64_t *d) {
+  auto A = lt(a, D);
+  if (kind == 0) {
+    auto B = lt(b, D);
+    return m.getSubmanifoldRuleBook(A, B, true);
+  }
+  if (kind == 1) {
+    auto B = lt(b, D), C = lt(c, D), Dd = lt(d, D);
+    return m.getRuleBook(A, B, C, Dd, true);
+  }
+  return m.getSparseToDenseRuleBook(A, true);
+}
+
+}  // namespace
+
+#define DISPATCH(h, ...)                                     \
+  switch (((Handle *)h)->dim) {                              \
+  case 1: { constexpr Int D = 1; auto &m = *(Metadata<1> *)((Handle *)h)->m; __VA_ARGS__; } break; \
+  case 2: { constexpr Int D = 2; auto &m = *(Metadata<2> *)((Handle *)h)->m; __VA_ARGS__; } break; \
+  case 3: { constexpr Int D = 3; auto &m = *(Metadata<3> *)((Handle *)h)->m; __VA_ARGS__; } break; \
+  case 4: { constexpr Int D = 4; auto &m = *(Metadata<4> *)((Handle *)h)->m; __VA_ARGS__; } break; \
+  }
+
+extern "C" {
+
+void *ref_md_create(int dim) {
+  Handle *h = new Handle{dim, nullptr};
+  switch (dim) {
+  case 1: h->m = new Metadata<1>(); break;
+  case 2: h->m = new Metadata<2>(); break;
+  case 3: h->m = new Metadata<3>(); break;
+  case 4: h->m = new Metadata<4>(); break;
+  default: delete h; return nullptr;
+  }
+  return h;
+}
+void ref_md_destroy(void *h) {
+  DISPATCH(h, (void)D; delete &m);
+  delete (Handle *)h;
+}
+int ref_input_layer(void *h, const int64_t *spatial, const int64_t *coords, int n, int ncols,
+                    int batchSize, int mode) {
+  int r = 0;
+  DISPATCH(h, auto S = lt(spatial, D);
+           auto C = torch::from_blob((void *)coords, {n, ncols}, at::kLong).clone();
+           m.inputLayer(S, C, batchSize, mode); r = *m.inputNActive);
+  return r;
+}
+void ref_input_rules_header(void *h, int *hdr) {
+  DISPATCH(h, (void)D; for (int i = 0; i < 4; i++) hdr[i] = m.inputLayerRuleBook[0][i]);
+}
+void ref_input_rules(void *h, int *rows) {
+  DISPATCH(h, (void)D; if (m.inputLayerRuleBook.size() > 1) std::memcpy(
+                           rows, m.inputLayerRuleBook[1].data(),
+                           m.inputLayerRuleBook[1].size() * sizeof(Int)));
+}
+int ref_nactive(void *h, const int64_t *spatial) {
+  int r = 0;
+  DISPATCH(h, auto S = lt(spatial, D); r = m.getNActive(S));
+  return r;
+}
+int ref_batch_size(void *h, const int64_t *spatial) {
+  int r = 0;
+  DISPATCH(h, auto S = lt(spatial, D); r = m.getBatchSize(S));
+  return r;
+}
+void ref_spatial_locations(void *h, const int64_t *spatial, int64_t *out) {
+  DISPATCH(h, auto S = lt(spatial, D); auto t = m.getSpatialLocations(S);
+           std::memcpy(out, t.data_ptr<long>(), sizeof(int64_t) * t.numel()));
+}
+int ref_rb_noffsets(void *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                    const int64_t *d) {
+  int r = 0;
+  DISPATCH(h, r = (int)rb_get<D>(m, kind, a, b, c, d).size());
+  return r;
+}
+void ref_rb_counts(void *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                   const int64_t *d, int64_t *counts) {
+  DISPATCH(h, auto &rb = rb_get<D>(m, kind, a, b, c, d);
+           for (size_t k = 0; k < rb.size(); k++) counts[k] = (int64_t)rb[k].size() / 2);
+}
+void ref_rb_copy(void *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                 const int64_t *d, int k, int *pairs) {
+  DISPATCH(h, auto &rb = rb_get<D>(m, kind, a, b, c, d);
+           std::memcpy(pairs, rb[k].data(), rb[k].size() * sizeof(Int)));
+}
+
+double ref_subm_conv(void *h, const int64_t *spatial, const int64_t *filter, const float *in,
+                     float *out, const float *w, const float *bias, int nIn, int nOut, int groups) {
+  double macs = 0;
+  DISPATCH(h, auto S = lt(spatial, D); auto F = lt(filter, D); Int n = m.getNActive(S);
+           auto I = ft(in, {n, nIn}); auto O = torch::empty({0}, at::kFloat);
+           auto W = ft(w, {F.prod().item<int64_t>(), groups, nIn / groups, nOut / groups});
+           auto B = ft(bias, {nOut});
+           macs = cpu_SubmanifoldConvolution_updateOutput<float, D>(S, F, m, I, O, W, B);
+           copy_out(O, out));
+  return macs;
+}
+double ref_conv(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                const int64_t *stride, const float *in, float *out, const float *w,
+                const float *bias, int nIn, int nOut, int groups) {
+  double macs = 0;
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(filter, D);
+           auto St = lt(stride, D); Int n = m.getNActive(IS); auto I = ft(in, {n, nIn});
+           auto O = torch::empty({0}, at::kFloat);
+           auto W = ft(w, {F.prod().item<int64_t>(), groups, nIn / groups, nOut / groups});
+           auto B = ft(bias, {nOut});
+           macs = cpu_Convolution_updateOutput<float, D>(IS, OS, F, St, m, I, O, W, B);
+           copy_out(O, out));
+  return macs;
+}
+double ref_deconv(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                  const int64_t *stride, const float *in, float *out, const float *w,
+                  const float *bias, int nIn, int nOut, int groups) {
+  double macs = 0;
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(filter, D);
+           auto St = lt(stride, D); Int n = m.getNActive(IS); auto I = ft(in, {n, nIn});
+           auto O = torch::empty({0}, at::kFloat);
+           auto W = ft(w, {F.prod().item<int64_t>(), groups, nIn / groups, nOut / groups});
+           auto B = ft(bias, {nOut});
+           macs = cpu_Deconvolution_updateOutput<float, D>(IS, OS, F, St, m, I, O, W, B);
+           copy_out(O, out));
+  return macs;
+}
+void ref_maxpool(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                 const int64_t *stride, const float *in, int inStride, float *out, int nPlanes,
+                 int nFeaturesToDrop) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(size, D);
+           auto St = lt(stride, D); Int n = m.getNActive(IS);
+           auto I = ft(in, {n, inStride}); auto O = torch::empty({0}, at::kFloat);
+           (void)nPlanes;
+           cpu_MaxPooling_updateOutput<float, D>(IS, OS, F, St, m, I, O, nFeaturesToDrop);
+           copy_out(O, out));
+}
+void ref_bn_eval(const float *in, float *out, int nActive, int nPlanes, int inStride,
+                 int outStride, const float *runningMean, const float *runningVar,
+                 const float *weight, const float *bias, float eps, float leakiness) {
+  std::vector<float> sm(nPlanes), si(nPlanes);
+  BatchNormalization_ForwardPass<float>((float *)in, out, nPlanes, inStride, outStride, nActive,
+                                        sm.data(), si.data(), (float *)runningMean,
+                                        (float *)runningVar, (float *)weight, (float *)bias, eps,
+                                        0.99f, false, leakiness);
+}
+void ref_input_fwd(void *h, const float *in, float *out, int nPlanes) {
+  // The rule list was built by ref_input_layer; this is the body of
+  // cpu_InputLayer_updateOutput after m.inputLayer(...) (CPU/IOLayers.cpp:57-71).
+  DISPATCH(h, (void)D; auto &rules = m.inputLayerRuleBook; Int mode = rules[0][0];
+           Int maxActive = rules[0][1]; Int nRows = rules[0][3];
+           if (mode == 0) { std::memcpy(out, in, sizeof(float) * (size_t)rules[0][2] * nPlanes); }
+           else {
+             std::memset(out, 0, sizeof(float) * (size_t)nRows * nPlanes);
+             InputLayer_ForwardPass<float>((float *)in, out, nRows, maxActive, nPlanes,
+                                           &rules[1][0], mode == 4);
+           });
+}
+void ref_output_fwd(void *h, const float *in, float *out, int nPlanes) {
+  DISPATCH(h, auto I = ft(in, {(int64_t)m.inputLayerRuleBook[0][3], nPlanes});
+           auto O = torch::empty({0}, at::kFloat);
+           cpu_OutputLayer_updateOutput<float, D>(m, I, O); copy_out(O, out));
+}
+void ref_s2d(void *h, const int64_t *spatial, const float *in, float *out, int nPlanes) {
+  DISPATCH(h, auto S = lt(spatial, D); Int n = m.getNActive(S); auto I = ft(in, {n, nPlanes});
+           auto O = torch::empty({0}, at::kFloat);
+           cpu_SparseToDense_updateOutput<float, D>(S, m, I, O, nPlanes); copy_out(O, out));
+}
+
+}  // extern "C"

@@ -1,0 +1,669 @@
+// CPU oracle for the sparse-convolution forward path.
+//
+// TEST INFRASTRUCTURE ONLY.  This file restates, on the CPU, the algorithm of
+// the reference implementation (facebookresearch/SparseConvNet, directory
+// sparseconvnet/SCN) for the forward pass: coordinate hash grids, rulebook
+// generation, gather -> GEMM -> scatter-add convolutions, eval-mode batch
+// norm, max pooling and the input / output / sparse-to-dense layers.  It is
+// the checker the GPU library is compared with and the "port" flavour of the
+// CPU baseline; nothing in the shipped library links or calls it.
+//
+// Every function cites the reference file:line it follows.  Row numbering of
+// levels created by a strided convolution follows this file's own hash-bucket
+// iteration, as the reference's follows google::dense_hash_map's; comparisons
+// therefore go through coordinates (orc_spatial_locations), never raw rows.
+//
+// Pinned by tests/test_oracle_*.py: brute-force dictionaries on small inputs,
+// dense torch convolutions / pooling / batch-norm, closed-form invariants, and
+// (where oracle/_ref builds) the compiled reference itself.
+//
+// Build: g++ -O3 -fopenmp -shared -fPIC scn_oracle.cpp -o libscn_oracle.so
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <vector>
+
+typedef int32_t Int;  // Metadata/32bits.h:11
+static const int MAXD = 6;  // sparseconvnet_cpu.cpp:14-20 instantiates 1..6
+
+struct Pt {
+  Int x[MAXD];
+};
+
+// Open-addressing map Point -> Int.  Hash function as Metadata/32bits.h:57-66
+// (32-bit wrap-around multiply by 2166136261 then xor, seed 16777619).
+// Iteration is in bucket order, as with the reference's dense_hash_map
+// (Metadata/Metadata.h:24-28); the probe sequence and growth policy are this
+// file's own, so the order differs from the reference's, which is allowed.
+struct Grid {
+  Int ctr = 0;  // Metadata/Metadata.h:31
+  int dim = 0;
+  std::vector<Pt> keys;
+  std::vector<Int> vals;
+  std::vector<uint8_t> used;
+  size_t count = 0;
+  void init(int d) {
+    dim = d;
+    keys.assign(32, Pt());
+    vals.assign(32, 0);
+    used.assign(32, 0);
+    count = 0;
+  }
+  size_t hash(const Pt &p) const {
+    uint32_t h = 16777619u;
+    for (int i = 0; i < dim; i++) {
+      h *= 2166136261u;
+      h ^= (uint32_t)p.x[i];
+    }
+    return (size_t)(int64_t)(int32_t)h;
+  }
+  bool eq(const Pt &a, const Pt &b) const {
+    for (int i = 0; i < dim; i++)
+      if (a.x[i] != b.x[i]) return false;
+    return true;
+  }
+  void grow() {
+    std::vector<Pt> ok;
+    std::vector<Int> ov;
+    std::vector<uint8_t> ou;
+    ok.swap(keys);
+    ov.swap(vals);
+    ou.swap(used);
+    size_t nb = ou.size() * 2;
+    keys.assign(nb, Pt());
+    vals.assign(nb, 0);
+    used.assign(nb, 0);
+    count = 0;
+    for (size_t i = 0; i < ou.size(); i++)
+      if (ou[i]) *insert(ok[i], ov[i]).first = ov[i];
+  }
+  // Returns (pointer to value, inserted?) like dense_hash_map::insert.
+  std::pair<Int *, bool> insert(const Pt &p, Int v) {
+    if ((count + 1) * 2 > used.size()) grow();
+    size_t mask = used.size() - 1, b = hash(p) & mask;
+    while (used[b]) {
+      if (eq(keys[b], p)) return {&vals[b], false};
+      b = (b + 1) & mask;
+    }
+    used[b] = 1;
+    keys[b] = p;
+    vals[b] = v;
+    count++;
+    return {&vals[b], true};
+  }
+  const Int *find(const Pt &p) const {
+    size_t mask = used.size() - 1, b = hash(p) & mask;
+    while (used[b]) {
+      if (eq(keys[b], p)) return &vals[b];
+      b = (b + 1) & mask;
+    }
+    return nullptr;
+  }
+};
+
+typedef std::vector<Grid> Grids;                 // Metadata/Metadata.h:34
+typedef std::vector<std::vector<Int>> RuleBook;  // Metadata/Metadata.h:35
+typedef std::vector<int64_t> Key;
+
+// Metadata/Metadata.h:44-74: per-spatial-size active counts and grids, and
+// lazily built rulebooks cached by (size || filter [|| stride]).
+struct Metadata {
+  int dim;
+  std::map<Key, Int> nActive;
+  std::map<Key, Grids> grids;
+  RuleBook inputLayerRuleBook;
+  std::map<Key, RuleBook> submanifoldRuleBooks;
+  std::map<Key, RuleBook> ruleBooks;
+  std::map<Key, RuleBook> sparseToDenseRuleBooks;
+  Key inputSpatialSize;
+};
+
+static Key mkkey(int dim, const int64_t *a, const int64_t *b = nullptr,
+                 const int64_t *c = nullptr) {
+  Key k(a, a + dim);
+  if (b) k.insert(k.end(), b, b + dim);
+  if (c) k.insert(k.end(), c, c + dim);
+  return k;
+}
+
+static void resize_grids(Grids &g, size_t n, int dim) {
+  size_t old = g.size();
+  g.resize(n);
+  for (size_t i = old; i < n; i++) g[i].init(dim);
+}
+
+static Int volume(int dim, const int64_t *s) {  // Metadata/Metadata.cpp volume<>
+  Int v = 1;
+  for (int i = 0; i < dim; i++) v *= (Int)s[i];
+  return v;
+}
+
+// Metadata/IOLayersRules.h:18-121
+static void inputLayerRules(Grids &SGs, RuleBook &rules, const int64_t *coords,
+                            Int nInputRows, Int nInputColumns, Int batchSize,
+                            Int mode, Int &nActive, int dim) {
+  resize_grids(SGs, batchSize, dim);  // :25 minimum batch size
+  Pt p = Pt();
+  if (mode == 0) {  // :28-58
+    nActive = nInputRows;
+    rules.resize(1);
+    rules[0] = {mode, 1, nInputRows, nInputRows};
+    if (nInputColumns == dim) {
+      SGs.clear();
+      resize_grids(SGs, 1, dim);
+      for (Int i = 0; i < nInputRows; ++i) {
+        for (int j = 0; j < dim; j++) p.x[j] = (Int)coords[j];
+        coords += dim;
+        *SGs[0].insert(p, i).first = i;
+      }
+    } else {
+      for (Int i = 0; i < nInputRows; ++i) {
+        for (int j = 0; j < dim; j++) p.x[j] = (Int)coords[j];
+        Int idx = (Int)coords[dim];
+        coords += dim + 1;
+        if (idx + 1 >= (Int)SGs.size()) resize_grids(SGs, idx + 1, dim);
+        *SGs[idx].insert(p, i).first = i;
+      }
+    }
+    return;
+  }
+  std::vector<std::vector<Int>> outputRows;  // :61-89
+  if (nInputColumns == dim) {
+    SGs.clear();
+    resize_grids(SGs, 1, dim);
+  }
+  for (Int i = 0; i < nInputRows; ++i) {
+    for (int j = 0; j < dim; j++) p.x[j] = (Int)coords[j];
+    Int idx = 0;
+    if (nInputColumns == dim) {
+      coords += dim;
+    } else {
+      idx = (Int)coords[dim];
+      coords += dim + 1;
+      if (idx + 1 >= (Int)SGs.size()) resize_grids(SGs, idx + 1, dim);
+    }
+    auto r = SGs[idx].insert(p, nActive);
+    if (r.second) outputRows.resize(++nActive);
+    outputRows[*r.first].push_back(i);
+  }
+  rules.resize(2);  // :90-94
+  rules[0] = {mode, 1, nInputRows, (Int)outputRows.size()};
+  auto &rule = rules[1];
+  if (mode == 1)  // :96-101 first occurrence
+    for (Int i = 0; i < nActive; ++i) {
+      rule.push_back(1);
+      rule.push_back(outputRows[i].front());
+    }
+  if (mode == 2)  // :102-107 last occurrence
+    for (Int i = 0; i < nActive; ++i) {
+      rule.push_back(1);
+      rule.push_back(outputRows[i].back());
+    }
+  if (mode == 3 || mode == 4) {  // :108-119
+    Int maxActive = 0;
+    for (auto &row : outputRows) maxActive = std::max(maxActive, (Int)row.size());
+    rules[0][1] = maxActive;
+    for (auto &row : outputRows) {
+      rule.push_back((Int)row.size());
+      for (auto r : row) rule.push_back(r);
+      rule.resize((rule.size() + maxActive) / (maxActive + 1) * (maxActive + 1));
+    }
+  }
+}
+
+// Row-major offset of p inside the box [lb, ub], last dimension fastest:
+// Metadata/RectangularRegions.h:30-38.
+static Int region_offset(int dim, const Int *lb, const Int *ub, const Int *p) {
+  Int of = 0, m = 1;
+  for (int i = dim - 1; i >= 0; i--) {
+    of += m * (p[i] - lb[i]);
+    m *= ub[i] - lb[i] + 1;
+  }
+  return of;
+}
+
+// Visit every point of the box [lb, ub] with the last dimension fastest
+// (Metadata/RectangularRegions.h:43-71).  Empty when some lb[i] > ub[i].
+template <class F>
+static void for_region(int dim, const Int *lb, const Int *ub, F f) {
+  Pt p = Pt();
+  for (int i = 0; i < dim; i++) {
+    if (lb[i] > ub[i]) return;
+    p.x[i] = lb[i];
+  }
+  for (;;) {
+    f(p);
+    int i = dim - 1;
+    for (;;) {
+      if (++p.x[i] <= ub[i]) break;
+      p.x[i] = lb[i];
+      if (--i < 0) return;
+    }
+  }
+}
+
+// Metadata/SubmanifoldConvolutionRules.h:11-45
+static double subm_SgToRules(const Grid &grid, RuleBook &rules,
+                             const int64_t *size, int dim) {
+  double count = 0;
+  for (size_t b = 0; b < grid.used.size(); b++) {
+    if (!grid.used[b]) continue;
+    const Pt &out = grid.keys[b];
+    Int lb[MAXD], ub[MAXD];
+    for (int i = 0; i < dim; i++) {
+      Int pad = (Int)size[i] / 2;
+      lb[i] = out.x[i] - pad;
+      ub[i] = out.x[i] + (Int)size[i] - 1 - pad;
+    }
+    Int rulesOffset = 0;
+    for_region(dim, lb, ub, [&](const Pt &in) {
+      const Int *v = grid.find(in);
+      if (v) {
+        rules[rulesOffset].push_back(*v + grid.ctr);
+        rules[rulesOffset].push_back(grid.vals[b] + grid.ctr);
+        count++;
+      }
+      rulesOffset++;
+    });
+  }
+  return count;
+}
+
+// Metadata/SubmanifoldConvolutionRules.h:59-87: samples in parallel, then
+// per-offset concatenation in sample order.
+static void subm_SgsToRules(const Grids &SGs, RuleBook &rules,
+                            const int64_t *size, int dim) {
+  Int sd = volume(dim, size);
+  std::vector<RuleBook> rbs(SGs.size());
+  rules.clear();
+  rules.resize(sd);
+#pragma omp parallel for schedule(dynamic, 1)
+  for (Int i = 0; i < (Int)SGs.size(); i++) {
+    rbs[i].resize(sd);
+    subm_SgToRules(SGs[i], rbs[i], size, dim);
+  }
+#pragma omp parallel for
+  for (Int k = 0; k < sd; k++)
+    for (auto &rb : rbs) rules[k].insert(rules[k].end(), rb[k].begin(), rb[k].end());
+}
+
+// Metadata/ConvolutionRules.h:11-34 with the region calculators of
+// Metadata/RectangularRegions.h:95-119.
+static void conv_InputSgToRulesAndOutputSg(const Grid &inG, Grid &outG,
+                                           RuleBook &rules, const int64_t *size,
+                                           const int64_t *stride,
+                                           const int64_t *outSz, int dim) {
+  rules.resize(volume(dim, size));
+  for (size_t b = 0; b < inG.used.size(); b++) {
+    if (!inG.used[b]) continue;
+    const Pt &in = inG.keys[b];
+    Int lb[MAXD], ub[MAXD];
+    for (int i = 0; i < dim; i++) {  // OutputRegionCalculator :109-119
+      lb[i] = (Int)std::max<int64_t>(0, (in.x[i] - size[i] + stride[i]) / stride[i]);
+      ub[i] = (Int)std::min<int64_t>(outSz[i] - 1, in.x[i] / stride[i]);
+    }
+    for_region(dim, lb, ub, [&](const Pt &j) {
+      Int ilb[MAXD], iub[MAXD];
+      for (int i = 0; i < dim; i++) {  // InputRegionCalculator :95-105
+        ilb[i] = j.x[i] * (Int)stride[i];
+        iub[i] = ilb[i] + (Int)size[i] - 1;
+      }
+      Int rulesOffset = region_offset(dim, ilb, iub, in.x);
+      auto mv = outG.insert(j, 0);
+      if (mv.second) *mv.first = outG.ctr++;
+      rules[rulesOffset].push_back(inG.vals[b] + inG.ctr);
+      rules[rulesOffset].push_back(*mv.first);
+    });
+  }
+}
+
+// Metadata/ConvolutionRules.h:61-105
+static Int conv_InputSgsToRulesAndOutputSgs(const Grids &inSGs, Grids &outSGs,
+                                            RuleBook &rules, const int64_t *size,
+                                            const int64_t *stride,
+                                            const int64_t *outSz, int dim) {
+  rules.clear();
+  rules.resize(volume(dim, size));
+  outSGs.clear();
+  Int batchSize = (Int)inSGs.size();
+  resize_grids(outSGs, batchSize, dim);
+  std::vector<RuleBook> rbs(batchSize);
+#pragma omp parallel for schedule(dynamic, 1)
+  for (Int i = 0; i < batchSize; i++)
+    conv_InputSgToRulesAndOutputSg(inSGs[i], outSGs[i], rbs[i], size, stride, outSz, dim);
+  Int output_nActive = 0;
+  for (Int i = 0; i < batchSize; i++) {  // :80-88 ctr <- prefix sum
+    Int tmp = output_nActive;
+    output_nActive += outSGs[i].ctr;
+    outSGs[i].ctr = tmp;
+  }
+#pragma omp parallel for
+  for (Int k = 0; k < (Int)rules.size(); k++) {
+    auto &R = rules[k];
+    for (Int j = 0; j < batchSize; j++) {
+      auto &r = rbs[j][k];
+      Int offset = outSGs[j].ctr;
+      for (size_t q = 0; q < r.size(); q += 2) {
+        R.push_back(r[q]);
+        R.push_back(r[q + 1] + offset);
+      }
+    }
+  }
+  return output_nActive;
+}
+
+// Metadata/ConvolutionRules.h:130-151
+static void s2d_rules(const Grids &SGs, RuleBook &rules, const int64_t *spatial, int dim) {
+  rules.clear();
+  rules.resize(SGs.size());
+  Int lb[MAXD], ub[MAXD];
+  for (int i = 0; i < dim; i++) {
+    lb[i] = 0;
+    ub[i] = (Int)spatial[i] - 1;
+  }
+  for (size_t s = 0; s < SGs.size(); s++) {
+    const Grid &g = SGs[s];
+    for (size_t b = 0; b < g.used.size(); b++)
+      if (g.used[b]) {
+        rules[s].push_back(g.vals[b] + g.ctr);
+        rules[s].push_back(region_offset(dim, lb, ub, g.keys[b].x));
+      }
+  }
+}
+
+// Metadata/Metadata.cpp:437-451
+static RuleBook &getSubmanifoldRuleBook(Metadata &m, const int64_t *spatial, const int64_t *size) {
+  auto &rb = m.submanifoldRuleBooks[mkkey(m.dim, spatial, size)];
+  if (rb.empty()) subm_SgsToRules(m.grids[mkkey(m.dim, spatial)], rb, size, m.dim);
+  return rb;
+}
+// Metadata/Metadata.cpp:492-518
+static RuleBook &getRuleBook(Metadata &m, const int64_t *inSz, const int64_t *outSz,
+                             const int64_t *size, const int64_t *stride) {
+  auto &rb = m.ruleBooks[mkkey(m.dim, inSz, size, stride)];
+  if (rb.empty()) {
+    auto &iSGs = m.grids[mkkey(m.dim, inSz)];
+    auto &oSGs = m.grids[mkkey(m.dim, outSz)];
+    m.nActive[mkkey(m.dim, outSz)] =
+        conv_InputSgsToRulesAndOutputSgs(iSGs, oSGs, rb, size, stride, outSz, m.dim);
+  }
+  return rb;
+}
+// Metadata/Metadata.cpp:476-491
+static RuleBook &getSparseToDenseRuleBook(Metadata &m, const int64_t *spatial) {
+  Key k = mkkey(m.dim, spatial);
+  auto &SGs = m.grids[k];
+  auto &rb = m.sparseToDenseRuleBooks[k];
+  if (rb.empty()) s2d_rules(SGs, rb, spatial, m.dim);
+  return rb;
+}
+
+// C = A[nRules x ip] * W[ip x op], row-major.  Stands in for at::matmul
+// (CPU/Convolution.cpp:74,145), a BLAS sgemm that is not part of the
+// reference's sources; plain triple loop, fp32 accumulate in k order.
+static void sgemm(const float *A, const float *W, float *C, Int n, Int ip, Int op) {
+#pragma omp parallel for
+  for (Int i = 0; i < n; i++) {
+    float *c = C + (size_t)i * op;
+    for (Int o = 0; o < op; o++) c[o] = 0.f;
+    const float *a = A + (size_t)i * ip;
+    for (Int k = 0; k < ip; k++) {
+      float av = a[k];
+      const float *w = W + (size_t)k * op;
+      for (Int o = 0; o < op; o++) c[o] += av * w[o];
+    }
+  }
+}
+
+// The loop shared by CPU/Convolution.cpp:45-79 (strided), :117-150
+// (submanifold) and CPU/Deconvolution.cpp:7-41 (columns swapped):
+// rule_index_select (:8-24) -> matmul -> rule_index_add_ (:28-43).
+static double conv_loop(const RuleBook &rules, int inCol, int outCol, const float *in,
+                        float *out, Int nOutRows, const float *w, const float *bias,
+                        Int nIn, Int nOut, Int groups) {
+  Int ip = nIn / groups, op = nOut / groups;
+  for (Int r = 0; r < nOutRows; r++)  // Convolution.cpp:127-131
+    for (Int c = 0; c < nOut; c++) out[(size_t)r * nOut + c] = (bias && nOutRows) ? bias[c] : 0.f;
+  double flops = 0;
+  std::vector<float> A, C;
+  for (size_t k = 0; k < rules.size(); k++) {
+    const auto &r = rules[k];
+    Int nRules = (Int)(r.size() / 2);
+    if (!nRules) continue;
+    flops += (double)nRules * ip * op * groups;  // Convolution.cpp:141
+    A.resize((size_t)nRules * ip);
+    C.resize((size_t)nRules * op);
+    for (Int g = 0; g < groups; g++) {
+      // weight[k][g] is [ip x op] (submanifoldConvolution.py:24-26)
+      const float *wk = w + (((size_t)k * groups + g) * ip) * op;
+#pragma omp parallel for
+      for (Int i = 0; i < nRules; i++)
+        std::memcpy(&A[(size_t)i * ip], in + ((size_t)r[2 * i + inCol] * groups + g) * ip,
+                    sizeof(float) * ip);
+      sgemm(A.data(), wk, C.data(), nRules, ip, op);
+#pragma omp parallel for
+      for (Int i = 0; i < nRules; i++) {
+        float *t = out + ((size_t)r[2 * i + outCol] * groups + g) * op;
+        const float *s = &C[(size_t)i * op];
+        for (Int j = 0; j < op; j++) t[j] += s[j];
+      }
+    }
+  }
+  return flops;
+}
+
+extern "C" {
+
+void *orc_md_create(int dim) {
+  if (dim < 1 || dim > MAXD) return nullptr;
+  Metadata *m = new Metadata();
+  m->dim = dim;
+  return m;
+}
+void orc_md_destroy(void *md) { delete (Metadata *)md; }
+
+// Metadata/Metadata.cpp:413-425.  Returns the number of active sites.
+int orc_input_layer(void *md, const int64_t *spatial, const int64_t *coords, int n,
+                    int ncols, int batchSize, int mode) {
+  Metadata &m = *(Metadata *)md;
+  m.inputSpatialSize = mkkey(m.dim, spatial);
+  Int &nA = m.nActive[m.inputSpatialSize];
+  inputLayerRules(m.grids[m.inputSpatialSize], m.inputLayerRuleBook, coords, n, ncols,
+                  batchSize, mode, nA, m.dim);
+  return nA;
+}
+// header: [mode, maxActive, nInputRows, nOutputRows]; Metadata/IOLayersRules.h:10-15
+void orc_input_rules_header(void *md, int *hdr) {
+  Metadata &m = *(Metadata *)md;
+  for (int i = 0; i < 4; i++) hdr[i] = m.inputLayerRuleBook[0][i];
+}
+// rows: nOutputRows x (1 + maxActive); only for mode != 0.
+void orc_input_rules(void *md, int *rows) {
+  Metadata &m = *(Metadata *)md;
+  if (m.inputLayerRuleBook.size() > 1)
+    std::memcpy(rows, m.inputLayerRuleBook[1].data(), m.inputLayerRuleBook[1].size() * sizeof(Int));
+}
+int orc_nactive(void *md, const int64_t *spatial) {  // Metadata/Metadata.cpp:67-70
+  Metadata &m = *(Metadata *)md;
+  return m.nActive[mkkey(m.dim, spatial)];
+}
+int orc_batch_size(void *md, const int64_t *spatial) {  // Metadata/Metadata.cpp:171-176
+  Metadata &m = *(Metadata *)md;
+  return (int)m.grids[mkkey(m.dim, spatial)].size();
+}
+// Metadata/Metadata.cpp:149-170: out is [nActive, dim+1] int64, zero-filled first.
+void orc_spatial_locations(void *md, const int64_t *spatial, int64_t *out) {
+  Metadata &m = *(Metadata *)md;
+  Key k = mkkey(m.dim, spatial);
+  Int nA = m.nActive[k];
+  std::memset(out, 0, sizeof(int64_t) * (size_t)nA * (m.dim + 1));
+  Grids &SGs = m.grids[k];
+  for (size_t s = 0; s < SGs.size(); s++) {
+    Grid &g = SGs[s];
+    for (size_t b = 0; b < g.used.size(); b++)
+      if (g.used[b]) {
+        int64_t *o = out + (size_t)(g.vals[b] + g.ctr) * (m.dim + 1);
+        for (int d = 0; d < m.dim; d++) o[d] = g.keys[b].x[d];
+        o[m.dim] = (int64_t)s;
+      }
+  }
+}
+
+// Rulebook access: kind 0 = submanifold(spatial=a, filter=b),
+// 1 = strided(in=a, out=b, filter=c, stride=d), 2 = sparse-to-dense(spatial=a).
+// Builds (and caches) on first use, like the getters in Metadata.cpp.
+static RuleBook &rb_get(Metadata &m, int kind, const int64_t *a, const int64_t *b,
+                        const int64_t *c, const int64_t *d) {
+  if (kind == 0) return getSubmanifoldRuleBook(m, a, b);
+  if (kind == 1) return getRuleBook(m, a, b, c, d);
+  return getSparseToDenseRuleBook(m, a);
+}
+int orc_rb_noffsets(void *md, int kind, const int64_t *a, const int64_t *b,
+                    const int64_t *c, const int64_t *d) {
+  return (int)rb_get(*(Metadata *)md, kind, a, b, c, d).size();
+}
+// counts[k] = number of (first, second) pairs in list k.
+void orc_rb_counts(void *md, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                   const int64_t *d, int64_t *counts) {
+  RuleBook &rb = rb_get(*(Metadata *)md, kind, a, b, c, d);
+  for (size_t k = 0; k < rb.size(); k++) counts[k] = (int64_t)rb[k].size() / 2;
+}
+void orc_rb_copy(void *md, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                 const int64_t *d, int k, int *pairs) {
+  RuleBook &rb = rb_get(*(Metadata *)md, kind, a, b, c, d);
+  std::memcpy(pairs, rb[k].data(), rb[k].size() * sizeof(Int));
+}
+
+// CPU/Convolution.cpp:117-150.  out is [nActive(spatial), nOut]; returns MACs.
+double orc_subm_conv(void *md, const int64_t *spatial, const int64_t *filter, const float *in,
+                     float *out, const float *w, const float *bias, int nIn, int nOut, int groups) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getSubmanifoldRuleBook(m, spatial, filter);
+  return conv_loop(rb, 0, 1, in, out, m.nActive[mkkey(m.dim, spatial)], w, bias, nIn, nOut, groups);
+}
+// CPU/Convolution.cpp:45-79.  out is [nActive(outSz), nOut].
+double orc_conv(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                const int64_t *stride, const float *in, float *out, const float *w,
+                const float *bias, int nIn, int nOut, int groups) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, inSz, outSz, filter, stride);
+  return conv_loop(rb, 0, 1, in, out, m.nActive[mkkey(m.dim, outSz)], w, bias, nIn, nOut, groups);
+}
+// CPU/Deconvolution.cpp:7-41: rulebook of (outSz -> inSz), gather column 1,
+// scatter column 0.  out is [nActive(outSz), nOut].
+double orc_deconv(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                  const int64_t *stride, const float *in, float *out, const float *w,
+                  const float *bias, int nIn, int nOut, int groups) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, outSz, inSz, filter, stride);
+  return conv_loop(rb, 1, 0, in, out, m.nActive[mkkey(m.dim, outSz)], w, bias, nIn, nOut, groups);
+}
+// CPU/MaxPooling.cpp:7-20,37-60.  in is [nIn rows, inStride]; out is
+// [nActive(outSz), nPlanes] with nPlanes = C - nFeaturesToDrop, zero-filled first.
+void orc_maxpool(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                 const int64_t *stride, const float *in, int inStride, float *out, int nPlanes,
+                 int nFeaturesToDrop) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, inSz, outSz, size, stride);
+  Int nA = m.nActive[mkkey(m.dim, outSz)];
+  std::memset(out, 0, sizeof(float) * (size_t)nA * nPlanes);
+  const float *iF = in + nFeaturesToDrop;
+  for (auto &r : rb) {
+    Int nHot = (Int)(r.size() / 2);
+#pragma omp parallel for
+    for (Int s = 0; s < nHot; s++) {
+      const float *i = iF + (size_t)r[2 * s] * inStride;
+      float *o = out + (size_t)r[2 * s + 1] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++)
+        if (o[p] < i[p]) o[p] = i[p];
+    }
+  }
+}
+// CPU/BatchNormalization.cpp:41-61 (eval branch) and :109-130.
+void orc_bn_eval(const float *in, float *out, int nActive, int nPlanes, int inStride,
+                 int outStride, const float *runningMean, const float *runningVar,
+                 const float *weight, const float *bias, float eps, float leakiness) {
+  std::vector<float> w(nPlanes), b(nPlanes);
+  for (int p = 0; p < nPlanes; p++) {
+    float invStd = powf(runningVar[p] + eps, -0.5f);
+    w[p] = invStd * (weight ? weight[p] : 1.f);
+    b[p] = -runningMean[p] * w[p] + (bias ? bias[p] : 0.f);
+  }
+  for (int row = 0; row < nActive; row++) {
+    const float *i = in + (size_t)row * inStride;
+    float *o = out + (size_t)row * outStride;
+    for (int p = 0; p < nPlanes; p++) {
+      float v = i[p] * w[p] + b[p];
+      const float r = (v > 0) ? 1.f : leakiness;
+      o[p] = v * r;
+    }
+  }
+}
+// CPU/IOLayers.cpp:11-29,49-72.  out is [nActive, nPlanes].
+void orc_input_fwd(void *md, const float *in, float *out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.inputLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][3];
+  if (mode == 0) {
+    std::memcpy(out, in, sizeof(float) * (size_t)rules[0][2] * nPlanes);
+    return;
+  }
+  std::memset(out, 0, sizeof(float) * (size_t)nRows * nPlanes);
+  const Int *R = rules[1].data();
+#pragma omp parallel for
+  for (Int row = 0; row < nRows; row++) {
+    const Int *r = R + (size_t)row * (1 + maxActive);
+    Int nA = r[0];
+    float mult = (mode == 4 && nA > 0) ? 1.f / nA : 1.f;
+    float *o = out + (size_t)row * nPlanes;
+    for (Int i = 1; i <= nA; ++i) {
+      const float *f = in + (size_t)r[i] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += mult * f[p];
+    }
+  }
+}
+// CPU/IOLayers.cpp:95-115 (InputLayer_BackwardPass :31-47 with average=false).
+// out is [nInputRows, nPlanes].
+void orc_output_fwd(void *md, const float *in, float *out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.inputLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][3];
+  if (mode == 0) {
+    std::memcpy(out, in, sizeof(float) * (size_t)rules[0][2] * nPlanes);
+    return;
+  }
+  std::memset(out, 0, sizeof(float) * (size_t)rules[0][2] * nPlanes);
+  const Int *R = rules[1].data();
+  for (Int row = 0; row < nRows; row++) {
+    const Int *r = R + (size_t)row * (1 + maxActive);
+    const float *f = in + (size_t)row * nPlanes;
+    for (Int i = 1; i <= r[0]; ++i) {
+      float *o = out + (size_t)r[i] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += f[p];
+    }
+  }
+}
+// CPU/SparseToDense.cpp:7-19,35-64.  out is [batch, nPlanes, spatial...], zeroed here.
+void orc_s2d(void *md, const int64_t *spatial, const float *in, float *out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getSparseToDenseRuleBook(m, spatial);
+  int64_t vol = 1;
+  for (int i = 0; i < m.dim; i++) vol *= spatial[i];
+  std::memset(out, 0, sizeof(float) * rb.size() * nPlanes * vol);
+  float *oF = out;
+  for (auto &r : rb) {
+    Int nHot = (Int)(r.size() / 2);
+    for (Int s = 0; s < nHot; s++) {
+      const float *i = in + (size_t)r[2 * s] * nPlanes;
+      float *o = oF + r[2 * s + 1];
+      for (Int p = 0; p < nPlanes; p++) o[(size_t)p * vol] = i[p];
+    }
+    oF += (size_t)nPlanes * vol;
+  }
+}
+
+}  // extern "C"

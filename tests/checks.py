@@ -1,0 +1,212 @@
+"""Checks of one implementation of the path against independent statements
+(tests/bruteforce.py).  `make(dim)` returns an object with the interface of
+oracle.cpu_path.CpuPath; the same checks run on the oracle, on the compiled
+reference (where present) and, through an adapter over the C-ABI, on the HIP
+library.  Floating-point tolerance: 1e-4 relative, 1e-5 absolute (fp32)."""
+import numpy as np
+
+import bruteforce as bf
+from oracle.cpu_path import canon_rules
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def assert_close(a, b, what=""):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    assert a.shape == b.shape, (what, a.shape, b.shape)
+    if a.size == 0:
+        return
+    scale = max(1.0, float(np.abs(b).max()))
+    err = np.abs(a - b)
+    bad = err > ATOL * scale + RTOL * np.abs(b)
+    assert not bad.any(), "%s: %d/%d off, max err %g" % (what, bad.sum(), bad.size, err.max())
+
+
+def check_input_layer(make, dim, mode, seed, n=300, spatial=9, batch=3, with_batch_col=True):
+    rng = np.random.default_rng(seed)
+    coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=0 if mode == 0 else n // 2)
+    if mode == 0:
+        coords = np.unique(coords, axis=0)
+        coords = coords[rng.permutation(len(coords))]
+    if not with_batch_col:
+        coords = coords[coords[:, -1] == 0][:, :dim]
+    feats = rng.normal(size=(len(coords), 5)).astype(np.float32)
+    p = make(dim)
+    n_active = p.input_layer(spatial, coords, 0, mode)
+    full = coords if with_batch_col else np.concatenate(
+        [coords, np.zeros((len(coords), 1), np.int64)], 1)
+    row_of, n_expected = bf.first_occurrence_rows(full)
+    if mode == 0:
+        assert n_active == len(coords)
+        loc = p.spatial_locations(spatial)
+        assert (loc == full).all()
+        assert_close(p.input_fwd(feats), feats)
+        assert_close(p.output_fwd(feats), feats)
+        return
+    assert n_active == n_expected
+    # row numbering: first-occurrence order over the whole input
+    loc = p.spatial_locations(spatial)
+    assert (loc[row_of] == full).all()
+    expect, _ = bf.input_layer_values(full, feats, mode)
+    assert_close(p.input_fwd(feats), expect, "input layer mode %d" % mode)
+    # rule table: header and per-row lists in input order
+    hdr, rows = p.input_rules()
+    counts = np.bincount(row_of, minlength=n_expected)
+    assert hdr[0] == mode and hdr[2] == len(coords) and hdr[3] == n_expected
+    if mode in (3, 4):
+        assert hdr[1] == counts.max()
+        assert (rows[:, 0] == counts).all()
+        for r in range(n_expected):
+            assert list(rows[r, 1:1 + counts[r]]) == list(np.nonzero(row_of == r)[0])
+    else:
+        assert hdr[1] == 1 and (rows[:, 0] == 1).all()
+        pick = [np.nonzero(row_of == r)[0][0 if mode == 1 else -1] for r in range(n_expected)]
+        assert list(rows[:, 1]) == pick
+    # output layer: every input point receives its site's row
+    y = rng.normal(size=(n_expected, 4)).astype(np.float32)
+    out = p.output_fwd(y)
+    if mode in (3, 4):
+        assert_close(out, y[row_of], "output layer")
+    else:
+        picked = np.zeros(len(coords), bool)
+        picked[rows[:, 1]] = True
+        assert_close(out[picked], y[row_of][picked])
+        assert (out[~picked] == 0).all()
+
+
+def _setup(make, dim, spatial, n, batch, seed, C):
+    rng = np.random.default_rng(seed)
+    coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=n // 4)
+    feats = rng.normal(size=(len(coords), C)).astype(np.float32)
+    p = make(dim)
+    p.input_layer(spatial, coords, 0, 3)
+    loc = p.spatial_locations(spatial)
+    x = p.input_fwd(feats)
+    return rng, p, loc, x
+
+
+def check_submanifold(make, dim, size, seed, spatial=8, n=200, batch=2, cin=3, cout=4, bias=False):
+    rng, p, loc, x = _setup(make, dim, spatial, n, batch, seed, cin)
+    rules = p.submanifold_rules(spatial, size)
+    K = int(np.prod(np.broadcast_to(np.asarray(size), (dim,))))
+    assert len(rules) == K
+    got = bf.triples_of(canon_rules(rules, loc, loc))
+    assert got == bf.submanifold_triples(loc, dim, size)
+    assert sum(len(r) for r in rules) == len(got)  # no duplicate rules
+    for r in rules:  # at most one rule per (offset, output row)
+        assert len(np.unique(r[:, 1])) == len(r)
+    sz = np.broadcast_to(np.asarray(size), (dim,))
+    if (sz % 2 == 1).all():
+        centre = rules[K // 2]  # centre tap = identity on all rows
+        assert len(centre) == len(loc) and (centre[:, 0] == centre[:, 1]).all()
+        # symmetry (k, i, j) <-> (K-1-k, j, i)
+        for k in range(K):
+            a = set(map(tuple, rules[k].tolist()))
+            b = set((j, i) for i, j in rules[K - 1 - k].tolist())
+            assert a == b
+    w = (rng.normal(size=(K, 1, cin, cout)) * 0.3).astype(np.float32)
+    b = rng.normal(size=cout).astype(np.float32) if bias else None
+    y, macs = p.subm_conv(spatial, size, x, w, b)
+    assert macs == len(got) * cin * cout
+    assert_close(y, bf.dense_subm_conv(loc, x, w, spatial, size, batch, b), "submanifold conv")
+
+
+def check_strided(make, dim, size, stride, seed, out_spatial=4, n=150, batch=2, cin=3, cout=4,
+                  bias=False):
+    size_a = np.broadcast_to(np.asarray(size), (dim,))
+    stride_a = np.broadcast_to(np.asarray(stride), (dim,))
+    out_sp = np.broadcast_to(np.asarray(out_spatial), (dim,))
+    in_sp = (out_sp - 1) * stride_a + size_a
+    rng = np.random.default_rng(seed)
+    pts = np.stack([rng.integers(0, s, n) for s in in_sp], 1)
+    coords = np.concatenate([pts, rng.integers(0, batch, (n, 1))], 1).astype(np.int64)
+    feats = rng.normal(size=(n, cin)).astype(np.float32)
+    p = make(dim)
+    p.input_layer(in_sp, coords, 0, 4)
+    loc = p.spatial_locations(in_sp)
+    x = p.input_fwd(feats)
+    rules = p.strided_rules(in_sp, out_sp, size, stride)
+    K = int(size_a.prod())
+    assert len(rules) == K
+    loc_out = p.spatial_locations(out_sp)
+    assert p.nactive(out_sp) == len(loc_out)
+    expect = bf.strided_triples(loc, dim, size, stride, out_sp)
+    got = bf.triples_of(canon_rules(rules, loc, loc_out))
+    assert got == expect
+    assert sum(len(r) for r in rules) == len(expect)
+    # active outputs = exactly the sites with at least one rule, each listed once
+    want_out = set(t[1 + dim + 1:] for t in expect)
+    assert set(map(tuple, loc_out.tolist())) == want_out and len(loc_out) == len(want_out)
+    for r in rules:
+        assert len(np.unique(r[:, 1])) == len(r)
+    assert p.batch_size(out_sp) == p.batch_size(in_sp)
+    # rows of one sample are contiguous and samples ascend at a created level
+    assert (np.diff(loc_out[:, -1]) >= 0).all()
+
+    w = (rng.normal(size=(K, 1, cin, cout)) * 0.3).astype(np.float32)
+    b = rng.normal(size=cout).astype(np.float32) if bias else None
+    y, macs = p.conv(in_sp, out_sp, size, stride, x, w, b)
+    assert macs == len(expect) * cin * cout
+    dense = bf.dense_strided_conv(loc, x, w, in_sp, size, stride, batch, b)
+    assert_close(y, bf.sample_dense(dense, loc_out), "strided conv")
+    # max pooling over the same rulebook: zero-initialised, so max(0, active inputs)
+    mp = p.maxpool(in_sp, out_sp, size, stride, x)
+    dmp = bf.dense_maxpool(loc, x, in_sp, size, stride, batch)
+    assert_close(mp, bf.sample_dense(dmp, loc_out), "max pooling")
+    mp1 = p.maxpool(in_sp, out_sp, size, stride, x, 1)
+    assert_close(mp1, mp[:, 1:], "max pooling nFeaturesToDrop")
+    # deconvolution back to the fine level: transposed conv masked to the fine active set
+    w2 = (rng.normal(size=(K, 1, cout, cin)) * 0.3).astype(np.float32)
+    z, macs2 = p.deconv(out_sp, in_sp, size, stride, y, w2)
+    assert macs2 == len(expect) * cin * cout
+    dz = bf.dense_deconv(loc_out, y, w2, out_sp, size, stride, batch)
+    assert_close(z, bf.sample_dense(dz, loc), "deconvolution")
+    return p
+
+
+def check_bn(make, seed, n=257, C=13):
+    rng = np.random.default_rng(seed)
+    import torch
+    import torch.nn.functional as F
+    x = rng.normal(size=(n, C)).astype(np.float32)
+    mean = rng.normal(size=C).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    g = rng.normal(size=C).astype(np.float32)
+    b = rng.normal(size=C).astype(np.float32)
+    p = make(2)
+    for leak in (0.0, 0.333, 1.0):
+        for affine in (True, False):
+            y = p.bn_eval(x, mean, var, g if affine else None, b if affine else None, 1e-4, leak)
+            t = F.batch_norm(torch.as_tensor(x, dtype=torch.float64), torch.as_tensor(mean).double(),
+                             torch.as_tensor(var).double(),
+                             torch.as_tensor(g).double() if affine else None,
+                             torch.as_tensor(b).double() if affine else None, False, 0.0, 1e-4)
+            t = torch.where(t > 0, t, t * leak)
+            assert_close(y, t.numpy(), "bn leak=%g" % leak)
+
+
+def check_s2d(make, dim, seed, spatial=6, n=80, batch=3, C=4):
+    rng, p, loc, x = _setup(make, dim, spatial, n, batch, seed, C)
+    d = p.s2d(spatial, x)
+    assert d.shape == (batch, C) + (spatial,) * dim
+    assert_close(d, bf.to_dense(loc, x, spatial, batch).numpy(), "sparse to dense")
+    rules = p.s2d_rules(spatial)
+    assert len(rules) == batch
+    for b, r in enumerate(rules):
+        sel = loc[r[:, 0]]
+        assert (sel[:, -1] == b).all()
+        off = np.ravel_multi_index(tuple(sel[:, i] for i in range(dim)), (spatial,) * dim)
+        assert (off == r[:, 1]).all()
+    assert sum(len(r) for r in rules) == len(loc)
+
+
+def check_empty(make, dim=3):
+    """Zero active sites: every op returns an empty result and 0 multiply-adds."""
+    p = make(dim)
+    n = p.input_layer(8, np.zeros((0, dim + 1), np.int64), 0, 3)
+    assert n == 0
+    rules = p.submanifold_rules(8, 3)
+    assert sum(len(r) for r in rules) == 0
+    y, macs = p.subm_conv(8, 3, np.zeros((0, 3), np.float32), np.ones((27, 1, 3, 2), np.float32))
+    assert y.shape == (0, 2) and macs == 0

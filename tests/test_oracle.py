@@ -1,0 +1,59 @@
+"""Pins the CPU oracle (oracle/scn_oracle.cpp) against independent statements:
+brute-force dictionaries, dense torch routines and closed-form invariants.
+The same checks run on the compiled reference where oracle/_ref exists, which
+shows that the statements themselves describe the reference."""
+import numpy as np
+import pytest
+
+import checks
+from oracle import cpu_path
+
+
+def _flavours():
+    out = ["oracle"]
+    if cpu_path.available("ref"):
+        out.append("ref")
+    return out
+
+
+@pytest.fixture(params=_flavours())
+def make(request, oracle_built):
+    fl = request.param
+    return lambda dim: cpu_path.CpuPath(dim, fl)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dim", [2, 3])
+def test_input_layer(make, dim, mode):
+    checks.check_input_layer(make, dim, mode, seed=10 * dim + mode)
+
+
+def test_input_layer_no_batch_column(make):
+    checks.check_input_layer(make, 3, 4, seed=5, with_batch_col=False)
+    checks.check_input_layer(make, 2, 0, seed=6, with_batch_col=False)
+
+
+@pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (2, (3, 1)), (3, (1, 3, 5)), (3, 2),
+                                      (4, 3)])
+def test_submanifold(make, dim, size):
+    checks.check_submanifold(make, dim, size, seed=7 + dim, spatial=8 if dim < 4 else 5,
+                             n=200 if dim < 4 else 250, bias=(dim == 2))
+
+
+@pytest.mark.parametrize("dim,size,stride", [(3, 2, 2), (3, 3, 2), (2, 3, 2), (2, 2, 2), (1, 3, 2),
+                                             (2, (3, 2), (2, 1)), (3, 4, 2), (2, 2, 3), (3, 3, 1)])
+def test_strided(make, dim, size, stride):
+    checks.check_strided(make, dim, size, stride, seed=3 + dim, bias=(dim == 2))
+
+
+def test_bn(make):
+    checks.check_bn(make, seed=1)
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3])
+def test_s2d(make, dim):
+    checks.check_s2d(make, dim, seed=2 + dim)
+
+
+def test_empty(make):
+    checks.check_empty(make)
