@@ -1,0 +1,152 @@
+/* C ABI of libscn_hip.so: the MI355X (gfx950) forward path of submanifold
+ * sparse convolutional networks.
+ *
+ * The library replaces what the reference binds through its pybind11 module
+ * `sparseconvnet.SCN` for the forward pass (reference paths are relative to
+ * sparseconvnet/SCN/): the `Metadata_<D>` class (pybind.cpp:11-33,
+ * Metadata/Metadata.h:44-167) and the `*_updateOutput` functions declared in
+ * sparseconvnet.h:22-246.  Signatures carry plain pointers and sizes only.
+ *
+ * Conventions
+ *  - every function returns 0 on success, non-zero on failure; the message is
+ *    read with scn_last_error() (thread-local).  The reference has no error
+ *    codes: its shape checks are Python asserts and C++ asserts.
+ *  - `spatial`, `filter`, `stride` arguments are HOST arrays of `dim` int64
+ *    (the reference passes 1-D CPU LongTensors, Metadata/32bits.h:17-24).
+ *  - feature / weight / coordinate pointers are DEVICE pointers; features are
+ *    fp32 row-major [rows, planes]; weights [K, groups, nIn/groups,
+ *    nOut/groups] as in sparseconvnet/submanifoldConvolution.py:24-26.
+ *  - outputs are allocated by the caller (the reference resizes the tensor it
+ *    is handed, CPU/Convolution.cpp:127): ask scn_md_nactive() for the row count
+ *    after the rulebook call that creates the level.
+ *  - `stream` is a hipStream_t (as void*); work is enqueued on it.  Calls that
+ *    return a host value (row counts, rule counts) synchronise that stream.
+ *  - a metadata handle is not thread-safe (neither is the reference's lazily
+ *    caching Metadata, Metadata/Metadata.cpp:442-449).
+ */
+#ifndef SCN_HIP_H
+#define SCN_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct scn_metadata scn_metadata;
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char *scn_last_error(void);
+/* 32: rule indices are int32, as the reference's n_rulebook_bits (pybind.cpp:235). */
+int scn_rulebook_bits(void);
+
+/* ---- Metadata (pybind.cpp:11-33; Metadata/Metadata.h:44-167) ------------ */
+
+/* Metadata_<dim>() constructor, dim in 1..6 (pybind.cpp:204-209). NULL on failure. */
+scn_metadata *scn_md_create(int dim);
+void scn_md_destroy(scn_metadata *md);
+/* Metadata::clear (Metadata/Metadata.cpp:52-66). */
+int scn_md_clear(scn_metadata *md);
+
+/* Metadata::inputLayer (Metadata/Metadata.cpp:413-425, Metadata/IOLayersRules.h:18-121).
+ * coords: device int64 [n, ncols], ncols = dim (one sample) or dim+1 (last column = sample
+ * index).  mode 0: rows = input order, no merging; 1: first, 2: last, 3: sum, 4: mean of the
+ * points that share a site; rows are numbered by first occurrence in input order.
+ * min_batch is the reference's batchSize argument (a lower bound on the number of samples).
+ * Coordinates outside [0, spatial) are an error (the reference leaves them undefined).
+ * Writes the number of active sites to *n_active. */
+int scn_md_input_layer(scn_metadata *md, const int64_t *spatial, const int64_t *coords,
+                       int64_t n, int ncols, int min_batch, int mode, void *stream,
+                       int64_t *n_active);
+/* Rule header [mode, maxActive, nInputRows, nOutputRows] (Metadata/IOLayersRules.h:10-15). */
+int scn_md_input_rules_header(scn_metadata *md, int32_t hdr[4]);
+/* Rule rows, device int32 [nOutputRows, 1+maxActive] = [count, input indices.., 0 pad]. */
+int scn_md_input_rules(scn_metadata *md, int32_t *rows, void *stream);
+
+/* Metadata::getNActive (Metadata/Metadata.cpp:67-70); 0 for an unknown level. */
+int scn_md_nactive(scn_metadata *md, const int64_t *spatial, int64_t *n_active);
+/* Metadata::getBatchSize (Metadata/Metadata.cpp:171-176). */
+int scn_md_batch_size(scn_metadata *md, const int64_t *spatial, int *batch);
+/* Metadata::getSpatialLocations (Metadata/Metadata.cpp:149-170): device int64
+ * [nActive, dim+1], coordinates then sample index. */
+int scn_md_spatial_locations(scn_metadata *md, const int64_t *spatial, int64_t *out,
+                             void *stream);
+
+/* Metadata::getSubmanifoldRuleBook (Metadata/Metadata.cpp:437-451,
+ * Metadata/SubmanifoldConvolutionRules.h:11-87): builds and caches the rulebook of
+ * (spatial, filter).  Idempotent. */
+int scn_md_submanifold_rules(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
+                             void *stream);
+/* Metadata::getRuleBook (Metadata/Metadata.cpp:492-518, Metadata/ConvolutionRules.h:11-105):
+ * builds and caches the rulebook of (in_size, filter, stride) and, as the reference does,
+ * REPLACES the level out_size with the sites the rules reach.  Rows of that level are
+ * numbered by sample, then along a space-filling curve (the reference's order is its hash
+ * map's bucket order; both are arbitrary, compare through scn_md_spatial_locations). */
+int scn_md_strided_rules(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                         const int64_t *filter, const int64_t *stride, void *stream);
+
+/* Rule export, for inspection and parity tests (the reference binds no rulebook getter;
+ * its lists are the RuleBook vectors of Metadata/Metadata.h:35).
+ * kind 0: submanifold (a=spatial, b=filter); kind 1: strided (a=in_size, b=out_size,
+ * c=filter, d=stride); kind 2: sparse-to-dense (a=spatial; one list per sample of
+ * (row, dense offset), Metadata/ConvolutionRules.h:130-151).  Builds the rulebook if needed.
+ * scn_rules_count: number of lists.  scn_rules_sizes: host int64[count] pairs per list.
+ * scn_rules_export: device int32 [sizes[k], 2] (first, second) pairs of list k. */
+int scn_rules_count(scn_metadata *md, int kind, const int64_t *a, const int64_t *b,
+                    const int64_t *c, const int64_t *d, void *stream, int *count);
+int scn_rules_sizes(scn_metadata *md, int kind, const int64_t *a, const int64_t *b,
+                    const int64_t *c, const int64_t *d, void *stream, int64_t *sizes);
+int scn_rules_export(scn_metadata *md, int kind, const int64_t *a, const int64_t *b,
+                     const int64_t *c, const int64_t *d, int k, int32_t *pairs, void *stream);
+
+/* ---- forward ops (sparseconvnet.h:22-246) -------------------------------- */
+
+/* InputLayer_updateOutput after the rules exist (pybind.cpp:155-159, CPU/IOLayers.cpp:49-72):
+ * in [nInputRows, planes] -> out [nActive, planes]. */
+int scn_input_layer_fwd(scn_metadata *md, const float *in, float *out, int planes, void *stream);
+/* OutputLayer_updateOutput (pybind.cpp:164-167, CPU/IOLayers.cpp:95-115):
+ * in [nActive, planes] -> out [nInputRows, planes]. */
+int scn_output_layer_fwd(scn_metadata *md, const float *in, float *out, int planes,
+                         void *stream);
+
+/* SubmanifoldConvolution_updateOutput (pybind.cpp:135-139, CPU/Convolution.cpp:117-150).
+ * in [nActive, nIn] -> out [nActive, nOut]; bias may be NULL; *macs receives the
+ * multiply-add count the reference returns (CPU/Convolution.cpp:141). */
+int scn_subm_conv_fwd(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
+                      const float *in, float *out, const float *weight, const float *bias,
+                      int n_in, int n_out, int groups, void *stream, double *macs);
+/* Convolution_updateOutput (pybind.cpp:55-60, CPU/Convolution.cpp:45-79).
+ * in [nActive(in_size), nIn] -> out [nActive(out_size), nOut]. */
+int scn_conv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                 const int64_t *filter, const int64_t *stride, const float *in, float *out,
+                 const float *weight, const float *bias, int n_in, int n_out, int groups,
+                 void *stream, double *macs);
+/* Deconvolution_updateOutput (pybind.cpp:79-84, CPU/Deconvolution.cpp:7-41): uses the
+ * rulebook of (out_size -> in_size) with its columns swapped.
+ * in [nActive(in_size), nIn] -> out [nActive(out_size), nOut]. */
+int scn_deconv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                   const int64_t *filter, const int64_t *stride, const float *in, float *out,
+                   const float *weight, const float *bias, int n_in, int n_out, int groups,
+                   void *stream, double *macs);
+/* MaxPooling_updateOutput (pybind.cpp:103-107, CPU/MaxPooling.cpp:37-60).
+ * in [nActive(in_size), in_stride] -> out [nActive(out_size), planes] where
+ * planes = in_stride - n_features_to_drop; the result is max(0, inputs of the window). */
+int scn_maxpool_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                    const int64_t *size, const int64_t *stride, const float *in, int in_stride,
+                    float *out, int planes, int n_features_to_drop, void *stream);
+/* BatchNormalization_updateOutput with train=false (pybind.cpp:220,
+ * CPU/BatchNormalization.cpp:41-61,109-130): out = leaky(x*w + b), w = gamma/sqrt(var+eps),
+ * b = beta - mean*w.  gamma/beta may be NULL.  Row strides in elements. */
+int scn_bn_eval_fwd(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                    int64_t out_stride, const float *running_mean, const float *running_var,
+                    const float *gamma, const float *beta, float eps, float leakiness,
+                    void *stream);
+/* SparseToDense_updateOutput (pybind.cpp:125-129, CPU/SparseToDense.cpp:35-64):
+ * in [nActive, planes] -> out [batch, planes, spatial...], zero-filled first. */
+int scn_s2d_fwd(scn_metadata *md, const int64_t *spatial, const float *in, float *out,
+                int planes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SCN_HIP_H */

@@ -1,0 +1,235 @@
+// extern "C" surface of libscn_hip.so (declared in include/scn_hip.h).
+#include "../../include/scn_hip.h"
+
+#include "metadata.h"
+
+using namespace scn;
+
+struct scn_metadata {
+  Metadata m;
+};
+
+static thread_local std::string g_error;
+
+template <class F> static int guarded(F f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception &e) {
+    g_error = e.what();
+    return 1;
+  } catch (...) {
+    g_error = "unknown failure";
+    return 1;
+  }
+}
+
+static Metadata &md(scn_metadata *h) {
+  if (!h) throw Error("null metadata handle");
+  return h->m;
+}
+static hipStream_t st(void *s) { return (hipStream_t)s; }
+
+static Level *find_level(Metadata &m, const int64_t *spatial) {
+  auto it = m.levels.find(mk(m.dim, spatial));
+  return it == m.levels.end() ? nullptr : &it->second;
+}
+
+extern "C" {
+
+const char *scn_last_error(void) { return g_error.c_str(); }
+int scn_rulebook_bits(void) { return 32; }
+
+scn_metadata *scn_md_create(int dim) {
+  if (dim < 1 || dim > SCN_MAXD) {
+    g_error = "dimension must be 1..6";
+    return nullptr;
+  }
+  try {
+    scn_metadata *h = new scn_metadata();
+    h->m.dim = dim;
+    return h;
+  } catch (const std::exception &e) {
+    g_error = e.what();
+    return nullptr;
+  }
+}
+void scn_md_destroy(scn_metadata *h) { delete h; }
+int scn_md_clear(scn_metadata *h) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    int dim = m.dim;
+    m.levels.clear();
+    m.subm.clear();
+    m.strided.clear();
+    m.input = InputRules();
+    m.input_size.clear();
+    m.dim = dim;
+  });
+}
+
+int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *coords, int64_t n,
+                       int ncols, int min_batch, int mode, void *stream, int64_t *n_active) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (n < 0) throw Error("negative point count");
+    if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
+    build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, st(stream));
+    if (n_active) *n_active = m.input.n_out;
+  });
+}
+int scn_md_input_rules_header(scn_metadata *h, int32_t hdr[4]) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (m.input.mode < 0) throw Error("input layer rules have not been built");
+    hdr[0] = m.input.mode;
+    hdr[1] = m.input.max_active;
+    hdr[2] = (int32_t)m.input.n_in;
+    hdr[3] = (int32_t)m.input.n_out;
+  });
+}
+int scn_md_input_rules(scn_metadata *h, int32_t *rows, void *stream) {
+  return guarded([&] { export_input_rules(md(h), rows, st(stream)); });
+}
+int scn_md_nactive(scn_metadata *h, const int64_t *spatial, int64_t *n_active) {
+  return guarded([&] {
+    Level *l = find_level(md(h), spatial);
+    *n_active = l ? l->n : 0;
+  });
+}
+int scn_md_batch_size(scn_metadata *h, const int64_t *spatial, int *batch) {
+  return guarded([&] {
+    Level *l = find_level(md(h), spatial);
+    *batch = l ? l->batch : 0;
+  });
+}
+int scn_md_spatial_locations(scn_metadata *h, const int64_t *spatial, int64_t *out, void *stream) {
+  return guarded([&] { spatial_locations(md(h), spatial, out, st(stream)); });
+}
+int scn_md_submanifold_rules(scn_metadata *h, const int64_t *spatial, const int64_t *filter, void *stream) {
+  return guarded([&] { submanifold_rules(md(h), spatial, filter, st(stream)); });
+}
+int scn_md_strided_rules(scn_metadata *h, const int64_t *in_size, const int64_t *out_size,
+                         const int64_t *filter, const int64_t *stride, void *stream) {
+  return guarded([&] { strided_rules(md(h), in_size, out_size, filter, stride, st(stream)); });
+}
+
+int scn_rules_count(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                    const int64_t *d, void *stream, int *count) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (kind == 0)
+      *count = submanifold_rules(m, a, b, st(stream)).K;
+    else if (kind == 1)
+      *count = strided_rules(m, a, b, c, d, st(stream)).by_out.K;
+    else if (kind == 2) {
+      Level *l = find_level(m, a);
+      *count = l ? l->batch : 0;
+    } else
+      throw Error("unknown rulebook kind");
+  });
+}
+int scn_rules_sizes(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                    const int64_t *d, void *stream, int64_t *sizes) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    std::vector<int64_t> v;
+    if (kind == 0)
+      v = submanifold_rules(m, a, b, st(stream)).counts;
+    else if (kind == 1)
+      v = strided_rules(m, a, b, c, d, st(stream)).by_out.counts;
+    else if (kind == 2)
+      v = s2d_sizes(m, a, st(stream));
+    else
+      throw Error("unknown rulebook kind");
+    for (size_t i = 0; i < v.size(); i++) sizes[i] = v[i];
+  });
+}
+int scn_rules_export(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                     const int64_t *d, int k, int32_t *pairs, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (kind == 0) {
+      Table &t = submanifold_rules(m, a, b, st(stream));
+      Level *l = find_level(m, a);
+      export_table_pairs(m, t, l ? l->sched_ptr() : nullptr, k, false, pairs, st(stream));
+    } else if (kind == 1) {
+      StridedRules &r = strided_rules(m, a, b, c, d, st(stream));
+      export_table_pairs(m, r.by_out, nullptr, k, false, pairs, st(stream));
+    } else if (kind == 2) {
+      export_s2d_pairs(m, a, k, pairs, st(stream));
+    } else
+      throw Error("unknown rulebook kind");
+  });
+}
+
+int scn_input_layer_fwd(scn_metadata *h, const float *in, float *out, int planes, void *stream) {
+  return guarded([&] { input_forward(md(h).input, in, out, planes, st(stream)); });
+}
+int scn_output_layer_fwd(scn_metadata *h, const float *in, float *out, int planes, void *stream) {
+  return guarded([&] { output_forward(md(h).input, in, out, planes, st(stream)); });
+}
+
+int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,
+                      float *out, const float *weight, const float *bias, int n_in, int n_out,
+                      int groups, void *stream, double *macs) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    Table &t = submanifold_rules(m, spatial, filter, st(stream));
+    Level *l = find_level(m, spatial);
+    conv_forward(t, l ? l->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
+    // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
+    if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
+  });
+}
+int scn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                 const int64_t *stride, const float *in, float *out, const float *weight,
+                 const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
+    conv_forward(r.by_out, nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
+    if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
+  });
+}
+int scn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                   const int64_t *stride, const float *in, float *out, const float *weight,
+                   const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
+    StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
+    Level *fine = find_level(m, out_size);
+    conv_forward(r.by_in, fine ? fine->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups,
+                 st(stream));
+    if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
+  });
+}
+int scn_maxpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
+                    const int64_t *stride, const float *in, int in_stride, float *out, int planes,
+                    int n_features_to_drop, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
+    StridedRules &r = strided_rules(m, in_size, out_size, size, stride, st(stream));
+    maxpool_forward(r.by_out, in, in_stride, out, planes, n_features_to_drop, st(stream));
+  });
+}
+int scn_bn_eval_fwd(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                    int64_t out_stride, const float *running_mean, const float *running_var,
+                    const float *gamma, const float *beta, float eps, float leakiness, void *stream) {
+  return guarded([&] {
+    bn_eval_forward(in, out, rows, planes, in_stride, out_stride, running_mean, running_var, gamma, beta,
+                    eps, leakiness, st(stream));
+  });
+}
+int scn_s2d_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float *out, int planes,
+                void *stream) {
+  return guarded([&] {
+    Level *l = find_level(md(h), spatial);
+    if (!l) throw Error("sparse to dense: unknown spatial size");
+    s2d_forward(*l, in, out, planes, st(stream));
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,145 @@
+// Shared host/device helpers of libscn_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#define SCN_MAXD 6
+#define SCN_EMPTY_KEY 0xFFFFFFFFFFFFFFFFull
+
+namespace scn {
+
+struct Error : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+inline void hip_check(hipError_t e, const char *what, const char *file, int line) {
+  if (e != hipSuccess) {
+    char buf[512];
+    snprintf(buf, sizeof buf, "%s failed: %s (%s:%d)", what, hipGetErrorString(e), file, line);
+    throw Error(buf);
+  }
+}
+#define HIP_CHECK(x) ::scn::hip_check((x), #x, __FILE__, __LINE__)
+#define LAUNCH_CHECK() ::scn::hip_check(hipGetLastError(), "kernel launch", __FILE__, __LINE__)
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+
+// Owning device buffer.  Grows by reallocation (contents discarded).
+template <class T> struct DevBuf {
+  T *p = nullptr;
+  size_t cap = 0;  // elements
+  DevBuf() = default;
+  DevBuf(const DevBuf &) = delete;
+  DevBuf &operator=(const DevBuf &) = delete;
+  DevBuf(DevBuf &&o) noexcept : p(o.p), cap(o.cap) { o.p = nullptr; o.cap = 0; }
+  DevBuf &operator=(DevBuf &&o) noexcept {
+    if (this != &o) {
+      release();
+      p = o.p;
+      cap = o.cap;
+      o.p = nullptr;
+      o.cap = 0;
+    }
+    return *this;
+  }
+  ~DevBuf() { release(); }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    cap = 0;
+  }
+  void reserve(size_t n) {
+    if (n <= cap) return;
+    release();
+    HIP_CHECK(hipMalloc((void **)&p, n * sizeof(T)));
+    cap = n;
+  }
+  size_t bytes() const { return cap * sizeof(T); }
+};
+
+// Geometry of one level (one spatial size) and the packing of (sample, coordinates) into
+// a 64-bit site key.  dim <= 3: Morton interleave of `bits` bits per coordinate with the
+// sample index above, so ascending keys walk each sample along a Z-order curve; dim >= 4:
+// row-major linear index.  Either way the key is a bijection on valid sites.
+struct Geom {
+  int dim;
+  int bits;       // Morton bits per coordinate (dim <= 3)
+  int64_t size[SCN_MAXD];
+  int64_t vol;    // product of sizes (dim >= 4)
+  int64_t max_batch;  // exclusive bound on the sample index that still fits the key
+};
+
+__host__ __device__ inline uint64_t spread2(uint64_t v) {  // 32 bits -> every 2nd bit
+  v &= 0xFFFFFFFFull;
+  v = (v | (v << 16)) & 0x0000FFFF0000FFFFull;
+  v = (v | (v << 8)) & 0x00FF00FF00FF00FFull;
+  v = (v | (v << 4)) & 0x0F0F0F0F0F0F0F0Full;
+  v = (v | (v << 2)) & 0x3333333333333333ull;
+  v = (v | (v << 1)) & 0x5555555555555555ull;
+  return v;
+}
+__host__ __device__ inline uint64_t spread3(uint64_t v) {  // 21 bits -> every 3rd bit
+  v &= 0x1FFFFFull;
+  v = (v | (v << 32)) & 0x001F00000000FFFFull;
+  v = (v | (v << 16)) & 0x001F0000FF0000FFull;
+  v = (v | (v << 8)) & 0x100F00F00F00F00Full;
+  v = (v | (v << 4)) & 0x10C30C30C30C30C3ull;
+  v = (v | (v << 2)) & 0x1249249249249249ull;
+  return v;
+}
+
+// c: dim coordinates, all inside [0, size).  The last coordinate varies fastest.
+__host__ __device__ inline uint64_t site_key(const Geom &g, const int *c, int batch) {
+  switch (g.dim) {
+  case 1:
+    return ((uint64_t)batch << g.bits) | (uint64_t)c[0];
+  case 2:
+    return ((uint64_t)batch << (2 * g.bits)) | (spread2(c[0]) << 1) | spread2(c[1]);
+  case 3:
+    return ((uint64_t)batch << (3 * g.bits)) | (spread3(c[0]) << 2) | (spread3(c[1]) << 1) |
+           spread3(c[2]);
+  default: {
+    uint64_t k = (uint64_t)batch;
+    for (int d = 0; d < g.dim; d++) k = k * (uint64_t)g.size[d] + (uint64_t)c[d];
+    return k;
+  }
+  }
+}
+
+__device__ inline uint64_t hash64(uint64_t k) {  // murmur3 finaliser
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 33;
+  k *= 0xc4ceb9fe1a85ec53ull;
+  k ^= k >> 33;
+  return k;
+}
+
+// Open-addressing table entry: 16 bytes so that one probe is one aligned 128-bit load.
+struct __attribute__((aligned(16))) HashEntry {
+  unsigned long long key;
+  int row;
+  int pad;
+};
+
+__device__ inline int hash_find(const HashEntry *table, uint64_t mask, uint64_t key) {
+  uint64_t b = hash64(key) & mask;
+  // The table is at most half full, so an empty slot ends every miss; the trip count is
+  // bounded by the table size all the same so that no wave can spin on a damaged table.
+  for (uint64_t i = 0; i <= mask; i++) {
+    const uint4 e = *reinterpret_cast<const uint4 *>(table + b);
+    unsigned long long k = ((unsigned long long)e.y << 32) | e.x;
+    if (k == key) return (int)e.z;
+    if (k == SCN_EMPTY_KEY) return -1;
+    b = (b + 1) & mask;
+  }
+  return -1;
+}
+
+}  // namespace scn

@@ -1,0 +1,107 @@
+// Host-side state behind a scn_metadata handle: levels (one per spatial size), the input
+// layer's rule lists and the cached neighbour tables.
+#pragma once
+#include <map>
+#include <memory>
+
+#include "common.h"
+
+namespace scn {
+
+typedef std::vector<int64_t> SizeKey;
+
+// One spatial size: which sites are active and where each row sits.
+struct Level {
+  Geom g{};
+  int64_t n = 0;     // active sites
+  int64_t npad = 0;  // n rounded up to 64: stride of the SoA arrays below
+  int batch = 0;     // number of samples
+  DevBuf<int> coords;                // [(dim+1)][npad]: coordinates, then sample index
+  DevBuf<unsigned long long> keys;   // [n] site key of each row
+  // Schedule: sched[t] = row, rows listed by ascending site key.  Kernels walk rows in
+  // this order so that one workgroup's rows are neighbours in space whatever order the
+  // caller's points came in.  Null when rows are already numbered by ascending key.
+  DevBuf<int> sched;
+  bool identity_sched = false;
+  DevBuf<HashEntry> table;  // key -> row, built on first use
+  uint64_t mask = 0;
+  bool hash_built = false;
+  const int *sched_ptr() const { return identity_sched ? nullptr : sched.p; }
+};
+
+// Neighbour table: nbr[k * npad + t] = row feeding filter tap k of the output row at
+// schedule position t, or -1.  counts[k] = number of non-negative entries of tap k.
+struct Table {
+  int K = 0;
+  int64_t n = 0, npad = 0;
+  DevBuf<int> nbr;
+  std::vector<int64_t> counts;
+  int64_t total() const {
+    int64_t s = 0;
+    for (auto c : counts) s += c;
+    return s;
+  }
+};
+
+struct StridedRules {
+  Table by_out;  // indexed by rows of the coarse (output) level: value = fine row
+  Table by_in;   // indexed by schedule positions of the fine level: value = coarse row
+  SizeKey in_size, out_size;
+};
+
+struct InputRules {
+  int mode = -1;
+  int max_active = 0;
+  int64_t n_in = 0, n_out = 0;
+  DevBuf<int> row_of_input;  // [n_in]
+  DevBuf<int> sorted_idx;    // [n_in] input indices grouped by site, input order inside a group
+  DevBuf<int> run_start;     // [n_out] first position of the row's group in sorted_idx
+  DevBuf<int> run_len;       // [n_out]
+};
+
+struct Metadata {
+  int dim = 0;
+  std::map<SizeKey, Level> levels;
+  InputRules input;
+  SizeKey input_size;
+  std::map<SizeKey, Table> subm;            // key: spatial || filter
+  std::map<SizeKey, StridedRules> strided;  // key: in_size || filter || stride
+  // scratch reused by the builders
+  DevBuf<unsigned char> tmp;
+  DevBuf<unsigned long long> k0, k1;
+  DevBuf<int> v0, v1, f0, f1, s0, s1;
+  DevBuf<long long> dcounts;
+  DevBuf<int> dflags;
+};
+
+SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);
+Geom make_geom(int dim, const int64_t *spatial);
+
+void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
+                       int ncols, int min_batch, int mode, hipStream_t s);
+void export_input_rules(Metadata &m, int *rows, hipStream_t s);
+void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStream_t s);
+Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s);
+StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
+                            const int64_t *filter, const int64_t *stride, hipStream_t s);
+// Pairs of tap k of a table: (value, row at position t), ordered by t.  Returns the count.
+int64_t export_table_pairs(Metadata &m, const Table &t, const int *sched, int k, bool swap,
+                           int *pairs, hipStream_t s);
+std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t s);
+int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *pairs,
+                         hipStream_t s);
+
+// ops.hip / conv.hip
+void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);
+void conv_forward(const Table &t, const int *rowmap, const float *in, float *out, const float *w,
+                  const float *bias, int n_in, int n_out, int groups, hipStream_t s);
+void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
+                     int drop, hipStream_t s);
+void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                     int64_t out_stride, const float *mean, const float *var, const float *gamma,
+                     const float *beta, float eps, float leak, hipStream_t s);
+void input_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s);
+void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s);
+void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStream_t s);
+
+}  // namespace scn

@@ -1,0 +1,709 @@
+// Levels, input-layer rules and rulebook construction on the GPU.
+//
+// The reference builds all of this on the host, one hash map per sample, one thread per
+// sample (Metadata/IOLayersRules.h:18-121, Metadata/SubmanifoldConvolutionRules.h:26-87,
+// Metadata/ConvolutionRules.h:11-105).  Here every step is data-parallel over sites:
+//   * sites are packed into 64-bit keys (common.h) and radix-sorted; equal keys become
+//     adjacent, which yields duplicate groups (input layer), the distinct output sites of
+//     a strided convolution, and a spatially coherent row schedule, all without atomics;
+//   * submanifold neighbours are found in an open-addressing table of (key -> row);
+//   * rules are stored output-stationary as a table nbr[tap][position] instead of
+//     per-tap pair lists; pair lists are produced on demand by ballot/prefix compaction.
+#include <hipcub/hipcub.hpp>
+
+#include "metadata.h"
+
+namespace scn {
+
+static const int TB = 256;
+static inline dim3 grid_for(int64_t n, int tb = TB) { return dim3((unsigned)std::max<int64_t>(1, ceil_div(n, tb))); }
+
+SizeKey mk(int dim, const int64_t *a, const int64_t *b, const int64_t *c) {
+  SizeKey k(a, a + dim);
+  if (b) k.insert(k.end(), b, b + dim);
+  if (c) k.insert(k.end(), c, c + dim);
+  return k;
+}
+
+Geom make_geom(int dim, const int64_t *spatial) {
+  Geom g{};
+  g.dim = dim;
+  g.vol = 1;
+  int bits = 1;
+  for (int d = 0; d < dim; d++) {
+    if (spatial[d] < 1 || spatial[d] > (int64_t)1 << 30) throw Error("spatial size out of range");
+    g.size[d] = spatial[d];
+    while (((int64_t)1 << bits) < spatial[d]) bits++;
+    if (dim >= 4) {
+      if (g.vol > ((int64_t)1 << 62) / spatial[d]) throw Error("spatial volume does not fit a 64-bit site key");
+      g.vol *= spatial[d];
+    }
+  }
+  g.bits = bits;
+  if (dim <= 3) {
+    if ((dim == 3 && bits > 21) || (dim == 2 && bits > 31) || dim * bits > 62)
+      throw Error("spatial size too large for the site key");
+    int free_bits = 63 - dim * bits;
+    g.max_batch = free_bits >= 31 ? ((int64_t)1 << 31) - 1 : (int64_t)1 << free_bits;
+  } else {
+    g.max_batch = std::min<int64_t>(((int64_t)1 << 31) - 1, ((int64_t)1 << 62) / g.vol);
+  }
+  return g;
+}
+
+// ---- small utilities -------------------------------------------------------------------
+
+__global__ void k_fill32(uint32_t *p, uint32_t v, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = v;
+}
+void fill32(void *p, uint32_t v, int64_t n, hipStream_t s) {
+  if (n <= 0) return;
+  int64_t blocks = std::min<int64_t>(ceil_div(n, TB), 256 * 32);
+  k_fill32<<<dim3((unsigned)blocks), TB, 0, s>>>((uint32_t *)p, v, n);
+  LAUNCH_CHECK();
+}
+
+static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout,
+                       const int *vin, int *vout, int64_t n, hipStream_t s) {
+  size_t bytes = 0;
+  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, 64, s));
+  m.tmp.reserve(bytes + 16);
+  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, 64, s));
+}
+static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipStream_t s) {
+  size_t bytes = 0;
+  HIP_CHECK(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, in, out, (int)n, s));
+  m.tmp.reserve(bytes + 16);
+  HIP_CHECK(hipcub::DeviceScan::ExclusiveSum(m.tmp.p, bytes, in, out, (int)n, s));
+}
+template <class T> static T read_back(const T *dev, hipStream_t s) {
+  T h;
+  HIP_CHECK(hipMemcpyAsync(&h, dev, sizeof(T), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  return h;
+}
+
+static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
+  l.g = g;
+  l.n = n;
+  l.npad = round_up(std::max<int64_t>(n, 1), 64);
+  l.batch = batch;
+  l.coords.reserve((size_t)(g.dim + 1) * l.npad);
+  l.keys.reserve((size_t)l.npad);
+  l.hash_built = false;
+}
+
+// ---- input layer -----------------------------------------------------------------------
+
+// flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
+// flags[1] = max sample index seen.
+__global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols,
+                             unsigned long long *keys, int *idx, int *flags) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t *c = coords + i * ncols;
+  int cc[SCN_MAXD];
+  bool ok = true;
+  for (int d = 0; d < g.dim; d++) {
+    int64_t v = c[d];
+    if (v < 0 || v >= g.size[d]) ok = false;
+    cc[d] = (int)v;
+  }
+  int64_t b = ncols > g.dim ? c[g.dim] : 0;
+  if (b < 0 || b >= g.max_batch) {
+    atomicOr(&flags[0], 2);
+    ok = false;
+    b = 0;
+  } else {
+    atomicMax(&flags[1], (int)b);
+  }
+  if (!ok) {
+    atomicOr(&flags[0], 1);
+    keys[i] = SCN_EMPTY_KEY;
+  } else {
+    keys[i] = site_key(g, cc, (int)b);
+  }
+  idx[i] = (int)i;
+}
+
+// mode 0: row = input index.
+__global__ void k_input_rows_identity(Geom g, const int64_t *coords, int64_t n, int ncols,
+                                      int64_t npad, int *soa) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t *c = coords + i * ncols;
+  for (int d = 0; d < g.dim; d++) soa[d * npad + i] = (int)c[d];
+  soa[g.dim * npad + i] = ncols > g.dim ? (int)c[g.dim] : 0;
+}
+
+// After the stable sort: head[p] marks the first point of each group of equal keys;
+// is_first[i] marks input points that are the first occurrence of their site.
+__global__ void k_group_heads(const unsigned long long *skeys, const int *sidx, int64_t n,
+                              int *head, int *is_first) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  int h = (p == 0 || skeys[p] != skeys[p - 1]) ? 1 : 0;
+  head[p] = h;
+  is_first[sidx[p]] = h;
+}
+
+// Heads: row = rank of the first occurrence in input order (Metadata/IOLayersRules.h:84-87).
+__global__ void k_assign_rows(Geom g, const int64_t *coords, int ncols, const unsigned long long *skeys,
+                              const int *sidx, const int *head, const int *head_scan,
+                              const int *first_scan, int64_t n, int64_t npad, int *soa,
+                              unsigned long long *level_keys, int *sched, int *row_of_group,
+                              int *head_pos) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n || !head[p]) return;
+  int i = sidx[p];
+  int row = first_scan[i];
+  int u = head_scan[p];
+  sched[u] = row;
+  row_of_group[u] = row;
+  head_pos[u] = (int)p;
+  level_keys[row] = skeys[p];
+  const int64_t *c = coords + (int64_t)i * ncols;
+  for (int d = 0; d < g.dim; d++) soa[d * npad + row] = (int)c[d];
+  soa[g.dim * npad + row] = ncols > g.dim ? (int)c[g.dim] : 0;
+}
+
+__global__ void k_finish_groups(const int *sidx, const int *head, const int *head_scan,
+                                const int *row_of_group, const int *head_pos, int64_t n,
+                                int n_groups, int *row_of_input, int *run_start, int *run_len,
+                                int *max_active) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  int u = head_scan[p] + head[p] - 1;
+  int row = row_of_group[u];
+  row_of_input[sidx[p]] = row;
+  if (head[p]) {
+    int next = (u + 1 < n_groups) ? head_pos[u + 1] : (int)n;
+    int len = next - (int)p;
+    run_start[row] = (int)p;
+    run_len[row] = len;
+    atomicMax(max_active, len);
+  }
+}
+
+void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
+                       int ncols, int min_batch, int mode, hipStream_t s) {
+  if (ncols != m.dim && ncols != m.dim + 1) throw Error("coords must have dim or dim+1 columns");
+  if (mode < 0 || mode > 4) throw Error("input layer mode must be 0..4");
+  if (n >= ((int64_t)1 << 31) - 64) throw Error("too many input points for int32 rule indices");
+  Geom g = make_geom(m.dim, spatial);
+  SizeKey key = mk(m.dim, spatial);
+  m.input_size = key;
+  Level &L = m.levels[key];
+  InputRules &R = m.input;
+  R.mode = mode;
+  R.n_in = n;
+  R.max_active = 1;
+  int batch_floor = ncols == m.dim ? 1 : std::max(min_batch, 0);
+  if (n == 0) {
+    alloc_level(L, g, 0, batch_floor);
+    L.identity_sched = true;
+    R.n_out = 0;
+    return;
+  }
+  m.k0.reserve(n);
+  m.k1.reserve(n);
+  m.v0.reserve(n);
+  m.v1.reserve(n);
+  m.dflags.reserve(8);
+  fill32(m.dflags.p, 0, 8, s);
+  k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, m.k0.p, m.v0.p, m.dflags.p);
+  LAUNCH_CHECK();
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s);
+  int hflags[2];
+  HIP_CHECK(hipMemcpyAsync(hflags, m.dflags.p, sizeof hflags, hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
+  if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");
+  // Metadata/IOLayersRules.h:25,46-47,76-77: the batch is at least min_batch and grows to
+  // the largest sample index + 1; without a sample column there is exactly one sample.
+  int batch = ncols == m.dim ? 1 : std::max(batch_floor, hflags[1] + 1);
+
+  if (mode == 0) {
+    alloc_level(L, g, n, batch);
+    L.sched.reserve(n);
+    L.identity_sched = false;
+    k_input_rows_identity<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, L.npad, L.coords.p);
+    LAUNCH_CHECK();
+    HIP_CHECK(hipMemcpyAsync(L.keys.p, m.k0.p, n * sizeof(unsigned long long), hipMemcpyDeviceToDevice, s));
+    HIP_CHECK(hipMemcpyAsync(L.sched.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
+    R.n_out = n;
+    return;
+  }
+
+  m.f0.reserve(n);  // head
+  m.f1.reserve(n);  // is_first
+  m.s0.reserve(n + 1);  // head_scan
+  m.s1.reserve(n + 1);  // first_scan
+  k_group_heads<<<grid_for(n), TB, 0, s>>>(m.k1.p, m.v1.p, n, m.f0.p, m.f1.p);
+  LAUNCH_CHECK();
+  exclusive_scan(m, m.f0.p, m.s0.p, n, s);
+  exclusive_scan(m, m.f1.p, m.s1.p, n, s);
+  int last[2];
+  HIP_CHECK(hipMemcpyAsync(&last[0], m.s0.p + (n - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipMemcpyAsync(&last[1], m.f0.p + (n - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  int64_t N = (int64_t)last[0] + last[1];
+  alloc_level(L, g, N, batch);
+  L.sched.reserve(N);
+  L.identity_sched = false;
+  R.n_out = N;
+  R.row_of_input.reserve(n);
+  R.sorted_idx.reserve(n);
+  R.run_start.reserve(N);
+  R.run_len.reserve(N);
+  m.v0.reserve(std::max<int64_t>(n, 2 * N + 2));  // reused: row_of_group | head_pos
+  int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
+  fill32(m.dflags.p, 0, 8, s);
+  k_assign_rows<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, m.k1.p, m.v1.p, m.f0.p, m.s0.p, m.s1.p,
+                                           n, L.npad, L.coords.p, L.keys.p, L.sched.p, row_of_group,
+                                           head_pos);
+  LAUNCH_CHECK();
+  k_finish_groups<<<grid_for(n), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, row_of_group, head_pos, n, (int)N,
+                                             R.row_of_input.p, R.run_start.p, R.run_len.p,
+                                             m.dflags.p + 2);
+  LAUNCH_CHECK();
+  HIP_CHECK(hipMemcpyAsync(R.sorted_idx.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
+  int ma = read_back(m.dflags.p + 2, s);
+  // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2.
+  R.max_active = (mode == 3 || mode == 4) ? ma : 1;
+}
+
+// Reference layout of the rule rows (Metadata/IOLayersRules.h:96-119).
+__global__ void k_export_input_rules(const int *sorted_idx, const int *run_start, const int *run_len,
+                                     int64_t n_out, int mode, int max_active, int *rows) {
+  int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_out) return;
+  int *o = rows + r * (1 + max_active);
+  int st = run_start[r], len = run_len[r];
+  if (mode == 1) {
+    o[0] = 1;
+    o[1] = sorted_idx[st];
+  } else if (mode == 2) {
+    o[0] = 1;
+    o[1] = sorted_idx[st + len - 1];
+  } else {
+    o[0] = len;
+    for (int q = 0; q < max_active; q++) o[1 + q] = q < len ? sorted_idx[st + q] : 0;
+  }
+}
+void export_input_rules(Metadata &m, int *rows, hipStream_t s) {
+  InputRules &R = m.input;
+  if (R.mode <= 0 || R.n_out == 0) return;
+  k_export_input_rules<<<grid_for(R.n_out), TB, 0, s>>>(R.sorted_idx.p, R.run_start.p, R.run_len.p,
+                                                        R.n_out, R.mode, R.max_active, rows);
+  LAUNCH_CHECK();
+}
+
+__global__ void k_locations(const int *soa, int64_t n, int64_t npad, int dim, int64_t *out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * (dim + 1)) return;
+  int64_t r = i / (dim + 1);
+  int d = (int)(i - r * (dim + 1));
+  out[i] = soa[d * npad + r];
+}
+void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStream_t s) {
+  auto it = m.levels.find(mk(m.dim, spatial));
+  if (it == m.levels.end() || it->second.n == 0) return;
+  Level &L = it->second;
+  k_locations<<<grid_for(L.n * (m.dim + 1)), TB, 0, s>>>(L.coords.p, L.n, L.npad, m.dim, out);
+  LAUNCH_CHECK();
+}
+
+// ---- hash table of a level -------------------------------------------------------------
+
+// Later rows win on equal keys, as repeated `mp[p] = i` does for input-layer mode 0
+// (Metadata/IOLayersRules.h:41,54); all other levels have distinct keys.
+__global__ void k_hash_insert(const unsigned long long *keys, int64_t n, HashEntry *table,
+                              unsigned long long mask) {
+  int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n) return;
+  unsigned long long key = keys[r];
+  unsigned long long b = hash64(key) & mask;
+  for (unsigned long long i = 0; i <= mask; i++) {
+    unsigned long long old = atomicCAS(&table[b].key, SCN_EMPTY_KEY, key);
+    if (old == SCN_EMPTY_KEY || old == key) {
+      atomicMax(&table[b].row, (int)r);
+      return;
+    }
+    b = (b + 1) & mask;
+  }
+}
+static void ensure_hash(Level &L, hipStream_t s) {
+  if (L.hash_built) return;
+  uint64_t cap = 64;
+  while (cap < (uint64_t)L.n * 2) cap <<= 1;
+  L.table.reserve(cap);
+  L.mask = cap - 1;
+  fill32(L.table.p, 0xFFFFFFFFu, (int64_t)cap * 4, s);  // key = EMPTY, row = -1
+  if (L.n) {
+    k_hash_insert<<<grid_for(L.n), TB, 0, s>>>(L.keys.p, L.n, L.table.p, L.mask);
+    LAUNCH_CHECK();
+  }
+  L.hash_built = true;
+}
+
+// ---- submanifold rules -----------------------------------------------------------------
+
+struct Filt {
+  int dim, K, M;
+  int size[SCN_MAXD], stride[SCN_MAXD], out_size[SCN_MAXD], m[SCN_MAXD];
+};
+
+// One thread per schedule position t: probe the filter box around the row's site
+// (Metadata/SubmanifoldConvolutionRules.h:11-45; taps enumerate the box row-major with the
+// last dimension fastest, Metadata/RectangularRegions.h:56-71).
+__global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, int64_t n,
+                             int64_t npad, const HashEntry *table, unsigned long long mask,
+                             int *nbr, unsigned long long *counts) {
+  extern __shared__ int lcount[];
+  for (int k = threadIdx.x; k < f.K; k += blockDim.x) lcount[k] = 0;
+  __syncthreads();
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) {
+    int row = sched ? sched[t] : (int)t;
+    int c[SCN_MAXD], tap[SCN_MAXD], q[SCN_MAXD];
+    for (int d = 0; d < g.dim; d++) {
+      c[d] = soa[d * npad + row];
+      tap[d] = 0;
+    }
+    int b = soa[g.dim * npad + row];
+    for (int k = 0; k < f.K; k++) {
+      bool inside = true;
+      for (int d = 0; d < g.dim; d++) {
+        q[d] = c[d] + tap[d] - f.size[d] / 2;
+        if (q[d] < 0 || q[d] >= g.size[d]) inside = false;
+      }
+      int j = -1;
+      if (inside) j = hash_find(table, mask, site_key(g, q, b));
+      nbr[(int64_t)k * npad + t] = j;
+      if (j >= 0) atomicAdd(&lcount[k], 1);
+      for (int d = g.dim - 1; d >= 0; d--) {  // next tap, last dimension fastest
+        if (++tap[d] < f.size[d]) break;
+        tap[d] = 0;
+      }
+    }
+  }
+  __syncthreads();
+  for (int k = threadIdx.x; k < f.K; k += blockDim.x)
+    if (lcount[k]) atomicAdd(&counts[k], (unsigned long long)lcount[k]);
+}
+
+static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const int64_t *out_size) {
+  Filt f{};
+  f.dim = dim;
+  int64_t K = 1, M = 1;
+  for (int d = 0; d < dim; d++) {
+    if (size[d] < 1 || size[d] > 64) throw Error("filter size must be in 1..64");
+    f.size[d] = (int)size[d];
+    f.stride[d] = stride ? (int)stride[d] : 1;
+    if (f.stride[d] < 1) throw Error("filter stride must be positive");
+    f.out_size[d] = out_size ? (int)out_size[d] : 0;
+    f.m[d] = (f.size[d] + f.stride[d] - 1) / f.stride[d];
+    K *= size[d];
+    M *= f.m[d];
+    if (K > 4096) throw Error("filter volume above 4096 is not supported");
+  }
+  f.K = (int)K;
+  f.M = (int)M;
+  return f;
+}
+
+static void fetch_counts(Metadata &m, Table &t, hipStream_t s) {
+  std::vector<unsigned long long> h(t.K);
+  HIP_CHECK(hipMemcpyAsync(h.data(), m.dcounts.p, t.K * sizeof(long long), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  t.counts.assign(h.begin(), h.end());
+}
+
+Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s) {
+  SizeKey key = mk(m.dim, spatial, filter);
+  auto it = m.subm.find(key);
+  if (it != m.subm.end()) return it->second;
+  Filt f = make_filt(m.dim, filter, nullptr, nullptr);
+  Table t;
+  t.K = f.K;
+  auto lit = m.levels.find(mk(m.dim, spatial));
+  if (lit == m.levels.end() || lit->second.n == 0) {
+    // Metadata/Metadata.cpp:445: an unknown level is an empty one.
+    t.n = 0;
+    t.npad = 64;
+    t.counts.assign(f.K, 0);
+    return m.subm.emplace(key, std::move(t)).first->second;
+  }
+  Level &L = lit->second;
+  ensure_hash(L, s);
+  t.n = L.n;
+  t.npad = L.npad;
+  t.nbr.reserve((size_t)f.K * t.npad);
+  m.dcounts.reserve(4096);
+  fill32(m.dcounts.p, 0, 2 * f.K, s);
+  k_subm_rules<<<grid_for(L.n), TB, f.K * sizeof(int), s>>>(L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad,
+                                                            L.table.p, L.mask, t.nbr.p,
+                                                            (unsigned long long *)m.dcounts.p);
+  LAUNCH_CHECK();
+  fetch_counts(m, t, s);
+  return m.subm.emplace(key, std::move(t)).first->second;
+}
+
+// ---- strided rules ---------------------------------------------------------------------
+
+// Candidate output sites of every input site (Metadata/RectangularRegions.h:109-119):
+// per dimension j in [max(0, ceil((p-size+1)/stride)), min(out-1, floor(p/stride))].
+// Slot e = t * M + m holds the key of the m-th candidate of the row at position t, or EMPTY.
+__device__ inline bool candidate(const Geom &gi, const Filt &f, const int *p, int m, int *j) {
+  for (int d = f.dim - 1; d >= 0; d--) {
+    int md = m % f.m[d];
+    m /= f.m[d];
+    int num = p[d] - f.size[d] + 1;
+    int lb = num <= 0 ? 0 : (num + f.stride[d] - 1) / f.stride[d];
+    int ub = min(f.out_size[d] - 1, p[d] / f.stride[d]);
+    j[d] = lb + md;
+    if (j[d] > ub) return false;
+  }
+  return true;
+}
+
+__global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, const int *sched,
+                                     int64_t n, int64_t npad, unsigned long long *keys, int *payload) {
+  int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n * f.M) return;
+  int64_t t = e / f.M;
+  int m = (int)(e - t * f.M);
+  int row = sched ? sched[t] : (int)t;
+  int p[SCN_MAXD], j[SCN_MAXD];
+  for (int d = 0; d < f.dim; d++) p[d] = soa[d * npad + row];
+  int b = soa[f.dim * npad + row];
+  keys[e] = candidate(gi, f, p, m, j) ? site_key(go, j, b) : SCN_EMPTY_KEY;
+  payload[e] = (int)e;
+}
+
+__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  head[p] = (skeys[p] != SCN_EMPTY_KEY && (p == 0 || skeys[p] != skeys[p - 1])) ? 1 : 0;
+}
+
+// One thread per sorted candidate: output row = number of heads before it; the filter tap
+// is the input site's offset inside the output's input box (Metadata/ConvolutionRules.h:19-31,
+// Metadata/RectangularRegions.h:30-38,95-105).
+__global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched, int64_t npad_in,
+                               const unsigned long long *skeys, const int *spayload, const int *head,
+                               const int *head_scan, int64_t n_cand, int64_t npad_out, int *by_out,
+                               int *by_in, int *out_soa, unsigned long long *out_keys,
+                               unsigned long long *counts) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n_cand) return;
+  unsigned long long key = skeys[p];
+  if (key == SCN_EMPTY_KEY) return;
+  int e = spayload[p];
+  int t = e / f.M, m = e - t * f.M;
+  int row = sched ? sched[t] : t;
+  int pc[SCN_MAXD], j[SCN_MAXD];
+  for (int d = 0; d < f.dim; d++) pc[d] = soa[d * npad_in + row];
+  candidate(gi, f, pc, m, j);
+  int k = 0;
+  for (int d = 0; d < f.dim; d++) k = k * f.size[d] + (pc[d] - j[d] * f.stride[d]);
+  int o = head_scan[p] + head[p] - 1;
+  by_out[(int64_t)k * npad_out + o] = row;
+  by_in[(int64_t)k * npad_in + t] = o;
+  atomicAdd(&counts[k], 1ull);
+  if (head[p]) {
+    for (int d = 0; d < f.dim; d++) out_soa[d * npad_out + o] = j[d];
+    out_soa[f.dim * npad_out + o] = soa[f.dim * npad_in + row];
+    out_keys[o] = key;
+  }
+}
+
+StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
+                            const int64_t *filter, const int64_t *stride, hipStream_t s) {
+  SizeKey key = mk(m.dim, in_size, filter, stride);
+  auto it = m.strided.find(key);
+  if (it != m.strided.end()) return it->second;
+  Filt f = make_filt(m.dim, filter, stride, out_size);
+  Geom go = make_geom(m.dim, out_size);
+  StridedRules R;
+  R.in_size = mk(m.dim, in_size);
+  R.out_size = mk(m.dim, out_size);
+  R.by_out.K = R.by_in.K = f.K;
+  R.by_out.counts.assign(f.K, 0);
+  R.by_in.counts.assign(f.K, 0);
+  if (R.in_size == R.out_size) throw Error("strided rules: input and output spatial size coincide");
+
+  auto lit = m.levels.find(R.in_size);
+  int64_t n = lit == m.levels.end() ? 0 : lit->second.n;
+  int batch = lit == m.levels.end() ? 0 : lit->second.batch;
+  // Building a strided rulebook replaces the output level (Metadata/ConvolutionRules.h:68-70)
+  // and whatever was cached for it.
+  for (auto i = m.subm.begin(); i != m.subm.end();)
+    i = std::equal(R.out_size.begin(), R.out_size.end(), i->first.begin()) ? m.subm.erase(i) : std::next(i);
+  Level &LO = m.levels[R.out_size];
+  LO = Level();
+  LO.identity_sched = true;
+  if (n == 0) {
+    alloc_level(LO, go, 0, batch);
+    R.by_out.n = 0;
+    R.by_out.npad = 64;
+    R.by_in.n = 0;
+    R.by_in.npad = 64;
+    return m.strided.emplace(key, std::move(R)).first->second;
+  }
+  Level &LI = m.levels[R.in_size];
+  int64_t nc = n * f.M;
+  if (nc >= ((int64_t)1 << 31) - 64) throw Error("strided rules: too many candidate pairs for int32 indices");
+  m.k0.reserve(nc);
+  m.k1.reserve(nc);
+  m.v0.reserve(nc);
+  m.v1.reserve(nc);
+  m.f0.reserve(nc);
+  m.s0.reserve(nc + 1);
+  k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), n, LI.npad,
+                                                   m.k0.p, m.v0.p);
+  LAUNCH_CHECK();
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s);
+  k_strided_heads<<<grid_for(nc), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
+  LAUNCH_CHECK();
+  exclusive_scan(m, m.f0.p, m.s0.p, nc, s);
+  int last[2];
+  HIP_CHECK(hipMemcpyAsync(&last[0], m.s0.p + (nc - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipMemcpyAsync(&last[1], m.f0.p + (nc - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  int64_t n_out = (int64_t)last[0] + last[1];
+  alloc_level(LO, go, n_out, batch);
+  R.by_out.n = n_out;
+  R.by_out.npad = LO.npad;
+  R.by_in.n = n;
+  R.by_in.npad = LI.npad;
+  R.by_out.nbr.reserve((size_t)f.K * LO.npad);
+  R.by_in.nbr.reserve((size_t)f.K * LI.npad);
+  fill32(R.by_out.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LO.npad, s);
+  fill32(R.by_in.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LI.npad, s);
+  m.dcounts.reserve(4096);
+  fill32(m.dcounts.p, 0, 2 * f.K, s);
+  k_strided_emit<<<grid_for(nc), TB, 0, s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), LI.npad, m.k1.p, m.v1.p,
+                                             m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
+                                             LO.coords.p, LO.keys.p, (unsigned long long *)m.dcounts.p);
+  LAUNCH_CHECK();
+  fetch_counts(m, R.by_out, s);
+  R.by_in.counts = R.by_out.counts;
+  return m.strided.emplace(key, std::move(R)).first->second;
+}
+
+// ---- pair-list export (ballot / prefix compaction) --------------------------------------
+
+// Each wavefront counts its hits with a ballot, one lane reserves the range in the block's
+// LDS counter, and lanes write at their prefix rank; blocks take their base from a scan of
+// the per-block totals, so the list is ordered by schedule position and deterministic.
+__global__ void k_tap_block_counts(const int *nbr, int64_t n, int *block_counts) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  bool hit = t < n && nbr[t] >= 0;
+  unsigned long long bal = __ballot(hit);
+  __shared__ int total;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) atomicAdd(&total, __popcll(bal));
+  __syncthreads();
+  if (threadIdx.x == 0) block_counts[blockIdx.x] = total;
+}
+__global__ void k_tap_compact(const int *nbr, const int *sched, int64_t n, const int *block_base,
+                              bool swap, int *pairs) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int v = t < n ? nbr[t] : -1;
+  bool hit = v >= 0;
+  unsigned long long bal = __ballot(hit);
+  int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ int wave_base[TB / 64];
+  if (lane == 0) wave_base[wave] = __popcll(bal);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int w = 0; w < TB / 64; w++) {
+      int c = wave_base[w];
+      wave_base[w] = acc;
+      acc += c;
+    }
+  }
+  __syncthreads();
+  if (hit) {
+    int rank = __popcll(bal & ((1ull << lane) - 1ull));
+    int64_t pos = (int64_t)block_base[blockIdx.x] + wave_base[wave] + rank;
+    int row = sched ? sched[t] : (int)t;
+    pairs[2 * pos + (swap ? 1 : 0)] = v;
+    pairs[2 * pos + (swap ? 0 : 1)] = row;
+  }
+}
+int64_t export_table_pairs(Metadata &m, const Table &t, const int *sched, int k, bool swap, int *pairs,
+                           hipStream_t s) {
+  if (k < 0 || k >= t.K) throw Error("rule list index out of range");
+  if (t.n == 0 || t.counts[k] == 0) return 0;
+  int64_t blocks = ceil_div(t.n, TB);
+  m.f1.reserve(blocks + 1);
+  m.s1.reserve(blocks + 1);
+  const int *col = t.nbr.p + (int64_t)k * t.npad;
+  k_tap_block_counts<<<dim3((unsigned)blocks), TB, 0, s>>>(col, t.n, m.f1.p);
+  LAUNCH_CHECK();
+  exclusive_scan(m, m.f1.p, m.s1.p, blocks, s);
+  k_tap_compact<<<dim3((unsigned)blocks), TB, 0, s>>>(col, sched, t.n, m.s1.p, swap, pairs);
+  LAUNCH_CHECK();
+  return t.counts[k];
+}
+
+// Sparse-to-dense lists: per sample, (row, row-major offset) (Metadata/ConvolutionRules.h:130-151).
+__global__ void k_sample_hist(const int *soa_batch, int64_t n, int batch, unsigned long long *hist) {
+  int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < n) {
+    int b = soa_batch[r];
+    if (b >= 0 && b < batch) atomicAdd(&hist[b], 1ull);
+  }
+}
+std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t s) {
+  auto it = m.levels.find(mk(m.dim, spatial));
+  if (it == m.levels.end()) return {};
+  Level &L = it->second;
+  std::vector<int64_t> out(L.batch, 0);
+  if (L.n == 0 || L.batch == 0) return out;
+  DevBuf<unsigned long long> hist;
+  hist.reserve(L.batch);
+  fill32(hist.p, 0, 2 * (int64_t)L.batch, s);
+  k_sample_hist<<<grid_for(L.n), TB, 0, s>>>(L.coords.p + (int64_t)m.dim * L.npad, L.n, L.batch, hist.p);
+  LAUNCH_CHECK();
+  std::vector<unsigned long long> h(L.batch);
+  HIP_CHECK(hipMemcpyAsync(h.data(), hist.p, L.batch * sizeof(long long), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  out.assign(h.begin(), h.end());
+  return out;
+}
+__global__ void k_s2d_flags(Geom g, const int *soa, int64_t n, int64_t npad, int sample, int *flag) {
+  int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < n) flag[r] = soa[g.dim * npad + r] == sample ? 1 : 0;
+}
+__global__ void k_s2d_pairs(Geom g, const int *soa, int64_t n, int64_t npad, const int *flag,
+                            const int *scan, int *pairs) {
+  int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n || !flag[r]) return;
+  int64_t off = 0;
+  for (int d = 0; d < g.dim; d++) off = off * g.size[d] + soa[d * npad + r];
+  pairs[2 * scan[r]] = (int)r;
+  pairs[2 * scan[r] + 1] = (int)off;
+}
+int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *pairs, hipStream_t s) {
+  auto it = m.levels.find(mk(m.dim, spatial));
+  if (it == m.levels.end() || it->second.n == 0) return 0;
+  Level &L = it->second;
+  m.f1.reserve(L.n + 1);
+  m.s1.reserve(L.n + 1);
+  k_s2d_flags<<<grid_for(L.n), TB, 0, s>>>(L.g, L.coords.p, L.n, L.npad, sample, m.f1.p);
+  LAUNCH_CHECK();
+  exclusive_scan(m, m.f1.p, m.s1.p, L.n, s);
+  k_s2d_pairs<<<grid_for(L.n), TB, 0, s>>>(L.g, L.coords.p, L.n, L.npad, m.f1.p, m.s1.p, pairs);
+  LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace scn

@@ -1,0 +1,197 @@
+// Bandwidth-bound forward ops: eval batch-norm + leaky ReLU, max pooling, the input and
+// output layers and sparse-to-dense.  Each is a single pass that reads its input once
+// and writes its output once with 16-byte accesses where the row length allows.
+#include "metadata.h"
+
+namespace scn {
+
+static const int TB = 256;
+
+// ---- batch norm (eval) + leaky ReLU -----------------------------------------------------
+// CPU/BatchNormalization.cpp:41-61: w = gamma / sqrt(var + eps), b = beta - mean * w,
+// y = x * w + b, y *= (y > 0 ? 1 : leakiness).
+template <int V>
+__global__ void k_bn_eval(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                          int64_t out_stride, const float *mean, const float *var, const float *gamma,
+                          const float *beta, float eps, float leak) {
+  // thread -> (row, group of V planes); consecutive threads cover one row, then the next
+  int groups = planes / V;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = rows * groups;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    int64_t r = i / groups;
+    int p0 = (int)(i - r * groups) * V;
+    float x[V], w[V], b[V];
+    if (V == 4) {
+      float4 t = *reinterpret_cast<const float4 *>(in + r * in_stride + p0);
+      x[0] = t.x, x[1] = t.y, x[2] = t.z, x[3] = t.w;
+    } else {
+      for (int v = 0; v < V; v++) x[v] = in[r * in_stride + p0 + v];
+    }
+    for (int v = 0; v < V; v++) {
+      float inv = 1.0f / sqrtf(var[p0 + v] + eps);
+      w[v] = inv * (gamma ? gamma[p0 + v] : 1.0f);
+      b[v] = -mean[p0 + v] * w[v] + (beta ? beta[p0 + v] : 0.0f);
+      float y = x[v] * w[v] + b[v];
+      x[v] = y * (y > 0 ? 1.0f : leak);
+    }
+    if (V == 4) {
+      *reinterpret_cast<float4 *>(out + r * out_stride + p0) = make_float4(x[0], x[1], x[2], x[3]);
+    } else {
+      for (int v = 0; v < V; v++) out[r * out_stride + p0 + v] = x[v];
+    }
+  }
+}
+
+void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                     int64_t out_stride, const float *mean, const float *var, const float *gamma,
+                     const float *beta, float eps, float leak, hipStream_t s) {
+  if (rows <= 0 || planes <= 0) return;
+  bool vec = planes % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 &&
+             ((uintptr_t)in % 16 == 0) && ((uintptr_t)out % 16 == 0);
+  int64_t total = rows * (vec ? planes / 4 : planes);
+  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  if (vec)
+    k_bn_eval<4><<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, mean,
+                                                       var, gamma, beta, eps, leak);
+  else
+    k_bn_eval<1><<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, mean,
+                                                       var, gamma, beta, eps, leak);
+  LAUNCH_CHECK();
+}
+
+// ---- max pooling ------------------------------------------------------------------------
+// CPU/MaxPooling.cpp:7-20,50: the output starts at zero and takes every input of its window
+// that compares greater, so the result is max(0, active inputs); output-stationary here.
+__global__ void k_maxpool(const int *nbr, int K, int64_t n_out, int64_t npad, const float *in,
+                          int in_stride, float *out, int planes) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = n_out * planes;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    int64_t o = i / planes;
+    int p = (int)(i - o * planes);
+    float acc = 0.0f;
+    for (int k = 0; k < K; k++) {
+      int j = nbr[(int64_t)k * npad + o];
+      if (j >= 0) {
+        float v = in[(int64_t)j * in_stride + p];
+        if (acc < v) acc = v;
+      }
+    }
+    out[i] = acc;
+  }
+}
+void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
+                     hipStream_t s) {
+  if (t.n == 0 || planes <= 0) return;
+  int64_t total = t.n * planes;
+  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  k_maxpool<<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, in + drop, in_stride, out,
+                                                  planes);
+  LAUNCH_CHECK();
+}
+
+// ---- input / output layers --------------------------------------------------------------
+// CPU/IOLayers.cpp:11-29: out[row] = sum over the row's points, in input order, of
+// mult * in[point], mult = 1/count for mode 4.  Modes 1 / 2 copy the first / last point.
+__global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const int *run_len,
+                            int64_t n_out, int mode, const float *in, float *out, int planes) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = n_out * planes;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    int64_t r = i / planes;
+    int p = (int)(i - r * planes);
+    int st = run_start[r], len = run_len[r];
+    float acc = 0.0f;
+    if (mode == 1) {
+      acc += in[(int64_t)sorted_idx[st] * planes + p];
+    } else if (mode == 2) {
+      acc += in[(int64_t)sorted_idx[st + len - 1] * planes + p];
+    } else {
+      float mult = (mode == 4 && len > 0) ? 1.0f / (float)len : 1.0f;
+      for (int q = 0; q < len; q++) acc += mult * in[(int64_t)sorted_idx[st + q] * planes + p];
+    }
+    out[i] = acc;
+  }
+}
+void input_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s) {
+  if (r.mode < 0) throw Error("input layer rules have not been built");
+  if (planes <= 0) return;
+  if (r.mode == 0) {
+    if (r.n_in)
+      HIP_CHECK(hipMemcpyAsync(out, in, sizeof(float) * r.n_in * planes, hipMemcpyDeviceToDevice, s));
+    return;
+  }
+  if (r.n_out == 0) return;
+  int64_t total = r.n_out * planes;
+  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.n_out,
+                                                    r.mode, in, out, planes);
+  LAUNCH_CHECK();
+}
+
+// CPU/IOLayers.cpp:95-115 (InputLayer_BackwardPass :31-47 without averaging): every input
+// point listed in its site's rule receives the site's row; as a gather per input point.
+// Modes 1 / 2 list a single point per site, the others get zeros.
+__global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, const int *run_start,
+                             const int *run_len, int64_t n_in, int mode, const float *in, float *out,
+                             int planes) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = n_in * planes;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    int64_t pt = i / planes;
+    int p = (int)(i - pt * planes);
+    int row = row_of_input[pt];
+    bool listed = true;
+    if (mode == 1) listed = sorted_idx[run_start[row]] == (int)pt;
+    if (mode == 2) listed = sorted_idx[run_start[row] + run_len[row] - 1] == (int)pt;
+    out[i] = listed ? in[(int64_t)row * planes + p] : 0.0f;
+  }
+}
+void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s) {
+  if (r.mode < 0) throw Error("input layer rules have not been built");
+  if (planes <= 0 || r.n_in == 0) return;
+  if (r.mode == 0) {
+    HIP_CHECK(hipMemcpyAsync(out, in, sizeof(float) * r.n_in * planes, hipMemcpyDeviceToDevice, s));
+    return;
+  }
+  int64_t total = r.n_in * planes;
+  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  k_output_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
+                                                     r.run_len.p, r.n_in, r.mode, in, out, planes);
+  LAUNCH_CHECK();
+}
+
+// ---- sparse to dense --------------------------------------------------------------------
+// CPU/SparseToDense.cpp:7-19,35-64: out[sample][plane][offset(site)] = in[row][plane] on a
+// zero-filled [batch, planes, spatial...] tensor.
+__global__ void k_s2d(Geom g, const int *soa, int64_t n, int64_t npad, const float *in, float *out,
+                      int planes, int64_t vol) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = n * planes;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    int64_t r = i / planes;
+    int p = (int)(i - r * planes);
+    int64_t off = 0;
+    for (int d = 0; d < g.dim; d++) off = off * g.size[d] + soa[d * npad + r];
+    int b = soa[g.dim * npad + r];
+    out[((int64_t)b * planes + p) * vol + off] = in[i];
+  }
+}
+void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStream_t s) {
+  int64_t vol = 1;
+  for (int d = 0; d < l.g.dim; d++) vol *= l.g.size[d];
+  fill32(out, 0, (int64_t)l.batch * planes * vol, s);
+  if (l.n == 0 || planes <= 0) return;
+  int64_t total = l.n * planes;
+  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  k_s2d<<<dim3((unsigned)blocks), TB, 0, s>>>(l.g, l.coords.p, l.n, l.npad, in, out, planes, vol);
+  LAUNCH_CHECK();
+}
+
+}  // namespace scn

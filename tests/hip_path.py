@@ -1,0 +1,175 @@
+"""The C ABI of libscn_hip.so behind the interface of oracle.cpu_path.CpuPath, so that the
+checks written for the CPU implementations run unchanged on the GPU library.  numpy in,
+numpy out; device memory and the stream come from torch."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from sparseconvnet_amd import _lib
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(a, dtype):
+    return torch.as_tensor(np.ascontiguousarray(a), dtype=dtype).cuda().contiguous()
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None and t.numel() else C.c_void_p(0)
+
+
+class HipPath:
+    def __init__(self, dim):
+        self.L = _lib.lib()
+        self.dim = dim
+        self.h = self.L.scn_md_create(dim)
+        if not self.h:
+            raise _lib.ScnError(self.L.scn_last_error().decode())
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.L.scn_md_destroy(self.h)
+            self.h = None
+
+    def _s(self, x):
+        return _lib.sizes(self.dim, x) if x is not None else None
+
+    # -- metadata ---------------------------------------------------------
+    def input_layer(self, spatial, coords, batch_size=0, mode=3):
+        coords = np.ascontiguousarray(coords, dtype=np.int64)
+        c = _dev(coords, torch.int64)
+        n = C.c_int64(0)
+        _lib.check(self.L.scn_md_input_layer(self.h, self._s(spatial), _ptr(c), coords.shape[0],
+                                             coords.shape[1], batch_size, mode, _stream(), C.byref(n)))
+        return n.value
+
+    def input_rules(self):
+        hdr = (C.c_int32 * 4)()
+        _lib.check(self.L.scn_md_input_rules_header(self.h, hdr))
+        mode, max_active, n_in, n_out = [int(v) for v in hdr]
+        rows = torch.zeros((n_out, 1 + max_active), dtype=torch.int32, device="cuda")
+        if mode != 0 and n_out:
+            _lib.check(self.L.scn_md_input_rules(self.h, _ptr(rows), _stream()))
+        return np.array(list(hdr), np.int32), rows.cpu().numpy()
+
+    def nactive(self, spatial):
+        n = C.c_int64(0)
+        _lib.check(self.L.scn_md_nactive(self.h, self._s(spatial), C.byref(n)))
+        return n.value
+
+    def batch_size(self, spatial):
+        b = C.c_int(0)
+        _lib.check(self.L.scn_md_batch_size(self.h, self._s(spatial), C.byref(b)))
+        return b.value
+
+    def spatial_locations(self, spatial):
+        n = self.nactive(spatial)
+        out = torch.zeros((n, self.dim + 1), dtype=torch.int64, device="cuda")
+        if n:
+            _lib.check(self.L.scn_md_spatial_locations(self.h, self._s(spatial), _ptr(out), _stream()))
+        return out.cpu().numpy()
+
+    def _rules(self, kind, a, b=None, c=None, d=None):
+        args = [self._s(v) for v in (a, b, c, d)]
+        cnt = C.c_int(0)
+        _lib.check(self.L.scn_rules_count(self.h, kind, *args, _stream(), C.byref(cnt)))
+        sizes = (C.c_int64 * max(1, cnt.value))()
+        _lib.check(self.L.scn_rules_sizes(self.h, kind, *args, _stream(), sizes))
+        out = []
+        for k in range(cnt.value):
+            pairs = torch.zeros((int(sizes[k]), 2), dtype=torch.int32, device="cuda")
+            if sizes[k]:
+                _lib.check(self.L.scn_rules_export(self.h, kind, *args, k, _ptr(pairs), _stream()))
+            out.append(pairs.cpu().numpy())
+        return out
+
+    def submanifold_rules(self, spatial, filter_size):
+        return self._rules(0, spatial, filter_size)
+
+    def strided_rules(self, in_size, out_size, filter_size, stride):
+        return self._rules(1, in_size, out_size, filter_size, stride)
+
+    def s2d_rules(self, spatial):
+        return self._rules(2, spatial)
+
+    # -- forward ops ------------------------------------------------------
+    def _conv(self, fn, sizes, n_rows, x, w, bias):
+        groups = w.shape[1]
+        n_in, n_out = w.shape[2] * groups, w.shape[3] * groups
+        xd, wd = _dev(x, torch.float32), _dev(w, torch.float32)
+        bd = _dev(bias, torch.float32) if bias is not None else None
+        out = torch.full((n_rows, n_out), float("nan"), dtype=torch.float32, device="cuda")
+        macs = C.c_double(0)
+        _lib.check(fn(self.h, *sizes, _ptr(xd), _ptr(out), _ptr(wd), _ptr(bd), n_in, n_out, groups,
+                      _stream(), C.byref(macs)))
+        return out.cpu().numpy(), macs.value
+
+    def subm_conv(self, spatial, filter_size, x, w, bias=None):
+        _lib.check(self.L.scn_md_submanifold_rules(self.h, self._s(spatial), self._s(filter_size),
+                                                   _stream()))
+        return self._conv(self.L.scn_subm_conv_fwd, (self._s(spatial), self._s(filter_size)),
+                          self.nactive(spatial), x, w, bias)
+
+    def conv(self, in_size, out_size, filter_size, stride, x, w, bias=None):
+        sizes = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        _lib.check(self.L.scn_md_strided_rules(self.h, *sizes, _stream()))
+        return self._conv(self.L.scn_conv_fwd, sizes, self.nactive(out_size), x, w, bias)
+
+    def deconv(self, in_size, out_size, filter_size, stride, x, w, bias=None):
+        sizes = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
+        _lib.check(self.L.scn_md_strided_rules(self.h, *rb, _stream()))
+        return self._conv(self.L.scn_deconv_fwd, sizes, self.nactive(out_size), x, w, bias)
+
+    def maxpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
+        sizes = [self._s(v) for v in (in_size, out_size, size, stride)]
+        _lib.check(self.L.scn_md_strided_rules(self.h, *sizes, _stream()))
+        xd = _dev(x, torch.float32)
+        planes = x.shape[1] - n_features_to_drop
+        out = torch.full((self.nactive(out_size), planes), float("nan"), dtype=torch.float32,
+                         device="cuda")
+        _lib.check(self.L.scn_maxpool_fwd(self.h, *sizes, _ptr(xd), x.shape[1], _ptr(out), planes,
+                                          n_features_to_drop, _stream()))
+        return out.cpu().numpy()
+
+    def bn_eval(self, x, mean, var, weight=None, bias=None, eps=1e-4, leakiness=1.0):
+        xd = _dev(x, torch.float32)
+        out = torch.full_like(xd, float("nan"))
+        md, vd = _dev(mean, torch.float32), _dev(var, torch.float32)
+        gd = _dev(weight, torch.float32) if weight is not None else None
+        bd = _dev(bias, torch.float32) if bias is not None else None
+        _lib.check(self.L.scn_bn_eval_fwd(_ptr(xd), _ptr(out), x.shape[0], x.shape[1], x.shape[1],
+                                          x.shape[1], _ptr(md), _ptr(vd), _ptr(gd), _ptr(bd), eps,
+                                          leakiness, _stream()))
+        return out.cpu().numpy()
+
+    def input_fwd(self, x):
+        hdr = self._hdr()
+        xd = _dev(x, torch.float32)
+        out = torch.full((int(hdr[3]), x.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_input_layer_fwd(self.h, _ptr(xd), _ptr(out), x.shape[1], _stream()))
+        return out.cpu().numpy()
+
+    def _hdr(self):
+        hdr = (C.c_int32 * 4)()
+        _lib.check(self.L.scn_md_input_rules_header(self.h, hdr))
+        return [int(v) for v in hdr]
+
+    def output_fwd(self, x):
+        hdr = self._hdr()
+        xd = _dev(x, torch.float32)
+        out = torch.full((hdr[2], x.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_output_layer_fwd(self.h, _ptr(xd), _ptr(out), x.shape[1], _stream()))
+        return out.cpu().numpy()
+
+    def s2d(self, spatial, x):
+        s = [int(v) for v in self._s(spatial)]
+        xd = _dev(x, torch.float32)
+        out = torch.full([self.batch_size(spatial), x.shape[1]] + s, float("nan"), dtype=torch.float32,
+                         device="cuda")
+        _lib.check(self.L.scn_s2d_fwd(self.h, self._s(spatial), _ptr(xd), _ptr(out), x.shape[1],
+                                      _stream()))
+        return out.cpu().numpy()

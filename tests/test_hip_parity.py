@@ -1,0 +1,122 @@
+"""Parity of the HIP library, called through its C ABI, with the independent statements of
+tests/checks.py, with the golden fixtures written by the compiled reference, and with the
+CPU oracle on the same seeded inputs.  Rulebooks bit-exact as canonically sorted
+(offset, in-site, out-site) sets; features within 1e-4 relative / 1e-5 absolute (fp32)."""
+import numpy as np
+import pytest
+
+import checks
+from oracle import cpu_path
+from oracle.cpu_path import canon_rows, canon_rules
+from sparseconvnet_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def make():
+    import torch
+    assert torch.cuda.is_available()
+    from hip_path import HipPath
+    return lambda dim: HipPath(dim)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dim", [2, 3])
+def test_input_layer(make, dim, mode):
+    checks.check_input_layer(make, dim, mode, seed=10 * dim + mode)
+
+
+def test_input_layer_no_batch_column(make):
+    checks.check_input_layer(make, 3, 4, seed=5, with_batch_col=False)
+    checks.check_input_layer(make, 2, 0, seed=6, with_batch_col=False)
+
+
+@pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (2, (3, 1)), (3, (1, 3, 5)), (3, 2),
+                                      (4, 3)])
+def test_submanifold(make, dim, size):
+    checks.check_submanifold(make, dim, size, seed=7 + dim, spatial=8 if dim < 4 else 5,
+                             n=200 if dim < 4 else 250, bias=(dim == 2))
+
+
+@pytest.mark.parametrize("dim,size,stride", [(3, 2, 2), (3, 3, 2), (2, 3, 2), (2, 2, 2), (1, 3, 2),
+                                             (2, (3, 2), (2, 1)), (3, 4, 2), (2, 2, 3), (3, 3, 1)])
+def test_strided(make, dim, size, stride):
+    checks.check_strided(make, dim, size, stride, seed=3 + dim, bias=(dim == 2))
+
+
+def test_bn(make):
+    checks.check_bn(make, seed=1)
+    checks.check_bn(make, seed=2, n=1000, C=32)
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3])
+def test_s2d(make, dim):
+    checks.check_s2d(make, dim, seed=2 + dim)
+
+
+def test_empty(make):
+    checks.check_empty(make)
+
+
+def test_golden(make, tmp_path):
+    from test_golden import compare_with_golden, make_golden
+    for name in sorted(make_golden.FIXTURES):
+        compare_with_golden(name, make, tmp_path)
+
+
+def _both(dim, oracle_built):
+    from hip_path import HipPath
+    return HipPath(dim), cpu_path.CpuPath(dim, "oracle")
+
+
+@pytest.mark.parametrize("cin,cout,groups", [(16, 16, 1), (3, 32, 1), (8, 12, 2), (32, 32, 1), (64, 64, 1)])
+def test_config1_vs_oracle(oracle_built, cin, cout, groups):
+    """Configuration 1 (batch 2, 128^3, ~40k sites per sample, 3^3 submanifold convolution)."""
+    g, o = _both(3, oracle_built)
+    coords = synthetic.config1()
+    rng = np.random.default_rng(1)
+    x = rng.normal(size=(len(coords), cin)).astype(np.float32)
+    w = (rng.normal(size=(27, groups, cin // groups, cout // groups)) * (2.0 / (cin * 27)) ** 0.5).astype(
+        np.float32)
+    for p in (g, o):
+        assert p.input_layer(128, coords, 0, 0) == len(coords)
+    lg, lo = g.spatial_locations(128), o.spatial_locations(128)
+    assert (lg == lo).all() and (lg == coords).all()
+    rg, ro = g.submanifold_rules(128, 3), o.submanifold_rules(128, 3)
+    assert (canon_rules(rg, lg, lg) == canon_rules(ro, lo, lo)).all()
+    yg, mg = g.subm_conv(128, 3, x, w)
+    yo, mo = o.subm_conv(128, 3, x, w)
+    assert mg == mo
+    checks.assert_close(yg, yo, "config 1 conv")
+
+
+def test_strided_tree_vs_oracle(oracle_built):
+    """Configuration 4's tree at 254^3 with 60k points, duplicates merged by mode 4."""
+    g, o = _both(3, oracle_built)
+    coords = synthetic.room_scene(seed=4000, target=60000, spatial=254, duplicate_fraction=0.3)
+    rng = np.random.default_rng(4)
+    f = rng.uniform(-1, 1, size=(len(coords), 32)).astype(np.float32)
+    w1 = (rng.normal(size=(8, 1, 32, 64)) * 0.1).astype(np.float32)
+    w2 = (rng.normal(size=(8, 1, 64, 32)) * 0.1).astype(np.float32)
+    res = []
+    for p in (g, o):
+        p.input_layer(254, coords, 0, 4)
+        l0 = p.spatial_locations(254)
+        x = p.input_fwd(f)
+        r1 = p.strided_rules(254, 127, 2, 2)
+        l1 = p.spatial_locations(127)
+        h, m1 = p.conv(254, 127, 2, 2, x, w1)
+        r2 = p.strided_rules(127, 63, 3, 2)
+        l2 = p.spatial_locations(63)
+        mp = p.maxpool(127, 63, 3, 2, h)
+        u, m2 = p.deconv(127, 254, 2, 2, h, w2)
+        res.append(dict(l0=l0, x=x, r1=canon_rules(r1, l0, l1), l1=l1[canon_rows(l1)], h=h[canon_rows(l1)],
+                        m1=m1, r2=canon_rules(r2, l1, l2), mp=mp[canon_rows(l2)], u=u, m2=m2,
+                        back=p.output_fwd(u)))
+    a, b = res
+    for k in ("l0", "r1", "l1", "r2"):
+        assert a[k].shape == b[k].shape and (a[k] == b[k]).all(), k
+    assert a["m1"] == b["m1"] and a["m2"] == b["m2"]
+    for k in ("x", "h", "mp", "u", "back"):
+        checks.assert_close(a[k], b[k], k)
