@@ -1,0 +1,202 @@
+"""Benchmark of the sparse-convolution forward path on one MI355X.
+
+Default workload ("sweep"): the single-layer configuration at scene scale - one synthetic
+room of 1,000,000 active voxels in a 4096^3 grid, SubmanifoldConvolution 3^3, fp32, for
+(nIn, nOut) in {(3,32), (32,32), (64,64), (128,128), (256,256)}.  One step = one forward of
+each of the five convolutions with the rulebook already built (its build time is reported
+separately as `rulebook_ms`).  `value` = sum of 2*MACs / sum of time, in GFLOP/s, with MACs
+counted as the reference counts them (sum over filter taps of rules * nIn * nOut).
+
+Prints ONE JSON line.  `roofline` describes the kernel that takes the largest share of the
+step; `sweep` lists every channel pair with its own roofline; `cpu_baseline` times the
+reference's CPU path (oracle/_ref, else the oracle port) on a bounded sample."""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+MFMA_FP32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PAIRS = [(3, 32), (32, 32), (64, 64), (128, 128), (256, 256)]
+
+
+def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
+    """Algorithmic bytes of one convolution forward: gathered input rows + int32 rule pairs +
+    output written once + weights once."""
+    return R * cin * s + 8 * R + n_out_rows * cout * s + K * cin * cout * s
+
+
+def roofline_for(cin, cout, R, n, K, ms):
+    flops = 2.0 * R * cin * cout
+    byts = conv_bytes(R, n, K, cin, cout)
+    t_mfma = flops / (MFMA_FP32_TFLOPS * 1e12)
+    t_hbm = byts / (HBM_PEAK_GBS * 1e9)
+    if t_mfma >= t_hbm:
+        ach = flops / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_FP32_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach / MFMA_FP32_TFLOPS, 4), "traffic": None}
+    ach = byts / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
+
+
+def cpu_baseline(sample_sites, seed):
+    """Reference CPU path (compiled reference if oracle/_ref is there, else the oracle port) on
+    a smaller scene of the same generator: the same five convolutions, once each."""
+    from oracle import cpu_path
+    from sparseconvnet_amd import synthetic
+    kind = "reference" if cpu_path.available("ref") else "port"
+    flavour = "ref" if kind == "reference" else "oracle"
+    if flavour == "oracle" and not cpu_path.available("oracle"):
+        return None
+    coords = synthetic.room_scene(seed=seed, target=sample_sites, spatial=4096)
+    p = cpu_path.CpuPath(3, flavour)
+    p.input_layer(4096, coords, 0, 0)
+    t0 = time.time()
+    rules = p.submanifold_rules(4096, 3)
+    t_rules = time.time() - t0
+    R = sum(len(r) for r in rules)
+    rng = np.random.default_rng(0)
+    flops = 0.0
+    secs = 0.0
+    for cin, cout in PAIRS:
+        x = rng.normal(size=(len(coords), cin)).astype(np.float32)
+        w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
+        t0 = time.time()
+        _, macs = p.subm_conv(4096, 3, x, w)
+        secs += time.time() - t0
+        flops += 2.0 * macs
+    try:
+        import torch
+        cores = torch.get_num_threads() if kind == "reference" else int(os.environ.get("OMP_NUM_THREADS", os.cpu_count()))
+    except Exception:
+        cores = os.cpu_count()
+    return {"value": round(flops / secs / 1e9, 2), "unit": "GFLOP/s", "cores": int(cores), "kind": kind,
+            "sample": "same sweep of 5 SubmanifoldConvolution 3^3 forwards, once each, on a %d-site room "
+                      "scene (%d rules); rulebook build %.2f s single-threaded, not included"
+                      % (len(coords), R, t_rules)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--sites", type=int, default=1000000)
+    ap.add_argument("--seed", type=int, default=3000)
+    ap.add_argument("--order", default="shuffled", choices=["shuffled", "scan"])
+    ap.add_argument("--cpu-sites", type=int, default=200000)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--pairs", default="")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from sparseconvnet_amd import _lib, synthetic
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    L = _lib.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    pairs = PAIRS if not args.pairs else [tuple(int(v) for v in p.split("x")) for p in args.pairs.split(",")]
+
+    coords = synthetic.room_scene(seed=args.seed, target=args.sites, spatial=4096, order=args.order)
+    cd = torch.as_tensor(coords).cuda()
+    sp, fs = _lib.sizes(3, 4096), _lib.sizes(3, 3)
+
+    def build():
+        h = L.scn_md_create(3)
+        n = C.c_int64(0)
+        _lib.check(L.scn_md_input_layer(h, sp, C.c_void_p(cd.data_ptr()), len(coords), 4, 0, 0, stream,
+                                        C.byref(n)))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _lib.check(L.scn_md_submanifold_rules(h, sp, fs, stream))
+        torch.cuda.synchronize()
+        return h, int(n.value), (time.perf_counter() - t0) * 1e3
+
+    rb_ms = []
+    for _ in range(4):
+        h, n, ms = build()
+        rb_ms.append(ms)
+        L.scn_md_destroy(h)
+    h, n, ms = build()
+    rb_ms.append(ms)
+    rulebook_ms = float(np.median(rb_ms[1:]))
+    sizes = (C.c_int64 * 27)()
+    _lib.check(L.scn_rules_sizes(h, 0, sp, fs, None, None, stream, sizes))
+    R = int(sum(sizes))
+
+    g = torch.Generator(device="cuda").manual_seed(0)
+    work = []
+    for cin, cout in pairs:
+        x = torch.randn((n, cin), device="cuda", generator=g)
+        w = torch.randn((27, 1, cin, cout), device="cuda", generator=g) * (2.0 / (cin * 27)) ** 0.5
+        y = torch.empty((n, cout), device="cuda")
+        work.append((cin, cout, x, w, y))
+
+    macs = C.c_double(0)
+
+    def conv(cin, cout, x, w, y):
+        _lib.check(L.scn_subm_conv_fwd(h, sp, fs, C.c_void_p(x.data_ptr()), C.c_void_p(y.data_ptr()),
+                                       C.c_void_p(w.data_ptr()), None, cin, cout, 1, stream, C.byref(macs)))
+
+    for _ in range(args.warmup):
+        for wk in work:
+            conv(*wk)
+    torch.cuda.synchronize()
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in work]
+          for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        for i, wk in enumerate(work):
+            ev[s][i][0].record()
+            conv(*wk)
+            ev[s][i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    per_pair_ms = [float(np.mean([ev[s][i][0].elapsed_time(ev[s][i][1]) for s in range(args.steps)]))
+                   for i in range(len(work))]
+    total_flops = sum(2.0 * R * cin * cout for cin, cout in pairs)
+    value = total_flops / (ms_per_step * 1e-3) / 1e9
+
+    sweep = []
+    for (cin, cout), ms in zip(pairs, per_pair_ms):
+        sweep.append({"nIn": cin, "nOut": cout, "ms": round(ms, 4),
+                      "gflops": round(2.0 * R * cin * cout / (ms * 1e-3) / 1e9, 1),
+                      "sites_per_s": round(n / (ms * 1e-3)),
+                      "roofline": roofline_for(cin, cout, R, n, 27, ms)})
+    dom = int(np.argmax(per_pair_ms))
+    roof = dict(sweep[dom]["roofline"])
+    roof["kernel"] = "submanifold conv %d->%d" % pairs[dom]
+
+    out = {
+        "metric": "SubmanifoldConv GFLOP/s & % roofline; 3D U-Net ms/scene at 1 GPU",
+        "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[2]: 3D single-layer sweep, SubmanifoldConvolution 3^3 on one "
+                               "%d-voxel room scene in 4096^3 (%s point order), (nIn,nOut) in %s, "
+                               "rulebook warm" % (n, args.order, pairs),
+                   "active_sites": n, "rules": R},
+        "rulebook_ms": round(rulebook_ms, 3),
+        "rulebook_sites_per_s": round(n / (rulebook_ms * 1e-3)),
+        "roofline": roof, "sweep": sweep,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sites, args.seed)
+    L.scn_md_destroy(h)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -177,7 +177,7 @@ int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *fi
     Metadata &m = md(h);
     Table &t = submanifold_rules(m, spatial, filter, st(stream));
     Level *l = find_level(m, spatial);
-    conv_forward(t, l ? l->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
+    conv_forward(m, t, l ? l->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
     // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
     if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
   });
@@ -188,7 +188,7 @@ int scn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_siz
   return guarded([&] {
     Metadata &m = md(h);
     StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
-    conv_forward(r.by_out, nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
+    conv_forward(m, r.by_out, nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
     if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
   });
 }
@@ -200,7 +200,7 @@ int scn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
     // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
     StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
     Level *fine = find_level(m, out_size);
-    conv_forward(r.by_in, fine ? fine->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups,
+    conv_forward(m, r.by_in, fine ? fine->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups,
                  st(stream));
     if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
   });

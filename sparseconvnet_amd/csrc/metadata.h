@@ -72,6 +72,7 @@ struct Metadata {
   DevBuf<int> v0, v1, f0, f1, s0, s1;
   DevBuf<long long> dcounts;
   DevBuf<int> dflags;
+  DevBuf<float> wpack;  // weights of the running convolution in MFMA operand order
 };
 
 SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);
@@ -93,7 +94,7 @@ int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *p
 
 // ops.hip / conv.hip
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);
-void conv_forward(const Table &t, const int *rowmap, const float *in, float *out, const float *w,
+void conv_forward(Metadata &m, const Table &t, const int *rowmap, const float *in, float *out, const float *w,
                   const float *bias, int n_in, int n_out, int groups, hipStream_t s);
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
                      int drop, hipStream_t s);
