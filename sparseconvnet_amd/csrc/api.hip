@@ -151,11 +151,10 @@ int scn_rules_export(scn_metadata *h, int kind, const int64_t *a, const int64_t 
     Metadata &m = md(h);
     if (kind == 0) {
       Table &t = submanifold_rules(m, a, b, st(stream));
-      Level *l = find_level(m, a);
-      export_table_pairs(m, t, l ? l->sched_ptr() : nullptr, k, false, pairs, st(stream));
+      export_table_pairs(m, t, k, false, pairs, st(stream));
     } else if (kind == 1) {
       StridedRules &r = strided_rules(m, a, b, c, d, st(stream));
-      export_table_pairs(m, r.by_out, nullptr, k, false, pairs, st(stream));
+      export_table_pairs(m, r.by_out, k, false, pairs, st(stream));
     } else if (kind == 2) {
       export_s2d_pairs(m, a, k, pairs, st(stream));
     } else
@@ -176,8 +175,7 @@ int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *fi
   return guarded([&] {
     Metadata &m = md(h);
     Table &t = submanifold_rules(m, spatial, filter, st(stream));
-    Level *l = find_level(m, spatial);
-    conv_forward(m, t, l ? l->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
+    conv_forward(m, t, in, out, weight, bias, n_in, n_out, groups, st(stream));
     // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
     if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
   });
@@ -188,7 +186,7 @@ int scn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_siz
   return guarded([&] {
     Metadata &m = md(h);
     StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
-    conv_forward(m, r.by_out, nullptr, in, out, weight, bias, n_in, n_out, groups, st(stream));
+    conv_forward(m, r.by_out, in, out, weight, bias, n_in, n_out, groups, st(stream));
     if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
   });
 }
@@ -199,9 +197,7 @@ int scn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
     Metadata &m = md(h);
     // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
     StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
-    Level *fine = find_level(m, out_size);
-    conv_forward(m, r.by_in, fine ? fine->sched_ptr() : nullptr, in, out, weight, bias, n_in, n_out, groups,
-                 st(stream));
+    conv_forward(m, r.by_in, in, out, weight, bias, n_in, n_out, groups, st(stream));
     if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
   });
 }

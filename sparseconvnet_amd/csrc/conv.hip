@@ -5,15 +5,11 @@
 // (CPU/Convolution.cpp:45-79,117-150, CPU/Deconvolution.cpp:7-41); they differ only in
 // the table they pass.
 //
-// MFMA kernel (groups == 1).  A workgroup owns WAVES*16 consecutive schedule positions;
-// each wavefront owns a granule of 16 of them and keeps that granule's [16 x nOut]
-// accumulators in registers for the whole filter.  Per tap the wavefront gathers its 16
-// input rows straight from HBM/L2 into v_mfma_f32_16x16x4_f32 A-operand registers (16-byte
-// loads; the reduction dimension is consumed in a lane-permuted order that the packed
-// weights mirror), multiplies with the tap's weight slab that the workgroup has staged in
-// LDS in B-operand order, and skips the tap altogether when none of its 16 rows has that
-// neighbour.  Rows arrive in Z-order, so a granule's rows mostly share one neighbour
-// pattern and the skipped taps carry almost all of the sparsity.
+// MFMA kernel (groups == 1): fp32 v_mfma_f32_16x16x4_f32, accumulators in registers for the
+// whole filter, gathered rows and packed weights staged through double-buffered LDS, taps
+// skipped per 16-row granule.  Positions arrive in Z-order and pattern-sorted, so a
+// granule's rows mostly share one neighbour pattern and the skipped (granule, tap) pairs
+// carry almost all of the sparsity.
 #include "metadata.h"
 
 namespace scn {
@@ -46,163 +42,304 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
 }
 
 // ---- weight packing ---------------------------------------------------------------------
-// wp[k][slab][s][cb][lane][jj] = W[k][channel (slab*SS+s)*16 + 4*(lane/16) + jj][16*cb + lane%16]
-// (zero outside [nIn) x [nOut)): the order in which lane `lane` of a wavefront consumes B
-// operands, so that staging a slab into LDS is a straight copy and each lane reads the four
-// operands of one 16-channel step with a single 16-byte LDS load.
+// wp[k][slab][e], e < SLAB_STRIDE (floats), with for e = ((s*NCB + cb)*64 + lane)*4 + jj
+//   wp = W[k][channel (slab*SS+s)*16 + 4*(lane/16) + jj][16*cb + lane%16]
+// (zero outside [nIn) x [nOut) and in the padding up to SLAB_STRIDE): the order in which
+// lane `lane` of a wavefront consumes B operands, so that staging a slab into LDS is a
+// straight copy and each lane reads the four operands of one 16-channel step with a single
+// 16-byte LDS load.
 __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n_out, int n_slab, int SS,
-                               int NCB) {
+                               int NCB, int slab_stride) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = (int64_t)K * n_slab * SS * NCB * 256;
+  int64_t total = (int64_t)K * n_slab * slab_stride;
   if (i >= total) return;
-  int jj = (int)(i & 3);
-  int lane = (int)((i >> 2) & 63);
-  int64_t r = i >> 8;
-  int cb = (int)(r % NCB);
-  r /= NCB;
-  int s = (int)(r % SS);
-  r /= SS;
+  int e = (int)(i % slab_stride);
+  int64_t r = i / slab_stride;
   int sl = (int)(r % n_slab);
   int k = (int)(r / n_slab);
-  int ch = (sl * SS + s) * 16 + 4 * (lane >> 4) + jj;
-  int col = 16 * cb + (lane & 15);
-  wp[i] = (ch < n_in && col < n_out) ? w[((int64_t)k * n_in + ch) * n_out + col] : 0.0f;
+  float v = 0.0f;
+  if (e < SS * NCB * 256) {
+    int jj = e & 3;
+    int lane = (e >> 2) & 63;
+    int q = e >> 8;
+    int cb = q % NCB;
+    int s = q / NCB;
+    int ch = (sl * SS + s) * 16 + 4 * (lane >> 4) + jj;
+    int col = 16 * cb + (lane & 15);
+    if (ch < n_in && col < n_out) v = w[((int64_t)k * n_in + ch) * n_out + col];
+  }
+  wp[i] = v;
 }
 
 // ---- MFMA kernel ------------------------------------------------------------------------
-template <int NCB, bool VEC4, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void k_conv_mfma(
+// A workgroup of 4 wavefronts owns a tile of G = GW*WR granules (16 rows each).  The
+// wavefronts form a WR x WC grid: wavefront (wr, wc) keeps, in registers, the accumulators
+// of granules [wr*GW, (wr+1)*GW) x column blocks [wc*NCBW, (wc+1)*NCBW) (16 columns each).
+// With WC = 4 every wavefront works on every granule, so the MFMA work of a tap is split
+// evenly whatever the neighbour pattern of the rows.
+//
+// Per (tap, slab of SS*16 input channels) iteration, for the granules that have the tap:
+//   gathered input rows  HBM/L2 -> registers -> LDS, in A-operand order
+//   the weight slab      HBM/L2 -> registers -> LDS, in B-operand order (see k_pack_weights)
+//   MFMAs out of LDS into the accumulators
+// as a software pipeline with one barrier per iteration: iteration it+1's loads are in
+// flight while iteration it computes; both LDS areas are double-buffered.  Every global
+// load of the pipeline is unconditional (granules without the tap and absent rows read
+// row 0 and are zeroed by a select), so the count of loads in flight is a compile-time
+// constant and the compiler can wait for exactly the loads it needs.
+template <int NCBW, int WC, int GW, int SS, bool VEC4>
+__global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
-    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int SS, int tiles_per_xcd,
-    int n_tiles) {
+    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles) {
+  constexpr int WR = 4 / WC;
+  constexpr int NCB = NCBW * WC;
+  constexpr int G = GW * WR;
+  constexpr int TM = G * 16;
+  constexpr int SLAB_F4 = SS * NCB * 64;      // float4 of one weight slab
+  constexpr int WPT = (SLAB_F4 + 255) / 256;  // float4 staged per thread
+  constexpr int SLAB_STRIDE_F4 = WPT * 256;   // padded slab, in global memory and LDS
+  constexpr int NFRAG = G * SS;               // A fragments (granule, step) per iteration
+  constexpr int FPW = NFRAG / 4;              // fragments gathered per wavefront
+  static_assert(NFRAG % 4 == 0, "fragments must divide over 4 wavefronts");
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int TM = WAVES * 16;
-  int *tapflag = reinterpret_cast<int *>(lds + (size_t)SS * NCB * 256);  // [K]
+  v4f *wbuf = reinterpret_cast<v4f *>(lds);   // [2][SLAB_STRIDE_F4]
+  v4f *abuf = wbuf + 2 * SLAB_STRIDE_F4;      // [2][NFRAG * 64]
+  int *jtab = reinterpret_cast<int *>(abuf + 2 * NFRAG * 64);  // [G][K][16]
+  unsigned *gmask = reinterpret_cast<unsigned *>(jtab + G * K * 16);  // [K] granules having tap k
+  int *taplist = reinterpret_cast<int *>(gmask + K);           // [K]
+  int *ntaps_p = taplist + K;                                  // [1]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
+  const int wr = wave / WC, wc = wave % WC;
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of
   // tiles so that neighbouring tiles (which gather the same rows) share one L2.
   const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
   if (tile >= n_tiles) return;  // whole workgroup leaves: no barrier is skipped
-  const int64_t t0 = (int64_t)tile * TM + wave * 16;
-  const int64_t t = t0 + r16;
-  const bool live = t < n;
+  const int64_t tbase = (int64_t)tile * TM;
 
-  for (int k = threadIdx.x; k < K; k += WAVES * 64) tapflag[k] = 0;
+  for (int k = threadIdx.x; k < K; k += 256) gmask[k] = 0u;
   __syncthreads();
-  for (int k = 0; k < K; k++) {
-    int j = live ? nbr[(int64_t)k * npad + t] : -1;
-    if (__ballot(j >= 0) != 0ull && lane == 0) tapflag[k] = 1;
+  // Neighbour rows of the tile -> LDS, four taps per pass (one per 16-lane group).
+  for (int gr = wave; gr < G; gr += 4) {
+    const int64_t t = tbase + gr * 16 + r16;
+    for (int kb = 0; kb < K; kb += 4) {
+      const int k = kb + g;
+      int j = -1;
+      if (k < K && t < n) j = nbr[(int64_t)k * npad + t];
+      if (k < K) jtab[(gr * K + k) * 16 + r16] = j;
+      const unsigned long long bal = __ballot(j >= 0);
+      if (lane == 0) {
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++)
+          if ((bal >> (16 * gg)) & 0xFFFFull) atomicOr(&gmask[kb + gg], 1u << gr);
+      }
+    }
   }
   __syncthreads();
+  if (threadIdx.x == 0) {
+    int c = 0;
+    for (int k = 0; k < K; k++)
+      if (gmask[k]) taplist[c++] = k;
+    *ntaps_p = c;
+  }
+  __syncthreads();
+  const int total = *ntaps_p * n_slab;
 
-  v4f acc[NCB];
+  v4f acc[GW][NCBW];
 #pragma unroll
-  for (int cb = 0; cb < NCB; cb++) acc[cb] = (v4f){0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < GW; q++)
+#pragma unroll
+    for (int c = 0; c < NCBW; c++) acc[q][c] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  const int slab_f4 = SS * NCB * 64;  // float4 per slab
-  for (int k = 0; k < K; k++) {
-    if (!tapflag[k]) continue;  // uniform over the workgroup
-    const int j = live ? nbr[(int64_t)k * npad + t] : -1;
-    const bool wave_has = __ballot(j >= 0) != 0ull;
-    const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
-    for (int sl = 0; sl < n_slab; sl++) {
-      __syncthreads();  // everyone is done with the previous slab
-      const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * slab_f4;
-      for (int e = threadIdx.x; e < slab_f4; e += WAVES * 64) reinterpret_cast<v4f *>(lds)[e] = wsrc[e];
-      __syncthreads();
-      if (!wave_has) continue;  // uniform over the wavefront
+  v4f wreg[WPT];
+  v4f areg[FPW];
+  unsigned gm_nxt = 0, gm_cur = 0;  // granule mask of the tap (uniform)
+  unsigned aok_nxt = 0;             // bit i: this lane's row of fragment i exists
+  int sl_nxt = 0;
+
+  // Issue the loads of iteration `it`: its weight slab into wreg; this wavefront's share of
+  // the A fragments (granule, step) into areg.
+  auto issue = [&](int it) {
+    const int ti = it / n_slab, sl = it - ti * n_slab;
+    const int k = taplist[ti];
+    const unsigned gm = gmask[k];
+    gm_nxt = gm;
+    sl_nxt = sl;
+    aok_nxt = 0;
+    const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
+#pragma unroll
+    for (int i = 0; i < WPT; i++) wreg[i] = wsrc[threadIdx.x + i * 256];
+#pragma unroll
+    for (int i = 0; i < FPW; i++) {
+      const int f = wave + 4 * i;  // fragment f = (granule f / SS, step f % SS)
+      const int gr = f / SS, s = f % SS;
+      const int j = jtab[(gr * K + k) * 16 + r16];
+      if (j >= 0) aok_nxt |= 1u << i;
+      const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
+      const int c0 = (sl * SS + s) * 16 + 4 * g;
+      v4f v;
+      if (VEC4) {
+        const int cc = c0 < n_in ? c0 : n_in - 4;
+        v = *reinterpret_cast<const v4f *>(src + cc);
+      } else {
+        v.x = src[min(c0 + 0, n_in - 1)];
+        v.y = src[min(c0 + 1, n_in - 1)];
+        v.z = src[min(c0 + 2, n_in - 1)];
+        v.w = src[min(c0 + 3, n_in - 1)];
+      }
+      areg[i] = v;
+    }
+  };
+
+  if (total > 0) issue(0);
+  for (int it = 0; it < total; it++) {
+    v4f *wb = wbuf + (it & 1) * SLAB_STRIDE_F4;
+    v4f *ab = abuf + (it & 1) * (NFRAG * 64);
+#pragma unroll
+    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * 256] = wreg[i];
+    // Absent rows and channels past nIn become zeros on their way into LDS.
+#pragma unroll
+    for (int i = 0; i < FPW; i++) {
+      const int f = wave + 4 * i;
+      const int c0 = (sl_nxt * SS + f % SS) * 16 + 4 * g;
+      const bool ok = (aok_nxt >> i) & 1u;
+      v4f v = areg[i];
+      if (VEC4) {
+        if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
+      } else {
+        if (!(ok && c0 + 0 < n_in)) v.x = 0.f;
+        if (!(ok && c0 + 1 < n_in)) v.y = 0.f;
+        if (!(ok && c0 + 2 < n_in)) v.z = 0.f;
+        if (!(ok && c0 + 3 < n_in)) v.w = 0.f;
+      }
+      ab[f * 64 + lane] = v;
+    }
+    gm_cur = gm_nxt;
+    // After this barrier the buffers of `it` are visible, and every wavefront has finished
+    // the MFMAs of it-1, so the other buffers may be overwritten at the top of it+1.
+    __syncthreads();
+    if (it + 1 < total) issue(it + 1);
+
+    v4f b[SS][NCBW];
+#pragma unroll
+    for (int s = 0; s < SS; s++)
+#pragma unroll
+      for (int c = 0; c < NCBW; c++) b[s][c] = wb[(s * NCB + wc * NCBW + c) * 64 + lane];
+#pragma unroll
+    for (int q = 0; q < GW; q++) {
+      const int gr = wr * GW + q;
+      if (!((gm_cur >> gr) & 1u)) continue;  // uniform over the workgroup
+#pragma unroll
       for (int s = 0; s < SS; s++) {
-        const int c0 = (sl * SS + s) * 16 + 4 * g;
-        v4f a = (v4f){0.f, 0.f, 0.f, 0.f};
-        if (j >= 0) {
-          if (VEC4) {
-            if (c0 < n_in) a = *reinterpret_cast<const v4f *>(src + c0);
-          } else {
-            if (c0 + 0 < n_in) a.x = src[c0 + 0];
-            if (c0 + 1 < n_in) a.y = src[c0 + 1];
-            if (c0 + 2 < n_in) a.z = src[c0 + 2];
-            if (c0 + 3 < n_in) a.w = src[c0 + 3];
-          }
-        }
+        const v4f av = ab[(gr * SS + s) * 64 + lane];
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) {
-          const v4f b = reinterpret_cast<const v4f *>(lds)[(s * NCB + cb) * 64 + lane];
-          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc[cb], 0, 0, 0);
-          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc[cb], 0, 0, 0);
-          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc[cb], 0, 0, 0);
-          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc[cb], 0, 0, 0);
-        }
+        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][c].x, acc[q][c], 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][c].y, acc[q][c], 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][c].z, acc[q][c], 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][c].w, acc[q][c], 0, 0, 0);
       }
     }
   }
 
-  // acc[cb][r] = result for local row 4*g + r, column 16*cb + r16
+  // acc[q][c][r] = result for position tbase + 16*(wr*GW+q) + 4*g + r, column 16*(wc*NCBW+c) + r16
+  float bv[NCBW];
 #pragma unroll
-  for (int r = 0; r < 4; r++) {
-    const int64_t pos = t0 + 4 * g + r;
-    if (pos >= n) continue;
-    const int64_t row = rowmap ? rowmap[pos] : pos;
-    float *o = out + row * n_out;
+  for (int c = 0; c < NCBW; c++) {
+    const int col = 16 * (wc * NCBW + c) + r16;
+    bv[c] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+  }
 #pragma unroll
-    for (int cb = 0; cb < NCB; cb++) {
-      const int col = 16 * cb + r16;
-      if (col < n_out) o[col] = acc[cb][r] + (bias ? bias[col] : 0.0f);
+  for (int q = 0; q < GW; q++) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int64_t pos = tbase + (wr * GW + q) * 16 + 4 * g + r;
+      if (pos >= n) continue;
+      const int64_t row = rowmap ? rowmap[pos] : pos;
+      float *o = out + row * n_out;
+#pragma unroll
+      for (int c = 0; c < NCBW; c++) {
+        const int col = 16 * (wc * NCBW + c) + r16;
+        if (col < n_out) o[col] = acc[q][c][r] + bv[c];
+      }
     }
   }
 }
 
-template <int NCB, bool VEC4>
-static void launch_mfma(Metadata &m, const Table &t, const int *rowmap, const float *in, float *out,
-                        const float *w, const float *bias, int n_in, int n_out, hipStream_t s) {
-  constexpr int WAVES = 4;
+template <int NCBW, int WC, int GW, int SS, bool VEC4>
+static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                        const float *bias, int n_in, int n_out, hipStream_t s) {
+  constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
+  constexpr int WPT = (SS * NCB * 64 + 255) / 256;
+  constexpr int SLAB_STRIDE = WPT * 256 * 4;  // floats
+  const size_t lds_bytes = (size_t)2 * SLAB_STRIDE * sizeof(float) + (size_t)2 * G * SS * 64 * 16 +
+                           ((size_t)G * t.K * 16 + 2 * t.K + 4) * sizeof(int);
+  if (lds_bytes > 160 * 1024) return false;
   const int cin16 = (int)ceil_div(n_in, 16);
-  int SS = std::max(1, std::min(cin16, 32 / NCB));
-  SS = std::min(SS, 8);
   const int n_slab = (int)ceil_div(cin16, SS);
-  const int64_t packed = (int64_t)t.K * n_slab * SS * NCB * 256;
+  const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
   m.wpack.reserve(packed);
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB);
+                                                                      SS, NCB, SLAB_STRIDE);
   LAUNCH_CHECK();
-  const int n_tiles = (int)ceil_div(t.n, WAVES * 16);
+  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  160 * 1024));
+    attr_set = true;
+  }
+  const int n_tiles = (int)ceil_div(t.n, G * 16);
   const int tiles_per_xcd = (int)ceil_div(n_tiles, 8);
-  const size_t lds_bytes = (size_t)SS * NCB * 256 * sizeof(float) + (size_t)t.K * sizeof(int);
-  k_conv_mfma<NCB, VEC4, WAVES><<<dim3((unsigned)(tiles_per_xcd * 8)), WAVES * 64, lds_bytes, s>>>(
-      t.nbr.p, rowmap, t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, SS, tiles_per_xcd,
-      n_tiles);
+  kern<<<dim3((unsigned)(tiles_per_xcd * 8)), 256, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in,
+                                                                   out, m.wpack.p, bias, n_in, n_out, n_slab,
+                                                                   tiles_per_xcd, n_tiles);
   LAUNCH_CHECK();
+  return true;
 }
 
+// Picks the instantiation from the number of 16-column blocks of the output.  Tiles are 8
+// granules (128 rows); registers and LDS are sized so that two workgroups share a CU and one
+// hides the other's staging.  A slab is one 16-channel step when nIn <= 16 or nOut > 128.
 template <bool VEC4>
-static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const int *rowmap, const float *in, float *out,
-                         const float *w, const float *bias, int n_in, int n_out, hipStream_t s) {
-#define SCN_CASE(N)                                                              \
-  if (ncb <= N) {                                                                \
-    launch_mfma<N, VEC4>(m, t, rowmap, in, out, w, bias, n_in, n_out, s);        \
-    return true;                                                                 \
-  }
-  SCN_CASE(1) SCN_CASE(2) SCN_CASE(4) SCN_CASE(6) SCN_CASE(8) SCN_CASE(10) SCN_CASE(12) SCN_CASE(14) SCN_CASE(16)
+static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                         const float *bias, int n_in, int n_out, hipStream_t s) {
+  const bool narrow = n_in <= 16;
+#define SCN_CASE(N, NCBW, WC, GW, SSW)                                                                 \
+  if (ncb <= N)                                                                                        \
+    return narrow ? launch_mfma<NCBW, WC, GW, 1, VEC4>(m, t, in, out, w, bias, n_in, n_out, s)         \
+                  : launch_mfma<NCBW, WC, GW, SSW, VEC4>(m, t, in, out, w, bias, n_in, n_out, s);
+  SCN_CASE(1, 1, 1, 2, 2)
+  SCN_CASE(2, 1, 2, 4, 2)
+  SCN_CASE(4, 1, 4, 8, 2)
+  SCN_CASE(6, 3, 2, 4, 2)
+  SCN_CASE(8, 2, 4, 8, 2)
+  SCN_CASE(10, 5, 2, 4, 1)
+  SCN_CASE(12, 3, 4, 8, 1)
+  SCN_CASE(14, 7, 2, 4, 1)
+  SCN_CASE(16, 4, 4, 8, 1)
 #undef SCN_CASE
   return false;
 }
 
-void conv_forward(Metadata &m, const Table &t, const int *rowmap, const float *in, float *out, const float *w,
-                  const float *bias, int n_in, int n_out, int groups, hipStream_t s) {
+void conv_forward(Metadata &m, const Table &t, const float *in, float *out, const float *w, const float *bias,
+                  int n_in, int n_out, int groups, hipStream_t s) {
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
   if (groups == 1 && t.K <= 1024) {
     const int ncb = (int)ceil_div(n_out, 16);
     const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
-    bool done = vec4 ? dispatch_ncb<true>(ncb, m, t, rowmap, in, out, w, bias, n_in, n_out, s)
-                     : dispatch_ncb<false>(ncb, m, t, rowmap, in, out, w, bias, n_in, n_out, s);
+    bool done = vec4 ? dispatch_ncb<true>(ncb, m, t, in, out, w, bias, n_in, n_out, s)
+                     : dispatch_ncb<false>(ncb, m, t, in, out, w, bias, n_in, n_out, s);
     if (done) return;
   }
   int64_t total = t.n * n_out;
-  k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, rowmap, t.K, t.n, t.npad, in,
+  k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in,
                                                                        out, w, bias, n_in, n_out, groups);
   LAUNCH_CHECK();
 }

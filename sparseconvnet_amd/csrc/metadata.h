@@ -30,11 +30,17 @@ struct Level {
 };
 
 // Neighbour table: nbr[k * npad + t] = row feeding filter tap k of the output row at
-// schedule position t, or -1.  counts[k] = number of non-negative entries of tap k.
+// position t, or -1; rowmap[t] = that output row.  Positions follow the level's schedule
+// (ascending site key), then inside every block of 256 positions they are sorted by
+// neighbour pattern (the bit mask of present taps), so that the 16 positions a wavefront
+// works on mostly need the same taps.  counts[k] = number of non-negative entries of tap k.
 struct Table {
   int K = 0;
   int64_t n = 0, npad = 0;
   DevBuf<int> nbr;
+  DevBuf<int> rowmap;
+  bool identity_rows = false;  // rowmap[t] == t: kernels skip the indirection
+  const int *rowmap_ptr() const { return identity_rows ? nullptr : rowmap.p; }
   std::vector<int64_t> counts;
   int64_t total() const {
     int64_t s = 0;
@@ -86,16 +92,15 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
                             const int64_t *filter, const int64_t *stride, hipStream_t s);
 // Pairs of tap k of a table: (value, row at position t), ordered by t.  Returns the count.
-int64_t export_table_pairs(Metadata &m, const Table &t, const int *sched, int k, bool swap,
-                           int *pairs, hipStream_t s);
+int64_t export_table_pairs(Metadata &m, const Table &t, int k, bool swap, int *pairs, hipStream_t s);
 std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t s);
 int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *pairs,
                          hipStream_t s);
 
 // ops.hip / conv.hip
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);
-void conv_forward(Metadata &m, const Table &t, const int *rowmap, const float *in, float *out, const float *w,
-                  const float *bias, int n_in, int n_out, int groups, hipStream_t s);
+void conv_forward(Metadata &m, const Table &t, const float *in, float *out, const float *w, const float *bias,
+                  int n_in, int n_out, int groups, hipStream_t s);
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
                      int drop, hipStream_t s);
 void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,

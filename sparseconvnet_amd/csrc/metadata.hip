@@ -66,11 +66,11 @@ void fill32(void *p, uint32_t v, int64_t n, hipStream_t s) {
 }
 
 static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout,
-                       const int *vin, int *vout, int64_t n, hipStream_t s) {
+                       const int *vin, int *vout, int64_t n, hipStream_t s, int end_bit = 64) {
   size_t bytes = 0;
-  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, 64, s));
+  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
   m.tmp.reserve(bytes + 16);
-  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, 64, s));
+  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
 }
 static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipStream_t s) {
   size_t bytes = 0;
@@ -395,6 +395,71 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
     if (lcount[k]) atomicAdd(&counts[k], (unsigned long long)lcount[k]);
 }
 
+
+// ---- pattern-sorted positions ----------------------------------------------------------
+
+static const int BLOCK_SHIFT = 8;  // positions are re-sorted inside blocks of 256
+
+__global__ void k_table_masks(const int *nbr, int K, int64_t n, int64_t npad, unsigned long long *keys,
+                              int *idx) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  unsigned long long mask = 0;
+  for (int k = 0; k < K; k++)
+    if (nbr[(int64_t)k * npad + t] >= 0) mask |= 1ull << k;
+  keys[t] = ((unsigned long long)(t >> BLOCK_SHIFT) << K) | mask;
+  idx[t] = (int)t;
+}
+__global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, const int *perm,
+                                const int *base, int *nbr2, int *rowmap) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * K) return;
+  int k = (int)(i / n);
+  int64_t t = i - (int64_t)k * n;
+  int src = perm[t];
+  nbr2[(int64_t)k * npad + t] = nbr[(int64_t)k * npad + src];
+  if (k == 0) rowmap[t] = base ? base[src] : src;
+}
+__global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) rowmap[t] = base ? base[t] : (int)t;
+}
+
+// t.nbr is indexed by the level's schedule (base[t] = row, or t itself when base is null).
+// Re-sort positions by neighbour pattern inside blocks and record the position -> row map.
+static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s) {
+  if (t.n == 0) {
+    t.identity_rows = true;
+    return;
+  }
+  t.rowmap.reserve(t.npad);
+  int block_bits = 1;
+  while (((int64_t)1 << block_bits) <= (t.n >> BLOCK_SHIFT)) block_bits++;
+  if (t.K + block_bits > 62) {  // the pattern does not fit the sort key: keep schedule order
+    t.identity_rows = base == nullptr;
+    if (base) {
+      k_copy_rowmap<<<grid_for(t.n), TB, 0, s>>>(base, t.n, t.rowmap.p);
+      LAUNCH_CHECK();
+    }
+    return;
+  }
+  m.k0.reserve(t.n);
+  m.k1.reserve(t.n);
+  m.v0.reserve(t.n);
+  m.v1.reserve(t.n);
+  k_table_masks<<<grid_for(t.n), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p);
+  LAUNCH_CHECK();
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, t.K + block_bits);
+  DevBuf<int> nbr2;
+  nbr2.reserve((size_t)t.K * t.npad);
+  k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
+                                                     t.rowmap.p);
+  LAUNCH_CHECK();
+  HIP_CHECK(hipStreamSynchronize(s));  // the old table is freed when nbr2 replaces it
+  t.nbr = std::move(nbr2);
+  t.identity_rows = false;
+}
+
 static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const int64_t *out_size) {
   Filt f{};
   f.dim = dim;
@@ -434,6 +499,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
     // Metadata/Metadata.cpp:445: an unknown level is an empty one.
     t.n = 0;
     t.npad = 64;
+    t.identity_rows = true;
     t.counts.assign(f.K, 0);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
@@ -449,6 +515,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
                                                             (unsigned long long *)m.dcounts.p);
   LAUNCH_CHECK();
   fetch_counts(m, t, s);
+  finalize_table(m, t, L.sched_ptr(), s);
   return m.subm.emplace(key, std::move(t)).first->second;
 }
 
@@ -552,6 +619,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     R.by_out.npad = 64;
     R.by_in.n = 0;
     R.by_in.npad = 64;
+    R.by_out.identity_rows = R.by_in.identity_rows = true;
     return m.strided.emplace(key, std::move(R)).first->second;
   }
   Level &LI = m.levels[R.in_size];
@@ -592,6 +660,8 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   LAUNCH_CHECK();
   fetch_counts(m, R.by_out, s);
   R.by_in.counts = R.by_out.counts;
+  finalize_table(m, R.by_out, nullptr, s);
+  finalize_table(m, R.by_in, LI.sched_ptr(), s);
   return m.strided.emplace(key, std::move(R)).first->second;
 }
 
@@ -638,8 +708,8 @@ __global__ void k_tap_compact(const int *nbr, const int *sched, int64_t n, const
     pairs[2 * pos + (swap ? 0 : 1)] = row;
   }
 }
-int64_t export_table_pairs(Metadata &m, const Table &t, const int *sched, int k, bool swap, int *pairs,
-                           hipStream_t s) {
+int64_t export_table_pairs(Metadata &m, const Table &t, int k, bool swap, int *pairs, hipStream_t s) {
+  const int *sched = t.rowmap_ptr();
   if (k < 0 || k >= t.K) throw Error("rule list index out of range");
   if (t.n == 0 || t.counts[k] == 0) return 0;
   int64_t blocks = ceil_div(t.n, TB);

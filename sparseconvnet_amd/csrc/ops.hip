@@ -64,8 +64,8 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
 // ---- max pooling ------------------------------------------------------------------------
 // CPU/MaxPooling.cpp:7-20,50: the output starts at zero and takes every input of its window
 // that compares greater, so the result is max(0, active inputs); output-stationary here.
-__global__ void k_maxpool(const int *nbr, int K, int64_t n_out, int64_t npad, const float *in,
-                          int in_stride, float *out, int planes) {
+__global__ void k_maxpool(const int *nbr, const int *rowmap, int K, int64_t n_out, int64_t npad,
+                          const float *in, int in_stride, float *out, int planes) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = n_out * planes;
   int64_t step = (int64_t)gridDim.x * blockDim.x;
@@ -80,7 +80,8 @@ __global__ void k_maxpool(const int *nbr, int K, int64_t n_out, int64_t npad, co
         if (acc < v) acc = v;
       }
     }
-    out[i] = acc;
+    int64_t row = rowmap ? rowmap[o] : o;
+    out[row * planes + p] = acc;
   }
 }
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
@@ -88,8 +89,8 @@ void maxpool_forward(const Table &t, const float *in, int in_stride, float *out,
   if (t.n == 0 || planes <= 0) return;
   int64_t total = t.n * planes;
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
-  k_maxpool<<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, in + drop, in_stride, out,
-                                                  planes);
+  k_maxpool<<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+                                                  in_stride, out, planes);
   LAUNCH_CHECK();
 }
 
