@@ -84,6 +84,47 @@ def cpu_baseline(sample_sites, seed):
                       % (len(coords), R, t_rules)}
 
 
+def unet_scene(sites, seed, reps=3):
+    """3D U-Net forward of examples/ScanNet/unet.py:25-38 with m=32, block_reps=2 (7 levels,
+    [32..224] planes), InputLayer mode 4 on a room scene with ~30% duplicated points, eval,
+    random-init weights, batch 1.  cold = new Metadata per scene, as a user runs it (input layer,
+    every rulebook and all layers); warm = the same scene again with its rulebooks cached."""
+    import torch
+    import sparseconvnet_amd as scn
+    from sparseconvnet_amd import synthetic
+    m = 32
+    torch.manual_seed(0)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m, 5 * m, 6 * m, 7 * m], False)).add(scn.OutputLayer(3)).cuda().eval()
+    linear = torch.nn.Linear(m, 20).cuda()
+    coords = synthetic.room_scene(seed=seed, target=sites, spatial=4096, duplicate_fraction=0.3)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    feats = torch.rand((len(coords), 3), device="cuda", generator=g) * 2 - 1
+    cd = torch.as_tensor(coords).cuda()
+    inp_layer = scn.InputLayer(3, 4096, mode=4)
+    cold, warm = [], []
+    with torch.no_grad():
+        for r in range(reps + 1):
+            scn.forward_pass_multiplyAdd_count = 0
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            x = inp_layer([cd, feats])
+            y = linear(model(x))
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            y = linear(model(x))
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            if r:  # first pass warms allocators and code objects
+                cold.append((t1 - t0) * 1e3)
+                warm.append((t2 - t1) * 1e3)
+            macs = scn.forward_pass_multiplyAdd_count / 2
+    return {"unet_ms_per_scene": round(float(np.median(cold)), 3), "unet_warm_ms": round(float(np.median(warm)), 3),
+            "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
+            "unet_gflop": round(2 * macs / 1e9, 2),
+            "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +136,8 @@ def main():
     ap.add_argument("--cpu-sites", type=int, default=200000)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pairs", default="")
+    ap.add_argument("--no-unet", action="store_true")
+    ap.add_argument("--unet-sites", type=int, default=1000000)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -192,9 +235,12 @@ def main():
         "rulebook_sites_per_s": round(n / (rulebook_ms * 1e-3)),
         "roofline": roof, "sweep": sweep,
     }
+    L.scn_md_destroy(h)
+    del work
+    if not args.no_unet:
+        out["unet"] = unet_scene(args.unet_sites, 5000)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sites, args.seed)
-    L.scn_md_destroy(h)
     print(json.dumps(out))
 
 

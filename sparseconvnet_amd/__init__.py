@@ -1,0 +1,28 @@
+"""sparseconvnet_amd: the forward pass of submanifold sparse convolutional networks on
+AMD MI355X, with the module API of facebookresearch/SparseConvNet (`import sparseconvnet_amd
+as scn`).  The modules call hand-written gfx950 kernels in libscn_hip.so through its C ABI
+(include/scn_hip.h); tensors are ordinary PyTorch-ROCm tensors."""
+
+# Counters the reference keeps at package level (sparseconvnet/__init__.py:7-8): multiply-adds
+# and output elements of the convolutions run so far.
+forward_pass_multiplyAdd_count = 0
+forward_pass_hidden_states = 0
+
+from .containers import AddTable, ConcatTable, JoinTable, Sequential  # noqa: E402
+from .layers import (BatchNormalization, BatchNormLeakyReLU, BatchNormReLU, Convolution,  # noqa: E402
+                     Deconvolution, Identity, InputLayer, MaxPooling, OutputLayer, SparseToDense,
+                     SubmanifoldConvolution, ValidConvolution)
+from .metadata import Metadata  # noqa: E402
+from .networks import SparseVggNet, UNet  # noqa: E402
+from .tensor import SparseConvNetTensor  # noqa: E402
+from .utils import optionalTensor, toLongTensor  # noqa: E402
+
+
+def is_hip_build():
+    """True when libscn_hip.so is present and loadable (the reference's SCN.is_cuda_build)."""
+    from . import _lib
+    try:
+        _lib.lib()
+        return True
+    except Exception:
+        return False

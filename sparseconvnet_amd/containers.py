@@ -1,0 +1,82 @@
+"""Containers: Sequential and the table modules (reference: sequential.py:10-35,
+tables.py:13-55).  They only route SparseConvNetTensors; feature concatenation and addition
+are plain torch ops on the GPU."""
+import torch
+
+from .tensor import SparseConvNetTensor
+
+
+class Sequential(torch.nn.Sequential):
+    def input_spatial_size(self, out_size):
+        for m in reversed(self._modules):
+            out_size = self._modules[m].input_spatial_size(out_size)
+        return out_size
+
+    def __add__(self, x):
+        r = Sequential()
+        for m in self:
+            r.append(m)
+        for m in x:
+            r.append(m)
+        return r
+
+    def add(self, module):
+        self._modules[str(len(self._modules))] = module
+        return self
+
+    def insert(self, index, module):
+        for i in range(len(self._modules), index, -1):
+            self._modules[str(i)] = self._modules[str(i - 1)]
+        self._modules[str(index)] = module
+
+    def append(self, module):
+        self._modules[str(len(self._modules))] = module
+        return self
+
+
+class _Table(torch.nn.Sequential):
+    def __init__(self, *args):
+        torch.nn.Sequential.__init__(self, *args)
+
+    def add(self, module):
+        self._modules[str(len(self._modules))] = module
+        return self
+
+
+class ConcatTable(_Table):
+    """Applies every child to the same input; returns the list of results."""
+
+    def forward(self, input):
+        return [module(input) for module in self._modules.values()]
+
+    def input_spatial_size(self, out_size):
+        return self._modules['0'].input_spatial_size(out_size)
+
+
+class JoinTable(_Table):
+    """Concatenates the feature planes of a list of tensors on one level."""
+
+    def forward(self, input):
+        output = SparseConvNetTensor()
+        output.metadata = input[0].metadata
+        output.spatial_size = input[0].spatial_size
+        output.features = torch.cat([i.features for i in input], 1) if input[0].features.numel() \
+            else input[0].features
+        return output
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+
+class AddTable(_Table):
+    """Adds the features of a list of tensors on one level."""
+
+    def forward(self, input):
+        output = SparseConvNetTensor()
+        output.metadata = input[0].metadata
+        output.spatial_size = input[0].spatial_size
+        output.features = sum([i.features for i in input])
+        return output
+
+    def input_spatial_size(self, out_size):
+        return out_size

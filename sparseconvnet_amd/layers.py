@@ -1,0 +1,345 @@
+"""The forward-pass modules, with the constructor signatures, attribute names, parameter
+shapes, initialisation, spatial-size arithmetic and repr of the reference's Python modules
+(cited per class; paths relative to the reference's sparseconvnet/ directory).  Each forward
+calls the HIP library through sparseconvnet_amd.metadata; there is no backward: this build
+covers inference, and differentiating through a module raises."""
+import torch
+from torch.autograd import Function
+from torch.nn import Module, Parameter
+
+import sparseconvnet_amd as _pkg
+
+from . import metadata as _md
+from .tensor import SparseConvNetTensor
+from .utils import optionalTensor, toLongTensor
+
+
+class _ForwardOnly(Function):
+    """Runs `fn(*tensors)` outside autograd; backward is not part of this build."""
+
+    @staticmethod
+    def forward(ctx, fn, *tensors):
+        return fn(*tensors)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("sparseconvnet_amd implements the forward (inference) pass only")
+
+
+def _run(fn, *tensors):
+    if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors):
+        return _ForwardOnly.apply(fn, *tensors)
+    return fn(*tensors)
+
+
+def _size_repr(prefix, size, stride=None):
+    """'C3', 'C(3,1,3)', 'C3/2', 'C(3,3)/(2,1)' ... as the reference prints filter sizes."""
+    uniform = size.max().item() == size.min().item() and (
+        stride is None or stride.max().item() == stride.min().item())
+    if uniform:
+        s = prefix + str(size[0].item())
+        if stride is not None:
+            s += '/' + str(stride[0].item())
+        return s
+    s = prefix + '(' + ','.join(str(v.item()) for v in size) + ')'
+    if stride is not None:
+        s += '/(' + ','.join(str(v.item()) for v in stride) + ')'
+    return s
+
+
+def _conv_weight(filter_volume, groups, nIn, nOut):
+    # N(0, sqrt(2 * groups / (nIn * filter_volume))): submanifoldConvolution.py:23-26
+    std = (2.0 * groups / nIn / filter_volume) ** 0.5
+    return Parameter(torch.Tensor(filter_volume, groups, nIn // groups, nOut // groups).normal_(0, std))
+
+
+def _count(macs, out):
+    _pkg.forward_pass_multiplyAdd_count += macs
+    _pkg.forward_pass_hidden_states += out.nelement()
+
+
+class SubmanifoldConvolution(Module):
+    """submanifoldConvolution.py:14-61."""
+
+    def __init__(self, dimension, nIn, nOut, filter_size, bias, groups=1):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.groups = groups
+        self.nIn = nIn
+        self.nOut = nOut
+        self.filter_size = toLongTensor(dimension, filter_size)
+        self.filter_volume = self.filter_size.prod().item()
+        self.weight = _conv_weight(self.filter_volume, groups, nIn, nOut)
+        if bias:
+            self.bias = Parameter(torch.Tensor(nOut).zero_())
+
+    def forward(self, input):
+        assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, self.nOut, input)
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = input.spatial_size
+        md, sz, fs = input.metadata, input.spatial_size, self.filter_size
+
+        def fn(x, w, b):
+            y, macs = md.submanifoldConvolution(sz, fs, x, w, b)
+            _count(macs, y)
+            return y
+        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        return output
+
+    def __repr__(self):
+        return 'SubmanifoldConvolution ' + str(self.nIn) + '->' + str(self.nOut) + _size_repr(' C', self.filter_size)
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+
+class ValidConvolution(SubmanifoldConvolution):
+    pass
+
+
+class Convolution(Module):
+    """convolution.py:13-70."""
+
+    def __init__(self, dimension, nIn, nOut, filter_size, filter_stride, bias, groups=1):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.groups = groups
+        self.nIn = nIn
+        self.nOut = nOut
+        self.filter_size = toLongTensor(dimension, filter_size)
+        self.filter_volume = self.filter_size.prod().item()
+        self.filter_stride = toLongTensor(dimension, filter_stride)
+        self.weight = _conv_weight(self.filter_volume, groups, nIn, nOut)
+        if bias:
+            self.bias = Parameter(torch.Tensor(nOut).zero_())
+
+    def forward(self, input):
+        assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = (input.spatial_size - self.filter_size).div(
+            self.filter_stride, rounding_mode='trunc') + 1
+        assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
+            input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+
+        def fn(x, w, b):
+            y, macs = md.convolution(*a, x, w, b)
+            _count(macs, y)
+            return y
+        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        return output
+
+    def __repr__(self):
+        return 'Convolution ' + str(self.nIn) + '->' + str(self.nOut) + _size_repr(
+            ' C', self.filter_size, self.filter_stride)
+
+    def input_spatial_size(self, out_size):
+        return (out_size - 1) * self.filter_stride + self.filter_size
+
+
+class Deconvolution(Module):
+    """deconvolution.py:13-47,76-100: undoes the matching Convolution's change of level."""
+
+    def __init__(self, dimension, nIn, nOut, filter_size, filter_stride, bias, groups=1):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.groups = groups
+        self.nIn = nIn
+        self.nOut = nOut
+        self.filter_size = toLongTensor(dimension, filter_size)
+        self.filter_volume = self.filter_size.prod().item()
+        self.filter_stride = toLongTensor(dimension, filter_stride)
+        self.weight = _conv_weight(self.filter_volume, groups, nIn, nOut)
+        if bias:
+            self.bias = Parameter(torch.Tensor(nOut).zero_())
+
+    def forward(self, input):
+        assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
+        md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+
+        def fn(x, w, b):
+            y, macs = md.deconvolution(*a, x, w, b)
+            _count(macs, y)
+            return y
+        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        return output
+
+    def __repr__(self):
+        return 'Deconvolution ' + str(self.nIn) + '->' + str(self.nOut) + _size_repr(
+            ' C', self.filter_size, self.filter_stride)
+
+    def input_spatial_size(self, out_size):
+        in_size = (out_size - self.filter_size) / self.filter_stride + 1
+        assert ((in_size - 1) * self.filter_stride + self.filter_size == out_size).all()
+        return in_size
+
+
+class BatchNormalization(Module):
+    """batchNormalization.py:13-71.  leakiness: 0 = ReLU, (0,1) = leaky ReLU, 1 = none.
+    Only eval mode is implemented: the running statistics are used as they are."""
+
+    def __init__(self, nPlanes, eps=1e-4, momentum=0.99, affine=True, leakiness=1):
+        Module.__init__(self)
+        self.nPlanes = nPlanes
+        self.eps = eps
+        self.momentum = momentum
+        self.affine = affine
+        self.leakiness = leakiness
+        self.register_buffer("running_mean", torch.Tensor(nPlanes).fill_(0))
+        self.register_buffer("running_var", torch.Tensor(nPlanes).fill_(1))
+        if affine:
+            self.weight = Parameter(torch.Tensor(nPlanes).fill_(1))
+            self.bias = Parameter(torch.Tensor(nPlanes).fill_(0))
+
+    def forward(self, input):
+        if input.features.nelement() == 0:
+            return input
+        assert input.features.size(1) == self.nPlanes, (self.nPlanes, input.features.shape)
+        if self.training:
+            raise NotImplementedError("sparseconvnet_amd batch normalisation runs in eval mode only; "
+                                      "call .eval() on the model")
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = input.spatial_size
+        eps, leak, mean, var = self.eps, self.leakiness, self.running_mean, self.running_var
+        output.features = _run(lambda x, w, b: _md.batchNormEval(x, mean, var, w, b, eps, leak),
+                               input.features, optionalTensor(self, 'weight'), optionalTensor(self, 'bias'))
+        return output
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+    def __repr__(self):
+        s = 'BatchNorm(' + str(self.nPlanes) + ',eps=' + str(self.eps) + ',momentum=' + str(self.momentum) + \
+            ',affine=' + str(self.affine)
+        if self.leakiness > 0:
+            s = s + ',leakiness=' + str(self.leakiness)
+        return s + ')'
+
+
+class BatchNormReLU(BatchNormalization):
+    """batchNormalization.py:74-81."""
+
+    def __init__(self, nPlanes, eps=1e-4, momentum=0.99):
+        BatchNormalization.__init__(self, nPlanes, eps, momentum, True, 0)
+
+    def __repr__(self):
+        return 'BatchNormReLU(' + str(self.nPlanes) + ',eps=' + str(self.eps) + ',momentum=' + \
+            str(self.momentum) + ',affine=' + str(self.affine) + ')'
+
+
+class BatchNormLeakyReLU(BatchNormalization):
+    """batchNormalization.py:84-91."""
+
+    def __init__(self, nPlanes, eps=1e-4, momentum=0.99, leakiness=0.333):
+        BatchNormalization.__init__(self, nPlanes, eps, momentum, True, leakiness)
+
+    def __repr__(self):
+        return 'BatchNormLeakyReLU(' + str(self.nPlanes) + ',eps=' + str(self.eps) + ',momentum=' + \
+            str(self.momentum) + ',affine=' + str(self.affine) + ',leakiness=' + str(self.leakiness) + ')'
+
+
+class MaxPooling(Module):
+    """maxPooling.py:74-117."""
+
+    def __init__(self, dimension, pool_size, pool_stride, nFeaturesToDrop=0):
+        super(MaxPooling, self).__init__()
+        self.dimension = dimension
+        self.pool_size = toLongTensor(dimension, pool_size)
+        self.pool_stride = toLongTensor(dimension, pool_stride)
+        self.nFeaturesToDrop = nFeaturesToDrop
+
+    def forward(self, input):
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = (input.spatial_size - self.pool_size).div(
+            self.pool_stride, rounding_mode='trunc') + 1
+        assert ((output.spatial_size - 1) * self.pool_stride + self.pool_size == input.spatial_size).all()
+        md, a, drop = input.metadata, (input.spatial_size, output.spatial_size, self.pool_size,
+                                       self.pool_stride), self.nFeaturesToDrop
+        output.features = _run(lambda x: md.maxPooling(*a, x, drop), input.features)
+        return output
+
+    def input_spatial_size(self, out_size):
+        return (out_size - 1) * self.pool_stride + self.pool_size
+
+    def __repr__(self):
+        s = _size_repr('MaxPooling', self.pool_size, self.pool_stride)
+        if self.nFeaturesToDrop > 0:
+            s = s + ' nFeaturesToDrop = ' + str(self.nFeaturesToDrop)
+        return s
+
+
+class InputLayer(Module):
+    """ioLayers.py:15-65.  forward takes (coords, features[, batch_size]): coords is an int64
+    tensor [N, dimension] (one sample) or [N, dimension+1] (last column = sample index),
+    features a float tensor [N, planes].  Points that share a site are merged according to
+    mode: 0 none (rows = points), 1 first, 2 last, 3 sum, 4 mean - as the reference's rule
+    builder behaves (Metadata/IOLayersRules.h:96-107), not as its docstring says for 1 and 2."""
+
+    def __init__(self, dimension, spatial_size, mode=3):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.spatial_size = toLongTensor(dimension, spatial_size)
+        self.mode = mode
+        self.device = None
+
+    def to(self, device):
+        self.device = device
+        return self
+
+    def forward(self, input):
+        output = SparseConvNetTensor(metadata=_md.Metadata(self.dimension), spatial_size=self.spatial_size)
+        feats = input[1].to(self.device) if self.device else input[1]
+        if not feats.is_cuda:
+            feats = feats.cuda()
+        md, sz, coords, mode = output.metadata, self.spatial_size, input[0], self.mode
+        batch_size = 0 if len(input) == 2 else input[2]
+        output.features = _run(lambda f: md.inputLayer(sz, coords, f, batch_size, mode), feats.float())
+        return output
+
+
+class OutputLayer(Module):
+    """ioLayers.py:68-89: one row per original input point."""
+
+    def __init__(self, dimension):
+        Module.__init__(self)
+        self.dimension = dimension
+
+    def forward(self, input):
+        md = input.metadata
+        return _run(lambda x: md.outputLayer(x), input.features)
+
+
+class SparseToDense(Module):
+    """sparseToDense.py:56-78: dense [batch, nPlanes, spatial...] tensor, zeros elsewhere."""
+
+    def __init__(self, dimension, nPlanes):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.nPlanes = nPlanes
+
+    def forward(self, input):
+        md, sz, planes = input.metadata, input.spatial_size, self.nPlanes
+        return _run(lambda x: md.sparseToDense(sz, x, planes), input.features)
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+    def __repr__(self):
+        return 'SparseToDense(' + str(self.dimension) + ',' + str(self.nPlanes) + ')'
+
+
+class Identity(Module):
+    """identity.py:10-15."""
+
+    def forward(self, input):
+        return input
+
+    def input_spatial_size(self, out_size):
+        return out_size

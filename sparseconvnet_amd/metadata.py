@@ -1,0 +1,146 @@
+"""Metadata: which sites are active at every spatial size, plus the cached rulebooks.
+
+Mirrors the object the reference exposes as `sparseconvnet.Metadata(dim)`
+(sparseconvnet/metadata.py:16-17 -> pybind class Metadata_<D>, SCN/pybind.cpp:11-33),
+as a thin owner of a handle of libscn_hip.so.  Everything lives on the GPU; only counts
+cross back to the host."""
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None and t.numel() else C.c_void_p(0)
+
+
+def _features(t, what):
+    if not t.is_cuda:
+        raise _lib.ScnError("%s must be a CUDA tensor: this library has no CPU path" % what)
+    if t.dtype != torch.float32:
+        raise _lib.ScnError("%s must be float32" % what)
+    return t.contiguous()
+
+
+class Metadata:
+    def __init__(self, dimension):
+        self.dimension = dimension
+        self._L = _lib.lib()
+        self._h = self._L.scn_md_create(dimension)
+        if not self._h:
+            raise _lib.ScnError(self._L.scn_last_error().decode())
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._L.scn_md_destroy(h)
+
+    def _s(self, x):
+        return _lib.sizes(self.dimension, x)
+
+    # ---- what the reference binds on Metadata_<D> ------------------------------------
+    def clear(self):
+        _lib.check(self._L.scn_md_clear(self._h))
+
+    def getNActive(self, spatial_size):
+        n = C.c_int64(0)
+        _lib.check(self._L.scn_md_nactive(self._h, self._s(spatial_size), C.byref(n)))
+        return n.value
+
+    def getBatchSize(self, spatial_size):
+        b = C.c_int(0)
+        _lib.check(self._L.scn_md_batch_size(self._h, self._s(spatial_size), C.byref(b)))
+        return b.value
+
+    def getSpatialLocations(self, spatial_size):
+        """LongTensor [nActive, dimension+1] on the CPU: coordinates, then sample index."""
+        n = self.getNActive(spatial_size)
+        out = torch.zeros((n, self.dimension + 1), dtype=torch.int64, device="cuda")
+        if n:
+            _lib.check(self._L.scn_md_spatial_locations(self._h, self._s(spatial_size), _ptr(out), _stream()))
+        return out.cpu()
+
+    # ---- forward ops; each returns a new CUDA tensor ---------------------------------
+    def inputLayer(self, spatial_size, coords, features, batch_size, mode):
+        coords = coords.to(device=features.device, dtype=torch.int64).contiguous()
+        assert coords.dim() == 2 and coords.size(0) == features.size(0)
+        features = _features(features, "input features")
+        n = C.c_int64(0)
+        _lib.check(self._L.scn_md_input_layer(self._h, self._s(spatial_size), _ptr(coords), coords.size(0),
+                                              coords.size(1), int(batch_size), int(mode), _stream(),
+                                              C.byref(n)))
+        out = torch.empty((n.value, features.size(1)), dtype=torch.float32, device=features.device)
+        _lib.check(self._L.scn_input_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
+        return out
+
+    def outputLayer(self, features):
+        features = _features(features, "features")
+        hdr = (C.c_int32 * 4)()
+        _lib.check(self._L.scn_md_input_rules_header(self._h, hdr))
+        out = torch.empty((hdr[2], features.size(1)), dtype=torch.float32, device=features.device)
+        _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
+        return out
+
+    def _conv(self, fn, size_args, n_rows, features, weight, bias):
+        features = _features(features, "features")
+        weight = _features(weight, "weight")
+        K, groups, ip, op = weight.shape
+        bias_t = _features(bias, "bias") if bias is not None and bias.numel() else None
+        out = torch.empty((n_rows, groups * op), dtype=torch.float32, device=features.device)
+        macs = C.c_double(0)
+        _lib.check(fn(self._h, *size_args, _ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t), groups * ip,
+                      groups * op, groups, _stream(), C.byref(macs)))
+        return out, macs.value
+
+    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias):
+        sp, fs = self._s(spatial_size), self._s(filter_size)
+        _lib.check(self._L.scn_md_submanifold_rules(self._h, sp, fs, _stream()))
+        return self._conv(self._L.scn_subm_conv_fwd, (sp, fs), self.getNActive(spatial_size), features, weight,
+                          bias)
+
+    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias):
+        a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
+        return self._conv(self._L.scn_conv_fwd, a, self.getNActive(out_size), features, weight, bias)
+
+    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias):
+        a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
+        _lib.check(self._L.scn_md_strided_rules(self._h, *rb, _stream()))
+        return self._conv(self._L.scn_deconv_fwd, a, self.getNActive(out_size), features, weight, bias)
+
+    def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
+        features = _features(features, "features")
+        planes = features.size(1) - n_features_to_drop
+        out = torch.empty((self.getNActive(out_size), planes), dtype=torch.float32, device=features.device)
+        _lib.check(self._L.scn_maxpool_fwd(self._h, *a, _ptr(features), features.size(1), _ptr(out), planes,
+                                           n_features_to_drop, _stream()))
+        return out
+
+    def sparseToDense(self, spatial_size, features, n_planes):
+        features = _features(features, "features")
+        sp = [int(v) for v in self._s(spatial_size)]
+        out = torch.empty([self.getBatchSize(spatial_size), n_planes] + sp, dtype=torch.float32,
+                          device=features.device)
+        _lib.check(self._L.scn_s2d_fwd(self._h, self._s(spatial_size), _ptr(features), _ptr(out), n_planes,
+                                       _stream()))
+        return out
+
+
+def batchNormEval(features, running_mean, running_var, weight, bias, eps, leakiness):
+    features = _features(features, "features")
+    out = torch.empty_like(features)
+    w = weight if weight is not None and weight.numel() else None
+    b = bias if bias is not None and bias.numel() else None
+    _lib.check(_lib.lib().scn_bn_eval_fwd(_ptr(features), _ptr(out), features.size(0), features.size(1),
+                                          features.stride(0), out.stride(0), _ptr(running_mean),
+                                          _ptr(running_var), _ptr(w), _ptr(b), float(eps), float(leakiness),
+                                          _stream()))
+    return out

@@ -1,0 +1,129 @@
+"""The Python module API against what the reference's modules promise (constructor
+signatures, attribute names, parameter shapes and initialisation, spatial-size arithmetic,
+repr strings, state_dict layout).  No GPU needed.  Citations: reference sparseconvnet/*.py."""
+import math
+
+import pytest
+import torch
+
+import sparseconvnet_amd as scn
+
+
+def hello_world_model():
+    # examples/hello-world.py:19-30
+    return scn.Sequential().add(
+        scn.SparseVggNet(2, 1, [['C', 8], ['C', 8], ['MP', 3, 2], ['C', 16], ['C', 16], ['MP', 3, 2],
+                                ['C', 24], ['C', 24], ['MP', 3, 2]])
+    ).add(scn.SubmanifoldConvolution(2, 24, 32, 3, False)).add(scn.BatchNormReLU(32)).add(scn.SparseToDense(2, 32))
+
+
+def test_exports():
+    for name in ["SubmanifoldConvolution", "ValidConvolution", "Convolution", "Deconvolution",
+                 "BatchNormalization", "BatchNormReLU", "BatchNormLeakyReLU", "MaxPooling", "InputLayer",
+                 "OutputLayer", "SparseToDense", "Metadata", "SparseConvNetTensor", "Sequential", "ConcatTable",
+                 "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor"]:
+        assert hasattr(scn, name), name
+    assert scn.forward_pass_multiplyAdd_count == 0 and scn.forward_pass_hidden_states == 0
+
+
+def test_conv_parameters_and_repr():
+    # submanifoldConvolution.py:15-28,45-56; convolution.py:14-29,53-67
+    c = scn.SubmanifoldConvolution(3, 16, 32, 3, False)
+    assert tuple(c.weight.shape) == (27, 1, 16, 32) and not hasattr(c, 'bias')
+    assert c.filter_volume == 27 and c.filter_size.tolist() == [3, 3, 3] and c.dimension == 3
+    assert repr(c) == 'SubmanifoldConvolution 16->32 C3'
+    assert repr(scn.SubmanifoldConvolution(3, 4, 4, [3, 1, 3], True)) == 'SubmanifoldConvolution 4->4 C(3,1,3)'
+    g = scn.SubmanifoldConvolution(2, 8, 12, 3, True, groups=2)
+    assert tuple(g.weight.shape) == (9, 2, 4, 6) and tuple(g.bias.shape) == (12,) and (g.bias == 0).all()
+    d = scn.Convolution(3, 32, 64, 2, 2, False)
+    assert tuple(d.weight.shape) == (8, 1, 32, 64) and repr(d) == 'Convolution 32->64 C2/2'
+    assert repr(scn.Convolution(2, 1, 1, [3, 2], [2, 1], False)) == 'Convolution 1->1 C(3,2)/(2,1)'
+    u = scn.Deconvolution(3, 64, 32, 2, 2, False)
+    assert tuple(u.weight.shape) == (8, 1, 64, 32) and repr(u) == 'Deconvolution 64->32 C2/2'
+    assert issubclass(scn.ValidConvolution, scn.SubmanifoldConvolution)
+
+
+def test_weight_initialisation_scale():
+    # std = sqrt(2 * groups / (nIn * filter_volume)), submanifoldConvolution.py:23-26
+    torch.manual_seed(0)
+    c = scn.SubmanifoldConvolution(3, 64, 64, 3, False)
+    want = math.sqrt(2.0 / (64 * 27))
+    assert abs(c.weight.std().item() / want - 1) < 0.02 and abs(c.weight.mean().item()) < 0.1 * want
+
+
+def test_spatial_size_arithmetic():
+    t = torch.LongTensor
+    assert scn.Convolution(3, 1, 1, 2, 2, False).input_spatial_size(t([64] * 3)).tolist() == [128] * 3
+    assert scn.Convolution(2, 1, 1, 3, 2, False).input_spatial_size(t([7, 7])).tolist() == [15, 15]
+    assert scn.MaxPooling(2, 3, 2).input_spatial_size(t([8, 8])).tolist() == [17, 17]
+    assert scn.SubmanifoldConvolution(2, 1, 1, 3, False).input_spatial_size(t([9, 9])).tolist() == [9, 9]
+    # hello world: three MP3/2 need 8k+7 (README "Output is 2x32x10x10" for input 87)
+    m = hello_world_model()
+    assert m.input_spatial_size(t([10, 10])).tolist() == [87, 87]
+    assert m.input_spatial_size(t([8, 8])).tolist() == [71, 71]
+
+
+def test_bn_modules():
+    # batchNormalization.py:13-91
+    b = scn.BatchNormalization(5)
+    assert b.eps == 1e-4 and b.momentum == 0.99 and b.leakiness == 1 and b.affine
+    assert (b.running_mean == 0).all() and (b.running_var == 1).all() and (b.weight == 1).all()
+    assert sorted(b.state_dict()) == ['bias', 'running_mean', 'running_var', 'weight']
+    assert scn.BatchNormReLU(4).leakiness == 0
+    assert scn.BatchNormLeakyReLU(4).leakiness == 0.333
+    assert repr(scn.BatchNormReLU(32)) == 'BatchNormReLU(32,eps=0.0001,momentum=0.99,affine=True)'
+    assert repr(scn.BatchNormLeakyReLU(8, leakiness=0)) == \
+        'BatchNormLeakyReLU(8,eps=0.0001,momentum=0.99,affine=True,leakiness=0)'
+    assert repr(scn.BatchNormalization(3)) == 'BatchNorm(3,eps=0.0001,momentum=0.99,affine=True,leakiness=1)'
+
+
+def test_containers():
+    s = scn.Sequential().add(scn.Identity()).add(scn.BatchNormReLU(3))
+    assert len(s) == 2 and isinstance(s[1], scn.BatchNormReLU)
+    s2 = s + scn.Sequential().add(scn.Identity())
+    assert len(s2) == 3
+    s.insert(0, scn.MaxPooling(2, 3, 2))
+    assert isinstance(s[0], scn.MaxPooling) and len(s) == 3
+    ct = scn.ConcatTable().add(scn.Identity()).add(scn.Identity())
+    assert len(ct) == 2
+    a = scn.SparseConvNetTensor(torch.ones(3, 2), None, torch.LongTensor([4, 4]))
+    b = scn.SparseConvNetTensor(2 * torch.ones(3, 5), None, torch.LongTensor([4, 4]))
+    j = scn.JoinTable()(ct(a)[:1] + [b])
+    assert tuple(j.features.shape) == (3, 7) and j.spatial_size is a.spatial_size
+    assert (scn.AddTable()([a, a]).features == 2).all()
+
+
+def test_unet_structure_and_state_dict():
+    # networkArchitectures.py:203-257 with examples/ScanNet/unet.py:25-38 (m=32, reps=2, 7 levels)
+    m = 32
+    planes = [m * i for i in range(1, 8)]
+    u = scn.UNet(3, 2, planes, False)
+    convs = [x for x in u.modules() if isinstance(x, scn.SubmanifoldConvolution)]
+    downs = [x for x in u.modules() if isinstance(x, scn.Convolution)]
+    ups = [x for x in u.modules() if isinstance(x, scn.Deconvolution)]
+    bns = [x for x in u.modules() if isinstance(x, scn.BatchNormalization)]
+    assert len(convs) == 2 * 7 + 2 * 6 and len(downs) == 6 and len(ups) == 6 and len(bns) == 26 + 12
+    assert [(c.nIn, c.nOut) for c in downs] == [(planes[i], planes[i + 1]) for i in range(6)]
+    assert sorted((c.nIn, c.nOut) for c in ups) == sorted((planes[i + 1], planes[i]) for i in range(6))
+    assert (64, 32) in [(c.nIn, c.nOut) for c in convs] and (448, 224) not in [(c.nIn, c.nOut) for c in convs]
+    assert all(b.leakiness == 0 for b in bns)
+    # first block, as torch names it: sequential indices nest exactly as in the reference
+    sd = u.state_dict()
+    assert tuple(sd['0.1.weight'].shape) == (27, 1, 32, 32) and '0.0.running_mean' in sd
+    assert tuple(sd['2.1.1.weight'].shape) == (8, 1, 32, 64)      # Convolution 32->64 C2/2
+    assert tuple(sd['2.1.4.weight'].shape) == (8, 1, 64, 32)      # Deconvolution 64->32 C2/2
+    assert tuple(sd['4.1.weight'].shape) == (27, 1, 64, 32)       # first block after the join
+    with pytest.raises(NotImplementedError):
+        scn.UNet(3, 1, [8, 16], residual_blocks=True)
+
+
+def test_no_cpu_fallback():
+    from sparseconvnet_amd._lib import ScnError
+    layer = scn.InputLayer(2, 8, mode=3)
+    coords = torch.LongTensor([[1, 2, 0], [3, 4, 0]])
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    with pytest.raises((ScnError, RuntimeError, AssertionError)):
+        layer([coords, torch.ones(2, 1)])
+    with pytest.raises(ScnError):
+        scn.metadata.batchNormEval(torch.ones(2, 3), torch.zeros(3), torch.ones(3), None, None, 1e-4, 0)

@@ -1,0 +1,117 @@
+"""Whole networks through the module API on the GPU against the CPU oracle run over the same
+module tree and parameters (tests/oracle_model.py).  fp32 tolerance 1e-4 rel / 1e-5 abs."""
+import numpy as np
+import pytest
+import torch
+
+import checks
+import oracle_model
+import sparseconvnet_amd as scn
+from oracle import cpu_path
+from sparseconvnet_amd import synthetic
+from test_modules_api import hello_world_model
+
+pytestmark = pytest.mark.gpu
+
+
+def randomise_bn(model, seed):
+    g = torch.Generator().manual_seed(seed)
+    for m in model.modules():
+        if isinstance(m, scn.BatchNormalization):
+            m.running_mean.copy_(torch.randn(m.nPlanes, generator=g))
+            m.running_var.copy_(torch.rand(m.nPlanes, generator=g) + 0.5)
+
+
+def test_hello_world_shape():
+    # examples/hello-world.py: the output of the two-sample message batch is 2x32x10x10
+    torch.manual_seed(0)
+    model = hello_world_model().cuda().eval()
+    size = model.input_spatial_size(torch.LongTensor([10, 10]))
+    msgs = [[" X   X  XXX  X    X    XX     X       X   XX   XXX   X    XXX   ",
+             " X   X  X    X    X   X  X    X       X  X  X  X  X  X    X  X  ",
+             " XXXXX  XX   X    X   X  X    X   X   X  X  X  XXX   X    X   X ",
+             " X   X  X    X    X   X  X     X X X X   X  X  X  X  X    X  X  ",
+             " X   X  XXX  XXX  XXX  XX       X   X     XX   X  X  XXX  XXX   "],
+            [" XXX              XXXXX      x   x     x  xxxxx  xxx ",
+             " X  X  X   XXX       X       x   x x   x  x     x  x ",
+             " XXX                X        x   xxxx  x  xxxx   xxx ",
+             " X     X   XXX       X       x     x   x      x    x ",
+             " X     X          XXXX   x   x     x   x  xxxx     x "]]
+    loc, feat = [], []
+    for b, msg in enumerate(msgs):
+        for y, line in enumerate(msg):
+            for x, c in enumerate(line):
+                if c == 'X':
+                    loc.append([y, x, b])
+                    feat.append([1.0])
+    inp = scn.InputLayer(2, size)([torch.LongTensor(loc), torch.FloatTensor(feat).cuda()])
+    assert inp.batch_size() == 2 and inp.features.shape == (len(loc), 1)
+    assert (inp.get_spatial_locations() == torch.LongTensor(loc)).all()
+    with torch.no_grad():
+        out = model(inp)
+    assert tuple(out.shape) == (2, 32, 10, 10) and out.is_cuda
+    assert torch.isfinite(out).all() and (out >= 0).all() and out.abs().sum() > 0
+
+
+def _run_both(model, inp_layer, x):
+    p = cpu_path.CpuPath(inp_layer.dimension, "oracle")
+    t = oracle_model.run(inp_layer, p, x)
+    want = oracle_model.run(model, p, t)
+    with torch.no_grad():
+        got = model.cuda()(inp_layer([x[0], x[1].cuda()]))
+    return got, want, p
+
+
+def test_unet_vs_oracle(oracle_built):
+    """Configuration 5 at reduced width and size: InputLayer mode 4 (duplicates averaged),
+    SubmanifoldConvolution 3->8, UNet(reps=2, 4 levels), OutputLayer, Linear."""
+    torch.manual_seed(5)
+    m = 8
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m], False)).add(scn.OutputLayer(3)).eval()
+    randomise_bn(model, 5)
+    linear = torch.nn.Linear(m, 20)
+    coords = synthetic.scene_batch(seed=5000, batch=2, target=6000, spatial=64, n_boxes=8,
+                                   duplicate_fraction=0.3)
+    rng = np.random.default_rng(5)
+    feats = rng.uniform(-1, 1, size=(len(coords), 3)).astype(np.float32)
+    inp_layer = scn.InputLayer(3, 64, mode=4)
+    x = [torch.as_tensor(coords), torch.as_tensor(feats)]
+    got, want, p = _run_both(model, inp_layer, x)
+    assert got.shape == (len(coords), m)
+    checks.assert_close(got.cpu().numpy(), want, "U-Net output rows")
+    with torch.no_grad():
+        logits = linear.cuda()(got)
+    assert logits.shape == (len(coords), 20)
+
+
+def test_vgg2d_vs_oracle(oracle_built):
+    torch.manual_seed(2)
+    model = hello_world_model().eval()
+    randomise_bn(model, 2)
+    coords = synthetic.strokes2d(seed=2000, batch=100, canvas=64, spatial=71)
+    feats = np.ones((len(coords), 1), np.float32)
+    inp_layer = scn.InputLayer(2, 71, mode=3)
+    got, want, _ = _run_both(model, inp_layer, [torch.as_tensor(coords), torch.as_tensor(feats)])
+    assert tuple(got.shape) == (100, 32, 8, 8)
+    checks.assert_close(got.cpu().numpy(), want, "2-D VGG dense output")
+
+
+def test_training_mode_and_backward_are_refused():
+    bn = scn.BatchNormReLU(4).cuda()
+    t = scn.InputLayer(2, 8)([torch.LongTensor([[1, 1, 0]]), torch.ones(1, 4).cuda()])
+    with pytest.raises(NotImplementedError):
+        bn(t)  # training mode
+    conv = scn.SubmanifoldConvolution(2, 4, 4, 3, False).cuda()
+    y = conv(t).features
+    assert y.requires_grad
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        y.sum().backward()
+
+
+def test_empty_input_passes_through():
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, 4, 3, False)).add(scn.BatchNormReLU(4)).cuda().eval()
+    t = scn.InputLayer(3, 16, mode=4)([torch.zeros((0, 4), dtype=torch.int64), torch.zeros((0, 3)).cuda()])
+    with torch.no_grad():
+        out = model(t)
+    assert out.features.shape == (0, 4)
