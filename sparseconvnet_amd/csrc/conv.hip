@@ -71,6 +71,26 @@ __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n
   wp[i] = v;
 }
 
+// Packs rows [0, n_in_part) of every tap's weight slice, where the slice of tap k starts at
+// w + k * w_rows * n_out (w already points at the first row of the range), as one slab per tap
+// in the layout of k_pack_weights.
+__global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows, int n_in_part, int n_out,
+                                    int SS, int NCB) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)K * SS * NCB * 256;
+  if (i >= total) return;
+  int e = (int)(i % (SS * NCB * 256));
+  int k = (int)(i / (SS * NCB * 256));
+  int jj = e & 3;
+  int lane = (e >> 2) & 63;
+  int q = e >> 8;
+  int cb = q % NCB;
+  int s = q / NCB;
+  int ch = s * 16 + 4 * (lane >> 4) + jj;
+  int col = 16 * cb + (lane & 15);
+  wp[i] = (ch < n_in_part && col < n_out) ? w[((int64_t)k * w_rows + ch) * n_out + col] : 0.0f;
+}
+
 // ---- MFMA kernel ------------------------------------------------------------------------
 // A workgroup of 4 wavefronts owns a tile of G = GW*WR granules (16 rows each).  The
 // wavefronts form a WR x WC grid: wavefront (wr, wc) keeps, in registers, the accumulators
@@ -326,11 +346,253 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
   return false;
 }
 
+// ---- resident-weights kernel for narrow layers ------------------------------------------
+// When the packed weights of all taps fit in LDS (K * ceil(nIn/16) * NCB KiB), a persistent
+// workgroup loads them once and its wavefronts then work independently, with no barrier:
+// each takes sets of RG granules, keeps their accumulators in registers, and walks the taps
+// that any of its 64 rows has (a bit mask scanned with ffs).  The walk is a three-stage
+// register pipeline: neighbour indices of tap i+2 and input rows of tap i+1 are in flight
+// while tap i runs its MFMAs; all loads are unconditional (absent rows read row 0 and are
+// zeroed by a select), past the last tap the pipeline reloads the last tap.  Granules none
+// of whose rows has the tap skip their MFMAs.
+// With accumulate != 0 the kernel adds to `out` instead of overwriting it (used to split a
+// wide nIn into several launches).
+template <int NCB, int RG, int SS, bool VEC4, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
+    const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
+    const float *__restrict__ in, int in_stride, float *__restrict__ out, const float *__restrict__ wp,
+    const float *__restrict__ bias, int n_in, int n_out, int n_sets, int sets_per_xcd, int accumulate) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  v4f *wl = reinterpret_cast<v4f *>(lds);  // [K][SS][NCB][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int total_f4 = K * SS * NCB * 64;
+  for (int e = threadIdx.x; e < total_f4; e += WAVES * 64) wl[e] = reinterpret_cast<const v4f *>(wp)[e];
+  __syncthreads();  // the only barrier; every wavefront reaches it
+
+  float bv[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; cb++) {
+    const int col = 16 * cb + r16;
+    bv[cb] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+  }
+  // Sets are dealt so that one XCD (blocks b, b+8, ...) walks a contiguous range.
+  const int xcd = blockIdx.x & 7, blk = blockIdx.x >> 3, blocks_per_xcd = gridDim.x >> 3;
+  for (int ls = blk * WAVES + wave; ls < sets_per_xcd; ls += blocks_per_xcd * WAVES) {
+    const int set = xcd * sets_per_xcd + ls;
+    if (set >= n_sets) break;
+    const int64_t t0 = (int64_t)set * (RG * 16);
+    // which taps does any row of the set have?  lane group g looks at taps 4*kk + g
+    unsigned tapmask = 0;
+    for (int kb = 0; kb < K; kb += 4) {
+      const int k = kb + g;
+      bool any = false;
+#pragma unroll
+      for (int q = 0; q < RG; q++) {
+        const int64_t t = t0 + q * 16 + r16;
+        if (k < K && t < n) any |= nbr[(int64_t)k * npad + t] >= 0;
+      }
+      const unsigned long long bal = __ballot(any);
+#pragma unroll
+      for (int gg = 0; gg < 4; gg++)
+        if ((bal >> (16 * gg)) & 0xFFFFull) tapmask |= 1u << (kb + gg);
+    }
+    tapmask = __builtin_amdgcn_readfirstlane(tapmask);
+    const int ntaps = __popc(tapmask);
+
+    v4f acc[RG][NCB];
+#pragma unroll
+    for (int q = 0; q < RG; q++)
+#pragma unroll
+      for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    if (ntaps > 0) {
+      int64_t tq[RG];
+#pragma unroll
+      for (int q = 0; q < RG; q++) tq[q] = min(t0 + q * 16 + r16, n - 1);
+      unsigned rest = tapmask;
+      auto next_tap = [&]() {  // next set bit; sticks at the last one
+        const int k = __ffs(rest) - 1;
+        if (rest & (rest - 1)) rest &= rest - 1;
+        return k;
+      };
+      auto load_j = [&](int k, int *j) {
+#pragma unroll
+        for (int q = 0; q < RG; q++) j[q] = nbr[(int64_t)k * npad + tq[q]];
+      };
+      auto load_a = [&](const int *j, v4f (*a)[SS]) {
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+          const float *src = in + (int64_t)(j[q] < 0 ? 0 : j[q]) * in_stride;
+#pragma unroll
+          for (int s = 0; s < SS; s++) {
+            const int c0 = s * 16 + 4 * g;
+            if (VEC4) {
+              const int cc = c0 < n_in ? c0 : n_in - 4;
+              a[q][s] = *reinterpret_cast<const v4f *>(src + cc);
+            } else {
+              a[q][s].x = src[min(c0 + 0, n_in - 1)];
+              a[q][s].y = src[min(c0 + 1, n_in - 1)];
+              a[q][s].z = src[min(c0 + 2, n_in - 1)];
+              a[q][s].w = src[min(c0 + 3, n_in - 1)];
+            }
+          }
+        }
+      };
+      int k_cur, k_nxt, k_nn;
+      int j_nxt[RG], j_nn[RG], j_cur[RG];
+      v4f a_nxt[RG][SS], a_cur[RG][SS];
+      k_nxt = next_tap();
+      load_j(k_nxt, j_nxt);
+      k_nn = next_tap();
+      load_j(k_nn, j_nn);
+      load_a(j_nxt, a_nxt);
+      for (int i = 0; i < ntaps; i++) {
+        k_cur = k_nxt;
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+          j_cur[q] = (t0 + q * 16 + r16 < n) ? j_nxt[q] : -1;
+#pragma unroll
+          for (int s = 0; s < SS; s++) a_cur[q][s] = a_nxt[q][s];
+        }
+        // advance the pipeline: rows of the next tap, indices of the one after
+        k_nxt = k_nn;
+#pragma unroll
+        for (int q = 0; q < RG; q++) j_nxt[q] = j_nn[q];
+        load_a(j_nxt, a_nxt);
+        k_nn = next_tap();
+        load_j(k_nn, j_nn);
+
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+          const bool ok = j_cur[q] >= 0;
+          if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
+#pragma unroll
+          for (int s = 0; s < SS; s++) {
+            const int c0 = s * 16 + 4 * g;
+            v4f av = a_cur[q][s];
+            if (VEC4) {
+              if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
+            } else {
+              if (!(ok && c0 + 0 < n_in)) av.x = 0.f;
+              if (!(ok && c0 + 1 < n_in)) av.y = 0.f;
+              if (!(ok && c0 + 2 < n_in)) av.z = 0.f;
+              if (!(ok && c0 + 3 < n_in)) av.w = 0.f;
+            }
+            v4f b[NCB];
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) b[cb] = wl[((k_cur * SS + s) * NCB + cb) * 64 + lane];
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[cb].x, acc[q][cb], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[cb].y, acc[q][cb], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[cb].z, acc[q][cb], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[cb].w, acc[q][cb], 0, 0, 0);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < RG; q++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int64_t pos = t0 + q * 16 + 4 * g + r;
+        if (pos >= n) continue;
+        const int64_t row = rowmap ? rowmap[pos] : pos;
+        float *o = out + row * n_out;
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) {
+          const int col = 16 * cb + r16;
+          if (col < n_out) o[col] = acc[q][cb][r] + (accumulate ? o[col] : bv[cb]);
+        }
+      }
+    }
+  }
+}
+
+// One launch over channels [c_lo, c_lo + n_in_part) of the input rows.
+template <int NCB, int SS, bool VEC4>
+static void launch_resident_part(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
+                                 const float *w, int w_in_stride_rows, const float *bias, int n_in_part,
+                                 int n_out, int accumulate, hipStream_t s) {
+  constexpr int RG = 4;
+  const int64_t packed = (int64_t)t.K * SS * NCB * 256;
+  m.wpack.reserve(packed);
+  // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
+  k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, w_in_stride_rows,
+                                                                           n_in_part, n_out, SS, NCB);
+  LAUNCH_CHECK();
+  const size_t lds_bytes = (size_t)packed * sizeof(float);
+  const int n_sets = (int)ceil_div(t.n, RG * 16);
+  const int sets_per_xcd = (int)ceil_div(n_sets, 8);
+  if (lds_bytes > 80 * 1024) {
+    constexpr int WAVES = 12;  // 3 wavefronts per SIMD: up to 170 registers each, no spills
+    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      attr_set = true;
+    }
+    const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32, ceil_div(sets_per_xcd, WAVES)));
+    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
+                                                     m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
+                                                     accumulate);
+  } else {
+    constexpr int WAVES = 8;
+    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      attr_set = true;
+    }
+    const int per_cu = lds_bytes > 40 * 1024 ? 1 : (lds_bytes > 20 * 1024 ? 2 : 4);
+    const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
+    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
+                                                     m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
+                                                     accumulate);
+  }
+  LAUNCH_CHECK();
+}
+
+// Narrow layers: nOut <= 32, any nIn, K <= 32.  nIn is processed in parts of up to 32
+// channels so that every part's weights fit in LDS; parts after the first accumulate.
+static bool try_resident(Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                         const float *bias, int n_in, int n_out, hipStream_t s) {
+  if (t.K > 32 || n_out > 32) return false;
+  const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
+  const int ncb = (int)ceil_div(n_out, 16);
+  for (int c_lo = 0; c_lo < n_in; c_lo += 32) {
+    const int part = std::min(32, n_in - c_lo);
+    const float *in_p = in + c_lo;
+    const float *w_p = w + (int64_t)c_lo * n_out;
+    const int acc = c_lo > 0;
+    const float *b = acc ? nullptr : bias;
+#define SCN_RES(NCBV, SSV)                                                                               \
+  do {                                                                                                   \
+    if (vec4)                                                                                            \
+      launch_resident_part<NCBV, SSV, true>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc, s);   \
+    else                                                                                                 \
+      launch_resident_part<NCBV, SSV, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc, s);  \
+  } while (0)
+    if (ncb == 1 && part <= 16) SCN_RES(1, 1);
+    else if (ncb == 1) SCN_RES(1, 2);
+    else if (part <= 16) SCN_RES(2, 1);
+    else SCN_RES(2, 2);
+#undef SCN_RES
+  }
+  return true;
+}
+
 void conv_forward(Metadata &m, const Table &t, const float *in, float *out, const float *w, const float *bias,
                   int n_in, int n_out, int groups, hipStream_t s) {
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
+  if (groups == 1 && try_resident(m, t, in, out, w, bias, n_in, n_out, s)) return;
   if (groups == 1 && t.K <= 1024) {
     const int ncb = (int)ceil_div(n_out, 16);
     const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);

@@ -565,27 +565,33 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
                                const int *head_scan, int64_t n_cand, int64_t npad_out, int *by_out,
                                int *by_in, int *out_soa, unsigned long long *out_keys,
                                unsigned long long *counts) {
+  extern __shared__ int lcount[];  // per-block rule counts, flushed with one atomic per tap
+  for (int k = threadIdx.x; k < f.K; k += blockDim.x) lcount[k] = 0;
+  __syncthreads();
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= n_cand) return;
-  unsigned long long key = skeys[p];
-  if (key == SCN_EMPTY_KEY) return;
-  int e = spayload[p];
-  int t = e / f.M, m = e - t * f.M;
-  int row = sched ? sched[t] : t;
-  int pc[SCN_MAXD], j[SCN_MAXD];
-  for (int d = 0; d < f.dim; d++) pc[d] = soa[d * npad_in + row];
-  candidate(gi, f, pc, m, j);
-  int k = 0;
-  for (int d = 0; d < f.dim; d++) k = k * f.size[d] + (pc[d] - j[d] * f.stride[d]);
-  int o = head_scan[p] + head[p] - 1;
-  by_out[(int64_t)k * npad_out + o] = row;
-  by_in[(int64_t)k * npad_in + t] = o;
-  atomicAdd(&counts[k], 1ull);
-  if (head[p]) {
-    for (int d = 0; d < f.dim; d++) out_soa[d * npad_out + o] = j[d];
-    out_soa[f.dim * npad_out + o] = soa[f.dim * npad_in + row];
-    out_keys[o] = key;
+  unsigned long long key = p < n_cand ? skeys[p] : SCN_EMPTY_KEY;
+  if (key != SCN_EMPTY_KEY) {
+    int e = spayload[p];
+    int t = e / f.M, m = e - t * f.M;
+    int row = sched ? sched[t] : t;
+    int pc[SCN_MAXD], j[SCN_MAXD];
+    for (int d = 0; d < f.dim; d++) pc[d] = soa[d * npad_in + row];
+    candidate(gi, f, pc, m, j);
+    int k = 0;
+    for (int d = 0; d < f.dim; d++) k = k * f.size[d] + (pc[d] - j[d] * f.stride[d]);
+    int o = head_scan[p] + head[p] - 1;
+    by_out[(int64_t)k * npad_out + o] = row;
+    by_in[(int64_t)k * npad_in + t] = o;
+    atomicAdd(&lcount[k], 1);
+    if (head[p]) {
+      for (int d = 0; d < f.dim; d++) out_soa[d * npad_out + o] = j[d];
+      out_soa[f.dim * npad_out + o] = soa[f.dim * npad_in + row];
+      out_keys[o] = key;
+    }
   }
+  __syncthreads();
+  for (int k = threadIdx.x; k < f.K; k += blockDim.x)
+    if (lcount[k]) atomicAdd(&counts[k], (unsigned long long)lcount[k]);
 }
 
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
@@ -654,7 +660,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   fill32(R.by_in.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LI.npad, s);
   m.dcounts.reserve(4096);
   fill32(m.dcounts.p, 0, 2 * f.K, s);
-  k_strided_emit<<<grid_for(nc), TB, 0, s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), LI.npad, m.k1.p, m.v1.p,
+  k_strided_emit<<<grid_for(nc), TB, f.K * sizeof(int), s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), LI.npad, m.k1.p, m.v1.p,
                                              m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
                                              LO.coords.p, LO.keys.p, (unsigned long long *)m.dcounts.p);
   LAUNCH_CHECK();
