@@ -11,6 +11,63 @@ struct scn_metadata {
 
 static thread_local std::string g_error;
 
+// ---- block cache behind DevBuf (see common.h) -----------------------------------------------
+#include <map>
+#include <mutex>
+
+namespace scn {
+namespace {
+std::mutex g_pool_mutex;
+std::multimap<std::pair<int, size_t>, void *> g_pool;  // (device, size class) -> free blocks
+
+int current_device() {
+  int d = 0;
+  (void)hipGetDevice(&d);
+  return d;
+}
+
+// Size classes: multiples of an eighth of the next power of two (at most 12.5% slack).
+size_t size_class(size_t bytes) {
+  size_t p2 = 4096;
+  while (p2 < bytes) p2 <<= 1;
+  size_t step = p2 / 8;
+  return (bytes + step - 1) / step * step;
+}
+}  // namespace
+
+void *pool_alloc(size_t bytes) {
+  const size_t cls = size_class(bytes ? bytes : 1);
+  {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    auto it = g_pool.find(std::make_pair(current_device(), cls));
+    if (it != g_pool.end()) {
+      void *p = it->second;
+      g_pool.erase(it);
+      return p;
+    }
+  }
+  void *p = nullptr;
+  hipError_t e = hipMalloc(&p, cls);
+  if (e != hipSuccess) {
+    // give cached blocks back to the driver and try once more
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    for (auto &kv : g_pool) (void)hipFree(kv.second);
+    g_pool.clear();
+    (void)hipGetLastError();
+    HIP_CHECK(hipMalloc(&p, cls));
+  }
+  return p;
+}
+
+void pool_free(void *p, size_t bytes) {
+  if (!p) return;
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  hipPointerAttribute_t attr;
+  int dev = hipPointerGetAttributes(&attr, p) == hipSuccess ? attr.device : current_device();
+  g_pool.emplace(std::make_pair(dev, size_class(bytes ? bytes : 1)), p);
+}
+}  // namespace scn
+
 template <class F> static int guarded(F f) {
   try {
     f();

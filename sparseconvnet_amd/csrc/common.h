@@ -30,6 +30,14 @@ inline void hip_check(hipError_t e, const char *what, const char *file, int line
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 
+// Device memory for the library's own buffers comes from a process-wide cache: blocks freed
+// by one metadata object are handed to the next instead of going back to the driver, so a
+// steady stream of scenes performs no hipMalloc / hipFree (each of which stalls the host,
+// and hipFree the whole device).  Blocks are reused in the order work is enqueued: callers
+// that drive one process from several streams must order those streams themselves.
+void *pool_alloc(size_t bytes);
+void pool_free(void *p, size_t bytes);
+
 // Owning device buffer.  Grows by reallocation (contents discarded).
 template <class T> struct DevBuf {
   T *p = nullptr;
@@ -50,14 +58,14 @@ template <class T> struct DevBuf {
   }
   ~DevBuf() { release(); }
   void release() {
-    if (p) (void)hipFree(p);
+    if (p) pool_free(p, cap * sizeof(T));
     p = nullptr;
     cap = 0;
   }
   void reserve(size_t n) {
     if (n <= cap) return;
     release();
-    HIP_CHECK(hipMalloc((void **)&p, n * sizeof(T)));
+    p = static_cast<T *>(pool_alloc(n * sizeof(T)));
     cap = n;
   }
   size_t bytes() const { return cap * sizeof(T); }

@@ -455,7 +455,6 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
                                                      t.rowmap.p);
   LAUNCH_CHECK();
-  HIP_CHECK(hipStreamSynchronize(s));  // the old table is freed when nbr2 replaces it
   t.nbr = std::move(nbr2);
   t.identity_rows = false;
 }
