@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_FP32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PAIRS = [(3, 32), (32, 32), (64, 64), (128, 128), (256, 256)]
+# HBM-side bytes per launch on the default workload (1,000,000 sites, seed 3000, shuffled), from
+# rocprofv3 FETCH_SIZE / WRITE_SIZE passes scaled by a 1 GiB copy kernel (x2.000 / x1.000):
+# profiles/conv256_sweep1M_pmc.txt.  Only reported when the run is that workload.
+MEASURED_TRAFFIC = {(256, 256): 25.93e9, (128, 128): 3.43e9, (64, 64): 0.66e9, (32, 32): 0.46e9, (3, 32): 0.40e9}
 
 
 def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
@@ -33,7 +37,7 @@ def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
     return R * cin * s + 8 * R + n_out_rows * cout * s + K * cin * cout * s
 
 
-def roofline_for(cin, cout, R, n, K, ms):
+def roofline_for(cin, cout, R, n, K, ms, traffic=None):
     flops = 2.0 * R * cin * cout
     byts = conv_bytes(R, n, K, cin, cout)
     t_mfma = flops / (MFMA_FP32_TFLOPS * 1e12)
@@ -41,10 +45,10 @@ def roofline_for(cin, cout, R, n, K, ms):
     if t_mfma >= t_hbm:
         ach = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_FP32_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(ach / MFMA_FP32_TFLOPS, 4), "traffic": None}
+                "frac": round(ach / MFMA_FP32_TFLOPS, 4), "traffic": traffic}
     ach = byts / (ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
+            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic}
 
 
 def cpu_baseline(sample_sites, seed):
@@ -137,6 +141,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pairs", default="")
     ap.add_argument("--no-unet", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy 3 times, to scale profiler byte counters")
     ap.add_argument("--unet-sites", type=int, default=1000000)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -212,12 +218,14 @@ def main():
     total_flops = sum(2.0 * R * cin * cout for cin, cout in pairs)
     value = total_flops / (ms_per_step * 1e-3) / 1e9
 
+    default_workload = args.sites == 1000000 and args.seed == 3000 and args.order == "shuffled"
     sweep = []
     for (cin, cout), ms in zip(pairs, per_pair_ms):
         sweep.append({"nIn": cin, "nOut": cout, "ms": round(ms, 4),
                       "gflops": round(2.0 * R * cin * cout / (ms * 1e-3) / 1e9, 1),
                       "sites_per_s": round(n / (ms * 1e-3)),
-                      "roofline": roofline_for(cin, cout, R, n, 27, ms)})
+                      "roofline": roofline_for(cin, cout, R, n, 27, ms,
+                                               MEASURED_TRAFFIC.get((cin, cout)) if default_workload else None)})
     dom = int(np.argmax(per_pair_ms))
     roof = dict(sweep[dom]["roofline"])
     roof["kernel"] = "submanifold conv %d->%d" % pairs[dom]
@@ -237,6 +245,13 @@ def main():
     }
     L.scn_md_destroy(h)
     del work
+    if args.calibrate_copy:
+        a = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     if not args.no_unet:
         out["unet"] = unet_scene(args.unet_sites, 5000)
     if not args.no_cpu:

@@ -247,13 +247,20 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     for (int s = 0; s < SS; s++)
 #pragma unroll
       for (int c = 0; c < NCBW; c++) b[s][c] = wb[(s * NCB + wc * NCBW + c) * 64 + lane];
+    // all A fragments of this wavefront's granules are fetched before the first MFMA, so that
+    // no MFMA waits on LDS
+    v4f afrag[GW][SS];
+#pragma unroll
+    for (int q = 0; q < GW; q++)
+#pragma unroll
+      for (int s = 0; s < SS; s++) afrag[q][s] = ab[((wr * GW + q) * SS + s) * 64 + lane];
 #pragma unroll
     for (int q = 0; q < GW; q++) {
       const int gr = wr * GW + q;
       if (!((gm_cur >> gr) & 1u)) continue;  // uniform over the workgroup
 #pragma unroll
       for (int s = 0; s < SS; s++) {
-        const v4f av = ab[(gr * SS + s) * 64 + lane];
+        const v4f av = afrag[q][s];
 #pragma unroll
         for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][c].x, acc[q][c], 0, 0, 0);
 #pragma unroll
