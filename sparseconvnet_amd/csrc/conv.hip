@@ -111,7 +111,8 @@ template <int NCBW, int WC, int GW, int SS, bool VEC4>
 __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
-    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles) {
+    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
+    int n_split, float *__restrict__ partial) {
   constexpr int WR = 4 / WC;
   constexpr int NCB = NCBW * WC;
   constexpr int G = GW * WR;
@@ -158,10 +159,13 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     }
   }
   __syncthreads();
+  // With n_split > 1 the taps of a tile are dealt over n_split workgroups (blockIdx.y), each
+  // of which writes a partial tile that k_conv_reduce sums: small levels have too few tiles
+  // to fill the GPU and too long a serial tap loop otherwise.
   if (threadIdx.x == 0) {
     int c = 0;
     for (int k = 0; k < K; k++)
-      if (gmask[k]) taplist[c++] = k;
+      if (gmask[k] && (n_split == 1 || k % n_split == (int)blockIdx.y)) taplist[c++] = k;
     *ntaps_p = c;
   }
   __syncthreads();
@@ -274,6 +278,17 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   }
 
   // acc[q][c][r] = result for position tbase + 16*(wr*GW+q) + 4*g + r, column 16*(wc*NCBW+c) + r16
+  if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
+    float *pt = partial + ((int64_t)blockIdx.y * n_tiles * TM + tbase) * (NCB * 16);
+#pragma unroll
+    for (int q = 0; q < GW; q++)
+#pragma unroll
+      for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int c = 0; c < NCBW; c++)
+          pt[(int64_t)((wr * GW + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * (wc * NCBW + c) + r16] = acc[q][c][r];
+    return;
+  }
   float bv[NCBW];
 #pragma unroll
   for (int c = 0; c < NCBW; c++) {
@@ -295,6 +310,19 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       }
     }
   }
+}
+
+// out[rowmap[pos]][col] = bias[col] + sum over splits of partial[split][pos][col]
+__global__ void k_conv_reduce(const float *partial, int n_split, int64_t split_stride, int ld, const int *rowmap,
+                              int64_t n, const float *bias, float *out, int n_out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * n_out) return;
+  int64_t pos = i / n_out;
+  int col = (int)(i - pos * n_out);
+  float acc = bias ? bias[col] : 0.0f;
+  for (int sp = 0; sp < n_split; sp++) acc += partial[sp * split_stride + pos * ld + col];
+  int64_t row = rowmap ? rowmap[pos] : pos;
+  out[row * n_out + col] = acc;
 }
 
 template <int NCBW, int WC, int GW, int SS, bool VEC4>
@@ -322,10 +350,24 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   }
   const int n_tiles = (int)ceil_div(t.n, G * 16);
   const int tiles_per_xcd = (int)ceil_div(n_tiles, 8);
-  kern<<<dim3((unsigned)(tiles_per_xcd * 8)), 256, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in,
-                                                                   out, m.wpack.p, bias, n_in, n_out, n_slab,
-                                                                   tiles_per_xcd, n_tiles);
+  // Few tiles: deal the taps of every tile over several workgroups (about two per CU in all).
+  int n_split = 1;
+  if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
+  float *partial = nullptr;
+  const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
+  if (n_split > 1) {
+    m.partial.reserve((size_t)n_split * split_stride);
+    partial = m.partial.p;
+  }
+  kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), 256, lds_bytes, s>>>(
+      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, tiles_per_xcd,
+      n_tiles, n_split, partial);
   LAUNCH_CHECK();
+  if (n_split > 1) {
+    k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
+                                                                          t.rowmap_ptr(), t.n, bias, out, n_out);
+    LAUNCH_CHECK();
+  }
   return true;
 }
 

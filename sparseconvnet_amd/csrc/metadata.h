@@ -78,7 +78,8 @@ struct Metadata {
   DevBuf<int> v0, v1, f0, f1, s0, s1;
   DevBuf<long long> dcounts;
   DevBuf<int> dflags;
-  DevBuf<float> wpack;  // weights of the running convolution in MFMA operand order
+  DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
+  DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
 };
 
 SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);
