@@ -566,7 +566,7 @@ template <int NCB, int SS, bool VEC4>
 static void launch_resident_part(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
                                  const float *w, int w_in_stride_rows, const float *bias, int n_in_part,
                                  int n_out, int accumulate, hipStream_t s) {
-  constexpr int RG = 4;
+  constexpr int RG = 2;  // 32 rows per set: measured faster than 64 (more wavefronts in flight)
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
   m.wpack.reserve(packed);
   // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
@@ -577,7 +577,7 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
   const int n_sets = (int)ceil_div(t.n, RG * 16);
   const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   if (lds_bytes > 80 * 1024) {
-    constexpr int WAVES = 12;  // 3 wavefronts per SIMD: up to 170 registers each, no spills
+    constexpr int WAVES = 16;
     auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -598,7 +598,7 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
       attr_set = true;
     }
-    const int per_cu = lds_bytes > 40 * 1024 ? 1 : (lds_bytes > 20 * 1024 ? 2 : 4);
+    const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / std::max<size_t>(lds_bytes, 1)));
     const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
     kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
                                                      m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
