@@ -129,21 +129,27 @@ __device__ inline uint64_t hash64(uint64_t k) {  // murmur3 finaliser
   return k;
 }
 
-// Open-addressing table entry: 16 bytes so that one probe is one aligned 128-bit load.
-struct __attribute__((aligned(16))) HashEntry {
-  unsigned long long key;
-  int row;
-  int pad;
+// Site lookup.  Sites of a level, sorted by key, are cut into blocks of 64 consecutive key
+// values (key >> 6: a 4x4x4 cell in 3-D, 8x8 in 2-D).  A block is one 32-byte entry of a small
+// open-addressing table: its key, the 64-bit occupancy mask of its sites and the rank of its
+// first site in the sorted order.  Looking a site up is one probe of that table (it holds
+// about N/16 entries for surfaces, so it stays in L2) plus a popcount:
+// rank = base + popcount(mask below the site's bit).  The 27 neighbours of a site fall into
+// at most 8 blocks, and consecutive taps usually share one.
+struct __attribute__((aligned(32))) BlockEntry {
+  unsigned long long key;   // block key = site key >> 6, or SCN_EMPTY_KEY
+  unsigned long long mask;  // bit i set: site with key (key << 6 | i) is active
+  int base;                 // rank of the block's first site among the level's distinct sites
+  int pad[3];
 };
 
-__device__ inline int hash_find(const HashEntry *table, uint64_t mask, uint64_t key) {
-  uint64_t b = hash64(key) & mask;
-  // The table is at most half full, so an empty slot ends every miss; the trip count is
-  // bounded by the table size all the same so that no wave can spin on a damaged table.
+// Slot of the block with key bkey, or -1.  The table is at most half full; the trip count is
+// bounded by the table size all the same so that no wave can spin on a damaged table.
+__device__ inline int64_t block_find(const BlockEntry *table, uint64_t mask, uint64_t bkey) {
+  uint64_t b = hash64(bkey) & mask;
   for (uint64_t i = 0; i <= mask; i++) {
-    const uint4 e = *reinterpret_cast<const uint4 *>(table + b);
-    unsigned long long k = ((unsigned long long)e.y << 32) | e.x;
-    if (k == key) return (int)e.z;
+    const unsigned long long k = table[b].key;
+    if (k == bkey) return (int64_t)b;
     if (k == SCN_EMPTY_KEY) return -1;
     b = (b + 1) & mask;
   }

@@ -23,9 +23,14 @@ struct Level {
   // caller's points came in.  Null when rows are already numbered by ascending key.
   DevBuf<int> sched;
   bool identity_sched = false;
-  DevBuf<HashEntry> table;  // key -> row, built on first use
+  // Site lookup (common.h: BlockEntry), built on first use: block table + row of every
+  // distinct site in key order.  `dups` marks levels whose keys may repeat (input-layer mode 0
+  // with repeated points: the last one wins, as with `mp[p] = i` in the reference).
+  DevBuf<BlockEntry> table;
   uint64_t mask = 0;
-  bool hash_built = false;
+  DevBuf<int> urow;
+  bool grid_built = false;
+  bool dups = false;
   const int *sched_ptr() const { return identity_sched ? nullptr : sched.p; }
 };
 

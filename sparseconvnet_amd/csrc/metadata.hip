@@ -92,7 +92,7 @@ static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
   l.batch = batch;
   l.coords.reserve((size_t)(g.dim + 1) * l.npad);
   l.keys.reserve((size_t)l.npad);
-  l.hash_built = false;
+  l.grid_built = false;
 }
 
 // ---- input layer -----------------------------------------------------------------------
@@ -229,6 +229,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
     alloc_level(L, g, n, batch);
     L.sched.reserve(n);
     L.identity_sched = false;
+    L.dups = true;  // mode 0 does not merge repeated points
     k_input_rows_identity<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, L.npad, L.coords.p);
     LAUNCH_CHECK();
     HIP_CHECK(hipMemcpyAsync(L.keys.p, m.k0.p, n * sizeof(unsigned long long), hipMemcpyDeviceToDevice, s));
@@ -316,37 +317,117 @@ void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStr
   LAUNCH_CHECK();
 }
 
-// ---- hash table of a level -------------------------------------------------------------
+// ---- site lookup of a level -------------------------------------------------------------
 
-// Later rows win on equal keys, as repeated `mp[p] = i` does for input-layer mode 0
-// (Metadata/IOLayersRules.h:41,54); all other levels have distinct keys.
-__global__ void k_hash_insert(const unsigned long long *keys, int64_t n, HashEntry *table,
-                              unsigned long long mask) {
-  int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= n) return;
-  unsigned long long key = keys[r];
-  unsigned long long b = hash64(key) & mask;
+// skey[t] = key of the row at schedule position t (ascending).
+__global__ void k_sorted_keys(const unsigned long long *keys, const int *sched, int64_t n,
+                              unsigned long long *skey) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) skey[t] = keys[sched ? sched[t] : t];
+}
+// Distinct sites: flag the last position of every run of equal keys.
+__global__ void k_run_tails(const unsigned long long *skey, int64_t n, int *tail) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) tail[t] = (t == n - 1 || skey[t + 1] != skey[t]) ? 1 : 0;
+}
+// ukey[u], urow[u] for the u-th distinct site: the last row of its run wins
+// (Metadata/IOLayersRules.h:41,54: repeated `mp[p] = i`).
+__global__ void k_compact_sites(const unsigned long long *skey, const int *sched, const int *tail,
+                                const int *tail_scan, int64_t n, unsigned long long *ukey, int *urow) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n || !tail[t]) return;
+  int u = tail_scan[t];
+  ukey[u] = skey[t];
+  urow[u] = sched ? sched[t] : (int)t;
+}
+__global__ void k_copy_rows(const int *sched, int64_t n, int *urow) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) urow[t] = sched ? sched[t] : (int)t;
+}
+__global__ void k_block_heads(const unsigned long long *ukey, int64_t n, int *head) {
+  int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (u < n) head[u] = (u == 0 || (ukey[u] >> 6) != (ukey[u - 1] >> 6)) ? 1 : 0;
+}
+// Block heads claim a slot and record their rank.
+__global__ void k_block_insert(const unsigned long long *ukey, const int *head, int64_t n, BlockEntry *table,
+                               unsigned long long mask) {
+  int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (u >= n || !head[u]) return;
+  unsigned long long bkey = ukey[u] >> 6;
+  unsigned long long b = hash64(bkey) & mask;
   for (unsigned long long i = 0; i <= mask; i++) {
-    unsigned long long old = atomicCAS(&table[b].key, SCN_EMPTY_KEY, key);
-    if (old == SCN_EMPTY_KEY || old == key) {
-      atomicMax(&table[b].row, (int)r);
+    unsigned long long old = atomicCAS(&table[b].key, SCN_EMPTY_KEY, bkey);
+    if (old == SCN_EMPTY_KEY) {
+      table[b].base = (int)u;
       return;
     }
     b = (b + 1) & mask;
   }
 }
-static void ensure_hash(Level &L, hipStream_t s) {
-  if (L.hash_built) return;
+// Every distinct site sets its bit in its block's mask.
+__global__ void k_block_masks(const unsigned long long *ukey, int64_t n, BlockEntry *table,
+                              unsigned long long mask) {
+  int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (u >= n) return;
+  unsigned long long key = ukey[u];
+  int64_t slot = block_find(table, mask, key >> 6);
+  if (slot >= 0) atomicOr(&table[slot].mask, 1ull << (key & 63));
+}
+
+__global__ void k_block_zero_masks(BlockEntry *table, int64_t cap) {
+  int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < cap) table[b].mask = 0ull;
+}
+
+static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
+  if (L.grid_built) return;
+  const int64_t n = L.n;
+  int64_t U = n, nblocks = 0;
+  m.k0.reserve(n + 1);
+  m.k1.reserve(n + 1);
+  m.f0.reserve(n + 1);
+  m.s0.reserve(n + 1);
+  L.urow.reserve(std::max<int64_t>(n, 1));
+  unsigned long long *ukey = m.k0.p;
+  if (n) {
+    k_sorted_keys<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, m.k0.p);
+    LAUNCH_CHECK();
+    if (L.dups) {
+      k_run_tails<<<grid_for(n), TB, 0, s>>>(m.k0.p, n, m.f0.p);
+      LAUNCH_CHECK();
+      exclusive_scan(m, m.f0.p, m.s0.p, n, s);
+      k_compact_sites<<<grid_for(n), TB, 0, s>>>(m.k0.p, L.sched_ptr(), m.f0.p, m.s0.p, n, m.k1.p, L.urow.p);
+      LAUNCH_CHECK();
+      U = read_back(m.s0.p + (n - 1), s) + 1;  // the last position always ends a run
+      ukey = m.k1.p;
+    } else {
+      k_copy_rows<<<grid_for(n), TB, 0, s>>>(L.sched_ptr(), n, L.urow.p);
+      LAUNCH_CHECK();
+    }
+    k_block_heads<<<grid_for(U), TB, 0, s>>>(ukey, U, m.f0.p);
+    LAUNCH_CHECK();
+    exclusive_scan(m, m.f0.p, m.s0.p, U, s);
+    int last[2];
+    HIP_CHECK(hipMemcpyAsync(&last[0], m.s0.p + (U - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipMemcpyAsync(&last[1], m.f0.p + (U - 1), sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    nblocks = (int64_t)last[0] + last[1];
+  }
   uint64_t cap = 64;
-  while (cap < (uint64_t)L.n * 2) cap <<= 1;
+  while (cap < (uint64_t)nblocks * 2) cap <<= 1;
   L.table.reserve(cap);
   L.mask = cap - 1;
-  fill32(L.table.p, 0xFFFFFFFFu, (int64_t)cap * 4, s);  // key = EMPTY, row = -1
-  if (L.n) {
-    k_hash_insert<<<grid_for(L.n), TB, 0, s>>>(L.keys.p, L.n, L.table.p, L.mask);
+  // key = EMPTY (all ones); masks must start at zero
+  fill32(L.table.p, 0xFFFFFFFFu, (int64_t)cap * 8, s);
+  if (n) {
+    k_block_insert<<<grid_for(U), TB, 0, s>>>(ukey, m.f0.p, U, L.table.p, L.mask);
+    LAUNCH_CHECK();
+    k_block_zero_masks<<<grid_for((int64_t)cap), TB, 0, s>>>(L.table.p, (int64_t)cap);
+    LAUNCH_CHECK();
+    k_block_masks<<<grid_for(U), TB, 0, s>>>(ukey, U, L.table.p, L.mask);
     LAUNCH_CHECK();
   }
-  L.hash_built = true;
+  L.grid_built = true;
 }
 
 // ---- submanifold rules -----------------------------------------------------------------
@@ -360,8 +441,8 @@ struct Filt {
 // (Metadata/SubmanifoldConvolutionRules.h:11-45; taps enumerate the box row-major with the
 // last dimension fastest, Metadata/RectangularRegions.h:56-71).
 __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, int64_t n,
-                             int64_t npad, const HashEntry *table, unsigned long long mask,
-                             int *nbr, unsigned long long *counts) {
+                             int64_t npad, const BlockEntry *table, unsigned long long mask,
+                             const int *urow, int *nbr, unsigned long long *counts) {
   extern __shared__ int lcount[];
   for (int k = threadIdx.x; k < f.K; k += blockDim.x) lcount[k] = 0;
   __syncthreads();
@@ -374,6 +455,8 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
       tap[d] = 0;
     }
     int b = soa[g.dim * npad + row];
+    unsigned long long last_bkey = SCN_EMPTY_KEY, last_mask = 0;  // block of the previous tap
+    int last_base = 0;
     for (int k = 0; k < f.K; k++) {
       bool inside = true;
       for (int d = 0; d < g.dim; d++) {
@@ -381,7 +464,18 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
         if (q[d] < 0 || q[d] >= g.size[d]) inside = false;
       }
       int j = -1;
-      if (inside) j = hash_find(table, mask, site_key(g, q, b));
+      if (inside) {
+        const unsigned long long key = site_key(g, q, b);
+        const unsigned long long bkey = key >> 6;
+        if (bkey != last_bkey) {
+          last_bkey = bkey;
+          const int64_t slot = block_find(table, mask, bkey);
+          last_mask = slot >= 0 ? table[slot].mask : 0ull;
+          last_base = slot >= 0 ? table[slot].base : 0;
+        }
+        const unsigned long long bit = 1ull << (key & 63);
+        if (last_mask & bit) j = urow[last_base + __popcll(last_mask & (bit - 1))];
+      }
       nbr[(int64_t)k * npad + t] = j;
       if (j >= 0) atomicAdd(&lcount[k], 1);
       for (int d = g.dim - 1; d >= 0; d--) {  // next tap, last dimension fastest
@@ -503,14 +597,14 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
     return m.subm.emplace(key, std::move(t)).first->second;
   }
   Level &L = lit->second;
-  ensure_hash(L, s);
+  ensure_grid(m, L, s);
   t.n = L.n;
   t.npad = L.npad;
   t.nbr.reserve((size_t)f.K * t.npad);
   m.dcounts.reserve(4096);
   fill32(m.dcounts.p, 0, 2 * f.K, s);
   k_subm_rules<<<grid_for(L.n), TB, f.K * sizeof(int), s>>>(L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad,
-                                                            L.table.p, L.mask, t.nbr.p,
+                                                            L.table.p, L.mask, L.urow.p, t.nbr.p,
                                                             (unsigned long long *)m.dcounts.p);
   LAUNCH_CHECK();
   fetch_counts(m, t, s);
