@@ -98,7 +98,6 @@ static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
 // ---- input layer -----------------------------------------------------------------------
 
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
-// flags[1] = max sample index seen.
 __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols,
                              unsigned long long *keys, int *idx, int *flags) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -116,8 +115,6 @@ __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols
     atomicOr(&flags[0], 2);
     ok = false;
     b = 0;
-  } else {
-    atomicMax(&flags[1], (int)b);
   }
   if (!ok) {
     atomicOr(&flags[0], 1);
@@ -217,13 +214,16 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   LAUNCH_CHECK();
   sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s);
   int hflags[2];
+  unsigned long long top_key = 0;  // keys ascend with the sample index: the last one has the largest
   HIP_CHECK(hipMemcpyAsync(hflags, m.dflags.p, sizeof hflags, hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipMemcpyAsync(&top_key, m.k1.p + (n - 1), sizeof top_key, hipMemcpyDeviceToHost, s));
   HIP_CHECK(hipStreamSynchronize(s));
   if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
   if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");
+  const int top_batch = g.dim <= 3 ? (int)(top_key >> (g.dim * g.bits)) : (int)(top_key / (unsigned long long)g.vol);
   // Metadata/IOLayersRules.h:25,46-47,76-77: the batch is at least min_batch and grows to
   // the largest sample index + 1; without a sample column there is exactly one sample.
-  int batch = ncols == m.dim ? 1 : std::max(batch_floor, hflags[1] + 1);
+  int batch = ncols == m.dim ? 1 : std::max(batch_floor, top_batch + 1);
 
   if (mode == 0) {
     alloc_level(L, g, n, batch);
@@ -442,22 +442,33 @@ struct Filt {
 // last dimension fastest, Metadata/RectangularRegions.h:56-71).
 __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, int64_t n,
                              int64_t npad, const BlockEntry *table, unsigned long long mask,
-                             const int *urow, int *nbr, unsigned long long *counts) {
+                             const int *urow, int *nbr, unsigned long long *counts, int parts) {
+  // blockDim = 64 * parts: wavefront p of the block handles taps [p*K/parts, (p+1)*K/parts)
+  // (one slice of the first filter dimension) of the block's 64 positions.
   extern __shared__ int lcount[];
   for (int k = threadIdx.x; k < f.K; k += blockDim.x) lcount[k] = 0;
   __syncthreads();
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t < n) {
+  const int part = threadIdx.x >> 6;
+  int64_t t = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63);
+  const bool live = t < n;
+  if (!live) t = n - 1;  // idle lanes shadow the last position so that ballots see whole wavefronts
+  {
     int row = sched ? sched[t] : (int)t;
     int c[SCN_MAXD], tap[SCN_MAXD], q[SCN_MAXD];
-    for (int d = 0; d < g.dim; d++) {
-      c[d] = soa[d * npad + row];
-      tap[d] = 0;
+    const int per = f.K / parts;
+    const int k0 = part * per;
+    {
+      int r = k0;
+      for (int d = g.dim - 1; d >= 0; d--) {
+        tap[d] = r % f.size[d];
+        r /= f.size[d];
+      }
     }
+    for (int d = 0; d < g.dim; d++) c[d] = soa[d * npad + row];
     int b = soa[g.dim * npad + row];
     unsigned long long last_bkey = SCN_EMPTY_KEY, last_mask = 0;  // block of the previous tap
     int last_base = 0;
-    for (int k = 0; k < f.K; k++) {
+    for (int k = k0; k < k0 + per; k++) {
       bool inside = true;
       for (int d = 0; d < g.dim; d++) {
         q[d] = c[d] + tap[d] - f.size[d] / 2;
@@ -476,8 +487,9 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
         const unsigned long long bit = 1ull << (key & 63);
         if (last_mask & bit) j = urow[last_base + __popcll(last_mask & (bit - 1))];
       }
-      nbr[(int64_t)k * npad + t] = j;
-      if (j >= 0) atomicAdd(&lcount[k], 1);
+      if (live) nbr[(int64_t)k * npad + t] = j;
+      const unsigned long long hits = __ballot(live && j >= 0);
+      if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&lcount[k], __popcll(hits));
       for (int d = g.dim - 1; d >= 0; d--) {  // next tap, last dimension fastest
         if (++tap[d] < f.size[d]) break;
         tap[d] = 0;
@@ -488,7 +500,6 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
   for (int k = threadIdx.x; k < f.K; k += blockDim.x)
     if (lcount[k]) atomicAdd(&counts[k], (unsigned long long)lcount[k]);
 }
-
 
 // ---- pattern-sorted positions ----------------------------------------------------------
 
@@ -553,6 +564,74 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   t.identity_rows = false;
 }
 
+// Filter 3 in every dimension, dim 2 or 3 (the common case): the Morton key of a neighbour
+// is the OR of per-coordinate spread values, so each coordinate is spread three times per
+// site (for c-1, c, c+1) instead of once per tap, and the tap loop is fully unrolled.
+// One wavefront per slice of the first filter dimension, as in k_subm_rules.
+template <int DIM>
+__global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_t n, int64_t npad,
+                                const BlockEntry *table, unsigned long long mask, const int *urow, int *nbr,
+                                unsigned long long *counts) {
+  constexpr int K = DIM == 3 ? 27 : 9;
+  constexpr int PER = K / 3;
+  __shared__ int lcount[K];
+  if (threadIdx.x < K) lcount[threadIdx.x] = 0;
+  __syncthreads();
+  const int part = threadIdx.x >> 6;  // offset -1, 0, +1 along the first dimension
+  int64_t t = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63);
+  const bool live = t < n;
+  if (!live) t = n - 1;
+  const int row = sched ? sched[t] : (int)t;
+  unsigned long long sp[DIM][3];
+  bool okc[DIM][3];
+#pragma unroll
+  for (int d = 0; d < DIM; d++) {
+    const int c = soa[d * npad + row];
+#pragma unroll
+    for (int o = 0; o < 3; o++) {
+      const int v = c + o - 1;
+      okc[d][o] = v >= 0 && v < g.size[d];
+      const unsigned long long s = DIM == 3 ? spread3((unsigned)v) : spread2((unsigned)v);
+      sp[d][o] = s << (DIM - 1 - d);
+    }
+  }
+  const unsigned long long bpart = (unsigned long long)soa[DIM * npad + row] << (DIM * g.bits);
+  unsigned long long last_bkey = SCN_EMPTY_KEY, last_mask = 0;
+  int last_base = 0;
+#pragma unroll
+  for (int kk = 0; kk < PER; kk++) {
+    const int k = part * PER + kk;
+    // taps enumerate the box with the last dimension fastest
+    const int o1 = DIM == 3 ? kk / 3 : kk, o2 = kk % 3;
+    bool inside;
+    unsigned long long key;
+    if (DIM == 3) {
+      inside = okc[0][part] && okc[1][o1] && okc[2][o2];
+      key = bpart | sp[0][part] | sp[1][o1] | sp[2][o2];
+    } else {
+      inside = okc[0][part] && okc[1][o1];
+      key = bpart | sp[0][part] | sp[1][o1];
+    }
+    int j = -1;
+    if (inside) {
+      const unsigned long long bkey = key >> 6;
+      if (bkey != last_bkey) {
+        last_bkey = bkey;
+        const int64_t slot = block_find(table, mask, bkey);
+        last_mask = slot >= 0 ? table[slot].mask : 0ull;
+        last_base = slot >= 0 ? table[slot].base : 0;
+      }
+      const unsigned long long bit = 1ull << (key & 63);
+      if (last_mask & bit) j = urow[last_base + __popcll(last_mask & (bit - 1))];
+    }
+    if (live) nbr[(int64_t)k * npad + t] = j;
+    const unsigned long long hits = __ballot(live && j >= 0);
+    if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&lcount[k], __popcll(hits));
+  }
+  __syncthreads();
+  if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&counts[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
+}
+
 static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const int64_t *out_size) {
   Filt f{};
   f.dim = dim;
@@ -603,9 +682,27 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   t.nbr.reserve((size_t)f.K * t.npad);
   m.dcounts.reserve(4096);
   fill32(m.dcounts.p, 0, 2 * f.K, s);
-  k_subm_rules<<<grid_for(L.n), TB, f.K * sizeof(int), s>>>(L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad,
-                                                            L.table.p, L.mask, L.urow.p, t.nbr.p,
-                                                            (unsigned long long *)m.dcounts.p);
+  bool all3 = true;
+  for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
+  if (all3 && (m.dim == 2 || m.dim == 3)) {
+    if (m.dim == 3)
+      k_subm_rules_s3<3><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
+                                                           L.mask, L.urow.p, t.nbr.p,
+                                                           (unsigned long long *)m.dcounts.p);
+    else
+      k_subm_rules_s3<2><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
+                                                           L.mask, L.urow.p, t.nbr.p,
+                                                           (unsigned long long *)m.dcounts.p);
+    LAUNCH_CHECK();
+    fetch_counts(m, t, s);
+    finalize_table(m, t, L.sched_ptr(), s);
+    return m.subm.emplace(key, std::move(t)).first->second;
+  }
+  // one wavefront per slice of the first filter dimension when that divides the taps evenly
+  const int parts = (m.dim >= 2 && f.size[0] <= 4) ? f.size[0] : 1;
+  k_subm_rules<<<grid_for(L.n, 64), 64 * parts, f.K * sizeof(int), s>>>(
+      L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p, L.mask, L.urow.p, t.nbr.p,
+      (unsigned long long *)m.dcounts.p, parts);
   LAUNCH_CHECK();
   fetch_counts(m, t, s);
   finalize_table(m, t, L.sched_ptr(), s);
