@@ -395,6 +395,240 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
   return false;
 }
 
+// ---- row-owner kernel for mid-width layers ----------------------------------------------
+// NW wavefronts, each owning RG granules of a tile of NW*RG granules.  Only the weight slab
+// goes through (double-buffered) LDS; every wavefront gathers the input rows of its own
+// granules straight into A-operand registers, one (tap, slab) iteration ahead, and keeps its
+// granules' [16 x nOut] accumulators in registers.  Compared with k_conv_mfma the gathered
+// rows never touch LDS and one weight slab serves NW*RG*16 rows (up to 512), at the price of
+// uneven MFMA work between wavefronts, which three to four wavefronts per SIMD even out.
+template <int NCB, int RG, int SS, bool VEC4, int NW>
+__global__ __launch_bounds__(NW * 64) void k_conv_rows(
+    const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
+    const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
+    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
+    int n_split, float *__restrict__ partial) {
+  constexpr int NT = NW * 64;
+  constexpr int G = NW * RG;
+  constexpr int TM = G * 16;
+  constexpr int SLAB_F4 = SS * NCB * 64;
+  constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
+  constexpr int SLAB_STRIDE_F4 = ((SLAB_F4 + 255) / 256) * 256;  // as packed by k_pack_weights
+  constexpr int LDS_SLAB_F4 = WPT * NT;                         // >= SLAB_STRIDE_F4 not required
+  static_assert(G <= 32, "granule mask is 32 bits");
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  v4f *wbuf = reinterpret_cast<v4f *>(lds);                      // [2][LDS_SLAB_F4]
+  int *jtab = reinterpret_cast<int *>(wbuf + 2 * LDS_SLAB_F4);   // [G][K][16]
+  unsigned *gmask = reinterpret_cast<unsigned *>(jtab + G * K * 16);
+  int *taplist = reinterpret_cast<int *>(gmask + K);
+  int *ntaps_p = taplist + K;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+
+  const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+  if (tile >= n_tiles) return;
+  const int64_t tbase = (int64_t)tile * TM;
+
+  for (int k = threadIdx.x; k < K; k += NT) gmask[k] = 0u;
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < RG; q++) {
+    const int gr = wave * RG + q;
+    const int64_t t = tbase + gr * 16 + r16;
+    for (int kb = 0; kb < K; kb += 4) {
+      const int k = kb + g;
+      int j = -1;
+      if (k < K && t < n) j = nbr[(int64_t)k * npad + t];
+      if (k < K) jtab[(gr * K + k) * 16 + r16] = j;
+      const unsigned long long bal = __ballot(j >= 0);
+      if (lane == 0) {
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++)
+          if ((bal >> (16 * gg)) & 0xFFFFull) atomicOr(&gmask[kb + gg], 1u << gr);
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int c = 0;
+    for (int k = 0; k < K; k++)
+      if (gmask[k] && (n_split == 1 || k % n_split == (int)blockIdx.y)) taplist[c++] = k;
+    *ntaps_p = c;
+  }
+  __syncthreads();
+  const int total = *ntaps_p * n_slab;
+
+  v4f acc[RG][NCB];
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  v4f wreg[WPT];
+  v4f a_nxt[RG][SS], a_cur[RG][SS];
+  unsigned gm_nxt = 0, gm_cur = 0, ok_nxt = 0;
+  int sl_nxt = 0;
+
+  auto issue = [&](int it) {
+    const int ti = it / n_slab, sl = it - ti * n_slab;
+    const int k = taplist[ti];
+    gm_nxt = gmask[k];
+    sl_nxt = sl;
+    ok_nxt = 0;
+    const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
+#pragma unroll
+    for (int i = 0; i < WPT; i++) {
+      const int e = threadIdx.x + i * NT;
+      wreg[i] = wsrc[e < SLAB_F4 ? e : 0];
+    }
+#pragma unroll
+    for (int q = 0; q < RG; q++) {
+      const int j = jtab[((wave * RG + q) * K + k) * 16 + r16];
+      if (j >= 0) ok_nxt |= 1u << q;
+      const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
+#pragma unroll
+      for (int s = 0; s < SS; s++) {
+        const int c0 = (sl * SS + s) * 16 + 4 * g;
+        if (VEC4) {
+          const int cc = c0 < n_in ? c0 : n_in - 4;
+          a_nxt[q][s] = *reinterpret_cast<const v4f *>(src + cc);
+        } else {
+          a_nxt[q][s].x = src[min(c0 + 0, n_in - 1)];
+          a_nxt[q][s].y = src[min(c0 + 1, n_in - 1)];
+          a_nxt[q][s].z = src[min(c0 + 2, n_in - 1)];
+          a_nxt[q][s].w = src[min(c0 + 3, n_in - 1)];
+        }
+      }
+    }
+  };
+
+  if (total > 0) issue(0);
+  for (int it = 0; it < total; it++) {
+    v4f *wb = wbuf + (it & 1) * LDS_SLAB_F4;
+#pragma unroll
+    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * NT] = wreg[i];
+#pragma unroll
+    for (int q = 0; q < RG; q++) {
+      const bool ok = (ok_nxt >> q) & 1u;
+#pragma unroll
+      for (int s = 0; s < SS; s++) {
+        const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
+        v4f v = a_nxt[q][s];
+        if (VEC4) {
+          if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
+        } else {
+          if (!(ok && c0 + 0 < n_in)) v.x = 0.f;
+          if (!(ok && c0 + 1 < n_in)) v.y = 0.f;
+          if (!(ok && c0 + 2 < n_in)) v.z = 0.f;
+          if (!(ok && c0 + 3 < n_in)) v.w = 0.f;
+        }
+        a_cur[q][s] = v;
+      }
+    }
+    gm_cur = gm_nxt;
+    __syncthreads();  // slab of `it` visible; every wavefront is done with the other buffer
+    if (it + 1 < total) issue(it + 1);
+    if (((gm_cur >> (wave * RG)) & ((1u << RG) - 1u)) == 0u) continue;  // none of my granules has the tap
+#pragma unroll
+    for (int s = 0; s < SS; s++) {
+      v4f b[NCB];
+#pragma unroll
+      for (int cb = 0; cb < NCB; cb++) b[cb] = wb[(s * NCB + cb) * 64 + lane];
+#pragma unroll
+      for (int q = 0; q < RG; q++) {
+        if (!((gm_cur >> (wave * RG + q)) & 1u)) continue;  // uniform over the wavefront
+        const v4f av = a_cur[q][s];
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[cb].x, acc[q][cb], 0, 0, 0);
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[cb].y, acc[q][cb], 0, 0, 0);
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[cb].z, acc[q][cb], 0, 0, 0);
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[cb].w, acc[q][cb], 0, 0, 0);
+      }
+    }
+  }
+
+  if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
+    float *pt = partial + ((int64_t)blockIdx.y * n_tiles * TM + tbase) * (NCB * 16);
+#pragma unroll
+    for (int q = 0; q < RG; q++)
+#pragma unroll
+      for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++)
+          pt[(int64_t)((wave * RG + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * cb + r16] = acc[q][cb][r];
+    return;
+  }
+  float bv[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; cb++) {
+    const int col = 16 * cb + r16;
+    bv[cb] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+  }
+#pragma unroll
+  for (int q = 0; q < RG; q++) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int64_t pos = tbase + (wave * RG + q) * 16 + 4 * g + r;
+      if (pos >= n) continue;
+      const int64_t row = rowmap ? rowmap[pos] : pos;
+      float *o = out + row * n_out;
+#pragma unroll
+      for (int cb = 0; cb < NCB; cb++) {
+        const int col = 16 * cb + r16;
+        if (col < n_out) o[col] = acc[q][cb][r] + bv[cb];
+      }
+    }
+  }
+}
+
+template <int NCB, int RG, int SS, bool VEC4, int NW>
+static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                        const float *bias, int n_in, int n_out, hipStream_t s) {
+  constexpr int NT = NW * 64, G = NW * RG;
+  constexpr int SLAB_F4 = SS * NCB * 64;
+  constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
+  constexpr int SLAB_STRIDE = ((SLAB_F4 + 255) / 256) * 256 * 4;  // floats, as k_pack_weights lays slabs out
+  const size_t lds_bytes = (size_t)2 * WPT * NT * 16 + ((size_t)G * t.K * 16 + 2 * t.K + 4) * sizeof(int);
+  if (lds_bytes > 160 * 1024) return false;
+  const int cin16 = (int)ceil_div(n_in, 16);
+  const int n_slab = (int)ceil_div(cin16, SS);
+  const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
+  m.wpack.reserve(packed);
+  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
+                                                                      SS, NCB, SLAB_STRIDE);
+  LAUNCH_CHECK();
+  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  160 * 1024));
+    attr_set = true;
+  }
+  const int n_tiles = (int)ceil_div(t.n, G * 16);
+  const int tiles_per_xcd = (int)ceil_div(n_tiles, 8);
+  int n_split = 1;
+  if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
+  float *partial = nullptr;
+  const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
+  if (n_split > 1) {
+    m.partial.reserve((size_t)n_split * split_stride);
+    partial = m.partial.p;
+  }
+  kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), NT, lds_bytes, s>>>(
+      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, tiles_per_xcd,
+      n_tiles, n_split, partial);
+  LAUNCH_CHECK();
+  if (n_split > 1) {
+    k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
+                                                                          t.rowmap_ptr(), t.n, bias, out, n_out);
+    LAUNCH_CHECK();
+  }
+  return true;
+}
+
 // ---- resident-weights kernel for narrow layers ------------------------------------------
 // When the packed weights of all taps fit in LDS (K * ceil(nIn/16) * NCB KiB), a persistent
 // workgroup loads them once and its wavefronts then work independently, with no barrier:
@@ -636,12 +870,37 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
   return true;
 }
 
+// Mid-width layers (32 < nOut <= 128): row-owner kernel.  Measured best on the 1 M-site
+// scene: 8 wavefronts x 2 granules for nOut <= 64, 16 wavefronts x 1 granule above.
+template <bool VEC4>
+static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                          const float *bias, int n_in, int n_out, hipStream_t s) {
+  const int ncb = (int)ceil_div(n_out, 16);
+  const bool narrow = n_in <= 16;
+  if (ncb <= 4)
+    return narrow ? launch_rows<4, 2, 1, VEC4, 8>(m, t, in, out, w, bias, n_in, n_out, s)
+                  : launch_rows<4, 2, 2, VEC4, 8>(m, t, in, out, w, bias, n_in, n_out, s);
+  if (ncb <= 6)
+    return narrow ? launch_rows<6, 1, 1, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s)
+                  : launch_rows<6, 1, 2, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s);
+  if (ncb <= 8)
+    return narrow ? launch_rows<8, 1, 1, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s)
+                  : launch_rows<8, 1, 2, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s);
+  return false;
+}
+
 void conv_forward(Metadata &m, const Table &t, const float *in, float *out, const float *w, const float *bias,
                   int n_in, int n_out, int groups, hipStream_t s) {
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
   if (groups == 1 && try_resident(m, t, in, out, w, bias, n_in, n_out, s)) return;
+  if (groups == 1 && n_out <= 128 && t.K <= 1024) {
+    const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
+    if (vec4 ? dispatch_rows<true>(m, t, in, out, w, bias, n_in, n_out, s)
+             : dispatch_rows<false>(m, t, in, out, w, bias, n_in, n_out, s))
+      return;
+  }
   if (groups == 1 && t.K <= 1024) {
     const int ncb = (int)ceil_div(n_out, 16);
     const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
