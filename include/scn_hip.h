@@ -128,6 +128,27 @@ int scn_deconv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_
                    const int64_t *filter, const int64_t *stride, const float *in, float *out,
                    const float *weight, const float *bias, int n_in, int n_out, int groups,
                    void *stream, double *macs);
+/* Fused pairs: an eval-mode batch norm + leaky ReLU on the input rows followed by one of the
+ * three convolutions above, i.e. BatchNormalization_updateOutput(train=false) (pybind.cpp:220,
+ * CPU/BatchNormalization.cpp:41-61) then the convolution, without writing the normalised rows
+ * to memory.  This is the order of every U-Net block (networkArchitectures.py:232-234).
+ * Same arguments as the plain calls plus the batch-norm tensors (device, [n_in]; gamma/beta
+ * may be NULL).  Results equal the two separate calls up to fp32 rounding. */
+int scn_bn_subm_conv_fwd(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
+                         const float *in, float *out, const float *weight, const float *bias,
+                         int n_in, int n_out, int groups, const float *running_mean,
+                         const float *running_var, const float *gamma, const float *beta, float eps,
+                         float leakiness, void *stream, double *macs);
+int scn_bn_conv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                    const int64_t *filter, const int64_t *stride, const float *in, float *out,
+                    const float *weight, const float *bias, int n_in, int n_out, int groups,
+                    const float *running_mean, const float *running_var, const float *gamma,
+                    const float *beta, float eps, float leakiness, void *stream, double *macs);
+int scn_bn_deconv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                      const int64_t *filter, const int64_t *stride, const float *in, float *out,
+                      const float *weight, const float *bias, int n_in, int n_out, int groups,
+                      const float *running_mean, const float *running_var, const float *gamma,
+                      const float *beta, float eps, float leakiness, void *stream, double *macs);
 /* MaxPooling_updateOutput (pybind.cpp:103-107, CPU/MaxPooling.cpp:37-60).
  * in [nActive(in_size), in_stride] -> out [nActive(out_size), planes] where
  * planes = in_stride - n_features_to_drop; the result is max(0, inputs of the window). */

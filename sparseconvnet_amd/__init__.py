@@ -7,6 +7,10 @@ as scn`).  The modules call hand-written gfx950 kernels in libscn_hip.so through
 # and output elements of the convolutions run so far.
 forward_pass_multiplyAdd_count = 0
 forward_pass_hidden_states = 0
+# Sequential hands an eval-mode batch normalisation that sits directly in front of a
+# convolution to that convolution (one pass over the rows instead of two).  False: run
+# every module as a pass of its own.
+fuse_batchnorm = True
 
 from .containers import AddTable, ConcatTable, JoinTable, Sequential  # noqa: E402
 from .layers import (BatchNormalization, BatchNormLeakyReLU, BatchNormReLU, Convolution,  # noqa: E402

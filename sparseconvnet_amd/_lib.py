@@ -38,6 +38,14 @@ SIGNATURES = {
                                C.c_int, _vp, C.POINTER(C.c_double)]),
     "scn_deconv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
                                  C.c_int, _vp, C.POINTER(C.c_double)]),
+    "scn_bn_subm_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int,
+                                       _vp, _vp, _vp, _vp, C.c_float, C.c_float, _vp, C.POINTER(C.c_double)]),
+    "scn_bn_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
+                                  C.c_int, _vp, _vp, _vp, _vp, C.c_float, C.c_float, _vp,
+                                  C.POINTER(C.c_double)]),
+    "scn_bn_deconv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
+                                    C.c_int, _vp, _vp, _vp, _vp, C.c_float, C.c_float, _vp,
+                                    C.POINTER(C.c_double)]),
     "scn_maxpool_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int,
                                   _vp]),
     "scn_bn_eval_fwd": (C.c_int, [_vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp,

@@ -7,6 +7,22 @@ from .tensor import SparseConvNetTensor
 
 
 class Sequential(torch.nn.Sequential):
+    def forward(self, input):
+        # Same chain as sequential.py:10-35, except that an eval-mode batch normalisation
+        # directly in front of a convolution is applied inside that convolution's gather.
+        from .layers import fusable_pair
+        mods = list(self._modules.values())
+        i = 0
+        while i < len(mods):
+            if i + 1 < len(mods) and isinstance(input, SparseConvNetTensor) and \
+                    fusable_pair(mods[i], mods[i + 1], input):
+                input = mods[i + 1](input, pre_bn=mods[i])
+                i += 2
+            else:
+                input = mods[i](input)
+                i += 1
+        return input
+
     def input_spatial_size(self, out_size):
         for m in reversed(self._modules):
             out_size = self._modules[m].input_spatial_size(out_size)

@@ -226,36 +226,84 @@ int scn_output_layer_fwd(scn_metadata *h, const float *in, float *out, int plane
   return guarded([&] { output_forward(md(h).input, in, out, planes, st(stream)); });
 }
 
+static int64_t level_rows(Metadata &m, const int64_t *spatial) {
+  Level *l = find_level(m, spatial);
+  return l ? l->n : 0;
+}
+static void subm_conv(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in, float *out,
+                      const float *weight, const float *bias, int n_in, int n_out, int groups, const BnArgs *bn,
+                      void *stream, double *macs) {
+  Metadata &m = md(h);
+  Table &t = submanifold_rules(m, spatial, filter, st(stream));
+  conv_forward(m, t, in, level_rows(m, spatial), out, weight, bias, n_in, n_out, groups, bn, st(stream));
+  // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
+  if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
+}
+static void strided_conv(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                         const int64_t *stride, const float *in, float *out, const float *weight,
+                         const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, void *stream,
+                         double *macs) {
+  Metadata &m = md(h);
+  StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
+  conv_forward(m, r.by_out, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, bn, st(stream));
+  if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
+}
+static void deconv(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                   const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
+                   int n_in, int n_out, int groups, const BnArgs *bn, void *stream, double *macs) {
+  Metadata &m = md(h);
+  // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
+  StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
+  conv_forward(m, r.by_in, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, bn, st(stream));
+  if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
+}
+
 int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,
                       float *out, const float *weight, const float *bias, int n_in, int n_out,
                       int groups, void *stream, double *macs) {
-  return guarded([&] {
-    Metadata &m = md(h);
-    Table &t = submanifold_rules(m, spatial, filter, st(stream));
-    conv_forward(m, t, in, out, weight, bias, n_in, n_out, groups, st(stream));
-    // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
-    if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
-  });
+  return guarded([&] { subm_conv(h, spatial, filter, in, out, weight, bias, n_in, n_out, groups, nullptr, stream, macs); });
 }
 int scn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                  const int64_t *stride, const float *in, float *out, const float *weight,
                  const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {
   return guarded([&] {
-    Metadata &m = md(h);
-    StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
-    conv_forward(m, r.by_out, in, out, weight, bias, n_in, n_out, groups, st(stream));
-    if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
+    strided_conv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, nullptr, stream, macs);
   });
 }
 int scn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                    const int64_t *stride, const float *in, float *out, const float *weight,
                    const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {
   return guarded([&] {
-    Metadata &m = md(h);
-    // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
-    StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
-    conv_forward(m, r.by_in, in, out, weight, bias, n_in, n_out, groups, st(stream));
-    if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
+    deconv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, nullptr, stream, macs);
+  });
+}
+int scn_bn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,
+                         float *out, const float *weight, const float *bias, int n_in, int n_out, int groups,
+                         const float *running_mean, const float *running_var, const float *gamma,
+                         const float *beta, float eps, float leakiness, void *stream, double *macs) {
+  return guarded([&] {
+    BnArgs bn{running_mean, running_var, gamma, beta, eps, leakiness};
+    subm_conv(h, spatial, filter, in, out, weight, bias, n_in, n_out, groups, &bn, stream, macs);
+  });
+}
+int scn_bn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                    const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
+                    int n_in, int n_out, int groups, const float *running_mean, const float *running_var,
+                    const float *gamma, const float *beta, float eps, float leakiness, void *stream,
+                    double *macs) {
+  return guarded([&] {
+    BnArgs bn{running_mean, running_var, gamma, beta, eps, leakiness};
+    strided_conv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, &bn, stream, macs);
+  });
+}
+int scn_bn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                      const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
+                      int n_in, int n_out, int groups, const float *running_mean, const float *running_var,
+                      const float *gamma, const float *beta, float eps, float leakiness, void *stream,
+                      double *macs) {
+  return guarded([&] {
+    BnArgs bn{running_mean, running_var, gamma, beta, eps, leakiness};
+    deconv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, &bn, stream, macs);
   });
 }
 int scn_maxpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,

@@ -16,6 +16,31 @@ namespace scn {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// Optional pre-activation of the gathered input values (eval batch norm + leaky ReLU of the
+// layer in front, CPU/BatchNormalization.cpp:41-61, fused into the gather): y = x*sc + sh,
+// y *= (y > 0 ? 1 : leak).  sc / sh are per input channel, zero-padded to a multiple of 64.
+template <bool PRE> __device__ inline v4f pre_act(v4f v, v4f sc, v4f sh, float leak) {
+  if (!PRE) return v;
+  v4f y = v * sc + sh;
+  y.x *= (y.x > 0.f ? 1.f : leak);
+  y.y *= (y.y > 0.f ? 1.f : leak);
+  y.z *= (y.z > 0.f ? 1.f : leak);
+  y.w *= (y.w > 0.f ? 1.f : leak);
+  return y;
+}
+__global__ void k_pre_coeffs(const float *mean, const float *var, const float *gamma, const float *beta, float eps,
+                             int n_in, int n_pad, float *sc, float *sh) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_pad) return;
+  float w = 0.f, b = 0.f;
+  if (c < n_in) {
+    w = (1.0f / sqrtf(var[c] + eps)) * (gamma ? gamma[c] : 1.0f);
+    b = -mean[c] * w + (beta ? beta[c] : 0.0f);
+  }
+  sc[c] = w;
+  sh[c] = b;
+}
+
 // ---- generic kernel: any channel counts, any groups -------------------------------------
 __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad,
                                const float *in, float *out, const float *w, const float *bias, int n_in,
@@ -107,12 +132,13 @@ __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows
 // load of the pipeline is unconditional (granules without the tap and absent rows read
 // row 0 and are zeroed by a select), so the count of loads in flight is a compile-time
 // constant and the compiler can wait for exactly the loads it needs.
-template <int NCBW, int WC, int GW, int SS, bool VEC4>
+template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE>
 __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
-    int n_split, float *__restrict__ partial) {
+    int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
+    const float *__restrict__ pre_sh, float pre_leak) {
   constexpr int WR = 4 / WC;
   constexpr int NCB = NCBW * WC;
   constexpr int G = GW * WR;
@@ -179,6 +205,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 
   v4f wreg[WPT];
   v4f areg[FPW];
+  v4f psc[FPW], psh[FPW];           // pre-activation coefficients of the fragments' channels
   unsigned gm_nxt = 0, gm_cur = 0;  // granule mask of the tap (uniform)
   unsigned aok_nxt = 0;             // bit i: this lane's row of fragment i exists
   int sl_nxt = 0;
@@ -203,6 +230,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       if (j >= 0) aok_nxt |= 1u << i;
       const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
       const int c0 = (sl * SS + s) * 16 + 4 * g;
+      if (PRE) {
+        psc[i] = *reinterpret_cast<const v4f *>(pre_sc + c0);
+        psh[i] = *reinterpret_cast<const v4f *>(pre_sh + c0);
+      }
       v4f v;
       if (VEC4) {
         const int cc = c0 < n_in ? c0 : n_in - 4;
@@ -229,7 +260,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       const int f = wave + 4 * i;
       const int c0 = (sl_nxt * SS + f % SS) * 16 + 4 * g;
       const bool ok = (aok_nxt >> i) & 1u;
-      v4f v = areg[i];
+      v4f v = pre_act<PRE>(areg[i], psc[i], psh[i], pre_leak);
       if (VEC4) {
         if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
       } else {
@@ -325,9 +356,14 @@ __global__ void k_conv_reduce(const float *partial, int n_split, int64_t split_s
   out[row * n_out + col] = acc;
 }
 
-template <int NCBW, int WC, int GW, int SS, bool VEC4>
+struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
+  const float *sc = nullptr, *sh = nullptr;
+  float leak = 1.0f;
+};
+
+template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE>
 static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                        const float *bias, int n_in, int n_out, hipStream_t s) {
+                        const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
   constexpr int WPT = (SS * NCB * 64 + 255) / 256;
   constexpr int SLAB_STRIDE = WPT * 256 * 4;  // floats
@@ -341,7 +377,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE);
   LAUNCH_CHECK();
-  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4>;
+  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -361,7 +397,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   }
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), 256, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial);
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak);
   LAUNCH_CHECK();
   if (n_split > 1) {
     k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
@@ -374,14 +410,14 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
 // Picks the instantiation from the number of 16-column blocks of the output.  Tiles are 8
 // granules (128 rows); registers and LDS are sized so that two workgroups share a CU and one
 // hides the other's staging.  A slab is one 16-channel step when nIn <= 16 or nOut > 128.
-template <bool VEC4>
+template <bool VEC4, bool PRE>
 static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                         const float *bias, int n_in, int n_out, hipStream_t s) {
+                         const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   const bool narrow = n_in <= 16;
-#define SCN_CASE(N, NCBW, WC, GW, SSW)                                                                 \
-  if (ncb <= N)                                                                                        \
-    return narrow ? launch_mfma<NCBW, WC, GW, 1, VEC4>(m, t, in, out, w, bias, n_in, n_out, s)         \
-                  : launch_mfma<NCBW, WC, GW, SSW, VEC4>(m, t, in, out, w, bias, n_in, n_out, s);
+#define SCN_CASE(N, NCBW, WC, GW, SSW)                                                                      \
+  if (ncb <= N)                                                                                             \
+    return narrow ? launch_mfma<NCBW, WC, GW, 1, VEC4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)    \
+                  : launch_mfma<NCBW, WC, GW, SSW, VEC4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
   SCN_CASE(1, 1, 1, 2, 2)
   SCN_CASE(2, 1, 2, 4, 2)
   SCN_CASE(4, 1, 4, 8, 2)
@@ -402,12 +438,13 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
 // granules' [16 x nOut] accumulators in registers.  Compared with k_conv_mfma the gathered
 // rows never touch LDS and one weight slab serves NW*RG*16 rows (up to 512), at the price of
 // uneven MFMA work between wavefronts, which three to four wavefronts per SIMD even out.
-template <int NCB, int RG, int SS, bool VEC4, int NW>
+template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE>
 __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
-    int n_split, float *__restrict__ partial) {
+    int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
+    const float *__restrict__ pre_sh, float pre_leak) {
   constexpr int NT = NW * 64;
   constexpr int G = NW * RG;
   constexpr int TM = G * 16;
@@ -466,6 +503,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 
   v4f wreg[WPT];
   v4f a_nxt[RG][SS], a_cur[RG][SS];
+  v4f psc[SS], psh[SS];
   unsigned gm_nxt = 0, gm_cur = 0, ok_nxt = 0;
   int sl_nxt = 0;
 
@@ -475,6 +513,13 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     gm_nxt = gmask[k];
     sl_nxt = sl;
     ok_nxt = 0;
+    if (PRE) {
+#pragma unroll
+      for (int s = 0; s < SS; s++) {
+        psc[s] = *reinterpret_cast<const v4f *>(pre_sc + (sl * SS + s) * 16 + 4 * g);
+        psh[s] = *reinterpret_cast<const v4f *>(pre_sh + (sl * SS + s) * 16 + 4 * g);
+      }
+    }
     const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
 #pragma unroll
     for (int i = 0; i < WPT; i++) {
@@ -513,7 +558,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 #pragma unroll
       for (int s = 0; s < SS; s++) {
         const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
-        v4f v = a_nxt[q][s];
+        v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
         if (VEC4) {
           if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
         } else {
@@ -584,9 +629,9 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   }
 }
 
-template <int NCB, int RG, int SS, bool VEC4, int NW>
+template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE>
 static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                        const float *bias, int n_in, int n_out, hipStream_t s) {
+                        const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   constexpr int NT = NW * 64, G = NW * RG;
   constexpr int SLAB_F4 = SS * NCB * 64;
   constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
@@ -600,7 +645,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE);
   LAUNCH_CHECK();
-  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW>;
+  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -619,7 +664,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   }
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), NT, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial);
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak);
   LAUNCH_CHECK();
   if (n_split > 1) {
     k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
@@ -640,11 +685,12 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
 // of whose rows has the tap skip their MFMAs.
 // With accumulate != 0 the kernel adds to `out` instead of overwriting it (used to split a
 // wide nIn into several launches).
-template <int NCB, int RG, int SS, bool VEC4, int WAVES>
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, int in_stride, float *__restrict__ out, const float *__restrict__ wp,
-    const float *__restrict__ bias, int n_in, int n_out, int n_sets, int sets_per_xcd, int accumulate) {
+    const float *__restrict__ bias, int n_in, int n_out, int n_sets, int sets_per_xcd, int accumulate,
+    const float *__restrict__ pre_sc, const float *__restrict__ pre_sh, float pre_leak) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   v4f *wl = reinterpret_cast<v4f *>(lds);  // [K][SS][NCB][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -658,6 +704,12 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   for (int cb = 0; cb < NCB; cb++) {
     const int col = 16 * cb + r16;
     bv[cb] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+  }
+  v4f psc[SS], psh[SS];  // this lane always handles channels s*16 + 4*g .. +3
+#pragma unroll
+  for (int s = 0; s < SS; s++) {
+    psc[s] = PRE ? *reinterpret_cast<const v4f *>(pre_sc + s * 16 + 4 * g) : (v4f){1.f, 1.f, 1.f, 1.f};
+    psh[s] = PRE ? *reinterpret_cast<const v4f *>(pre_sh + s * 16 + 4 * g) : (v4f){0.f, 0.f, 0.f, 0.f};
   }
   // Sets are dealt so that one XCD (blocks b, b+8, ...) walks a contiguous range.
   const int xcd = blockIdx.x & 7, blk = blockIdx.x >> 3, blocks_per_xcd = gridDim.x >> 3;
@@ -753,7 +805,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 #pragma unroll
           for (int s = 0; s < SS; s++) {
             const int c0 = s * 16 + 4 * g;
-            v4f av = a_cur[q][s];
+            v4f av = pre_act<PRE>(a_cur[q][s], psc[s], psh[s], pre_leak);
             if (VEC4) {
               if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
             } else {
@@ -796,10 +848,10 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 }
 
 // One launch over channels [c_lo, c_lo + n_in_part) of the input rows.
-template <int NCB, int SS, bool VEC4>
+template <int NCB, int SS, bool VEC4, bool PRE>
 static void launch_resident_part(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
                                  const float *w, int w_in_stride_rows, const float *bias, int n_in_part,
-                                 int n_out, int accumulate, hipStream_t s) {
+                                 int n_out, int accumulate, PreArgs pre, hipStream_t s) {
   constexpr int RG = 2;  // 32 rows per set: measured faster than 64 (more wavefronts in flight)
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
   m.wpack.reserve(packed);
@@ -812,7 +864,7 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
   const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   if (lds_bytes > 80 * 1024) {
     constexpr int WAVES = 16;
-    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES>;
+    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, PRE>;
     static bool attr_set = false;
     if (!attr_set) {
       HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -822,10 +874,10 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
     const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32, ceil_div(sets_per_xcd, WAVES)));
     kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
                                                      m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                     accumulate);
+                                                     accumulate, pre.sc, pre.sh, pre.leak);
   } else {
     constexpr int WAVES = 8;
-    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES>;
+    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, PRE>;
     static bool attr_set = false;
     if (!attr_set) {
       HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -836,16 +888,21 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
     const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
     kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
                                                      m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                     accumulate);
+                                                     accumulate, pre.sc, pre.sh, pre.leak);
   }
   LAUNCH_CHECK();
 }
 
 // Narrow layers: nOut <= 32, any nIn, K <= 32.  nIn is processed in parts of up to 32
 // channels so that every part's weights fit in LDS; parts after the first accumulate.
+static bool resident_fits(const Table &t, int n_out) { return t.K <= 32 && n_out <= 32; }
+
+// No fused batch norm here: this kernel's time goes into the vector instructions around its
+// small MFMA blocks, and normalising every gathered value (each row is gathered once per tap
+// that reaches it) costs more than one extra pass over the rows.
 static bool try_resident(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                          const float *bias, int n_in, int n_out, hipStream_t s) {
-  if (t.K > 32 || n_out > 32) return false;
+  if (!resident_fits(t, n_out)) return false;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   const int ncb = (int)ceil_div(n_out, 16);
   for (int c_lo = 0; c_lo < n_in; c_lo += 32) {
@@ -854,12 +911,14 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
     const float *w_p = w + (int64_t)c_lo * n_out;
     const int acc = c_lo > 0;
     const float *b = acc ? nullptr : bias;
-#define SCN_RES(NCBV, SSV)                                                                               \
-  do {                                                                                                   \
-    if (vec4)                                                                                            \
-      launch_resident_part<NCBV, SSV, true>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc, s);   \
-    else                                                                                                 \
-      launch_resident_part<NCBV, SSV, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc, s);  \
+#define SCN_RES(NCBV, SSV)                                                                                   \
+  do {                                                                                                       \
+    if (vec4)                                                                                                \
+      launch_resident_part<NCBV, SSV, true, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc,    \
+                                                   PreArgs(), s);                                            \
+    else                                                                                                     \
+      launch_resident_part<NCBV, SSV, false, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc,   \
+                                                    PreArgs(), s);                                           \
   } while (0)
     if (ncb == 1 && part <= 16) SCN_RES(1, 1);
     else if (ncb == 1) SCN_RES(1, 2);
@@ -870,46 +929,76 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
   return true;
 }
 
-// Mid-width layers (32 < nOut <= 128): row-owner kernel.  Measured best on the 1 M-site
-// scene: 8 wavefronts x 2 granules for nOut <= 64, 16 wavefronts x 1 granule above.
-template <bool VEC4>
+// Mid-width layers (32 < nOut <= 128): row-owner kernel with 128-row workgroups (measured
+// best on room scenes: small workgroups, five or more per CU, even out the work between
+// barriers better than 256- or 512-row ones).  Above 128 outputs the accumulators of a
+// granule no longer leave room for this layout's operands and k_conv_mfma is as fast.
+template <bool VEC4, bool PRE>
 static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                          const float *bias, int n_in, int n_out, hipStream_t s) {
+                          const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   const int ncb = (int)ceil_div(n_out, 16);
   const bool narrow = n_in <= 16;
   if (ncb <= 4)
-    return narrow ? launch_rows<4, 2, 1, VEC4, 8>(m, t, in, out, w, bias, n_in, n_out, s)
-                  : launch_rows<4, 2, 2, VEC4, 8>(m, t, in, out, w, bias, n_in, n_out, s);
+    return narrow ? launch_rows<4, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
+                  : launch_rows<4, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
   if (ncb <= 6)
-    return narrow ? launch_rows<6, 1, 1, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s)
-                  : launch_rows<6, 1, 2, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s);
+    return narrow ? launch_rows<6, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
+                  : launch_rows<6, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
   if (ncb <= 8)
-    return narrow ? launch_rows<8, 1, 1, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s)
-                  : launch_rows<8, 1, 2, VEC4, 16>(m, t, in, out, w, bias, n_in, n_out, s);
+    return narrow ? launch_rows<8, 1, 1, VEC4, 8, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
+                  : launch_rows<8, 1, 2, VEC4, 8, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
   return false;
 }
 
-void conv_forward(Metadata &m, const Table &t, const float *in, float *out, const float *w, const float *bias,
-                  int n_in, int n_out, int groups, hipStream_t s) {
+template <bool PRE>
+static bool conv_mfma_paths(Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                            const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+  if (!PRE && try_resident(m, t, in, out, w, bias, n_in, n_out, s)) return true;
+  const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
+  if (n_out <= 128 && t.K <= 1024) {
+    if (vec4 ? dispatch_rows<true, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
+             : dispatch_rows<false, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s))
+      return true;
+  }
+  if (t.K <= 1024) {
+    const int ncb = (int)ceil_div(n_out, 16);
+    if (vec4 ? dispatch_ncb<true, PRE>(ncb, m, t, in, out, w, bias, n_in, n_out, pre, s)
+             : dispatch_ncb<false, PRE>(ncb, m, t, in, out, w, bias, n_in, n_out, pre, s))
+      return true;
+  }
+  return false;
+}
+
+// bn: optional eval batch norm + leaky ReLU applied to the input rows before the convolution
+// (what a BatchNormalization module in front of the convolution computes), fused into the
+// gather; nullptr for a plain convolution.
+void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
+                  const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, hipStream_t s) {
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
-  if (groups == 1 && try_resident(m, t, in, out, w, bias, n_in, n_out, s)) return;
-  if (groups == 1 && n_out <= 128 && t.K <= 1024) {
-    const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
-    if (vec4 ? dispatch_rows<true>(m, t, in, out, w, bias, n_in, n_out, s)
-             : dispatch_rows<false>(m, t, in, out, w, bias, n_in, n_out, s))
-      return;
+  if (bn && groups == 1 && !resident_fits(t, n_out)) {
+    const int n_pad = (int)round_up(n_in, 64) + 64;
+    m.prebuf.reserve(2 * (size_t)n_pad);
+    k_pre_coeffs<<<dim3((unsigned)ceil_div(n_pad, 256)), 256, 0, s>>>(bn->mean, bn->var, bn->gamma, bn->beta, bn->eps,
+                                                                     n_in, n_pad, m.prebuf.p, m.prebuf.p + n_pad);
+    LAUNCH_CHECK();
+    PreArgs pre;
+    pre.sc = m.prebuf.p;
+    pre.sh = m.prebuf.p + n_pad;
+    pre.leak = bn->leak;
+    if (conv_mfma_paths<true>(m, t, in, out, w, bias, n_in, n_out, pre, s)) return;
   }
-  if (groups == 1 && t.K <= 1024) {
-    const int ncb = (int)ceil_div(n_out, 16);
-    const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
-    bool done = vec4 ? dispatch_ncb<true>(ncb, m, t, in, out, w, bias, n_in, n_out, s)
-                     : dispatch_ncb<false>(ncb, m, t, in, out, w, bias, n_in, n_out, s);
-    if (done) return;
+  const float *src = in;
+  if (bn) {  // no fused kernel for this shape: normalise the rows in a pass of their own
+    m.bntmp.reserve((size_t)std::max<int64_t>(n_in_rows, 1) * n_in);
+    bn_eval_forward(in, m.bntmp.p, n_in_rows, n_in, n_in, n_in, bn->mean, bn->var, bn->gamma, bn->beta, bn->eps,
+                    bn->leak, s);
+    src = m.bntmp.p;
   }
+  if (groups == 1 && conv_mfma_paths<false>(m, t, src, out, w, bias, n_in, n_out, PreArgs(), s)) return;
   int64_t total = t.n * n_out;
-  k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in,
+  k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, src,
                                                                        out, w, bias, n_in, n_out, groups);
   LAUNCH_CHECK();
 }

@@ -85,6 +85,8 @@ struct Metadata {
   DevBuf<int> dflags;
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
+  DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
+  DevBuf<float> bntmp;    // normalised input when a fused batch norm has no fused kernel
 };
 
 SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);
@@ -105,8 +107,12 @@ int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *p
 
 // ops.hip / conv.hip
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);
-void conv_forward(Metadata &m, const Table &t, const float *in, float *out, const float *w, const float *bias,
-                  int n_in, int n_out, int groups, hipStream_t s);
+struct BnArgs {  // eval batch norm + leaky ReLU in front of a convolution (device pointers)
+  const float *mean, *var, *gamma, *beta;
+  float eps, leak;
+};
+void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
+                  const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, hipStream_t s);
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
                      int drop, hipStream_t s);
 void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,

@@ -503,16 +503,23 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
 
 // ---- pattern-sorted positions ----------------------------------------------------------
 
-static const int BLOCK_SHIFT = 8;  // positions are re-sorted inside blocks of 256
+// Positions are re-sorted by neighbour pattern inside PATTERN_WINDOWS equal ranges of the
+// space-filling-curve order.  A convolution workgroup takes consecutive positions, so after
+// the sort its rows share one or two patterns: it walks only the taps those patterns have and
+// every 16-row granule is busy on each of them.  One range per XCD (workgroups are dealt to
+// XCDs in contiguous ranges) keeps an XCD's gathers inside one compact region of space;
+// measured on room scenes of 60k..4M sites, 8 or 16 ranges beat both 256-position blocks
+// (by 20-30% for 64..256 channels) and one global sort (which loses the locality).
+static const int PATTERN_WINDOWS = 8;
 
-__global__ void k_table_masks(const int *nbr, int K, int64_t n, int64_t npad, unsigned long long *keys,
+__global__ void k_table_masks(int64_t window, const int *nbr, int K, int64_t n, int64_t npad, unsigned long long *keys,
                               int *idx) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n) return;
   unsigned long long mask = 0;
   for (int k = 0; k < K; k++)
     if (nbr[(int64_t)k * npad + t] >= 0) mask |= 1ull << k;
-  keys[t] = ((unsigned long long)(t >> BLOCK_SHIFT) << K) | mask;
+  keys[t] = ((unsigned long long)(t / window) << K) | mask;
   idx[t] = (int)t;
 }
 __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, const int *perm,
@@ -531,15 +538,16 @@ __global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
 }
 
 // t.nbr is indexed by the level's schedule (base[t] = row, or t itself when base is null).
-// Re-sort positions by neighbour pattern inside blocks and record the position -> row map.
+// Re-sort positions by neighbour pattern inside windows and record the position -> row map.
 static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s) {
   if (t.n == 0) {
     t.identity_rows = true;
     return;
   }
   t.rowmap.reserve(t.npad);
+  const int64_t window = std::max<int64_t>(256, round_up(ceil_div(t.n, PATTERN_WINDOWS), 256));
   int block_bits = 1;
-  while (((int64_t)1 << block_bits) <= (t.n >> BLOCK_SHIFT)) block_bits++;
+  while (((int64_t)1 << block_bits) <= t.n / window) block_bits++;
   if (t.K + block_bits > 62) {  // the pattern does not fit the sort key: keep schedule order
     t.identity_rows = base == nullptr;
     if (base) {
@@ -552,7 +560,7 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   m.k1.reserve(t.n);
   m.v0.reserve(t.n);
   m.v1.reserve(t.n);
-  k_table_masks<<<grid_for(t.n), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p);
+  k_table_masks<<<grid_for(t.n), TB, 0, s>>>(window, t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p);
   LAUNCH_CHECK();
   sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, t.K + block_bits);
   DevBuf<int> nbr2;

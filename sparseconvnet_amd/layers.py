@@ -58,6 +58,27 @@ def _count(macs, out):
     _pkg.forward_pass_hidden_states += out.nelement()
 
 
+def _bn_args(bn):
+    """The tensors and constants of an eval-mode BatchNormalization module that a convolution
+    applies to its input rows itself (None: nothing to apply)."""
+    if bn is None:
+        return None
+    return (bn.running_mean, bn.running_var, optionalTensor(bn, 'weight').detach(),
+            optionalTensor(bn, 'bias').detach(), bn.eps, bn.leakiness)
+
+
+def fusable_pair(bn, conv, input):
+    """True when Sequential may hand the batch normalisation `bn` to the convolution `conv`
+    that follows it instead of running it as a pass of its own: the result is the same, the
+    normalised rows are just never written to memory."""
+    return (_pkg.fuse_batchnorm and type(bn) in (BatchNormalization, BatchNormReLU, BatchNormLeakyReLU)
+            and type(conv) in (SubmanifoldConvolution, ValidConvolution, Convolution, Deconvolution)
+            and not bn.training and conv.groups == 1 and bn.nPlanes == conv.nIn
+            and not bn._forward_hooks and not bn._forward_pre_hooks
+            and not conv._forward_hooks and not conv._forward_pre_hooks
+            and input.features.nelement() > 0 and input.features.size(1) == bn.nPlanes)
+
+
 class SubmanifoldConvolution(Module):
     """submanifoldConvolution.py:14-61."""
 
@@ -73,15 +94,15 @@ class SubmanifoldConvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input):
+    def forward(self, input, pre_bn=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, self.nOut, input)
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
-        md, sz, fs = input.metadata, input.spatial_size, self.filter_size
+        md, sz, fs, bn = input.metadata, input.spatial_size, self.filter_size, _bn_args(pre_bn)
 
         def fn(x, w, b):
-            y, macs = md.submanifoldConvolution(sz, fs, x, w, b)
+            y, macs = md.submanifoldConvolution(sz, fs, x, w, b, bn)
             _count(macs, y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
@@ -114,7 +135,7 @@ class Convolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input):
+    def forward(self, input, pre_bn=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
@@ -123,9 +144,10 @@ class Convolution(Module):
         assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
             input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        bn = _bn_args(pre_bn)
 
         def fn(x, w, b):
-            y, macs = md.convolution(*a, x, w, b)
+            y, macs = md.convolution(*a, x, w, b, bn)
             _count(macs, y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
@@ -155,15 +177,16 @@ class Deconvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input):
+    def forward(self, input, pre_bn=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
         md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        bn = _bn_args(pre_bn)
 
         def fn(x, w, b):
-            y, macs = md.deconvolution(*a, x, w, b)
+            y, macs = md.deconvolution(*a, x, w, b, bn)
             _count(macs, y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))

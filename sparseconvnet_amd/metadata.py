@@ -86,33 +86,44 @@ class Metadata:
         _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out
 
-    def _conv(self, fn, size_args, n_rows, features, weight, bias):
+    def _conv(self, name, size_args, n_rows, features, weight, bias, bn):
+        """bn: None, or (running_mean, running_var, weight, bias, eps, leakiness) of an eval-mode
+        batch normalisation applied to `features` inside the convolution's gather."""
         features = _features(features, "features")
         weight = _features(weight, "weight")
         K, groups, ip, op = weight.shape
         bias_t = _features(bias, "bias") if bias is not None and bias.numel() else None
         out = torch.empty((n_rows, groups * op), dtype=torch.float32, device=features.device)
         macs = C.c_double(0)
-        _lib.check(fn(self._h, *size_args, _ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t), groups * ip,
-                      groups * op, groups, _stream(), C.byref(macs)))
+        head = (self._h, *size_args, _ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t), groups * ip,
+                groups * op, groups)
+        if bn is None:
+            _lib.check(getattr(self._L, "scn_" + name)(*head, _stream(), C.byref(macs)))
+        else:
+            mean, var, g, b, eps, leak = bn
+            assert mean.numel() == groups * ip and var.numel() == groups * ip
+            g = _features(g, "bn weight") if g is not None and g.numel() else None
+            b = _features(b, "bn bias") if b is not None and b.numel() else None
+            _lib.check(getattr(self._L, "scn_bn_" + name)(
+                *head, _ptr(_features(mean, "running_mean")), _ptr(_features(var, "running_var")), _ptr(g),
+                _ptr(b), float(eps), float(leak), _stream(), C.byref(macs)))
         return out, macs.value
 
-    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias):
+    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias, bn=None):
         sp, fs = self._s(spatial_size), self._s(filter_size)
         _lib.check(self._L.scn_md_submanifold_rules(self._h, sp, fs, _stream()))
-        return self._conv(self._L.scn_subm_conv_fwd, (sp, fs), self.getNActive(spatial_size), features, weight,
-                          bias)
+        return self._conv("subm_conv_fwd", (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn)
 
-    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias):
+    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
-        return self._conv(self._L.scn_conv_fwd, a, self.getNActive(out_size), features, weight, bias)
+        return self._conv("conv_fwd", a, self.getNActive(out_size), features, weight, bias, bn)
 
-    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias):
+    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *rb, _stream()))
-        return self._conv(self._L.scn_deconv_fwd, a, self.getNActive(out_size), features, weight, bias)
+        return self._conv("deconv_fwd", a, self.getNActive(out_size), features, weight, bias, bn)
 
     def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
         a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]

@@ -115,3 +115,26 @@ def test_empty_input_passes_through():
     with torch.no_grad():
         out = model(t)
     assert out.features.shape == (0, 4)
+
+
+def test_fused_and_unfused_sequential_agree():
+    """Sequential hands a batch normalisation in front of a convolution to that convolution;
+    with sparseconvnet_amd.fuse_batchnorm off every module runs by itself.  Same result."""
+    torch.manual_seed(7)
+    m = 16
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m], False, leakiness=0.2)).add(scn.BatchNormReLU(m)).add(
+        scn.OutputLayer(3)).cuda().eval()
+    randomise_bn(model, 7)
+    coords = synthetic.scene_batch(seed=7000, batch=2, target=8000, spatial=64, n_boxes=8)
+    feats = torch.rand(len(coords), 3).cuda()
+    inp_layer = scn.InputLayer(3, 64, mode=4)
+    outs = []
+    for fuse in (True, False):
+        scn.fuse_batchnorm = fuse
+        try:
+            with torch.no_grad():
+                outs.append(model(inp_layer([torch.as_tensor(coords), feats])).cpu().numpy())
+        finally:
+            scn.fuse_batchnorm = True
+    checks.assert_close(outs[0], outs[1], "fused vs unfused")
