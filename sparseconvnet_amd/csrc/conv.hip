@@ -12,6 +12,8 @@
 // carry almost all of the sparsity.
 #include "metadata.h"
 
+#include <type_traits>
+
 namespace scn {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -99,8 +101,10 @@ __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n
 // Packs rows [0, n_in_part) of every tap's weight slice, where the slice of tap k starts at
 // w + k * w_rows * n_out (w already points at the first row of the range), as one slab per tap
 // in the layout of k_pack_weights.
+// Also clears the eight set counters (one per XCD, 128 bytes apart) of the launch it precedes.
 __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows, int n_in_part, int n_out,
-                                    int SS, int NCB) {
+                                    int SS, int NCB, int *queue) {
+  if (blockIdx.x == 0 && threadIdx.x < 8) queue[threadIdx.x * 32] = 0;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = (int64_t)K * SS * NCB * 256;
   if (i >= total) return;
@@ -676,24 +680,29 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
 
 // ---- resident-weights kernel for narrow layers ------------------------------------------
 // When the packed weights of all taps fit in LDS (K * ceil(nIn/16) * NCB KiB), a persistent
-// workgroup loads them once and its wavefronts then work independently, with no barrier:
-// each takes sets of RG granules, keeps their accumulators in registers, and walks the taps
-// that any of its 64 rows has (a bit mask scanned with ffs).  The walk is a three-stage
-// register pipeline: neighbour indices of tap i+2 and input rows of tap i+1 are in flight
-// while tap i runs its MFMAs; all loads are unconditional (absent rows read row 0 and are
-// zeroed by a select), past the last tap the pipeline reloads the last tap.  Granules none
-// of whose rows has the tap skip their MFMAs.
+// workgroup loads them once and its wavefronts then work independently, with no barrier.
+// A wavefront takes sets of RG granules and, for each set, the taps that any of its rows
+// has (the OR of the table's per-granule tap masks).  The (set, tap) pairs of a wavefront
+// form one stream that runs through a register pipeline four items deep: the neighbour
+// indices of items i+3 and i+4 and the input rows of items i+1 and i+2 are in flight while
+// item i runs its MFMAs (one item of look-ahead does not cover the latency of a gather that
+// misses L2), also across the boundary between two sets, so the pipeline drains only once,
+// at the wavefront's end.
+// All loads are unconditional (absent rows read row 0 and are zeroed by a select; items past
+// the end re-read the first set).  Granules none of whose rows has the tap skip their MFMAs.
 // With accumulate != 0 the kernel adds to `out` instead of overwriting it (used to split a
 // wide nIn into several launches).
 template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
-    const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
-    const float *__restrict__ in, int in_stride, float *__restrict__ out, const float *__restrict__ wp,
-    const float *__restrict__ bias, int n_in, int n_out, int n_sets, int sets_per_xcd, int accumulate,
-    const float *__restrict__ pre_sc, const float *__restrict__ pre_sh, float pre_leak) {
+    const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
+    int64_t n, int64_t npad, const float *__restrict__ in, int in_stride, float *__restrict__ out,
+    const float *__restrict__ wp, const float *__restrict__ bias, int n_in, int n_out, int n_sets,
+    int sets_per_xcd, int accumulate, const float *__restrict__ pre_sc, const float *__restrict__ pre_sh,
+    float pre_leak, int *__restrict__ queue) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   v4f *wl = reinterpret_cast<v4f *>(lds);  // [K][SS][NCB][64]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
   const int total_f4 = K * SS * NCB * 64;
   for (int e = threadIdx.x; e < total_f4; e += WAVES * 64) wl[e] = reinterpret_cast<const v4f *>(wp)[e];
@@ -711,139 +720,190 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     psc[s] = PRE ? *reinterpret_cast<const v4f *>(pre_sc + s * 16 + 4 * g) : (v4f){1.f, 1.f, 1.f, 1.f};
     psh[s] = PRE ? *reinterpret_cast<const v4f *>(pre_sh + s * 16 + 4 * g) : (v4f){0.f, 0.f, 0.f, 0.f};
   }
-  // Sets are dealt so that one XCD (blocks b, b+8, ...) walks a contiguous range.
-  const int xcd = blockIdx.x & 7, blk = blockIdx.x >> 3, blocks_per_xcd = gridDim.x >> 3;
-  for (int ls = blk * WAVES + wave; ls < sets_per_xcd; ls += blocks_per_xcd * WAVES) {
-    const int set = xcd * sets_per_xcd + ls;
-    if (set >= n_sets) break;
-    const int64_t t0 = (int64_t)set * (RG * 16);
-    // which taps does any row of the set have?  lane group g looks at taps 4*kk + g
-    unsigned tapmask = 0;
-    for (int kb = 0; kb < K; kb += 4) {
-      const int k = kb + g;
-      bool any = false;
-#pragma unroll
-      for (int q = 0; q < RG; q++) {
-        const int64_t t = t0 + q * 16 + r16;
-        if (k < K && t < n) any |= nbr[(int64_t)k * npad + t] >= 0;
-      }
-      const unsigned long long bal = __ballot(any);
-#pragma unroll
-      for (int gg = 0; gg < 4; gg++)
-        if ((bal >> (16 * gg)) & 0xFFFFull) tapmask |= 1u << (kb + gg);
-    }
-    tapmask = __builtin_amdgcn_readfirstlane(tapmask);
-    const int ntaps = __popc(tapmask);
-
-    v4f acc[RG][NCB];
-#pragma unroll
-    for (int q = 0; q < RG; q++)
-#pragma unroll
-      for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    if (ntaps > 0) {
-      int64_t tq[RG];
-#pragma unroll
-      for (int q = 0; q < RG; q++) tq[q] = min(t0 + q * 16 + r16, n - 1);
-      unsigned rest = tapmask;
-      auto next_tap = [&]() {  // next set bit; sticks at the last one
-        const int k = __ffs(rest) - 1;
-        if (rest & (rest - 1)) rest &= rest - 1;
-        return k;
-      };
-      auto load_j = [&](int k, int *j) {
-#pragma unroll
-        for (int q = 0; q < RG; q++) j[q] = nbr[(int64_t)k * npad + tq[q]];
-      };
-      auto load_a = [&](const int *j, v4f (*a)[SS]) {
-#pragma unroll
-        for (int q = 0; q < RG; q++) {
-          const float *src = in + (int64_t)(j[q] < 0 ? 0 : j[q]) * in_stride;
-#pragma unroll
-          for (int s = 0; s < SS; s++) {
-            const int c0 = s * 16 + 4 * g;
-            if (VEC4) {
-              const int cc = c0 < n_in ? c0 : n_in - 4;
-              a[q][s] = *reinterpret_cast<const v4f *>(src + cc);
-            } else {
-              a[q][s].x = src[min(c0 + 0, n_in - 1)];
-              a[q][s].y = src[min(c0 + 1, n_in - 1)];
-              a[q][s].z = src[min(c0 + 2, n_in - 1)];
-              a[q][s].w = src[min(c0 + 3, n_in - 1)];
-            }
-          }
-        }
-      };
-      int k_cur, k_nxt, k_nn;
-      int j_nxt[RG], j_nn[RG], j_cur[RG];
-      v4f a_nxt[RG][SS], a_cur[RG][SS];
-      k_nxt = next_tap();
-      load_j(k_nxt, j_nxt);
-      k_nn = next_tap();
-      load_j(k_nn, j_nn);
-      load_a(j_nxt, a_nxt);
-      for (int i = 0; i < ntaps; i++) {
-        k_cur = k_nxt;
-#pragma unroll
-        for (int q = 0; q < RG; q++) {
-          j_cur[q] = (t0 + q * 16 + r16 < n) ? j_nxt[q] : -1;
-#pragma unroll
-          for (int s = 0; s < SS; s++) a_cur[q][s] = a_nxt[q][s];
-        }
-        // advance the pipeline: rows of the next tap, indices of the one after
-        k_nxt = k_nn;
-#pragma unroll
-        for (int q = 0; q < RG; q++) j_nxt[q] = j_nn[q];
-        load_a(j_nxt, a_nxt);
-        k_nn = next_tap();
-        load_j(k_nn, j_nn);
-
-#pragma unroll
-        for (int q = 0; q < RG; q++) {
-          const bool ok = j_cur[q] >= 0;
-          if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
-#pragma unroll
-          for (int s = 0; s < SS; s++) {
-            const int c0 = s * 16 + 4 * g;
-            v4f av = pre_act<PRE>(a_cur[q][s], psc[s], psh[s], pre_leak);
-            if (VEC4) {
-              if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
-            } else {
-              if (!(ok && c0 + 0 < n_in)) av.x = 0.f;
-              if (!(ok && c0 + 1 < n_in)) av.y = 0.f;
-              if (!(ok && c0 + 2 < n_in)) av.z = 0.f;
-              if (!(ok && c0 + 3 < n_in)) av.w = 0.f;
-            }
-            v4f b[NCB];
-#pragma unroll
-            for (int cb = 0; cb < NCB; cb++) b[cb] = wl[((k_cur * SS + s) * NCB + cb) * 64 + lane];
-#pragma unroll
-            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[cb].x, acc[q][cb], 0, 0, 0);
-#pragma unroll
-            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[cb].y, acc[q][cb], 0, 0, 0);
-#pragma unroll
-            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[cb].z, acc[q][cb], 0, 0, 0);
-#pragma unroll
-            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[cb].w, acc[q][cb], 0, 0, 0);
-          }
-        }
-      }
-    }
+  const int64_t n_granules = (n + 15) >> 4;
+  // Tap mask of a set; a set without any rule still runs one (empty) tap so that its rows
+  // get their bias.  The index is clamped: the caller decides whether the set exists.
+  auto set_mask = [&](int set) {
+    unsigned m = 0;
 #pragma unroll
     for (int q = 0; q < RG; q++) {
+      const int64_t gi = (int64_t)set * RG + q;
+      m |= gmask[gi < n_granules ? gi : n_granules - 1];
+    }
+    return m ? m : 1u;
+  };
+  // One XCD (blocks b, b+8, ...) walks a contiguous range of sets.  A wavefront's first set
+  // is fixed; the following ones it takes from the XCD's counter, one set ahead of the set
+  // it is generating items for.  (With a fixed share per wavefront the kernel ran as long as
+  // its slowest wavefront: the SIMD's arbiter favours its oldest wavefront, so the four
+  // wavefronts of a SIMD finish one after the other, and shares differ in their tap counts.)
+  // Every counter value is handed out once, values past the range end a wavefront's stream.
+  const int xcd = blockIdx.x & 7, blk = blockIdx.x >> 3, blocks_per_xcd = gridDim.x >> 3;
+  const int set_begin = xcd * sets_per_xcd;
+  const int set_end = min(n_sets, set_begin + sets_per_xcd);
+  const int first_round = blocks_per_xcd * WAVES;
+  int *ctr = queue + xcd * 32;
+  auto take = [&]() {
+    int v = 0;
+    if (lane == 0) v = atomicAdd(ctr, 1);
+    return set_begin + first_round + __builtin_amdgcn_readfirstlane(v);
+  };
+  // generator of the item stream (wave-uniform state)
+  int g_set = set_begin + blk * WAVES + wave;
+  bool g_has = g_set < set_end;
+  unsigned g_rest = g_has ? set_mask(g_set) : 0u;
+  int g_next = take();           // the set after g_set
+  unsigned g_mask_next = 0;      // its tap mask, read two items after g_next was requested
+  int g_age = 0;
+  struct Item {
+    int k, set;
+    bool last, valid;
+  };
+  auto gen = [&]() {
+    if (++g_age == 2) g_mask_next = set_mask(min(g_next, n_sets - 1));
+    Item it;
+    it.valid = g_has;
+    it.set = g_has ? g_set : 0;
+    it.k = g_has ? __ffs(g_rest) - 1 : 0;
+    g_rest &= g_rest - 1;
+    it.last = g_has && g_rest == 0u;
+    if (it.last) {
+      if (g_age < 2) g_mask_next = set_mask(min(g_next, n_sets - 1));  // a set of one or two taps
+      g_set = g_next;
+      g_has = g_set < set_end;
+      g_rest = g_mask_next;
+      if (g_has) {
+        g_next = take();
+        g_age = 0;
+      }
+    }
+    return it;
+  };
+  // Register rings, indexed by item number mod 3 (the loop below is unrolled three times so
+  // that every index is a constant): neighbour indices, gathered rows, row-present bits.
+  int jr[3][RG];
+  v4f ar[3][RG][SS];
+  unsigned okr[3];
+  auto issue_j = [&](const Item &it, int *j) {
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int64_t pos = t0 + q * 16 + 4 * g + r;
-        if (pos >= n) continue;
-        const int64_t row = rowmap ? rowmap[pos] : pos;
-        float *o = out + row * n_out;
+    for (int q = 0; q < RG; q++) {
+      const int64_t t = min((int64_t)it.set * (RG * 16) + q * 16 + r16, n - 1);
+      j[q] = nbr[(int64_t)it.k * npad + t];
+    }
+  };
+  auto issue_a = [&](const Item &it, const int *j, v4f (*a)[SS], unsigned &okbits) {
+    okbits = 0;
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) {
-          const int col = 16 * cb + r16;
-          if (col < n_out) o[col] = acc[q][cb][r] + (accumulate ? o[col] : bv[cb]);
+    for (int q = 0; q < RG; q++) {
+      const bool ok = j[q] >= 0 && (int64_t)it.set * (RG * 16) + q * 16 + r16 < n;
+      okbits |= ok ? 1u << q : 0u;
+      const float *src = in + (int64_t)(ok ? j[q] : 0) * in_stride;
+#pragma unroll
+      for (int s = 0; s < SS; s++) {
+        const int c0 = s * 16 + 4 * g;
+        if (VEC4) {
+          const int cc = c0 < n_in ? c0 : n_in - 4;
+          a[q][s] = *reinterpret_cast<const v4f *>(src + cc);
+        } else {
+          a[q][s].x = src[min(c0 + 0, n_in - 1)];
+          a[q][s].y = src[min(c0 + 1, n_in - 1)];
+          a[q][s].z = src[min(c0 + 2, n_in - 1)];
+          a[q][s].w = src[min(c0 + 3, n_in - 1)];
         }
       }
     }
+  };
+
+  v4f acc[RG][NCB];
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  // Items in flight: I0 runs its MFMAs now, I1's rows are on their way, I2's indices have
+  // arrived (its rows are requested next), I3's indices are on their way.
+  Item I0 = gen(), I1 = gen(), I2 = gen(), I3 = gen();
+  issue_j(I0, jr[0]);
+  issue_j(I1, jr[1]);
+  issue_a(I0, jr[0], ar[0], okr[0]);
+  issue_j(I2, jr[2]);
+  issue_a(I1, jr[1], ar[1], okr[1]);
+  issue_j(I3, jr[0]);
+
+  auto step = [&](auto slot) {
+    constexpr int S = decltype(slot)::value, S1 = (S + 1) % 3, S2 = (S + 2) % 3;
+    issue_a(I2, jr[S2], ar[S2], okr[S2]);
+    const Item I4 = gen();
+    issue_j(I4, jr[S1]);
+
+    const int64_t t0 = (int64_t)I0.set * (RG * 16);
+    const int k_cur = I0.k;
+    const unsigned okb = okr[S];
+    if (__ballot(okb != 0u) != 0ull) {
+      v4f b[SS][NCB];
+#pragma unroll
+      for (int s = 0; s < SS; s++)
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) b[s][cb] = wl[((k_cur * SS + s) * NCB + cb) * 64 + lane];
+#pragma unroll
+      for (int q = 0; q < RG; q++) {
+        const bool ok = (okb >> q) & 1u;
+        if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
+#pragma unroll
+        for (int s = 0; s < SS; s++) {
+          const int c0 = s * 16 + 4 * g;
+          v4f av = pre_act<PRE>(ar[S][q][s], psc[s], psh[s], pre_leak);
+          if (VEC4) {
+            if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
+          } else {
+            if (!(ok && c0 + 0 < n_in)) av.x = 0.f;
+            if (!(ok && c0 + 1 < n_in)) av.y = 0.f;
+            if (!(ok && c0 + 2 < n_in)) av.z = 0.f;
+            if (!(ok && c0 + 3 < n_in)) av.w = 0.f;
+          }
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][cb].x, acc[q][cb], 0, 0, 0);
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][cb].y, acc[q][cb], 0, 0, 0);
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][cb].z, acc[q][cb], 0, 0, 0);
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][cb].w, acc[q][cb], 0, 0, 0);
+        }
+      }
+    }
+    if (I0.last) {  // the set is complete: write its rows, start the next set from zero
+#pragma unroll
+      for (int q = 0; q < RG; q++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int64_t pos = t0 + q * 16 + 4 * g + r;
+          if (pos < n) {
+            const int64_t row = rowmap ? rowmap[pos] : pos;
+            float *o = out + row * n_out;
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) {
+              const int col = 16 * cb + r16;
+              if (col < n_out) o[col] = acc[q][cb][r] + (accumulate ? o[col] : bv[cb]);
+            }
+          }
+        }
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    I0 = I1;
+    I1 = I2;
+    I2 = I3;
+    I3 = I4;
+  };
+  while (true) {  // items after the last valid one are invalid: every wavefront leaves here
+    if (!I0.valid) break;
+    step(std::integral_constant<int, 0>{});
+    if (!I0.valid) break;
+    step(std::integral_constant<int, 1>{});
+    if (!I0.valid) break;
+    step(std::integral_constant<int, 2>{});
   }
 }
 
@@ -856,8 +916,9 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
   m.wpack.reserve(packed);
   // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
+  m.queue.reserve(8 * 32);
   k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, w_in_stride_rows,
-                                                                           n_in_part, n_out, SS, NCB);
+                                                                           n_in_part, n_out, SS, NCB, m.queue.p);
   LAUNCH_CHECK();
   const size_t lds_bytes = (size_t)packed * sizeof(float);
   const int n_sets = (int)ceil_div(t.n, RG * 16);
@@ -872,9 +933,9 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
       attr_set = true;
     }
     const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32, ceil_div(sets_per_xcd, WAVES)));
-    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
+    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride, out,
                                                      m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                     accumulate, pre.sc, pre.sh, pre.leak);
+                                                     accumulate, pre.sc, pre.sh, pre.leak, m.queue.p);
   } else {
     constexpr int WAVES = 8;
     auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, PRE>;
@@ -886,16 +947,16 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
     }
     const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / std::max<size_t>(lds_bytes, 1)));
     const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
-    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, in_stride, out,
+    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride, out,
                                                      m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                     accumulate, pre.sc, pre.sh, pre.leak);
+                                                     accumulate, pre.sc, pre.sh, pre.leak, m.queue.p);
   }
   LAUNCH_CHECK();
 }
 
 // Narrow layers: nOut <= 32, any nIn, K <= 32.  nIn is processed in parts of up to 32
 // channels so that every part's weights fit in LDS; parts after the first accumulate.
-static bool resident_fits(const Table &t, int n_out) { return t.K <= 32 && n_out <= 32; }
+static bool resident_fits(const Table &t, int n_out) { return t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr; }
 
 // No fused batch norm here: this kernel's time goes into the vector instructions around its
 // small MFMA blocks, and normalising every gathered value (each row is gathered once per tap

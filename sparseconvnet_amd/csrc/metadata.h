@@ -44,6 +44,7 @@ struct Table {
   int64_t n = 0, npad = 0;
   DevBuf<int> nbr;
   DevBuf<int> rowmap;
+  DevBuf<unsigned> gmask;  // K <= 32 and pattern-sorted: bit k of gmask[i] = some position of granule i (16 positions) has tap k
   bool identity_rows = false;  // rowmap[t] == t: kernels skip the indirection
   const int *rowmap_ptr() const { return identity_rows ? nullptr : rowmap.p; }
   std::vector<int64_t> counts;
@@ -85,6 +86,7 @@ struct Metadata {
   DevBuf<int> dflags;
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
+  DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
   DevBuf<float> bntmp;    // normalised input when a fused batch norm has no fused kernel
 };

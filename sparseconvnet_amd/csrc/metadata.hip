@@ -512,14 +512,19 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
 // (by 20-30% for 64..256 channels) and one global sort (which loses the locality).
 static const int PATTERN_WINDOWS = 8;
 
-__global__ void k_table_masks(int64_t window, const int *nbr, int K, int64_t n, int64_t npad, unsigned long long *keys,
-                              int *idx) {
+// Sort key of a position: window, then (when the bits allow) the number of absent taps, then
+// the tap mask.  Inside a window the positions with the most taps come first and the
+// cheapest last, which shortens the tail of kernels that hand positions out in order.
+__global__ void k_table_masks(int64_t window, int pc_bits, const int *nbr, int K, int64_t n, int64_t npad,
+                              unsigned long long *keys, int *idx) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n) return;
   unsigned long long mask = 0;
   for (int k = 0; k < K; k++)
     if (nbr[(int64_t)k * npad + t] >= 0) mask |= 1ull << k;
-  keys[t] = ((unsigned long long)(t / window) << K) | mask;
+  unsigned long long hi = (unsigned long long)(t / window);
+  if (pc_bits) hi = (hi << pc_bits) | (unsigned long long)(K - __popcll(mask));
+  keys[t] = (hi << K) | mask;
   idx[t] = (int)t;
 }
 __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, const int *perm,
@@ -531,6 +536,18 @@ __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, 
   int src = perm[t];
   nbr2[(int64_t)k * npad + t] = nbr[(int64_t)k * npad + src];
   if (k == 0) rowmap[t] = base ? base[src] : src;
+}
+// sorted keys carry each position's tap mask in their low K bits (K <= 32)
+__global__ void k_granule_masks(const unsigned long long *skeys, int K, int64_t n, int64_t n_granules,
+                                unsigned *gmask) {
+  int64_t gi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gi >= n_granules) return;
+  unsigned long long m = 0;
+  for (int r = 0; r < 16; r++) {
+    const int64_t t = gi * 16 + r;
+    if (t < n) m |= skeys[t];
+  }
+  gmask[gi] = (unsigned)(m & ((1ull << K) - 1ull));
 }
 __global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -560,9 +577,12 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   m.k1.reserve(t.n);
   m.v0.reserve(t.n);
   m.v1.reserve(t.n);
-  k_table_masks<<<grid_for(t.n), TB, 0, s>>>(window, t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p);
+  int pc_bits = 1;
+  while ((1 << pc_bits) <= t.K) pc_bits++;
+  if (t.K + pc_bits + block_bits > 62) pc_bits = 0;
+  k_table_masks<<<grid_for(t.n), TB, 0, s>>>(window, pc_bits, t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p);
   LAUNCH_CHECK();
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, t.K + block_bits);
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, t.K + pc_bits + block_bits);
   DevBuf<int> nbr2;
   nbr2.reserve((size_t)t.K * t.npad);
   k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
@@ -570,6 +590,12 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   LAUNCH_CHECK();
   t.nbr = std::move(nbr2);
   t.identity_rows = false;
+  if (t.K <= 32) {
+    const int64_t n_granules = ceil_div(t.n, 16);
+    t.gmask.reserve(n_granules);
+    k_granule_masks<<<grid_for(n_granules), TB, 0, s>>>(m.k1.p, t.K, t.n, n_granules, t.gmask.p);
+    LAUNCH_CHECK();
+  }
 }
 
 // Filter 3 in every dimension, dim 2 or 3 (the common case): the Morton key of a neighbour
