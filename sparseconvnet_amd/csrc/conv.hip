@@ -692,19 +692,22 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
 // the end re-read the first set).  Granules none of whose rows has the tap skip their MFMAs.
 // With accumulate != 0 the kernel adds to `out` instead of overwriting it (used to split a
 // wide nIn into several launches).
-template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool PRE>
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4>
 __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
     int64_t n, int64_t npad, const float *__restrict__ in, int in_stride, float *__restrict__ out,
     const float *__restrict__ wp, const float *__restrict__ bias, int n_in, int n_out, int n_sets,
-    int sets_per_xcd, int accumulate, const float *__restrict__ pre_sc, const float *__restrict__ pre_sh,
-    float pre_leak, int *__restrict__ queue) {
+    int sets_per_xcd, int accumulate, int *__restrict__ queue) {
+  static_assert(!C4 || SS == 1, "the four-channel layout has one slab");
+  // C4 (nIn <= 4): the MFMA's k index is the input channel itself, so a lane gathers one
+  // float (row r16, channel g) and a tap costs one MFMA per column block instead of four.
+  using AV = typename std::conditional<C4, float, v4f>::type;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  v4f *wl = reinterpret_cast<v4f *>(lds);  // [K][SS][NCB][64]
+  v4f *wl = reinterpret_cast<v4f *>(lds);  // [K][SS][NCB][64] float4, C4: [K][NCB][64] float
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
-  const int total_f4 = K * SS * NCB * 64;
+  const int total_f4 = C4 ? K * NCB * 16 : K * SS * NCB * 64;
   for (int e = threadIdx.x; e < total_f4; e += WAVES * 64) wl[e] = reinterpret_cast<const v4f *>(wp)[e];
   __syncthreads();  // the only barrier; every wavefront reaches it
 
@@ -713,12 +716,6 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   for (int cb = 0; cb < NCB; cb++) {
     const int col = 16 * cb + r16;
     bv[cb] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
-  }
-  v4f psc[SS], psh[SS];  // this lane always handles channels s*16 + 4*g .. +3
-#pragma unroll
-  for (int s = 0; s < SS; s++) {
-    psc[s] = PRE ? *reinterpret_cast<const v4f *>(pre_sc + s * 16 + 4 * g) : (v4f){1.f, 1.f, 1.f, 1.f};
-    psh[s] = PRE ? *reinterpret_cast<const v4f *>(pre_sh + s * 16 + 4 * g) : (v4f){0.f, 0.f, 0.f, 0.f};
   }
   const int64_t n_granules = (n + 15) >> 4;
   // Tap mask of a set; a set without any rule still runs one (empty) tap so that its rows
@@ -782,7 +779,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   // Register rings, indexed by item number mod 3 (the loop below is unrolled three times so
   // that every index is a constant): neighbour indices, gathered rows, row-present bits.
   int jr[3][RG];
-  v4f ar[3][RG][SS];
+  AV ar[3][RG][SS];
   unsigned okr[3];
   auto issue_j = [&](const Item &it, int *j) {
 #pragma unroll
@@ -791,7 +788,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
       j[q] = nbr[(int64_t)it.k * npad + t];
     }
   };
-  auto issue_a = [&](const Item &it, const int *j, v4f (*a)[SS], unsigned &okbits) {
+  auto issue_a = [&](const Item &it, const int *j, AV (*a)[SS], unsigned &okbits) {
     okbits = 0;
 #pragma unroll
     for (int q = 0; q < RG; q++) {
@@ -801,7 +798,9 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 #pragma unroll
       for (int s = 0; s < SS; s++) {
         const int c0 = s * 16 + 4 * g;
-        if (VEC4) {
+        if constexpr (C4) {
+          a[q][s] = src[min(g, n_in - 1)];
+        } else if constexpr (VEC4) {
           const int cc = c0 < n_in ? c0 : n_in - 4;
           a[q][s] = *reinterpret_cast<const v4f *>(src + cc);
         } else {
@@ -840,35 +839,49 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int k_cur = I0.k;
     const unsigned okb = okr[S];
     if (__ballot(okb != 0u) != 0ull) {
-      v4f b[SS][NCB];
+      if constexpr (C4) {
+        float b[NCB];
 #pragma unroll
-      for (int s = 0; s < SS; s++)
+        for (int cb = 0; cb < NCB; cb++) b[cb] = lds[(k_cur * NCB + cb) * 64 + lane];
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) b[s][cb] = wl[((k_cur * SS + s) * NCB + cb) * 64 + lane];
+        for (int q = 0; q < RG; q++) {
+          const bool ok = (okb >> q) & 1u;
+          if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
+          const float av = (ok && g < n_in) ? ar[S][q][0] : 0.f;
 #pragma unroll
-      for (int q = 0; q < RG; q++) {
-        const bool ok = (okb >> q) & 1u;
-        if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[cb], acc[q][cb], 0, 0, 0);
+        }
+      } else {
+        v4f b[SS][NCB];
 #pragma unroll
-        for (int s = 0; s < SS; s++) {
-          const int c0 = s * 16 + 4 * g;
-          v4f av = pre_act<PRE>(ar[S][q][s], psc[s], psh[s], pre_leak);
-          if (VEC4) {
-            if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
-          } else {
-            if (!(ok && c0 + 0 < n_in)) av.x = 0.f;
-            if (!(ok && c0 + 1 < n_in)) av.y = 0.f;
-            if (!(ok && c0 + 2 < n_in)) av.z = 0.f;
-            if (!(ok && c0 + 3 < n_in)) av.w = 0.f;
+        for (int s = 0; s < SS; s++)
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) b[s][cb] = wl[((k_cur * SS + s) * NCB + cb) * 64 + lane];
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+          const bool ok = (okb >> q) & 1u;
+          if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
+#pragma unroll
+          for (int s = 0; s < SS; s++) {
+            const int c0 = s * 16 + 4 * g;
+            v4f av = ar[S][q][s];
+            if (VEC4) {
+              if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
+            } else {
+              if (!(ok && c0 + 0 < n_in)) av.x = 0.f;
+              if (!(ok && c0 + 1 < n_in)) av.y = 0.f;
+              if (!(ok && c0 + 2 < n_in)) av.z = 0.f;
+              if (!(ok && c0 + 3 < n_in)) av.w = 0.f;
+            }
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][cb].x, acc[q][cb], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][cb].y, acc[q][cb], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][cb].z, acc[q][cb], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][cb].w, acc[q][cb], 0, 0, 0);
           }
-#pragma unroll
-          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][cb].x, acc[q][cb], 0, 0, 0);
-#pragma unroll
-          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][cb].y, acc[q][cb], 0, 0, 0);
-#pragma unroll
-          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][cb].z, acc[q][cb], 0, 0, 0);
-#pragma unroll
-          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][cb].w, acc[q][cb], 0, 0, 0);
         }
       }
     }
@@ -907,51 +920,73 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   }
 }
 
+// B operands of the four-channel layout: wp[(k * NCB + cb) * 64 + lane] = w[k][lane / 16][16 cb + lane % 16].
+// Also clears the set counters, as k_pack_weights_part does.
+__global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, int n_out, int NCB, int *queue) {
+  if (blockIdx.x == 0 && threadIdx.x < 8) queue[threadIdx.x * 32] = 0;
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= K * NCB * 64) return;
+  const int lane = i & 63, cb = (i >> 6) % NCB, k = i / (64 * NCB);
+  const int ch = lane >> 4, col = 16 * cb + (lane & 15);
+  wp[i] = (ch < n_in && col < n_out) ? w[((int64_t)k * n_in + ch) * n_out + col] : 0.0f;
+}
+
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4>
+static void launch_resident_kernel(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
+                                   const float *bias, int n_in_part, int n_out, int accumulate, size_t lds_bytes,
+                                   int per_cu, hipStream_t s) {
+  auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, C4>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  160 * 1024));
+    attr_set = true;
+  }
+  const int n_sets = (int)ceil_div(t.n, RG * 16);
+  const int sets_per_xcd = (int)ceil_div(n_sets, 8);
+  const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
+  kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
+                                                   out, m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
+                                                   accumulate, m.queue.p);
+  LAUNCH_CHECK();
+}
+
 // One launch over channels [c_lo, c_lo + n_in_part) of the input rows.
-template <int NCB, int SS, bool VEC4, bool PRE>
+template <int NCB, int SS, bool VEC4>
 static void launch_resident_part(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
                                  const float *w, int w_in_stride_rows, const float *bias, int n_in_part,
-                                 int n_out, int accumulate, PreArgs pre, hipStream_t s) {
+                                 int n_out, int accumulate, hipStream_t s) {
   constexpr int RG = 2;  // 32 rows per set: measured faster than 64 (more wavefronts in flight)
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
   m.wpack.reserve(packed);
-  // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
   m.queue.reserve(8 * 32);
+  // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
   k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, w_in_stride_rows,
                                                                            n_in_part, n_out, SS, NCB, m.queue.p);
   LAUNCH_CHECK();
   const size_t lds_bytes = (size_t)packed * sizeof(float);
-  const int n_sets = (int)ceil_div(t.n, RG * 16);
-  const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   if (lds_bytes > 80 * 1024) {
-    constexpr int WAVES = 16;
-    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, PRE>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      attr_set = true;
-    }
-    const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32, ceil_div(sets_per_xcd, WAVES)));
-    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride, out,
-                                                     m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                     accumulate, pre.sc, pre.sh, pre.leak, m.queue.p);
+    launch_resident_kernel<NCB, RG, SS, VEC4, 16, false>(m, t, in, in_stride, out, bias, n_in_part, n_out, accumulate,
+                                                         lds_bytes, 1, s);
   } else {
-    constexpr int WAVES = 8;
-    auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, PRE>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      attr_set = true;
-    }
     const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / std::max<size_t>(lds_bytes, 1)));
-    const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
-    kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride, out,
-                                                     m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                     accumulate, pre.sc, pre.sh, pre.leak, m.queue.p);
+    launch_resident_kernel<NCB, RG, SS, VEC4, 8, false>(m, t, in, in_stride, out, bias, n_in_part, n_out, accumulate,
+                                                        lds_bytes, per_cu, s);
   }
+}
+
+// nIn <= 4 (the first layer of most networks): four-channel layout, 64 rows per set.
+template <int NCB>
+static void launch_resident_c4(Metadata &m, const Table &t, const float *in, float *out, const float *w,
+                               const float *bias, int n_in, int n_out, hipStream_t s) {
+  const int packed = t.K * NCB * 64;
+  m.wpack.reserve(packed);
+  m.queue.reserve(8 * 32);
+  k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, NCB,
+                                                                        m.queue.p);
   LAUNCH_CHECK();
+  launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, bias, n_in, n_out, 0,
+                                                    (size_t)packed * sizeof(float), 3, s);
 }
 
 // Narrow layers: nOut <= 32, any nIn, K <= 32.  nIn is processed in parts of up to 32
@@ -966,6 +1001,11 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
   if (!resident_fits(t, n_out)) return false;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   const int ncb = (int)ceil_div(n_out, 16);
+  if (n_in <= 4) {
+    if (ncb == 1) launch_resident_c4<1>(m, t, in, out, w, bias, n_in, n_out, s);
+    else launch_resident_c4<2>(m, t, in, out, w, bias, n_in, n_out, s);
+    return true;
+  }
   for (int c_lo = 0; c_lo < n_in; c_lo += 32) {
     const int part = std::min(32, n_in - c_lo);
     const float *in_p = in + c_lo;
@@ -975,11 +1015,9 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
 #define SCN_RES(NCBV, SSV)                                                                                   \
   do {                                                                                                       \
     if (vec4)                                                                                                \
-      launch_resident_part<NCBV, SSV, true, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc,    \
-                                                   PreArgs(), s);                                            \
+      launch_resident_part<NCBV, SSV, true>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc, s);       \
     else                                                                                                     \
-      launch_resident_part<NCBV, SSV, false, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc,   \
-                                                    PreArgs(), s);                                           \
+      launch_resident_part<NCBV, SSV, false>(m, t, in_p, n_in, out, w_p, n_in, b, part, n_out, acc, s);      \
   } while (0)
     if (ncb == 1 && part <= 16) SCN_RES(1, 1);
     else if (ncb == 1) SCN_RES(1, 2);
