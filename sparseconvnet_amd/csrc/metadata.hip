@@ -51,6 +51,21 @@ Geom make_geom(int dim, const int64_t *spatial) {
   return g;
 }
 
+// Number of low key bits that can be non-zero for sample indices below `batch`.
+static int key_bits(const Geom &g, int64_t batch) {
+  auto bitlen = [](uint64_t v) {
+    int b = 0;
+    while (v) {
+      b++;
+      v >>= 1;
+    }
+    return b;
+  };
+  batch = std::max<int64_t>(batch, 1);
+  if (g.dim <= 3) return g.dim * g.bits + bitlen((uint64_t)batch - 1);
+  return bitlen((uint64_t)batch * (uint64_t)g.vol - 1);
+}
+
 // ---- small utilities -------------------------------------------------------------------
 
 __global__ void k_fill32(uint32_t *p, uint32_t v, int64_t n) {
@@ -100,29 +115,35 @@ static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
 __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols,
                              unsigned long long *keys, int *idx, int *flags) {
+  // flags[0]: error bits, flags[3]: largest sample index (one atomic per wavefront)
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int64_t *c = coords + i * ncols;
-  int cc[SCN_MAXD];
-  bool ok = true;
-  for (int d = 0; d < g.dim; d++) {
-    int64_t v = c[d];
-    if (v < 0 || v >= g.size[d]) ok = false;
-    cc[d] = (int)v;
+  int bmax = 0;
+  if (i < n) {
+    const int64_t *c = coords + i * ncols;
+    int cc[SCN_MAXD];
+    bool ok = true;
+    for (int d = 0; d < g.dim; d++) {
+      int64_t v = c[d];
+      if (v < 0 || v >= g.size[d]) ok = false;
+      cc[d] = (int)v;
+    }
+    int64_t b = ncols > g.dim ? c[g.dim] : 0;
+    if (b < 0 || b >= g.max_batch) {
+      atomicOr(&flags[0], 2);
+      ok = false;
+      b = 0;
+    }
+    if (!ok) {
+      atomicOr(&flags[0], 1);
+      keys[i] = SCN_EMPTY_KEY;
+    } else {
+      keys[i] = site_key(g, cc, (int)b);
+    }
+    idx[i] = (int)i;
+    bmax = (int)b;
   }
-  int64_t b = ncols > g.dim ? c[g.dim] : 0;
-  if (b < 0 || b >= g.max_batch) {
-    atomicOr(&flags[0], 2);
-    ok = false;
-    b = 0;
-  }
-  if (!ok) {
-    atomicOr(&flags[0], 1);
-    keys[i] = SCN_EMPTY_KEY;
-  } else {
-    keys[i] = site_key(g, cc, (int)b);
-  }
-  idx[i] = (int)i;
+  for (int off = 32; off; off >>= 1) bmax = max(bmax, __shfl_xor(bmax, off));
+  if ((threadIdx.x & 63) == 0 && bmax > 0) atomicMax(&flags[3], bmax);
 }
 
 // mode 0: row = input index.
@@ -212,15 +233,14 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   fill32(m.dflags.p, 0, 8, s);
   k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, m.k0.p, m.v0.p, m.dflags.p);
   LAUNCH_CHECK();
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s);
-  int hflags[2];
-  unsigned long long top_key = 0;  // keys ascend with the sample index: the last one has the largest
+  int hflags[4];
   HIP_CHECK(hipMemcpyAsync(hflags, m.dflags.p, sizeof hflags, hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipMemcpyAsync(&top_key, m.k1.p + (n - 1), sizeof top_key, hipMemcpyDeviceToHost, s));
   HIP_CHECK(hipStreamSynchronize(s));
   if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
   if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");
-  const int top_batch = g.dim <= 3 ? (int)(top_key >> (g.dim * g.bits)) : (int)(top_key / (unsigned long long)g.vol);
+  const int top_batch = hflags[3];
+  // only the key bits that samples 0..top_batch can set take part in the sort
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s, key_bits(g, (int64_t)top_batch + 1));
   // Metadata/IOLayersRules.h:25,46-47,76-77: the batch is at least min_batch and grows to
   // the largest sample index + 1; without a sample column there is exactly one sample.
   int batch = ncols == m.dim ? 1 : std::max(batch_floor, top_batch + 1);
@@ -864,7 +884,19 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), n, LI.npad,
                                                    m.k0.p, m.v0.p);
   LAUNCH_CHECK();
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s);
+  // Filter = stride = 2 in every dimension over exactly fitting sizes (the U-Net's and most
+  // networks' downsampling): each site has one candidate, the Morton key of its coordinates
+  // halved, which ascends with the site's own key, so the schedule order is already sorted.
+  bool presorted = m.dim <= 3 && f.M == 1;
+  for (int d = 0; d < m.dim; d++)
+    presorted = presorted && filter[d] == 2 && stride[d] == 2 && in_size[d] == 2 * out_size[d];
+  if (presorted) {
+    std::swap(m.k0, m.k1);
+    std::swap(m.v0, m.v1);
+  } else {
+    // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
+    sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
+  }
   k_strided_heads<<<grid_for(nc), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
   LAUNCH_CHECK();
   exclusive_scan(m, m.f0.p, m.s0.p, nc, s);
