@@ -991,14 +991,19 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
 
 // Narrow layers: nOut <= 32, any nIn, K <= 32.  nIn is processed in parts of up to 32
 // channels so that every part's weights fit in LDS; parts after the first accumulate.
-static bool resident_fits(const Table &t, int n_out) { return t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr; }
+// The resident kernel serves nOut <= 32 with up to 32 taps.  It takes the input channels in
+// parts of 32 and has no fused batch norm, so from 128 input channels on, or from 64 when a
+// batch norm comes with the call, the row-owner kernel is at least as fast (measured).
+static bool resident_fits(const Table &t, int n_in, int n_out, bool with_bn) {
+  return t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr && n_in < (with_bn ? 64 : 128);
+}
 
 // No fused batch norm here: this kernel's time goes into the vector instructions around its
 // small MFMA blocks, and normalising every gathered value (each row is gathered once per tap
 // that reaches it) costs more than one extra pass over the rows.
 static bool try_resident(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                          const float *bias, int n_in, int n_out, hipStream_t s) {
-  if (!resident_fits(t, n_out)) return false;
+  if (!resident_fits(t, n_in, n_out, false)) return false;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   const int ncb = (int)ceil_div(n_out, 16);
   if (n_in <= 4) {
@@ -1037,6 +1042,9 @@ static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *o
                           const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   const int ncb = (int)ceil_div(n_out, 16);
   const bool narrow = n_in <= 16;
+  if (ncb <= 2)
+    return narrow ? launch_rows<2, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
+                  : launch_rows<2, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
   if (ncb <= 4)
     return narrow ? launch_rows<4, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
                   : launch_rows<4, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
@@ -1076,7 +1084,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
-  if (bn && groups == 1 && !resident_fits(t, n_out)) {
+  if (bn && groups == 1 && !resident_fits(t, n_in, n_out, true)) {
     const int n_pad = (int)round_up(n_in, 64) + 64;
     m.prebuf.reserve(2 * (size_t)n_pad);
     k_pre_coeffs<<<dim3((unsigned)ceil_div(n_pad, 256)), 256, 0, s>>>(bn->mean, bn->var, bn->gamma, bn->beta, bn->eps,
