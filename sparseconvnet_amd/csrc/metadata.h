@@ -36,9 +36,10 @@ struct Level {
 
 // Neighbour table: nbr[k * npad + t] = row feeding filter tap k of the output row at
 // position t, or -1; rowmap[t] = that output row.  Positions follow the level's schedule
-// (ascending site key), then inside every block of 256 positions they are sorted by
-// neighbour pattern (the bit mask of present taps), so that the 16 positions a wavefront
-// works on mostly need the same taps.  counts[k] = number of non-negative entries of tap k.
+// (ascending site key), then inside each of a few equal ranges of that order they are sorted
+// by neighbour pattern (number of absent taps, then the bit mask of present taps), so that
+// the positions a workgroup takes mostly need the same taps.  counts[k] = number of
+// non-negative entries of tap k.
 struct Table {
   int K = 0;
   int64_t n = 0, npad = 0;

@@ -6,7 +6,9 @@
 //   * sites are packed into 64-bit keys (common.h) and radix-sorted; equal keys become
 //     adjacent, which yields duplicate groups (input layer), the distinct output sites of
 //     a strided convolution, and a spatially coherent row schedule, all without atomics;
-//   * submanifold neighbours are found in an open-addressing table of (key -> row);
+//   * neighbours are found through a block-occupancy grid: one table entry per block of 64
+//     consecutive key values (occupancy mask + rank of its first site), so the taps of a
+//     filter box mostly re-use the entry of the previous tap;
 //   * rules are stored output-stationary as a table nbr[tap][position] instead of
 //     per-tap pair lists; pair lists are produced on demand by ballot/prefix compaction.
 #include <hipcub/hipcub.hpp>
