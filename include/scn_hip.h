@@ -128,27 +128,26 @@ int scn_deconv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_
                    const int64_t *filter, const int64_t *stride, const float *in, float *out,
                    const float *weight, const float *bias, int n_in, int n_out, int groups,
                    void *stream, double *macs);
-/* Fused pairs: an eval-mode batch norm + leaky ReLU on the input rows followed by one of the
- * three convolutions above, i.e. BatchNormalization_updateOutput(train=false) (pybind.cpp:220,
- * CPU/BatchNormalization.cpp:41-61) then the convolution, without writing the normalised rows
- * to memory.  This is the order of every U-Net block (networkArchitectures.py:232-234).
- * Same arguments as the plain calls plus the batch-norm tensors (device, [n_in]; gamma/beta
- * may be NULL).  Results equal the two separate calls up to fp32 rounding. */
-int scn_bn_subm_conv_fwd(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
-                         const float *in, float *out, const float *weight, const float *bias,
-                         int n_in, int n_out, int groups, const float *running_mean,
-                         const float *running_var, const float *gamma, const float *beta, float eps,
-                         float leakiness, void *stream, double *macs);
-int scn_bn_conv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
-                    const int64_t *filter, const int64_t *stride, const float *in, float *out,
+/* A convolution with the eval-mode batch norms + leaky ReLUs next to it folded in:
+ * BatchNormalization_updateOutput(train=false) (pybind.cpp:220, CPU/BatchNormalization.cpp:41-61)
+ * of the layer in front (`pre`, over the n_in input planes, applied while the input rows are
+ * gathered) and / or of the layer behind (`post`, over the n_out output planes, applied as the
+ * output rows are stored), so that neither layer reads and writes the feature matrix itself.
+ * Every block of the reference's U-Net is such a pair (networkArchitectures.py:232-234).
+ * kind 0: SubmanifoldConvolution (a = spatial, b = filter, c = d = NULL); 1: Convolution,
+ * 2: Deconvolution (a = in_size, b = out_size, c = filter, d = stride); the other arguments
+ * are those of the plain calls.  pre / post may be NULL.  Results equal the separate calls up
+ * to fp32 rounding. */
+typedef struct scn_bn_params {
+  const float *running_mean, *running_var; /* device, [planes] */
+  const float *gamma, *beta;               /* device, [planes], or NULL */
+  float eps, leakiness;
+} scn_bn_params;
+int scn_conv_bn_fwd(scn_metadata *md, int kind, const int64_t *a, const int64_t *b,
+                    const int64_t *c, const int64_t *d, const float *in, float *out,
                     const float *weight, const float *bias, int n_in, int n_out, int groups,
-                    const float *running_mean, const float *running_var, const float *gamma,
-                    const float *beta, float eps, float leakiness, void *stream, double *macs);
-int scn_bn_deconv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
-                      const int64_t *filter, const int64_t *stride, const float *in, float *out,
-                      const float *weight, const float *bias, int n_in, int n_out, int groups,
-                      const float *running_mean, const float *running_var, const float *gamma,
-                      const float *beta, float eps, float leakiness, void *stream, double *macs);
+                    const scn_bn_params *pre, const scn_bn_params *post, void *stream,
+                    double *macs);
 /* MaxPooling_updateOutput (pybind.cpp:103-107, CPU/MaxPooling.cpp:37-60).
  * in [nActive(in_size), in_stride] -> out [nActive(out_size), planes] where
  * planes = in_stride - n_features_to_drop; the result is max(0, inputs of the window). */

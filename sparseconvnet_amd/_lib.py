@@ -12,6 +12,13 @@ LIB_PATH = os.path.join(_HERE, "libscn_hip.so")
 _i64p = C.POINTER(C.c_int64)
 _vp = C.c_void_p
 
+
+class BnParams(C.Structure):
+    """scn_bn_params of include/scn_hip.h: an eval-mode batch norm + leaky ReLU."""
+    _fields_ = [("running_mean", _vp), ("running_var", _vp), ("gamma", _vp), ("beta", _vp),
+                ("eps", C.c_float), ("leakiness", C.c_float)]
+
+
 # name -> (restype, argtypes); mirrors include/scn_hip.h line by line
 SIGNATURES = {
     "scn_last_error": (C.c_char_p, []),
@@ -38,14 +45,8 @@ SIGNATURES = {
                                C.c_int, _vp, C.POINTER(C.c_double)]),
     "scn_deconv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
                                  C.c_int, _vp, C.POINTER(C.c_double)]),
-    "scn_bn_subm_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int,
-                                       _vp, _vp, _vp, _vp, C.c_float, C.c_float, _vp, C.POINTER(C.c_double)]),
-    "scn_bn_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
-                                  C.c_int, _vp, _vp, _vp, _vp, C.c_float, C.c_float, _vp,
-                                  C.POINTER(C.c_double)]),
-    "scn_bn_deconv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
-                                    C.c_int, _vp, _vp, _vp, _vp, C.c_float, C.c_float, _vp,
-                                    C.POINTER(C.c_double)]),
+    "scn_conv_bn_fwd": (C.c_int, [_vp, C.c_int, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
+                                  C.c_int, C.POINTER(BnParams), C.POINTER(BnParams), _vp, C.POINTER(C.c_double)]),
     "scn_maxpool_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int,
                                   _vp]),
     "scn_bn_eval_fwd": (C.c_int, [_vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp,

@@ -7,20 +7,33 @@ from .tensor import SparseConvNetTensor
 
 
 class Sequential(torch.nn.Sequential):
+    def _chain(self):
+        """The modules this container runs, with nested plain Sequentials (no hooks of their
+        own) spliced in, so that a batch normalisation and a convolution that meet across the
+        boundary of two blocks can still be run as one."""
+        out = []
+        for m in self._modules.values():
+            if type(m) is Sequential and not m._forward_hooks and not m._forward_pre_hooks:
+                out.extend(m._chain())
+            else:
+                out.append(m)
+        return out
+
     def forward(self, input):
-        # Same chain as sequential.py:10-35, except that an eval-mode batch normalisation
-        # directly in front of a convolution is applied inside that convolution's gather.
-        from .layers import fusable_pair
-        mods = list(self._modules.values())
+        # Same chain as sequential.py:10-35, except that eval-mode batch normalisations next
+        # to a convolution are applied inside that convolution (layers.fuse_plan).
+        from .layers import fuse_plan
+        mods = self._chain()
         i = 0
         while i < len(mods):
-            if i + 1 < len(mods) and isinstance(input, SparseConvNetTensor) and \
-                    fusable_pair(mods[i], mods[i + 1], input):
-                input = mods[i + 1](input, pre_bn=mods[i])
-                i += 2
-            else:
+            plan = fuse_plan(mods[i:i + 3], input) if isinstance(input, SparseConvNetTensor) else None
+            if plan is None:
                 input = mods[i](input)
                 i += 1
+            else:
+                conv, pre, post, used = plan
+                input = conv(input, pre_bn=pre, post_bn=post)
+                i += used
         return input
 
     def input_spatial_size(self, out_size):

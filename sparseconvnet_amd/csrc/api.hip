@@ -231,79 +231,80 @@ static int64_t level_rows(Metadata &m, const int64_t *spatial) {
   return l ? l->n : 0;
 }
 static void subm_conv(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in, float *out,
-                      const float *weight, const float *bias, int n_in, int n_out, int groups, const BnArgs *bn,
-                      void *stream, double *macs) {
+                      const float *weight, const float *bias, int n_in, int n_out, int groups, const BnArgs *pre,
+                      const BnArgs *post, void *stream, double *macs) {
   Metadata &m = md(h);
   Table &t = submanifold_rules(m, spatial, filter, st(stream));
-  conv_forward(m, t, in, level_rows(m, spatial), out, weight, bias, n_in, n_out, groups, bn, st(stream));
+  conv_forward(m, t, in, level_rows(m, spatial), out, weight, bias, n_in, n_out, groups, pre, post, st(stream));
   // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
   if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
 }
 static void strided_conv(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                          const int64_t *stride, const float *in, float *out, const float *weight,
-                         const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, void *stream,
-                         double *macs) {
+                         const float *bias, int n_in, int n_out, int groups, const BnArgs *pre, const BnArgs *post,
+                         void *stream, double *macs) {
   Metadata &m = md(h);
   StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
-  conv_forward(m, r.by_out, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, bn, st(stream));
+  conv_forward(m, r.by_out, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
+               st(stream));
   if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
 }
 static void deconv(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                    const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
-                   int n_in, int n_out, int groups, const BnArgs *bn, void *stream, double *macs) {
+                   int n_in, int n_out, int groups, const BnArgs *pre, const BnArgs *post, void *stream,
+                   double *macs) {
   Metadata &m = md(h);
   // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
   StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
-  conv_forward(m, r.by_in, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, bn, st(stream));
+  conv_forward(m, r.by_in, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
+               st(stream));
   if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
 }
 
 int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,
                       float *out, const float *weight, const float *bias, int n_in, int n_out,
                       int groups, void *stream, double *macs) {
-  return guarded([&] { subm_conv(h, spatial, filter, in, out, weight, bias, n_in, n_out, groups, nullptr, stream, macs); });
+  return guarded([&] {
+    subm_conv(h, spatial, filter, in, out, weight, bias, n_in, n_out, groups, nullptr, nullptr, stream, macs);
+  });
 }
 int scn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                  const int64_t *stride, const float *in, float *out, const float *weight,
                  const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {
   return guarded([&] {
-    strided_conv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, nullptr, stream, macs);
+    strided_conv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, nullptr, nullptr,
+                 stream, macs);
   });
 }
 int scn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                    const int64_t *stride, const float *in, float *out, const float *weight,
                    const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {
   return guarded([&] {
-    deconv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, nullptr, stream, macs);
+    deconv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, nullptr, nullptr, stream,
+           macs);
   });
 }
-int scn_bn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,
-                         float *out, const float *weight, const float *bias, int n_in, int n_out, int groups,
-                         const float *running_mean, const float *running_var, const float *gamma,
-                         const float *beta, float eps, float leakiness, void *stream, double *macs) {
+int scn_conv_bn_fwd(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
+                    const int64_t *d, const float *in, float *out, const float *weight, const float *bias,
+                    int n_in, int n_out, int groups, const scn_bn_params *pre, const scn_bn_params *post,
+                    void *stream, double *macs) {
   return guarded([&] {
-    BnArgs bn{running_mean, running_var, gamma, beta, eps, leakiness};
-    subm_conv(h, spatial, filter, in, out, weight, bias, n_in, n_out, groups, &bn, stream, macs);
-  });
-}
-int scn_bn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
-                    const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
-                    int n_in, int n_out, int groups, const float *running_mean, const float *running_var,
-                    const float *gamma, const float *beta, float eps, float leakiness, void *stream,
-                    double *macs) {
-  return guarded([&] {
-    BnArgs bn{running_mean, running_var, gamma, beta, eps, leakiness};
-    strided_conv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, &bn, stream, macs);
-  });
-}
-int scn_bn_deconv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
-                      const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
-                      int n_in, int n_out, int groups, const float *running_mean, const float *running_var,
-                      const float *gamma, const float *beta, float eps, float leakiness, void *stream,
-                      double *macs) {
-  return guarded([&] {
-    BnArgs bn{running_mean, running_var, gamma, beta, eps, leakiness};
-    deconv(h, in_size, out_size, filter, stride, in, out, weight, bias, n_in, n_out, groups, &bn, stream, macs);
+    BnArgs pre_a{}, post_a{};
+    auto conv = [](const scn_bn_params *p, BnArgs &o) -> const BnArgs * {
+      if (!p) return nullptr;
+      if (!p->running_mean || !p->running_var) throw Error("batch norm parameters need running_mean and running_var");
+      o = BnArgs{p->running_mean, p->running_var, p->gamma, p->beta, p->eps, p->leakiness};
+      return &o;
+    };
+    const BnArgs *pa = conv(pre, pre_a), *po = conv(post, post_a);
+    if (kind == 0)
+      subm_conv(h, a, b, in, out, weight, bias, n_in, n_out, groups, pa, po, stream, macs);
+    else if (kind == 1)
+      strided_conv(h, a, b, c, d, in, out, weight, bias, n_in, n_out, groups, pa, po, stream, macs);
+    else if (kind == 2)
+      deconv(h, a, b, c, d, in, out, weight, bias, n_in, n_out, groups, pa, po, stream, macs);
+    else
+      throw Error("scn_conv_bn_fwd: kind must be 0 (submanifold), 1 (strided) or 2 (transposed)");
   });
 }
 int scn_maxpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,

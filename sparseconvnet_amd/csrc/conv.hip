@@ -30,6 +30,18 @@ template <bool PRE> __device__ inline v4f pre_act(v4f v, v4f sc, v4f sh, float l
   y.w *= (y.w > 0.f ? 1.f : leak);
   return y;
 }
+// What happens to an accumulated output value before it is stored: + bias, then optionally the
+// eval batch norm + leaky ReLU of the layer that follows (folded to scale / shift per output
+// channel), so that layer needs no pass of its own.
+struct Epi {
+  const float *bias = nullptr;               // [nOut] or null
+  const float *sc = nullptr, *sh = nullptr;  // [nOut] each, or nulls
+  float leak = 1.0f;
+};
+__device__ inline float epi_act(float v, float sc, float sh, float leak) {
+  const float y = v * sc + sh;
+  return y > 0.f ? y : y * leak;
+}
 __global__ void k_pre_coeffs(const float *mean, const float *var, const float *gamma, const float *beta, float eps,
                              int n_in, int n_pad, float *sc, float *sh) {
   int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -45,7 +57,7 @@ __global__ void k_pre_coeffs(const float *mean, const float *var, const float *g
 
 // ---- generic kernel: any channel counts, any groups -------------------------------------
 __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad,
-                               const float *in, float *out, const float *w, const float *bias, int n_in,
+                               const float *in, float *out, const float *w, Epi epi, int n_in,
                                int n_out, int groups) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = n * n_out;
@@ -54,7 +66,7 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
   int oc = (int)(i - t * n_out);
   int ip = n_in / groups, op = n_out / groups;
   int g = oc / op, ocg = oc - g * op;
-  float acc = bias ? bias[oc] : 0.0f;
+  float acc = epi.bias ? epi.bias[oc] : 0.0f;
   for (int k = 0; k < K; k++) {
     int j = nbr[(int64_t)k * npad + t];
     if (j < 0) continue;
@@ -64,6 +76,7 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
     for (int c = 0; c < ip; c++) a += x[c] * wk[(int64_t)c * op];
     acc += a;
   }
+  if (epi.sc) acc = epi_act(acc, epi.sc[oc], epi.sh[oc], epi.leak);
   int64_t row = rowmap ? rowmap[t] : t;
   out[row * n_out + oc] = acc;
 }
@@ -140,7 +153,7 @@ template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE>
 __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
-    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
+    Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak) {
   constexpr int WR = 4 / WC;
@@ -324,11 +337,14 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
           pt[(int64_t)((wr * GW + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * (wc * NCBW + c) + r16] = acc[q][c][r];
     return;
   }
-  float bv[NCBW];
+  float bv[NCBW], es[NCBW], eh[NCBW];
+  const bool post = epi.sc != nullptr;
 #pragma unroll
   for (int c = 0; c < NCBW; c++) {
     const int col = 16 * (wc * NCBW + c) + r16;
-    bv[c] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+    bv[c] = (epi.bias != nullptr && col < n_out) ? epi.bias[col] : 0.0f;
+    es[c] = (post && col < n_out) ? epi.sc[col] : 1.0f;
+    eh[c] = (post && col < n_out) ? epi.sh[col] : 0.0f;
   }
 #pragma unroll
   for (int q = 0; q < GW; q++) {
@@ -341,21 +357,24 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 #pragma unroll
       for (int c = 0; c < NCBW; c++) {
         const int col = 16 * (wc * NCBW + c) + r16;
-        if (col < n_out) o[col] = acc[q][c][r] + bv[c];
+        float v = acc[q][c][r] + bv[c];
+        if (post) v = epi_act(v, es[c], eh[c], epi.leak);
+        if (col < n_out) o[col] = v;
       }
     }
   }
 }
 
-// out[rowmap[pos]][col] = bias[col] + sum over splits of partial[split][pos][col]
+// out[rowmap[pos]][col] = epilogue(bias[col] + sum over splits of partial[split][pos][col])
 __global__ void k_conv_reduce(const float *partial, int n_split, int64_t split_stride, int ld, const int *rowmap,
-                              int64_t n, const float *bias, float *out, int n_out) {
+                              int64_t n, Epi epi, float *out, int n_out) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n * n_out) return;
   int64_t pos = i / n_out;
   int col = (int)(i - pos * n_out);
-  float acc = bias ? bias[col] : 0.0f;
+  float acc = epi.bias ? epi.bias[col] : 0.0f;
   for (int sp = 0; sp < n_split; sp++) acc += partial[sp * split_stride + pos * ld + col];
+  if (epi.sc) acc = epi_act(acc, epi.sc[col], epi.sh[col], epi.leak);
   int64_t row = rowmap ? rowmap[pos] : pos;
   out[row * n_out + col] = acc;
 }
@@ -367,7 +386,7 @@ struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
 
 template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE>
 static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                        const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+                        Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
   constexpr int WPT = (SS * NCB * 64 + 255) / 256;
   constexpr int SLAB_STRIDE = WPT * 256 * 4;  // floats
@@ -400,12 +419,12 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
     partial = m.partial.p;
   }
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), 256, lds_bytes, s>>>(
-      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, tiles_per_xcd,
+      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, epi, n_in, n_out, n_slab, tiles_per_xcd,
       n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak);
   LAUNCH_CHECK();
   if (n_split > 1) {
     k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
-                                                                          t.rowmap_ptr(), t.n, bias, out, n_out);
+                                                                          t.rowmap_ptr(), t.n, epi, out, n_out);
     LAUNCH_CHECK();
   }
   return true;
@@ -416,12 +435,12 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
 // hides the other's staging.  A slab is one 16-channel step when nIn <= 16 or nOut > 128.
 template <bool VEC4, bool PRE>
 static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                         const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   const bool narrow = n_in <= 16;
 #define SCN_CASE(N, NCBW, WC, GW, SSW)                                                                      \
   if (ncb <= N)                                                                                             \
-    return narrow ? launch_mfma<NCBW, WC, GW, 1, VEC4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)    \
-                  : launch_mfma<NCBW, WC, GW, SSW, VEC4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
+    return narrow ? launch_mfma<NCBW, WC, GW, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)    \
+                  : launch_mfma<NCBW, WC, GW, SSW, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
   SCN_CASE(1, 1, 1, 2, 2)
   SCN_CASE(2, 1, 2, 4, 2)
   SCN_CASE(4, 1, 4, 8, 2)
@@ -446,7 +465,7 @@ template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE>
 __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
-    const float *__restrict__ bias, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
+    Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak) {
   constexpr int NT = NW * 64;
@@ -610,11 +629,14 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
           pt[(int64_t)((wave * RG + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * cb + r16] = acc[q][cb][r];
     return;
   }
-  float bv[NCB];
+  float bv[NCB], es[NCB], eh[NCB];
+  const bool post = epi.sc != nullptr;
 #pragma unroll
   for (int cb = 0; cb < NCB; cb++) {
     const int col = 16 * cb + r16;
-    bv[cb] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+    bv[cb] = (epi.bias != nullptr && col < n_out) ? epi.bias[col] : 0.0f;
+    es[cb] = (post && col < n_out) ? epi.sc[col] : 1.0f;
+    eh[cb] = (post && col < n_out) ? epi.sh[col] : 0.0f;
   }
 #pragma unroll
   for (int q = 0; q < RG; q++) {
@@ -627,7 +649,9 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 #pragma unroll
       for (int cb = 0; cb < NCB; cb++) {
         const int col = 16 * cb + r16;
-        if (col < n_out) o[col] = acc[q][cb][r] + bv[cb];
+        float v = acc[q][cb][r] + bv[cb];
+        if (post) v = epi_act(v, es[cb], eh[cb], epi.leak);
+        if (col < n_out) o[col] = v;
       }
     }
   }
@@ -635,7 +659,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 
 template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE>
 static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                        const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+                        Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   constexpr int NT = NW * 64, G = NW * RG;
   constexpr int SLAB_F4 = SS * NCB * 64;
   constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
@@ -667,12 +691,12 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
     partial = m.partial.p;
   }
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), NT, lds_bytes, s>>>(
-      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, bias, n_in, n_out, n_slab, tiles_per_xcd,
+      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, epi, n_in, n_out, n_slab, tiles_per_xcd,
       n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak);
   LAUNCH_CHECK();
   if (n_split > 1) {
     k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
-                                                                          t.rowmap_ptr(), t.n, bias, out, n_out);
+                                                                          t.rowmap_ptr(), t.n, epi, out, n_out);
     LAUNCH_CHECK();
   }
   return true;
@@ -696,7 +720,7 @@ template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4>
 __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
     int64_t n, int64_t npad, const float *__restrict__ in, int in_stride, float *__restrict__ out,
-    const float *__restrict__ wp, const float *__restrict__ bias, int n_in, int n_out, int n_sets,
+    const float *__restrict__ wp, Epi epi, int n_in, int n_out, int n_sets,
     int sets_per_xcd, int accumulate, int *__restrict__ queue) {
   static_assert(!C4 || SS == 1, "the four-channel layout has one slab");
   // C4 (nIn <= 4): the MFMA's k index is the input channel itself, so a lane gathers one
@@ -711,11 +735,14 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   for (int e = threadIdx.x; e < total_f4; e += WAVES * 64) wl[e] = reinterpret_cast<const v4f *>(wp)[e];
   __syncthreads();  // the only barrier; every wavefront reaches it
 
-  float bv[NCB];
+  float bv[NCB], es[NCB], eh[NCB];
+  const bool post = epi.sc != nullptr;
 #pragma unroll
   for (int cb = 0; cb < NCB; cb++) {
     const int col = 16 * cb + r16;
-    bv[cb] = (bias != nullptr && col < n_out) ? bias[col] : 0.0f;
+    bv[cb] = (epi.bias != nullptr && col < n_out) ? epi.bias[col] : 0.0f;
+    es[cb] = (post && col < n_out) ? epi.sc[col] : 1.0f;
+    eh[cb] = (post && col < n_out) ? epi.sh[col] : 0.0f;
   }
   const int64_t n_granules = (n + 15) >> 4;
   // Tap mask of a set; a set without any rule still runs one (empty) tap so that its rows
@@ -897,7 +924,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 #pragma unroll
             for (int cb = 0; cb < NCB; cb++) {
               const int col = 16 * cb + r16;
-              if (col < n_out) o[col] = acc[q][cb][r] + (accumulate ? o[col] : bv[cb]);
+              if (col < n_out) {
+                float v = acc[q][cb][r] + (accumulate ? o[col] : bv[cb]);
+                if (post) v = epi_act(v, es[cb], eh[cb], epi.leak);
+                o[col] = v;
+              }
             }
           }
         }
@@ -933,7 +964,7 @@ __global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, in
 
 template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4>
 static void launch_resident_kernel(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
-                                   const float *bias, int n_in_part, int n_out, int accumulate, size_t lds_bytes,
+                                   Epi epi, int n_in_part, int n_out, int accumulate, size_t lds_bytes,
                                    int per_cu, hipStream_t s) {
   auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, C4>;
   static bool attr_set = false;
@@ -946,7 +977,7 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
   const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
   kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
-                                                   out, m.wpack.p, bias, n_in_part, n_out, n_sets, sets_per_xcd,
+                                                   out, m.wpack.p, epi, n_in_part, n_out, n_sets, sets_per_xcd,
                                                    accumulate, m.queue.p);
   LAUNCH_CHECK();
 }
@@ -954,7 +985,7 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
 // One launch over channels [c_lo, c_lo + n_in_part) of the input rows.
 template <int NCB, int SS, bool VEC4>
 static void launch_resident_part(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
-                                 const float *w, int w_in_stride_rows, const float *bias, int n_in_part,
+                                 const float *w, int w_in_stride_rows, Epi epi, int n_in_part,
                                  int n_out, int accumulate, hipStream_t s) {
   constexpr int RG = 2;  // 32 rows per set: measured faster than 64 (more wavefronts in flight)
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
@@ -966,11 +997,11 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
   LAUNCH_CHECK();
   const size_t lds_bytes = (size_t)packed * sizeof(float);
   if (lds_bytes > 80 * 1024) {
-    launch_resident_kernel<NCB, RG, SS, VEC4, 16, false>(m, t, in, in_stride, out, bias, n_in_part, n_out, accumulate,
+    launch_resident_kernel<NCB, RG, SS, VEC4, 16, false>(m, t, in, in_stride, out, epi, n_in_part, n_out, accumulate,
                                                          lds_bytes, 1, s);
   } else {
     const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / std::max<size_t>(lds_bytes, 1)));
-    launch_resident_kernel<NCB, RG, SS, VEC4, 8, false>(m, t, in, in_stride, out, bias, n_in_part, n_out, accumulate,
+    launch_resident_kernel<NCB, RG, SS, VEC4, 8, false>(m, t, in, in_stride, out, epi, n_in_part, n_out, accumulate,
                                                         lds_bytes, per_cu, s);
   }
 }
@@ -978,14 +1009,14 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
 // nIn <= 4 (the first layer of most networks): four-channel layout, 64 rows per set.
 template <int NCB>
 static void launch_resident_c4(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                               const float *bias, int n_in, int n_out, hipStream_t s) {
+                               Epi epi, int n_in, int n_out, hipStream_t s) {
   const int packed = t.K * NCB * 64;
   m.wpack.reserve(packed);
   m.queue.reserve(8 * 32);
   k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, NCB,
                                                                         m.queue.p);
   LAUNCH_CHECK();
-  launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, bias, n_in, n_out, 0,
+  launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, epi, n_in, n_out, 0,
                                                     (size_t)packed * sizeof(float), 3, s);
 }
 
@@ -1002,13 +1033,13 @@ static bool resident_fits(const Table &t, int n_in, int n_out, bool with_bn) {
 // small MFMA blocks, and normalising every gathered value (each row is gathered once per tap
 // that reaches it) costs more than one extra pass over the rows.
 static bool try_resident(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                         const float *bias, int n_in, int n_out, hipStream_t s) {
+                         Epi epi, int n_in, int n_out, hipStream_t s) {
   if (!resident_fits(t, n_in, n_out, false)) return false;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   const int ncb = (int)ceil_div(n_out, 16);
   if (n_in <= 4) {
-    if (ncb == 1) launch_resident_c4<1>(m, t, in, out, w, bias, n_in, n_out, s);
-    else launch_resident_c4<2>(m, t, in, out, w, bias, n_in, n_out, s);
+    if (ncb == 1) launch_resident_c4<1>(m, t, in, out, w, epi, n_in, n_out, s);
+    else launch_resident_c4<2>(m, t, in, out, w, epi, n_in, n_out, s);
     return true;
   }
   for (int c_lo = 0; c_lo < n_in; c_lo += 32) {
@@ -1016,7 +1047,13 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
     const float *in_p = in + c_lo;
     const float *w_p = w + (int64_t)c_lo * n_out;
     const int acc = c_lo > 0;
-    const float *b = acc ? nullptr : bias;
+    Epi b;  // bias with the first part, the following layer's batch norm with the last
+    if (!acc) b.bias = epi.bias;
+    if (c_lo + 32 >= n_in) {
+      b.sc = epi.sc;
+      b.sh = epi.sh;
+      b.leak = epi.leak;
+    }
 #define SCN_RES(NCBV, SSV)                                                                                   \
   do {                                                                                                       \
     if (vec4)                                                                                                \
@@ -1039,38 +1076,38 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
 // granule no longer leave room for this layout's operands and k_conv_mfma is as fast.
 template <bool VEC4, bool PRE>
 static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                          const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+                          Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   const int ncb = (int)ceil_div(n_out, 16);
   const bool narrow = n_in <= 16;
   if (ncb <= 2)
-    return narrow ? launch_rows<2, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
-                  : launch_rows<2, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
+    return narrow ? launch_rows<2, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
+                  : launch_rows<2, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
   if (ncb <= 4)
-    return narrow ? launch_rows<4, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
-                  : launch_rows<4, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
+    return narrow ? launch_rows<4, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
+                  : launch_rows<4, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
   if (ncb <= 6)
-    return narrow ? launch_rows<6, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
-                  : launch_rows<6, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
+    return narrow ? launch_rows<6, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
+                  : launch_rows<6, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
   if (ncb <= 8)
-    return narrow ? launch_rows<8, 1, 1, VEC4, 8, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
-                  : launch_rows<8, 1, 2, VEC4, 8, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s);
+    return narrow ? launch_rows<8, 1, 1, VEC4, 8, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
+                  : launch_rows<8, 1, 2, VEC4, 8, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
   return false;
 }
 
 template <bool PRE>
 static bool conv_mfma_paths(Metadata &m, const Table &t, const float *in, float *out, const float *w,
-                            const float *bias, int n_in, int n_out, PreArgs pre, hipStream_t s) {
-  if (!PRE && try_resident(m, t, in, out, w, bias, n_in, n_out, s)) return true;
+                            Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+  if (!PRE && try_resident(m, t, in, out, w, epi, n_in, n_out, s)) return true;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   if (n_out <= 128 && t.K <= 1024) {
-    if (vec4 ? dispatch_rows<true, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s)
-             : dispatch_rows<false, PRE>(m, t, in, out, w, bias, n_in, n_out, pre, s))
+    if (vec4 ? dispatch_rows<true, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
+             : dispatch_rows<false, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s))
       return true;
   }
   if (t.K <= 1024) {
     const int ncb = (int)ceil_div(n_out, 16);
-    if (vec4 ? dispatch_ncb<true, PRE>(ncb, m, t, in, out, w, bias, n_in, n_out, pre, s)
-             : dispatch_ncb<false, PRE>(ncb, m, t, in, out, w, bias, n_in, n_out, pre, s))
+    if (vec4 ? dispatch_ncb<true, PRE>(ncb, m, t, in, out, w, epi, n_in, n_out, pre, s)
+             : dispatch_ncb<false, PRE>(ncb, m, t, in, out, w, epi, n_in, n_out, pre, s))
       return true;
   }
   return false;
@@ -1078,12 +1115,26 @@ static bool conv_mfma_paths(Metadata &m, const Table &t, const float *in, float 
 
 // bn: optional eval batch norm + leaky ReLU applied to the input rows before the convolution
 // (what a BatchNormalization module in front of the convolution computes), fused into the
-// gather; nullptr for a plain convolution.
+// gather; post: the same for a BatchNormalization module behind the convolution, applied to
+// the output values as they are stored.  nullptr for a plain convolution.
 void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
-                  const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, hipStream_t s) {
+                  const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, const BnArgs *post,
+                  hipStream_t s) {
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
+  Epi epi;
+  epi.bias = bias;
+  if (post) {
+    m.postbuf.reserve(2 * (size_t)n_out);
+    k_pre_coeffs<<<dim3((unsigned)ceil_div(n_out, 256)), 256, 0, s>>>(post->mean, post->var, post->gamma, post->beta,
+                                                                     post->eps, n_out, n_out, m.postbuf.p,
+                                                                     m.postbuf.p + n_out);
+    LAUNCH_CHECK();
+    epi.sc = m.postbuf.p;
+    epi.sh = m.postbuf.p + n_out;
+    epi.leak = post->leak;
+  }
   if (bn && groups == 1 && !resident_fits(t, n_in, n_out, true)) {
     const int n_pad = (int)round_up(n_in, 64) + 64;
     m.prebuf.reserve(2 * (size_t)n_pad);
@@ -1094,7 +1145,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     pre.sc = m.prebuf.p;
     pre.sh = m.prebuf.p + n_pad;
     pre.leak = bn->leak;
-    if (conv_mfma_paths<true>(m, t, in, out, w, bias, n_in, n_out, pre, s)) return;
+    if (conv_mfma_paths<true>(m, t, in, out, w, epi, n_in, n_out, pre, s)) return;
   }
   const float *src = in;
   if (bn) {  // no fused kernel for this shape: normalise the rows in a pass of their own
@@ -1103,10 +1154,10 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
                     bn->leak, s);
     src = m.bntmp.p;
   }
-  if (groups == 1 && conv_mfma_paths<false>(m, t, src, out, w, bias, n_in, n_out, PreArgs(), s)) return;
+  if (groups == 1 && conv_mfma_paths<false>(m, t, src, out, w, epi, n_in, n_out, PreArgs(), s)) return;
   int64_t total = t.n * n_out;
   k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, src,
-                                                                       out, w, bias, n_in, n_out, groups);
+                                                                       out, w, epi, n_in, n_out, groups);
   LAUNCH_CHECK();
 }
 

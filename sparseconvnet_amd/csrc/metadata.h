@@ -88,6 +88,7 @@ struct Metadata {
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
   DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
+  DevBuf<float> postbuf;  // scale / shift of a batch norm fused into the running convolution's stores
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
   DevBuf<float> bntmp;    // normalised input when a fused batch norm has no fused kernel
 };
@@ -115,7 +116,8 @@ struct BnArgs {  // eval batch norm + leaky ReLU in front of a convolution (devi
   float eps, leak;
 };
 void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
-                  const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, hipStream_t s);
+                  const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, const BnArgs *post,
+                  hipStream_t s);
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
                      int drop, hipStream_t s);
 void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,

@@ -67,16 +67,38 @@ def _bn_args(bn):
             optionalTensor(bn, 'bias').detach(), bn.eps, bn.leakiness)
 
 
-def fusable_pair(bn, conv, input):
-    """True when Sequential may hand the batch normalisation `bn` to the convolution `conv`
-    that follows it instead of running it as a pass of its own: the result is the same, the
-    normalised rows are just never written to memory."""
-    return (_pkg.fuse_batchnorm and type(bn) in (BatchNormalization, BatchNormReLU, BatchNormLeakyReLU)
-            and type(conv) in (SubmanifoldConvolution, ValidConvolution, Convolution, Deconvolution)
-            and not bn.training and conv.groups == 1 and bn.nPlanes == conv.nIn
-            and not bn._forward_hooks and not bn._forward_pre_hooks
-            and not conv._forward_hooks and not conv._forward_pre_hooks
-            and input.features.nelement() > 0 and input.features.size(1) == bn.nPlanes)
+def _plain(module, classes):
+    return type(module) in classes and not module._forward_hooks and not module._forward_pre_hooks
+
+
+def _is_bn(module):
+    return (_plain(module, (BatchNormalization, BatchNormReLU, BatchNormLeakyReLU)) and not module.training)
+
+
+def _is_conv(module):
+    return (_plain(module, (SubmanifoldConvolution, ValidConvolution, Convolution, Deconvolution))
+            and module.groups == 1)
+
+
+def fuse_plan(mods, input):
+    """How Sequential runs the first module(s) of `mods` on `input`: (convolution, batch norm in
+    front or None, batch norm behind or None, number of modules consumed), or None when the
+    first module runs by itself.  An eval-mode batch normalisation next to a convolution gives
+    the same result applied inside the convolution, without a pass over the rows of its own."""
+    if not _pkg.fuse_batchnorm or input.features.nelement() == 0:
+        return None
+    pre, i = None, 0
+    if len(mods) > 1 and _is_bn(mods[0]) and _is_conv(mods[1]) and mods[0].nPlanes == mods[1].nIn:
+        pre, i = mods[0], 1
+    if not _is_conv(mods[i]) or input.features.size(1) != mods[i].nIn:
+        return None
+    conv = mods[i]
+    post = None
+    if len(mods) > i + 1 and _is_bn(mods[i + 1]) and mods[i + 1].nPlanes == conv.nOut:
+        post = mods[i + 1]
+    if pre is None and post is None:
+        return None
+    return conv, pre, post, i + 1 + (post is not None)
 
 
 class SubmanifoldConvolution(Module):
@@ -94,15 +116,15 @@ class SubmanifoldConvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None):
+    def forward(self, input, pre_bn=None, post_bn=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, self.nOut, input)
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
-        md, sz, fs, bn = input.metadata, input.spatial_size, self.filter_size, _bn_args(pre_bn)
+        md, sz, fs, bn, post = input.metadata, input.spatial_size, self.filter_size, _bn_args(pre_bn), _bn_args(post_bn)
 
         def fn(x, w, b):
-            y, macs = md.submanifoldConvolution(sz, fs, x, w, b, bn)
+            y, macs = md.submanifoldConvolution(sz, fs, x, w, b, bn, post)
             _count(macs, y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
@@ -135,7 +157,7 @@ class Convolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None):
+    def forward(self, input, pre_bn=None, post_bn=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
@@ -144,10 +166,10 @@ class Convolution(Module):
         assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
             input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
-        bn = _bn_args(pre_bn)
+        bn, post = _bn_args(pre_bn), _bn_args(post_bn)
 
         def fn(x, w, b):
-            y, macs = md.convolution(*a, x, w, b, bn)
+            y, macs = md.convolution(*a, x, w, b, bn, post)
             _count(macs, y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
@@ -177,16 +199,16 @@ class Deconvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None):
+    def forward(self, input, pre_bn=None, post_bn=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
         md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
-        bn = _bn_args(pre_bn)
+        bn, post = _bn_args(pre_bn), _bn_args(post_bn)
 
         def fn(x, w, b):
-            y, macs = md.deconvolution(*a, x, w, b, bn)
+            y, macs = md.deconvolution(*a, x, w, b, bn, post)
             _count(macs, y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))

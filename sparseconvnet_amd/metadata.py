@@ -86,44 +86,53 @@ class Metadata:
         _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out
 
-    def _conv(self, name, size_args, n_rows, features, weight, bias, bn):
-        """bn: None, or (running_mean, running_var, weight, bias, eps, leakiness) of an eval-mode
-        batch normalisation applied to `features` inside the convolution's gather."""
+    def _conv(self, kind, size_args, n_rows, features, weight, bias, bn, post):
+        """kind 0 / 1 / 2: submanifold / strided / transposed convolution.  bn, post: None, or
+        (running_mean, running_var, weight, bias, eps, leakiness) of an eval-mode batch
+        normalisation in front of / behind the convolution, applied inside it."""
         features = _features(features, "features")
         weight = _features(weight, "weight")
         K, groups, ip, op = weight.shape
         bias_t = _features(bias, "bias") if bias is not None and bias.numel() else None
         out = torch.empty((n_rows, groups * op), dtype=torch.float32, device=features.device)
         macs = C.c_double(0)
-        head = (self._h, *size_args, _ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t), groups * ip,
-                groups * op, groups)
-        if bn is None:
-            _lib.check(getattr(self._L, "scn_" + name)(*head, _stream(), C.byref(macs)))
+        tail = (_ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t), groups * ip, groups * op, groups)
+        if bn is None and post is None:
+            fn = (self._L.scn_subm_conv_fwd, self._L.scn_conv_fwd, self._L.scn_deconv_fwd)[kind]
+            _lib.check(fn(self._h, *size_args, *tail, _stream(), C.byref(macs)))
         else:
-            mean, var, g, b, eps, leak = bn
-            assert mean.numel() == groups * ip and var.numel() == groups * ip
-            g = _features(g, "bn weight") if g is not None and g.numel() else None
-            b = _features(b, "bn bias") if b is not None and b.numel() else None
-            _lib.check(getattr(self._L, "scn_bn_" + name)(
-                *head, _ptr(_features(mean, "running_mean")), _ptr(_features(var, "running_var")), _ptr(g),
-                _ptr(b), float(eps), float(leak), _stream(), C.byref(macs)))
+            keep = []  # tensors behind the raw pointers stay alive until the call has been issued
+
+            def params(p, planes):
+                if p is None:
+                    return None
+                mean, var, g, b, eps, leak = p
+                assert mean.numel() == planes and var.numel() == planes, (mean.shape, planes)
+                t = [_features(mean, "running_mean"), _features(var, "running_var"),
+                     _features(g, "bn weight") if g is not None and g.numel() else None,
+                     _features(b, "bn bias") if b is not None and b.numel() else None]
+                keep.extend(t)
+                return C.byref(_lib.BnParams(*[_ptr(x) for x in t], float(eps), float(leak)))
+            sizes = list(size_args) + [None] * (4 - len(size_args))
+            _lib.check(self._L.scn_conv_bn_fwd(self._h, kind, *sizes, *tail, params(bn, groups * ip),
+                                               params(post, groups * op), _stream(), C.byref(macs)))
         return out, macs.value
 
-    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias, bn=None):
+    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias, bn=None, post=None):
         sp, fs = self._s(spatial_size), self._s(filter_size)
         _lib.check(self._L.scn_md_submanifold_rules(self._h, sp, fs, _stream()))
-        return self._conv("subm_conv_fwd", (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn)
+        return self._conv(0, (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn, post)
 
-    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None):
+    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
-        return self._conv("conv_fwd", a, self.getNActive(out_size), features, weight, bias, bn)
+        return self._conv(1, a, self.getNActive(out_size), features, weight, bias, bn, post)
 
-    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None):
+    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *rb, _stream()))
-        return self._conv("deconv_fwd", a, self.getNActive(out_size), features, weight, bias, bn)
+        return self._conv(2, a, self.getNActive(out_size), features, weight, bias, bn, post)
 
     def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
         a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]

@@ -96,40 +96,49 @@ class HipPath:
         return self._rules(2, spatial)
 
     # -- forward ops ------------------------------------------------------
-    def _conv(self, name, sizes, n_rows, x, w, bias, bn=None):
-        """bn: None or dict(mean, var, weight, bias, eps, leakiness): the fused entry point."""
+    def _conv(self, kind, sizes, n_rows, x, w, bias, bn=None, post=None):
+        """bn / post: None or dict(mean, var, weight, bias, eps, leakiness) of a batch norm in
+        front of / behind the convolution: the fused entry point scn_conv_bn_fwd."""
         groups = w.shape[1]
         n_in, n_out = w.shape[2] * groups, w.shape[3] * groups
         xd, wd = _dev(x, torch.float32), _dev(w, torch.float32)
         bd = _dev(bias, torch.float32) if bias is not None else None
         out = torch.full((n_rows, n_out), float("nan"), dtype=torch.float32, device="cuda")
         macs = C.c_double(0)
-        head = (self.h, *sizes, _ptr(xd), _ptr(out), _ptr(wd), _ptr(bd), n_in, n_out, groups)
-        if bn is None:
-            _lib.check(getattr(self.L, "scn_" + name)(*head, _stream(), C.byref(macs)))
+        tail = (_ptr(xd), _ptr(out), _ptr(wd), _ptr(bd), n_in, n_out, groups)
+        if bn is None and post is None:
+            fn = (self.L.scn_subm_conv_fwd, self.L.scn_conv_fwd, self.L.scn_deconv_fwd)[kind]
+            _lib.check(fn(self.h, *sizes, *tail, _stream(), C.byref(macs)))
         else:
-            t = [_dev(bn[k], torch.float32) if bn.get(k) is not None else None
-                 for k in ("mean", "var", "weight", "bias")]
-            _lib.check(getattr(self.L, "scn_bn_" + name)(*head, *[_ptr(v) for v in t], bn["eps"],
-                                                         bn["leakiness"], _stream(), C.byref(macs)))
+            keep = []
+
+            def params(p):
+                if p is None:
+                    return None
+                t = [_dev(p[k], torch.float32) if p.get(k) is not None else None
+                     for k in ("mean", "var", "weight", "bias")]
+                keep.extend(t)
+                return C.byref(_lib.BnParams(*[_ptr(v) for v in t], p["eps"], p["leakiness"]))
+            sz = list(sizes) + [None] * (4 - len(sizes))
+            _lib.check(self.L.scn_conv_bn_fwd(self.h, kind, *sz, *tail, params(bn), params(post), _stream(),
+                                              C.byref(macs)))
         return out.cpu().numpy(), macs.value
 
-    def subm_conv(self, spatial, filter_size, x, w, bias=None, bn=None):
+    def subm_conv(self, spatial, filter_size, x, w, bias=None, bn=None, post=None):
         _lib.check(self.L.scn_md_submanifold_rules(self.h, self._s(spatial), self._s(filter_size),
                                                    _stream()))
-        return self._conv("subm_conv_fwd", (self._s(spatial), self._s(filter_size)),
-                          self.nactive(spatial), x, w, bias, bn)
+        return self._conv(0, (self._s(spatial), self._s(filter_size)), self.nactive(spatial), x, w, bias, bn, post)
 
-    def conv(self, in_size, out_size, filter_size, stride, x, w, bias=None, bn=None):
+    def conv(self, in_size, out_size, filter_size, stride, x, w, bias=None, bn=None, post=None):
         sizes = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         _lib.check(self.L.scn_md_strided_rules(self.h, *sizes, _stream()))
-        return self._conv("conv_fwd", sizes, self.nactive(out_size), x, w, bias, bn)
+        return self._conv(1, sizes, self.nactive(out_size), x, w, bias, bn, post)
 
-    def deconv(self, in_size, out_size, filter_size, stride, x, w, bias=None, bn=None):
+    def deconv(self, in_size, out_size, filter_size, stride, x, w, bias=None, bn=None, post=None):
         sizes = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
         _lib.check(self.L.scn_md_strided_rules(self.h, *rb, _stream()))
-        return self._conv("deconv_fwd", sizes, self.nactive(out_size), x, w, bias, bn)
+        return self._conv(2, sizes, self.nactive(out_size), x, w, bias, bn, post)
 
     def maxpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
         sizes = [self._s(v) for v in (in_size, out_size, size, stride)]

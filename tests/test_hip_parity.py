@@ -123,41 +123,57 @@ def test_strided_tree_vs_oracle(oracle_built):
 
 
 @pytest.mark.parametrize("cin,cout,groups", [(3, 32, 1), (32, 32, 1), (40, 16, 1), (48, 64, 1), (64, 96, 1),
-                                             (96, 128, 1), (128, 160, 1), (30, 50, 1), (8, 12, 2)])
+                                             (96, 128, 1), (128, 160, 1), (30, 50, 1), (64, 32, 1), (8, 12, 2)])
 def test_fused_bn_conv_vs_oracle(oracle_built, cin, cout, groups):
-    """The fused entry points (eval batch norm + leaky ReLU inside the convolution's gather)
-    against the oracle's two separate passes, over every convolution kernel's channel range,
-    for the submanifold, strided and transposed convolutions."""
+    """The fused entry point (eval batch norm + leaky ReLU in front of the convolution applied
+    in its gather, the one behind it applied to its stores) against the oracle's separate
+    passes, over every convolution kernel's channel range, for the submanifold, strided and
+    transposed convolutions."""
     g, o = _both(3, oracle_built)
     coords = synthetic.room_scene(seed=4100, target=20000, spatial=126, duplicate_fraction=0.0)
     rng = np.random.default_rng(cin * 1000 + cout)
     x = rng.normal(size=(len(coords), cin)).astype(np.float32)
-    bn = dict(mean=rng.normal(size=cin).astype(np.float32), var=rng.uniform(0.5, 1.5, cin).astype(np.float32),
-              weight=rng.uniform(0.5, 1.5, cin).astype(np.float32), bias=rng.normal(size=cin).astype(np.float32),
-              eps=1e-4, leakiness=0.0)
+
+    def bn_of(planes, leak, affine=True):
+        return dict(mean=rng.normal(size=planes).astype(np.float32),
+                    var=rng.uniform(0.5, 1.5, planes).astype(np.float32),
+                    weight=rng.uniform(0.5, 1.5, planes).astype(np.float32) if affine else None,
+                    bias=rng.normal(size=planes).astype(np.float32) if affine else None, eps=1e-4, leakiness=leak)
+
+    def apply(p, bn, v):
+        return p.bn_eval(v, bn["mean"], bn["var"], bn["weight"], bn["bias"], bn["eps"], bn["leakiness"])
 
     def w(k, a, b):
         return (rng.normal(size=(k, groups, a // groups, b // groups)) * (2.0 / (a * k)) ** 0.5).astype(np.float32)
+    pre, post, post_leaky = bn_of(cin, 0.0), bn_of(cout, 0.0), bn_of(cout, 0.333, affine=False)
     w_s, w_d, w_u = w(27, cin, cout), w(8, cin, cout), w(8, cin, cout)
     bias = rng.normal(size=cout).astype(np.float32)
     for p in (g, o):
         assert p.input_layer(126, coords, 0, 3) == len(coords)
         p.strided_rules(126, 63, 2, 2)
     lg, lo = g.spatial_locations(63), o.spatial_locations(63)
-    xn = o.bn_eval(x, bn["mean"], bn["var"], bn["weight"], bn["bias"], bn["eps"], bn["leakiness"])
-    got, _ = g.subm_conv(126, 3, x, w_s, bias, bn=bn)
-    want, _ = o.subm_conv(126, 3, xn, w_s, bias)
-    checks.assert_close(got, want, "bn + submanifold convolution")
-    got, m1 = g.conv(126, 63, 2, 2, x, w_d, None, bn=bn)
+    xn = apply(o, pre, x)
+    # batch norm in front and behind
+    got, _ = g.subm_conv(126, 3, x, w_s, bias, bn=pre, post=post)
+    want = apply(o, post, o.subm_conv(126, 3, xn, w_s, bias)[0])
+    checks.assert_close(got, want, "bn + submanifold convolution + bn")
+    # only behind
+    got, _ = g.subm_conv(126, 3, x, w_s, None, post=post_leaky)
+    want = apply(o, post_leaky, o.subm_conv(126, 3, x, w_s, None)[0])
+    checks.assert_close(got, want, "submanifold convolution + bn")
+    # only in front
+    got, m1 = g.conv(126, 63, 2, 2, x, w_d, None, bn=pre)
     want, m2 = o.conv(126, 63, 2, 2, xn, w_d, None)
     assert m1 == m2
     checks.assert_close(got[canon_rows(lg)], want[canon_rows(lo)], "bn + strided convolution")
+    got, _ = g.conv(126, 63, 2, 2, x, w_d, bias, post=post)
+    want = apply(o, post, o.conv(126, 63, 2, 2, x, w_d, bias)[0])
+    checks.assert_close(got[canon_rows(lg)], want[canon_rows(lo)], "strided convolution + bn")
     # transposed convolution: rows of the 63^3 level in, rows of the 126^3 level out
     xc = rng.normal(size=(len(lo), cin)).astype(np.float32)
     xg = np.empty_like(xc)
     xg[canon_rows(lg)] = xc[canon_rows(lo)]  # the same site gets the same row of values
-    leaky = dict(bn, leakiness=0.333, weight=None, bias=None)
-    xcn = o.bn_eval(xc, bn["mean"], bn["var"], None, None, bn["eps"], 0.333)
-    got, _ = g.deconv(63, 126, 2, 2, xg, w_u, bias, bn=leaky)
-    want, _ = o.deconv(63, 126, 2, 2, xcn, w_u, bias)
-    checks.assert_close(got, want, "bn + transposed convolution")
+    leaky = bn_of(cin, 0.333, affine=False)
+    got, _ = g.deconv(63, 126, 2, 2, xg, w_u, bias, bn=leaky, post=post)
+    want = apply(o, post, o.deconv(63, 126, 2, 2, apply(o, leaky, xc), w_u, bias)[0])
+    checks.assert_close(got, want, "bn + transposed convolution + bn")
