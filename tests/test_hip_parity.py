@@ -177,3 +177,83 @@ def test_fused_bn_conv_vs_oracle(oracle_built, cin, cout, groups):
     got, _ = g.deconv(63, 126, 2, 2, xg, w_u, bias, bn=leaky, post=post)
     want = apply(o, post, o.deconv(63, 126, 2, 2, apply(o, leaky, xc), w_u, bias)[0])
     checks.assert_close(got, want, "bn + transposed convolution + bn")
+
+
+def _neighbour_counts(coords, spatial):
+    """Per site and tap: is the neighbour active?  Independent of oracle and library: sorted
+    linear indices and a binary search (numpy)."""
+    c = coords[:, :3].astype(np.int64)
+    lin = ((coords[:, 3].astype(np.int64) * spatial + c[:, 0]) * spatial + c[:, 1]) * spatial + c[:, 2]
+    order = np.argsort(lin)
+    s = lin[order]
+    present = np.zeros((27, len(c)), bool)
+    k = 0
+    for dx in (-1, 0, 1):
+        for dy in (-1, 0, 1):
+            for dz in (-1, 0, 1):
+                q = lin + (dx * spatial + dy) * spatial + dz
+                ok = ((c[:, 0] + dx >= 0) & (c[:, 0] + dx < spatial) & (c[:, 1] + dy >= 0) & (c[:, 1] + dy < spatial)
+                      & (c[:, 2] + dz >= 0) & (c[:, 2] + dz < spatial))
+                i = np.minimum(np.searchsorted(s, q), len(s) - 1)
+                present[k] = ok & (s[i] == q)
+                k += 1
+    return present
+
+
+def test_full_size_sweep_scene_properties():
+    """Configuration 3 at its full size (one room scene of 1,000,000 sites in 4096^3, the
+    bench workload), through properties that do not need the oracle to finish: the rule count
+    per tap equals an independent numpy count; a convolution whose weights are all ones on a
+    feature of ones returns each site's neighbour count; the centre-tap identity returns the
+    input; the map is linear; fused and separate batch norm agree."""
+    from hip_path import HipPath
+    g = HipPath(3)
+    coords = synthetic.room_scene(seed=3000, target=1000000, spatial=4096)
+    assert g.input_layer(4096, coords, 0, 0) == len(coords)
+    present = _neighbour_counts(coords, 4096)
+    rules = g.submanifold_rules(4096, 3)
+    assert [len(r) for r in rules] == present.sum(1).tolist()
+    # taps are mirror images of each other: rule (i -> j) of tap k is rule (j -> i) of tap 26 - k
+    for k in (0, 5, 13):
+        a, b = rules[k], rules[26 - k]
+        ka = np.sort(a[:, 0].astype(np.int64) * len(coords) + a[:, 1])
+        kb = np.sort(b[:, 1].astype(np.int64) * len(coords) + b[:, 0])
+        assert (ka == kb).all()
+    n = len(coords)
+    ones = np.ones((n, 1), np.float32)
+    y, macs = g.subm_conv(4096, 3, ones, np.ones((27, 1, 1, 1), np.float32))
+    assert macs == present.sum()
+    assert (y[:, 0] == present.sum(0)).all()  # small integers: exact in fp32
+    rng = np.random.default_rng(3)
+    for cin, cout in ((32, 32), (64, 64), (128, 128)):
+        x = rng.normal(size=(n, cin)).astype(np.float32)
+        w = np.zeros((27, 1, cin, cout), np.float32)
+        w[13, 0] = np.eye(cin, cout)
+        y, _ = g.subm_conv(4096, 3, x, w)
+        assert (y == x[:, :cout]).all()  # centre tap, identity weights: a copy
+    x1, x2 = rng.normal(size=(n, 64)).astype(np.float32), rng.normal(size=(n, 64)).astype(np.float32)
+    w = (rng.normal(size=(27, 1, 64, 64)) * (2.0 / (64 * 27)) ** 0.5).astype(np.float32)
+    y1, y2, y12 = (g.subm_conv(4096, 3, v, w)[0] for v in (x1, x2, x1 + 2 * x2))
+    checks.assert_close(y12, y1 + 2 * y2, "linearity at 1 M sites")
+    # one output row recomputed by hand from the numpy neighbour table
+    lin = ((coords[:, 0].astype(np.int64)) * 4096 + coords[:, 1]) * 4096 + coords[:, 2]
+    order = np.argsort(lin)
+    for row in (0, n // 2, n - 1):
+        acc = np.zeros(64, np.float64)
+        k = 0
+        for dx in (-1, 0, 1):
+            for dy in (-1, 0, 1):
+                for dz in (-1, 0, 1):
+                    if present[k, row]:
+                        q = lin[row] + (dx * 4096 + dy) * 4096 + dz
+                        j = order[np.searchsorted(lin[order], q)]
+                        acc += x1[j].astype(np.float64) @ w[k, 0].astype(np.float64)
+                    k += 1
+        checks.assert_close(y1[row], acc, "row %d by hand" % row)
+    bn = dict(mean=rng.normal(size=64).astype(np.float32), var=rng.uniform(0.5, 1.5, 64).astype(np.float32),
+              weight=rng.uniform(0.5, 1.5, 64).astype(np.float32), bias=rng.normal(size=64).astype(np.float32),
+              eps=1e-4, leakiness=0.0)
+    fused, _ = g.subm_conv(4096, 3, x1, w, None, bn=bn, post=bn)
+    sep = g.bn_eval(g.subm_conv(4096, 3, g.bn_eval(x1, bn["mean"], bn["var"], bn["weight"], bn["bias"], 1e-4, 0.0),
+                                w)[0], bn["mean"], bn["var"], bn["weight"], bn["bias"], 1e-4, 0.0)
+    checks.assert_close(fused, sep, "fused vs separate batch norm at 1 M sites")
