@@ -42,17 +42,32 @@ __device__ inline float epi_act(float v, float sc, float sh, float leak) {
   const float y = v * sc + sh;
   return y > 0.f ? y : y * leak;
 }
-__global__ void k_pre_coeffs(const float *mean, const float *var, const float *gamma, const float *beta, float eps,
-                             int n_in, int n_pad, float *sc, float *sh) {
-  int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= n_pad) return;
-  float w = 0.f, b = 0.f;
-  if (c < n_in) {
-    w = (1.0f / sqrtf(var[c] + eps)) * (gamma ? gamma[c] : 1.0f);
-    b = -mean[c] * w + (beta ? beta[c] : 0.0f);
+// Folding a batch norm to scale / shift (sc[c] = gamma / sqrt(var + eps), sh[c] = beta -
+// mean * sc, zeros from n to n_pad) is a few hundred values: the weight-packing launch that
+// precedes every MFMA convolution does it on the side (its first workgroup), so it costs no
+// launch of its own.  CoefJobs lives in metadata.h.
+__device__ inline void coef_job(const CoefJob &j) {
+  for (int c = threadIdx.x; c < j.n_pad; c += blockDim.x) {
+    float w = 0.f, b = 0.f;
+    if (c < j.n) {
+      w = (1.0f / sqrtf(j.var[c] + j.eps)) * (j.gamma ? j.gamma[c] : 1.0f);
+      b = -j.mean[c] * w + (j.beta ? j.beta[c] : 0.0f);
+    }
+    j.sc[c] = w;
+    j.sh[c] = b;
   }
-  sc[c] = w;
-  sh[c] = b;
+}
+__device__ inline void coef_jobs(const CoefJobs &jobs) {
+  if (blockIdx.x != 0) return;
+  if (jobs.pre.n_pad) coef_job(jobs.pre);
+  if (jobs.post.n_pad) coef_job(jobs.post);
+}
+__global__ void k_coefs(CoefJobs jobs) { coef_jobs(jobs); }
+// Hands the pending jobs to the launch being prepared (and forgets them).
+static CoefJobs take_jobs(Metadata &m) {
+  CoefJobs j = m.jobs;
+  m.jobs = CoefJobs();
+  return j;
 }
 
 // ---- generic kernel: any channel counts, any groups -------------------------------------
@@ -89,7 +104,8 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
 // straight copy and each lane reads the four operands of one 16-channel step with a single
 // 16-byte LDS load.
 __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n_out, int n_slab, int SS,
-                               int NCB, int slab_stride) {
+                               int NCB, int slab_stride, CoefJobs jobs) {
+  coef_jobs(jobs);
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = (int64_t)K * n_slab * slab_stride;
   if (i >= total) return;
@@ -116,7 +132,8 @@ __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n
 // in the layout of k_pack_weights.
 // Also clears the eight set counters (one per XCD, 128 bytes apart) of the launch it precedes.
 __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows, int n_in_part, int n_out,
-                                    int SS, int NCB, int *queue) {
+                                    int SS, int NCB, int *queue, CoefJobs jobs) {
+  coef_jobs(jobs);
   if (blockIdx.x == 0 && threadIdx.x < 8) queue[threadIdx.x * 32] = 0;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = (int64_t)K * SS * NCB * 256;
@@ -398,7 +415,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
   m.wpack.reserve(packed);
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB, SLAB_STRIDE);
+                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m));
   LAUNCH_CHECK();
   auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE>;
   static bool attr_set = false;
@@ -671,7 +688,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
   m.wpack.reserve(packed);
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB, SLAB_STRIDE);
+                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m));
   LAUNCH_CHECK();
   auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE>;
   static bool attr_set = false;
@@ -953,7 +970,9 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 
 // B operands of the four-channel layout: wp[(k * NCB + cb) * 64 + lane] = w[k][lane / 16][16 cb + lane % 16].
 // Also clears the set counters, as k_pack_weights_part does.
-__global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, int n_out, int NCB, int *queue) {
+__global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, int n_out, int NCB, int *queue,
+                                  CoefJobs jobs) {
+  coef_jobs(jobs);
   if (blockIdx.x == 0 && threadIdx.x < 8) queue[threadIdx.x * 32] = 0;
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= K * NCB * 64) return;
@@ -993,7 +1012,8 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
   m.queue.reserve(8 * 32);
   // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
   k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, w_in_stride_rows,
-                                                                           n_in_part, n_out, SS, NCB, m.queue.p);
+                                                                           n_in_part, n_out, SS, NCB, m.queue.p,
+                                                                           take_jobs(m));
   LAUNCH_CHECK();
   const size_t lds_bytes = (size_t)packed * sizeof(float);
   if (lds_bytes > 80 * 1024) {
@@ -1014,7 +1034,7 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
   m.wpack.reserve(packed);
   m.queue.reserve(8 * 32);
   k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, NCB,
-                                                                        m.queue.p);
+                                                                        m.queue.p, take_jobs(m));
   LAUNCH_CHECK();
   launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, epi, n_in, n_out, 0,
                                                     (size_t)packed * sizeof(float), 3, s);
@@ -1125,12 +1145,11 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   if (t.n == 0) return;
   Epi epi;
   epi.bias = bias;
+  m.jobs = CoefJobs();
   if (post) {
     m.postbuf.reserve(2 * (size_t)n_out);
-    k_pre_coeffs<<<dim3((unsigned)ceil_div(n_out, 256)), 256, 0, s>>>(post->mean, post->var, post->gamma, post->beta,
-                                                                     post->eps, n_out, n_out, m.postbuf.p,
-                                                                     m.postbuf.p + n_out);
-    LAUNCH_CHECK();
+    m.jobs.post = CoefJob{post->mean, post->var, post->gamma, post->beta, post->eps, n_out, n_out, m.postbuf.p,
+                          m.postbuf.p + n_out};
     epi.sc = m.postbuf.p;
     epi.sh = m.postbuf.p + n_out;
     epi.leak = post->leak;
@@ -1138,14 +1157,14 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   if (bn && groups == 1 && !resident_fits(t, n_in, n_out, true)) {
     const int n_pad = (int)round_up(n_in, 64) + 64;
     m.prebuf.reserve(2 * (size_t)n_pad);
-    k_pre_coeffs<<<dim3((unsigned)ceil_div(n_pad, 256)), 256, 0, s>>>(bn->mean, bn->var, bn->gamma, bn->beta, bn->eps,
-                                                                     n_in, n_pad, m.prebuf.p, m.prebuf.p + n_pad);
-    LAUNCH_CHECK();
+    m.jobs.pre = CoefJob{bn->mean, bn->var, bn->gamma, bn->beta, bn->eps, n_in, n_pad, m.prebuf.p,
+                         m.prebuf.p + n_pad};
     PreArgs pre;
     pre.sc = m.prebuf.p;
     pre.sh = m.prebuf.p + n_pad;
     pre.leak = bn->leak;
     if (conv_mfma_paths<true>(m, t, in, out, w, epi, n_in, n_out, pre, s)) return;
+    m.jobs.pre = CoefJob();
   }
   const float *src = in;
   if (bn) {  // no fused kernel for this shape: normalise the rows in a pass of their own
@@ -1155,6 +1174,10 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     src = m.bntmp.p;
   }
   if (groups == 1 && conv_mfma_paths<false>(m, t, src, out, w, epi, n_in, n_out, PreArgs(), s)) return;
+  if (m.jobs.post.n_pad) {  // no packing launch on this path: fold the coefficients by themselves
+    k_coefs<<<dim3(1), 256, 0, s>>>(take_jobs(m));
+    LAUNCH_CHECK();
+  }
   int64_t total = t.n * n_out;
   k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, src,
                                                                        out, w, epi, n_in, n_out, groups);

@@ -62,6 +62,17 @@ struct StridedRules {
   SizeKey in_size, out_size;
 };
 
+// A batch norm to fold to scale / shift arrays (device pointers); n_pad == 0: nothing to do.
+struct CoefJob {
+  const float *mean = nullptr, *var = nullptr, *gamma = nullptr, *beta = nullptr;
+  float eps = 0.f;
+  int n = 0, n_pad = 0;
+  float *sc = nullptr, *sh = nullptr;
+};
+struct CoefJobs {
+  CoefJob pre, post;
+};
+
 struct InputRules {
   int mode = -1;
   int max_active = 0;
@@ -88,6 +99,7 @@ struct Metadata {
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
   DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
+  CoefJobs jobs;          // coefficient arrays the next weight-packing launch has to fill
   DevBuf<float> postbuf;  // scale / shift of a batch norm fused into the running convolution's stores
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
   DevBuf<float> bntmp;    // normalised input when a fused batch norm has no fused kernel
