@@ -98,8 +98,16 @@ int scn_rules_sizes(scn_metadata *md, int kind, const int64_t *a, const int64_t 
                     const int64_t *c, const int64_t *d, void *stream, int64_t *sizes);
 int scn_rules_export(scn_metadata *md, int kind, const int64_t *a, const int64_t *b,
                      const int64_t *c, const int64_t *d, int k, int32_t *pairs, void *stream);
-
 /* ---- forward ops (sparseconvnet.h:22-246) -------------------------------- */
+
+/* The convolution calls below return the multiply-add count the reference returns
+ * (CPU/Convolution.cpp:141) through `macs`; the first time a rulebook is used that costs a
+ * stream synchronisation (the rule counts are tallied on the device).  A caller that passes
+ * macs = NULL has the count added to a per-metadata total instead, which this call returns
+ * and resets (one synchronisation for everything that is still outstanding): asked once,
+ * after a network has been enqueued, it keeps the GPU busy in between.  The reference has no
+ * counterpart; its Python layer sums the per-call values (sparseconvnet/__init__.py:7). */
+int scn_md_take_macs(scn_metadata *md, void *stream, double *macs);
 
 /* InputLayer_updateOutput after the rules exist (pybind.cpp:155-159, CPU/IOLayers.cpp:49-72):
  * in [nInputRows, planes] -> out [nActive, planes]. */
@@ -111,7 +119,7 @@ int scn_output_layer_fwd(scn_metadata *md, const float *in, float *out, int plan
 
 /* SubmanifoldConvolution_updateOutput (pybind.cpp:135-139, CPU/Convolution.cpp:117-150).
  * in [nActive, nIn] -> out [nActive, nOut]; bias may be NULL; *macs receives the
- * multiply-add count the reference returns (CPU/Convolution.cpp:141). */
+ * multiply-add count the reference returns (CPU/Convolution.cpp:141); macs may be NULL. */
 int scn_subm_conv_fwd(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
                       const float *in, float *out, const float *weight, const float *bias,
                       int n_in, int n_out, int groups, void *stream, double *macs);

@@ -4,8 +4,9 @@ as scn`).  The modules call hand-written gfx950 kernels in libscn_hip.so through
 (include/scn_hip.h); tensors are ordinary PyTorch-ROCm tensors."""
 
 # Counters the reference keeps at package level (sparseconvnet/__init__.py:7-8): multiply-adds
-# and output elements of the convolutions run so far.
-forward_pass_multiplyAdd_count = 0
+# and output elements of the convolutions run so far.  forward_pass_multiplyAdd_count is a
+# property of this module (see the end of the file): reading it collects the counts the
+# library has been keeping on the GPU side.
 forward_pass_hidden_states = 0
 # Sequential hands an eval-mode batch normalisation that sits directly in front of a
 # convolution to that convolution (one pass over the rows instead of two).  False: run
@@ -30,3 +31,22 @@ def is_hip_build():
         return True
     except Exception:
         return False
+
+
+import sys as _sys  # noqa: E402
+import types as _types  # noqa: E402
+
+from .metadata import mac_counter as _mac_counter  # noqa: E402
+
+
+class _Package(_types.ModuleType):
+    @property
+    def forward_pass_multiplyAdd_count(self):
+        return _mac_counter.read()
+
+    @forward_pass_multiplyAdd_count.setter
+    def forward_pass_multiplyAdd_count(self, value):
+        _mac_counter.reset(value)
+
+
+_sys.modules[__name__].__class__ = _Package

@@ -37,6 +37,7 @@ SIGNATURES = {
     "scn_rules_count": (C.c_int, [_vp, C.c_int, _i64p, _i64p, _i64p, _i64p, _vp, C.POINTER(C.c_int)]),
     "scn_rules_sizes": (C.c_int, [_vp, C.c_int, _i64p, _i64p, _i64p, _i64p, _vp, _i64p]),
     "scn_rules_export": (C.c_int, [_vp, C.c_int, _i64p, _i64p, _i64p, _i64p, C.c_int, _vp, _vp]),
+    "scn_md_take_macs": (C.c_int, [_vp, _vp, C.POINTER(C.c_double)]),
     "scn_input_layer_fwd": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp]),
     "scn_output_layer_fwd": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp]),
     "scn_subm_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int,

@@ -186,16 +186,19 @@ int scn_rules_count(scn_metadata *h, int kind, const int64_t *a, const int64_t *
       throw Error("unknown rulebook kind");
   });
 }
+int scn_md_take_macs(scn_metadata *h, void *stream, double *macs) {
+  return guarded([&] { *macs = take_macs(md(h), st(stream)); });
+}
 int scn_rules_sizes(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
                     const int64_t *d, void *stream, int64_t *sizes) {
   return guarded([&] {
     Metadata &m = md(h);
     std::vector<int64_t> v;
-    if (kind == 0)
-      v = submanifold_rules(m, a, b, st(stream)).counts;
-    else if (kind == 1)
-      v = strided_rules(m, a, b, c, d, st(stream)).by_out.counts;
-    else if (kind == 2)
+    if (kind == 0) {
+      v = submanifold_rules(m, a, b, st(stream)).counts(st(stream));
+    } else if (kind == 1) {
+      v = strided_rules(m, a, b, c, d, st(stream)).by_out.counts(st(stream));
+    } else if (kind == 2)
       v = s2d_sizes(m, a, st(stream));
     else
       throw Error("unknown rulebook kind");
@@ -237,7 +240,7 @@ static void subm_conv(scn_metadata *h, const int64_t *spatial, const int64_t *fi
   Table &t = submanifold_rules(m, spatial, filter, st(stream));
   conv_forward(m, t, in, level_rows(m, spatial), out, weight, bias, n_in, n_out, groups, pre, post, st(stream));
   // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
-  if (macs) *macs = (double)t.total() * (n_in / groups) * (n_out / groups) * groups;
+  note_macs(m, t, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
 }
 static void strided_conv(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                          const int64_t *stride, const float *in, float *out, const float *weight,
@@ -247,7 +250,7 @@ static void strided_conv(scn_metadata *h, const int64_t *in_size, const int64_t 
   StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
   conv_forward(m, r.by_out, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
                st(stream));
-  if (macs) *macs = (double)r.by_out.total() * (n_in / groups) * (n_out / groups) * groups;
+  note_macs(m, r.by_out, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
 }
 static void deconv(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                    const int64_t *stride, const float *in, float *out, const float *weight, const float *bias,
@@ -258,7 +261,7 @@ static void deconv(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
   StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
   conv_forward(m, r.by_in, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
                st(stream));
-  if (macs) *macs = (double)r.by_in.total() * (n_in / groups) * (n_out / groups) * groups;
+  note_macs(m, r.by_in, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
 }
 
 int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,

@@ -23,14 +23,17 @@ struct Level {
   // caller's points came in.  Null when rows are already numbered by ascending key.
   DevBuf<int> sched;
   bool identity_sched = false;
-  // Site lookup (common.h: BlockEntry), built on first use: block table + row of every
-  // distinct site in key order.  `dups` marks levels whose keys may repeat (input-layer mode 0
-  // with repeated points: the last one wins, as with `mp[p] = i` in the reference).
+  // Site lookup (common.h: BlockEntry), built on first use: block table, its mask (capacity
+  // - 1, decided and kept on the device: gridp[0]) and the row of every distinct site in key
+  // order.  `dups` marks levels whose keys may repeat (input-layer mode 0 with repeated
+  // points: the last one wins, as with `mp[p] = i` in the reference); only those need `urow`,
+  // elsewhere the u-th distinct site is schedule position u.
   DevBuf<BlockEntry> table;
-  uint64_t mask = 0;
+  DevBuf<unsigned long long> gridp;
   DevBuf<int> urow;
   bool grid_built = false;
   bool dups = false;
+  const int *urow_ptr() const { return dups ? urow.p : sched_ptr(); }
   const int *sched_ptr() const { return identity_sched ? nullptr : sched.p; }
 };
 
@@ -40,6 +43,24 @@ struct Level {
 // by neighbour pattern (number of absent taps, then the bit mask of present taps), so that
 // the positions a workgroup takes mostly need the same taps.  counts[k] = number of
 // non-negative entries of tap k.
+// Rule counts per tap of a rulebook.  They are tallied on the device while the rules are
+// written and fetched only when somebody needs them on the host (multiply-add counts, list
+// sizes of the export), so that building a rulebook needs no host round trip for them.  The
+// two tables of a strided rulebook share one object; so do deferred multiply-add counts
+// (Metadata::pending_macs), which is why it is held by shared_ptr.
+struct Counts {
+  int K = 0;
+  DevBuf<long long> dev;
+  std::vector<int64_t> host;
+  bool ready = false;  // host is valid
+  int64_t total() const {
+    int64_t s = 0;
+    for (auto c : host) s += c;
+    return s;
+  }
+};
+void ensure_counts(Counts &c, hipStream_t s);  // fetches dev into host (one stream synchronisation)
+
 struct Table {
   int K = 0;
   int64_t n = 0, npad = 0;
@@ -48,11 +69,14 @@ struct Table {
   DevBuf<unsigned> gmask;  // K <= 32 and pattern-sorted: bit k of gmask[i] = some position of granule i (16 positions) has tap k
   bool identity_rows = false;  // rowmap[t] == t: kernels skip the indirection
   const int *rowmap_ptr() const { return identity_rows ? nullptr : rowmap.p; }
-  std::vector<int64_t> counts;
-  int64_t total() const {
-    int64_t s = 0;
-    for (auto c : counts) s += c;
-    return s;
+  std::shared_ptr<Counts> cnt;  // never null once the table has been built
+  const std::vector<int64_t> &counts(hipStream_t s) {
+    ensure_counts(*cnt, s);
+    return cnt->host;
+  }
+  int64_t total(hipStream_t s) {
+    ensure_counts(*cnt, s);
+    return cnt->total();
   }
 };
 
@@ -99,6 +123,10 @@ struct Metadata {
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
   DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
+  // Multiply-add counts of forward calls that did not ask for theirs (macs == NULL): settled
+  // ones summed, the others as (counts, multiply-adds per rule) until take_macs() fetches them.
+  double macs_settled = 0;
+  std::vector<std::pair<std::shared_ptr<Counts>, double>> pending_macs;
   CoefJobs jobs;          // coefficient arrays the next weight-packing launch has to fill
   DevBuf<float> postbuf;  // scale / shift of a batch norm fused into the running convolution's stores
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
@@ -116,7 +144,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
                             const int64_t *filter, const int64_t *stride, hipStream_t s);
 // Pairs of tap k of a table: (value, row at position t), ordered by t.  Returns the count.
-int64_t export_table_pairs(Metadata &m, const Table &t, int k, bool swap, int *pairs, hipStream_t s);
+int64_t export_table_pairs(Metadata &m, Table &t, int k, bool swap, int *pairs, hipStream_t s);
 std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t s);
 int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *pairs,
                          hipStream_t s);
@@ -127,6 +155,8 @@ struct BnArgs {  // eval batch norm + leaky ReLU in front of a convolution (devi
   const float *mean, *var, *gamma, *beta;
   float eps, leak;
 };
+void note_macs(Metadata &m, Table &t, double per_rule, double *macs, hipStream_t s);
+double take_macs(Metadata &m, hipStream_t s);
 void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
                   const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, const BnArgs *post,
                   hipStream_t s);

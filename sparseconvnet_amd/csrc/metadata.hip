@@ -362,91 +362,112 @@ __global__ void k_compact_sites(const unsigned long long *skey, const int *sched
   ukey[u] = skey[t];
   urow[u] = sched ? sched[t] : (int)t;
 }
-__global__ void k_copy_rows(const int *sched, int64_t n, int *urow) {
+// The size of a level's block table is decided on the device (no host round trip): from the
+// number of blocks, capacity = the power of two >= 2 * blocks (at least 64).
+__device__ inline unsigned long long grid_capacity(long long nblocks) {
+  unsigned long long cap = 64;
+  while (cap < (unsigned long long)nblocks * 2ull) cap <<= 1;
+  return cap;
+}
+// skey[t] = key of the row at schedule position t; head[t] = 1 where a block of 64 keys starts.
+__global__ void k_grid_heads(const unsigned long long *keys, const int *sched, int64_t n,
+                             unsigned long long *skey, int *head) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t < n) urow[t] = sched ? sched[t] : (int)t;
+  if (t >= n) return;
+  const unsigned long long k = keys[sched ? sched[t] : t];
+  skey[t] = k;
+  head[t] = (t == 0 || (k >> 6) != (keys[sched ? sched[t - 1] : t - 1] >> 6)) ? 1 : 0;
 }
 __global__ void k_block_heads(const unsigned long long *ukey, int64_t n, int *head) {
   int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (u < n) head[u] = (u == 0 || (ukey[u] >> 6) != (ukey[u - 1] >> 6)) ? 1 : 0;
 }
-// Block heads claim a slot and record their rank.
-__global__ void k_block_insert(const unsigned long long *ukey, const int *head, int64_t n, BlockEntry *table,
-                               unsigned long long mask) {
+// Empties the part of the table that will be used and records its mask (capacity - 1) for the
+// kernels that follow.  n_sites_dev: the number of distinct sites when it is only known on
+// the device (levels with repeated keys), else null.
+__global__ void k_block_clear(BlockEntry *table, int64_t cap_alloc, const int *head, const int *head_scan,
+                              int64_t n_sites, const int *n_sites_dev, unsigned long long *mask_out) {
+  int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t U = n_sites_dev ? (int64_t)*n_sites_dev + 1 : n_sites;
+  const unsigned long long cap = grid_capacity(U > 0 ? (long long)head_scan[U - 1] + head[U - 1] : 0);
+  if (b == 0) *mask_out = cap - 1;
+  if (b < cap_alloc && (unsigned long long)b < cap) {
+    table[b].key = SCN_EMPTY_KEY;
+    table[b].mask = 0ull;
+    table[b].base = 0;
+  }
+}
+// The first site of every block collects the occupancy bits of its block (its run of at most
+// 64 consecutive distinct keys), claims a slot and stores key, mask and its own rank.
+__global__ void k_block_insert(const unsigned long long *ukey, const int *head, int64_t n_sites,
+                               const int *n_sites_dev, BlockEntry *table, const unsigned long long *mask_p) {
   int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (u >= n || !head[u]) return;
-  unsigned long long bkey = ukey[u] >> 6;
+  const int64_t U = n_sites_dev ? (int64_t)*n_sites_dev + 1 : n_sites;
+  if (u >= U || !head[u]) return;
+  const unsigned long long mask = *mask_p;
+  const unsigned long long bkey = ukey[u] >> 6;
+  unsigned long long bits = 0;
+  for (int64_t v = u; v < U && v < u + 64; v++) {
+    const unsigned long long k = ukey[v];
+    if ((k >> 6) != bkey) break;
+    bits |= 1ull << (k & 63);
+  }
   unsigned long long b = hash64(bkey) & mask;
   for (unsigned long long i = 0; i <= mask; i++) {
     unsigned long long old = atomicCAS(&table[b].key, SCN_EMPTY_KEY, bkey);
     if (old == SCN_EMPTY_KEY) {
+      table[b].mask = bits;
       table[b].base = (int)u;
       return;
     }
     b = (b + 1) & mask;
   }
 }
-// Every distinct site sets its bit in its block's mask.
-__global__ void k_block_masks(const unsigned long long *ukey, int64_t n, BlockEntry *table,
-                              unsigned long long mask) {
-  int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (u >= n) return;
-  unsigned long long key = ukey[u];
-  int64_t slot = block_find(table, mask, key >> 6);
-  if (slot >= 0) atomicOr(&table[slot].mask, 1ull << (key & 63));
-}
-
-__global__ void k_block_zero_masks(BlockEntry *table, int64_t cap) {
-  int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (b < cap) table[b].mask = 0ull;
-}
 
 static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   if (L.grid_built) return;
   const int64_t n = L.n;
-  int64_t U = n, nblocks = 0;
   m.k0.reserve(n + 1);
   m.k1.reserve(n + 1);
   m.f0.reserve(n + 1);
   m.s0.reserve(n + 1);
-  L.urow.reserve(std::max<int64_t>(n, 1));
-  unsigned long long *ukey = m.k0.p;
+  L.gridp.reserve(2);
+  // every site could be a block of its own: room for that, of which only the part the
+  // device-side capacity covers is ever touched
+  uint64_t cap_alloc = 64;
+  while (cap_alloc < (uint64_t)n * 2) cap_alloc <<= 1;
+  L.table.reserve(cap_alloc);
+  const unsigned long long *ukey = m.k0.p;
+  const int *n_sites_dev = nullptr;
   if (n) {
-    k_sorted_keys<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, m.k0.p);
-    LAUNCH_CHECK();
     if (L.dups) {
-      k_run_tails<<<grid_for(n), TB, 0, s>>>(m.k0.p, n, m.f0.p);
+      // distinct sites first: ukey / urow by compaction; their number stays on the device
+      k_sorted_keys<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, m.k0.p);
       LAUNCH_CHECK();
-      exclusive_scan(m, m.f0.p, m.s0.p, n, s);
-      k_compact_sites<<<grid_for(n), TB, 0, s>>>(m.k0.p, L.sched_ptr(), m.f0.p, m.s0.p, n, m.k1.p, L.urow.p);
+      m.f1.reserve(n + 1);
+      m.s1.reserve(n + 1);
+      L.urow.reserve(n);
+      k_run_tails<<<grid_for(n), TB, 0, s>>>(m.k0.p, n, m.f1.p);
       LAUNCH_CHECK();
-      U = read_back(m.s0.p + (n - 1), s) + 1;  // the last position always ends a run
+      exclusive_scan(m, m.f1.p, m.s1.p, n, s);
+      k_compact_sites<<<grid_for(n), TB, 0, s>>>(m.k0.p, L.sched_ptr(), m.f1.p, m.s1.p, n, m.k1.p, L.urow.p);
+      LAUNCH_CHECK();
+      n_sites_dev = m.s1.p + (n - 1);  // index of the last distinct site (the last position ends a run)
       ukey = m.k1.p;
+      // positions past the last distinct site hold stale keys: heads there are never read
+      k_block_heads<<<grid_for(n), TB, 0, s>>>(ukey, n, m.f0.p);
+      LAUNCH_CHECK();
     } else {
-      k_copy_rows<<<grid_for(n), TB, 0, s>>>(L.sched_ptr(), n, L.urow.p);
+      k_grid_heads<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, m.k0.p, m.f0.p);
       LAUNCH_CHECK();
     }
-    k_block_heads<<<grid_for(U), TB, 0, s>>>(ukey, U, m.f0.p);
-    LAUNCH_CHECK();
-    exclusive_scan(m, m.f0.p, m.s0.p, U, s);
-    int last[2];
-    HIP_CHECK(hipMemcpyAsync(&last[0], m.s0.p + (U - 1), sizeof(int), hipMemcpyDeviceToHost, s));
-    HIP_CHECK(hipMemcpyAsync(&last[1], m.f0.p + (U - 1), sizeof(int), hipMemcpyDeviceToHost, s));
-    HIP_CHECK(hipStreamSynchronize(s));
-    nblocks = (int64_t)last[0] + last[1];
+    exclusive_scan(m, m.f0.p, m.s0.p, n, s);
   }
-  uint64_t cap = 64;
-  while (cap < (uint64_t)nblocks * 2) cap <<= 1;
-  L.table.reserve(cap);
-  L.mask = cap - 1;
-  // key = EMPTY (all ones); masks must start at zero
-  fill32(L.table.p, 0xFFFFFFFFu, (int64_t)cap * 8, s);
+  k_block_clear<<<grid_for((int64_t)cap_alloc), TB, 0, s>>>(L.table.p, (int64_t)cap_alloc, m.f0.p, m.s0.p, n,
+                                                           n_sites_dev, L.gridp.p);
+  LAUNCH_CHECK();
   if (n) {
-    k_block_insert<<<grid_for(U), TB, 0, s>>>(ukey, m.f0.p, U, L.table.p, L.mask);
-    LAUNCH_CHECK();
-    k_block_zero_masks<<<grid_for((int64_t)cap), TB, 0, s>>>(L.table.p, (int64_t)cap);
-    LAUNCH_CHECK();
-    k_block_masks<<<grid_for(U), TB, 0, s>>>(ukey, U, L.table.p, L.mask);
+    k_block_insert<<<grid_for(n), TB, 0, s>>>(ukey, m.f0.p, n, n_sites_dev, L.table.p, L.gridp.p);
     LAUNCH_CHECK();
   }
   L.grid_built = true;
@@ -463,8 +484,9 @@ struct Filt {
 // (Metadata/SubmanifoldConvolutionRules.h:11-45; taps enumerate the box row-major with the
 // last dimension fastest, Metadata/RectangularRegions.h:56-71).
 __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, int64_t n,
-                             int64_t npad, const BlockEntry *table, unsigned long long mask,
+                             int64_t npad, const BlockEntry *table, const unsigned long long *mask_p,
                              const int *urow, int *nbr, unsigned long long *counts, int parts) {
+  const unsigned long long mask = *mask_p;
   // blockDim = 64 * parts: wavefront p of the block handles taps [p*K/parts, (p+1)*K/parts)
   // (one slice of the first filter dimension) of the block's 64 positions.
   extern __shared__ int lcount[];
@@ -507,7 +529,10 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
           last_base = slot >= 0 ? table[slot].base : 0;
         }
         const unsigned long long bit = 1ull << (key & 63);
-        if (last_mask & bit) j = urow[last_base + __popcll(last_mask & (bit - 1))];
+        if (last_mask & bit) {
+          const int r = last_base + __popcll(last_mask & (bit - 1));
+          j = urow ? urow[r] : r;
+        }
       }
       if (live) nbr[(int64_t)k * npad + t] = j;
       const unsigned long long hits = __ballot(live && j >= 0);
@@ -626,8 +651,9 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
 // One wavefront per slice of the first filter dimension, as in k_subm_rules.
 template <int DIM>
 __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_t n, int64_t npad,
-                                const BlockEntry *table, unsigned long long mask, const int *urow, int *nbr,
-                                unsigned long long *counts) {
+                                const BlockEntry *table, const unsigned long long *mask_p, const int *urow,
+                                int *nbr, unsigned long long *counts) {
+  const unsigned long long mask = *mask_p;
   constexpr int K = DIM == 3 ? 27 : 9;
   constexpr int PER = K / 3;
   __shared__ int lcount[K];
@@ -678,7 +704,10 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
         last_base = slot >= 0 ? table[slot].base : 0;
       }
       const unsigned long long bit = 1ull << (key & 63);
-      if (last_mask & bit) j = urow[last_base + __popcll(last_mask & (bit - 1))];
+      if (last_mask & bit) {
+        const int r = last_base + __popcll(last_mask & (bit - 1));
+        j = urow ? urow[r] : r;
+      }
     }
     if (live) nbr[(int64_t)k * npad + t] = j;
     const unsigned long long hits = __ballot(live && j >= 0);
@@ -708,11 +737,65 @@ static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const
   return f;
 }
 
-static void fetch_counts(Metadata &m, Table &t, hipStream_t s) {
-  std::vector<unsigned long long> h(t.K);
-  HIP_CHECK(hipMemcpyAsync(h.data(), m.dcounts.p, t.K * sizeof(long long), hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipStreamSynchronize(s));
-  t.counts.assign(h.begin(), h.end());
+static void start_counts(Table &t, hipStream_t s) {
+  t.cnt = std::make_shared<Counts>();
+  t.cnt->K = t.K;
+  t.cnt->dev.reserve(std::max(t.K, 1));
+  fill32(t.cnt->dev.p, 0, 2 * (int64_t)std::max(t.K, 1), s);
+}
+static void zero_counts(Table &t) {  // a table without rules
+  t.cnt = std::make_shared<Counts>();
+  t.cnt->K = t.K;
+  t.cnt->host.assign(t.K, 0);
+  t.cnt->ready = true;
+}
+void ensure_counts(Counts &c, hipStream_t s) {
+  if (c.ready) return;
+  std::vector<unsigned long long> h(c.K);
+  if (c.K && c.dev.p) {
+    HIP_CHECK(hipMemcpyAsync(h.data(), c.dev.p, c.K * sizeof(long long), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+  }
+  c.host.assign(h.begin(), h.end());
+  c.ready = true;
+}
+// A forward call over table t did per_rule multiply-adds per rule.  With macs != NULL the
+// caller wants the number now; otherwise it is remembered and summed up by take_macs().
+void note_macs(Metadata &m, Table &t, double per_rule, double *macs, hipStream_t s) {
+  if (macs) {
+    *macs = (double)t.total(s) * per_rule;
+  } else if (t.cnt->ready) {
+    m.macs_settled += (double)t.cnt->total() * per_rule;
+  } else {
+    m.pending_macs.emplace_back(t.cnt, per_rule);
+  }
+}
+// Sum of the deferred multiply-add counts since the last call; at most one synchronisation
+// (all copies are queued first).
+double take_macs(Metadata &m, hipStream_t s) {
+  std::vector<std::vector<unsigned long long>> tmp(m.pending_macs.size());
+  bool queued = false;
+  for (size_t i = 0; i < m.pending_macs.size(); i++) {
+    Counts &c = *m.pending_macs[i].first;
+    if (c.ready || !c.K || !c.dev.p) continue;
+    tmp[i].resize(c.K);
+    HIP_CHECK(hipMemcpyAsync(tmp[i].data(), c.dev.p, c.K * sizeof(long long), hipMemcpyDeviceToHost, s));
+    queued = true;
+  }
+  if (queued) HIP_CHECK(hipStreamSynchronize(s));
+  for (size_t i = 0; i < m.pending_macs.size(); i++) {
+    Counts &c = *m.pending_macs[i].first;
+    if (!c.ready) {
+      c.host.assign(tmp[i].begin(), tmp[i].end());
+      if (c.host.empty()) c.host.assign(c.K, 0);
+      c.ready = true;
+    }
+    m.macs_settled += (double)c.total() * m.pending_macs[i].second;
+  }
+  m.pending_macs.clear();
+  double r = m.macs_settled;
+  m.macs_settled = 0;
+  return r;
 }
 
 Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s) {
@@ -728,7 +811,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
     t.n = 0;
     t.npad = 64;
     t.identity_rows = true;
-    t.counts.assign(f.K, 0);
+    zero_counts(t);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
   Level &L = lit->second;
@@ -736,31 +819,28 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   t.n = L.n;
   t.npad = L.npad;
   t.nbr.reserve((size_t)f.K * t.npad);
-  m.dcounts.reserve(4096);
-  fill32(m.dcounts.p, 0, 2 * f.K, s);
+  start_counts(t, s);
   bool all3 = true;
   for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
   if (all3 && (m.dim == 2 || m.dim == 3)) {
     if (m.dim == 3)
       k_subm_rules_s3<3><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
-                                                           L.mask, L.urow.p, t.nbr.p,
-                                                           (unsigned long long *)m.dcounts.p);
+                                                           L.gridp.p, L.urow_ptr(), t.nbr.p,
+                                                           (unsigned long long *)t.cnt->dev.p);
     else
       k_subm_rules_s3<2><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
-                                                           L.mask, L.urow.p, t.nbr.p,
-                                                           (unsigned long long *)m.dcounts.p);
+                                                           L.gridp.p, L.urow_ptr(), t.nbr.p,
+                                                           (unsigned long long *)t.cnt->dev.p);
     LAUNCH_CHECK();
-    fetch_counts(m, t, s);
     finalize_table(m, t, L.sched_ptr(), s);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
   // one wavefront per slice of the first filter dimension when that divides the taps evenly
   const int parts = (m.dim >= 2 && f.size[0] <= 4) ? f.size[0] : 1;
   k_subm_rules<<<grid_for(L.n, 64), 64 * parts, f.K * sizeof(int), s>>>(
-      L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p, L.mask, L.urow.p, t.nbr.p,
-      (unsigned long long *)m.dcounts.p, parts);
+      L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p, L.gridp.p, L.urow_ptr(), t.nbr.p,
+      (unsigned long long *)t.cnt->dev.p, parts);
   LAUNCH_CHECK();
-  fetch_counts(m, t, s);
   finalize_table(m, t, L.sched_ptr(), s);
   return m.subm.emplace(key, std::move(t)).first->second;
 }
@@ -851,8 +931,8 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   R.in_size = mk(m.dim, in_size);
   R.out_size = mk(m.dim, out_size);
   R.by_out.K = R.by_in.K = f.K;
-  R.by_out.counts.assign(f.K, 0);
-  R.by_in.counts.assign(f.K, 0);
+  zero_counts(R.by_out);
+  R.by_in.cnt = R.by_out.cnt;  // until rules are emitted below
   if (R.in_size == R.out_size) throw Error("strided rules: input and output spatial size coincide");
 
   auto lit = m.levels.find(R.in_size);
@@ -916,14 +996,12 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   R.by_in.nbr.reserve((size_t)f.K * LI.npad);
   fill32(R.by_out.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LO.npad, s);
   fill32(R.by_in.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LI.npad, s);
-  m.dcounts.reserve(4096);
-  fill32(m.dcounts.p, 0, 2 * f.K, s);
+  start_counts(R.by_out, s);
   k_strided_emit<<<grid_for(nc), TB, f.K * sizeof(int), s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), LI.npad, m.k1.p, m.v1.p,
                                              m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
-                                             LO.coords.p, LO.keys.p, (unsigned long long *)m.dcounts.p);
+                                             LO.coords.p, LO.keys.p, (unsigned long long *)R.by_out.cnt->dev.p);
   LAUNCH_CHECK();
-  fetch_counts(m, R.by_out, s);
-  R.by_in.counts = R.by_out.counts;
+  R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
   finalize_table(m, R.by_out, nullptr, s);
   finalize_table(m, R.by_in, LI.sched_ptr(), s);
   return m.strided.emplace(key, std::move(R)).first->second;
@@ -972,10 +1050,11 @@ __global__ void k_tap_compact(const int *nbr, const int *sched, int64_t n, const
     pairs[2 * pos + (swap ? 0 : 1)] = row;
   }
 }
-int64_t export_table_pairs(Metadata &m, const Table &t, int k, bool swap, int *pairs, hipStream_t s) {
+int64_t export_table_pairs(Metadata &m, Table &t, int k, bool swap, int *pairs, hipStream_t s) {
   const int *sched = t.rowmap_ptr();
   if (k < 0 || k >= t.K) throw Error("rule list index out of range");
-  if (t.n == 0 || t.counts[k] == 0) return 0;
+  const int64_t count_k = t.counts(s)[k];
+  if (t.n == 0 || count_k == 0) return 0;
   int64_t blocks = ceil_div(t.n, TB);
   m.f1.reserve(blocks + 1);
   m.s1.reserve(blocks + 1);
@@ -985,7 +1064,7 @@ int64_t export_table_pairs(Metadata &m, const Table &t, int k, bool swap, int *p
   exclusive_scan(m, m.f1.p, m.s1.p, blocks, s);
   k_tap_compact<<<dim3((unsigned)blocks), TB, 0, s>>>(col, sched, t.n, m.s1.p, swap, pairs);
   LAUNCH_CHECK();
-  return t.counts[k];
+  return count_k;
 }
 
 // Sparse-to-dense lists: per sample, (row, row-major offset) (Metadata/ConvolutionRules.h:130-151).

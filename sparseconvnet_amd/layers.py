@@ -53,8 +53,8 @@ def _conv_weight(filter_volume, groups, nIn, nOut):
     return Parameter(torch.Tensor(filter_volume, groups, nIn // groups, nOut // groups).normal_(0, std))
 
 
-def _count(macs, out):
-    _pkg.forward_pass_multiplyAdd_count += macs
+def _count(out):
+    # the multiply-adds are counted by the library (Metadata.takeMacs), see metadata.MacCounter
     _pkg.forward_pass_hidden_states += out.nelement()
 
 
@@ -124,8 +124,8 @@ class SubmanifoldConvolution(Module):
         md, sz, fs, bn, post = input.metadata, input.spatial_size, self.filter_size, _bn_args(pre_bn), _bn_args(post_bn)
 
         def fn(x, w, b):
-            y, macs = md.submanifoldConvolution(sz, fs, x, w, b, bn, post)
-            _count(macs, y)
+            y, _ = md.submanifoldConvolution(sz, fs, x, w, b, bn, post, want_macs=False)
+            _count(y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
         return output
@@ -169,8 +169,8 @@ class Convolution(Module):
         bn, post = _bn_args(pre_bn), _bn_args(post_bn)
 
         def fn(x, w, b):
-            y, macs = md.convolution(*a, x, w, b, bn, post)
-            _count(macs, y)
+            y, _ = md.convolution(*a, x, w, b, bn, post, want_macs=False)
+            _count(y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
         return output
@@ -208,8 +208,8 @@ class Deconvolution(Module):
         bn, post = _bn_args(pre_bn), _bn_args(post_bn)
 
         def fn(x, w, b):
-            y, macs = md.deconvolution(*a, x, w, b, bn, post)
-            _count(macs, y)
+            y, _ = md.deconvolution(*a, x, w, b, bn, post, want_macs=False)
+            _count(y)
             return y
         output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
         return output

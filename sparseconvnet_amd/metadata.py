@@ -5,6 +5,7 @@ Mirrors the object the reference exposes as `sparseconvnet.Metadata(dim)`
 as a thin owner of a handle of libscn_hip.so.  Everything lives on the GPU; only counts
 cross back to the host."""
 import ctypes as C
+import weakref
 
 import torch
 
@@ -27,6 +28,30 @@ def _features(t, what):
     return t.contiguous()
 
 
+class MacCounter:
+    """The package's forward_pass_multiplyAdd_count (sparseconvnet/__init__.py:7).  The
+    convolutions do not fetch their rule counts when they run (that would stall the GPU once
+    per rulebook); the library keeps a running total per Metadata, which is collected here
+    when somebody reads the counter or the Metadata goes away."""
+
+    def __init__(self):
+        self.base = 0.0
+        self.live = weakref.WeakSet()
+
+    def read(self):
+        for md in list(self.live):
+            self.base += md.takeMacs()
+        return self.base
+
+    def reset(self, value):
+        for md in list(self.live):
+            md.takeMacs()
+        self.base = value
+
+
+mac_counter = MacCounter()
+
+
 class Metadata:
     def __init__(self, dimension):
         self.dimension = dimension
@@ -34,11 +59,24 @@ class Metadata:
         self._h = self._L.scn_md_create(dimension)
         if not self._h:
             raise _lib.ScnError(self._L.scn_last_error().decode())
+        mac_counter.live.add(self)
 
     def __del__(self):
-        h, self._h = getattr(self, "_h", None), None
+        h = getattr(self, "_h", None)
         if h:
+            try:
+                mac_counter.base += self.takeMacs()
+            except Exception:  # interpreter shutdown, lost device: the count is not worth an error
+                pass
+            self._h = None
             self._L.scn_md_destroy(h)
+
+    def takeMacs(self):
+        """Multiply-adds of the convolutions run on this Metadata since the last call whose
+        count was not returned to the caller directly (synchronises the stream once)."""
+        macs = C.c_double(0)
+        _lib.check(self._L.scn_md_take_macs(self._h, _stream(), C.byref(macs)))
+        return macs.value
 
     def _s(self, x):
         return _lib.sizes(self.dimension, x)
@@ -86,20 +124,23 @@ class Metadata:
         _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out
 
-    def _conv(self, kind, size_args, n_rows, features, weight, bias, bn, post):
+    def _conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs):
         """kind 0 / 1 / 2: submanifold / strided / transposed convolution.  bn, post: None, or
         (running_mean, running_var, weight, bias, eps, leakiness) of an eval-mode batch
-        normalisation in front of / behind the convolution, applied inside it."""
+        normalisation in front of / behind the convolution, applied inside it.  want_macs:
+        return the multiply-add count (a stream synchronisation the first time a rulebook is
+        used); otherwise the library adds it to this Metadata's running total (takeMacs)."""
         features = _features(features, "features")
         weight = _features(weight, "weight")
         K, groups, ip, op = weight.shape
         bias_t = _features(bias, "bias") if bias is not None and bias.numel() else None
         out = torch.empty((n_rows, groups * op), dtype=torch.float32, device=features.device)
         macs = C.c_double(0)
+        macs_p = C.byref(macs) if want_macs else None
         tail = (_ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t), groups * ip, groups * op, groups)
         if bn is None and post is None:
             fn = (self._L.scn_subm_conv_fwd, self._L.scn_conv_fwd, self._L.scn_deconv_fwd)[kind]
-            _lib.check(fn(self._h, *size_args, *tail, _stream(), C.byref(macs)))
+            _lib.check(fn(self._h, *size_args, *tail, _stream(), macs_p))
         else:
             keep = []  # tensors behind the raw pointers stay alive until the call has been issued
 
@@ -115,24 +156,27 @@ class Metadata:
                 return C.byref(_lib.BnParams(*[_ptr(x) for x in t], float(eps), float(leak)))
             sizes = list(size_args) + [None] * (4 - len(size_args))
             _lib.check(self._L.scn_conv_bn_fwd(self._h, kind, *sizes, *tail, params(bn, groups * ip),
-                                               params(post, groups * op), _stream(), C.byref(macs)))
-        return out, macs.value
+                                               params(post, groups * op), _stream(), macs_p))
+        return out, (macs.value if want_macs else None)
 
-    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias, bn=None, post=None):
+    def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias, bn=None, post=None,
+                               want_macs=True):
         sp, fs = self._s(spatial_size), self._s(filter_size)
         _lib.check(self._L.scn_md_submanifold_rules(self._h, sp, fs, _stream()))
-        return self._conv(0, (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn, post)
+        return self._conv(0, (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn, post, want_macs)
 
-    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None):
+    def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None,
+                    want_macs=True):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
-        return self._conv(1, a, self.getNActive(out_size), features, weight, bias, bn, post)
+        return self._conv(1, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs)
 
-    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None):
+    def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None,
+                      want_macs=True):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *rb, _stream()))
-        return self._conv(2, a, self.getNActive(out_size), features, weight, bias, bn, post)
+        return self._conv(2, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs)
 
     def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
         a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]

@@ -138,3 +138,44 @@ def test_fused_and_unfused_sequential_agree():
         finally:
             scn.fuse_batchnorm = True
     checks.assert_close(outs[0], outs[1], "fused vs unfused")
+
+
+def test_multiply_add_counter_matches_oracle(oracle_built):
+    """forward_pass_multiplyAdd_count (sparseconvnet/__init__.py:7) is collected lazily from
+    the library; it must equal the sum of the counts the reference returns per layer
+    (CPU/Convolution.cpp:141), also when read twice, after a reset, and when the Metadata has
+    already been dropped."""
+    torch.manual_seed(11)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, 8, 3, False)).add(
+        scn.Convolution(3, 8, 16, 2, 2, False)).add(scn.SubmanifoldConvolution(3, 16, 16, 3, True)).add(
+        scn.Deconvolution(3, 16, 8, 2, 2, False)).cuda().eval()
+    coords = synthetic.scene_batch(seed=1100, batch=2, target=3000, spatial=32, n_boxes=5)
+    feats = np.random.default_rng(11).normal(size=(len(coords), 3)).astype(np.float32)
+    p = cpu_path.CpuPath(3, "oracle")
+    p.input_layer(32, coords, 0, 4)
+    x = p.input_fwd(feats)
+    want = 0.0
+    h, m1 = p.subm_conv(32, 3, x, np.zeros((27, 1, 3, 8), np.float32))
+    p.strided_rules(32, 16, 2, 2)
+    h, m2 = p.conv(32, 16, 2, 2, h, np.zeros((8, 1, 8, 16), np.float32))
+    h, m3 = p.subm_conv(16, 3, h, np.zeros((27, 1, 16, 16), np.float32))
+    h, m4 = p.deconv(16, 32, 2, 2, h, np.zeros((8, 1, 16, 8), np.float32))
+    want = m1 + m2 + m3 + m4
+    scn.forward_pass_multiplyAdd_count = 0
+    scn.forward_pass_hidden_states = 0
+    inp = scn.InputLayer(3, 32, mode=4)([torch.as_tensor(coords), torch.as_tensor(feats).cuda()])
+    with torch.no_grad():
+        out = model(inp)
+    assert scn.forward_pass_multiplyAdd_count == want
+    assert scn.forward_pass_multiplyAdd_count == want  # reading does not consume it
+    with torch.no_grad():
+        model(inp)  # rulebooks cached: the counts are known without a round trip
+    assert scn.forward_pass_multiplyAdd_count == 2 * want
+    scn.forward_pass_multiplyAdd_count = 0
+    with torch.no_grad():
+        out = model(scn.InputLayer(3, 32, mode=4)([torch.as_tensor(coords), torch.as_tensor(feats).cuda()]))
+    del out, inp
+    import gc
+    gc.collect()
+    assert scn.forward_pass_multiplyAdd_count == want
+    assert scn.forward_pass_hidden_states > 0
