@@ -13,6 +13,8 @@
 //     per-tap pair lists; pair lists are produced on demand by ballot/prefix compaction.
 #include <hipcub/hipcub.hpp>
 
+#include <algorithm>
+
 #include "metadata.h"
 
 namespace scn {
@@ -770,28 +772,41 @@ void note_macs(Metadata &m, Table &t, double per_rule, double *macs, hipStream_t
     m.pending_macs.emplace_back(t.cnt, per_rule);
   }
 }
-// Sum of the deferred multiply-add counts since the last call; at most one synchronisation
-// (all copies are queued first).
+// Sum of the deferred multiply-add counts since the last call.  Every rulebook whose counts
+// are still on the device is copied once, through a pinned staging buffer so that the copies
+// are asynchronous, with one synchronisation per staging buffer's worth (in practice one).
 double take_macs(Metadata &m, hipStream_t s) {
-  std::vector<std::vector<unsigned long long>> tmp(m.pending_macs.size());
-  bool queued = false;
-  for (size_t i = 0; i < m.pending_macs.size(); i++) {
-    Counts &c = *m.pending_macs[i].first;
-    if (c.ready || !c.K || !c.dev.p) continue;
-    tmp[i].resize(c.K);
-    HIP_CHECK(hipMemcpyAsync(tmp[i].data(), c.dev.p, c.K * sizeof(long long), hipMemcpyDeviceToHost, s));
-    queued = true;
-  }
-  if (queued) HIP_CHECK(hipStreamSynchronize(s));
-  for (size_t i = 0; i < m.pending_macs.size(); i++) {
-    Counts &c = *m.pending_macs[i].first;
-    if (!c.ready) {
-      c.host.assign(tmp[i].begin(), tmp[i].end());
-      if (c.host.empty()) c.host.assign(c.K, 0);
-      c.ready = true;
+  static thread_local long long *stage = nullptr;
+  constexpr size_t STAGE = 8192;  // entries
+  if (!stage) HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&stage), STAGE * sizeof(long long), hipHostMallocDefault));
+  std::vector<Counts *> batch;
+  size_t used = 0;
+  auto flush = [&]() {
+    if (batch.empty()) return;
+    HIP_CHECK(hipStreamSynchronize(s));
+    size_t off = 0;
+    for (Counts *c : batch) {
+      c->host.assign(stage + off, stage + off + c->K);
+      c->ready = true;
+      off += c->K;
     }
-    m.macs_settled += (double)c.total() * m.pending_macs[i].second;
+    batch.clear();
+    used = 0;
+  };
+  for (auto &pm : m.pending_macs) {
+    Counts &c = *pm.first;
+    if (c.ready || std::find(batch.begin(), batch.end(), &c) != batch.end()) continue;
+    if (!c.K || !c.dev.p || (size_t)c.K > STAGE) {  // nothing on the device (or absurdly many taps): the slow way
+      ensure_counts(c, s);
+      continue;
+    }
+    if (used + c.K > STAGE) flush();
+    HIP_CHECK(hipMemcpyAsync(stage + used, c.dev.p, c.K * sizeof(long long), hipMemcpyDeviceToHost, s));
+    used += c.K;
+    batch.push_back(&c);
   }
+  flush();
+  for (auto &pm : m.pending_macs) m.macs_settled += (double)pm.first->total() * pm.second;
   m.pending_macs.clear();
   double r = m.macs_settled;
   m.macs_settled = 0;
