@@ -196,17 +196,21 @@ __global__ void k_finish_groups(const int *sidx, const int *head, const int *hea
                                 int n_groups, int *row_of_input, int *run_start, int *run_len,
                                 int *max_active) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= n) return;
-  int u = head_scan[p] + head[p] - 1;
-  int row = row_of_group[u];
-  row_of_input[sidx[p]] = row;
-  if (head[p]) {
-    int next = (u + 1 < n_groups) ? head_pos[u + 1] : (int)n;
-    int len = next - (int)p;
-    run_start[row] = (int)p;
-    run_len[row] = len;
-    atomicMax(max_active, len);
+  int len = 0;
+  if (p < n) {
+    int u = head_scan[p] + head[p] - 1;
+    int row = row_of_group[u];
+    row_of_input[sidx[p]] = row;
+    if (head[p]) {
+      int next = (u + 1 < n_groups) ? head_pos[u + 1] : (int)n;
+      len = next - (int)p;
+      run_start[row] = (int)p;
+      run_len[row] = len;
+    }
   }
+  // longest run: one atomic per wavefront, and only when it can raise the maximum
+  for (int off = 32; off; off >>= 1) len = max(len, __shfl_xor(len, off));
+  if ((threadIdx.x & 63) == 0 && len > 1) atomicMax(max_active, len);
 }
 
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
@@ -295,7 +299,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
                                              m.dflags.p + 2);
   LAUNCH_CHECK();
   HIP_CHECK(hipMemcpyAsync(R.sorted_idx.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
-  int ma = read_back(m.dflags.p + 2, s);
+  int ma = std::max(1, read_back(m.dflags.p + 2, s));  // runs of one never touch the counter
   // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2.
   R.max_active = (mode == 3 || mode == 4) ? ma : 1;
 }
