@@ -478,13 +478,14 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
 // granules' [16 x nOut] accumulators in registers.  Compared with k_conv_mfma the gathered
 // rows never touch LDS and one weight slab serves NW*RG*16 rows (up to 512), at the price of
 // uneven MFMA work between wavefronts, which three to four wavefronts per SIMD even out.
-template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE>
+template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF>
 __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
-    const float *__restrict__ pre_sh, float pre_leak) {
+    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
+  static_assert(!BUF || (VEC4 && !PRE), "buffer gathers: float4 rows, no pre-activation");
   constexpr int NT = NW * 64;
   constexpr int G = NW * RG;
   constexpr int TM = G * 16;
@@ -547,6 +548,10 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   unsigned gm_nxt = 0, gm_cur = 0, ok_nxt = 0;
   int sl_nxt = 0;
 
+  typedef int v4i_t __attribute__((ext_vector_type(4)));
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
+  const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
   auto issue = [&](int it) {
     const int ti = it / n_slab, sl = it - ti * n_slab;
     const int k = taplist[ti];
@@ -569,6 +574,18 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 #pragma unroll
     for (int q = 0; q < RG; q++) {
       const int j = jtab[((wave * RG + q) * K + k) * 16 + r16];
+      if constexpr (BUF) {
+        // Buffer loads return zeros past the end of the buffer: an absent row becomes an
+        // offset of 2 GiB (the launcher only takes this path for smaller inputs, whole slabs
+        // and fewer than 2^24 rows), so no select is needed afterwards and the address is
+        // one 24-bit multiply-add.
+        const unsigned voff = j >= 0 ? __umul24((unsigned)j, row_bytes) + lane_off : 0x80000000u;
+#pragma unroll
+        for (int s = 0; s < SS; s++)
+          a_nxt[q][s] = __builtin_bit_cast(
+              v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, (sl * SS + s) * 64, 0));
+        continue;
+      }
       if (j >= 0) ok_nxt |= 1u << q;
       const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
 #pragma unroll
@@ -597,6 +614,10 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
       const bool ok = (ok_nxt >> q) & 1u;
 #pragma unroll
       for (int s = 0; s < SS; s++) {
+        if constexpr (BUF) {
+          a_cur[q][s] = a_nxt[q][s];
+          continue;
+        }
         const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
         v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
         if (VEC4) {
@@ -674,9 +695,16 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   }
 }
 
-template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE>
+template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF = false>
 static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+  if constexpr (VEC4 && !PRE && !BUF) {
+    // gathers through buffer loads (no per-element selects, 32-bit addressing) when the input
+    // is below 2 GiB and 2^24 rows and consists of whole slabs
+    if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
+        m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24))
+      return launch_rows<NCB, RG, SS, VEC4, NW, PRE, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+  }
   constexpr int NT = NW * 64, G = NW * RG;
   constexpr int SLAB_F4 = SS * NCB * 64;
   constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
@@ -690,7 +718,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE, take_jobs(m));
   LAUNCH_CHECK();
-  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE>;
+  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE, BUF>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -709,7 +737,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   }
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), NT, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak);
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
   if (n_split > 1) {
     k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
@@ -1146,6 +1174,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   Epi epi;
   epi.bias = bias;
   m.jobs = CoefJobs();
+  m.cur_in_rows = n_in_rows;
   if (post) {
     m.postbuf.reserve(2 * (size_t)n_out);
     m.jobs.post = CoefJob{post->mean, post->var, post->gamma, post->beta, post->eps, n_out, n_out, m.postbuf.p,
