@@ -761,12 +761,13 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
 // the end re-read the first set).  Granules none of whose rows has the tap skip their MFMAs.
 // With accumulate != 0 the kernel adds to `out` instead of overwriting it (used to split a
 // wide nIn into several launches).
-template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4>
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF>
 __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
     int64_t n, int64_t npad, const float *__restrict__ in, int in_stride, float *__restrict__ out,
     const float *__restrict__ wp, Epi epi, int n_in, int n_out, int n_sets,
-    int sets_per_xcd, int accumulate, int *__restrict__ queue) {
+    int sets_per_xcd, int accumulate, int *__restrict__ queue, unsigned in_bytes, unsigned nbr_bytes) {
+  static_assert(!BUF || VEC4 || C4, "buffer gathers need float4 rows or the four-channel layout");
   static_assert(!C4 || SS == 1, "the four-channel layout has one slab");
   // C4 (nIn <= 4): the MFMA's k index is the input channel itself, so a lane gathers one
   // float (row r16, channel g) and a tap costs one MFMA per column block instead of four.
@@ -853,11 +854,26 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   int jr[3][RG];
   AV ar[3][RG][SS];
   unsigned okr[3];
+  // BUF: neighbour table and input rows are read through buffer loads (32-bit offsets; an
+  // offset of 2 GiB is past the end and reads as zero, which replaces the selects that zero
+  // absent rows).  The launcher takes this variant when both buffers are below 2 GiB, the rows
+  // fewer than 2^24 and the channel part a whole number of slabs.
+  const __amdgpu_buffer_rsrc_t in_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t nbr_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(nbr), 0, BUF ? (int)nbr_bytes : 0, 0x00020000);
+  const unsigned row_bytes = (unsigned)in_stride * 4u;
+  const unsigned lane_off = C4 ? (g < n_in ? 4u * (unsigned)g : 0x80000000u) : 16u * (unsigned)g;
   auto issue_j = [&](const Item &it, int *j) {
 #pragma unroll
     for (int q = 0; q < RG; q++) {
-      const int64_t t = min((int64_t)it.set * (RG * 16) + q * 16 + r16, n - 1);
-      j[q] = nbr[(int64_t)it.k * npad + t];
+      if constexpr (BUF) {
+        const unsigned t = min((unsigned)it.set * (RG * 16) + q * 16 + r16, (unsigned)(n - 1));
+        j[q] = __builtin_amdgcn_raw_buffer_load_b32(nbr_rsrc, t * 4u, (unsigned)it.k * (unsigned)npad * 4u, 0);
+      } else {
+        const int64_t t = min((int64_t)it.set * (RG * 16) + q * 16 + r16, n - 1);
+        j[q] = nbr[(int64_t)it.k * npad + t];
+      }
     }
   };
   auto issue_a = [&](const Item &it, const int *j, AV (*a)[SS], unsigned &okbits) {
@@ -866,6 +882,17 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     for (int q = 0; q < RG; q++) {
       const bool ok = j[q] >= 0 && (int64_t)it.set * (RG * 16) + q * 16 + r16 < n;
       okbits |= ok ? 1u << q : 0u;
+      if constexpr (BUF) {
+        const unsigned voff = ok ? (__umul24((unsigned)j[q], row_bytes) + lane_off) : 0x80000000u;
+#pragma unroll
+        for (int s = 0; s < SS; s++) {
+          if constexpr (C4)
+            a[q][s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(in_rsrc, voff, 0, 0));
+          else
+            a[q][s] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(in_rsrc, voff, s * 64, 0));
+        }
+        continue;
+      }
       const float *src = in + (int64_t)(ok ? j[q] : 0) * in_stride;
 #pragma unroll
       for (int s = 0; s < SS; s++) {
@@ -919,7 +946,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
         for (int q = 0; q < RG; q++) {
           const bool ok = (okb >> q) & 1u;
           if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
-          const float av = (ok && g < n_in) ? ar[S][q][0] : 0.f;
+          const float av = BUF ? ar[S][q][0] : ((ok && g < n_in) ? ar[S][q][0] : 0.f);
 #pragma unroll
           for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[cb], acc[q][cb], 0, 0, 0);
         }
@@ -937,7 +964,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
           for (int s = 0; s < SS; s++) {
             const int c0 = s * 16 + 4 * g;
             v4f av = ar[S][q][s];
-            if (VEC4) {
+            if (BUF) {
+            } else if (VEC4) {
               if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};
             } else {
               if (!(ok && c0 + 0 < n_in)) av.x = 0.f;
@@ -1009,11 +1037,23 @@ __global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, in
   wp[i] = (ch < n_in && col < n_out) ? w[((int64_t)k * n_in + ch) * n_out + col] : 0.0f;
 }
 
-template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4>
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF = false>
 static void launch_resident_kernel(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
                                    Epi epi, int n_in_part, int n_out, int accumulate, size_t lds_bytes,
                                    int per_cu, hipStream_t s) {
-  auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, C4>;
+  // bytes from `in` (which may point at a channel offset inside the first row) to the end
+  const int64_t in_bytes = (m.cur_in_rows * in_stride - (in - m.cur_in_base)) * 4;
+  const int64_t nbr_bytes = (int64_t)t.K * t.npad * 4;
+  if constexpr ((VEC4 || C4) && !BUF) {
+    const bool whole = C4 || n_in_part == 16 * SS;
+    if (whole && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) && in_stride * 4 < (1 << 24) && in_bytes > 0 &&
+        in_bytes < ((int64_t)1 << 31) && nbr_bytes < ((int64_t)1 << 31)) {
+      launch_resident_kernel<NCB, RG, SS, VEC4, WAVES, C4, true>(m, t, in, in_stride, out, epi, n_in_part, n_out,
+                                                                 accumulate, lds_bytes, per_cu, s);
+      return;
+    }
+  }
+  auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, C4, BUF>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1025,7 +1065,7 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
   const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
   kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
                                                    out, m.wpack.p, epi, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                   accumulate, m.queue.p);
+                                                   accumulate, m.queue.p, (unsigned)in_bytes, (unsigned)nbr_bytes);
   LAUNCH_CHECK();
 }
 
@@ -1175,6 +1215,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   epi.bias = bias;
   m.jobs = CoefJobs();
   m.cur_in_rows = n_in_rows;
+  m.cur_in_base = in;
   if (post) {
     m.postbuf.reserve(2 * (size_t)n_out);
     m.jobs.post = CoefJob{post->mean, post->var, post->gamma, post->beta, post->eps, n_out, n_out, m.postbuf.p,
@@ -1201,6 +1242,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     bn_eval_forward(in, m.bntmp.p, n_in_rows, n_in, n_in, n_in, bn->mean, bn->var, bn->gamma, bn->beta, bn->eps,
                     bn->leak, s);
     src = m.bntmp.p;
+    m.cur_in_base = src;
   }
   if (groups == 1 && conv_mfma_paths<false>(m, t, src, out, w, epi, n_in, n_out, PreArgs(), s)) return;
   if (m.jobs.post.n_pad) {  // no packing launch on this path: fold the coefficients by themselves

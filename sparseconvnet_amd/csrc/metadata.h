@@ -127,7 +127,8 @@ struct Metadata {
   // ones summed, the others as (counts, multiply-adds per rule) until take_macs() fetches them.
   double macs_settled = 0;
   std::vector<std::pair<std::shared_ptr<Counts>, double>> pending_macs;
-  int64_t cur_in_rows = 0;  // rows of the input matrix of the convolution being launched
+  int64_t cur_in_rows = 0;  // rows and start of the input matrix of the convolution being launched
+  const float *cur_in_base = nullptr;
   CoefJobs jobs;          // coefficient arrays the next weight-packing launch has to fill
   DevBuf<float> postbuf;  // scale / shift of a batch norm fused into the running convolution's stores
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
