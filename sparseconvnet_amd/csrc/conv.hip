@@ -166,13 +166,14 @@ __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows
 // load of the pipeline is unconditional (granules without the tap and absent rows read
 // row 0 and are zeroed by a select), so the count of loads in flight is a compile-time
 // constant and the compiler can wait for exactly the loads it needs.
-template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE>
+template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF>
 __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
-    const float *__restrict__ pre_sh, float pre_leak) {
+    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
+  static_assert(!BUF || (VEC4 && !PRE), "buffer gathers: float4 rows, no pre-activation");
   constexpr int WR = 4 / WC;
   constexpr int NCB = NCBW * WC;
   constexpr int G = GW * WR;
@@ -246,6 +247,11 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 
   // Issue the loads of iteration `it`: its weight slab into wreg; this wavefront's share of
   // the A fragments (granule, step) into areg.
+  // BUF: gathers through buffer loads; an absent row becomes an offset of 2 GiB, which is past
+  // the end and reads as zeros (see k_conv_rows).
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
+  const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
   auto issue = [&](int it) {
     const int ti = it / n_slab, sl = it - ti * n_slab;
     const int k = taplist[ti];
@@ -261,6 +267,11 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       const int f = wave + 4 * i;  // fragment f = (granule f / SS, step f % SS)
       const int gr = f / SS, s = f % SS;
       const int j = jtab[(gr * K + k) * 16 + r16];
+      if constexpr (BUF) {
+        const unsigned voff = j >= 0 ? __umul24((unsigned)j, row_bytes) + lane_off : 0x80000000u;
+        areg[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, (sl * SS + s) * 64, 0));
+        continue;
+      }
       if (j >= 0) aok_nxt |= 1u << i;
       const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
       const int c0 = (sl * SS + s) * 16 + 4 * g;
@@ -295,7 +306,8 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       const int c0 = (sl_nxt * SS + f % SS) * 16 + 4 * g;
       const bool ok = (aok_nxt >> i) & 1u;
       v4f v = pre_act<PRE>(areg[i], psc[i], psh[i], pre_leak);
-      if (VEC4) {
+      if (BUF) {
+      } else if (VEC4) {
         if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
       } else {
         if (!(ok && c0 + 0 < n_in)) v.x = 0.f;
@@ -401,9 +413,14 @@ struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
   float leak = 1.0f;
 };
 
-template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE>
+template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF = false>
 static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+  if constexpr (VEC4 && !PRE && !BUF) {
+    if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
+        m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24))
+      return launch_mfma<NCBW, WC, GW, SS, VEC4, PRE, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+  }
   constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
   constexpr int WPT = (SS * NCB * 64 + 255) / 256;
   constexpr int SLAB_STRIDE = WPT * 256 * 4;  // floats
@@ -417,7 +434,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE, take_jobs(m));
   LAUNCH_CHECK();
-  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE>;
+  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE, BUF>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -437,7 +454,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   }
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), 256, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak);
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
   if (n_split > 1) {
     k_conv_reduce<<<dim3((unsigned)ceil_div(t.n * n_out, 256)), 256, 0, s>>>(partial, n_split, split_stride, NCB * 16,
