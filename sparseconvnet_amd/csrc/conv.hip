@@ -502,7 +502,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
-  static_assert(!BUF || (VEC4 && !PRE), "buffer gathers: float4 rows, no pre-activation");
+  static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   constexpr int NT = NW * 64;
   constexpr int G = NW * RG;
   constexpr int TM = G * 16;
@@ -597,6 +597,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
         // and fewer than 2^24 rows), so no select is needed afterwards and the address is
         // one 24-bit multiply-add.
         const unsigned voff = j >= 0 ? __umul24((unsigned)j, row_bytes) + lane_off : 0x80000000u;
+        if (PRE && j >= 0) ok_nxt |= 1u << q;  // zero must stay zero through the pre-activation
 #pragma unroll
         for (int s = 0; s < SS; s++)
           a_nxt[q][s] = __builtin_bit_cast(
@@ -631,8 +632,13 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
       const bool ok = (ok_nxt >> q) & 1u;
 #pragma unroll
       for (int s = 0; s < SS; s++) {
-        if constexpr (BUF) {
+        if constexpr (BUF && !PRE) {
           a_cur[q][s] = a_nxt[q][s];
+          continue;
+        }
+        if constexpr (BUF && PRE) {
+          const v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
+          a_cur[q][s] = ok ? v : (v4f){0.f, 0.f, 0.f, 0.f};
           continue;
         }
         const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
@@ -715,7 +721,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF = false>
 static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
-  if constexpr (VEC4 && !PRE && !BUF) {
+  if constexpr (VEC4 && !BUF) {
     // gathers through buffer loads (no per-element selects, 32-bit addressing) when the input
     // is below 2 GiB and 2^24 rows and consists of whole slabs
     if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
