@@ -569,9 +569,14 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
   const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
-  auto issue = [&](int it) {
-    const int ti = it / n_slab, sl = it - ti * n_slab;
-    const int k = taplist[ti];
+  int nx_ti = 0, nx_sl = 0;  // (tap index, slab) of the next iteration to issue; issue() runs in sequence
+  auto issue = [&](int) {
+    const int sl = nx_sl;
+    const int k = taplist[nx_ti];
+    if (++nx_sl == n_slab) {
+      nx_sl = 0;
+      nx_ti++;
+    }
     gm_nxt = gmask[k];
     sl_nxt = sl;
     ok_nxt = 0;
