@@ -179,3 +179,41 @@ def test_multiply_add_counter_matches_oracle(oracle_built):
     gc.collect()
     assert scn.forward_pass_multiplyAdd_count == want
     assert scn.forward_pass_hidden_states > 0
+
+
+def test_unet_scene_scale_invariants():
+    """The ScanNet-style U-Net (m = 32, 7 levels, mode-4 input with duplicated points) on a
+    250,000-point scene, where the oracle is too slow: the result does not depend on the order
+    of the input points (rows follow their points), is bit-identical between a cold pass and a
+    pass over cached rulebooks, and the fused and unfused batch norms agree."""
+    torch.manual_seed(21)
+    m = 32
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m, 5 * m, 6 * m, 7 * m], False)).add(scn.BatchNormReLU(m)).add(
+        scn.OutputLayer(3)).cuda().eval()
+    randomise_bn(model, 21)
+    coords = synthetic.room_scene(seed=2100, target=200000, spatial=4096, duplicate_fraction=0.3)
+    rng = np.random.default_rng(21)
+    feats = rng.uniform(-1, 1, size=(len(coords), 3)).astype(np.float32)
+    layer = scn.InputLayer(3, 4096, mode=4)
+
+    def run(c, f, twice=False):
+        with torch.no_grad():
+            x = layer([torch.as_tensor(c).cuda(), torch.as_tensor(f).cuda()])
+            y = model(x)
+            if twice:
+                return y.cpu().numpy(), model(x).cpu().numpy()
+            return y.cpu().numpy()
+    cold, warm = run(coords, feats, twice=True)
+    assert cold.shape == (len(coords), m) and np.isfinite(cold).all() and np.abs(cold).max() > 0
+    assert (cold == warm).all()
+    perm = rng.permutation(len(coords))
+    shuffled = run(coords[perm], feats[perm])
+    # summation orders inside duplicate groups and pattern-sorted tiles may differ: tolerance, not bits
+    checks.assert_close(shuffled, cold[perm], "permuted input points")
+    scn.fuse_batchnorm = False
+    try:
+        unfused = run(coords, feats)
+    finally:
+        scn.fuse_batchnorm = True
+    checks.assert_close(cold, unfused, "fused vs unfused U-Net")
