@@ -254,8 +254,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
   auto issue = [&](int it) {
     const int ti = it / n_slab, sl = it - ti * n_slab;
-    const int k = taplist[ti];
-    const unsigned gm = gmask[k];
+    // LDS values every lane reads alike: tell the compiler, so that what follows from them
+    // (weight address, branches on the granule mask) is scalar work
+    const int k = __builtin_amdgcn_readfirstlane(taplist[ti]);
+    const unsigned gm = __builtin_amdgcn_readfirstlane(gmask[k]);
     gm_nxt = gm;
     sl_nxt = sl;
     aok_nxt = 0;
@@ -572,12 +574,14 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   int nx_ti = 0, nx_sl = 0;  // (tap index, slab) of the next iteration to issue; issue() runs in sequence
   auto issue = [&](int) {
     const int sl = nx_sl;
-    const int k = taplist[nx_ti];
+    // LDS values every lane reads alike: tell the compiler, so that what follows from them
+    // (weight address, branches on the granule mask) is scalar work
+    const int k = __builtin_amdgcn_readfirstlane(taplist[nx_ti]);
     if (++nx_sl == n_slab) {
       nx_sl = 0;
       nx_ti++;
     }
-    gm_nxt = gmask[k];
+    gm_nxt = __builtin_amdgcn_readfirstlane(gmask[k]);
     sl_nxt = sl;
     ok_nxt = 0;
     if (PRE) {

@@ -118,7 +118,6 @@ struct Metadata {
   DevBuf<unsigned char> tmp;
   DevBuf<unsigned long long> k0, k1;
   DevBuf<int> v0, v1, f0, f1, s0, s1;
-  DevBuf<long long> dcounts;
   DevBuf<int> dflags;
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
