@@ -5,11 +5,17 @@
 // (CPU/Convolution.cpp:45-79,117-150, CPU/Deconvolution.cpp:7-41); they differ only in
 // the table they pass.
 //
-// MFMA kernel (groups == 1): fp32 v_mfma_f32_16x16x4_f32, accumulators in registers for the
-// whole filter, gathered rows and packed weights staged through double-buffered LDS, taps
-// skipped per 16-row granule.  Positions arrive in Z-order and pattern-sorted, so a
-// granule's rows mostly share one neighbour pattern and the skipped (granule, tap) pairs
-// carry almost all of the sparsity.
+// Three MFMA kernels (groups == 1, fp32 v_mfma_f32_16x16x4_f32, accumulators in registers
+// for the whole filter, taps skipped per 16-row granule), chosen by the output width:
+//   k_conv_resident  nOut <= 32   all taps' weights resident in LDS, wavefronts run alone
+//   k_conv_rows      nOut <= 128  wavefronts own rows, the weight slab goes through LDS
+//   k_conv_mfma      wider        wavefronts own columns, rows and weights go through LDS
+// and k_conv_generic for everything else (groups > 1).  Positions arrive in Z-order and
+// pattern-sorted, so a granule's rows mostly share one neighbour pattern and the skipped
+// (granule, tap) pairs carry almost all of the sparsity.  Template flag BUF: the gathers are
+// buffer loads, for which an absent row is an offset past the end that reads as zeros;
+// without it absent rows read row 0 and are zeroed by a select.  PRE / Epi: the batch norm +
+// leaky ReLU of the layer in front / behind, applied to the gathered / stored values.
 #include "metadata.h"
 
 #include <type_traits>
