@@ -129,6 +129,117 @@ def unet_scene(sites, seed, reps=3):
             "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1)}
 
 
+def other_ops(sites, seed):
+    """The rest of the path on the same kind of scene, each op by itself with inputs resident
+    in HBM: ms (median of 5, HIP events on the launch stream) and the algorithmic bytes it has
+    to move, against the 8 TB/s of HBM.  Rulebook builds are timed from the host (they
+    synchronise)."""
+    import torch
+    import sparseconvnet_amd as scn
+    from sparseconvnet_amd import metadata as M
+    from sparseconvnet_amd import synthetic
+
+    def timed(fn, reps=5):
+        fn()
+        ms = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        return float(np.median(ms))
+
+    def host_timed(fn, reps=4):
+        ms = []
+        for _ in range(reps + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            keep = fn()
+            torch.cuda.synchronize()
+            ms.append((time.perf_counter() - t0) * 1e3)
+            del keep
+        return float(np.median(ms[1:]))
+
+    def row(name, ms, byts, **extra):
+        d = {"op": name, "ms": round(ms, 4), "algorithmic_MB": round(byts / 1e6, 1),
+             "GB_per_s": round(byts / (ms * 1e-3) / 1e9, 1), "frac_hbm": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        d.update(extra)
+        return d
+
+    coords = synthetic.room_scene(seed=seed, target=sites, spatial=4096, duplicate_fraction=0.3)
+    npts = len(coords)
+    cd = torch.as_tensor(coords).cuda()
+    g = torch.Generator(device="cuda").manual_seed(2)
+    feats = torch.rand((npts, 3), device="cuda", generator=g)
+    sz, half = torch.LongTensor([4096] * 3), torch.LongTensor([2048] * 3)
+    two = torch.LongTensor([2] * 3)
+    out = []
+
+    def input_layer():
+        md = M.Metadata(3)
+        md.inputLayer(sz, cd, feats, 0, 4)
+        return md
+    ms = host_timed(input_layer)
+    md = M.Metadata(3)
+    x3 = md.inputLayer(sz, cd, feats, 0, 4)
+    n = x3.shape[0]
+    # coordinates read (4 int64 per point), level written (4 int32 + key per site), rules (2 int32 per point)
+    out.append(row("InputLayer mode 4: rules + level (%d points -> %d sites)" % (npts, n), ms,
+                   npts * 32 + n * 24 + npts * 8, points_per_s=round(npts / (ms * 1e-3))))
+    L, stream = md._L, C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    y3 = torch.empty((n, 3), device="cuda")
+    ms = timed(lambda: M._lib.check(L.scn_input_layer_fwd(md._h, M._ptr(feats), M._ptr(y3), 3, stream)))
+    out.append(row("InputLayer forward (mean of duplicates), 3 planes", ms, npts * 12 + npts * 4 + n * 12 + n * 8))
+    x32 = torch.randn((n, 32), device="cuda", generator=g)
+    x64 = torch.randn((n, 64), device="cuda", generator=g)
+    ms = timed(lambda: md.outputLayer(x32))
+    out.append(row("OutputLayer forward, 32 planes", ms, npts * 4 + npts * 128 + n * 128))
+    mean, var = torch.zeros(64, device="cuda"), torch.ones(64, device="cuda")
+    ms = timed(lambda: M.batchNormEval(x64, mean, var, None, None, 1e-4, 0.0))
+    out.append(row("BatchNormReLU eval (stand-alone pass), 64 planes", ms, 2 * n * 64 * 4))
+
+    def strided():
+        m2 = M.Metadata(3)
+        m2.inputLayer(sz, cd, feats, 0, 4)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        M._lib.check(L.scn_md_strided_rules(m2._h, m2._s(sz), m2._s(half), m2._s(two), m2._s(two), stream))
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3, m2
+    t = []
+    for _ in range(4):
+        dt, m2 = strided()
+        t.append(dt)
+        del m2
+    ms = float(np.median(t[1:]))
+    w_dn = torch.randn((8, 1, 32, 64), device="cuda", generator=g) * 0.1
+    w_up = torch.randn((8, 1, 64, 32), device="cuda", generator=g) * 0.1
+    yc, _ = md.convolution(sz, half, two, two, x32, w_dn, None)
+    nc = yc.shape[0]
+    # input keys read, output level written, both rule tables written (8 taps)
+    out.append(row("strided rulebook 2^3 / stride 2 + output level (%d -> %d sites)" % (n, nc), ms,
+                   n * 8 + nc * 24 + 8 * 4 * (n + nc) + 8 * n, sites_per_s=round(n / (ms * 1e-3))))
+    ms = timed(lambda: md.convolution(sz, half, two, two, x32, w_dn, None, want_macs=False))
+    out.append(row("Convolution 2^3 / stride 2, 32 -> 64", ms, n * 32 * 4 + 8 * n + nc * 64 * 4 + 8 * 32 * 64 * 4,
+                   gflops=round(2.0 * n * 32 * 64 / (ms * 1e-3) / 1e9, 1)))
+    ms = timed(lambda: md.deconvolution(half, sz, two, two, yc, w_up, None, want_macs=False))
+    out.append(row("Deconvolution 2^3 / stride 2, 64 -> 32", ms, nc * 64 * 4 + 8 * n + n * 32 * 4 + 8 * 64 * 32 * 4,
+                   gflops=round(2.0 * n * 64 * 32 / (ms * 1e-3) / 1e9, 1)))
+    ms = timed(lambda: md.maxPooling(sz, half, two, two, x32, 0))
+    out.append(row("MaxPooling 2^3 / stride 2, 32 planes", ms, n * 32 * 4 + 8 * n + nc * 32 * 4))
+    # sparse to dense on a grid that can be dense: the same scene generator at 128^3, 16 planes
+    c2 = synthetic.room_scene(seed=seed + 1, target=200000, spatial=128)
+    md2 = M.Metadata(3)
+    s128 = torch.LongTensor([128] * 3)
+    f2 = torch.randn((len(c2), 16), device="cuda", generator=g)
+    xs = md2.inputLayer(s128, torch.as_tensor(c2).cuda(), f2, 0, 3)
+    ms = timed(lambda: md2.sparseToDense(s128, xs, 16))
+    out.append(row("SparseToDense 128^3, 16 planes (%d sites)" % xs.shape[0], ms, xs.shape[0] * 16 * 4 + 128 ** 3 * 16 * 4))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,6 +252,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pairs", default="")
     ap.add_argument("--no-unet", action="store_true")
+    ap.add_argument("--no-ops", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times, to scale profiler byte counters")
     ap.add_argument("--unet-sites", type=int, default=1000000)
@@ -252,6 +364,8 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
+    if not args.no_ops:
+        out["other_ops"] = other_ops(args.unet_sites, 5000)
     if not args.no_unet:
         out["unet"] = unet_scene(args.unet_sites, 5000)
     if not args.no_cpu:

@@ -1150,9 +1150,14 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
 // channels so that every part's weights fit in LDS; parts after the first accumulate.
 // The resident kernel serves nOut <= 32 with up to 32 taps.  It takes the input channels in
 // parts of 32 and has no fused batch norm, so from 128 input channels on, or from 64 when a
-// batch norm comes with the call, the row-owner kernel is at least as fast (measured).
+// batch norm comes with the call or the filter has few taps, the row-owner kernel is at
+// least as fast (measured).
 static bool resident_fits(const Table &t, int n_in, int n_out, bool with_bn) {
-  return t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr && n_in < (with_bn ? 64 : 128);
+  if (!(t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr)) return false;
+  // several parts re-read and re-write the output once per part: with few taps (strided and
+  // transposed convolutions) that costs more than the convolution itself
+  if (n_in > 32 && t.K <= 8) return false;
+  return n_in < (with_bn ? 64 : 128);
 }
 
 // No fused batch norm here: this kernel's time goes into the vector instructions around its

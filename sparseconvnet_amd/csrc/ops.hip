@@ -14,15 +14,23 @@ template <int V>
 __global__ void k_bn_eval(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
                           int64_t out_stride, const float *mean, const float *var, const float *gamma,
                           const float *beta, float eps, float leak) {
+  // scale / shift of every plane once per workgroup (LDS), then a pure streaming pass:
   // thread -> (row, group of V planes); consecutive threads cover one row, then the next
-  int groups = planes / V;
+  extern __shared__ float coef[];  // [planes] scale | [planes] shift
+  for (int c = threadIdx.x; c < planes; c += blockDim.x) {
+    const float w = (1.0f / sqrtf(var[c] + eps)) * (gamma ? gamma[c] : 1.0f);
+    coef[c] = w;
+    coef[planes + c] = -mean[c] * w + (beta ? beta[c] : 0.0f);
+  }
+  __syncthreads();
+  const int groups = planes / V;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = rows * groups;
-  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  const int64_t total = rows * groups;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
   for (; i < total; i += step) {
-    int64_t r = i / groups;
-    int p0 = (int)(i - r * groups) * V;
-    float x[V], w[V], b[V];
+    const int64_t r = i / groups;
+    const int p0 = (int)(i - r * groups) * V;
+    float x[V];
     if (V == 4) {
       float4 t = *reinterpret_cast<const float4 *>(in + r * in_stride + p0);
       x[0] = t.x, x[1] = t.y, x[2] = t.z, x[3] = t.w;
@@ -30,10 +38,7 @@ __global__ void k_bn_eval(const float *in, float *out, int64_t rows, int planes,
       for (int v = 0; v < V; v++) x[v] = in[r * in_stride + p0 + v];
     }
     for (int v = 0; v < V; v++) {
-      float inv = 1.0f / sqrtf(var[p0 + v] + eps);
-      w[v] = inv * (gamma ? gamma[p0 + v] : 1.0f);
-      b[v] = -mean[p0 + v] * w[v] + (beta ? beta[p0 + v] : 0.0f);
-      float y = x[v] * w[v] + b[v];
+      const float y = x[v] * coef[p0 + v] + coef[planes + p0 + v];
       x[v] = y * (y > 0 ? 1.0f : leak);
     }
     if (V == 4) {
@@ -48,15 +53,16 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
                      int64_t out_stride, const float *mean, const float *var, const float *gamma,
                      const float *beta, float eps, float leak, hipStream_t s) {
   if (rows <= 0 || planes <= 0) return;
+  if (planes > 8192) throw Error("batch norm: more than 8192 planes");
   bool vec = planes % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 &&
              ((uintptr_t)in % 16 == 0) && ((uintptr_t)out % 16 == 0);
   int64_t total = rows * (vec ? planes / 4 : planes);
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   if (vec)
-    k_bn_eval<4><<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, mean,
+    k_bn_eval<4><<<dim3((unsigned)blocks), TB, 2 * planes * sizeof(float), s>>>(in, out, rows, planes, in_stride, out_stride, mean,
                                                        var, gamma, beta, eps, leak);
   else
-    k_bn_eval<1><<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, mean,
+    k_bn_eval<1><<<dim3((unsigned)blocks), TB, 2 * planes * sizeof(float), s>>>(in, out, rows, planes, in_stride, out_stride, mean,
                                                        var, gamma, beta, eps, leak);
   LAUNCH_CHECK();
 }
@@ -64,33 +70,54 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
 // ---- max pooling ------------------------------------------------------------------------
 // CPU/MaxPooling.cpp:7-20,50: the output starts at zero and takes every input of its window
 // that compares greater, so the result is max(0, active inputs); output-stationary here.
+template <int V>
 __global__ void k_maxpool(const int *nbr, const int *rowmap, int K, int64_t n_out, int64_t npad,
                           const float *in, int in_stride, float *out, int planes) {
+  // thread -> (output position, group of V planes)
+  const int groups = planes / V;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = n_out * planes;
-  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  const int64_t total = n_out * groups;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
   for (; i < total; i += step) {
-    int64_t o = i / planes;
-    int p = (int)(i - o * planes);
-    float acc = 0.0f;
+    const int64_t o = i / groups;
+    const int p = (int)(i - o * groups) * V;
+    float acc[V];
+    for (int v = 0; v < V; v++) acc[v] = 0.0f;
     for (int k = 0; k < K; k++) {
-      int j = nbr[(int64_t)k * npad + o];
+      const int j = nbr[(int64_t)k * npad + o];
       if (j >= 0) {
-        float v = in[(int64_t)j * in_stride + p];
-        if (acc < v) acc = v;
+        const float *src = in + (int64_t)j * in_stride + p;
+        if (V == 4) {
+          const float4 t = *reinterpret_cast<const float4 *>(src);
+          acc[0] = acc[0] < t.x ? t.x : acc[0];
+          acc[1] = acc[1] < t.y ? t.y : acc[1];
+          acc[2] = acc[2] < t.z ? t.z : acc[2];
+          acc[3] = acc[3] < t.w ? t.w : acc[3];
+        } else {
+          for (int v = 0; v < V; v++) acc[v] = acc[v] < src[v] ? src[v] : acc[v];
+        }
       }
     }
-    int64_t row = rowmap ? rowmap[o] : o;
-    out[row * planes + p] = acc;
+    const int64_t row = rowmap ? rowmap[o] : o;
+    if (V == 4)
+      *reinterpret_cast<float4 *>(out + row * planes + p) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    else
+      for (int v = 0; v < V; v++) out[row * planes + p + v] = acc[v];
   }
 }
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
                      hipStream_t s) {
   if (t.n == 0 || planes <= 0) return;
-  int64_t total = t.n * planes;
+  const bool vec = planes % 4 == 0 && in_stride % 4 == 0 && drop % 4 == 0 && ((uintptr_t)in % 16 == 0) &&
+                   ((uintptr_t)out % 16 == 0);
+  int64_t total = t.n * (vec ? planes / 4 : planes);
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
-  k_maxpool<<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
-                                                  in_stride, out, planes);
+  if (vec)
+    k_maxpool<4><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+                                                       in_stride, out, planes);
+  else
+    k_maxpool<1><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+                                                       in_stride, out, planes);
   LAUNCH_CHECK();
 }
 
