@@ -88,18 +88,21 @@ def cpu_baseline(sample_sites, seed):
                       % (len(coords), R, t_rules)}
 
 
-def unet_scene(sites, seed, reps=3):
+def unet_scene(sites, seed, reps=3, residual=False):
     """3D U-Net forward of examples/ScanNet/unet.py:25-38 with m=32, block_reps=2 (7 levels,
     [32..224] planes), InputLayer mode 4 on a room scene with ~30% duplicated points, eval,
     random-init weights, batch 1.  cold = new Metadata per scene, as a user runs it (input layer,
-    every rulebook and all layers); warm = the same scene again with its rulebooks cached."""
+    every rulebook and all layers); warm = the same scene again with its rulebooks cached.
+    residual: the builder's ResNet-style blocks (networkArchitectures.py:222-230) instead of
+    the VGG-style ones the example uses."""
     import torch
     import sparseconvnet_amd as scn
     from sparseconvnet_amd import synthetic
     m = 32
     torch.manual_seed(0)
     model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
-        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m, 5 * m, 6 * m, 7 * m], False)).add(scn.OutputLayer(3)).cuda().eval()
+        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m, 5 * m, 6 * m, 7 * m], residual)).add(
+        scn.OutputLayer(3)).cuda().eval()
     linear = torch.nn.Linear(m, 20).cuda()
     coords = synthetic.room_scene(seed=seed, target=sites, spatial=4096, duplicate_fraction=0.3)
     g = torch.Generator(device="cuda").manual_seed(1)
@@ -123,6 +126,10 @@ def unet_scene(sites, seed, reps=3):
                 cold.append((t1 - t0) * 1e3)
                 warm.append((t2 - t1) * 1e3)
             macs = scn.forward_pass_multiplyAdd_count / 2
+    if residual:
+        return {"unet_residual_ms_per_scene": round(float(np.median(cold)), 3),
+                "unet_residual_warm_ms": round(float(np.median(warm)), 3),
+                "unet_residual_gflop": round(2 * macs / 1e9, 2)}
     return {"unet_ms_per_scene": round(float(np.median(cold)), 3), "unet_warm_ms": round(float(np.median(warm)), 3),
             "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
             "unet_gflop": round(2 * macs / 1e9, 2),
@@ -226,6 +233,10 @@ def other_ops(sites, seed):
                    gflops=round(2.0 * n * 32 * 64 / (ms * 1e-3) / 1e9, 1)))
     ms = timed(lambda: md.deconvolution(half, sz, two, two, yc, w_up, None, want_macs=False))
     out.append(row("Deconvolution 2^3 / stride 2, 64 -> 32", ms, nc * 64 * 4 + 8 * n + n * 32 * 4 + 8 * 64 * 32 * 4,
+                   gflops=round(2.0 * n * 64 * 32 / (ms * 1e-3) / 1e9, 1)))
+    w_nin = torch.randn((64, 32), device="cuda", generator=g) * 0.1
+    ms = timed(lambda: md.networkInNetwork(x64, w_nin, None, want_macs=False))
+    out.append(row("NetworkInNetwork 64 -> 32", ms, n * 64 * 4 + n * 32 * 4 + 64 * 32 * 4,
                    gflops=round(2.0 * n * 64 * 32 / (ms * 1e-3) / 1e9, 1)))
     ms = timed(lambda: md.maxPooling(sz, half, two, two, x32, 0))
     out.append(row("MaxPooling 2^3 / stride 2, 32 planes", ms, n * 32 * 4 + 8 * n + nc * 32 * 4))
@@ -368,6 +379,7 @@ def main():
         out["other_ops"] = other_ops(args.unet_sites, 5000)
     if not args.no_unet:
         out["unet"] = unet_scene(args.unet_sites, 5000)
+        out["unet"].update(unet_scene(args.unet_sites, 5000, residual=True))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sites, args.seed)
     print(json.dumps(out))

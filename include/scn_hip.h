@@ -156,6 +156,15 @@ int scn_conv_bn_fwd(scn_metadata *md, int kind, const int64_t *a, const int64_t 
                     const float *weight, const float *bias, int n_in, int n_out, int groups,
                     const scn_bn_params *pre, const scn_bn_params *post, void *stream,
                     double *macs);
+/* NetworkInNetwork_updateOutput (pybind.cpp:225, sparseconvnet.h:51-54, CPU/NetworkInNetwork.cpp:7-23):
+ * out [rows, n_out] = bias + in [rows, n_in] * weight [n_in, n_out]; a convolution with one
+ * tap.  The reference call takes no metadata; here the handle of the tensor's metadata owns
+ * the scratch the kernels use (packed weights, the one-tap table for this row count), which
+ * the caller has at hand (SparseConvNetTensor.metadata).  macs as for the convolutions
+ * (rows * n_in * n_out). */
+int scn_nin_fwd(scn_metadata *md, const float *in, float *out, const float *weight,
+                const float *bias, int64_t rows, int n_in, int n_out, void *stream,
+                double *macs);
 /* MaxPooling_updateOutput (pybind.cpp:103-107, CPU/MaxPooling.cpp:37-60).
  * in [nActive(in_size), in_stride] -> out [nActive(out_size), planes] where
  * planes = in_stride - n_features_to_drop; the result is max(0, inputs of the window). */

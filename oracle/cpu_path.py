@@ -56,6 +56,7 @@ def _load(flavour):
                                 _f32p, C.c_int, C.c_int, C.c_int]),
         "maxpool": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p,
                            C.c_int, C.c_int]),
+        "nin": (C.c_double, [_f32p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]),
         "bn_eval": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p, _f32p,
                            _f32p, C.c_float, C.c_float]),
         "input_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
@@ -197,6 +198,13 @@ class CpuPath:
         self.f["maxpool"](self.h, *[_p64(s) for s in sizes], _pf(x), x.shape[1], _pf(out), planes,
                           n_features_to_drop)
         return out
+
+    def nin(self, x, w, bias=None):
+        """NetworkInNetwork: returns (bias + x @ w, multiply-adds)."""
+        x, w, bias = _f32(x), _f32(w), _f32(bias)
+        out = np.zeros((x.shape[0], w.shape[1]), np.float32)
+        macs = self.f["nin"](_pf(x), _pf(out), _pf(w), _pf(bias), x.shape[0], w.shape[0], w.shape[1])
+        return out, macs
 
     def bn_eval(self, x, mean, var, weight=None, bias=None, eps=1e-4, leakiness=1.0):
         x = _f32(x)

@@ -25,6 +25,7 @@ template class Metadata<4>;
 #include "CPU/Deconvolution.cpp"
 #include "CPU/IOLayers.cpp"
 #include "CPU/MaxPooling.cpp"
+#include "CPU/NetworkInNetwork.cpp"
 #include "CPU/SparseToDense.cpp"
 
 #include <cstring>
@@ -183,6 +184,16 @@ void ref_maxpool(void *h, const int64_t *inSz, const int64_t *outSz, const int64
            (void)nPlanes;
            cpu_MaxPooling_updateOutput<float, D>(IS, OS, F, St, m, I, O, nFeaturesToDrop);
            copy_out(O, out));
+}
+double ref_nin(const float *in, float *out, const float *w, const float *bias, int nActive, int nIn,
+               int nOut) {
+  auto I = ft(in, {nActive, nIn});
+  auto O = torch::empty({0}, at::kFloat);
+  auto W = ft(w, {nIn, nOut});
+  auto B = ft(bias, {nOut});
+  double macs = cpu_NetworkInNetwork_updateOutput<float>(I, O, W, B);
+  copy_out(O, out);
+  return macs;
 }
 void ref_bn_eval(const float *in, float *out, int nActive, int nPlanes, int inStride,
                  int outStride, const float *runningMean, const float *runningVar,

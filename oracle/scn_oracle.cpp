@@ -583,6 +583,23 @@ void orc_maxpool(void *md, const int64_t *inSz, const int64_t *outSz, const int6
     }
   }
 }
+// CPU/NetworkInNetwork.cpp:7-23: out = bias (or 0), then out += in * weight
+// (weight [nIn, nOut] row-major); returns nActive * nIn * nOut.
+double orc_nin(const float *in, float *out, const float *weight, const float *bias, int nActive,
+               int nIn, int nOut) {
+#pragma omp parallel for
+  for (int row = 0; row < nActive; row++) {
+    float *o = out + (size_t)row * nOut;
+    for (int q = 0; q < nOut; q++) o[q] = bias ? bias[q] : 0.f;
+    const float *i = in + (size_t)row * nIn;
+    for (int p = 0; p < nIn; p++) {
+      const float v = i[p];
+      const float *w = weight + (size_t)p * nOut;
+      for (int q = 0; q < nOut; q++) o[q] += v * w[q];
+    }
+  }
+  return (double)nActive * nIn * nOut;
+}
 // CPU/BatchNormalization.cpp:41-61 (eval branch) and :109-130.
 void orc_bn_eval(const float *in, float *out, int nActive, int nPlanes, int inStride,
                  int outStride, const float *runningMean, const float *runningVar,

@@ -15,7 +15,7 @@ fuse_batchnorm = True
 
 from .containers import AddTable, ConcatTable, JoinTable, Sequential  # noqa: E402
 from .layers import (BatchNormalization, BatchNormLeakyReLU, BatchNormReLU, Convolution,  # noqa: E402
-                     Deconvolution, Identity, InputLayer, MaxPooling, OutputLayer, SparseToDense,
+                     Deconvolution, Identity, InputLayer, MaxPooling, NetworkInNetwork, OutputLayer, SparseToDense,
                      SubmanifoldConvolution, ValidConvolution)
 from .metadata import Metadata  # noqa: E402
 from .networks import SparseVggNet, UNet  # noqa: E402

@@ -48,6 +48,7 @@ SIGNATURES = {
                                  C.c_int, _vp, C.POINTER(C.c_double)]),
     "scn_conv_bn_fwd": (C.c_int, [_vp, C.c_int, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
                                   C.c_int, C.POINTER(BnParams), C.POINTER(BnParams), _vp, C.POINTER(C.c_double)]),
+    "scn_nin_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, C.c_int, _vp, C.POINTER(C.c_double)]),
     "scn_maxpool_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int,
                                   _vp]),
     "scn_bn_eval_fwd": (C.c_int, [_vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp,

@@ -310,6 +310,17 @@ int scn_conv_bn_fwd(scn_metadata *h, int kind, const int64_t *a, const int64_t *
       throw Error("scn_conv_bn_fwd: kind must be 0 (submanifold), 1 (strided) or 2 (transposed)");
   });
 }
+int scn_nin_fwd(scn_metadata *h, const float *in, float *out, const float *weight, const float *bias,
+                int64_t rows, int n_in, int n_out, void *stream, double *macs) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (rows < 0 || rows >= ((int64_t)1 << 31)) throw Error("network in network: row count out of range");
+    Table &t = identity_table(m, rows, st(stream));
+    conv_forward(m, t, in, rows, out, weight, bias, n_in, n_out, 1, nullptr, nullptr, st(stream));
+    // CPU/NetworkInNetwork.cpp:22: nActive * input_nPlanes * output_nPlanes
+    note_macs(m, t, (double)n_in * n_out, macs, st(stream));
+  });
+}
 int scn_maxpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
                     const int64_t *stride, const float *in, int in_stride, float *out, int planes,
                     int n_features_to_drop, void *stream) {

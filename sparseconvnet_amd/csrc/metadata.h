@@ -114,6 +114,7 @@ struct Metadata {
   SizeKey input_size;
   std::map<SizeKey, Table> subm;            // key: spatial || filter
   std::map<SizeKey, StridedRules> strided;  // key: in_size || filter || stride
+  std::map<int64_t, Table> ident;           // key: rows; one tap, row t feeds row t (NetworkInNetwork)
   // scratch reused by the builders
   DevBuf<unsigned char> tmp;
   DevBuf<unsigned long long> k0, k1;
@@ -144,6 +145,8 @@ void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStr
 Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s);
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
                             const int64_t *filter, const int64_t *stride, hipStream_t s);
+// The one-tap table over `rows` rows whose only rule list is the identity.
+Table &identity_table(Metadata &m, int64_t rows, hipStream_t s);
 // Pairs of tap k of a table: (value, row at position t), ordered by t.  Returns the count.
 int64_t export_table_pairs(Metadata &m, Table &t, int k, bool swap, int *pairs, hipStream_t s);
 std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t s);

@@ -1026,6 +1026,37 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   return m.strided.emplace(key, std::move(R)).first->second;
 }
 
+// ---- identity table -----------------------------------------------------------------------
+
+__global__ void k_identity_table(int64_t n, int64_t npad, int *nbr, unsigned *gmask) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < npad) nbr[t] = t < n ? (int)t : -1;
+  if (t < (n + 15) / 16) gmask[t] = 1u;
+}
+
+// A 1x1 convolution (NetworkInNetwork, CPU/NetworkInNetwork.cpp:7-23) is the convolution
+// over this table: one tap, position t reads row t and writes row t.
+Table &identity_table(Metadata &m, int64_t rows, hipStream_t s) {
+  auto it = m.ident.find(rows);
+  if (it != m.ident.end()) return it->second;
+  Table t;
+  t.K = 1;
+  t.n = rows;
+  t.npad = round_up(std::max<int64_t>(rows, 1), 64);
+  t.identity_rows = true;
+  t.cnt = std::make_shared<Counts>();
+  t.cnt->K = 1;
+  t.cnt->host.assign(1, rows);
+  t.cnt->ready = true;
+  if (rows > 0) {
+    t.nbr.reserve(t.npad);
+    t.gmask.reserve(ceil_div(rows, 16));
+    k_identity_table<<<grid_for(t.npad), TB, 0, s>>>(rows, t.npad, t.nbr.p, t.gmask.p);
+    LAUNCH_CHECK();
+  }
+  return m.ident.emplace(rows, std::move(t)).first->second;
+}
+
 // ---- pair-list export (ballot / prefix compaction) --------------------------------------
 
 // Each wavefront counts its hits with a ballot, one lane reserves the range in the block's

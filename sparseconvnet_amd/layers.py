@@ -224,6 +224,40 @@ class Deconvolution(Module):
         return in_size
 
 
+class NetworkInNetwork(Module):
+    """networkInNetwork.py:57-93: a 1x1 convolution, out = bias + in @ weight."""
+
+    def __init__(self, nIn, nOut, bias):
+        Module.__init__(self)
+        self.nIn = nIn
+        self.nOut = nOut
+        std = (2.0 / nIn)**0.5
+        self.weight = Parameter(torch.Tensor(nIn, nOut).normal_(0, std))
+        if bias:
+            self.bias = Parameter(torch.Tensor(nOut).zero_())
+
+    def forward(self, input):
+        assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, \
+            (self.nIn, input.features.shape)
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = input.spatial_size
+        md = input.metadata
+
+        def fn(x, w, b):
+            y, _ = md.networkInNetwork(x, w, b, want_macs=False)
+            _count(y)
+            return y
+        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        return output
+
+    def __repr__(self):
+        return 'NetworkInNetwork' + str(self.nIn) + '->' + str(self.nOut)
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+
 class BatchNormalization(Module):
     """batchNormalization.py:13-71.  leakiness: 0 = ReLU, (0,1) = leaky ReLU, 1 = none.
     Only eval mode is implemented: the running statistics are used as they are."""

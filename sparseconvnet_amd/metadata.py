@@ -178,6 +178,20 @@ class Metadata:
         _lib.check(self._L.scn_md_strided_rules(self._h, *rb, _stream()))
         return self._conv(2, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs)
 
+    def networkInNetwork(self, features, weight, bias, want_macs=True):
+        """out = bias + features @ weight (weight [nIn, nOut]): a convolution with one tap."""
+        features = _features(features, "features")
+        weight = _features(weight, "weight")
+        bias_t = _features(bias, "bias") if bias is not None and bias.numel() else None
+        n_in, n_out = weight.shape
+        assert features.size(0) == 0 or features.size(1) == n_in, (features.shape, weight.shape)
+        out = torch.empty((features.size(0), n_out), dtype=torch.float32, device=features.device)
+        macs = C.c_double(0)
+        _lib.check(self._L.scn_nin_fwd(self._h, _ptr(features), _ptr(out), _ptr(weight), _ptr(bias_t),
+                                       features.size(0), n_in, n_out, _stream(),
+                                       C.byref(macs) if want_macs else None))
+        return out, (macs.value if want_macs else None)
+
     def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
         a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))

@@ -186,6 +186,22 @@ def check_bn(make, seed, n=257, C=13):
             assert_close(y, t.numpy(), "bn leak=%g" % leak)
 
 
+def check_nin(make, seed, shapes=((257, 13, 7), (64, 32, 32), (1, 5, 3), (300, 64, 96), (0, 4, 4))):
+    """NetworkInNetwork against the float64 matrix product of numpy, with and without bias."""
+    rng = np.random.default_rng(seed)
+    p = make(3)
+    for n, cin, cout in shapes:
+        x = rng.normal(size=(n, cin)).astype(np.float32)
+        w = (rng.normal(size=(cin, cout)) * 0.3).astype(np.float32)
+        b = rng.normal(size=cout).astype(np.float32)
+        for bias in (None, b):
+            y, macs = p.nin(x, w, bias)
+            expect = x.astype(np.float64) @ w.astype(np.float64) + (0 if bias is None else bias.astype(np.float64))
+            assert y.shape == (n, cout)
+            assert_close(y, expect, "network in network %s" % ((n, cin, cout),))
+            assert macs == n * cin * cout
+
+
 def check_s2d(make, dim, seed, spatial=6, n=80, batch=3, C=4):
     rng, p, loc, x = _setup(make, dim, spatial, n, batch, seed, C)
     d = p.s2d(spatial, x)

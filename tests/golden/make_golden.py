@@ -103,8 +103,38 @@ def vgg2d(path, make):
                         bn1_var=bn1[1], bn2_mean=bn2[0], bn2_var=bn2[1], dense=dense)
 
 
+def residual_block(path, make):
+    """One residual block of the U-Net builder (networkArchitectures.py:222-230) at 24^3,
+    6 -> 10 planes: NetworkInNetwork(x) + SC(BNReLU(SC(BNReLU(x)))), and a second
+    NetworkInNetwork with bias on the sum."""
+    rng = np.random.default_rng(106)
+    coords = synthetic.config1(seed=6000, batch=2, spatial=24, target=500)
+    feats = rng.normal(size=(len(coords), 6)).astype(np.float32)
+    wn = (rng.normal(size=(6, 10)) * (2.0 / 6) ** 0.5).astype(np.float32)
+    w1 = (rng.normal(size=(27, 1, 6, 10)) * (2.0 / (6 * 27)) ** 0.5).astype(np.float32)
+    w2 = (rng.normal(size=(27, 1, 10, 10)) * (2.0 / (10 * 27)) ** 0.5).astype(np.float32)
+    wn2 = (rng.normal(size=(10, 4)) * (2.0 / 10) ** 0.5).astype(np.float32)
+    bias2 = rng.normal(size=4).astype(np.float32)
+    bn1 = [rng.normal(size=6).astype(np.float32), rng.uniform(0.5, 1.5, 6).astype(np.float32)]
+    bn2 = [rng.normal(size=10).astype(np.float32), rng.uniform(0.5, 1.5, 10).astype(np.float32)]
+    p = make(3)
+    p.input_layer(24, coords, 0, 0)
+    loc = p.spatial_locations(24)
+    skip, macs_nin = p.nin(feats, wn)
+    a = p.bn_eval(feats, bn1[0], bn1[1], None, None, 1e-4, 0.0)
+    a, _ = p.subm_conv(24, 3, a, w1)
+    a = p.bn_eval(a, bn2[0], bn2[1], None, None, 1e-4, 0.0)
+    a, _ = p.subm_conv(24, 3, a, w2)
+    y = skip + a
+    z, _ = p.nin(y, wn2, bias2)
+    np.savez_compressed(path, coords=coords, feats=feats, wn=wn, w1=w1, w2=w2, wn2=wn2, bias2=bias2,
+                        bn1_mean=bn1[0], bn1_var=bn1[1], bn2_mean=bn2[0], bn2_var=bn2[1],
+                        skip=canon_feats(loc, skip), macs_nin=macs_nin, y=canon_feats(loc, y),
+                        z=canon_feats(loc, z))
+
+
 FIXTURES = {"single_layer_32.npz": single_layer, "strided_tree_62.npz": strided_tree,
-            "vgg2d_31.npz": vgg2d}
+            "vgg2d_31.npz": vgg2d, "residual_block_24.npz": residual_block}
 
 if __name__ == "__main__":
     ref = lambda dim: CpuPath(dim, "ref")  # noqa: E731

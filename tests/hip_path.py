@@ -140,6 +140,15 @@ class HipPath:
         _lib.check(self.L.scn_md_strided_rules(self.h, *rb, _stream()))
         return self._conv(2, sizes, self.nactive(out_size), x, w, bias, bn, post)
 
+    def nin(self, x, w, bias=None):
+        xd, wd = _dev(x, torch.float32), _dev(w, torch.float32)
+        bd = _dev(bias, torch.float32) if bias is not None else None
+        out = torch.full((x.shape[0], w.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        macs = C.c_double(0)
+        _lib.check(self.L.scn_nin_fwd(self.h, _ptr(xd), _ptr(out), _ptr(wd), _ptr(bd), x.shape[0], w.shape[0],
+                                      w.shape[1], _stream(), C.byref(macs)))
+        return out.cpu().numpy(), macs.value
+
     def maxpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
         sizes = [self._s(v) for v in (in_size, out_size, size, stride)]
         _lib.check(self.L.scn_md_strided_rules(self.h, *sizes, _stream()))

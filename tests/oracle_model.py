@@ -42,6 +42,10 @@ def run(module, path, x):
         b = _np(module.bias) if hasattr(module, 'bias') else None
         y, _ = path.deconv(x.spatial, out_sp, fs, st, x.features, _np(module.weight), b)
         return CpuTensor(y, out_sp)
+    if isinstance(module, scn.NetworkInNetwork):
+        b = _np(module.bias) if hasattr(module, 'bias') else None
+        y, _ = path.nin(x.features, _np(module.weight), b)
+        return CpuTensor(y, x.spatial)
     if isinstance(module, scn.MaxPooling):
         ps, st = _np(module.pool_size), _np(module.pool_stride)
         out_sp = (x.spatial - ps) // st + 1

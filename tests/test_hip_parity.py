@@ -50,6 +50,13 @@ def test_bn(make):
     checks.check_bn(make, seed=2, n=1000, C=32)
 
 
+def test_nin(make):
+    checks.check_nin(make, seed=4)
+    # every convolution kernel family: few / many output planes, wide inputs, odd plane counts
+    checks.check_nin(make, seed=5, shapes=((5000, 64, 32), (5000, 32, 64), (3000, 96, 160), (2000, 256, 256),
+                                           (70000, 64, 32), (777, 33, 17), (4000, 3, 32), (1500, 448, 224)))
+
+
 @pytest.mark.parametrize("dim", [1, 2, 3])
 def test_s2d(make, dim):
     checks.check_s2d(make, dim, seed=2 + dim)

@@ -113,8 +113,26 @@ def test_unet_structure_and_state_dict():
     assert tuple(sd['2.1.1.weight'].shape) == (8, 1, 32, 64)      # Convolution 32->64 C2/2
     assert tuple(sd['2.1.4.weight'].shape) == (8, 1, 64, 32)      # Deconvolution 64->32 C2/2
     assert tuple(sd['4.1.weight'].shape) == (27, 1, 64, 32)       # first block after the join
-    with pytest.raises(NotImplementedError):
-        scn.UNet(3, 1, [8, 16], residual_blocks=True)
+
+
+def test_residual_unet_structure():
+    # networkArchitectures.py:222-230: a NetworkInNetwork only where a block changes the plane count
+    u = scn.UNet(3, 2, [8, 16, 24], residual_blocks=True, n_input_planes=5)
+    nins = [x for x in u.modules() if isinstance(x, scn.NetworkInNetwork)]
+    assert sorted((n.nIn, n.nOut) for n in nins) == [(5, 8), (16, 8), (32, 16)]
+    assert all(not hasattr(n, 'bias') and tuple(n.weight.shape) == (n.nIn, n.nOut) for n in nins)
+    adds = [x for x in u.modules() if isinstance(x, scn.AddTable)]
+    convs = [x for x in u.modules() if isinstance(x, scn.SubmanifoldConvolution)]
+    assert len(adds) == 2 * 3 + 2 * 2 and len(convs) == 2 * len(adds)
+    sd = u.state_dict()
+    # block 0: ConcatTable(NetworkInNetwork, Sequential(BN, conv, BN, conv)), then AddTable
+    assert tuple(sd['0.0.weight'].shape) == (5, 8)
+    assert tuple(sd['0.1.1.weight'].shape) == (27, 1, 5, 8) and tuple(sd['0.1.3.weight'].shape) == (27, 1, 8, 8)
+    # block 1 keeps the plane count: Identity has no parameters
+    assert '2.0.weight' not in sd and tuple(sd['2.1.1.weight'].shape) == (27, 1, 8, 8)
+    n = scn.NetworkInNetwork(6, 4, True)
+    assert tuple(n.bias.shape) == (4,) and (n.bias == 0).all()
+    assert abs(scn.NetworkInNetwork(400, 300, False).weight.std().item() - (2.0 / 400) ** 0.5) < 2e-3
 
 
 def test_no_cpu_fallback():

@@ -85,6 +85,24 @@ def test_unet_vs_oracle(oracle_built):
     assert logits.shape == (len(coords), 20)
 
 
+def test_residual_unet_vs_oracle(oracle_built):
+    """The ScanNet example's residual variant at reduced width: blocks of two BN + convolution
+    pairs added to the block input, through a NetworkInNetwork where the plane count changes."""
+    torch.manual_seed(6)
+    m = 8
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m], True)).add(scn.BatchNormReLU(m)).add(scn.OutputLayer(3)).eval()
+    randomise_bn(model, 6)
+    coords = synthetic.scene_batch(seed=5001, batch=2, target=6000, spatial=64, n_boxes=8,
+                                   duplicate_fraction=0.3)
+    rng = np.random.default_rng(6)
+    feats = rng.uniform(-1, 1, size=(len(coords), 3)).astype(np.float32)
+    inp_layer = scn.InputLayer(3, 64, mode=4)
+    got, want, p = _run_both(model, inp_layer, [torch.as_tensor(coords), torch.as_tensor(feats)])
+    assert got.shape == (len(coords), m)
+    checks.assert_close(got.cpu().numpy(), want, "residual U-Net output rows")
+
+
 def test_vgg2d_vs_oracle(oracle_built):
     torch.manual_seed(2)
     model = hello_world_model().eval()

@@ -50,6 +50,10 @@ def test_bn(make):
     checks.check_bn(make, seed=1)
 
 
+def test_nin(make):
+    checks.check_nin(make, seed=4)
+
+
 @pytest.mark.parametrize("dim", [1, 2, 3])
 def test_s2d(make, dim):
     checks.check_s2d(make, dim, seed=2 + dim)
