@@ -171,6 +171,19 @@ int scn_nin_fwd(scn_metadata *md, const float *in, float *out, const float *weig
 int scn_maxpool_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
                     const int64_t *size, const int64_t *stride, const float *in, int in_stride,
                     float *out, int planes, int n_features_to_drop, void *stream);
+/* AveragePooling_updateOutput (pybind.cpp:44-48, sparseconvnet.h:74-78,
+ * CPU/AveragePooling.cpp:38-61): as scn_maxpool_fwd, the result is the sum of the window's
+ * active inputs divided by the filter volume (absent sites count as zeros). */
+int scn_avgpool_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                    const int64_t *size, const int64_t *stride, const float *in, int in_stride,
+                    float *out, int planes, int n_features_to_drop, void *stream);
+/* UnPooling_updateOutput (pybind.cpp:189-193, sparseconvnet.h:230-234, CPU/UnPooling.cpp:34-57):
+ * in [nActive(in_size), in_stride] on the coarse level -> out [nActive(out_size), planes] on
+ * the finer level out_size, which must exist already (as for scn_deconv_fwd): every fine site
+ * receives the sum of the coarse rows whose windows hold it. */
+int scn_unpool_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                   const int64_t *size, const int64_t *stride, const float *in, int in_stride,
+                   float *out, int planes, int n_features_to_drop, void *stream);
 /* BatchNormalization_updateOutput with train=false (pybind.cpp:220,
  * CPU/BatchNormalization.cpp:41-61,109-130): out = leaky(x*w + b), w = gamma/sqrt(var+eps),
  * b = beta - mean*w.  gamma/beta may be NULL.  Row strides in elements. */

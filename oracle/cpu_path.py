@@ -56,6 +56,10 @@ def _load(flavour):
                                 _f32p, C.c_int, C.c_int, C.c_int]),
         "maxpool": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p,
                            C.c_int, C.c_int]),
+        "avgpool": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p,
+                           C.c_int, C.c_int]),
+        "unpool": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p,
+                          C.c_int, C.c_int]),
         "nin": (C.c_double, [_f32p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]),
         "bn_eval": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p, _f32p,
                            _f32p, C.c_float, C.c_float]),
@@ -197,6 +201,26 @@ class CpuPath:
         out = np.zeros((self.nactive(out_size), planes), np.float32)
         self.f["maxpool"](self.h, *[_p64(s) for s in sizes], _pf(x), x.shape[1], _pf(out), planes,
                           n_features_to_drop)
+        return out
+
+    def avgpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
+        x = _f32(x)
+        self.strided_rules(in_size, out_size, size, stride)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, size, stride)]
+        planes = x.shape[1] - n_features_to_drop
+        out = np.zeros((self.nactive(out_size), planes), np.float32)
+        self.f["avgpool"](self.h, *[_p64(s) for s in sizes], _pf(x), x.shape[1], _pf(out), planes,
+                          n_features_to_drop)
+        return out
+
+    def unpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
+        """x lives on the coarse level in_size; the result on the finer level out_size."""
+        x = _f32(x)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, size, stride)]
+        planes = x.shape[1] - n_features_to_drop
+        out = np.zeros((self.nactive(out_size), planes), np.float32)
+        self.f["unpool"](self.h, *[_p64(s) for s in sizes], _pf(x), x.shape[1], _pf(out), planes,
+                         n_features_to_drop)
         return out
 
     def nin(self, x, w, bias=None):

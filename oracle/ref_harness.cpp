@@ -24,7 +24,9 @@ template class Metadata<4>;
 #include "CPU/Convolution.cpp"
 #include "CPU/Deconvolution.cpp"
 #include "CPU/IOLayers.cpp"
+#include "CPU/AveragePooling.cpp"
 #include "CPU/MaxPooling.cpp"
+#include "CPU/UnPooling.cpp"
 #include "CPU/NetworkInNetwork.cpp"
 #include "CPU/SparseToDense.cpp"
 
@@ -183,6 +185,26 @@ void ref_maxpool(void *h, const int64_t *inSz, const int64_t *outSz, const int64
            auto I = ft(in, {n, inStride}); auto O = torch::empty({0}, at::kFloat);
            (void)nPlanes;
            cpu_MaxPooling_updateOutput<float, D>(IS, OS, F, St, m, I, O, nFeaturesToDrop);
+           copy_out(O, out));
+}
+void ref_avgpool(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                 const int64_t *stride, const float *in, int inStride, float *out, int nPlanes,
+                 int nFeaturesToDrop) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(size, D);
+           auto St = lt(stride, D); Int n = m.getNActive(IS);
+           auto I = ft(in, {n, inStride}); auto O = torch::empty({0}, at::kFloat);
+           (void)nPlanes;
+           cpu_AveragePooling_updateOutput<float, D>(IS, OS, F, St, m, I, O, nFeaturesToDrop);
+           copy_out(O, out));
+}
+void ref_unpool(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                const int64_t *stride, const float *in, int inStride, float *out, int nPlanes,
+                int nFeaturesToDrop) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(size, D);
+           auto St = lt(stride, D); Int n = m.getNActive(IS);
+           auto I = ft(in, {n, inStride}); auto O = torch::empty({0}, at::kFloat);
+           (void)nPlanes;
+           cpu_UnPooling_updateOutput<float, D>(IS, OS, F, St, m, I, O, nFeaturesToDrop);
            copy_out(O, out));
 }
 double ref_nin(const float *in, float *out, const float *w, const float *bias, int nActive, int nIn,

@@ -583,6 +583,45 @@ void orc_maxpool(void *md, const int64_t *inSz, const int64_t *outSz, const int6
     }
   }
 }
+// CPU/AveragePooling.cpp:7-20,38-61: out zero-filled, then per rule
+// out[o] += in[i] / filterVolume with filterVolume = number of rule lists.
+void orc_avgpool(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                 const int64_t *stride, const float *in, int inStride, float *out, int nPlanes,
+                 int nFeaturesToDrop) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, inSz, outSz, size, stride);
+  Int nA = m.nActive[mkkey(m.dim, outSz)];
+  std::memset(out, 0, sizeof(float) * (size_t)nA * nPlanes);
+  const float *iF = in + nFeaturesToDrop;
+  const Int filterVolume = (Int)rb.size();
+  for (auto &r : rb) {
+    Int nHot = (Int)(r.size() / 2);
+    for (Int s = 0; s < nHot; s++) {
+      const float *i = iF + (size_t)r[2 * s] * inStride;
+      float *o = out + (size_t)r[2 * s + 1] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += i[p] / filterVolume;
+    }
+  }
+}
+// CPU/UnPooling.cpp:7-20,34-57: the rulebook of (outSz -> inSz), i.e. outSz is the
+// finer level; out zero-filled, then out[rule[0]] += in[rule[1]].
+void orc_unpool(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                const int64_t *stride, const float *in, int inStride, float *out, int nPlanes,
+                int nFeaturesToDrop) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, outSz, inSz, size, stride);
+  Int nA = m.nActive[mkkey(m.dim, outSz)];
+  std::memset(out, 0, sizeof(float) * (size_t)nA * nPlanes);
+  const float *iF = in + nFeaturesToDrop;
+  for (auto &r : rb) {
+    Int nHot = (Int)(r.size() / 2);
+    for (Int s = 0; s < nHot; s++) {
+      const float *i = iF + (size_t)r[2 * s + 1] * inStride;
+      float *o = out + (size_t)r[2 * s] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += i[p];
+    }
+  }
+}
 // CPU/NetworkInNetwork.cpp:7-23: out = bias (or 0), then out += in * weight
 // (weight [nIn, nOut] row-major); returns nActive * nIn * nOut.
 double orc_nin(const float *in, float *out, const float *weight, const float *bias, int nActive,

@@ -51,6 +51,10 @@ SIGNATURES = {
     "scn_nin_fwd": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, C.c_int, _vp, C.POINTER(C.c_double)]),
     "scn_maxpool_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int,
                                   _vp]),
+    "scn_avgpool_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int,
+                                  _vp]),
+    "scn_unpool_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int,
+                                 _vp]),
     "scn_bn_eval_fwd": (C.c_int, [_vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp,
                                   C.c_float, C.c_float, _vp]),
     "scn_s2d_fwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, _vp]),

@@ -331,6 +331,27 @@ int scn_maxpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_
     maxpool_forward(r.by_out, in, in_stride, out, planes, n_features_to_drop, st(stream));
   });
 }
+int scn_avgpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
+                    const int64_t *stride, const float *in, int in_stride, float *out, int planes,
+                    int n_features_to_drop, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
+    StridedRules &r = strided_rules(m, in_size, out_size, size, stride, st(stream));
+    avgpool_forward(r.by_out, in, in_stride, out, planes, n_features_to_drop, st(stream));
+  });
+}
+int scn_unpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
+                   const int64_t *stride, const float *in, int in_stride, float *out, int planes,
+                   int n_features_to_drop, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
+    // CPU/UnPooling.cpp:43-44: the rulebook of (out_size -> in_size), read from the fine side
+    StridedRules &r = strided_rules(m, out_size, in_size, size, stride, st(stream));
+    unpool_forward(r.by_in, in, in_stride, out, planes, n_features_to_drop, st(stream));
+  });
+}
 int scn_bn_eval_fwd(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
                     int64_t out_stride, const float *running_mean, const float *running_var,
                     const float *gamma, const float *beta, float eps, float leakiness, void *stream) {

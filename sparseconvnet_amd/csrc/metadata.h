@@ -166,6 +166,10 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
                   hipStream_t s);
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
                      int drop, hipStream_t s);
+void avgpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
+                     int drop, hipStream_t s);
+void unpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes,
+                    int drop, hipStream_t s);
 void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
                      int64_t out_stride, const float *mean, const float *var, const float *gamma,
                      const float *beta, float eps, float leak, hipStream_t s);

@@ -67,14 +67,20 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
   LAUNCH_CHECK();
 }
 
-// ---- max pooling ------------------------------------------------------------------------
-// CPU/MaxPooling.cpp:7-20,50: the output starts at zero and takes every input of its window
-// that compares greater, so the result is max(0, active inputs); output-stationary here.
-template <int V>
-__global__ void k_maxpool(const int *nbr, const int *rowmap, int K, int64_t n_out, int64_t npad,
-                          const float *in, int in_stride, float *out, int planes) {
-  // thread -> (output position, group of V planes)
+// Pooling over a neighbour table, one thread per (output position, group of V planes).
+// MAX     CPU/MaxPooling.cpp:7-20,37-60: the output starts at zero, so the result is
+//         max(0, inputs of the window).
+// AVERAGE CPU/AveragePooling.cpp:7-20,38-61: sum over the window's active inputs of
+//         in / filter volume (absent sites count as zeros), taps in ascending order as the
+//         reference walks its rule lists.
+// UNPOOL  CPU/UnPooling.cpp:7-20,34-57: sum of the rows the table lists (over the fine level's
+//         table of a strided rulebook that is the copy of the one coarse row above each site).
+enum { POOL_MAX = 0, POOL_AVERAGE = 1, POOL_UNPOOL = 2 };
+template <int V, int MODE>
+__global__ void k_pool(const int *nbr, const int *rowmap, int K, int64_t n_out, int64_t npad,
+                       const float *in, int in_stride, float *out, int planes) {
   const int groups = planes / V;
+  const float volume = (float)K;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t total = n_out * groups;
   const int64_t step = (int64_t)gridDim.x * blockDim.x;
@@ -87,14 +93,20 @@ __global__ void k_maxpool(const int *nbr, const int *rowmap, int K, int64_t n_ou
       const int j = nbr[(int64_t)k * npad + o];
       if (j >= 0) {
         const float *src = in + (int64_t)j * in_stride + p;
+        float x[V];
         if (V == 4) {
           const float4 t = *reinterpret_cast<const float4 *>(src);
-          acc[0] = acc[0] < t.x ? t.x : acc[0];
-          acc[1] = acc[1] < t.y ? t.y : acc[1];
-          acc[2] = acc[2] < t.z ? t.z : acc[2];
-          acc[3] = acc[3] < t.w ? t.w : acc[3];
+          x[0] = t.x, x[1] = t.y, x[2] = t.z, x[3] = t.w;
         } else {
-          for (int v = 0; v < V; v++) acc[v] = acc[v] < src[v] ? src[v] : acc[v];
+          for (int v = 0; v < V; v++) x[v] = src[v];
+        }
+        for (int v = 0; v < V; v++) {
+          if (MODE == POOL_MAX)
+            acc[v] = acc[v] < x[v] ? x[v] : acc[v];
+          else if (MODE == POOL_AVERAGE)
+            acc[v] += x[v] / volume;
+          else
+            acc[v] += x[v];
         }
       }
     }
@@ -105,20 +117,33 @@ __global__ void k_maxpool(const int *nbr, const int *rowmap, int K, int64_t n_ou
       for (int v = 0; v < V; v++) out[row * planes + p + v] = acc[v];
   }
 }
-void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
-                     hipStream_t s) {
+template <int MODE>
+static void pool_launch(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
+                        hipStream_t s) {
   if (t.n == 0 || planes <= 0) return;
   const bool vec = planes % 4 == 0 && in_stride % 4 == 0 && drop % 4 == 0 && ((uintptr_t)in % 16 == 0) &&
                    ((uintptr_t)out % 16 == 0);
   int64_t total = t.n * (vec ? planes / 4 : planes);
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   if (vec)
-    k_maxpool<4><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
-                                                       in_stride, out, planes);
+    k_pool<4, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+                                                          in_stride, out, planes);
   else
-    k_maxpool<1><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
-                                                       in_stride, out, planes);
+    k_pool<1, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+                                                          in_stride, out, planes);
   LAUNCH_CHECK();
+}
+void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
+                     hipStream_t s) {
+  pool_launch<POOL_MAX>(t, in, in_stride, out, planes, drop, s);
+}
+void avgpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
+                     hipStream_t s) {
+  pool_launch<POOL_AVERAGE>(t, in, in_stride, out, planes, drop, s);
+}
+void unpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
+                    hipStream_t s) {
+  pool_launch<POOL_UNPOOL>(t, in, in_stride, out, planes, drop, s);
 }
 
 // ---- input / output layers --------------------------------------------------------------

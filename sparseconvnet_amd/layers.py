@@ -354,6 +354,54 @@ class MaxPooling(Module):
         return s
 
 
+class AveragePooling(MaxPooling):
+    """averagePooling.py:13-67: the sum of the window's active inputs over the filter volume."""
+
+    def forward(self, input):
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = (input.spatial_size - self.pool_size).div(
+            self.pool_stride, rounding_mode='trunc') + 1
+        assert ((output.spatial_size - 1) * self.pool_stride + self.pool_size == input.spatial_size).all()
+        md, a, drop = input.metadata, (input.spatial_size, output.spatial_size, self.pool_size,
+                                       self.pool_stride), self.nFeaturesToDrop
+        output.features = _run(lambda x: md.averagePooling(*a, x, drop), input.features)
+        return output
+
+    def __repr__(self):
+        return 'Average' + MaxPooling.__repr__(self)[3:]
+
+
+class UnPooling(Module):
+    """unPooling.py:59-96: every site of the finer level (which must exist in the metadata
+    already) receives the rows of the coarse sites whose pooling windows hold it."""
+
+    def __init__(self, dimension, pool_size, pool_stride, nFeaturesToDrop=0):
+        super(UnPooling, self).__init__()
+        self.dimension = dimension
+        self.pool_size = toLongTensor(dimension, pool_size)
+        self.pool_stride = toLongTensor(dimension, pool_stride)
+        self.nFeaturesToDrop = nFeaturesToDrop
+
+    def forward(self, input):
+        output = SparseConvNetTensor()
+        output.metadata = input.metadata
+        output.spatial_size = (input.spatial_size - 1) * self.pool_stride + self.pool_size
+        md, a, drop = input.metadata, (input.spatial_size, output.spatial_size, self.pool_size,
+                                       self.pool_stride), self.nFeaturesToDrop
+        output.features = _run(lambda x: md.unPooling(*a, x, drop), input.features)
+        return output
+
+    def input_spatial_size(self, out_size):
+        return (out_size - 1) * self.pool_stride + self.pool_size
+
+    def __repr__(self):
+        s = _size_repr('UnPooling', self.pool_size, self.pool_stride)
+        if self.nFeaturesToDrop > 0:
+            s = s + ' nFeaturesToDrop = ' + str(self.nFeaturesToDrop)
+        return s
+
+
 class InputLayer(Module):
     """ioLayers.py:15-65.  forward takes (coords, features[, batch_size]): coords is an int64
     tensor [N, dimension] (one sample) or [N, dimension+1] (last column = sample index),

@@ -192,15 +192,31 @@ class Metadata:
                                        C.byref(macs) if want_macs else None))
         return out, (macs.value if want_macs else None)
 
-    def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
-        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
-        _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
+    def _pool(self, fn, rule_sizes, a, n_rows, features, n_features_to_drop):
+        _lib.check(self._L.scn_md_strided_rules(self._h, *rule_sizes, _stream()))
         features = _features(features, "features")
         planes = features.size(1) - n_features_to_drop
-        out = torch.empty((self.getNActive(out_size), planes), dtype=torch.float32, device=features.device)
-        _lib.check(self._L.scn_maxpool_fwd(self._h, *a, _ptr(features), features.size(1), _ptr(out), planes,
-                                           n_features_to_drop, _stream()))
+        out = torch.empty((n_rows(), planes), dtype=torch.float32, device=features.device)
+        _lib.check(fn(self._h, *a, _ptr(features), features.size(1), _ptr(out), planes, n_features_to_drop,
+                      _stream()))
         return out
+
+    def maxPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        return self._pool(self._L.scn_maxpool_fwd, a, a, lambda: self.getNActive(out_size), features,
+                          n_features_to_drop)
+
+    def averagePooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        return self._pool(self._L.scn_avgpool_fwd, a, a, lambda: self.getNActive(out_size), features,
+                          n_features_to_drop)
+
+    def unPooling(self, in_size, out_size, pool_size, pool_stride, features, n_features_to_drop):
+        """in_size: the coarse level the features live on; out_size: the finer level."""
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        rb = [self._s(v) for v in (out_size, in_size, pool_size, pool_stride)]
+        return self._pool(self._L.scn_unpool_fwd, rb, a, lambda: self.getNActive(out_size), features,
+                          n_features_to_drop)
 
     def sparseToDense(self, spatial_size, features, n_planes):
         features = _features(features, "features")

@@ -110,6 +110,7 @@ def dense_weight(w, dim, size):
 
 _CONV = {1: F.conv1d, 2: F.conv2d, 3: F.conv3d}
 _CONVT = {1: F.conv_transpose1d, 2: F.conv_transpose2d, 3: F.conv_transpose3d}
+_AVG = {1: F.avg_pool1d, 2: F.avg_pool2d, 3: F.avg_pool3d}
 _POOL = {1: F.max_pool1d, 2: F.max_pool2d, 3: F.max_pool3d}
 
 
@@ -168,6 +169,15 @@ def dense_maxpool(loc, feats, spatial, size, stride, batch):
     # the output starts at zero and only grows (CPU/MaxPooling.cpp:17-18,50): a window whose
     # sites are all active and negative still yields 0
     return _POOL[dim](x, sz, st).clamp(min=0)
+
+
+def dense_avgpool(loc, feats, spatial, size, stride, batch):
+    """Sum of the window over its volume, absent sites as zeros (CPU/AveragePooling.cpp:19,59)."""
+    dim = loc.shape[1] - 1
+    x = to_dense(loc, feats, spatial, batch)
+    sz = [int(s) for s in np.broadcast_to(np.asarray(size), (dim,))]
+    st = [int(s) for s in np.broadcast_to(np.asarray(stride), (dim,))]
+    return _AVG[dim](x, sz, st)
 
 
 def active_mask(loc, spatial, batch):

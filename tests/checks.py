@@ -156,6 +156,17 @@ def check_strided(make, dim, size, stride, seed, out_spatial=4, n=150, batch=2, 
     assert_close(mp, bf.sample_dense(dmp, loc_out), "max pooling")
     mp1 = p.maxpool(in_sp, out_sp, size, stride, x, 1)
     assert_close(mp1, mp[:, 1:], "max pooling nFeaturesToDrop")
+    # average pooling: window sum over the filter volume, absent sites count as zeros
+    ap = p.avgpool(in_sp, out_sp, size, stride, x)
+    dap = bf.dense_avgpool(loc, x, in_sp, size, stride, batch)
+    assert_close(ap, bf.sample_dense(dap, loc_out), "average pooling")
+    assert_close(p.avgpool(in_sp, out_sp, size, stride, x, 2), ap[:, 2:], "average pooling nFeaturesToDrop")
+    # unpooling: the transposed convolution whose every tap is the identity matrix
+    eye = np.broadcast_to(np.eye(cout, dtype=np.float32), (K, 1, cout, cout)).copy()
+    up = p.unpool(out_sp, in_sp, size, stride, y)
+    dup = bf.dense_deconv(loc_out, y, eye, out_sp, size, stride, batch)
+    assert_close(up, bf.sample_dense(dup, loc), "unpooling")
+    assert_close(p.unpool(out_sp, in_sp, size, stride, y, 1), up[:, 1:], "unpooling nFeaturesToDrop")
     # deconvolution back to the fine level: transposed conv masked to the fine active set
     w2 = (rng.normal(size=(K, 1, cout, cin)) * 0.3).astype(np.float32)
     z, macs2 = p.deconv(out_sp, in_sp, size, stride, y, w2)

@@ -160,6 +160,27 @@ class HipPath:
                                           n_features_to_drop, _stream()))
         return out.cpu().numpy()
 
+    def avgpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
+        sizes = [self._s(v) for v in (in_size, out_size, size, stride)]
+        _lib.check(self.L.scn_md_strided_rules(self.h, *sizes, _stream()))
+        xd = _dev(x, torch.float32)
+        planes = x.shape[1] - n_features_to_drop
+        out = torch.full((self.nactive(out_size), planes), float("nan"), dtype=torch.float32,
+                         device="cuda")
+        _lib.check(self.L.scn_avgpool_fwd(self.h, *sizes, _ptr(xd), x.shape[1], _ptr(out), planes,
+                                          n_features_to_drop, _stream()))
+        return out.cpu().numpy()
+
+    def unpool(self, in_size, out_size, size, stride, x, n_features_to_drop=0):
+        sizes = [self._s(v) for v in (in_size, out_size, size, stride)]
+        xd = _dev(x, torch.float32)
+        planes = x.shape[1] - n_features_to_drop
+        out = torch.full((self.nactive(out_size), planes), float("nan"), dtype=torch.float32,
+                         device="cuda")
+        _lib.check(self.L.scn_unpool_fwd(self.h, *sizes, _ptr(xd), x.shape[1], _ptr(out), planes,
+                                         n_features_to_drop, _stream()))
+        return out.cpu().numpy()
+
     def bn_eval(self, x, mean, var, weight=None, bias=None, eps=1e-4, leakiness=1.0):
         xd = _dev(x, torch.float32)
         out = torch.full_like(xd, float("nan"))

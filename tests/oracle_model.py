@@ -46,6 +46,14 @@ def run(module, path, x):
         b = _np(module.bias) if hasattr(module, 'bias') else None
         y, _ = path.nin(x.features, _np(module.weight), b)
         return CpuTensor(y, x.spatial)
+    if isinstance(module, scn.AveragePooling):
+        ps, st = _np(module.pool_size), _np(module.pool_stride)
+        out_sp = (x.spatial - ps) // st + 1
+        return CpuTensor(path.avgpool(x.spatial, out_sp, ps, st, x.features, module.nFeaturesToDrop), out_sp)
+    if isinstance(module, scn.UnPooling):
+        ps, st = _np(module.pool_size), _np(module.pool_stride)
+        out_sp = (x.spatial - 1) * st + ps
+        return CpuTensor(path.unpool(x.spatial, out_sp, ps, st, x.features, module.nFeaturesToDrop), out_sp)
     if isinstance(module, scn.MaxPooling):
         ps, st = _np(module.pool_size), _np(module.pool_stride)
         out_sp = (x.spatial - ps) // st + 1

@@ -21,7 +21,8 @@ def test_exports():
     for name in ["SubmanifoldConvolution", "ValidConvolution", "Convolution", "Deconvolution",
                  "BatchNormalization", "BatchNormReLU", "BatchNormLeakyReLU", "MaxPooling", "InputLayer",
                  "OutputLayer", "SparseToDense", "Metadata", "SparseConvNetTensor", "Sequential", "ConcatTable",
-                 "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor"]:
+                 "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor",
+                 "NetworkInNetwork", "AveragePooling", "UnPooling"]:
         assert hasattr(scn, name), name
     assert scn.forward_pass_multiplyAdd_count == 0 and scn.forward_pass_hidden_states == 0
 
@@ -61,6 +62,16 @@ def test_spatial_size_arithmetic():
     m = hello_world_model()
     assert m.input_spatial_size(t([10, 10])).tolist() == [87, 87]
     assert m.input_spatial_size(t([8, 8])).tolist() == [71, 71]
+
+
+def test_pooling_modules():
+    # averagePooling.py:21-66, unPooling.py:59-96
+    a = scn.AveragePooling(3, 3, 2)
+    assert repr(a) == 'AveragePooling3/2' and (a.input_spatial_size(torch.LongTensor([7, 7, 7])) == 15).all()
+    assert repr(scn.AveragePooling(2, [3, 2], [2, 1])) == 'AveragePooling(3,2)/(2,1)'
+    u = scn.UnPooling(3, 2, 2)
+    assert repr(u) == 'UnPooling2/2' and (u.input_spatial_size(torch.LongTensor([4, 4, 4])) == 8).all()
+    assert u.nFeaturesToDrop == 0 and len(list(u.parameters())) == 0
 
 
 def test_bn_modules():

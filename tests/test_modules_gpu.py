@@ -103,6 +103,28 @@ def test_residual_unet_vs_oracle(oracle_built):
     checks.assert_close(got.cpu().numpy(), want, "residual U-Net output rows")
 
 
+def test_average_and_unpooling_modules_vs_oracle(oracle_built):
+    """AveragePooling down and UnPooling back up around a convolution, joined with the skip
+    path (the shape of FullyConvolutionalNet's levels, networkArchitectures.py:259-312)."""
+    torch.manual_seed(7)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, 8, 3, False)).add(scn.BatchNormReLU(8)).add(
+        scn.ConcatTable().add(scn.Identity()).add(
+            scn.Sequential().add(scn.AveragePooling(3, 2, 2)).add(scn.SubmanifoldConvolution(3, 8, 12, 3, True))
+            .add(scn.BatchNormLeakyReLU(12)).add(scn.UnPooling(3, 2, 2)))).add(scn.JoinTable()).add(
+        scn.AveragePooling(3, 2, 2, nFeaturesToDrop=4)).eval()
+    randomise_bn(model, 7)
+    assert (model.input_spatial_size(torch.LongTensor([15] * 3)) == 30).all()
+    coords = synthetic.scene_batch(seed=7000, batch=3, target=3000, spatial=30, n_boxes=5)
+    rng = np.random.default_rng(7)
+    feats = rng.uniform(-1, 1, size=(len(coords), 3)).astype(np.float32)
+    inp_layer = scn.InputLayer(3, 30, mode=3)
+    got, want, p = _run_both(model, inp_layer, [torch.as_tensor(coords), torch.as_tensor(feats)])
+    assert got.features.shape == (p.nactive(15), 16) and (got.spatial_size == 15).all()
+    rows = lambda loc: cpu_path.canon_rows(loc)  # noqa: E731
+    checks.assert_close(got.features.cpu().numpy()[rows(got.get_spatial_locations().numpy())],
+                        want.features[rows(p.spatial_locations(15))], "pooling network")
+
+
 def test_vgg2d_vs_oracle(oracle_built):
     torch.manual_seed(2)
     model = hello_world_model().eval()
