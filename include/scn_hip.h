@@ -62,6 +62,21 @@ int scn_md_input_layer(scn_metadata *md, const int64_t *spatial, const int64_t *
 int scn_md_input_rules_header(scn_metadata *md, int32_t hdr[4]);
 /* Rule rows, device int32 [nOutputRows, 1+maxActive] = [count, input indices.., 0 pad]. */
 int scn_md_input_rules(scn_metadata *md, int32_t *rows, void *stream);
+/* Metadata::blLayer (Metadata/Metadata.cpp:426-436, Metadata/IOLayersRules.h:132-286), the rule
+ * half of BLInputLayer_updateOutput (pybind.cpp:168-173 region, CPU/IOLayers.cpp:117-139).
+ * coords: device int64 [batch, length, dim]; a position whose first coordinate is negative is
+ * empty.  Sample b holds positions b*length .. (b+1)*length-1; rows are numbered by first
+ * occurrence, sample after sample.  mode 0: every position is a row of its own (none may be
+ * empty); 1: the last point of a site, 2: the first (the opposite of scn_md_input_layer, as
+ * in the reference); 3: sum; 4: mean.  The feature passes are scn_input_layer_fwd
+ * (in [batch*length, planes]) and scn_output_layer_fwd (out [batch*length, planes], zeros at
+ * empty positions: BLOutputLayer_updateOutput, CPU/IOLayers.cpp:186-206); the rule rows come
+ * from scn_md_input_rules. */
+int scn_md_bl_input_layer(scn_metadata *md, const int64_t *spatial, const int64_t *coords,
+                          int64_t batch, int64_t length, int mode, void *stream,
+                          int64_t *n_active);
+/* Rule header [mode, maxActive, batchSize, length, nOutputRows] (Metadata/IOLayersRules.h:122-128). */
+int scn_md_bl_rules_header(scn_metadata *md, int32_t hdr[5]);
 
 /* Metadata::getNActive (Metadata/Metadata.cpp:67-70); 0 for an unknown level. */
 int scn_md_nactive(scn_metadata *md, const int64_t *spatial, int64_t *n_active);

@@ -42,6 +42,11 @@ def _load(flavour):
         "input_layer": (C.c_int, [C.c_void_p, _i64p, _i64p, C.c_int, C.c_int, C.c_int, C.c_int]),
         "input_rules_header": (None, [C.c_void_p, _i32p]),
         "input_rules": (None, [C.c_void_p, _i32p]),
+        "bl_input_layer": (C.c_int, [C.c_void_p, _i64p, _i64p, C.c_int, C.c_int, C.c_int]),
+        "bl_rules_header": (None, [C.c_void_p, _i32p]),
+        "bl_rules": (None, [C.c_void_p, _i32p]),
+        "bl_input_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "bl_output_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
         "nactive": (C.c_int, [C.c_void_p, _i64p]),
         "batch_size": (C.c_int, [C.c_void_p, _i64p]),
         "spatial_locations": (None, [C.c_void_p, _i64p, _i64p]),
@@ -125,6 +130,37 @@ class CpuPath:
         if mode != 0 and n_out:
             self.f["input_rules"](self.h, rows.ctypes.data_as(_i32p))
         return hdr, rows
+
+    # batch-by-length input layer: coords [batch, length, dim], features [batch, length, planes]
+    def bl_input_layer(self, spatial, coords, mode=3):
+        coords = np.ascontiguousarray(coords, dtype=np.int64)
+        assert coords.ndim == 3 and coords.shape[2] == self.dim
+        return self.f["bl_input_layer"](self.h, _p64(_sz(self.dim, spatial)), _p64(coords),
+                                        coords.shape[0], coords.shape[1], mode)
+
+    def bl_rules(self):
+        """(header [mode, maxActive, batch, length, nOut], rows [nOut, 1 + maxActive])."""
+        hdr = np.zeros(5, np.int32)
+        self.f["bl_rules_header"](self.h, hdr.ctypes.data_as(_i32p))
+        rows = np.zeros((int(hdr[4]), 1 + int(hdr[1])), np.int32)
+        if hdr[0] != 0 and hdr[4]:
+            self.f["bl_rules"](self.h, rows.ctypes.data_as(_i32p))
+        return hdr, rows
+
+    def bl_input_fwd(self, x):
+        x = _f32(x)
+        hdr, _ = self.bl_rules()
+        flat = np.ascontiguousarray(x.reshape(-1, x.shape[-1]))
+        out = np.zeros((int(hdr[4]), x.shape[-1]), np.float32)
+        self.f["bl_input_fwd"](self.h, _pf(flat), _pf(out), x.shape[-1])
+        return out
+
+    def bl_output_fwd(self, x):
+        x = _f32(x)
+        hdr, _ = self.bl_rules()
+        out = np.zeros((int(hdr[2]), int(hdr[3]), x.shape[1]), np.float32)
+        self.f["bl_output_fwd"](self.h, _pf(x), _pf(out), x.shape[1])
+        return out
 
     def nactive(self, spatial):
         return self.f["nactive"](self.h, _p64(_sz(self.dim, spatial)))

@@ -243,6 +243,39 @@ void ref_output_fwd(void *h, const float *in, float *out, int nPlanes) {
            auto O = torch::empty({0}, at::kFloat);
            cpu_OutputLayer_updateOutput<float, D>(m, I, O); copy_out(O, out));
 }
+int ref_bl_input_layer(void *h, const int64_t *spatial, const int64_t *coords, int batchSize,
+                       int length, int mode) {
+  int r = 0;
+  DISPATCH(h, auto S = lt(spatial, D);
+           auto C = torch::from_blob((void *)coords, {batchSize, length, D}, at::kLong).clone();
+           m.blLayer(S, C, mode); r = *m.inputNActive);
+  return r;
+}
+void ref_bl_rules_header(void *h, int *hdr) {
+  DISPATCH(h, (void)D; for (int i = 0; i < 5; i++) hdr[i] = m.blLayerRuleBook[0][i]);
+}
+void ref_bl_rules(void *h, int *rows) {
+  DISPATCH(h, (void)D; if (m.blLayerRuleBook.size() > 1) std::memcpy(
+                           rows, m.blLayerRuleBook[1].data(),
+                           m.blLayerRuleBook[1].size() * sizeof(Int)));
+}
+void ref_bl_input_fwd(void *h, const float *in, float *out, int nPlanes) {
+  // The rule list was built by ref_bl_input_layer; this is the body of
+  // cpu_BLInputLayer_updateOutput after m.blLayer(...) (CPU/IOLayers.cpp:126-138).
+  DISPATCH(h, (void)D; auto &rules = m.blLayerRuleBook; Int mode = rules[0][0];
+           Int maxActive = rules[0][1]; Int nRows = rules[0][4];
+           if (mode == 0) { std::memcpy(out, in, sizeof(float) * (size_t)nRows * nPlanes); }
+           else {
+             std::memset(out, 0, sizeof(float) * (size_t)nRows * nPlanes);
+             InputLayer_ForwardPass<float>((float *)in, out, nRows, maxActive, nPlanes,
+                                           &rules[1][0], mode == 4);
+           });
+}
+void ref_bl_output_fwd(void *h, const float *in, float *out, int nPlanes) {
+  DISPATCH(h, auto I = ft(in, {(int64_t)m.blLayerRuleBook[0][4], nPlanes});
+           auto O = torch::empty({0}, at::kFloat);
+           cpu_BLOutputLayer_updateOutput<float, D>(m, I, O); copy_out(O, out));
+}
 void ref_s2d(void *h, const int64_t *spatial, const float *in, float *out, int nPlanes) {
   DISPATCH(h, auto S = lt(spatial, D); Int n = m.getNActive(S); auto I = ft(in, {n, nPlanes});
            auto O = torch::empty({0}, at::kFloat);

@@ -116,6 +116,7 @@ struct Metadata {
   std::map<Key, Int> nActive;
   std::map<Key, Grids> grids;
   RuleBook inputLayerRuleBook;
+  RuleBook blLayerRuleBook;
   std::map<Key, RuleBook> submanifoldRuleBooks;
   std::map<Key, RuleBook> ruleBooks;
   std::map<Key, RuleBook> sparseToDenseRuleBooks;
@@ -211,6 +212,71 @@ static void inputLayerRules(Grids &SGs, RuleBook &rules, const int64_t *coords,
       rule.push_back((Int)row.size());
       for (auto r : row) rule.push_back(r);
       rule.resize((rule.size() + maxActive) / (maxActive + 1) * (maxActive + 1));
+    }
+  }
+}
+
+// Metadata/IOLayersRules.h:132-286.  coords is [batchSize, length, dim]; a position whose
+// first coordinate is negative is empty.  Header (:122-128):
+// [mode, maxActive, batchSize, length, nOutputRows]; rows nOutputRows x (1 + maxActive).
+// Mode 1 keeps the LAST point of a site (:184-190), mode 2 the first (:199-207).
+static void blRules(Grids &SGs, RuleBook &rules, const int64_t *coords, Int batchSize, Int length,
+                    Int mode, Int &nActive, int dim) {
+  SGs.clear();
+  resize_grids(SGs, batchSize, dim);
+  Pt p = Pt();
+  if (mode == 0) {  // :141-162 every position is its own row
+    nActive = batchSize * length;
+    rules.resize(1);
+    rules[0] = {mode, 1, batchSize, length, nActive};
+    for (Int I = 0; I < batchSize; I++) {
+      SGs[I].ctr = I * length;
+      const int64_t *c = coords + (size_t)I * length * dim;
+      for (Int l = 0; l < length; ++l, c += dim) {
+        for (int j = 0; j < dim; j++) p.x[j] = (Int)c[j];
+        *SGs[I].insert(p, l).first = l;
+      }
+    }
+    return;
+  }
+  // per sample: the input rows of every output row, in input order (:165-252)
+  std::vector<std::vector<std::vector<Int>>> outputRows(batchSize);
+  for (Int I = 0; I < batchSize; I++) {
+    auto &ors = outputRows[I];
+    const int64_t *c = coords + (size_t)I * length * dim;
+    Int i = I * length;
+    for (Int l = 0; l < length; ++l, ++i, c += dim) {
+      for (int j = 0; j < dim; j++) p.x[j] = (Int)c[j];
+      if (p.x[0] < 0) continue;
+      auto r = SGs[I].insert(p, (Int)ors.size());
+      if (r.second) ors.emplace_back();
+      ors[*r.first].push_back(i);
+    }
+  }
+  for (Int I = 0; I < batchSize; I++) {  // :209-212,254-257
+    SGs[I].ctr = nActive;
+    nActive += (Int)outputRows[I].size();
+  }
+  Int maxActive = 1;
+  if (mode >= 3)
+    for (auto &ors : outputRows)
+      for (auto &row : ors) maxActive = std::max(maxActive, (Int)row.size());
+  rules.resize(2);
+  rules[0] = {mode, maxActive, batchSize, length, nActive};
+  auto &rule = rules[1];
+  rule.assign((size_t)(maxActive + 1) * nActive, 0);
+  for (Int I = 0; I < batchSize; I++) {
+    Int *rr = rule.data() + (size_t)SGs[I].ctr * (maxActive + 1);
+    for (auto &row : outputRows[I]) {
+      if (mode == 1) {
+        rr[0] = 1, rr[1] = row.back();
+      } else if (mode == 2) {
+        rr[0] = 1, rr[1] = row.front();
+      } else {
+        rr[0] = (Int)row.size();
+        for (size_t q = 0; q < row.size(); q++) rr[1 + q] = row[q];
+      }
+      rr += 1 + maxActive;
     }
   }
 }
@@ -660,6 +726,33 @@ void orc_bn_eval(const float *in, float *out, int nActive, int nPlanes, int inSt
   }
 }
 // CPU/IOLayers.cpp:11-29,49-72.  out is [nActive, nPlanes].
+// CPU/IOLayers.cpp:11-29: out (zero-filled by the caller) += mult * in over each row's list.
+static void input_forward_pass(const float *in, float *out, Int nRows, Int maxActive, int nPlanes,
+                               const Int *R, bool average) {
+#pragma omp parallel for
+  for (Int row = 0; row < nRows; row++) {
+    const Int *r = R + (size_t)row * (1 + maxActive);
+    Int nA = r[0];
+    float mult = (average && nA > 0) ? 1.f / nA : 1.f;
+    float *o = out + (size_t)row * nPlanes;
+    for (Int i = 1; i <= nA; ++i) {
+      const float *f = in + (size_t)r[i] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += mult * f[p];
+    }
+  }
+}
+// CPU/IOLayers.cpp:31-47 with average = false: every listed input point receives its row.
+static void input_backward_pass(float *points, const float *rows, Int nRows, Int maxActive, int nPlanes,
+                                const Int *R) {
+  for (Int row = 0; row < nRows; row++) {
+    const Int *r = R + (size_t)row * (1 + maxActive);
+    const float *f = rows + (size_t)row * nPlanes;
+    for (Int i = 1; i <= r[0]; ++i) {
+      float *o = points + (size_t)r[i] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += f[p];
+    }
+  }
+}
 void orc_input_fwd(void *md, const float *in, float *out, int nPlanes) {
   Metadata &m = *(Metadata *)md;
   auto &rules = m.inputLayerRuleBook;
@@ -669,18 +762,7 @@ void orc_input_fwd(void *md, const float *in, float *out, int nPlanes) {
     return;
   }
   std::memset(out, 0, sizeof(float) * (size_t)nRows * nPlanes);
-  const Int *R = rules[1].data();
-#pragma omp parallel for
-  for (Int row = 0; row < nRows; row++) {
-    const Int *r = R + (size_t)row * (1 + maxActive);
-    Int nA = r[0];
-    float mult = (mode == 4 && nA > 0) ? 1.f / nA : 1.f;
-    float *o = out + (size_t)row * nPlanes;
-    for (Int i = 1; i <= nA; ++i) {
-      const float *f = in + (size_t)r[i] * nPlanes;
-      for (Int p = 0; p < nPlanes; p++) o[p] += mult * f[p];
-    }
-  }
+  input_forward_pass(in, out, nRows, maxActive, nPlanes, rules[1].data(), mode == 4);
 }
 // CPU/IOLayers.cpp:95-115 (InputLayer_BackwardPass :31-47 with average=false).
 // out is [nInputRows, nPlanes].
@@ -693,15 +775,50 @@ void orc_output_fwd(void *md, const float *in, float *out, int nPlanes) {
     return;
   }
   std::memset(out, 0, sizeof(float) * (size_t)rules[0][2] * nPlanes);
-  const Int *R = rules[1].data();
-  for (Int row = 0; row < nRows; row++) {
-    const Int *r = R + (size_t)row * (1 + maxActive);
-    const float *f = in + (size_t)row * nPlanes;
-    for (Int i = 1; i <= r[0]; ++i) {
-      float *o = out + (size_t)r[i] * nPlanes;
-      for (Int p = 0; p < nPlanes; p++) o[p] += f[p];
-    }
+  input_backward_pass(out, in, nRows, maxActive, nPlanes, rules[1].data());
+}
+// Metadata/Metadata.cpp:426-436.  Returns the number of active sites.
+int orc_bl_input_layer(void *md, const int64_t *spatial, const int64_t *coords, int batchSize,
+                       int length, int mode) {
+  Metadata &m = *(Metadata *)md;
+  m.inputSpatialSize = mkkey(m.dim, spatial);
+  Int &nA = m.nActive[m.inputSpatialSize];
+  blRules(m.grids[m.inputSpatialSize], m.blLayerRuleBook, coords, batchSize, length, mode, nA, m.dim);
+  return nA;
+}
+void orc_bl_rules_header(void *md, int *hdr) {
+  Metadata &m = *(Metadata *)md;
+  for (int i = 0; i < 5; i++) hdr[i] = m.blLayerRuleBook[0][i];
+}
+void orc_bl_rules(void *md, int *rows) {
+  Metadata &m = *(Metadata *)md;
+  if (m.blLayerRuleBook.size() > 1)
+    std::memcpy(rows, m.blLayerRuleBook[1].data(), m.blLayerRuleBook[1].size() * sizeof(Int));
+}
+// CPU/IOLayers.cpp:117-139.  in is [batchSize * length, nPlanes], out [nActive, nPlanes].
+void orc_bl_input_fwd(void *md, const float *in, float *out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.blLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][4];
+  if (mode == 0) {
+    std::memcpy(out, in, sizeof(float) * (size_t)nRows * nPlanes);
+    return;
   }
+  std::memset(out, 0, sizeof(float) * (size_t)nRows * nPlanes);
+  input_forward_pass(in, out, nRows, maxActive, nPlanes, rules[1].data(), mode == 4);
+}
+// CPU/IOLayers.cpp:186-206.  out is [batchSize * length, nPlanes].
+void orc_bl_output_fwd(void *md, const float *in, float *out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.blLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][4];
+  size_t nPoints = (size_t)rules[0][2] * rules[0][3];
+  if (mode == 0) {
+    std::memcpy(out, in, sizeof(float) * nPoints * nPlanes);
+    return;
+  }
+  std::memset(out, 0, sizeof(float) * nPoints * nPlanes);
+  input_backward_pass(out, in, nRows, maxActive, nPlanes, rules[1].data());
 }
 // CPU/SparseToDense.cpp:7-19,35-64.  out is [batch, nPlanes, spatial...], zeroed here.
 void orc_s2d(void *md, const int64_t *spatial, const float *in, float *out, int nPlanes) {

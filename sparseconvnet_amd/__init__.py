@@ -14,9 +14,10 @@ forward_pass_hidden_states = 0
 fuse_batchnorm = True
 
 from .containers import AddTable, ConcatTable, JoinTable, Sequential  # noqa: E402
-from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, BatchNormReLU, Convolution,  # noqa: E402
-                     Deconvolution, Identity, InputLayer, MaxPooling, NetworkInNetwork, OutputLayer, SparseToDense,
-                     SubmanifoldConvolution, UnPooling, ValidConvolution)
+from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, BatchNormReLU,  # noqa: E402
+                     BLInputLayer, BLOutputLayer, Convolution, Deconvolution, Identity, InputLayer, MaxPooling,
+                     NetworkInNetwork, OutputLayer, SparseToDense, SubmanifoldConvolution, UnPooling,
+                     ValidConvolution)
 from .metadata import Metadata  # noqa: E402
 from .networks import SparseVggNet, UNet  # noqa: E402
 from .tensor import SparseConvNetTensor  # noqa: E402

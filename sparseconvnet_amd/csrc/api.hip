@@ -139,10 +139,32 @@ int scn_md_input_rules_header(scn_metadata *h, int32_t hdr[4]) {
   return guarded([&] {
     Metadata &m = md(h);
     if (m.input.mode < 0) throw Error("input layer rules have not been built");
-    hdr[0] = m.input.mode;
+    hdr[0] = m.input.user_mode;
     hdr[1] = m.input.max_active;
     hdr[2] = (int32_t)m.input.n_in;
     hdr[3] = (int32_t)m.input.n_out;
+  });
+}
+int scn_md_bl_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *coords, int64_t batch,
+                          int64_t length, int mode, void *stream, int64_t *n_active) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (batch < 0 || length < 0) throw Error("negative batch size or length");
+    if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
+    if (batch * length == 0) length = 1, batch = 0;
+    build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, st(stream), length);
+    if (n_active) *n_active = m.input.n_out;
+  });
+}
+int scn_md_bl_rules_header(scn_metadata *h, int32_t hdr[5]) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (m.input.mode < 0 || m.input.bl_length == 0) throw Error("batch-by-length input rules have not been built");
+    hdr[0] = m.input.user_mode;
+    hdr[1] = m.input.max_active;
+    hdr[2] = (int32_t)m.input.bl_batch;
+    hdr[3] = (int32_t)m.input.bl_length;
+    hdr[4] = (int32_t)m.input.n_out;
   });
 }
 int scn_md_input_rules(scn_metadata *h, int32_t *rows, void *stream) {

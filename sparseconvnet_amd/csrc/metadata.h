@@ -98,10 +98,12 @@ struct CoefJobs {
 };
 
 struct InputRules {
-  int mode = -1;
+  int mode = -1;      // 1: the first point of a site is listed, 2: the last, 3 / 4: all (sum / mean)
+  int user_mode = -1; // the mode the caller gave (the batch-by-length layer numbers 1 and 2 the other way round)
   int max_active = 0;
   int64_t n_in = 0, n_out = 0;
-  DevBuf<int> row_of_input;  // [n_in]
+  int64_t bl_batch = 0, bl_length = 0;  // batch-by-length input (BLInputLayer); 0: plain input layer
+  DevBuf<int> row_of_input;  // [n_in]; -1: an empty position of a batch-by-length input
   DevBuf<int> sorted_idx;    // [n_in] input indices grouped by site, input order inside a group
   DevBuf<int> run_start;     // [n_out] first position of the row's group in sorted_idx
   DevBuf<int> run_len;       // [n_out]
@@ -138,8 +140,10 @@ struct Metadata {
 SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);
 Geom make_geom(int dim, const int64_t *spatial);
 
+// bl_length > 0: coords is [n / bl_length, bl_length, dim] (BLInputLayer), the sample is the
+// first index and positions whose first coordinate is negative are empty.
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
-                       int ncols, int min_batch, int mode, hipStream_t s);
+                       int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length = 0);
 void export_input_rules(Metadata &m, int *rows, hipStream_t s);
 void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStream_t s);
 Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s);

@@ -117,27 +117,33 @@ static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
 // ---- input layer -----------------------------------------------------------------------
 
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
-__global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols,
+// bl_len > 0: the sample of point i is i / bl_len and a negative first coordinate marks an
+// empty position (Metadata/IOLayersRules.h:183,204,234): key EMPTY, counted in flags[4].
+__global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols, int64_t bl_len,
                              unsigned long long *keys, int *idx, int *flags) {
   // flags[0]: error bits, flags[3]: largest sample index (one atomic per wavefront)
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int bmax = 0;
+  bool empty = false;
   if (i < n) {
     const int64_t *c = coords + i * ncols;
     int cc[SCN_MAXD];
     bool ok = true;
+    empty = bl_len > 0 && c[0] < 0;
     for (int d = 0; d < g.dim; d++) {
       int64_t v = c[d];
       if (v < 0 || v >= g.size[d]) ok = false;
       cc[d] = (int)v;
     }
-    int64_t b = ncols > g.dim ? c[g.dim] : 0;
+    int64_t b = bl_len > 0 ? i / bl_len : (ncols > g.dim ? c[g.dim] : 0);
     if (b < 0 || b >= g.max_batch) {
       atomicOr(&flags[0], 2);
       ok = false;
       b = 0;
     }
-    if (!ok) {
+    if (empty) {
+      keys[i] = SCN_EMPTY_KEY;
+    } else if (!ok) {
       atomicOr(&flags[0], 1);
       keys[i] = SCN_EMPTY_KEY;
     } else {
@@ -148,31 +154,35 @@ __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols
   }
   for (int off = 32; off; off >>= 1) bmax = max(bmax, __shfl_xor(bmax, off));
   if ((threadIdx.x & 63) == 0 && bmax > 0) atomicMax(&flags[3], bmax);
+  const unsigned long long em = __ballot(empty);
+  if ((threadIdx.x & 63) == 0 && em) atomicAdd(&flags[4], __popcll(em));
 }
 
 // mode 0: row = input index.
-__global__ void k_input_rows_identity(Geom g, const int64_t *coords, int64_t n, int ncols,
+__global__ void k_input_rows_identity(Geom g, const int64_t *coords, int64_t n, int ncols, int64_t bl_len,
                                       int64_t npad, int *soa) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const int64_t *c = coords + i * ncols;
   for (int d = 0; d < g.dim; d++) soa[d * npad + i] = (int)c[d];
-  soa[g.dim * npad + i] = ncols > g.dim ? (int)c[g.dim] : 0;
+  soa[g.dim * npad + i] = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)c[g.dim] : 0);
 }
 
 // After the stable sort: head[p] marks the first point of each group of equal keys;
-// is_first[i] marks input points that are the first occurrence of their site.
-__global__ void k_group_heads(const unsigned long long *skeys, const int *sidx, int64_t n,
+// is_first[i] marks input points that are the first occurrence of their site.  Positions from
+// n_valid on hold the empty points of a batch-by-length input: no group, never first.
+__global__ void k_group_heads(const unsigned long long *skeys, const int *sidx, int64_t n, int64_t n_valid,
                               int *head, int *is_first) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n) return;
-  int h = (p == 0 || skeys[p] != skeys[p - 1]) ? 1 : 0;
+  int h = (p < n_valid && (p == 0 || skeys[p] != skeys[p - 1])) ? 1 : 0;
   head[p] = h;
   is_first[sidx[p]] = h;
 }
 
 // Heads: row = rank of the first occurrence in input order (Metadata/IOLayersRules.h:84-87).
-__global__ void k_assign_rows(Geom g, const int64_t *coords, int ncols, const unsigned long long *skeys,
+__global__ void k_assign_rows(Geom g, const int64_t *coords, int ncols, int64_t bl_len,
+                              const unsigned long long *skeys,
                               const int *sidx, const int *head, const int *head_scan,
                               const int *first_scan, int64_t n, int64_t npad, int *soa,
                               unsigned long long *level_keys, int *sched, int *row_of_group,
@@ -188,7 +198,7 @@ __global__ void k_assign_rows(Geom g, const int64_t *coords, int ncols, const un
   level_keys[row] = skeys[p];
   const int64_t *c = coords + (int64_t)i * ncols;
   for (int d = 0; d < g.dim; d++) soa[d * npad + row] = (int)c[d];
-  soa[g.dim * npad + row] = ncols > g.dim ? (int)c[g.dim] : 0;
+  soa[g.dim * npad + row] = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)c[g.dim] : 0);
 }
 
 __global__ void k_finish_groups(const int *sidx, const int *head, const int *head_scan,
@@ -214,8 +224,10 @@ __global__ void k_finish_groups(const int *sidx, const int *head, const int *hea
 }
 
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
-                       int ncols, int min_batch, int mode, hipStream_t s) {
-  if (ncols != m.dim && ncols != m.dim + 1) throw Error("coords must have dim or dim+1 columns");
+                       int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length) {
+  const bool bl = bl_length > 0;
+  if (bl ? ncols != m.dim : (ncols != m.dim && ncols != m.dim + 1))
+    throw Error(bl ? "coords must be [batch, length, dim]" : "coords must have dim or dim+1 columns");
   if (mode < 0 || mode > 4) throw Error("input layer mode must be 0..4");
   if (n >= ((int64_t)1 << 31) - 64) throw Error("too many input points for int32 rule indices");
   Geom g = make_geom(m.dim, spatial);
@@ -223,10 +235,15 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   m.input_size = key;
   Level &L = m.levels[key];
   InputRules &R = m.input;
-  R.mode = mode;
+  // Metadata/IOLayersRules.h:96-107 against :180-205: the plain layer lists the first point of
+  // a site in mode 1 and the last in mode 2, the batch-by-length layer the other way round.
+  R.user_mode = mode;
+  R.mode = (bl && (mode == 1 || mode == 2)) ? 3 - mode : mode;
   R.n_in = n;
   R.max_active = 1;
-  int batch_floor = ncols == m.dim ? 1 : std::max(min_batch, 0);
+  R.bl_length = bl_length;
+  R.bl_batch = bl ? n / bl_length : 0;
+  int batch_floor = bl ? (int)R.bl_batch : (ncols == m.dim ? 1 : std::max(min_batch, 0));
   if (n == 0) {
     alloc_level(L, g, 0, batch_floor);
     L.identity_sched = true;
@@ -239,26 +256,32 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   m.v1.reserve(n);
   m.dflags.reserve(8);
   fill32(m.dflags.p, 0, 8, s);
-  k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, m.k0.p, m.v0.p, m.dflags.p);
+  k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, bl_length, m.k0.p, m.v0.p, m.dflags.p);
   LAUNCH_CHECK();
-  int hflags[4];
+  int hflags[5];
   HIP_CHECK(hipMemcpyAsync(hflags, m.dflags.p, sizeof hflags, hipMemcpyDeviceToHost, s));
   HIP_CHECK(hipStreamSynchronize(s));
   if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
   if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");
   const int top_batch = hflags[3];
-  // only the key bits that samples 0..top_batch can set take part in the sort
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s, key_bits(g, (int64_t)top_batch + 1));
+  const int64_t n_empty = hflags[4], nv = n - n_empty;
+  if (n_empty && mode == 0) throw Error("batch-by-length input layer: mode 0 needs every position filled");
+  // only the key bits that samples 0..top_batch can set take part in the sort; one bit more
+  // keeps the EMPTY keys (all ones) of empty positions behind every real key
+  const int bits = key_bits(g, (int64_t)top_batch + 1) + (n_empty ? 1 : 0);
+  if (bits > 64) throw Error("batch-by-length input layer: grid too large for a layer with empty positions");
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s, bits);
   // Metadata/IOLayersRules.h:25,46-47,76-77: the batch is at least min_batch and grows to
   // the largest sample index + 1; without a sample column there is exactly one sample.
-  int batch = ncols == m.dim ? 1 : std::max(batch_floor, top_batch + 1);
+  // :140 batch-by-length: one grid per sample of the input, filled or not.
+  int batch = bl ? batch_floor : (ncols == m.dim ? 1 : std::max(batch_floor, top_batch + 1));
 
   if (mode == 0) {
     alloc_level(L, g, n, batch);
     L.sched.reserve(n);
     L.identity_sched = false;
     L.dups = true;  // mode 0 does not merge repeated points
-    k_input_rows_identity<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, L.npad, L.coords.p);
+    k_input_rows_identity<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, bl_length, L.npad, L.coords.p);
     LAUNCH_CHECK();
     HIP_CHECK(hipMemcpyAsync(L.keys.p, m.k0.p, n * sizeof(unsigned long long), hipMemcpyDeviceToDevice, s));
     HIP_CHECK(hipMemcpyAsync(L.sched.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
@@ -270,7 +293,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   m.f1.reserve(n);  // is_first
   m.s0.reserve(n + 1);  // head_scan
   m.s1.reserve(n + 1);  // first_scan
-  k_group_heads<<<grid_for(n), TB, 0, s>>>(m.k1.p, m.v1.p, n, m.f0.p, m.f1.p);
+  k_group_heads<<<grid_for(n), TB, 0, s>>>(m.k1.p, m.v1.p, n, nv, m.f0.p, m.f1.p);
   LAUNCH_CHECK();
   exclusive_scan(m, m.f0.p, m.s0.p, n, s);
   exclusive_scan(m, m.f1.p, m.s1.p, n, s);
@@ -285,20 +308,23 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   R.n_out = N;
   R.row_of_input.reserve(n);
   R.sorted_idx.reserve(n);
-  R.run_start.reserve(N);
-  R.run_len.reserve(N);
+  R.run_start.reserve(std::max<int64_t>(N, 1));
+  R.run_len.reserve(std::max<int64_t>(N, 1));
+  if (n_empty) fill32(R.row_of_input.p, 0xFFFFFFFFu, n, s);  // empty positions belong to no row
+  HIP_CHECK(hipMemcpyAsync(R.sorted_idx.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
+  if (N == 0) return;
   m.v0.reserve(std::max<int64_t>(n, 2 * N + 2));  // reused: row_of_group | head_pos
   int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
   fill32(m.dflags.p, 0, 8, s);
-  k_assign_rows<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, m.k1.p, m.v1.p, m.f0.p, m.s0.p, m.s1.p,
+  k_assign_rows<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, bl_length, m.k1.p, m.v1.p, m.f0.p, m.s0.p, m.s1.p,
                                            n, L.npad, L.coords.p, L.keys.p, L.sched.p, row_of_group,
                                            head_pos);
   LAUNCH_CHECK();
-  k_finish_groups<<<grid_for(n), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, row_of_group, head_pos, n, (int)N,
-                                             R.row_of_input.p, R.run_start.p, R.run_len.p,
-                                             m.dflags.p + 2);
+  // the groups end where the empty positions begin
+  k_finish_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, row_of_group, head_pos, nv, (int)N,
+                                              R.row_of_input.p, R.run_start.p, R.run_len.p,
+                                              m.dflags.p + 2);
   LAUNCH_CHECK();
-  HIP_CHECK(hipMemcpyAsync(R.sorted_idx.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
   int ma = std::max(1, read_back(m.dflags.p + 2, s));  // runs of one never touch the counter
   // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2.
   R.max_active = (mode == 3 || mode == 4) ? ma : 1;

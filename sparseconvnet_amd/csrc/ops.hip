@@ -199,9 +199,9 @@ __global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, con
     int64_t pt = i / planes;
     int p = (int)(i - pt * planes);
     int row = row_of_input[pt];
-    bool listed = true;
-    if (mode == 1) listed = sorted_idx[run_start[row]] == (int)pt;
-    if (mode == 2) listed = sorted_idx[run_start[row] + run_len[row] - 1] == (int)pt;
+    bool listed = row >= 0;  // empty positions of a batch-by-length input get zeros
+    if (listed && mode == 1) listed = sorted_idx[run_start[row]] == (int)pt;
+    if (listed && mode == 2) listed = sorted_idx[run_start[row] + run_len[row] - 1] == (int)pt;
     out[i] = listed ? in[(int64_t)row * planes + p] : 0.0f;
   }
 }
@@ -213,6 +213,10 @@ void output_forward(const InputRules &r, const float *in, float *out, int planes
     return;
   }
   int64_t total = r.n_in * planes;
+  if (r.n_out == 0) {  // every position empty
+    fill32(out, 0, total, s);
+    return;
+  }
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   k_output_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
                                                      r.run_len.p, r.n_in, r.mode, in, out, planes);

@@ -443,6 +443,45 @@ class OutputLayer(Module):
         return _run(lambda x: md.outputLayer(x), input.features)
 
 
+class BLInputLayer(Module):
+    """ioLayers.py:92-138.  forward takes (coords, features): coords an int64 tensor
+    [batch, length, dimension] whose positions with a negative first coordinate are empty,
+    features a float tensor [batch, length, planes].  mode 0: every position is a row;
+    1: the last point of a site, 2: the first, 3: sum, 4: mean."""
+
+    def __init__(self, dimension, spatial_size, mode=3):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.spatial_size = toLongTensor(dimension, spatial_size)
+        self.mode = mode
+        self.device = None
+
+    def to(self, device):
+        self.device = device
+        return self
+
+    def forward(self, input):
+        output = SparseConvNetTensor(metadata=_md.Metadata(self.dimension), spatial_size=self.spatial_size)
+        feats = input[1].to(self.device) if self.device else input[1]
+        if not feats.is_cuda:
+            feats = feats.cuda()
+        md, sz, coords, mode = output.metadata, self.spatial_size, input[0], self.mode
+        output.features = _run(lambda f: md.blInputLayer(sz, coords, f, mode), feats.float())
+        return output
+
+
+class BLOutputLayer(Module):
+    """ioLayers.py:141-160: [batch, length, planes], zeros at the empty positions."""
+
+    def __init__(self, dimension):
+        Module.__init__(self)
+        self.dimension = dimension
+
+    def forward(self, input):
+        md = input.metadata
+        return _run(lambda x: md.blOutputLayer(x), input.features)
+
+
 class SparseToDense(Module):
     """sparseToDense.py:56-78: dense [batch, nPlanes, spatial...] tensor, zeros elsewhere."""
 

@@ -124,6 +124,29 @@ class Metadata:
         _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out
 
+    def blInputLayer(self, spatial_size, coords, features, mode):
+        """coords [batch, length, dimension] (first coordinate < 0: empty position),
+        features [batch, length, planes] -> [nActive, planes]."""
+        coords = coords.to(device=features.device, dtype=torch.int64).contiguous()
+        assert coords.dim() == 3 and features.dim() == 3 and coords.shape[:2] == features.shape[:2], \
+            (coords.shape, features.shape)
+        features = _features(features, "input features")
+        n = C.c_int64(0)
+        _lib.check(self._L.scn_md_bl_input_layer(self._h, self._s(spatial_size), _ptr(coords), coords.size(0),
+                                                 coords.size(1), int(mode), _stream(), C.byref(n)))
+        out = torch.empty((n.value, features.size(2)), dtype=torch.float32, device=features.device)
+        _lib.check(self._L.scn_input_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(2), _stream()))
+        return out
+
+    def blOutputLayer(self, features):
+        """[nActive, planes] -> [batch, length, planes] of the batch-by-length input layer."""
+        features = _features(features, "features")
+        hdr = (C.c_int32 * 5)()
+        _lib.check(self._L.scn_md_bl_rules_header(self._h, hdr))
+        out = torch.empty((hdr[2], hdr[3], features.size(1)), dtype=torch.float32, device=features.device)
+        _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
+        return out
+
     def _conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs):
         """kind 0 / 1 / 2: submanifold / strided / transposed convolution.  bn, post: None, or
         (running_mean, running_var, weight, bias, eps, leakiness) of an eval-mode batch

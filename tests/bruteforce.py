@@ -43,6 +43,26 @@ def input_layer_values(coords, feats, mode):
     return out.astype(np.float32), row_of
 
 
+def bl_groups(coords):
+    """Batch-by-length input [B, L, d]: the flat input indices of every output row, rows in
+    first-occurrence order sample after sample, positions with a negative first coordinate
+    skipped; plus the (coords, sample) location of every row."""
+    B, L, d = coords.shape
+    groups, loc = [], []
+    for b in range(B):
+        seen = {}
+        for l in range(L):
+            c = tuple(int(v) for v in coords[b, l])
+            if c[0] < 0:
+                continue
+            if c not in seen:
+                seen[c] = len(groups)
+                groups.append([])
+                loc.append(c + (b,))
+            groups[seen[c]].append(b * L + l)
+    return groups, np.asarray(loc, np.int64).reshape(len(loc), d + 1)
+
+
 def submanifold_triples(loc, dim, size):
     """Set of (k, in_site, out_site) as coordinate tuples: in = out + tap - size//2, same sample."""
     size = np.broadcast_to(np.asarray(size), (dim,))

@@ -75,6 +75,63 @@ def check_input_layer(make, dim, mode, seed, n=300, spatial=9, batch=3, with_bat
         assert (out[~picked] == 0).all()
 
 
+def check_bl_input_layer(make, dim, mode, seed, batch=3, length=70, spatial=9, planes=5, empties=True):
+    """BLInputLayer / BLOutputLayer against a per-sample dictionary: row numbering, rule table,
+    merged features (mode 1 = last point of a site, 2 = first, 3 = sum, 4 = mean) and the way
+    back, with zeros at empty positions."""
+    rng = np.random.default_rng(seed)
+    coords = rng.integers(0, spatial, (batch, length, dim)).astype(np.int64)
+    if mode == 0:  # unique inside a sample, nothing empty
+        for b in range(batch):
+            cells = rng.permutation(spatial ** dim)[:length]
+            coords[b] = np.stack(np.unravel_index(cells, (spatial,) * dim), 1)
+    elif empties:
+        hole = rng.random((batch, length)) < 0.2
+        coords[hole] = -1
+        if batch > 2:
+            coords[1, :, :] = -1  # a sample without points still counts
+    feats = rng.normal(size=(batch, length, planes)).astype(np.float32)
+    flat = feats.reshape(-1, planes)
+    p = make(dim)
+    n_active = p.bl_input_layer(spatial, coords, mode)
+    hdr, rows = p.bl_rules()
+    if mode == 0:
+        assert n_active == batch * length and list(hdr) == [0, 1, batch, length, batch * length]
+        loc = p.spatial_locations(spatial)
+        want = np.concatenate([coords.reshape(-1, dim), np.repeat(np.arange(batch), length)[:, None]], 1)
+        assert (loc == want).all()
+        assert_close(p.bl_input_fwd(feats), flat)
+        assert_close(p.bl_output_fwd(flat), feats)
+        assert p.batch_size(spatial) == batch
+        return
+    groups, loc_want = bf.bl_groups(coords)
+    assert n_active == len(groups) and p.nactive(spatial) == len(groups)
+    assert (p.spatial_locations(spatial) == loc_want).all()
+    assert p.batch_size(spatial) == batch
+    longest = max([len(g) for g in groups] + [1])
+    assert list(hdr) == [mode, longest if mode >= 3 else 1, batch, length, len(groups)]
+    expect = np.zeros((len(groups), planes), np.float64)
+    for r, g in enumerate(groups):
+        if mode == 1:
+            assert list(rows[r]) == [1, g[-1]]
+            expect[r] = flat[g[-1]]
+        elif mode == 2:
+            assert list(rows[r]) == [1, g[0]]
+            expect[r] = flat[g[0]]
+        else:
+            assert rows[r, 0] == len(g) and list(rows[r, 1:1 + len(g)]) == g and (rows[r, 1 + len(g):] == 0).all()
+            expect[r] = flat[g].astype(np.float64).sum(0) / (len(g) if mode == 4 else 1)
+    assert_close(p.bl_input_fwd(feats), expect, "batch-by-length input, mode %d" % mode)
+    y = rng.normal(size=(len(groups), 4)).astype(np.float32)
+    back = np.zeros((batch * length, 4), np.float32)
+    for r, g in enumerate(groups):
+        listed = g if mode >= 3 else [g[-1] if mode == 1 else g[0]]
+        back[listed] = y[r]
+    out = p.bl_output_fwd(y)
+    assert out.shape == (batch, length, 4)
+    assert_close(out.reshape(-1, 4), back, "batch-by-length output, mode %d" % mode)
+
+
 def _setup(make, dim, spatial, n, batch, seed, C):
     rng = np.random.default_rng(seed)
     coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=n // 4)

@@ -55,6 +55,37 @@ class HipPath:
             _lib.check(self.L.scn_md_input_rules(self.h, _ptr(rows), _stream()))
         return np.array(list(hdr), np.int32), rows.cpu().numpy()
 
+    def bl_input_layer(self, spatial, coords, mode=3):
+        coords = np.ascontiguousarray(coords, dtype=np.int64)
+        c = _dev(coords, torch.int64)
+        n = C.c_int64(0)
+        _lib.check(self.L.scn_md_bl_input_layer(self.h, self._s(spatial), _ptr(c), coords.shape[0],
+                                                coords.shape[1], mode, _stream(), C.byref(n)))
+        return n.value
+
+    def bl_rules(self):
+        hdr = (C.c_int32 * 5)()
+        _lib.check(self.L.scn_md_bl_rules_header(self.h, hdr))
+        mode, max_active, _, _, n_out = [int(v) for v in hdr]
+        rows = torch.zeros((n_out, 1 + max_active), dtype=torch.int32, device="cuda")
+        if mode != 0 and n_out:
+            _lib.check(self.L.scn_md_input_rules(self.h, _ptr(rows), _stream()))
+        return np.array(list(hdr), np.int32), rows.cpu().numpy()
+
+    def bl_input_fwd(self, x):
+        hdr, _ = self.bl_rules()
+        xd = _dev(np.ascontiguousarray(x.reshape(-1, x.shape[-1])), torch.float32)
+        out = torch.full((int(hdr[4]), x.shape[-1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_input_layer_fwd(self.h, _ptr(xd), _ptr(out), x.shape[-1], _stream()))
+        return out.cpu().numpy()
+
+    def bl_output_fwd(self, x):
+        hdr, _ = self.bl_rules()
+        xd = _dev(x, torch.float32)
+        out = torch.full((int(hdr[2]), int(hdr[3]), x.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_output_layer_fwd(self.h, _ptr(xd), _ptr(out), x.shape[1], _stream()))
+        return out.cpu().numpy()
+
     def nactive(self, spatial):
         n = C.c_int64(0)
         _lib.check(self.L.scn_md_nactive(self.h, self._s(spatial), C.byref(n)))

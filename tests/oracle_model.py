@@ -24,6 +24,13 @@ def run(module, path, x):
         sp = _np(module.spatial_size)
         path.input_layer(sp, coords, 0 if len(x) == 2 else x[2], module.mode)
         return CpuTensor(path.input_fwd(feats), sp)
+    if isinstance(module, scn.BLInputLayer):
+        coords, feats = _np(x[0]), _np(x[1]).astype(np.float32)
+        sp = _np(module.spatial_size)
+        path.bl_input_layer(sp, coords, module.mode)
+        return CpuTensor(path.bl_input_fwd(feats), sp)
+    if isinstance(module, scn.BLOutputLayer):
+        return path.bl_output_fwd(x.features)
     if isinstance(module, scn.OutputLayer):
         return path.output_fwd(x.features)
     if isinstance(module, scn.SubmanifoldConvolution):

@@ -22,7 +22,7 @@ def test_exports():
                  "BatchNormalization", "BatchNormReLU", "BatchNormLeakyReLU", "MaxPooling", "InputLayer",
                  "OutputLayer", "SparseToDense", "Metadata", "SparseConvNetTensor", "Sequential", "ConcatTable",
                  "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor",
-                 "NetworkInNetwork", "AveragePooling", "UnPooling"]:
+                 "NetworkInNetwork", "AveragePooling", "UnPooling", "BLInputLayer", "BLOutputLayer"]:
         assert hasattr(scn, name), name
     assert scn.forward_pass_multiplyAdd_count == 0 and scn.forward_pass_hidden_states == 0
 

@@ -125,6 +125,23 @@ def test_average_and_unpooling_modules_vs_oracle(oracle_built):
                         want.features[rows(p.spatial_locations(15))], "pooling network")
 
 
+def test_bl_layers_network_vs_oracle(oracle_built):
+    """BLInputLayer (mode 4, with empty positions) -> convolutions -> BLOutputLayer."""
+    torch.manual_seed(8)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(2, 4, 8, 3, True)).add(scn.BatchNormReLU(8)).add(
+        scn.SubmanifoldConvolution(2, 8, 6, 3, False)).add(scn.BLOutputLayer(2)).eval()
+    randomise_bn(model, 8)
+    rng = np.random.default_rng(8)
+    coords = rng.integers(0, 24, (5, 200, 2)).astype(np.int64)
+    coords[rng.random((5, 200)) < 0.15] = -1
+    feats = rng.normal(size=(5, 200, 4)).astype(np.float32)
+    inp_layer = scn.BLInputLayer(2, 24, mode=4)
+    got, want, p = _run_both(model, inp_layer, [torch.as_tensor(coords), torch.as_tensor(feats)])
+    assert tuple(got.shape) == (5, 200, 6)
+    checks.assert_close(got.cpu().numpy(), want, "batch-by-length network")
+    assert (got.cpu().numpy()[coords[:, :, 0] < 0] == 0).all()
+
+
 def test_vgg2d_vs_oracle(oracle_built):
     torch.manual_seed(2)
     model = hello_world_model().eval()

@@ -33,6 +33,18 @@ def test_input_layer_no_batch_column(make):
     checks.check_input_layer(make, 2, 0, seed=6, with_batch_col=False)
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dim", [2, 3])
+def test_bl_input_layer(make, dim, mode):
+    checks.check_bl_input_layer(make, dim, mode, seed=20 * dim + mode)
+
+
+def test_bl_input_layer_edge_cases(make):
+    checks.check_bl_input_layer(make, 3, 3, seed=1, empties=False)
+    checks.check_bl_input_layer(make, 1, 4, seed=2, batch=1, length=300, spatial=40)
+    checks.check_bl_input_layer(make, 2, 1, seed=3, batch=5, length=1)
+
+
 @pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (2, (3, 1)), (3, (1, 3, 5)), (3, 2),
                                       (4, 3)])
 def test_submanifold(make, dim, size):
