@@ -21,7 +21,7 @@ from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, Bat
 from .metadata import Metadata  # noqa: E402
 from .networks import SparseVggNet, UNet  # noqa: E402
 from .tensor import SparseConvNetTensor  # noqa: E402
-from .utils import optionalTensor, toLongTensor  # noqa: E402
+from .utils import optionalTensor, prepare_BLInput, toLongTensor  # noqa: E402
 
 
 def is_hip_build():

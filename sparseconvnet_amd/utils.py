@@ -23,3 +23,18 @@ def optionalTensor(module, name):
 
 def optionalTensorReturn(a):
     return a if a.numel() else None
+
+
+def prepare_BLInput(batch):
+    """utils.py:127-136: pads a list of (locations [n_i, d], features [n_i, planes]) samples
+    to one [batch, max n_i, d] location tensor (filled up with -1 = empty) and one
+    [batch, max n_i, planes] feature tensor (filled up with zeros) for BLInputLayer."""
+    with torch.no_grad():
+        longest = max(loc.size(0) for loc, _ in batch)
+        loc0, feat0 = batch[0]
+        locations = torch.full((len(batch), longest, loc0.size(1)), -1, dtype=torch.int64)
+        features = torch.zeros(len(batch), longest, feat0.size(1))
+        for i, (loc, feat) in enumerate(batch):
+            locations[i, :loc.size(0)] = loc
+            features[i, :feat.size(0)] = feat
+    return [locations, features]

@@ -51,6 +51,17 @@ def test_hello_world_shape():
         out = model(inp)
     assert tuple(out.shape) == (2, 32, 10, 10) and out.is_cuda
     assert torch.isfinite(out).all() and (out >= 0).all() and out.abs().sum() > 0
+    # "Alternatively" (examples/hello-world.py:72-92): the same batch through BLInputLayer
+    batch = []
+    for b in range(2):
+        sel = [i for i, l in enumerate(loc) if l[2] == b]
+        batch.append([torch.LongTensor([loc[i][:2] for i in sel]), torch.FloatTensor([feat[i] for i in sel])])
+    batch = scn.prepare_BLInput(batch)
+    assert tuple(batch[0].shape) == (2, max(sum(l[2] == b for l in loc) for b in range(2)), 2)
+    batch[1] = batch[1].cuda()
+    with torch.no_grad():
+        out_bl = model(scn.BLInputLayer(2, size)(batch))
+    assert torch.allclose(out_bl, out, rtol=1e-4, atol=1e-5)
 
 
 def _run_both(model, inp_layer, x):
