@@ -264,6 +264,7 @@ def main():
     ap.add_argument("--pairs", default="")
     ap.add_argument("--no-unet", action="store_true")
     ap.add_argument("--no-ops", action="store_true")
+    ap.add_argument("--no-bf16", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times, to scale profiler byte counters")
     ap.add_argument("--unet-sites", type=int, default=1000000)
@@ -366,6 +367,30 @@ def main():
         "rulebook_sites_per_s": round(n / (rulebook_ms * 1e-3)),
         "roofline": roof, "sweep": sweep,
     }
+    if not args.no_bf16:
+        # Optional reduced-precision path (bf16 operands, fp32 accumulation), same work, listed
+        # beside the fp32 sweep; `value` and `roofline` above are fp32 only.
+        _lib.check(L.scn_md_set_bf16(h, 1))
+        wide = [(i, wk) for i, wk in enumerate(work) if wk[0] >= 64]
+        for _, wk in wide:
+            conv(*wk)
+        torch.cuda.synchronize()
+        bf = []
+        for i, wk in wide:
+            t = []
+            for _ in range(max(2, min(args.steps, 5))):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                conv(*wk)
+                e1.record()
+                torch.cuda.synchronize()
+                t.append(e0.elapsed_time(e1))
+            ms = float(np.mean(t))
+            bf.append({"nIn": wk[0], "nOut": wk[1], "ms": round(ms, 4),
+                       "gflops": round(2.0 * R * wk[0] * wk[1] / (ms * 1e-3) / 1e9, 1),
+                       "speedup_vs_f32": round(per_pair_ms[i] / ms, 2)})
+        out["sweep_bf16"] = bf
+        _lib.check(L.scn_md_set_bf16(h, 0))
     L.scn_md_destroy(h)
     del work
     if args.calibrate_copy:
@@ -380,6 +405,12 @@ def main():
     if not args.no_unet:
         out["unet"] = unet_scene(args.unet_sites, 5000)
         out["unet"].update(unet_scene(args.unet_sites, 5000, residual=True))
+        if not args.no_bf16:
+            import sparseconvnet_amd as scn
+            scn.bf16_mfma = True
+            u = unet_scene(args.unet_sites, 5000)
+            scn.bf16_mfma = False
+            out["unet"].update({"unet_bf16_ms_per_scene": u["unet_ms_per_scene"], "unet_bf16_warm_ms": u["unet_warm_ms"]})
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sites, args.seed)
     print(json.dumps(out))

@@ -48,6 +48,14 @@ void scn_md_destroy(scn_metadata *md);
 /* Metadata::clear (Metadata/Metadata.cpp:52-66). */
 int scn_md_clear(scn_metadata *md);
 
+/* Optional reduced-precision path (no counterpart in the reference, which computes in fp32
+ * throughout): with enable != 0 the convolutions of this handle whose input rows consist of
+ * whole 32-channel slabs and that run in the two wide kernel families (more than 32 output
+ * planes, or 128 and more input planes) round input rows and weights to bf16 (nearest even)
+ * and use the bf16 MFMA with fp32 accumulation; outputs, batch norms and everything else stay
+ * fp32.  Results then agree with the fp32 path to about 1e-2 relative to the output scale.
+ * Off by default. */
+int scn_md_set_bf16(scn_metadata *md, int enable);
 /* Metadata::inputLayer (Metadata/Metadata.cpp:413-425, Metadata/IOLayersRules.h:18-121).
  * coords: device int64 [n, ncols], ncols = dim (one sample) or dim+1 (last column = sample
  * index).  mode 0: rows = input order, no merging; 1: first, 2: last, 3: sum, 4: mean of the

@@ -12,6 +12,10 @@ forward_pass_hidden_states = 0
 # convolution to that convolution (one pass over the rows instead of two).  False: run
 # every module as a pass of its own.
 fuse_batchnorm = True
+# True: every Metadata created from now on runs its wide convolutions (more than 32 output
+# planes, or 128 and more input planes) with bf16 operands and fp32 accumulation.  The
+# reference computes in fp32 throughout, which is also the default here.
+bf16_mfma = False
 
 from .containers import AddTable, ConcatTable, JoinTable, Sequential  # noqa: E402
 from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, BatchNormReLU,  # noqa: E402

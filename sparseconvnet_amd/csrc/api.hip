@@ -125,6 +125,9 @@ int scn_md_clear(scn_metadata *h) {
   });
 }
 
+int scn_md_set_bf16(scn_metadata *h, int enable) {
+  return guarded([&] { md(h).bf16 = enable != 0; });
+}
 int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *coords, int64_t n,
                        int ncols, int min_batch, int mode, void *stream, int64_t *n_active) {
   return guarded([&] {

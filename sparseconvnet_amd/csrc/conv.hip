@@ -23,6 +23,14 @@
 namespace scn {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+// Four bf16 values in two registers: the A / B operand of v_mfma_f32_16x16x16_bf16, which
+// contracts the 16 channels that four fp32 MFMAs (16x16x4) take one after the other.  A lane
+// holds the same four consecutive channels in both layouts, so the reduced-precision kernels
+// differ from the fp32 ones only in a conversion (round to nearest even) where operands enter
+// LDS or the A registers, and in one MFMA instead of four.
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+__device__ inline v4s to_bf16x4(v4f v) { return __builtin_bit_cast(v4s, __builtin_convertvector(v, v4bf)); }
 
 // Optional pre-activation of the gathered input values (eval batch norm + leaky ReLU of the
 // layer in front, CPU/BatchNormalization.cpp:41-61, fused into the gather): y = x*sc + sh,
@@ -172,7 +180,7 @@ __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows
 // load of the pipeline is unconditional (granules without the tap and absent rows read
 // row 0 and are zeroed by a select), so the count of loads in flight is a compile-time
 // constant and the compiler can wait for exactly the loads it needs.
-template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF>
+template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF, bool BF16>
 __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
@@ -180,6 +188,8 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || (VEC4 && !PRE), "buffer gathers: float4 rows, no pre-activation");
+  static_assert(!BF16 || BUF, "the bf16 variant exists for buffer gathers only");
+  using OP = typename std::conditional<BF16, v4s, v4f>::type;  // an MFMA operand as LDS holds it
   constexpr int WR = 4 / WC;
   constexpr int NCB = NCBW * WC;
   constexpr int G = GW * WR;
@@ -306,7 +316,12 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     v4f *wb = wbuf + (it & 1) * SLAB_STRIDE_F4;
     v4f *ab = abuf + (it & 1) * (NFRAG * 64);
 #pragma unroll
-    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * 256] = wreg[i];
+    for (int i = 0; i < WPT; i++) {
+      if constexpr (BF16)
+        reinterpret_cast<v4s *>(wb)[threadIdx.x + i * 256] = to_bf16x4(wreg[i]);
+      else
+        wb[threadIdx.x + i * 256] = wreg[i];
+    }
     // Absent rows and channels past nIn become zeros on their way into LDS.
 #pragma unroll
     for (int i = 0; i < FPW; i++) {
@@ -323,7 +338,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
         if (!(ok && c0 + 2 < n_in)) v.z = 0.f;
         if (!(ok && c0 + 3 < n_in)) v.w = 0.f;
       }
-      ab[f * 64 + lane] = v;
+      if constexpr (BF16)
+        reinterpret_cast<v4s *>(ab)[f * 64 + lane] = to_bf16x4(v);
+      else
+        ab[f * 64 + lane] = v;
     }
     gm_cur = gm_nxt;
     // After this barrier the buffers of `it` are visible, and every wavefront has finished
@@ -331,33 +349,40 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     __syncthreads();
     if (it + 1 < total) issue(it + 1);
 
-    v4f b[SS][NCBW];
+    OP b[SS][NCBW];
 #pragma unroll
     for (int s = 0; s < SS; s++)
 #pragma unroll
-      for (int c = 0; c < NCBW; c++) b[s][c] = wb[(s * NCB + wc * NCBW + c) * 64 + lane];
+      for (int c = 0; c < NCBW; c++)
+        b[s][c] = reinterpret_cast<const OP *>(wb)[(s * NCB + wc * NCBW + c) * 64 + lane];
     // all A fragments of this wavefront's granules are fetched before the first MFMA, so that
     // no MFMA waits on LDS
-    v4f afrag[GW][SS];
+    OP afrag[GW][SS];
 #pragma unroll
     for (int q = 0; q < GW; q++)
 #pragma unroll
-      for (int s = 0; s < SS; s++) afrag[q][s] = ab[((wr * GW + q) * SS + s) * 64 + lane];
+      for (int s = 0; s < SS; s++) afrag[q][s] = reinterpret_cast<const OP *>(ab)[((wr * GW + q) * SS + s) * 64 + lane];
 #pragma unroll
     for (int q = 0; q < GW; q++) {
       const int gr = wr * GW + q;
       if (!((gm_cur >> gr) & 1u)) continue;  // uniform over the workgroup
 #pragma unroll
       for (int s = 0; s < SS; s++) {
-        const v4f av = afrag[q][s];
+        if constexpr (BF16) {
 #pragma unroll
-        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][c].x, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++)
+            acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(afrag[q][s], b[s][c], acc[q][c], 0, 0, 0);
+        } else {
+          const v4f av = afrag[q][s];
 #pragma unroll
-        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][c].y, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][c].x, acc[q][c], 0, 0, 0);
 #pragma unroll
-        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][c].z, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][c].y, acc[q][c], 0, 0, 0);
 #pragma unroll
-        for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][c].w, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][c].z, acc[q][c], 0, 0, 0);
+#pragma unroll
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][c].w, acc[q][c], 0, 0, 0);
+        }
       }
     }
   }
@@ -421,13 +446,16 @@ struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
   float leak = 1.0f;
 };
 
-template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF = false>
+template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF = false, bool BF16 = false>
 static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   if constexpr (VEC4 && !PRE && !BUF) {
     if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
-        m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24))
+        m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24)) {
+      if (m.bf16 && n_in >= 32)
+        return launch_mfma<NCBW, WC, GW, SS, VEC4, PRE, true, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
       return launch_mfma<NCBW, WC, GW, SS, VEC4, PRE, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+    }
   }
   constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
   constexpr int WPT = (SS * NCB * 64 + 255) / 256;
@@ -442,7 +470,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE, take_jobs(m));
   LAUNCH_CHECK();
-  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE, BUF>;
+  auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE, BUF, BF16>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -503,7 +531,7 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
 // granules' [16 x nOut] accumulators in registers.  Compared with k_conv_mfma the gathered
 // rows never touch LDS and one weight slab serves NW*RG*16 rows (up to 512), at the price of
 // uneven MFMA work between wavefronts, which three to four wavefronts per SIMD even out.
-template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF>
+template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF, bool BF16>
 __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
@@ -511,6 +539,8 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
+  static_assert(!BF16 || BUF, "the bf16 variant exists for buffer gathers only");
+  using OP = typename std::conditional<BF16, v4s, v4f>::type;  // an MFMA operand
   constexpr int NT = NW * 64;
   constexpr int G = NW * RG;
   constexpr int TM = G * 16;
@@ -568,7 +598,8 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   v4f wreg[WPT];
-  v4f a_nxt[RG][SS], a_cur[RG][SS];
+  v4f a_nxt[RG][SS];
+  OP a_cur[RG][SS];
   v4f psc[SS], psh[SS];
   unsigned gm_nxt = 0, gm_cur = 0, ok_nxt = 0;
   int sl_nxt = 0;
@@ -641,32 +672,48 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   for (int it = 0; it < total; it++) {
     v4f *wb = wbuf + (it & 1) * LDS_SLAB_F4;
 #pragma unroll
-    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * NT] = wreg[i];
+    for (int i = 0; i < WPT; i++) {
+      if constexpr (BF16)
+        reinterpret_cast<v4s *>(wb)[threadIdx.x + i * NT] = to_bf16x4(wreg[i]);
+      else
+        wb[threadIdx.x + i * NT] = wreg[i];
+    }
 #pragma unroll
     for (int q = 0; q < RG; q++) {
       const bool ok = (ok_nxt >> q) & 1u;
 #pragma unroll
       for (int s = 0; s < SS; s++) {
-        if constexpr (BUF && !PRE) {
+        if constexpr (BF16) {
+          v4f v = a_nxt[q][s];
+          if constexpr (PRE) {
+            v = pre_act<PRE>(v, psc[s], psh[s], pre_leak);
+            v = ok ? v : (v4f){0.f, 0.f, 0.f, 0.f};
+          }
+          a_cur[q][s] = to_bf16x4(v);
+          continue;
+        }
+        if constexpr (BUF && !PRE && !BF16) {
           a_cur[q][s] = a_nxt[q][s];
           continue;
         }
-        if constexpr (BUF && PRE) {
+        if constexpr (BUF && PRE && !BF16) {
           const v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
           a_cur[q][s] = ok ? v : (v4f){0.f, 0.f, 0.f, 0.f};
           continue;
         }
-        const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
-        v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
-        if (VEC4) {
-          if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
-        } else {
-          if (!(ok && c0 + 0 < n_in)) v.x = 0.f;
-          if (!(ok && c0 + 1 < n_in)) v.y = 0.f;
-          if (!(ok && c0 + 2 < n_in)) v.z = 0.f;
-          if (!(ok && c0 + 3 < n_in)) v.w = 0.f;
+        if constexpr (!BUF) {
+          const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
+          v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
+          if (VEC4) {
+            if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
+          } else {
+            if (!(ok && c0 + 0 < n_in)) v.x = 0.f;
+            if (!(ok && c0 + 1 < n_in)) v.y = 0.f;
+            if (!(ok && c0 + 2 < n_in)) v.z = 0.f;
+            if (!(ok && c0 + 3 < n_in)) v.w = 0.f;
+          }
+          a_cur[q][s] = v;
         }
-        a_cur[q][s] = v;
       }
     }
     gm_cur = gm_nxt;
@@ -675,21 +722,27 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     if (((gm_cur >> (wave * RG)) & ((1u << RG) - 1u)) == 0u) continue;  // none of my granules has the tap
 #pragma unroll
     for (int s = 0; s < SS; s++) {
-      v4f b[NCB];
+      OP b[NCB];
 #pragma unroll
-      for (int cb = 0; cb < NCB; cb++) b[cb] = wb[(s * NCB + cb) * 64 + lane];
+      for (int cb = 0; cb < NCB; cb++) b[cb] = reinterpret_cast<const OP *>(wb)[(s * NCB + cb) * 64 + lane];
 #pragma unroll
       for (int q = 0; q < RG; q++) {
         if (!((gm_cur >> (wave * RG + q)) & 1u)) continue;  // uniform over the wavefront
-        const v4f av = a_cur[q][s];
+        if constexpr (BF16) {
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[cb].x, acc[q][cb], 0, 0, 0);
+          for (int cb = 0; cb < NCB; cb++)
+            acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_cur[q][s], b[cb], acc[q][cb], 0, 0, 0);
+        } else {
+          const v4f av = a_cur[q][s];
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[cb].y, acc[q][cb], 0, 0, 0);
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[cb].x, acc[q][cb], 0, 0, 0);
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[cb].z, acc[q][cb], 0, 0, 0);
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[cb].y, acc[q][cb], 0, 0, 0);
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[cb].w, acc[q][cb], 0, 0, 0);
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[cb].z, acc[q][cb], 0, 0, 0);
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[cb].w, acc[q][cb], 0, 0, 0);
+        }
       }
     }
   }
@@ -733,15 +786,18 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   }
 }
 
-template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF = false>
+template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF = false, bool BF16 = false>
 static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   if constexpr (VEC4 && !BUF) {
     // gathers through buffer loads (no per-element selects, 32-bit addressing) when the input
     // is below 2 GiB and 2^24 rows and consists of whole slabs
     if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
-        m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24))
+        m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24)) {
+      if (m.bf16)
+        return launch_rows<NCB, RG, SS, VEC4, NW, PRE, true, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
       return launch_rows<NCB, RG, SS, VEC4, NW, PRE, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+    }
   }
   constexpr int NT = NW * 64, G = NW * RG;
   constexpr int SLAB_F4 = SS * NCB * 64;
@@ -756,7 +812,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE, take_jobs(m));
   LAUNCH_CHECK();
-  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE, BUF>;
+  auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE, BUF, BF16>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -135,6 +135,10 @@ struct Metadata {
   DevBuf<float> postbuf;  // scale / shift of a batch norm fused into the running convolution's stores
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
   DevBuf<float> bntmp;    // normalised input when a fused batch norm has no fused kernel
+  // The row-owner and LDS-tiled convolution kernels (more than 32 output planes, or wide
+  // inputs) round their operands to bf16 and run the bf16 MFMA with fp32 accumulation when the
+  // input consists of whole 32-channel slabs; off unless the caller asks for it.
+  bool bf16 = false;
 };
 
 SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);

@@ -218,9 +218,10 @@ __global__ void k_finish_groups(const int *sidx, const int *head, const int *hea
       run_len[row] = len;
     }
   }
-  // longest run: one atomic per wavefront, and only when it can raise the maximum
+  // longest run: one atomic per wavefront, and only when it can raise the maximum (the plain
+  // read may be stale, which only costs an atomic that changes nothing)
   for (int off = 32; off; off >>= 1) len = max(len, __shfl_xor(len, off));
-  if ((threadIdx.x & 63) == 0 && len > 1) atomicMax(max_active, len);
+  if ((threadIdx.x & 63) == 0 && len > 1 && len > __builtin_nontemporal_load(max_active)) atomicMax(max_active, len);
 }
 
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,

@@ -60,6 +60,14 @@ class Metadata:
         if not self._h:
             raise _lib.ScnError(self._L.scn_last_error().decode())
         mac_counter.live.add(self)
+        import sparseconvnet_amd
+        if getattr(sparseconvnet_amd, "bf16_mfma", False):
+            self.setBf16(True)
+
+    def setBf16(self, enable):
+        """Wide convolutions of this Metadata round their operands to bf16 and accumulate in
+        fp32 (about 1e-2 relative to the output scale); everything else stays fp32."""
+        _lib.check(self._L.scn_md_set_bf16(self._h, 1 if enable else 0))
 
     def __del__(self):
         h = getattr(self, "_h", None)

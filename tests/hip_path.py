@@ -29,6 +29,9 @@ class HipPath:
         if not self.h:
             raise _lib.ScnError(self.L.scn_last_error().decode())
 
+    def set_bf16(self, enable=True):
+        _lib.check(self.L.scn_md_set_bf16(self.h, 1 if enable else 0))
+
     def __del__(self):
         if getattr(self, "h", None):
             self.L.scn_md_destroy(self.h)

@@ -219,6 +219,53 @@ def _neighbour_counts(coords, spatial):
     return present
 
 
+@pytest.mark.parametrize("cin,cout", [(64, 64), (64, 32), (128, 128), (96, 160), (256, 256), (128, 32)])
+def test_bf16_path_vs_oracle(oracle_built, cin, cout):
+    """The optional bf16-operand path: submanifold convolution (with and without a batch norm
+    in front), strided convolution and deconvolution against the fp32 oracle, within 1e-2 of
+    the output scale; the fp32 path on the same handle stays within its own tolerance."""
+    hp, op = _both(3, oracle_built)
+    hp.set_bf16(True)
+    rng = np.random.default_rng(cin * 7 + cout)
+    coords = synthetic.scene_batch(seed=8000 + cin, batch=2, target=4000, spatial=64, n_boxes=8)
+    for p in (hp, op):
+        p.input_layer(64, coords, 0, 3)
+    x = rng.normal(size=(len(coords), cin)).astype(np.float32)
+    xo, xh = op.input_fwd(x), hp.input_fwd(x)
+    ro, rh = canon_rows(op.spatial_locations(64)), canon_rows(hp.spatial_locations(64))
+
+    def close(got, want, what):
+        scale = float(np.abs(want).max())
+        err = float(np.abs(got - want).max())
+        assert err <= 1e-2 * scale, "%s: max err %g against scale %g" % (what, err, scale)
+        assert err > 0  # the reduced-precision kernels did run
+
+    w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
+    yo, _ = op.subm_conv(64, 3, xo, w)
+    yh, _ = hp.subm_conv(64, 3, xh, w)
+    close(yh[rh], yo[ro], "submanifold")
+    bn = dict(mean=rng.normal(size=cin).astype(np.float32), var=rng.uniform(0.5, 1.5, cin).astype(np.float32),
+              weight=rng.normal(size=cin).astype(np.float32), bias=rng.normal(size=cin).astype(np.float32),
+              eps=1e-4, leakiness=0.0)
+    xb = op.bn_eval(xo, bn["mean"], bn["var"], bn["weight"], bn["bias"], 1e-4, 0.0)
+    yo, _ = op.subm_conv(64, 3, xb, w)
+    yh, _ = hp.subm_conv(64, 3, xh, w, bn=bn)
+    close(yh[rh], yo[ro], "batch norm + submanifold")
+    w2 = (rng.normal(size=(8, 1, cin, cout)) * (2.0 / (cin * 8)) ** 0.5).astype(np.float32)
+    co, _ = op.conv(64, 32, 2, 2, xo, w2)
+    ch, _ = hp.conv(64, 32, 2, 2, xh, w2)
+    r1o, r1h = canon_rows(op.spatial_locations(32)), canon_rows(hp.spatial_locations(32))
+    close(ch[r1h], co[r1o], "strided")
+    w3 = (rng.normal(size=(8, 1, cout, cin)) * (2.0 / (cout * 8)) ** 0.5).astype(np.float32)
+    do, _ = op.deconv(32, 64, 2, 2, co, w3)
+    dh, _ = hp.deconv(32, 64, 2, 2, co[r1o][np.argsort(r1h)], w3)
+    close(dh[rh], do[ro], "transposed")
+    hp.set_bf16(False)
+    yo, _ = op.subm_conv(64, 3, xo, w)
+    yh, _ = hp.subm_conv(64, 3, xh, w)
+    checks.assert_close(yh[rh], yo[ro], "fp32 again")
+
+
 def test_full_size_sweep_scene_properties():
     """Configuration 3 at its full size (one room scene of 1,000,000 sites in 4096^3, the
     bench workload), through properties that do not need the oracle to finish: the rule count
