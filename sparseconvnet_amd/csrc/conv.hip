@@ -30,11 +30,21 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // LDS or the A registers, and in one MFMA instead of four.
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 __device__ inline v4s to_bf16x4(v4f v) { return __builtin_bit_cast(v4s, __builtin_convertvector(v, v4bf)); }
+// The bf16 kernels take two 16-channel steps per v_mfma_f32_16x16x32_bf16: lane group g
+// contributes its four channels of either step (the instruction sums over all 32 (lane group,
+// element) pairs, in whatever order A and B agree on).  Operands of a pair of steps are kept
+// next to each other (16 bytes per lane) in LDS and in the packed weights, so that they
+// arrive in the four consecutive registers the instruction wants.
+__device__ inline v8s to_bf16x8(v4f lo, v4f hi) {
+  return __builtin_shufflevector(to_bf16x4(lo), to_bf16x4(hi), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+__device__ inline v4f mfma_bf16(v8s a, v8s b, v4f acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), acc, 0, 0, 0);
+}
 
-// Optional pre-activation of the gathered input values (eval batch norm + leaky ReLU of the
-// layer in front, CPU/BatchNormalization.cpp:41-61, fused into the gather): y = x*sc + sh,
-// y *= (y > 0 ? 1 : leak).  sc / sh are per input channel, zero-padded to a multiple of 64.
 template <bool PRE> __device__ inline v4f pre_act(v4f v, v4f sc, v4f sh, float leak) {
   if (!PRE) return v;
   v4f y = v * sc + sh;
@@ -110,6 +120,10 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
   out[row * n_out + oc] = acc;
 }
 
+// Elements of one packed weight slab (SS steps of 16 channels by NCB column blocks), padded to
+// a multiple of 256 lanes' worth so that a workgroup stages it without bounds checks.
+constexpr int packed_slab_floats(int SS, int NCB) { return (SS * NCB * 64 + 255) / 256 * 256 * 4; }
+
 // ---- weight packing ---------------------------------------------------------------------
 // wp[k][slab][e], e < SLAB_STRIDE (floats), with for e = ((s*NCB + cb)*64 + lane)*4 + jj
 //   wp = W[k][channel (slab*SS+s)*16 + 4*(lane/16) + jj][16*cb + lane%16]
@@ -117,8 +131,10 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
 // lane `lane` of a wavefront consumes B operands, so that staging a slab into LDS is a
 // straight copy and each lane reads the four operands of one 16-channel step with a single
 // 16-byte LDS load.
+// as_bf16 (SS even): 2-byte elements rounded to nearest even, the two steps of a pair next to
+// each other: e = (((sp*NCB + cb)*64 + lane)*2 + s%2)*4 + jj with sp = s/2.
 __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n_out, int n_slab, int SS,
-                               int NCB, int slab_stride, CoefJobs jobs) {
+                               int NCB, int slab_stride, CoefJobs jobs, bool as_bf16 = false) {
   coef_jobs(jobs);
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = (int64_t)K * n_slab * slab_stride;
@@ -134,11 +150,20 @@ __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n
     int q = e >> 8;
     int cb = q % NCB;
     int s = q / NCB;
+    if (as_bf16) {
+      lane = (e >> 3) & 63;
+      q = e >> 9;
+      cb = q % NCB;
+      s = 2 * (q / NCB) + ((e >> 2) & 1);
+    }
     int ch = (sl * SS + s) * 16 + 4 * (lane >> 4) + jj;
     int col = 16 * cb + (lane & 15);
     if (ch < n_in && col < n_out) v = w[((int64_t)k * n_in + ch) * n_out + col];
   }
-  wp[i] = v;
+  if (as_bf16)
+    reinterpret_cast<__bf16 *>(wp)[i] = (__bf16)v;
+  else
+    wp[i] = v;
 }
 
 // Packs rows [0, n_in_part) of every tap's weight slice, where the slice of tap k starts at
@@ -188,22 +213,26 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || (VEC4 && !PRE), "buffer gathers: float4 rows, no pre-activation");
-  static_assert(!BF16 || BUF, "the bf16 variant exists for buffer gathers only");
-  using OP = typename std::conditional<BF16, v4s, v4f>::type;  // an MFMA operand as LDS holds it
+  static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int WR = 4 / WC;
   constexpr int NCB = NCBW * WC;
   constexpr int G = GW * WR;
   constexpr int TM = G * 16;
-  constexpr int SLAB_F4 = SS * NCB * 64;      // float4 of one weight slab
-  constexpr int WPT = (SLAB_F4 + 255) / 256;  // float4 staged per thread
-  constexpr int SLAB_STRIDE_F4 = WPT * 256;   // padded slab, in global memory and LDS
+  // An operand is what one lane feeds one MFMA with: 16 bytes, either four fp32 channels of
+  // one 16-channel step or four bf16 channels of each step of a pair.
+  constexpr int WS = BF16 ? SS / 2 : SS;      // operands per slab, column block and lane
+  constexpr int SLAB_F4 = WS * NCB * 64;      // operands of one weight slab
+  constexpr int WPT = (SLAB_F4 + 255) / 256;  // operands staged per thread
+  constexpr int LDS_SLAB_F4 = WPT * 256;      // slab in LDS
+  constexpr int SLAB_STRIDE_F4 = packed_slab_floats(SS, NCB) / (BF16 ? 8 : 4);  // slab in global memory
   constexpr int NFRAG = G * SS;               // A fragments (granule, step) per iteration
   constexpr int FPW = NFRAG / 4;              // fragments gathered per wavefront
+  constexpr int A_F4 = G * WS * 64;           // A operands per iteration
   static_assert(NFRAG % 4 == 0, "fragments must divide over 4 wavefronts");
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  v4f *wbuf = reinterpret_cast<v4f *>(lds);   // [2][SLAB_STRIDE_F4]
-  v4f *abuf = wbuf + 2 * SLAB_STRIDE_F4;      // [2][NFRAG * 64]
-  int *jtab = reinterpret_cast<int *>(abuf + 2 * NFRAG * 64);  // [G][K][16]
+  v4f *wbuf = reinterpret_cast<v4f *>(lds);   // [2][LDS_SLAB_F4]
+  v4f *abuf = wbuf + 2 * LDS_SLAB_F4;         // [2][A_F4]
+  int *jtab = reinterpret_cast<int *>(abuf + 2 * A_F4);  // [G][K][16]
   unsigned *gmask = reinterpret_cast<unsigned *>(jtab + G * K * 16);  // [K] granules having tap k
   int *taplist = reinterpret_cast<int *>(gmask + K);           // [K]
   int *ntaps_p = taplist + K;                                  // [1]
@@ -279,7 +308,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     aok_nxt = 0;
     const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
 #pragma unroll
-    for (int i = 0; i < WPT; i++) wreg[i] = wsrc[threadIdx.x + i * 256];
+    for (int i = 0; i < WPT; i++) {
+      const int e = threadIdx.x + i * 256;
+      wreg[i] = wsrc[(SLAB_F4 % 256 == 0 || e < SLAB_F4) ? e : 0];
+    }
 #pragma unroll
     for (int i = 0; i < FPW; i++) {
       const int f = wave + 4 * i;  // fragment f = (granule f / SS, step f % SS)
@@ -313,15 +345,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 
   if (total > 0) issue(0);
   for (int it = 0; it < total; it++) {
-    v4f *wb = wbuf + (it & 1) * SLAB_STRIDE_F4;
-    v4f *ab = abuf + (it & 1) * (NFRAG * 64);
+    v4f *wb = wbuf + (it & 1) * LDS_SLAB_F4;
+    v4f *ab = abuf + (it & 1) * A_F4;
 #pragma unroll
-    for (int i = 0; i < WPT; i++) {
-      if constexpr (BF16)
-        reinterpret_cast<v4s *>(wb)[threadIdx.x + i * 256] = to_bf16x4(wreg[i]);
-      else
-        wb[threadIdx.x + i * 256] = wreg[i];
-    }
+    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * 256] = wreg[i];
     // Absent rows and channels past nIn become zeros on their way into LDS.
 #pragma unroll
     for (int i = 0; i < FPW; i++) {
@@ -338,8 +365,8 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
         if (!(ok && c0 + 2 < n_in)) v.z = 0.f;
         if (!(ok && c0 + 3 < n_in)) v.w = 0.f;
       }
-      if constexpr (BF16)
-        reinterpret_cast<v4s *>(ab)[f * 64 + lane] = to_bf16x4(v);
+      if constexpr (BF16)  // the half of the pair's operand that belongs to step f % SS
+        reinterpret_cast<v4s *>(ab)[(((f / SS) * WS + (f % SS) / 2) * 64 + lane) * 2 + (f & 1)] = to_bf16x4(v);
       else
         ab[f * 64 + lane] = v;
     }
@@ -349,29 +376,28 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     __syncthreads();
     if (it + 1 < total) issue(it + 1);
 
-    OP b[SS][NCBW];
+    v4f b[WS][NCBW];
 #pragma unroll
-    for (int s = 0; s < SS; s++)
+    for (int s = 0; s < WS; s++)
 #pragma unroll
-      for (int c = 0; c < NCBW; c++)
-        b[s][c] = reinterpret_cast<const OP *>(wb)[(s * NCB + wc * NCBW + c) * 64 + lane];
+      for (int c = 0; c < NCBW; c++) b[s][c] = wb[(s * NCB + wc * NCBW + c) * 64 + lane];
     // all A fragments of this wavefront's granules are fetched before the first MFMA, so that
     // no MFMA waits on LDS
-    OP afrag[GW][SS];
+    v4f afrag[GW][WS];
 #pragma unroll
     for (int q = 0; q < GW; q++)
 #pragma unroll
-      for (int s = 0; s < SS; s++) afrag[q][s] = reinterpret_cast<const OP *>(ab)[((wr * GW + q) * SS + s) * 64 + lane];
+      for (int s = 0; s < WS; s++) afrag[q][s] = ab[((wr * GW + q) * WS + s) * 64 + lane];
 #pragma unroll
     for (int q = 0; q < GW; q++) {
       const int gr = wr * GW + q;
       if (!((gm_cur >> gr) & 1u)) continue;  // uniform over the workgroup
 #pragma unroll
-      for (int s = 0; s < SS; s++) {
+      for (int s = 0; s < WS; s++) {
         if constexpr (BF16) {
 #pragma unroll
           for (int c = 0; c < NCBW; c++)
-            acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(afrag[q][s], b[s][c], acc[q][c], 0, 0, 0);
+            acc[q][c] = mfma_bf16(__builtin_bit_cast(v8s, afrag[q][s]), __builtin_bit_cast(v8s, b[s][c]), acc[q][c]);
         } else {
           const v4f av = afrag[q][s];
 #pragma unroll
@@ -452,15 +478,16 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   if constexpr (VEC4 && !PRE && !BUF) {
     if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
         m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24)) {
-      if (m.bf16 && n_in >= 32)
-        return launch_mfma<NCBW, WC, GW, SS, VEC4, PRE, true, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      if (m.bf16 && n_in % 32 == 0)  // half-size operands leave room for two steps per slab
+        return launch_mfma<NCBW, WC, GW, 2, VEC4, PRE, true, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
       return launch_mfma<NCBW, WC, GW, SS, VEC4, PRE, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     }
   }
   constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
-  constexpr int WPT = (SS * NCB * 64 + 255) / 256;
-  constexpr int SLAB_STRIDE = WPT * 256 * 4;  // floats
-  const size_t lds_bytes = (size_t)2 * SLAB_STRIDE * sizeof(float) + (size_t)2 * G * SS * 64 * 16 +
+  constexpr int WS = BF16 ? SS / 2 : SS;
+  constexpr int WPT = (WS * NCB * 64 + 255) / 256;
+  constexpr int SLAB_STRIDE = packed_slab_floats(SS, NCB);  // elements of a packed slab
+  const size_t lds_bytes = (size_t)2 * WPT * 256 * 16 + (size_t)2 * G * WS * 64 * 16 +
                            ((size_t)G * t.K * 16 + 2 * t.K + 4) * sizeof(int);
   if (lds_bytes > 160 * 1024) return false;
   const int cin16 = (int)ceil_div(n_in, 16);
@@ -468,7 +495,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
   m.wpack.reserve(packed);
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m));
+                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m), BF16);
   LAUNCH_CHECK();
   auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE, BUF, BF16>;
   static bool attr_set = false;
@@ -539,14 +566,14 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
-  static_assert(!BF16 || BUF, "the bf16 variant exists for buffer gathers only");
-  using OP = typename std::conditional<BF16, v4s, v4f>::type;  // an MFMA operand
+  static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int NT = NW * 64;
   constexpr int G = NW * RG;
   constexpr int TM = G * 16;
-  constexpr int SLAB_F4 = SS * NCB * 64;
+  constexpr int WS = BF16 ? SS / 2 : SS;  // 16-byte operands per slab, column block and lane (see k_conv_mfma)
+  constexpr int SLAB_F4 = WS * NCB * 64;
   constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
-  constexpr int SLAB_STRIDE_F4 = ((SLAB_F4 + 255) / 256) * 256;  // as packed by k_pack_weights
+  constexpr int SLAB_STRIDE_F4 = packed_slab_floats(SS, NCB) / (BF16 ? 8 : 4);  // as packed by k_pack_weights
   constexpr int LDS_SLAB_F4 = WPT * NT;                         // >= SLAB_STRIDE_F4 not required
   static_assert(G <= 32, "granule mask is 32 bits");
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -599,7 +626,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 
   v4f wreg[WPT];
   v4f a_nxt[RG][SS];
-  OP a_cur[RG][SS];
+  v4f a_cur[RG][WS];  // bf16: the eight values of a pair of steps
   v4f psc[SS], psh[SS];
   unsigned gm_nxt = 0, gm_cur = 0, ok_nxt = 0;
   int sl_nxt = 0;
@@ -672,26 +699,26 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   for (int it = 0; it < total; it++) {
     v4f *wb = wbuf + (it & 1) * LDS_SLAB_F4;
 #pragma unroll
-    for (int i = 0; i < WPT; i++) {
-      if constexpr (BF16)
-        reinterpret_cast<v4s *>(wb)[threadIdx.x + i * NT] = to_bf16x4(wreg[i]);
-      else
-        wb[threadIdx.x + i * NT] = wreg[i];
-    }
+    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * NT] = wreg[i];
 #pragma unroll
     for (int q = 0; q < RG; q++) {
       const bool ok = (ok_nxt >> q) & 1u;
+      if constexpr (BF16) {
+#pragma unroll
+        for (int s = 0; s < SS; s += 2) {
+          v4f v0 = a_nxt[q][s], v1 = a_nxt[q][s + 1];
+          if constexpr (PRE) {
+            v0 = pre_act<PRE>(v0, psc[s], psh[s], pre_leak);
+            v1 = pre_act<PRE>(v1, psc[s + 1], psh[s + 1], pre_leak);
+            v0 = ok ? v0 : (v4f){0.f, 0.f, 0.f, 0.f};
+            v1 = ok ? v1 : (v4f){0.f, 0.f, 0.f, 0.f};
+          }
+          a_cur[q][s / 2] = __builtin_bit_cast(v4f, to_bf16x8(v0, v1));
+        }
+        continue;
+      }
 #pragma unroll
       for (int s = 0; s < SS; s++) {
-        if constexpr (BF16) {
-          v4f v = a_nxt[q][s];
-          if constexpr (PRE) {
-            v = pre_act<PRE>(v, psc[s], psh[s], pre_leak);
-            v = ok ? v : (v4f){0.f, 0.f, 0.f, 0.f};
-          }
-          a_cur[q][s] = to_bf16x4(v);
-          continue;
-        }
         if constexpr (BUF && !PRE && !BF16) {
           a_cur[q][s] = a_nxt[q][s];
           continue;
@@ -721,17 +748,17 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     if (it + 1 < total) issue(it + 1);
     if (((gm_cur >> (wave * RG)) & ((1u << RG) - 1u)) == 0u) continue;  // none of my granules has the tap
 #pragma unroll
-    for (int s = 0; s < SS; s++) {
-      OP b[NCB];
+    for (int s = 0; s < WS; s++) {
+      v4f b[NCB];
 #pragma unroll
-      for (int cb = 0; cb < NCB; cb++) b[cb] = reinterpret_cast<const OP *>(wb)[(s * NCB + cb) * 64 + lane];
+      for (int cb = 0; cb < NCB; cb++) b[cb] = wb[(s * NCB + cb) * 64 + lane];
 #pragma unroll
       for (int q = 0; q < RG; q++) {
         if (!((gm_cur >> (wave * RG + q)) & 1u)) continue;  // uniform over the wavefront
         if constexpr (BF16) {
 #pragma unroll
           for (int cb = 0; cb < NCB; cb++)
-            acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_cur[q][s], b[cb], acc[q][cb], 0, 0, 0);
+            acc[q][cb] = mfma_bf16(__builtin_bit_cast(v8s, a_cur[q][s]), __builtin_bit_cast(v8s, b[cb]), acc[q][cb]);
         } else {
           const v4f av = a_cur[q][s];
 #pragma unroll
@@ -794,15 +821,17 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
     // is below 2 GiB and 2^24 rows and consists of whole slabs
     if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
         m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24)) {
-      if (m.bf16)
-        return launch_rows<NCB, RG, SS, VEC4, NW, PRE, true, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      if constexpr (SS % 2 == 0) {
+        if (m.bf16)
+          return launch_rows<NCB, RG, SS, VEC4, NW, PRE, true, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      }
       return launch_rows<NCB, RG, SS, VEC4, NW, PRE, true>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     }
   }
   constexpr int NT = NW * 64, G = NW * RG;
-  constexpr int SLAB_F4 = SS * NCB * 64;
+  constexpr int SLAB_F4 = (BF16 ? SS / 2 : SS) * NCB * 64;
   constexpr int WPT = (SLAB_F4 + NT - 1) / NT;
-  constexpr int SLAB_STRIDE = ((SLAB_F4 + 255) / 256) * 256 * 4;  // floats, as k_pack_weights lays slabs out
+  constexpr int SLAB_STRIDE = packed_slab_floats(SS, NCB);  // elements of a packed slab
   const size_t lds_bytes = (size_t)2 * WPT * NT * 16 + ((size_t)G * t.K * 16 + 2 * t.K + 4) * sizeof(int);
   if (lds_bytes > 160 * 1024) return false;
   const int cin16 = (int)ceil_div(n_in, 16);
@@ -810,7 +839,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
   m.wpack.reserve(packed);
   k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m));
+                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m), BF16);
   LAUNCH_CHECK();
   auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE, BUF, BF16>;
   static bool attr_set = false;
