@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
-  static_assert(!BUF || (VEC4 && !PRE), "buffer gathers: float4 rows, no pre-activation");
+  static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int WR = 4 / WC;
   constexpr int NCB = NCBW * WC;
@@ -320,6 +320,11 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       if constexpr (BUF) {
         const unsigned voff = j >= 0 ? __umul24((unsigned)j, row_bytes) + lane_off : 0x80000000u;
         areg[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, (sl * SS + s) * 64, 0));
+        if (PRE) {  // zero must stay zero through the pre-activation
+          if (j >= 0) aok_nxt |= 1u << i;
+          psc[i] = *reinterpret_cast<const v4f *>(pre_sc + (sl * SS + s) * 16 + 4 * g);
+          psh[i] = *reinterpret_cast<const v4f *>(pre_sh + (sl * SS + s) * 16 + 4 * g);
+        }
         continue;
       }
       if (j >= 0) aok_nxt |= 1u << i;
@@ -357,6 +362,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       const bool ok = (aok_nxt >> i) & 1u;
       v4f v = pre_act<PRE>(areg[i], psc[i], psh[i], pre_leak);
       if (BUF) {
+        if (PRE && !ok) v = (v4f){0.f, 0.f, 0.f, 0.f};
       } else if (VEC4) {
         if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
       } else {
@@ -475,7 +481,7 @@ struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
 template <int NCBW, int WC, int GW, int SS, bool VEC4, bool PRE, bool BUF = false, bool BF16 = false>
 static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                         Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
-  if constexpr (VEC4 && !PRE && !BUF) {
+  if constexpr (VEC4 && !BUF) {
     if (n_in % (16 * SS) == 0 && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) &&
         m.cur_in_rows * n_in * 4 < ((int64_t)1 << 31) && n_in * 4 < (1 << 24)) {
       if (m.bf16 && n_in % 32 == 0)  // half-size operands leave room for two steps per slab
@@ -1237,8 +1243,11 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
 // parts of 32 and has no fused batch norm, so from 128 input channels on, or from 64 when a
 // batch norm comes with the call or the filter has few taps, the row-owner kernel is at
 // least as fast (measured).
-static bool resident_fits(const Table &t, int n_in, int n_out, bool with_bn) {
+static bool resident_fits(const Metadata &m, const Table &t, int n_in, int n_out, bool with_bn) {
   if (!(t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr)) return false;
+  // the resident kernel computes in fp32 only; from two parts on the row-owner kernel's bf16
+  // variant is faster (measured)
+  if (m.bf16 && n_in >= 64 && n_in % 32 == 0) return false;
   // several parts re-read and re-write the output once per part: with few taps (strided and
   // transposed convolutions) that costs more than the convolution itself
   if (n_in > 32 && t.K <= 8) return false;
@@ -1250,7 +1259,7 @@ static bool resident_fits(const Table &t, int n_in, int n_out, bool with_bn) {
 // that reaches it) costs more than one extra pass over the rows.
 static bool try_resident(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                          Epi epi, int n_in, int n_out, hipStream_t s) {
-  if (!resident_fits(t, n_in, n_out, false)) return false;
+  if (!resident_fits(m, t, n_in, n_out, false)) return false;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   const int ncb = (int)ceil_div(n_out, 16);
   if (n_in <= 4) {
@@ -1352,7 +1361,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     epi.sh = m.postbuf.p + n_out;
     epi.leak = post->leak;
   }
-  if (bn && groups == 1 && !resident_fits(t, n_in, n_out, true)) {
+  if (bn && groups == 1 && !resident_fits(m, t, n_in, n_out, true)) {
     const int n_pad = (int)round_up(n_in, 64) + 64;
     m.prebuf.reserve(2 * (size_t)n_pad);
     m.jobs.pre = CoefJob{bn->mean, bn->var, bn->gamma, bn->beta, bn->eps, n_in, n_pad, m.prebuf.p,
