@@ -28,7 +28,7 @@ PAIRS = [(3, 32), (32, 32), (64, 64), (128, 128), (256, 256)]
 # HBM-side bytes per launch on the default workload (1,000,000 sites, seed 3000, shuffled), from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE passes scaled by a 1 GiB copy kernel (x2.000 / x1.000):
 # profiles/conv256_sweep1M_pmc.txt.  Only reported when the run is that workload.
-MEASURED_TRAFFIC = {(256, 256): 17.09e9, (128, 128): 3.69e9, (64, 64): 1.09e9, (32, 32): 0.430e9, (3, 32): 0.432e9}
+MEASURED_TRAFFIC = {(256, 256): 17.10e9, (128, 128): 3.71e9, (64, 64): 1.09e9, (32, 32): 0.429e9, (3, 32): 0.432e9}
 
 
 def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
@@ -265,6 +265,7 @@ def main():
     ap.add_argument("--no-unet", action="store_true")
     ap.add_argument("--no-ops", action="store_true")
     ap.add_argument("--no-bf16", action="store_true")
+    ap.add_argument("--no-residual", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times, to scale profiler byte counters")
     ap.add_argument("--unet-sites", type=int, default=1000000)
@@ -404,7 +405,8 @@ def main():
         out["other_ops"] = other_ops(args.unet_sites, 5000)
     if not args.no_unet:
         out["unet"] = unet_scene(args.unet_sites, 5000)
-        out["unet"].update(unet_scene(args.unet_sites, 5000, residual=True))
+        if not args.no_residual:
+            out["unet"].update(unet_scene(args.unet_sites, 5000, residual=True))
         if not args.no_bf16:
             import sparseconvnet_amd as scn
             scn.bf16_mfma = True
