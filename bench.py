@@ -259,7 +259,7 @@ def main():
     ap.add_argument("--sites", type=int, default=1000000)
     ap.add_argument("--seed", type=int, default=3000)
     ap.add_argument("--order", default="shuffled", choices=["shuffled", "scan"])
-    ap.add_argument("--cpu-sites", type=int, default=200000)
+    ap.add_argument("--cpu-sites", type=int, default=1000000)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pairs", default="")
     ap.add_argument("--no-unet", action="store_true")
