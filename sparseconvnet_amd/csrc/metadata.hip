@@ -77,8 +77,23 @@ __global__ void k_fill32(uint32_t *p, uint32_t v, int64_t n) {
   int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) p[i] = v;
 }
+// 16 bytes per store: p is 16-byte aligned, n4 counts groups of four words
+__global__ void k_fill128(uint4 *p, uint32_t v, int64_t n4) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const uint4 vv = make_uint4(v, v, v, v);
+  for (; i < n4; i += stride) p[i] = vv;
+}
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s) {
   if (n <= 0) return;
+  if (n >= 4096 && (uintptr_t)p % 16 == 0) {  // large fills: wide stores, the tail word by word
+    const int64_t n4 = n / 4;
+    k_fill128<<<dim3((unsigned)std::min<int64_t>(ceil_div(n4, TB), 256 * 32)), TB, 0, s>>>((uint4 *)p, v, n4);
+    LAUNCH_CHECK();
+    p = (uint32_t *)p + n4 * 4;
+    n -= n4 * 4;
+    if (n == 0) return;
+  }
   int64_t blocks = std::min<int64_t>(ceil_div(n, TB), 256 * 32);
   k_fill32<<<dim3((unsigned)blocks), TB, 0, s>>>((uint32_t *)p, v, n);
   LAUNCH_CHECK();

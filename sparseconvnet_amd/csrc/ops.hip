@@ -189,20 +189,29 @@ void input_forward(const InputRules &r, const float *in, float *out, int planes,
 // CPU/IOLayers.cpp:95-115 (InputLayer_BackwardPass :31-47 without averaging): every input
 // point listed in its site's rule receives the site's row; as a gather per input point.
 // Modes 1 / 2 list a single point per site, the others get zeros.
+template <int V>
 __global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, const int *run_start,
                              const int *run_len, int64_t n_in, int mode, const float *in, float *out,
                              int planes) {
+  // thread -> (input point, group of V planes)
+  const int groups = planes / V;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = n_in * planes;
-  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  const int64_t total = n_in * groups;
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
   for (; i < total; i += step) {
-    int64_t pt = i / planes;
-    int p = (int)(i - pt * planes);
-    int row = row_of_input[pt];
+    const int64_t pt = i / groups;
+    const int p = (int)(i - pt * groups) * V;
+    const int row = row_of_input[pt];
     bool listed = row >= 0;  // empty positions of a batch-by-length input get zeros
     if (listed && mode == 1) listed = sorted_idx[run_start[row]] == (int)pt;
     if (listed && mode == 2) listed = sorted_idx[run_start[row] + run_len[row] - 1] == (int)pt;
-    out[i] = listed ? in[(int64_t)row * planes + p] : 0.0f;
+    if (V == 4) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (listed) v = *reinterpret_cast<const float4 *>(in + (int64_t)row * planes + p);
+      *reinterpret_cast<float4 *>(out + pt * planes + p) = v;
+    } else {
+      out[pt * planes + p] = listed ? in[(int64_t)row * planes + p] : 0.0f;
+    }
   }
 }
 void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s) {
@@ -212,14 +221,19 @@ void output_forward(const InputRules &r, const float *in, float *out, int planes
     HIP_CHECK(hipMemcpyAsync(out, in, sizeof(float) * r.n_in * planes, hipMemcpyDeviceToDevice, s));
     return;
   }
-  int64_t total = r.n_in * planes;
   if (r.n_out == 0) {  // every position empty
-    fill32(out, 0, total, s);
+    fill32(out, 0, r.n_in * planes, s);
     return;
   }
-  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
-  k_output_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
-                                                     r.run_len.p, r.n_in, r.mode, in, out, planes);
+  const bool vec = planes % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0;
+  const int64_t total = r.n_in * (vec ? planes / 4 : planes);
+  const int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  if (vec)
+    k_output_fwd<4><<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
+                                                          r.run_len.p, r.n_in, r.mode, in, out, planes);
+  else
+    k_output_fwd<1><<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
+                                                          r.run_len.p, r.n_in, r.mode, in, out, planes);
   LAUNCH_CHECK();
 }
 
