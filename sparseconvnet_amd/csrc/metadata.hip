@@ -131,12 +131,38 @@ static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
 
 // ---- input layer -----------------------------------------------------------------------
 
+// A maximum over the whole grid without hammering one address: wavefront shuffle, one LDS
+// atomic per wavefront, then one global atomic per workgroup into one of 64 slots (a cache line
+// apart), and only when it can raise the slot (the plain read may be stale, which costs an
+// atomic that changes nothing).  20 000 same-address atomics cost ~130 us on a 1.3 M-point
+// input, this costs ~10.  Every thread of the workgroup must call it; values <= floor are
+// not reported.  The host takes the maximum over the slots (max_slots).
+static const int MAX_SLOTS = 64, MAX_SLOT_STRIDE = 16;
+__device__ inline void grid_max(int v, int floor, int *slots) {
+  __shared__ int block_max;
+  if (threadIdx.x == 0) block_max = floor;
+  __syncthreads();
+  for (int off = 32; off; off >>= 1) v = max(v, __shfl_xor(v, off));
+  if ((threadIdx.x & 63) == 0 && v > floor) atomicMax(&block_max, v);
+  __syncthreads();
+  int *slot = slots + MAX_SLOT_STRIDE * (blockIdx.x & (MAX_SLOTS - 1));
+  if (threadIdx.x == 0 && block_max > floor && block_max > __builtin_nontemporal_load(slot)) atomicMax(slot, block_max);
+}
+static int max_slots(const int *slots, hipStream_t s) {  // one stream synchronisation
+  int h[MAX_SLOTS * MAX_SLOT_STRIDE];
+  HIP_CHECK(hipMemcpyAsync(h, slots, sizeof h, hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  int v = 0;
+  for (int i = 0; i < MAX_SLOTS; i++) v = std::max(v, h[i * MAX_SLOT_STRIDE]);
+  return v;
+}
+
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
 // bl_len > 0: the sample of point i is i / bl_len and a negative first coordinate marks an
 // empty position (Metadata/IOLayersRules.h:183,204,234): key EMPTY, counted in flags[4].
 __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols, int64_t bl_len,
                              unsigned long long *keys, int *idx, int *flags) {
-  // flags[0]: error bits, flags[3]: largest sample index (one atomic per wavefront)
+  // flags[0]: error bits, flags[4]: empty positions, flags[8...]: slots of the largest sample index
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int bmax = 0;
   bool empty = false;
@@ -167,8 +193,7 @@ __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols
     idx[i] = (int)i;
     bmax = (int)b;
   }
-  for (int off = 32; off; off >>= 1) bmax = max(bmax, __shfl_xor(bmax, off));
-  if ((threadIdx.x & 63) == 0 && bmax > 0) atomicMax(&flags[3], bmax);
+  grid_max(bmax, 0, flags + 8);
   const unsigned long long em = __ballot(empty);
   if ((threadIdx.x & 63) == 0 && em) atomicAdd(&flags[4], __popcll(em));
 }
@@ -233,10 +258,7 @@ __global__ void k_finish_groups(const int *sidx, const int *head, const int *hea
       run_len[row] = len;
     }
   }
-  // longest run: one atomic per wavefront, and only when it can raise the maximum (the plain
-  // read may be stale, which only costs an atomic that changes nothing)
-  for (int off = 32; off; off >>= 1) len = max(len, __shfl_xor(len, off));
-  if ((threadIdx.x & 63) == 0 && len > 1 && len > __builtin_nontemporal_load(max_active)) atomicMax(max_active, len);
+  grid_max(len, 1, max_active);  // longest run; runs of one are the floor
 }
 
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
@@ -270,16 +292,18 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   m.k1.reserve(n);
   m.v0.reserve(n);
   m.v1.reserve(n);
-  m.dflags.reserve(8);
-  fill32(m.dflags.p, 0, 8, s);
+  const int n_flags = 8 + MAX_SLOTS * MAX_SLOT_STRIDE;
+  m.dflags.reserve(n_flags);
+  fill32(m.dflags.p, 0, n_flags, s);
   k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, bl_length, m.k0.p, m.v0.p, m.dflags.p);
   LAUNCH_CHECK();
-  int hflags[5];
-  HIP_CHECK(hipMemcpyAsync(hflags, m.dflags.p, sizeof hflags, hipMemcpyDeviceToHost, s));
+  std::vector<int> hflags(n_flags);
+  HIP_CHECK(hipMemcpyAsync(hflags.data(), m.dflags.p, n_flags * sizeof(int), hipMemcpyDeviceToHost, s));
   HIP_CHECK(hipStreamSynchronize(s));
   if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
   if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");
-  const int top_batch = hflags[3];
+  int top_batch = 0;
+  for (int i = 0; i < MAX_SLOTS; i++) top_batch = std::max(top_batch, hflags[8 + i * MAX_SLOT_STRIDE]);
   const int64_t n_empty = hflags[4], nv = n - n_empty;
   if (n_empty && mode == 0) throw Error("batch-by-length input layer: mode 0 needs every position filled");
   // only the key bits that samples 0..top_batch can set take part in the sort; one bit more
@@ -331,7 +355,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   if (N == 0) return;
   m.v0.reserve(std::max<int64_t>(n, 2 * N + 2));  // reused: row_of_group | head_pos
   int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
-  fill32(m.dflags.p, 0, 8, s);
+  fill32(m.dflags.p, 0, n_flags, s);
   k_assign_rows<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, bl_length, m.k1.p, m.v1.p, m.f0.p, m.s0.p, m.s1.p,
                                            n, L.npad, L.coords.p, L.keys.p, L.sched.p, row_of_group,
                                            head_pos);
@@ -339,9 +363,9 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   // the groups end where the empty positions begin
   k_finish_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, row_of_group, head_pos, nv, (int)N,
                                               R.row_of_input.p, R.run_start.p, R.run_len.p,
-                                              m.dflags.p + 2);
+                                              m.dflags.p + 8);
   LAUNCH_CHECK();
-  int ma = std::max(1, read_back(m.dflags.p + 2, s));  // runs of one never touch the counter
+  int ma = std::max(1, max_slots(m.dflags.p + 8, s));  // runs of one never touch the slots
   // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2.
   R.max_active = (mode == 3 || mode == 4) ? ma : 1;
 }
