@@ -72,6 +72,8 @@ static int key_bits(const Geom &g, int64_t batch) {
 
 // ---- small utilities -------------------------------------------------------------------
 
+static const int COUNT_SLOTS = 32;  // copies of a rulebook's per-tap counters (a power of two)
+
 __global__ void k_fill32(uint32_t *p, uint32_t v, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -616,8 +618,9 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
     }
   }
   __syncthreads();
+  unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * f.K;
   for (int k = threadIdx.x; k < f.K; k += blockDim.x)
-    if (lcount[k]) atomicAdd(&counts[k], (unsigned long long)lcount[k]);
+    if (lcount[k]) atomicAdd(&slot[k], (unsigned long long)lcount[k]);
 }
 
 // ---- pattern-sorted positions ----------------------------------------------------------
@@ -786,7 +789,8 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
     if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&lcount[k], __popcll(hits));
   }
   __syncthreads();
-  if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&counts[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
+  unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * K;
+  if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&slot[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
 }
 
 static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const int64_t *out_size) {
@@ -809,11 +813,28 @@ static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const
   return f;
 }
 
+// Rule counts are tallied per workgroup in LDS and flushed with one atomic per tap into one of
+// COUNT_SLOTS copies of the counter array (a million-site level has 15 000 workgroups; all of
+// them adding to the same K addresses cost 160 us of a 700 us rulebook build).  fold_counts
+// then sums the copies into the first one, which is the one everybody reads.
 static void start_counts(Table &t, hipStream_t s) {
   t.cnt = std::make_shared<Counts>();
   t.cnt->K = t.K;
-  t.cnt->dev.reserve(std::max(t.K, 1));
-  fill32(t.cnt->dev.p, 0, 2 * (int64_t)std::max(t.K, 1), s);
+  const int64_t words = (int64_t)COUNT_SLOTS * std::max(t.K, 1);
+  t.cnt->dev.reserve(words);
+  fill32(t.cnt->dev.p, 0, 2 * words, s);
+}
+__global__ void k_fold_counts(unsigned long long *counts, int K) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= K) return;
+  unsigned long long v = 0;
+  for (int sl = 1; sl < COUNT_SLOTS; sl++) v += counts[(size_t)sl * K + k];
+  counts[k] += v;
+}
+static void fold_counts(Table &t, hipStream_t s) {
+  if (t.K <= 0) return;
+  k_fold_counts<<<grid_for(t.K), TB, 0, s>>>((unsigned long long *)t.cnt->dev.p, t.K);
+  LAUNCH_CHECK();
 }
 static void zero_counts(Table &t) {  // a table without rules
   t.cnt = std::make_shared<Counts>();
@@ -917,6 +938,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
                                                            L.gridp.p, L.urow_ptr(), t.nbr.p,
                                                            (unsigned long long *)t.cnt->dev.p);
     LAUNCH_CHECK();
+    fold_counts(t, s);
     finalize_table(m, t, L.sched_ptr(), s);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
@@ -926,6 +948,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
       L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p, L.gridp.p, L.urow_ptr(), t.nbr.p,
       (unsigned long long *)t.cnt->dev.p, parts);
   LAUNCH_CHECK();
+  fold_counts(t, s);
   finalize_table(m, t, L.sched_ptr(), s);
   return m.subm.emplace(key, std::move(t)).first->second;
 }
@@ -1001,8 +1024,9 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
     }
   }
   __syncthreads();
+  unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * f.K;
   for (int k = threadIdx.x; k < f.K; k += blockDim.x)
-    if (lcount[k]) atomicAdd(&counts[k], (unsigned long long)lcount[k]);
+    if (lcount[k]) atomicAdd(&slot[k], (unsigned long long)lcount[k]);
 }
 
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
@@ -1086,6 +1110,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
                                              m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
                                              LO.coords.p, LO.keys.p, (unsigned long long *)R.by_out.cnt->dev.p);
   LAUNCH_CHECK();
+  fold_counts(R.by_out, s);
   R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
   finalize_table(m, R.by_out, nullptr, s);
   finalize_table(m, R.by_in, LI.sched_ptr(), s);
