@@ -222,25 +222,36 @@ __global__ void k_group_heads(const unsigned long long *skeys, const int *sidx, 
   is_first[sidx[p]] = h;
 }
 
-// Heads: row = rank of the first occurrence in input order (Metadata/IOLayersRules.h:84-87).
-__global__ void k_assign_rows(Geom g, const int64_t *coords, int ncols, int64_t bl_len,
-                              const unsigned long long *skeys,
-                              const int *sidx, const int *head, const int *head_scan,
-                              const int *first_scan, int64_t n, int64_t npad, int *soa,
-                              unsigned long long *level_keys, int *sched, int *row_of_group,
-                              int *head_pos) {
+// Row = rank of the first occurrence in input order (Metadata/IOLayersRules.h:84-87).
+// Two passes so that every array is written in ascending order (stream compaction) instead of
+// being scattered: one over the sorted points for what is indexed by group (key order) ...
+__global__ void k_assign_groups(const int *sidx, const int *head, const int *head_scan, const int *first_scan,
+                                int64_t n, int *sched, int *row_of_group, int *head_pos) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n || !head[p]) return;
-  int i = sidx[p];
-  int row = first_scan[i];
-  int u = head_scan[p];
+  const int row = first_scan[sidx[p]];
+  const int u = head_scan[p];
   sched[u] = row;
   row_of_group[u] = row;
   head_pos[u] = (int)p;
-  level_keys[row] = skeys[p];
-  const int64_t *c = coords + (int64_t)i * ncols;
-  for (int d = 0; d < g.dim; d++) soa[d * npad + row] = (int)c[d];
-  soa[g.dim * npad + row] = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)c[g.dim] : 0);
+}
+// ... and one over the points in input order for what is indexed by row: coordinates and key
+// of every first occurrence.
+__global__ void k_assign_coords(Geom g, const int64_t *coords, int ncols, int64_t bl_len, const int *is_first,
+                                const int *first_scan, int64_t n, int64_t npad, int *soa,
+                                unsigned long long *level_keys) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n || !is_first[i]) return;
+  const int row = first_scan[i];
+  const int64_t *c = coords + i * ncols;
+  int cc[SCN_MAXD];
+  for (int d = 0; d < g.dim; d++) {
+    cc[d] = (int)c[d];
+    soa[d * npad + row] = cc[d];
+  }
+  const int b = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)c[g.dim] : 0);
+  soa[g.dim * npad + row] = b;
+  level_keys[row] = site_key(g, cc, b);
 }
 
 __global__ void k_finish_groups(const int *sidx, const int *head, const int *head_scan,
@@ -358,9 +369,10 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   m.v0.reserve(std::max<int64_t>(n, 2 * N + 2));  // reused: row_of_group | head_pos
   int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
   fill32(m.dflags.p, 0, n_flags, s);
-  k_assign_rows<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, bl_length, m.k1.p, m.v1.p, m.f0.p, m.s0.p, m.s1.p,
-                                           n, L.npad, L.coords.p, L.keys.p, L.sched.p, row_of_group,
-                                           head_pos);
+  k_assign_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, m.s1.p, nv, L.sched.p, row_of_group, head_pos);
+  LAUNCH_CHECK();
+  k_assign_coords<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, bl_length, m.f1.p, m.s1.p, n, L.npad, L.coords.p,
+                                             L.keys.p);
   LAUNCH_CHECK();
   // the groups end where the empty positions begin
   k_finish_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, row_of_group, head_pos, nv, (int)N,
