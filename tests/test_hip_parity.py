@@ -323,3 +323,29 @@ def test_full_size_sweep_scene_properties():
     sep = g.bn_eval(g.subm_conv(4096, 3, g.bn_eval(x1, bn["mean"], bn["var"], bn["weight"], bn["bias"], 1e-4, 0.0),
                                 w)[0], bn["mean"], bn["var"], bn["weight"], bn["bias"], 1e-4, 0.0)
     checks.assert_close(fused, sep, "fused vs separate batch norm at 1 M sites")
+
+
+def test_input_above_2_gib_matches_split_channels():
+    """A feature matrix above 2 GiB takes the kernels' 64-bit addressing path (the buffer-load
+    gathers are for smaller inputs; the reference itself overflows its int32 offsets near this
+    size, CPU/Convolution.cpp:18,38).  Checked against the same convolution computed as the
+    sum of two half-width convolutions, each of which is below the limit."""
+    import torch
+    from sparseconvnet_amd import metadata as M
+    coords = synthetic.room_scene(seed=3100, target=1100000, spatial=4096)
+    n = len(coords)
+    md = M.Metadata(3)
+    sz, three = torch.LongTensor([4096] * 3), torch.LongTensor([3] * 3)
+    g = torch.Generator(device="cuda").manual_seed(31)
+    md.inputLayer(sz, torch.as_tensor(coords).cuda(), torch.zeros((n, 1), device="cuda"), 0, 0)
+    x = torch.randn((n, 512), device="cuda", generator=g)
+    assert x.numel() * 4 > 2 ** 31
+    for cout in (16, 144):  # row-owner kernel, LDS-tiled kernel
+        w = torch.randn((27, 1, 512, cout), device="cuda", generator=g) * 0.02
+        y, macs = md.submanifoldConvolution(sz, three, x, w, None)
+        ya, _ = md.submanifoldConvolution(sz, three, x[:, :256].contiguous(), w[:, :, :256].contiguous(), None)
+        yb, _ = md.submanifoldConvolution(sz, three, x[:, 256:].contiguous(), w[:, :, 256:].contiguous(), None)
+        want = (ya + yb).cpu().numpy()
+        checks.assert_close(y.cpu().numpy(), want, "512 -> %d above 2 GiB" % cout)
+        assert np.abs(want).max() > 0.1 and macs > 0
+        del y, ya, yb
