@@ -88,13 +88,14 @@ def cpu_baseline(sample_sites, seed):
                       % (len(coords), R, t_rules)}
 
 
-def unet_scene(sites, seed, reps=3, residual=False):
+def unet_scene(sites, seed, reps=3, residual=False, batch=1):
     """3D U-Net forward of examples/ScanNet/unet.py:25-38 with m=32, block_reps=2 (7 levels,
     [32..224] planes), InputLayer mode 4 on a room scene with ~30% duplicated points, eval,
     random-init weights, batch 1.  cold = new Metadata per scene, as a user runs it (input layer,
     every rulebook and all layers); warm = the same scene again with its rulebooks cached.
     residual: the builder's ResNet-style blocks (networkArchitectures.py:222-230) instead of
-    the VGG-style ones the example uses."""
+    the VGG-style ones the example uses.  batch: that many scenes of `sites` sites in one call
+    (examples/ScanNet/unet.py trains and validates with batches of scenes)."""
     import torch
     import sparseconvnet_amd as scn
     from sparseconvnet_amd import synthetic
@@ -104,7 +105,10 @@ def unet_scene(sites, seed, reps=3, residual=False):
         scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m, 5 * m, 6 * m, 7 * m], residual)).add(
         scn.OutputLayer(3)).cuda().eval()
     linear = torch.nn.Linear(m, 20).cuda()
-    coords = synthetic.room_scene(seed=seed, target=sites, spatial=4096, duplicate_fraction=0.3)
+    if batch == 1:
+        coords = synthetic.room_scene(seed=seed, target=sites, spatial=4096, duplicate_fraction=0.3)
+    else:
+        coords = synthetic.scene_batch(seed=seed, batch=batch, target=sites, spatial=4096, duplicate_fraction=0.3)
     g = torch.Generator(device="cuda").manual_seed(1)
     feats = torch.rand((len(coords), 3), device="cuda", generator=g) * 2 - 1
     cd = torch.as_tensor(coords).cuda()
@@ -126,6 +130,10 @@ def unet_scene(sites, seed, reps=3, residual=False):
                 cold.append((t1 - t0) * 1e3)
                 warm.append((t2 - t1) * 1e3)
             macs = scn.forward_pass_multiplyAdd_count / 2
+    if batch > 1:
+        return {"unet_batch%d_ms_per_batch" % batch: round(float(np.median(cold)), 3),
+                "unet_batch%d_warm_ms_per_batch" % batch: round(float(np.median(warm)), 3),
+                "unet_batch%d_active_sites" % batch: int(x.features.shape[0])}
     if residual:
         return {"unet_residual_ms_per_scene": round(float(np.median(cold)), 3),
                 "unet_residual_warm_ms": round(float(np.median(warm)), 3),
@@ -407,6 +415,7 @@ def main():
         out["unet"] = unet_scene(args.unet_sites, 5000)
         if not args.no_residual:
             out["unet"].update(unet_scene(args.unet_sites, 5000, residual=True))
+            out["unet"].update(unet_scene(args.unet_sites, 7000, reps=2, batch=4))
         if not args.no_bf16:
             import sparseconvnet_amd as scn
             scn.bf16_mfma = True
