@@ -221,17 +221,13 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   // An operand is what one lane feeds one MFMA with: 16 bytes, either four fp32 channels of
   // one 16-channel step or four bf16 channels of each step of a pair.
   constexpr int WS = BF16 ? SS / 2 : SS;      // operands per slab, column block and lane
-  constexpr int SLAB_F4 = WS * NCB * 64;      // operands of one weight slab
-  constexpr int WPT = (SLAB_F4 + 255) / 256;  // operands staged per thread
-  constexpr int LDS_SLAB_F4 = WPT * 256;      // slab in LDS
   constexpr int SLAB_STRIDE_F4 = packed_slab_floats(SS, NCB) / (BF16 ? 8 : 4);  // slab in global memory
   constexpr int NFRAG = G * SS;               // A fragments (granule, step) per iteration
   constexpr int FPW = NFRAG / 4;              // fragments gathered per wavefront
   constexpr int A_F4 = G * WS * 64;           // A operands per iteration
   static_assert(NFRAG % 4 == 0, "fragments must divide over 4 wavefronts");
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  v4f *wbuf = reinterpret_cast<v4f *>(lds);   // [2][LDS_SLAB_F4]
-  v4f *abuf = wbuf + 2 * LDS_SLAB_F4;         // [2][A_F4]
+  v4f *abuf = reinterpret_cast<v4f *>(lds);   // [2][A_F4]
   int *jtab = reinterpret_cast<int *>(abuf + 2 * A_F4);  // [G][K][16]
   unsigned *gmask = reinterpret_cast<unsigned *>(jtab + G * K * 16);  // [K] granules having tap k
   int *taplist = reinterpret_cast<int *>(gmask + K);           // [K]
@@ -283,22 +279,35 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 #pragma unroll
     for (int c = 0; c < NCBW; c++) acc[q][c] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  v4f wreg[WPT];
+  // Loads in flight, one iteration ahead.  The weights never pass through LDS: a wavefront's
+  // column blocks are its own (wavefronts that share a column range, WR = 2, each fetch their
+  // copy from L2), and the packed layout is the lane order of the B operand, so a lane's 16
+  // bytes per (step, column block) are one coalesced load.  They alternate between two register
+  // sets (iteration parity; the loop is unrolled twice so that the set is a constant), because
+  // the set of iteration it+1 is being filled while the MFMAs of iteration it read theirs.
+  // The gathered rows go through double-buffered LDS, since every wavefront needs all of them.
+  v4f breg[2][WS][NCBW];
   v4f areg[FPW];
   v4f psc[FPW], psh[FPW];           // pre-activation coefficients of the fragments' channels
   unsigned gm_nxt = 0, gm_cur = 0;  // granule mask of the tap (uniform)
   unsigned aok_nxt = 0;             // bit i: this lane's row of fragment i exists
   int sl_nxt = 0;
 
-  // Issue the loads of iteration `it`: its weight slab into wreg; this wavefront's share of
-  // the A fragments (granule, step) into areg.
   // BUF: gathers through buffer loads; an absent row becomes an offset of 2 GiB, which is past
   // the end and reads as zeros (see k_conv_rows).
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
   const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
-  auto issue = [&](int it) {
-    const int ti = it / n_slab, sl = it - ti * n_slab;
+  const int ntaps = *ntaps_p;
+  // Issue the loads of iteration `it`: this wavefront's weights into register set P (= it % 2)
+  // and its share of the A fragments (granule, step) into areg.
+  auto issue = [&](int it, auto par_c) {
+    constexpr int P = decltype(par_c)::value;
+    // Slab outer, tap inner: while a slab is being worked on, the tile and its neighbours in
+    // the XCD's range gather the same 64-byte columns of a few hundred rows over and over (a
+    // row feeds ~10 taps), a working set that stays in L2; with the tap outermost every
+    // gather of a 1 KiB row came from HBM (12 GB per launch at 256 planes).
+    const int sl = it / ntaps, ti = it - sl * ntaps;
     // LDS values every lane reads alike: tell the compiler, so that what follows from them
     // (weight address, branches on the granule mask) is scalar work
     const int k = __builtin_amdgcn_readfirstlane(taplist[ti]);
@@ -308,10 +317,9 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     aok_nxt = 0;
     const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
 #pragma unroll
-    for (int i = 0; i < WPT; i++) {
-      const int e = threadIdx.x + i * 256;
-      wreg[i] = wsrc[(SLAB_F4 % 256 == 0 || e < SLAB_F4) ? e : 0];
-    }
+    for (int s = 0; s < WS; s++)
+#pragma unroll
+      for (int c = 0; c < NCBW; c++) breg[P][s][c] = wsrc[(s * NCB + wc * NCBW + c) * 64 + lane];
 #pragma unroll
     for (int i = 0; i < FPW; i++) {
       const int f = wave + 4 * i;  // fragment f = (granule f / SS, step f % SS)
@@ -348,12 +356,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     }
   };
 
-  if (total > 0) issue(0);
-  for (int it = 0; it < total; it++) {
-    v4f *wb = wbuf + (it & 1) * LDS_SLAB_F4;
-    v4f *ab = abuf + (it & 1) * A_F4;
-#pragma unroll
-    for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * 256] = wreg[i];
+  // One iteration; P = it % 2 selects the LDS buffer of the rows and the weights' register set.
+  auto iterate = [&](int it, auto par_c) {
+    constexpr int P = decltype(par_c)::value;
+    v4f *ab = abuf + P * A_F4;
     // Absent rows and channels past nIn become zeros on their way into LDS.
 #pragma unroll
     for (int i = 0; i < FPW; i++) {
@@ -377,23 +383,20 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
         ab[f * 64 + lane] = v;
     }
     gm_cur = gm_nxt;
-    // After this barrier the buffers of `it` are visible, and every wavefront has finished
-    // the MFMAs of it-1, so the other buffers may be overwritten at the top of it+1.
+    // After this barrier the rows of `it` are visible, and every wavefront has finished the
+    // MFMAs of it-1, so the other buffer may be overwritten at the top of it+1.
     __syncthreads();
-    if (it + 1 < total) issue(it + 1);
+    if (it + 1 < total) issue(it + 1, std::integral_constant<int, 1 - P>{});
 
-    v4f b[WS][NCBW];
+    // fp32: all A fragments of this wavefront's granules are fetched before the first MFMA, so
+    // that no MFMA waits on LDS.  bf16: a granule's fragment is fetched when its turn comes.
+    v4f afrag[BF16 ? 1 : GW][WS];
+    if constexpr (!BF16) {
 #pragma unroll
-    for (int s = 0; s < WS; s++)
+      for (int q = 0; q < GW; q++)
 #pragma unroll
-      for (int c = 0; c < NCBW; c++) b[s][c] = wb[(s * NCB + wc * NCBW + c) * 64 + lane];
-    // all A fragments of this wavefront's granules are fetched before the first MFMA, so that
-    // no MFMA waits on LDS
-    v4f afrag[GW][WS];
-#pragma unroll
-    for (int q = 0; q < GW; q++)
-#pragma unroll
-      for (int s = 0; s < WS; s++) afrag[q][s] = ab[((wr * GW + q) * WS + s) * 64 + lane];
+        for (int s = 0; s < WS; s++) afrag[q][s] = ab[((wr * GW + q) * WS + s) * 64 + lane];
+    }
 #pragma unroll
     for (int q = 0; q < GW; q++) {
       const int gr = wr * GW + q;
@@ -401,22 +404,29 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 #pragma unroll
       for (int s = 0; s < WS; s++) {
         if constexpr (BF16) {
+          const v4f af = ab[((wr * GW + q) * WS + s) * 64 + lane];
 #pragma unroll
           for (int c = 0; c < NCBW; c++)
-            acc[q][c] = mfma_bf16(__builtin_bit_cast(v8s, afrag[q][s]), __builtin_bit_cast(v8s, b[s][c]), acc[q][c]);
+            acc[q][c] = mfma_bf16(__builtin_bit_cast(v8s, af), __builtin_bit_cast(v8s, breg[P][s][c]), acc[q][c]);
         } else {
           const v4f av = afrag[q][s];
 #pragma unroll
-          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, b[s][c].x, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, breg[P][s][c].x, acc[q][c], 0, 0, 0);
 #pragma unroll
-          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, b[s][c].y, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, breg[P][s][c].y, acc[q][c], 0, 0, 0);
 #pragma unroll
-          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, b[s][c].z, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, breg[P][s][c].z, acc[q][c], 0, 0, 0);
 #pragma unroll
-          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, b[s][c].w, acc[q][c], 0, 0, 0);
+          for (int c = 0; c < NCBW; c++) acc[q][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, breg[P][s][c].w, acc[q][c], 0, 0, 0);
         }
       }
     }
+  };
+
+  if (total > 0) issue(0, std::integral_constant<int, 0>{});
+  for (int it = 0; it < total; it += 2) {
+    iterate(it, std::integral_constant<int, 0>{});
+    if (it + 1 < total) iterate(it + 1, std::integral_constant<int, 1>{});
   }
 
   // acc[q][c][r] = result for position tbase + 16*(wr*GW+q) + 4*g + r, column 16*(wc*NCBW+c) + r16
@@ -491,10 +501,8 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   }
   constexpr int WR = 4 / WC, NCB = NCBW * WC, G = GW * WR;
   constexpr int WS = BF16 ? SS / 2 : SS;
-  constexpr int WPT = (WS * NCB * 64 + 255) / 256;
   constexpr int SLAB_STRIDE = packed_slab_floats(SS, NCB);  // elements of a packed slab
-  const size_t lds_bytes = (size_t)2 * WPT * 256 * 16 + (size_t)2 * G * WS * 64 * 16 +
-                           ((size_t)G * t.K * 16 + 2 * t.K + 4) * sizeof(int);
+  const size_t lds_bytes = (size_t)2 * G * WS * 64 * 16 + ((size_t)G * t.K * 16 + 2 * t.K + 4) * sizeof(int);
   if (lds_bytes > 160 * 1024) return false;
   const int cin16 = (int)ceil_div(n_in, 16);
   const int n_slab = (int)ceil_div(cin16, SS);
@@ -622,7 +630,8 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     *ntaps_p = c;
   }
   __syncthreads();
-  const int total = *ntaps_p * n_slab;
+  const int ntaps = *ntaps_p;
+  const int total = ntaps * n_slab;
 
   v4f acc[RG][NCB];
 #pragma unroll
@@ -647,9 +656,9 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     // LDS values every lane reads alike: tell the compiler, so that what follows from them
     // (weight address, branches on the granule mask) is scalar work
     const int k = __builtin_amdgcn_readfirstlane(taplist[nx_ti]);
-    if (++nx_sl == n_slab) {
-      nx_sl = 0;
-      nx_ti++;
+    if (++nx_ti == ntaps) {  // slab outer, tap inner (see k_conv_mfma)
+      nx_ti = 0;
+      nx_sl++;
     }
     gm_nxt = __builtin_amdgcn_readfirstlane(gmask[k]);
     sl_nxt = sl;
