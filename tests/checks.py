@@ -285,6 +285,43 @@ def check_s2d(make, dim, seed, spatial=6, n=80, batch=3, C=4):
     assert sum(len(r) for r in rules) == len(loc)
 
 
+def check_level_replacement(make, seed=11):
+    """What happens to a level that is built twice, as the reference does it
+    (Metadata/ConvolutionRules.h:68-70, Metadata/Metadata.cpp:492-518, CPU/Deconvolution.cpp:15-18):
+    operations with the same (input size, filter, stride) share one rulebook and one output
+    level; a strided rulebook with another key that lands on an existing spatial size builds
+    that level anew from its own input; a deconvolution towards a spatial size that was never
+    built finds an empty fine level, yields no rows and leaves the coarse level empty."""
+    rng = np.random.default_rng(seed)
+    dim, batch = 2, 2
+    coords = bf.random_sites(rng, dim, 9, 60, batch)
+    coords = np.unique(coords, axis=0)
+    x = rng.normal(size=(len(coords), 3)).astype(np.float32)
+    p = make(dim)
+    p.input_layer(9, coords, 0, 0)
+    loc = p.spatial_locations(9)
+    w = (rng.normal(size=(9, 1, 3, 2)) * 0.3).astype(np.float32)
+    y, _ = p.conv(9, 4, 3, 2, x, w)
+    loc_a = p.spatial_locations(4)
+    want_a = set(t[1 + dim + 1:] for t in bf.strided_triples(loc, dim, 3, 2, np.array([4, 4])))
+    assert set(map(tuple, loc_a.tolist())) == want_a
+    mp = p.maxpool(9, 4, 3, 2, x)  # same key: same rulebook, level untouched
+    assert (p.spatial_locations(4) == loc_a).all() and mp.shape == (len(loc_a), 3)
+    # another key onto spatial size 4: the level is rebuilt from this rulebook's outputs
+    w6 = (rng.normal(size=(36, 1, 3, 2)) * 0.1).astype(np.float32)
+    y6, _ = p.conv(9, 4, 6, 1, x, w6)
+    loc_b = p.spatial_locations(4)
+    want_b = set(t[1 + dim + 1:] for t in bf.strided_triples(loc, dim, 6, 1, np.array([4, 4])))
+    assert set(map(tuple, loc_b.tolist())) == want_b and p.nactive(4) == len(want_b) == len(y6)
+    dense = bf.dense_strided_conv(loc, x, w6, 9, 6, 1, batch)
+    assert_close(y6, bf.sample_dense(dense, loc_b), "second rulebook onto the same level")
+    # deconvolution towards a level nobody built: 4 -> (4-1)*3+3 = 12
+    wd = (rng.normal(size=(9, 1, 2, 3)) * 0.3).astype(np.float32)
+    z, macs = p.deconv(4, 12, 3, 3, y6, wd)
+    assert z.shape == (0, 3) and macs == 0
+    assert p.nactive(12) == 0 and p.nactive(4) == 0
+
+
 def check_empty(make, dim=3):
     """Zero active sites: every op returns an empty result and 0 multiply-adds."""
     p = make(dim)

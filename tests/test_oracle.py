@@ -71,5 +71,9 @@ def test_s2d(make, dim):
     checks.check_s2d(make, dim, seed=2 + dim)
 
 
+def test_level_replacement(make):
+    checks.check_level_replacement(make)
+
+
 def test_empty(make):
     checks.check_empty(make)
