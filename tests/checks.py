@@ -322,6 +322,49 @@ def check_level_replacement(make, seed=11):
     assert p.nactive(12) == 0 and p.nactive(4) == 0
 
 
+def check_special_values(make, seed=12):
+    """NaN, infinities, negative zero and all-negative windows: max pooling starts from zero and
+    replaces only when `out < in` (CPU/MaxPooling.cpp:17-18,50), so a NaN never enters and an
+    all-negative window gives +0; batch norm multiplies by the leakiness where y > 0 is false
+    (CPU/BatchNormalization.cpp:55-58), so ReLU maps negatives to -0.0 and NaN stays NaN."""
+    rng = np.random.default_rng(seed)
+    dim, batch = 2, 1
+    coords = np.unique(bf.random_sites(rng, dim, 8, 50, batch), axis=0)
+    n = len(coords)
+    x = rng.normal(size=(n, 4)).astype(np.float32)
+    x[rng.random(n) < 0.2, 0] = np.nan
+    x[:, 1] = -np.abs(x[:, 1]) - 0.5            # every window negative
+    x[rng.random(n) < 0.3, 2] = -0.0
+    x[rng.random(n) < 0.1, 3] = np.inf
+    p = make(dim)
+    p.input_layer(8, coords, 0, 0)
+    loc = p.spatial_locations(8)
+    rules = p.strided_rules(8, 4, 2, 2)
+    got = p.maxpool(8, 4, 2, 2, x)
+    want = np.zeros_like(got)
+    for r in rules:
+        for i, o in r:
+            lt = want[o] < x[i]                 # false for NaN
+            want[o][lt] = x[i][lt]
+    assert got.shape == want.shape
+    assert (np.isnan(got) == np.isnan(want)).all() and not np.isnan(got).any()
+    assert (got == want).all() and (np.signbit(got) == np.signbit(want)).all()
+    assert (got[:, 1] == 0).all() and not np.signbit(got[:, 1]).any()
+    mean, var = np.zeros(4, np.float32), np.ones(4, np.float32)
+    y = p.bn_eval(x, mean, var, None, None, 1e-4, 0.0)
+    w = np.float32(1.0) / np.sqrt(var + np.float32(1e-4))
+    b = -mean * w + np.float32(0)               # the reference's shift term: +0 here
+    t = x * w + b
+    with np.errstate(invalid="ignore"):
+        want = t * np.where(t > 0, np.float32(1), np.float32(0))
+    assert (np.isnan(y) == np.isnan(want)).all()
+    ok = np.isfinite(want)
+    assert (np.isinf(y) == np.isinf(want)).all()
+    assert_close(y[ok], want[ok], "batch norm special values")
+    ok = ~np.isnan(want)
+    assert (np.signbit(y[ok]) == np.signbit(want[ok])).all()   # negatives become -0.0, as in the reference
+
+
 def check_empty(make, dim=3):
     """Zero active sites: every op returns an empty result and 0 multiply-adds."""
     p = make(dim)

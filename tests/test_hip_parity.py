@@ -78,6 +78,10 @@ def test_level_replacement(make):
     checks.check_level_replacement(make)
 
 
+def test_special_values(make):
+    checks.check_special_values(make)
+
+
 def test_empty(make):
     checks.check_empty(make)
 
