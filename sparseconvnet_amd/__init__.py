@@ -25,7 +25,8 @@ from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, Bat
 from .metadata import Metadata  # noqa: E402
 from .networks import SparseVggNet, UNet  # noqa: E402
 from .tensor import SparseConvNetTensor  # noqa: E402
-from .utils import optionalTensor, prepare_BLInput, toLongTensor  # noqa: E402
+from .utils import (checkpoint_restore, checkpoint_save, is_power2, optionalTensor,  # noqa: E402
+                    prepare_BLInput, toLongTensor)
 
 
 def is_hip_build():

@@ -104,7 +104,10 @@ class AddTable(_Table):
         output = SparseConvNetTensor()
         output.metadata = input[0].metadata
         output.spatial_size = input[0].spatial_size
-        output.features = sum([i.features for i in input])
+        features = input[0].features  # the reference's sum(...) starts from 0: one pass more
+        for i in input[1:]:
+            features = features + i.features
+        output.features = features
         return output
 
     def input_spatial_size(self, out_size):

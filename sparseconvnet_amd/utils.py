@@ -1,5 +1,8 @@
 """Small helpers shared by the modules (same names and meaning as the reference's
 sparseconvnet/utils.py:11-26)."""
+import glob
+import os
+
 import torch
 
 
@@ -38,3 +41,45 @@ def prepare_BLInput(batch):
             locations[i, :loc.size(0)] = loc
             features[i, :feat.size(0)] = feat
     return [locations, features]
+
+
+def is_power2(num):
+    """utils.py:157-158."""
+    return num != 0 and ((num & (num - 1)) == 0)
+
+
+def checkpoint_restore(model, exp_name, name2, use_cuda=True, epoch=0):
+    """utils.py:138-155: loads `<exp_name>-<epoch, 9 digits>-<name2>.pth` (the newest one when
+    epoch is 0) into the model and returns the epoch to continue with; 1 when there is none.
+    The state dict is read with weights_only=True: parameter and buffer tensors only."""
+    if use_cuda:
+        model.cpu()
+    if epoch > 0:
+        f = exp_name + '-%09d-' % epoch + name2 + '.pth'
+        assert os.path.isfile(f)
+        print('Restore from ' + f)
+        model.load_state_dict(torch.load(f, weights_only=True))
+    else:
+        found = sorted(glob.glob(exp_name + '-*-' + name2 + '.pth'))
+        if len(found) > 0:
+            f = found[-1]
+            print('Restore from ' + f)
+            model.load_state_dict(torch.load(f, weights_only=True))
+            epoch = int(f[len(exp_name) + 1:-len(name2) - 5])
+    if use_cuda:
+        model.cuda()
+    return epoch + 1
+
+
+def checkpoint_save(model, exp_name, name2, epoch, use_cuda=True):
+    """utils.py:166-177: saves the state dict and removes the previous epoch's file unless its
+    number is a power of two."""
+    f = exp_name + '-%09d-' % epoch + name2 + '.pth'
+    model.cpu()
+    torch.save(model.state_dict(), f)
+    if use_cuda:
+        model.cuda()
+    epoch = epoch - 1
+    f = exp_name + '-%09d-' % epoch + name2 + '.pth'
+    if os.path.isfile(f) and not is_power2(epoch):
+        os.remove(f)

@@ -146,6 +146,23 @@ def test_residual_unet_structure():
     assert abs(scn.NetworkInNetwork(400, 300, False).weight.std().item() - (2.0 / 400) ** 0.5) < 2e-3
 
 
+def test_checkpoint_round_trip(tmp_path):
+    # utils.py:138-177: file naming, newest-epoch lookup, pruning of non-power-of-two epochs
+    torch.manual_seed(3)
+    a = scn.UNet(3, 1, [4, 8], False)
+    stem = str(tmp_path / "exp")
+    assert scn.checkpoint_restore(a, stem, "unet", use_cuda=False) == 1
+    for epoch in (1, 2, 3, 4, 5):
+        scn.checkpoint_save(a, stem, "unet", epoch, use_cuda=False)
+    kept = sorted(f.name for f in tmp_path.iterdir())
+    assert kept == ["exp-%09d-unet.pth" % e for e in (1, 2, 4, 5)]
+    b = scn.UNet(3, 1, [4, 8], False)
+    assert scn.checkpoint_restore(b, stem, "unet", use_cuda=False) == 6
+    for (ka, va), (kb, vb) in zip(a.state_dict().items(), b.state_dict().items()):
+        assert ka == kb and torch.equal(va, vb)
+    assert scn.is_power2(8) and not scn.is_power2(6) and not scn.is_power2(0)
+
+
 def test_no_cpu_fallback():
     from sparseconvnet_amd._lib import ScnError
     layer = scn.InputLayer(2, 8, mode=3)
