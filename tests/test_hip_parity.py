@@ -357,3 +357,52 @@ def test_input_above_2_gib_matches_split_channels():
         checks.assert_close(y.cpu().numpy(), want, "512 -> %d above 2 GiB" % cout)
         assert np.abs(want).max() > 0.1 and macs > 0
         del y, ya, yb
+
+
+def test_error_paths_leave_the_handle_usable(make):
+    """Every misuse comes back as a status plus message (ScnError here), no kernel runs on bad
+    operands, and the handle keeps working afterwards."""
+    import ctypes as C
+    import torch
+    from sparseconvnet_amd import _lib
+    from sparseconvnet_amd._lib import ScnError
+    L = _lib.lib()
+    assert L.scn_md_create(0) is None and L.scn_md_create(9) is None
+    assert b"dimension" in L.scn_last_error() or len(L.scn_last_error()) > 0
+    with pytest.raises(ScnError, match="null metadata handle"):
+        _lib.check(L.scn_md_clear(None))
+    p = make(3)
+    good = np.array([[1, 2, 3, 0], [4, 5, 6, 1], [1, 2, 3, 0]], np.int64)
+    for bad, what in (([[1, 2, 8, 0]], "outside"), ([[-1, 2, 3, 0]], "outside"), ([[1, 2, 3, -1]], "sample index")):
+        with pytest.raises(ScnError, match=what):
+            p.input_layer(8, np.array(bad, np.int64), 0, 3)
+        _lib.check(L.scn_md_clear(p.h))
+    with pytest.raises(ScnError, match="mode"):
+        p.input_layer(8, good, 0, 7)
+    _lib.check(L.scn_md_clear(p.h))
+    with pytest.raises(ScnError, match="every position filled"):
+        p.bl_input_layer(8, np.array([[[1, 1, 1], [-1, -1, -1]]], np.int64), 0)
+    _lib.check(L.scn_md_clear(p.h))
+    with pytest.raises(ScnError, match="not been built"):
+        p.input_rules()
+    assert p.input_layer(8, good, 0, 3) == 2
+    with pytest.raises(ScnError, match="already has an input layer"):
+        p.input_layer(8, good, 0, 3)
+    x = np.ones((2, 4), np.float32)
+    with pytest.raises(ScnError, match="kind"):
+        hdr = (C.c_int64 * 3)(8, 8, 8)
+        xd = torch.ones(2, 4, device="cuda")
+        _lib.check(L.scn_conv_bn_fwd(p.h, 5, hdr, hdr, None, None, C.c_void_p(xd.data_ptr()), C.c_void_p(xd.data_ptr()),
+                                     C.c_void_p(xd.data_ptr()), None, 4, 4, 1, None, None, None, None))
+    with pytest.raises(ScnError, match="planes must equal"):
+        sz = [p._s(v) for v in (8, 4, 2, 2)]
+        _lib.check(L.scn_md_strided_rules(p.h, *sz, None))
+        xd = torch.ones(2, 4, device="cuda")
+        _lib.check(L.scn_maxpool_fwd(p.h, *sz, C.c_void_p(xd.data_ptr()), 4, C.c_void_p(xd.data_ptr()), 4, 1, None))
+    with pytest.raises(ScnError, match="unknown spatial size"):
+        p.s2d(5, x)
+    with pytest.raises(ScnError, match="filter"):
+        p.submanifold_rules(8, 0)
+    # the handle still works
+    y, macs = p.subm_conv(8, 3, x, np.ones((27, 1, 4, 2), np.float32))
+    assert y.shape == (2, 2) and macs == 2 * 4 * 2 and (y == 4).all()
