@@ -171,7 +171,7 @@ __global__ void k_pack_weights(const float *w, float *wp, int K, int n_in, int n
 // in the layout of k_pack_weights.
 // Also clears the eight set counters (one per XCD, 128 bytes apart) of the launch it precedes.
 __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows, int n_in_part, int n_out,
-                                    int SS, int NCB, int *queue, CoefJobs jobs) {
+                                    int SS, int NCB, int *queue, CoefJobs jobs, bool as_bf16 = false) {
   coef_jobs(jobs);
   if (blockIdx.x == 0 && threadIdx.x < 8) queue[threadIdx.x * 32] = 0;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -184,9 +184,19 @@ __global__ void k_pack_weights_part(const float *w, float *wp, int K, int w_rows
   int q = e >> 8;
   int cb = q % NCB;
   int s = q / NCB;
+  if (as_bf16) {  // pairs of steps next to each other, 2-byte elements (see k_pack_weights)
+    lane = (e >> 3) & 63;
+    q = e >> 9;
+    cb = q % NCB;
+    s = 2 * (q / NCB) + ((e >> 2) & 1);
+  }
   int ch = s * 16 + 4 * (lane >> 4) + jj;
   int col = 16 * cb + (lane & 15);
-  wp[i] = (ch < n_in_part && col < n_out) ? w[((int64_t)k * w_rows + ch) * n_out + col] : 0.0f;
+  const float v = (ch < n_in_part && col < n_out) ? w[((int64_t)k * w_rows + ch) * n_out + col] : 0.0f;
+  if (as_bf16)
+    reinterpret_cast<__bf16 *>(wp)[i] = (__bf16)v;
+  else
+    wp[i] = v;
 }
 
 // ---- MFMA kernel ------------------------------------------------------------------------
@@ -899,7 +909,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
 // the end re-read the first set).  Granules none of whose rows has the tap skip their MFMAs.
 // With accumulate != 0 the kernel adds to `out` instead of overwriting it (used to split a
 // wide nIn into several launches).
-template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF>
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF, bool BF16>
 __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
     int64_t n, int64_t npad, const float *__restrict__ in, int in_stride, float *__restrict__ out,
@@ -907,6 +917,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     int sets_per_xcd, int accumulate, int *__restrict__ queue, unsigned in_bytes, unsigned nbr_bytes) {
   static_assert(!BUF || VEC4 || C4, "buffer gathers need float4 rows or the four-channel layout");
   static_assert(!C4 || SS == 1, "the four-channel layout has one slab");
+  static_assert(!BF16 || (BUF && !C4 && SS == 2), "the bf16 variant: buffer gathers, one pair of steps");
   // C4 (nIn <= 4): the MFMA's k index is the input channel itself, so a lane gathers one
   // float (row r16, channel g) and a tap costs one MFMA per column block instead of four.
   using AV = typename std::conditional<C4, float, v4f>::type;
@@ -915,7 +926,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r16 = lane & 15, g = lane >> 4;
-  const int total_f4 = C4 ? K * NCB * 16 : K * SS * NCB * 64;
+  const int total_f4 = C4 ? K * NCB * 16 : (BF16 ? K * NCB * 64 : K * SS * NCB * 64);
   for (int e = threadIdx.x; e < total_f4; e += WAVES * 64) wl[e] = reinterpret_cast<const v4f *>(wp)[e];
   __syncthreads();  // the only barrier; every wavefront reaches it
 
@@ -1088,6 +1099,19 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 #pragma unroll
           for (int cb = 0; cb < NCB; cb++) acc[q][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[cb], acc[q][cb], 0, 0, 0);
         }
+      } else if constexpr (BF16) {
+        // one operand per column block holds both steps (bf16); the gathered rows are rounded here
+        v4f b[NCB];
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) b[cb] = wl[(k_cur * NCB + cb) * 64 + lane];
+#pragma unroll
+        for (int q = 0; q < RG; q++) {
+          const bool ok = (okb >> q) & 1u;
+          if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
+          const v8s av = to_bf16x8(ar[S][q][0], ar[S][q][1]);
+#pragma unroll
+          for (int cb = 0; cb < NCB; cb++) acc[q][cb] = mfma_bf16(av, __builtin_bit_cast(v8s, b[cb]), acc[q][cb]);
+        }
       } else {
         v4f b[SS][NCB];
 #pragma unroll
@@ -1175,7 +1199,7 @@ __global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, in
   wp[i] = (ch < n_in && col < n_out) ? w[((int64_t)k * n_in + ch) * n_out + col] : 0.0f;
 }
 
-template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF = false>
+template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF = false, bool BF16 = false>
 static void launch_resident_kernel(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
                                    Epi epi, int n_in_part, int n_out, int accumulate, size_t lds_bytes,
                                    int per_cu, hipStream_t s) {
@@ -1186,12 +1210,15 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
     const bool whole = C4 || n_in_part == 16 * SS;
     if (whole && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) && in_stride * 4 < (1 << 24) && in_bytes > 0 &&
         in_bytes < ((int64_t)1 << 31) && nbr_bytes < ((int64_t)1 << 31)) {
-      launch_resident_kernel<NCB, RG, SS, VEC4, WAVES, C4, true>(m, t, in, in_stride, out, epi, n_in_part, n_out,
-                                                                 accumulate, lds_bytes, per_cu, s);
+      launch_resident_kernel<NCB, RG, SS, VEC4, WAVES, C4, true, BF16>(m, t, in, in_stride, out, epi, n_in_part,
+                                                                       n_out, accumulate, lds_bytes, per_cu, s);
       return;
     }
   }
-  auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, C4, BUF>;
+  if constexpr (BF16 && !BUF) {
+    throw Error("internal: the bf16 resident kernel needs buffer gathers");
+  } else {
+  auto kern = k_conv_resident<NCB, RG, SS, VEC4, WAVES, C4, BUF, BF16>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1205,6 +1232,15 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
                                                    out, m.wpack.p, epi, n_in_part, n_out, n_sets, sets_per_xcd,
                                                    accumulate, m.queue.p, (unsigned)in_bytes, (unsigned)nbr_bytes);
   LAUNCH_CHECK();
+  }
+}
+
+// Whether launch_resident_kernel would take its buffer-gather variant for this input.
+static bool resident_buffer_gathers(const Metadata &m, const Table &t, const float *in, int in_stride) {
+  const int64_t in_bytes = (m.cur_in_rows * in_stride - (in - m.cur_in_base)) * 4;
+  const int64_t nbr_bytes = (int64_t)t.K * t.npad * 4;
+  return m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) && in_stride * 4 < (1 << 24) && in_bytes > 0 &&
+         in_bytes < ((int64_t)1 << 31) && nbr_bytes < ((int64_t)1 << 31);
 }
 
 // One launch over channels [c_lo, c_lo + n_in_part) of the input rows.
@@ -1216,6 +1252,23 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
   m.wpack.reserve(packed);
   m.queue.reserve(8 * 32);
+  if constexpr (SS == 2 && VEC4) {
+    // bf16 operands (when asked for): a whole 32-channel part, buffer gathers
+    if (m.bf16 && n_in_part == 32 && resident_buffer_gathers(m, t, in, in_stride)) {
+      k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(
+          w, m.wpack.p, t.K, w_in_stride_rows, n_in_part, n_out, SS, NCB, m.queue.p, take_jobs(m), true);
+      LAUNCH_CHECK();
+      const size_t lds16 = (size_t)packed * 2;  // 2-byte elements
+      const int per_cu16 = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds16));
+      if (lds16 > 80 * 1024)
+        launch_resident_kernel<NCB, RG, SS, VEC4, 16, false, true, true>(m, t, in, in_stride, out, epi, n_in_part, n_out,
+                                                                         accumulate, lds16, 1, s);
+      else
+        launch_resident_kernel<NCB, RG, SS, VEC4, 8, false, true, true>(m, t, in, in_stride, out, epi, n_in_part, n_out,
+                                                                        accumulate, lds16, per_cu16, s);
+      return;
+    }
+  }
   // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
   k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, w_in_stride_rows,
                                                                            n_in_part, n_out, SS, NCB, m.queue.p,

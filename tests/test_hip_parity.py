@@ -227,7 +227,7 @@ def _neighbour_counts(coords, spatial):
     return present
 
 
-@pytest.mark.parametrize("cin,cout", [(64, 64), (64, 32), (128, 128), (96, 160), (256, 256), (128, 32)])
+@pytest.mark.parametrize("cin,cout", [(32, 32), (32, 16), (64, 64), (64, 32), (128, 128), (96, 160), (256, 256), (128, 32)])
 def test_bf16_path_vs_oracle(oracle_built, cin, cout):
     """The optional bf16-operand path: submanifold convolution (with and without a batch norm
     in front), strided convolution and deconvolution against the fp32 oracle, within 1e-2 of
