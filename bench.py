@@ -380,7 +380,7 @@ def main():
         # Optional reduced-precision path (bf16 operands, fp32 accumulation), same work, listed
         # beside the fp32 sweep; `value` and `roofline` above are fp32 only.
         _lib.check(L.scn_md_set_bf16(h, 1))
-        wide = [(i, wk) for i, wk in enumerate(work) if wk[0] >= 64]
+        wide = [(i, wk) for i, wk in enumerate(work) if wk[0] >= 32]
         for _, wk in wide:
             conv(*wk)
         torch.cuda.synchronize()
