@@ -1000,7 +1000,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   };
   // Register rings, indexed by item number mod 3 (the loop below is unrolled three times so
   // that every index is a constant): neighbour indices, gathered rows, row-present bits.
-  int jr[3][RG];
+  int jr[3][1];
   AV ar[3][RG][SS];
   unsigned okr[3];
   // BUF: neighbour table and input rows are read through buffer loads (32-bit offsets; an
@@ -1013,20 +1013,24 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
       __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(nbr), 0, BUF ? (int)nbr_bytes : 0, 0x00020000);
   const unsigned row_bytes = (unsigned)in_stride * 4u;
   const unsigned lane_off = C4 ? (g < n_in ? 4u * (unsigned)g : 0x80000000u) : 16u * (unsigned)g;
+  // One load fetches the indices of the whole set (lane l: row l of the set); issue_a hands
+  // each lane the index of its own row of every granule through a lane permute, which costs an
+  // LDS-crossbar instruction instead of a memory instruction per granule.
+  const int set_lane = lane % (RG * 16);
   auto issue_j = [&](const Item &it, int *j) {
-#pragma unroll
-    for (int q = 0; q < RG; q++) {
-      if constexpr (BUF) {
-        const unsigned t = min((unsigned)it.set * (RG * 16) + q * 16 + r16, (unsigned)(n - 1));
-        j[q] = __builtin_amdgcn_raw_buffer_load_b32(nbr_rsrc, t * 4u, (unsigned)it.k * (unsigned)npad * 4u, 0);
-      } else {
-        const int64_t t = min((int64_t)it.set * (RG * 16) + q * 16 + r16, n - 1);
-        j[q] = nbr[(int64_t)it.k * npad + t];
-      }
+    if constexpr (BUF) {
+      const unsigned t = min((unsigned)it.set * (RG * 16) + set_lane, (unsigned)(n - 1));
+      j[0] = __builtin_amdgcn_raw_buffer_load_b32(nbr_rsrc, t * 4u, (unsigned)it.k * (unsigned)npad * 4u, 0);
+    } else {
+      const int64_t t = min((int64_t)it.set * (RG * 16) + set_lane, n - 1);
+      j[0] = nbr[(int64_t)it.k * npad + t];
     }
   };
-  auto issue_a = [&](const Item &it, const int *j, AV (*a)[SS], unsigned &okbits) {
+  auto issue_a = [&](const Item &it, const int *jset, AV (*a)[SS], unsigned &okbits) {
     okbits = 0;
+    int j[RG];
+#pragma unroll
+    for (int q = 0; q < RG; q++) j[q] = __shfl(jset[0], q * 16 + r16, 64);
 #pragma unroll
     for (int q = 0; q < RG; q++) {
       const bool ok = j[q] >= 0 && (int64_t)it.set * (RG * 16) + q * 16 + r16 < n;
