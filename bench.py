@@ -28,7 +28,7 @@ PAIRS = [(3, 32), (32, 32), (64, 64), (128, 128), (256, 256)]
 # HBM-side bytes per launch on the default workload (1,000,000 sites, seed 3000, shuffled), from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE passes scaled by a 1 GiB copy kernel (x2.000 / x1.000):
 # profiles/conv256_sweep1M_pmc.txt.  Only reported when the run is that workload.
-MEASURED_TRAFFIC = {(256, 256): 7.77e9, (128, 128): 1.62e9, (64, 64): 0.783e9, (32, 32): 0.430e9, (3, 32): 0.432e9}
+MEASURED_TRAFFIC = {(256, 256): 7.70e9, (128, 128): 1.62e9, (64, 64): 0.782e9, (32, 32): 0.430e9, (3, 32): 0.501e9}
 
 
 def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
