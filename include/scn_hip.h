@@ -48,6 +48,15 @@ void scn_md_destroy(scn_metadata *md);
 /* Metadata::clear (Metadata/Metadata.cpp:52-66). */
 int scn_md_clear(scn_metadata *md);
 
+/* Rulebooks depend on coordinates only.  By default the library builds them on a stream of its
+ * own (one per device, default priority) and orders that stream against the stream argument of
+ * each call with events, so that the construction of the next level's rulebook runs beside the
+ * convolutions already enqueued: a new scene's forward pass then costs little more than its
+ * convolutions.  Results are the same either way.  enable = 0 builds on the caller's stream
+ * (also: SCN_BUILD_STREAM=0 in the environment); returns the previous setting.  Process-wide;
+ * affects constructions started afterwards.  No counterpart in the reference, whose rulebooks
+ * are built on the host. */
+int scn_set_build_stream(int enable);
 /* Optional reduced-precision path (no counterpart in the reference, which computes in fp32
  * throughout): with enable != 0 the convolutions of this handle whose input rows consist of
  * whole 32-channel slabs and that run in the two wide kernel families (more than 32 output

@@ -26,6 +26,7 @@ SIGNATURES = {
     "scn_md_create": (_vp, [C.c_int]),
     "scn_md_destroy": (None, [_vp]),
     "scn_md_clear": (C.c_int, [_vp]),
+    "scn_set_build_stream": (C.c_int, [C.c_int]),
     "scn_md_set_bf16": (C.c_int, [_vp, C.c_int]),
     "scn_md_input_layer": (C.c_int, [_vp, _i64p, _vp, C.c_int64, C.c_int, C.c_int, C.c_int, _vp, _i64p]),
     "scn_md_input_rules_header": (C.c_int, [_vp, C.POINTER(C.c_int32)]),

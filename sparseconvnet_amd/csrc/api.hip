@@ -12,13 +12,15 @@ struct scn_metadata {
 static thread_local std::string g_error;
 
 // ---- block cache behind DevBuf (see common.h) -----------------------------------------------
+#include <atomic>
 #include <map>
 #include <mutex>
+#include <tuple>
 
 namespace scn {
 namespace {
 std::mutex g_pool_mutex;
-std::multimap<std::pair<int, size_t>, void *> g_pool;  // (device, size class) -> free blocks
+std::multimap<std::tuple<int, int, size_t>, void *> g_pool;  // (device, cache, size class) -> free blocks
 
 int current_device() {
   int d = 0;
@@ -35,11 +37,16 @@ size_t size_class(size_t bytes) {
 }
 }  // namespace
 
-void *pool_alloc(size_t bytes) {
+int &pool_scope() {
+  static thread_local int scope = POOL_COMPUTE;
+  return scope;
+}
+
+void *pool_alloc(size_t bytes, int pool) {
   const size_t cls = size_class(bytes ? bytes : 1);
   {
     std::lock_guard<std::mutex> lock(g_pool_mutex);
-    auto it = g_pool.find(std::make_pair(current_device(), cls));
+    auto it = g_pool.find(std::make_tuple(current_device(), pool, cls));
     if (it != g_pool.end()) {
       void *p = it->second;
       g_pool.erase(it);
@@ -59,12 +66,12 @@ void *pool_alloc(size_t bytes) {
   return p;
 }
 
-void pool_free(void *p, size_t bytes) {
+void pool_free(void *p, size_t bytes, int pool) {
   if (!p) return;
   std::lock_guard<std::mutex> lock(g_pool_mutex);
   hipPointerAttribute_t attr;
   int dev = hipPointerGetAttributes(&attr, p) == hipSuccess ? attr.device : current_device();
-  g_pool.emplace(std::make_pair(dev, size_class(bytes ? bytes : 1)), p);
+  g_pool.emplace(std::make_tuple(dev, pool, size_class(bytes ? bytes : 1)), p);
 }
 }  // namespace scn
 
@@ -86,6 +93,144 @@ static Metadata &md(scn_metadata *h) {
   return h->m;
 }
 static hipStream_t st(void *s) { return (hipStream_t)s; }
+
+// ---- two streams -------------------------------------------------------------------------------
+// Rulebooks depend on coordinates only, never on features.  They are built on a stream of the
+// library's own (one per device, default priority), so that the many small kernels and the few
+// host round trips of a construction run beside the convolutions already enqueued on the
+// caller's stream instead of between them: the host gets ahead of the GPU, and a new scene's
+// forward pass costs little more than its convolutions.  Ordering:
+//   * a construction that reads the caller's data (the input layer's coordinates) first makes
+//     the build stream wait for the caller's stream;
+//   * behind every construction an event is recorded; every feature pass (and everything else
+//     that reads rulebooks on the caller's stream) first makes its stream wait for the latest one;
+//   * before a construction drops or overwrites something a feature pass may be reading, and
+//     before a handle is destroyed, the build stream waits for the caller's stream.
+// scn_set_build_stream(0), or SCN_BUILD_STREAM=0 in the environment, builds on the caller's
+// stream as a single-stream library would.
+static std::atomic<int> g_build_stream{-1};  // -1: not decided yet (environment), 0 / 1
+static bool use_build_stream() {
+  int v = g_build_stream.load();
+  if (v < 0) {
+    const char *e = getenv("SCN_BUILD_STREAM");
+    v = (e && e[0] == '0') ? 0 : 1;
+    g_build_stream.store(v);
+  }
+  return v != 0;
+}
+static hipStream_t device_build_stream() {
+  static std::mutex mu;
+  static std::map<int, hipStream_t> streams;
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = streams.find(dev);
+  if (it != streams.end()) return it->second;
+  hipStream_t s;
+  HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  streams[dev] = s;
+  return s;
+}
+
+struct BuildScope {
+  Metadata &m;
+  hipStream_t caller, bs;
+  uint64_t builds0;
+  int pool0;
+  bool force = false;  // record the event even if no construction was counted
+  // reads_caller_data: the construction reads buffers the caller filled on its stream, or
+  // writes buffers the caller will read there
+  BuildScope(Metadata &m_, void *stream, bool reads_caller_data = false)
+      : m(m_), caller(st(stream)), bs(use_build_stream() ? device_build_stream() : st(stream)),
+        builds0(m_.builds), pool0(pool_scope()) {
+    pool_scope() = POOL_BUILD;
+    if (bs != caller && reads_caller_data) {
+      hipEvent_t ev;
+      HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+      HIP_CHECK(hipEventRecord(ev, caller));
+      HIP_CHECK(hipStreamWaitEvent(bs, ev, 0));
+      HIP_CHECK(hipEventDestroy(ev));
+    }
+  }
+  hipStream_t s() const { return bs; }
+  ~BuildScope() {
+    pool_scope() = pool0;
+    if (bs == caller || (m.builds == builds0 && !force)) return;
+    m.build_stream = bs;
+    hipEvent_t &ev = m.ready[m.ready_next];
+    m.ready_next = (m.ready_next + 1) % 8;
+    if (!ev && hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+      ev = nullptr;
+      (void)hipStreamSynchronize(bs);  // no event to hand out: fall back to waiting here
+      m.last_ready = nullptr;
+      return;
+    }
+    if (hipEventRecord(ev, bs) != hipSuccess) {
+      (void)hipStreamSynchronize(bs);
+      m.last_ready = nullptr;
+      return;
+    }
+    m.last_ready = ev;
+    m.consumer_waited = false;
+  }
+};
+
+// Called by everything that reads rulebooks or levels on the caller's stream.
+static void consume(Metadata &m, hipStream_t s) {
+  if (m.last_ready && (!m.consumer_waited || !m.consumer_known || m.consumer != s))
+    HIP_CHECK(hipStreamWaitEvent(s, m.last_ready, 0));
+  m.consumer = s;
+  m.consumer_known = true;
+  m.consumer_waited = true;
+}
+
+static void retire(Metadata &m) {  // before the handle's buffers go back to the caches
+  if (m.build_stream) {
+    try {
+      wait_for_consumers(m, m.build_stream);
+    } catch (...) {
+      (void)hipDeviceSynchronize();
+    }
+  }
+  for (hipEvent_t &e : m.ready) {
+    if (e) (void)hipEventDestroy(e);
+    e = nullptr;
+  }
+  m.last_ready = nullptr;
+}
+
+// Table lookups that may have to build: the construction runs on the build stream, then the
+// caller's stream is made to wait for it.
+static Table &subm_table(Metadata &m, const int64_t *spatial, const int64_t *filter, void *stream) {
+  Table *t;
+  {
+    BuildScope b(m, stream);
+    t = &submanifold_rules(m, spatial, filter, b.s());
+  }
+  consume(m, st(stream));
+  return *t;
+}
+static StridedRules &strided_table(Metadata &m, const int64_t *in_size, const int64_t *out_size,
+                                   const int64_t *filter, const int64_t *stride, void *stream) {
+  StridedRules *r;
+  {
+    BuildScope b(m, stream);
+    r = &strided_rules(m, in_size, out_size, filter, stride, b.s());
+  }
+  consume(m, st(stream));
+  return *r;
+}
+// Exports and other rarely used calls run wholly on the build stream, ordered against the
+// caller's stream on both sides (they read and write the caller's buffers and use the
+// constructions' scratch).
+template <class F> static void on_build_stream(Metadata &m, void *stream, F f) {
+  {
+    BuildScope b(m, stream, true);
+    b.force = true;
+    f(b.s());
+  }
+  consume(m, st(stream));
+}
 
 static Level *find_level(Metadata &m, const int64_t *spatial) {
   auto it = m.levels.find(mk(m.dim, spatial));
@@ -111,10 +256,17 @@ scn_metadata *scn_md_create(int dim) {
     return nullptr;
   }
 }
-void scn_md_destroy(scn_metadata *h) { delete h; }
+void scn_md_destroy(scn_metadata *h) {
+  if (!h) return;
+  retire(h->m);
+  const int scope = pool_scope();
+  delete h;
+  pool_scope() = scope;
+}
 int scn_md_clear(scn_metadata *h) {
   return guarded([&] {
     Metadata &m = md(h);
+    retire(m);
     int dim = m.dim;
     m.levels.clear();
     m.subm.clear();
@@ -125,6 +277,11 @@ int scn_md_clear(scn_metadata *h) {
   });
 }
 
+int scn_set_build_stream(int enable) {
+  const int before = use_build_stream() ? 1 : 0;
+  g_build_stream.store(enable ? 1 : 0);
+  return before;
+}
 int scn_md_set_bf16(scn_metadata *h, int enable) {
   return guarded([&] { md(h).bf16 = enable != 0; });
 }
@@ -134,7 +291,8 @@ int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *c
     Metadata &m = md(h);
     if (n < 0) throw Error("negative point count");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
-    build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, st(stream));
+    BuildScope b(m, stream, true);
+    build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, b.s());
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -155,7 +313,8 @@ int scn_md_bl_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t
     if (batch < 0 || length < 0) throw Error("negative batch size or length");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
     if (batch * length == 0) length = 1, batch = 0;
-    build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, st(stream), length);
+    BuildScope b(m, stream, true);
+    build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, b.s(), length);
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -171,7 +330,10 @@ int scn_md_bl_rules_header(scn_metadata *h, int32_t hdr[5]) {
   });
 }
 int scn_md_input_rules(scn_metadata *h, int32_t *rows, void *stream) {
-  return guarded([&] { export_input_rules(md(h), rows, st(stream)); });
+  return guarded([&] {
+    Metadata &m = md(h);
+    on_build_stream(m, stream, [&](hipStream_t s) { export_input_rules(m, rows, s); });
+  });
 }
 int scn_md_nactive(scn_metadata *h, const int64_t *spatial, int64_t *n_active) {
   return guarded([&] {
@@ -186,14 +348,25 @@ int scn_md_batch_size(scn_metadata *h, const int64_t *spatial, int *batch) {
   });
 }
 int scn_md_spatial_locations(scn_metadata *h, const int64_t *spatial, int64_t *out, void *stream) {
-  return guarded([&] { spatial_locations(md(h), spatial, out, st(stream)); });
+  return guarded([&] {
+    Metadata &m = md(h);
+    on_build_stream(m, stream, [&](hipStream_t s) { spatial_locations(m, spatial, out, s); });
+  });
 }
 int scn_md_submanifold_rules(scn_metadata *h, const int64_t *spatial, const int64_t *filter, void *stream) {
-  return guarded([&] { submanifold_rules(md(h), spatial, filter, st(stream)); });
+  return guarded([&] {
+    Metadata &m = md(h);
+    BuildScope b(m, stream);
+    submanifold_rules(m, spatial, filter, b.s());
+  });
 }
 int scn_md_strided_rules(scn_metadata *h, const int64_t *in_size, const int64_t *out_size,
                          const int64_t *filter, const int64_t *stride, void *stream) {
-  return guarded([&] { strided_rules(md(h), in_size, out_size, filter, stride, st(stream)); });
+  return guarded([&] {
+    Metadata &m = md(h);
+    BuildScope b(m, stream);
+    strided_rules(m, in_size, out_size, filter, stride, b.s());
+  });
 }
 
 int scn_rules_count(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
@@ -201,9 +374,9 @@ int scn_rules_count(scn_metadata *h, int kind, const int64_t *a, const int64_t *
   return guarded([&] {
     Metadata &m = md(h);
     if (kind == 0)
-      *count = submanifold_rules(m, a, b, st(stream)).K;
+      *count = subm_table(m, a, b, stream).K;
     else if (kind == 1)
-      *count = strided_rules(m, a, b, c, d, st(stream)).by_out.K;
+      *count = strided_table(m, a, b, c, d, stream).by_out.K;
     else if (kind == 2) {
       Level *l = find_level(m, a);
       *count = l ? l->batch : 0;
@@ -212,7 +385,11 @@ int scn_rules_count(scn_metadata *h, int kind, const int64_t *a, const int64_t *
   });
 }
 int scn_md_take_macs(scn_metadata *h, void *stream, double *macs) {
-  return guarded([&] { *macs = take_macs(md(h), st(stream)); });
+  return guarded([&] {
+    Metadata &m = md(h);
+    consume(m, st(stream));
+    *macs = take_macs(m, st(stream));
+  });
 }
 int scn_rules_sizes(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
                     const int64_t *d, void *stream, int64_t *sizes) {
@@ -220,11 +397,11 @@ int scn_rules_sizes(scn_metadata *h, int kind, const int64_t *a, const int64_t *
     Metadata &m = md(h);
     std::vector<int64_t> v;
     if (kind == 0) {
-      v = submanifold_rules(m, a, b, st(stream)).counts(st(stream));
+      v = subm_table(m, a, b, stream).counts(st(stream));
     } else if (kind == 1) {
-      v = strided_rules(m, a, b, c, d, st(stream)).by_out.counts(st(stream));
+      v = strided_table(m, a, b, c, d, stream).by_out.counts(st(stream));
     } else if (kind == 2)
-      v = s2d_sizes(m, a, st(stream));
+      on_build_stream(m, stream, [&](hipStream_t s) { v = s2d_sizes(m, a, s); });
     else
       throw Error("unknown rulebook kind");
     for (size_t i = 0; i < v.size(); i++) sizes[i] = v[i];
@@ -235,23 +412,33 @@ int scn_rules_export(scn_metadata *h, int kind, const int64_t *a, const int64_t 
   return guarded([&] {
     Metadata &m = md(h);
     if (kind == 0) {
-      Table &t = submanifold_rules(m, a, b, st(stream));
-      export_table_pairs(m, t, k, false, pairs, st(stream));
+      on_build_stream(m, stream, [&](hipStream_t s) {
+        Table &t = submanifold_rules(m, a, b, s);
+        export_table_pairs(m, t, k, false, pairs, s);
+      });
     } else if (kind == 1) {
-      StridedRules &r = strided_rules(m, a, b, c, d, st(stream));
-      export_table_pairs(m, r.by_out, k, false, pairs, st(stream));
+      on_build_stream(m, stream, [&](hipStream_t s) {
+        StridedRules &r = strided_rules(m, a, b, c, d, s);
+        export_table_pairs(m, r.by_out, k, false, pairs, s);
+      });
     } else if (kind == 2) {
-      export_s2d_pairs(m, a, k, pairs, st(stream));
+      on_build_stream(m, stream, [&](hipStream_t s) { export_s2d_pairs(m, a, k, pairs, s); });
     } else
       throw Error("unknown rulebook kind");
   });
 }
 
 int scn_input_layer_fwd(scn_metadata *h, const float *in, float *out, int planes, void *stream) {
-  return guarded([&] { input_forward(md(h).input, in, out, planes, st(stream)); });
+  return guarded([&] {
+    consume(md(h), st(stream));
+    input_forward(md(h).input, in, out, planes, st(stream));
+  });
 }
 int scn_output_layer_fwd(scn_metadata *h, const float *in, float *out, int planes, void *stream) {
-  return guarded([&] { output_forward(md(h).input, in, out, planes, st(stream)); });
+  return guarded([&] {
+    consume(md(h), st(stream));
+    output_forward(md(h).input, in, out, planes, st(stream));
+  });
 }
 
 static int64_t level_rows(Metadata &m, const int64_t *spatial) {
@@ -262,7 +449,7 @@ static void subm_conv(scn_metadata *h, const int64_t *spatial, const int64_t *fi
                       const float *weight, const float *bias, int n_in, int n_out, int groups, const BnArgs *pre,
                       const BnArgs *post, void *stream, double *macs) {
   Metadata &m = md(h);
-  Table &t = submanifold_rules(m, spatial, filter, st(stream));
+  Table &t = subm_table(m, spatial, filter, stream);
   conv_forward(m, t, in, level_rows(m, spatial), out, weight, bias, n_in, n_out, groups, pre, post, st(stream));
   // CPU/Convolution.cpp:141: nRules * ip * op * groups per tap
   note_macs(m, t, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
@@ -272,7 +459,7 @@ static void strided_conv(scn_metadata *h, const int64_t *in_size, const int64_t 
                          const float *bias, int n_in, int n_out, int groups, const BnArgs *pre, const BnArgs *post,
                          void *stream, double *macs) {
   Metadata &m = md(h);
-  StridedRules &r = strided_rules(m, in_size, out_size, filter, stride, st(stream));
+  StridedRules &r = strided_table(m, in_size, out_size, filter, stride, stream);
   conv_forward(m, r.by_out, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
                st(stream));
   note_macs(m, r.by_out, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
@@ -283,7 +470,7 @@ static void deconv(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
                    double *macs) {
   Metadata &m = md(h);
   // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
-  StridedRules &r = strided_rules(m, out_size, in_size, filter, stride, st(stream));
+  StridedRules &r = strided_table(m, out_size, in_size, filter, stride, stream);
   conv_forward(m, r.by_in, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
                st(stream));
   note_macs(m, r.by_in, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
@@ -340,7 +527,13 @@ int scn_nin_fwd(scn_metadata *h, const float *in, float *out, const float *weigh
   return guarded([&] {
     Metadata &m = md(h);
     if (rows < 0 || rows >= ((int64_t)1 << 31)) throw Error("network in network: row count out of range");
-    Table &t = identity_table(m, rows, st(stream));
+    Table *tp;
+    {
+      BuildScope b(m, stream);
+      tp = &identity_table(m, rows, b.s());
+    }
+    consume(m, st(stream));
+    Table &t = *tp;
     conv_forward(m, t, in, rows, out, weight, bias, n_in, n_out, 1, nullptr, nullptr, st(stream));
     // CPU/NetworkInNetwork.cpp:22: nActive * input_nPlanes * output_nPlanes
     note_macs(m, t, (double)n_in * n_out, macs, st(stream));
@@ -352,7 +545,7 @@ int scn_maxpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_
   return guarded([&] {
     Metadata &m = md(h);
     if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
-    StridedRules &r = strided_rules(m, in_size, out_size, size, stride, st(stream));
+    StridedRules &r = strided_table(m, in_size, out_size, size, stride, stream);
     maxpool_forward(r.by_out, in, in_stride, out, planes, n_features_to_drop, st(stream));
   });
 }
@@ -362,7 +555,7 @@ int scn_avgpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_
   return guarded([&] {
     Metadata &m = md(h);
     if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
-    StridedRules &r = strided_rules(m, in_size, out_size, size, stride, st(stream));
+    StridedRules &r = strided_table(m, in_size, out_size, size, stride, stream);
     avgpool_forward(r.by_out, in, in_stride, out, planes, n_features_to_drop, st(stream));
   });
 }
@@ -373,7 +566,7 @@ int scn_unpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
     Metadata &m = md(h);
     if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
     // CPU/UnPooling.cpp:43-44: the rulebook of (out_size -> in_size), read from the fine side
-    StridedRules &r = strided_rules(m, out_size, in_size, size, stride, st(stream));
+    StridedRules &r = strided_table(m, out_size, in_size, size, stride, stream);
     unpool_forward(r.by_in, in, in_stride, out, planes, n_features_to_drop, st(stream));
   });
 }
@@ -390,6 +583,7 @@ int scn_s2d_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float 
   return guarded([&] {
     Level *l = find_level(md(h), spatial);
     if (!l) throw Error("sparse to dense: unknown spatial size");
+    consume(md(h), st(stream));
     s2d_forward(*l, in, out, planes, st(stream));
   });
 }

@@ -33,24 +33,32 @@ inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 // Device memory for the library's own buffers comes from a process-wide cache: blocks freed
 // by one metadata object are handed to the next instead of going back to the driver, so a
 // steady stream of scenes performs no hipMalloc / hipFree (each of which stalls the host,
-// and hipFree the whole device).  Blocks are reused in the order work is enqueued: callers
-// that drive one process from several streams must order those streams themselves.
-void *pool_alloc(size_t bytes);
-void pool_free(void *p, size_t bytes);
+// and hipFree the whole device).  Blocks are reused in the order work is enqueued.  The
+// library enqueues on two streams, the caller's (convolutions and the other feature passes)
+// and its own build stream (rulebook construction, see api.hip), so there are two caches and
+// a block never moves from one to the other: whatever a thread allocates while it builds
+// rulebooks (pool_scope() == POOL_BUILD) comes from and returns to the build cache.  Callers
+// that drive one process from several streams of their own must order those themselves.
+enum { POOL_COMPUTE = 0, POOL_BUILD = 1 };
+int &pool_scope();  // the calling thread's current cache
+void *pool_alloc(size_t bytes, int pool);
+void pool_free(void *p, size_t bytes, int pool);
 
 // Owning device buffer.  Grows by reallocation (contents discarded).
 template <class T> struct DevBuf {
   T *p = nullptr;
   size_t cap = 0;  // elements
+  int pool = POOL_COMPUTE;  // the cache the block came from
   DevBuf() = default;
   DevBuf(const DevBuf &) = delete;
   DevBuf &operator=(const DevBuf &) = delete;
-  DevBuf(DevBuf &&o) noexcept : p(o.p), cap(o.cap) { o.p = nullptr; o.cap = 0; }
+  DevBuf(DevBuf &&o) noexcept : p(o.p), cap(o.cap), pool(o.pool) { o.p = nullptr; o.cap = 0; }
   DevBuf &operator=(DevBuf &&o) noexcept {
     if (this != &o) {
       release();
       p = o.p;
       cap = o.cap;
+      pool = o.pool;
       o.p = nullptr;
       o.cap = 0;
     }
@@ -58,14 +66,15 @@ template <class T> struct DevBuf {
   }
   ~DevBuf() { release(); }
   void release() {
-    if (p) pool_free(p, cap * sizeof(T));
+    if (p) pool_free(p, cap * sizeof(T), pool);
     p = nullptr;
     cap = 0;
   }
   void reserve(size_t n) {
     if (n <= cap) return;
     release();
-    p = static_cast<T *>(pool_alloc(n * sizeof(T)));
+    pool = pool_scope();
+    p = static_cast<T *>(pool_alloc(n * sizeof(T), pool));
     cap = n;
   }
   size_t bytes() const { return cap * sizeof(T); }

@@ -139,7 +139,21 @@ struct Metadata {
   // inputs) round their operands to bf16 and run the bf16 MFMA with fp32 accumulation when the
   // input consists of whole 32-channel slabs; off unless the caller asks for it.
   bool bf16 = false;
+  // Ordering between the stream rulebooks are built on and the stream the caller's feature
+  // passes run on (api.hip: BuildScope, consume).
+  uint64_t builds = 0;              // bumped by every construction that enqueued work
+  hipStream_t build_stream = nullptr;  // where the last construction ran (null: none yet)
+  hipEvent_t ready[8] = {};         // ring of events recorded behind constructions
+  int ready_next = 0;
+  hipEvent_t last_ready = nullptr;  // what a feature pass has to wait for; null: nothing outstanding
+  hipStream_t consumer = nullptr;   // the stream feature passes were last enqueued on ...
+  bool consumer_known = false;
+  bool consumer_waited = true;      // ... and whether it has been made to wait for last_ready
 };
+
+// Makes stream s wait for the feature passes enqueued so far on the caller's stream (before a
+// construction overwrites or frees something they may still be reading).
+void wait_for_consumers(Metadata &m, hipStream_t s);
 
 SizeKey mk(int dim, const int64_t *a, const int64_t *b = nullptr, const int64_t *c = nullptr);
 Geom make_geom(int dim, const int64_t *spatial);

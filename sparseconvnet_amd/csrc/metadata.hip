@@ -72,6 +72,15 @@ static int key_bits(const Geom &g, int64_t batch) {
 
 // ---- small utilities -------------------------------------------------------------------
 
+void wait_for_consumers(Metadata &m, hipStream_t s) {
+  if (!m.consumer_known || m.consumer == s) return;
+  hipEvent_t ev;
+  HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  HIP_CHECK(hipEventRecord(ev, m.consumer));
+  HIP_CHECK(hipStreamWaitEvent(s, ev, 0));
+  HIP_CHECK(hipEventDestroy(ev));  // released once it has completed
+}
+
 static const int COUNT_SLOTS = 32;  // copies of a rulebook's per-tap counters (a power of two)
 
 __global__ void k_fill32(uint32_t *p, uint32_t v, int64_t n) {
@@ -295,6 +304,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   R.bl_length = bl_length;
   R.bl_batch = bl ? n / bl_length : 0;
   int batch_floor = bl ? (int)R.bl_batch : (ncols == m.dim ? 1 : std::max(min_batch, 0));
+  m.builds++;
   if (n == 0) {
     alloc_level(L, g, 0, batch_floor);
     L.identity_sched = true;
@@ -921,6 +931,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   auto it = m.subm.find(key);
   if (it != m.subm.end()) return it->second;
   Filt f = make_filt(m.dim, filter, nullptr, nullptr);
+  m.builds++;
   Table t;
   t.K = f.K;
   auto lit = m.levels.find(mk(m.dim, spatial));
@@ -1048,6 +1059,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   if (it != m.strided.end()) return it->second;
   Filt f = make_filt(m.dim, filter, stride, out_size);
   Geom go = make_geom(m.dim, out_size);
+  m.builds++;
   StridedRules R;
   R.in_size = mk(m.dim, in_size);
   R.out_size = mk(m.dim, out_size);
@@ -1061,6 +1073,8 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   int batch = lit == m.levels.end() ? 0 : lit->second.batch;
   // Building a strided rulebook replaces the output level (Metadata/ConvolutionRules.h:68-70)
   // and whatever was cached for it.
+  // Feature passes enqueued earlier may still be reading what is dropped here.
+  if (m.levels.count(R.out_size)) wait_for_consumers(m, s);
   for (auto i = m.subm.begin(); i != m.subm.end();)
     i = std::equal(R.out_size.begin(), R.out_size.end(), i->first.begin()) ? m.subm.erase(i) : std::next(i);
   Level &LO = m.levels[R.out_size];
@@ -1142,6 +1156,7 @@ __global__ void k_identity_table(int64_t n, int64_t npad, int *nbr, unsigned *gm
 Table &identity_table(Metadata &m, int64_t rows, hipStream_t s) {
   auto it = m.ident.find(rows);
   if (it != m.ident.end()) return it->second;
+  m.builds++;
   Table t;
   t.K = 1;
   t.n = rows;
