@@ -291,8 +291,13 @@ int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *c
     Metadata &m = md(h);
     if (n < 0) throw Error("negative point count");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
-    BuildScope b(m, stream, true);
-    build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, b.s());
+    {
+      BuildScope b(m, stream, true);
+      build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, b.s());
+    }
+    // the construction's last kernels may still be reading `coords`: whatever the caller does
+    // with that buffer next on its stream (free it, reuse it) is ordered behind them
+    consume(m, st(stream));
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -313,8 +318,11 @@ int scn_md_bl_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t
     if (batch < 0 || length < 0) throw Error("negative batch size or length");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
     if (batch * length == 0) length = 1, batch = 0;
-    BuildScope b(m, stream, true);
-    build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, b.s(), length);
+    {
+      BuildScope b(m, stream, true);
+      build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, b.s(), length);
+    }
+    consume(m, st(stream));  // as in scn_md_input_layer
     if (n_active) *n_active = m.input.n_out;
   });
 }
