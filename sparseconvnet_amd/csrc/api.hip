@@ -220,6 +220,18 @@ static StridedRules &strided_table(Metadata &m, const int64_t *in_size, const in
   consume(m, st(stream));
   return *r;
 }
+// The same rulebook read from the fine side (transposed convolution, unpooling).
+static StridedRules &strided_table_fine(Metadata &m, const int64_t *in_size, const int64_t *out_size,
+                                        const int64_t *filter, const int64_t *stride, void *stream) {
+  StridedRules *r;
+  {
+    BuildScope b(m, stream);
+    r = &strided_rules(m, in_size, out_size, filter, stride, b.s());
+    finish_by_in(m, *r, b.s());
+  }
+  consume(m, st(stream));
+  return *r;
+}
 // Exports and other rarely used calls run wholly on the build stream, ordered against the
 // caller's stream on both sides (they read and write the caller's buffers and use the
 // constructions' scratch).
@@ -478,7 +490,7 @@ static void deconv(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
                    double *macs) {
   Metadata &m = md(h);
   // CPU/Deconvolution.cpp:15-16: the rulebook of (out_size -> in_size), columns swapped.
-  StridedRules &r = strided_table(m, out_size, in_size, filter, stride, stream);
+  StridedRules &r = strided_table_fine(m, out_size, in_size, filter, stride, stream);
   conv_forward(m, r.by_in, in, level_rows(m, in_size), out, weight, bias, n_in, n_out, groups, pre, post,
                st(stream));
   note_macs(m, r.by_in, (double)(n_in / groups) * (n_out / groups) * groups, macs, st(stream));
@@ -574,7 +586,7 @@ int scn_unpool_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_s
     Metadata &m = md(h);
     if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
     // CPU/UnPooling.cpp:43-44: the rulebook of (out_size -> in_size), read from the fine side
-    StridedRules &r = strided_table(m, out_size, in_size, size, stride, stream);
+    StridedRules &r = strided_table_fine(m, out_size, in_size, size, stride, stream);
     unpool_forward(r.by_in, in, in_stride, out, planes, n_features_to_drop, st(stream));
   });
 }

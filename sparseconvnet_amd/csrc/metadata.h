@@ -83,6 +83,10 @@ struct Table {
 struct StridedRules {
   Table by_out;  // indexed by rows of the coarse (output) level: value = fine row
   Table by_in;   // indexed by schedule positions of the fine level: value = coarse row
+  // by_in is emitted with by_out but pattern-sorted only when somebody asks for it
+  // (finish_by_in): transposed convolutions and unpooling come long after the level was built,
+  // and the sort would sit on the path of the next level's construction.
+  bool by_in_final = false;
   SizeKey in_size, out_size;
 };
 
@@ -169,6 +173,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
                             const int64_t *filter, const int64_t *stride, hipStream_t s);
 // The one-tap table over `rows` rows whose only rule list is the identity.
 Table &identity_table(Metadata &m, int64_t rows, hipStream_t s);
+void finish_by_in(Metadata &m, StridedRules &r, hipStream_t s);
 // Pairs of tap k of a table: (value, row at position t), ordered by t.  Returns the count.
 int64_t export_table_pairs(Metadata &m, Table &t, int k, bool swap, int *pairs, hipStream_t s);
 std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t s);

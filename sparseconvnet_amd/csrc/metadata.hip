@@ -1087,6 +1087,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     R.by_in.n = 0;
     R.by_in.npad = 64;
     R.by_out.identity_rows = R.by_in.identity_rows = true;
+    R.by_in_final = true;
     return m.strided.emplace(key, std::move(R)).first->second;
   }
   Level &LI = m.levels[R.in_size];
@@ -1139,8 +1140,16 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   fold_counts(R.by_out, s);
   R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
   finalize_table(m, R.by_out, nullptr, s);
-  finalize_table(m, R.by_in, LI.sched_ptr(), s);
   return m.strided.emplace(key, std::move(R)).first->second;
+}
+
+void finish_by_in(Metadata &m, StridedRules &r, hipStream_t s) {
+  if (r.by_in_final) return;
+  auto li = m.levels.find(r.in_size);
+  if (li == m.levels.end()) throw Error("strided rules: the fine level is gone");
+  m.builds++;
+  finalize_table(m, r.by_in, li->second.sched_ptr(), s);
+  r.by_in_final = true;
 }
 
 // ---- identity table -----------------------------------------------------------------------
