@@ -75,6 +75,26 @@ int scn_md_set_bf16(scn_metadata *md, int enable);
 int scn_md_input_layer(scn_metadata *md, const int64_t *spatial, const int64_t *coords,
                        int64_t n, int ncols, int min_batch, int mode, void *stream,
                        int64_t *n_active);
+/* The point-at-a-time input of sparseconvnet/inputBatch.py, as one pass over everything the
+ * caller collected: Metadata::setInputSpatialSize / batchAddSample / setInputSpatialLocation(s)
+ * (Metadata/Metadata.cpp:74-147) with addPointToSparseGridMapAndFeatures (:29-46).  coords as
+ * for scn_md_input_layer, in the order the points were set; a site's row is the rank of its
+ * first point, and the site lists that point unless later points of the site have
+ * overwrite[i] != 0: then it lists the last of those (overwrite: device bytes [n], or NULL for
+ * "no point overwrites"; copied, so the caller may free it).  min_batch is the number of
+ * samples added so far (samples without points count).  scn_input_layer_fwd then gathers the
+ * listed points' vectors into the [n_active, planes] feature matrix the reference grows row by
+ * row.  scn_md_input_rules_header reports mode 5 (1 without flags), maxActive 1. */
+int scn_md_input_batch(scn_metadata *md, const int64_t *spatial, const int64_t *coords,
+                       const unsigned char *overwrite, int64_t n, int ncols, int min_batch,
+                       void *stream, int64_t *n_active);
+/* Metadata::generateRuleBooks2s2 / generateRuleBooks3s2 (Metadata/Metadata.cpp:351-411;
+ * InputBatch.precompute_metadata, sparseconvnet/inputBatch.py:72-82): starting at the input
+ * level, every level's 3^d submanifold rulebook and the size-`size` (2 or 3), stride-2 rulebook
+ * to the next level, until an extent no longer halves (size 2: even and >= 2; size 3: odd and
+ * >= 3).  Everything is enqueued on the library's build stream (see scn_set_build_stream); later
+ * calls that use one of the rulebooks wait for it there. */
+int scn_md_generate_rulebooks(scn_metadata *md, int size, void *stream);
 /* Rule header [mode, maxActive, nInputRows, nOutputRows] (Metadata/IOLayersRules.h:10-15). */
 int scn_md_input_rules_header(scn_metadata *md, int32_t hdr[4]);
 /* Rule rows, device int32 [nOutputRows, 1+maxActive] = [count, input indices.., 0 pad]. */

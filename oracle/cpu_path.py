@@ -47,6 +47,13 @@ def _load(flavour):
         "bl_rules": (None, [C.c_void_p, _i32p]),
         "bl_input_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
         "bl_output_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "set_input_spatial_size": (None, [C.c_void_p, _i64p]),
+        "batch_add_sample": (None, [C.c_void_p]),
+        "set_input_locations": (C.c_int, [C.c_void_p, _i64p, C.c_int, C.c_int, _f32p, C.c_int, C.c_int]),
+        "add_sample_from_tensor": (None, [C.c_void_p, _f32p, _i64p, C.c_int, _i64p, C.c_float]),
+        "batch_planes": (C.c_int, [C.c_void_p]),
+        "batch_features": (None, [C.c_void_p, _f32p]),
+        "generate_rulebooks": (None, [C.c_void_p, C.c_int]),
         "nactive": (C.c_int, [C.c_void_p, _i64p]),
         "batch_size": (C.c_int, [C.c_void_p, _i64p]),
         "spatial_locations": (None, [C.c_void_p, _i64p, _i64p]),
@@ -161,6 +168,42 @@ class CpuPath:
         out = np.zeros((int(hdr[2]), int(hdr[3]), x.shape[1]), np.float32)
         self.f["bl_output_fwd"](self.h, _pf(x), _pf(out), x.shape[1])
         return out
+
+    # point-at-a-time input (sparseconvnet/inputBatch.py)
+    def batch_begin(self, spatial):
+        self.input_spatial = _sz(self.dim, spatial)
+        self.f["set_input_spatial_size"](self.h, _p64(self.input_spatial))
+
+    def batch_add_sample(self):
+        self.f["batch_add_sample"](self.h)
+
+    def batch_set_locations(self, locations, vectors, overwrite=False):
+        locations = np.ascontiguousarray(locations, dtype=np.int64)
+        vectors = _f32(vectors)
+        assert locations.ndim == 2 and vectors.ndim == 2 and len(locations) == len(vectors)
+        r = self.f["set_input_locations"](self.h, _p64(locations), locations.shape[0], locations.shape[1],
+                                          _pf(vectors), vectors.shape[1], 1 if overwrite else 0)
+        if r:
+            raise RuntimeError("no current sample")
+
+    def batch_add_sample_from_tensor(self, tensor, offset, threshold=0.0):
+        tensor = _f32(tensor)
+        assert tensor.ndim == self.dim + 1
+        size = np.ascontiguousarray(tensor.shape[:-1], dtype=np.int64)
+        self.f["add_sample_from_tensor"](self.h, _pf(tensor), _p64(size), tensor.shape[-1],
+                                         _p64(_sz(self.dim, offset)), float(threshold))
+
+    def batch_end(self):  # the CPU implementations insert as they go: nothing left to do
+        pass
+
+    def batch_features(self):
+        out = np.zeros((self.nactive(self.input_spatial), self.f["batch_planes"](self.h)), np.float32)
+        if out.size:
+            self.f["batch_features"](self.h, _pf(out))
+        return out
+
+    def generate_rulebooks(self, size):
+        self.f["generate_rulebooks"](self.h, int(size))
 
     def nactive(self, spatial):
         return self.f["nactive"](self.h, _p64(_sz(self.dim, spatial)))

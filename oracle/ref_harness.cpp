@@ -37,6 +37,7 @@ namespace {
 struct Handle {
   int dim;
   void *m;
+  at::Tensor feats = torch::empty({0}, at::kFloat);  // what sparseconvnet/inputBatch.py:18 keeps beside its Metadata
 };
 
 at::Tensor lt(const int64_t *p, int n) {
@@ -280,6 +281,38 @@ void ref_s2d(void *h, const int64_t *spatial, const float *in, float *out, int n
   DISPATCH(h, auto S = lt(spatial, D); Int n = m.getNActive(S); auto I = ft(in, {n, nPlanes});
            auto O = torch::empty({0}, at::kFloat);
            cpu_SparseToDense_updateOutput<float, D>(S, m, I, O, nPlanes); copy_out(O, out));
+}
+
+// sparseconvnet/inputBatch.py's calls into Metadata, with the feature tensor it passes along
+// kept in the handle.
+void ref_set_input_spatial_size(void *h, const int64_t *spatial) {
+  DISPATCH(h, auto S = lt(spatial, D); m.setInputSpatialSize(S));
+}
+void ref_batch_add_sample(void *h) { DISPATCH(h, (void)D; m.batchAddSample()); }
+int ref_set_input_locations(void *h, const int64_t *locations, int n, int ncols, const float *vecs,
+                            int nPlanes, int overwrite) {
+  int r = 0;
+  DISPATCH(h, if (ncols == D && !m.inputSG) { r = -1; break; }
+           auto L = torch::from_blob((void *)locations, {n, ncols}, at::kLong).clone();
+           auto V = ft(vecs, {n, nPlanes}).clone();
+           m.setInputSpatialLocations(((Handle *)h)->feats, L, V, overwrite != 0));
+  return r;
+}
+void ref_add_sample_from_tensor(void *h, const float *tensor, const int64_t *size, int nPlanes,
+                                const int64_t *offset, float threshold) {
+  DISPATCH(h, std::vector<int64_t> shape(size, size + D); shape.push_back(nPlanes);
+           auto T = ft(tensor, shape).clone(); auto O = lt(offset, D);
+           auto S = torch::empty({D}, at::kLong);
+           for (int i = 0; i < D; i++) S.data_ptr<long>()[i] = m.inputSpatialSize[i];
+           m.addSampleFromThresholdedTensor(((Handle *)h)->feats, T, O, S, threshold));
+}
+int ref_batch_planes(void *h) {
+  auto &f = ((Handle *)h)->feats;
+  return f.dim() == 2 ? (int)f.size(1) : 0;
+}
+void ref_batch_features(void *h, float *out) { copy_out(((Handle *)h)->feats, out); }
+void ref_generate_rulebooks(void *h, int size) {
+  DISPATCH(h, (void)D; if (size == 2) m.generateRuleBooks2s2(); else m.generateRuleBooks3s2());
 }
 
 }  // extern "C"

@@ -121,6 +121,11 @@ struct Metadata {
   std::map<Key, RuleBook> ruleBooks;
   std::map<Key, RuleBook> sparseToDenseRuleBooks;
   Key inputSpatialSize;
+  // point-at-a-time input (Metadata/Metadata.h:62-64 inputSGs / inputSG / inputNActive, and
+  // the feature tensor that sparseconvnet/inputBatch.py:18 hands to every call)
+  Int currentSample = -1;
+  int batchPlanes = 0;
+  std::vector<float> batchFeatures;
 };
 
 static Key mkkey(int dim, const int64_t *a, const int64_t *b = nullptr,
@@ -836,6 +841,125 @@ void orc_s2d(void *md, const int64_t *spatial, const float *in, float *out, int 
       for (Int p = 0; p < nPlanes; p++) o[(size_t)p * vol] = i[p];
     }
     oF += (size_t)nPlanes * vol;
+  }
+}
+
+// ---- point-at-a-time input (sparseconvnet/inputBatch.py over Metadata/Metadata.cpp:74-147,296-411)
+
+// Metadata/Metadata.cpp:74-82
+void orc_set_input_spatial_size(void *md, const int64_t *spatial) {
+  Metadata &m = *(Metadata *)md;
+  m.inputSpatialSize = mkkey(m.dim, spatial);
+  m.grids[m.inputSpatialSize];
+  m.nActive[m.inputSpatialSize];
+}
+// Metadata/Metadata.cpp:83-87
+void orc_batch_add_sample(void *md) {
+  Metadata &m = *(Metadata *)md;
+  Grids &SGs = m.grids[m.inputSpatialSize];
+  resize_grids(SGs, SGs.size() + 1, m.dim);
+  m.currentSample = (Int)SGs.size() - 1;
+}
+// Metadata/Metadata.cpp:29-46: a new site takes the next row and the vector; a known site
+// keeps its vector unless overwrite is set.
+static void add_point(Metadata &m, Grid &mp, const Pt &p, const float *vec, int nPlanes, bool overwrite) {
+  Int &nActive = m.nActive[m.inputSpatialSize];
+  auto r = mp.insert(p, nActive);
+  if (r.second) {
+    nActive++;
+    m.batchPlanes = nPlanes;
+    m.batchFeatures.resize((size_t)nActive * nPlanes);
+    std::memcpy(m.batchFeatures.data() + (size_t)(nActive - 1) * nPlanes, vec, sizeof(float) * nPlanes);
+  } else if (overwrite) {
+    std::memcpy(m.batchFeatures.data() + (size_t)*r.first * nPlanes, vec, sizeof(float) * nPlanes);
+  }
+}
+// Metadata/Metadata.cpp:100-147: ncols == dim adds to the current sample, ncols == dim + 1
+// reads the sample from the last column and grows the batch as needed.  Returns 0, or -1
+// where the reference asserts (no current sample).
+int orc_set_input_locations(void *md, const int64_t *locations, int n, int ncols, const float *vecs,
+                            int nPlanes, int overwrite) {
+  Metadata &m = *(Metadata *)md;
+  Grids &SGs = m.grids[m.inputSpatialSize];
+  if (ncols == m.dim && m.currentSample < 0) return -1;
+  for (int i = 0; i < n; i++) {
+    Pt p = Pt();
+    for (int d = 0; d < m.dim; d++) p.x[d] = (Int)locations[(size_t)i * ncols + d];
+    Int b = m.currentSample;
+    if (ncols == m.dim + 1) {
+      b = (Int)locations[(size_t)i * ncols + m.dim];
+      if (b >= (Int)SGs.size()) resize_grids(SGs, b + 1, m.dim);
+    }
+    add_point(m, SGs[b], p, vecs + (size_t)i * nPlanes, nPlanes, overwrite != 0);
+  }
+  return 0;
+}
+// Metadata/Metadata.cpp:296-349: a new sample from a dense [size..., nPlanes] block placed at
+// offset; a cell is active when some plane exceeds the threshold in magnitude and the cell
+// lies inside the spatial size.  Cells are visited with the last dimension fastest
+// (Metadata/RectangularRegions.h:84-91).
+void orc_add_sample_from_tensor(void *md, const float *tensor, const int64_t *size, int nPlanes,
+                                const int64_t *offset, float threshold) {
+  Metadata &m = *(Metadata *)md;
+  Grids &SGs = m.grids[m.inputSpatialSize];
+  resize_grids(SGs, SGs.size() + 1, m.dim);
+  Grid &sg = SGs.back();
+  Int &nActive = m.nActive[m.inputSpatialSize];
+  int64_t vol = 1;
+  for (int d = 0; d < m.dim; d++) vol *= size[d];
+  m.batchPlanes = nPlanes;
+  Pt point = Pt();
+  for (int d = 0; d < m.dim; d++) point.x[d] = (Int)offset[d];
+  for (int64_t c = 0; c < vol; c++) {
+    bool active = false;
+    for (int i = 0; i < nPlanes; i++)
+      if (std::fabs(tensor[i]) > threshold) {
+        active = true;
+        break;
+      }
+    for (int d = 0; d < m.dim; d++)
+      if (point.x[d] < 0 || point.x[d] >= m.inputSpatialSize[d]) {
+        active = false;
+        break;
+      }
+    if (active) {
+      *sg.insert(point, nActive).first = nActive;
+      nActive++;
+      m.batchFeatures.insert(m.batchFeatures.end(), tensor, tensor + nPlanes);
+    }
+    tensor += nPlanes;
+    for (int d = m.dim - 1; d >= 0; d--) {
+      point.x[d]++;
+      if (point.x[d] < offset[d] + size[d]) break;
+      point.x[d] = (Int)offset[d];
+    }
+  }
+}
+int orc_batch_planes(void *md) { return ((Metadata *)md)->batchPlanes; }
+void orc_batch_features(void *md, float *out) {
+  Metadata &m = *(Metadata *)md;
+  if (!m.batchFeatures.empty()) std::memcpy(out, m.batchFeatures.data(), m.batchFeatures.size() * sizeof(float));
+}
+// Metadata/Metadata.cpp:351-411: every level's 3^d submanifold rulebook and the size-`size`
+// stride-2 rulebook to the next level, until a level's extent no longer halves (size 2:
+// even and >= 2; size 3: odd and >= 3).
+void orc_generate_rulebooks(void *md, int size) {
+  Metadata &m = *(Metadata *)md;
+  int64_t inS[MAXD], outS[MAXD], s3[MAXD], sz[MAXD], str[MAXD];
+  for (int d = 0; d < m.dim; d++) {
+    inS[d] = m.inputSpatialSize[d];
+    s3[d] = 3;
+    sz[d] = size;
+    str[d] = 2;
+  }
+  while (true) {
+    getSubmanifoldRuleBook(m, inS, s3);
+    for (int d = 0; d < m.dim; d++) {
+      if (size == 2 ? (inS[d] < 2 || inS[d] % 2 != 0) : (inS[d] < 3 || inS[d] % 2 != 1)) return;
+      outS[d] = size == 2 ? inS[d] / 2 : (inS[d] - 1) / 2;
+    }
+    getRuleBook(m, inS, outS, sz, str);
+    for (int d = 0; d < m.dim; d++) inS[d] = outS[d];
   }
 }
 

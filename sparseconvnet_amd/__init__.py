@@ -22,6 +22,7 @@ from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, Bat
                      BLInputLayer, BLOutputLayer, Convolution, Deconvolution, Identity, InputLayer, MaxPooling,
                      NetworkInNetwork, OutputLayer, SparseToDense, SubmanifoldConvolution, UnPooling,
                      ValidConvolution)
+from .inputBatch import InputBatch  # noqa: E402
 from .metadata import Metadata  # noqa: E402
 from .networks import SparseVggNet, UNet  # noqa: E402
 from .tensor import SparseConvNetTensor  # noqa: E402

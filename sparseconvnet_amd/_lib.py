@@ -33,6 +33,8 @@ SIGNATURES = {
     "scn_md_input_rules": (C.c_int, [_vp, _vp, _vp]),
     "scn_md_bl_input_layer": (C.c_int, [_vp, _i64p, _vp, C.c_int64, C.c_int64, C.c_int, _vp, _i64p]),
     "scn_md_bl_rules_header": (C.c_int, [_vp, C.POINTER(C.c_int32)]),
+    "scn_md_input_batch": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int64, C.c_int, C.c_int, _vp, _i64p]),
+    "scn_md_generate_rulebooks": (C.c_int, [_vp, C.c_int, _vp]),
     "scn_md_nactive": (C.c_int, [_vp, _i64p, _i64p]),
     "scn_md_batch_size": (C.c_int, [_vp, _i64p, C.POINTER(C.c_int)]),
     "scn_md_spatial_locations": (C.c_int, [_vp, _i64p, _vp, _vp]),

@@ -313,6 +313,28 @@ int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *c
     if (n_active) *n_active = m.input.n_out;
   });
 }
+int scn_md_input_batch(scn_metadata *h, const int64_t *spatial, const int64_t *coords,
+                       const unsigned char *overwrite, int64_t n, int ncols, int min_batch, void *stream,
+                       int64_t *n_active) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (n < 0) throw Error("negative point count");
+    if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
+    {
+      BuildScope b(m, stream, true);
+      build_input_layer(m, spatial, coords, n, ncols, min_batch, 5, b.s(), 0, overwrite);
+    }
+    consume(m, st(stream));  // as in scn_md_input_layer; `overwrite` was copied on the build stream too
+    if (n_active) *n_active = m.input.n_out;
+  });
+}
+int scn_md_generate_rulebooks(scn_metadata *h, int size, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    BuildScope b(m, stream);
+    generate_rulebooks(m, size, b.s());
+  });
+}
 int scn_md_input_rules_header(scn_metadata *h, int32_t hdr[4]) {
   return guarded([&] {
     Metadata &m = md(h);

@@ -102,7 +102,8 @@ struct CoefJobs {
 };
 
 struct InputRules {
-  int mode = -1;      // 1: the first point of a site is listed, 2: the last, 3 / 4: all (sum / mean)
+  int mode = -1;      // 1: the first point of a site is listed, 2: the last, 3 / 4: all (sum / mean),
+                      // 5: the first, unless later points of the site carry an overwrite flag: then the last of those
   int user_mode = -1; // the mode the caller gave (the batch-by-length layer numbers 1 and 2 the other way round)
   int max_active = 0;
   int64_t n_in = 0, n_out = 0;
@@ -111,7 +112,20 @@ struct InputRules {
   DevBuf<int> sorted_idx;    // [n_in] input indices grouped by site, input order inside a group
   DevBuf<int> run_start;     // [n_out] first position of the row's group in sorted_idx
   DevBuf<int> run_len;       // [n_out]
+  DevBuf<unsigned char> overwrite;  // [n_in], mode 5 only
 };
+
+// The one input point a site lists in modes 1, 2 and 5; [st, st + len) is the site's group in
+// sorted_idx, in input order.
+__device__ inline int listed_point(const int *sorted_idx, int st, int len, int mode, const unsigned char *overwrite) {
+  if (mode == 2) return sorted_idx[st + len - 1];
+  if (mode == 5)
+    for (int q = len - 1; q > 0; q--) {
+      const int i = sorted_idx[st + q];
+      if (overwrite[i]) return i;
+    }
+  return sorted_idx[st];
+}
 
 struct Metadata {
   int dim = 0;
@@ -164,8 +178,12 @@ Geom make_geom(int dim, const int64_t *spatial);
 
 // bl_length > 0: coords is [n / bl_length, bl_length, dim] (BLInputLayer), the sample is the
 // first index and positions whose first coordinate is negative are empty.
+// mode 5 (point-at-a-time input, Metadata/Metadata.cpp:29-46 as one pass): overwrite[i] != 0 marks
+// points that replace what their site holds; NULL: none does.
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
-                       int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length = 0);
+                       int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length = 0,
+                       const unsigned char *overwrite = nullptr);
+void generate_rulebooks(Metadata &m, int size, hipStream_t s);
 void export_input_rules(Metadata &m, int *rows, hipStream_t s);
 void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStream_t s);
 Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s);

@@ -284,11 +284,13 @@ __global__ void k_finish_groups(const int *sidx, const int *head, const int *hea
 }
 
 void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
-                       int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length) {
+                       int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length,
+                       const unsigned char *overwrite) {
   const bool bl = bl_length > 0;
   if (bl ? ncols != m.dim : (ncols != m.dim && ncols != m.dim + 1))
     throw Error(bl ? "coords must be [batch, length, dim]" : "coords must have dim or dim+1 columns");
-  if (mode < 0 || mode > 4) throw Error("input layer mode must be 0..4");
+  if (mode < 0 || mode > 5 || (mode == 5 && bl)) throw Error("input layer mode must be 0..4");
+  if (mode == 5 && !overwrite) mode = 1;  // nothing overwrites: every site keeps its first point
   if (n >= ((int64_t)1 << 31) - 64) throw Error("too many input points for int32 rule indices");
   Geom g = make_geom(m.dim, spatial);
   SizeKey key = mk(m.dim, spatial);
@@ -375,6 +377,10 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   R.run_len.reserve(std::max<int64_t>(N, 1));
   if (n_empty) fill32(R.row_of_input.p, 0xFFFFFFFFu, n, s);  // empty positions belong to no row
   HIP_CHECK(hipMemcpyAsync(R.sorted_idx.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
+  if (mode == 5) {  // the caller's flags are read again by every forward pass: keep a copy
+    R.overwrite.reserve(n);
+    HIP_CHECK(hipMemcpyAsync(R.overwrite.p, overwrite, n, hipMemcpyDeviceToDevice, s));
+  }
   if (N == 0) return;
   m.v0.reserve(std::max<int64_t>(n, 2 * N + 2));  // reused: row_of_group | head_pos
   int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
@@ -396,17 +402,15 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
 
 // Reference layout of the rule rows (Metadata/IOLayersRules.h:96-119).
 __global__ void k_export_input_rules(const int *sorted_idx, const int *run_start, const int *run_len,
-                                     int64_t n_out, int mode, int max_active, int *rows) {
+                                     const unsigned char *overwrite, int64_t n_out, int mode, int max_active,
+                                     int *rows) {
   int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= n_out) return;
   int *o = rows + r * (1 + max_active);
   int st = run_start[r], len = run_len[r];
-  if (mode == 1) {
+  if (mode == 1 || mode == 2 || mode == 5) {
     o[0] = 1;
-    o[1] = sorted_idx[st];
-  } else if (mode == 2) {
-    o[0] = 1;
-    o[1] = sorted_idx[st + len - 1];
+    o[1] = listed_point(sorted_idx, st, len, mode, overwrite);
   } else {
     o[0] = len;
     for (int q = 0; q < max_active; q++) o[1 + q] = q < len ? sorted_idx[st + q] : 0;
@@ -416,7 +420,7 @@ void export_input_rules(Metadata &m, int *rows, hipStream_t s) {
   InputRules &R = m.input;
   if (R.mode <= 0 || R.n_out == 0) return;
   k_export_input_rules<<<grid_for(R.n_out), TB, 0, s>>>(R.sorted_idx.p, R.run_start.p, R.run_len.p,
-                                                        R.n_out, R.mode, R.max_active, rows);
+                                                        R.overwrite.p, R.n_out, R.mode, R.max_active, rows);
   LAUNCH_CHECK();
 }
 
@@ -1294,6 +1298,30 @@ int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *p
   k_s2d_pairs<<<grid_for(L.n), TB, 0, s>>>(L.g, L.coords.p, L.n, L.npad, m.f1.p, m.s1.p, pairs);
   LAUNCH_CHECK();
   return 0;
+}
+
+// Metadata/Metadata.cpp:351-411 (generateRuleBooks2s2 / 3s2): from the input level down, every
+// level's 3^d submanifold table and the size-`size` stride-2 table to the next level, until an
+// extent no longer halves (size 2: even and >= 2; size 3: odd and >= 3).
+void generate_rulebooks(Metadata &m, int size, hipStream_t s) {
+  if (size != 2 && size != 3) throw Error("rulebooks are precomputed for filter size 2 or 3 (stride 2)");
+  if (m.input_size.empty()) throw Error("no input level to start from");
+  int64_t in_s[SCN_MAXD], out_s[SCN_MAXD], f3[SCN_MAXD], fs[SCN_MAXD], st[SCN_MAXD];
+  for (int d = 0; d < m.dim; d++) {
+    in_s[d] = m.input_size[d];
+    f3[d] = 3;
+    fs[d] = size;
+    st[d] = 2;
+  }
+  while (true) {
+    submanifold_rules(m, in_s, f3, s);
+    for (int d = 0; d < m.dim; d++) {
+      if (size == 2 ? (in_s[d] < 2 || in_s[d] % 2 != 0) : (in_s[d] < 3 || in_s[d] % 2 != 1)) return;
+      out_s[d] = size == 2 ? in_s[d] / 2 : (in_s[d] - 1) / 2;
+    }
+    strided_rules(m, in_s, out_s, fs, st, s);
+    for (int d = 0; d < m.dim; d++) in_s[d] = out_s[d];
+  }
 }
 
 }  // namespace scn

@@ -148,9 +148,11 @@ void unpool_forward(const Table &t, const float *in, int in_stride, float *out, 
 
 // ---- input / output layers --------------------------------------------------------------
 // CPU/IOLayers.cpp:11-29: out[row] = sum over the row's points, in input order, of
-// mult * in[point], mult = 1/count for mode 4.  Modes 1 / 2 copy the first / last point.
+// mult * in[point], mult = 1/count for mode 4.  Modes 1 / 2 / 5 copy the one point
+// the site lists.
 __global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const int *run_len,
-                            int64_t n_out, int mode, const float *in, float *out, int planes) {
+                            const unsigned char *overwrite, int64_t n_out, int mode, const float *in, float *out,
+                            int planes) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = n_out * planes;
   int64_t step = (int64_t)gridDim.x * blockDim.x;
@@ -159,10 +161,8 @@ __global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const i
     int p = (int)(i - r * planes);
     int st = run_start[r], len = run_len[r];
     float acc = 0.0f;
-    if (mode == 1) {
-      acc += in[(int64_t)sorted_idx[st] * planes + p];
-    } else if (mode == 2) {
-      acc += in[(int64_t)sorted_idx[st + len - 1] * planes + p];
+    if (mode == 1 || mode == 2 || mode == 5) {
+      acc += in[(int64_t)listed_point(sorted_idx, st, len, mode, overwrite) * planes + p];
     } else {
       float mult = (mode == 4 && len > 0) ? 1.0f / (float)len : 1.0f;
       for (int q = 0; q < len; q++) acc += mult * in[(int64_t)sorted_idx[st + q] * planes + p];
@@ -181,18 +181,18 @@ void input_forward(const InputRules &r, const float *in, float *out, int planes,
   if (r.n_out == 0) return;
   int64_t total = r.n_out * planes;
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
-  k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.n_out,
-                                                    r.mode, in, out, planes);
+  k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p,
+                                                    r.n_out, r.mode, in, out, planes);
   LAUNCH_CHECK();
 }
 
 // CPU/IOLayers.cpp:95-115 (InputLayer_BackwardPass :31-47 without averaging): every input
 // point listed in its site's rule receives the site's row; as a gather per input point.
-// Modes 1 / 2 list a single point per site, the others get zeros.
+// Modes 1 / 2 / 5 list a single point per site, the others get zeros.
 template <int V>
 __global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, const int *run_start,
-                             const int *run_len, int64_t n_in, int mode, const float *in, float *out,
-                             int planes) {
+                             const int *run_len, const unsigned char *overwrite, int64_t n_in, int mode,
+                             const float *in, float *out, int planes) {
   // thread -> (input point, group of V planes)
   const int groups = planes / V;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -203,8 +203,8 @@ __global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, con
     const int p = (int)(i - pt * groups) * V;
     const int row = row_of_input[pt];
     bool listed = row >= 0;  // empty positions of a batch-by-length input get zeros
-    if (listed && mode == 1) listed = sorted_idx[run_start[row]] == (int)pt;
-    if (listed && mode == 2) listed = sorted_idx[run_start[row] + run_len[row] - 1] == (int)pt;
+    if (listed && (mode == 1 || mode == 2 || mode == 5))
+      listed = listed_point(sorted_idx, run_start[row], run_len[row], mode, overwrite) == (int)pt;
     if (V == 4) {
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       if (listed) v = *reinterpret_cast<const float4 *>(in + (int64_t)row * planes + p);
@@ -230,10 +230,10 @@ void output_forward(const InputRules &r, const float *in, float *out, int planes
   const int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   if (vec)
     k_output_fwd<4><<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
-                                                          r.run_len.p, r.n_in, r.mode, in, out, planes);
+                                                          r.run_len.p, r.overwrite.p, r.n_in, r.mode, in, out, planes);
   else
     k_output_fwd<1><<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
-                                                          r.run_len.p, r.n_in, r.mode, in, out, planes);
+                                                          r.run_len.p, r.overwrite.p, r.n_in, r.mode, in, out, planes);
   LAUNCH_CHECK();
 }
 

@@ -124,6 +124,32 @@ class Metadata:
         _lib.check(self._L.scn_input_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out
 
+    def inputBatch(self, spatial_size, coords, vectors, overwrite, batch_size):
+        """Everything an InputBatch collected, in the order it was set: coords [n, dimension
+        (+1)], vectors [n, planes], overwrite None or a uint8 tensor [n] (points that replace
+        what their site holds) -> features [nActive, planes], rows by first occurrence."""
+        coords = coords.to(device=vectors.device, dtype=torch.int64).contiguous()
+        assert coords.dim() == 2 and coords.size(0) == vectors.size(0)
+        vectors = _features(vectors, "input vectors")
+        if overwrite is not None:
+            overwrite = overwrite.to(device=vectors.device, dtype=torch.uint8).contiguous()
+            assert overwrite.numel() == coords.size(0)
+        n = C.c_int64(0)
+        _lib.check(self._L.scn_md_input_batch(self._h, self._s(spatial_size), _ptr(coords), _ptr(overwrite),
+                                              coords.size(0), coords.size(1), int(batch_size), _stream(),
+                                              C.byref(n)))
+        out = torch.empty((n.value, vectors.size(1)), dtype=torch.float32, device=vectors.device)
+        _lib.check(self._L.scn_input_layer_fwd(self._h, _ptr(vectors), _ptr(out), vectors.size(1), _stream()))
+        return out
+
+    def generateRuleBooks2s2(self):
+        """3^d submanifold and 2^d / stride-2 rulebooks of every level, ahead of their use."""
+        _lib.check(self._L.scn_md_generate_rulebooks(self._h, 2, _stream()))
+
+    def generateRuleBooks3s2(self):
+        """3^d submanifold and 3^d / stride-2 rulebooks of every level, ahead of their use."""
+        _lib.check(self._L.scn_md_generate_rulebooks(self._h, 3, _stream()))
+
     def outputLayer(self, features):
         features = _features(features, "features")
         hdr = (C.c_int32 * 4)()

@@ -63,6 +63,41 @@ def bl_groups(coords):
     return groups, np.asarray(loc, np.int64).reshape(len(loc), d + 1)
 
 
+class PointTable:
+    """The point-at-a-time input as a dictionary: a new (coordinates, sample) takes the next
+    row and the vector; a known one keeps its vector unless the point overwrites."""
+
+    def __init__(self):
+        self.rows = {}
+        self.vectors = []
+
+    def set(self, key, vector, overwrite):
+        key = tuple(int(v) for v in key)
+        if key not in self.rows:
+            self.rows[key] = len(self.rows)
+            self.vectors.append(np.array(vector, np.float32))
+        elif overwrite:
+            self.vectors[self.rows[key]] = np.array(vector, np.float32)
+
+    def dense_block(self, tensor, offset, spatial, sample, threshold):
+        """Cells of a dense [size..., planes] block at `offset` with some |plane| > threshold,
+        inside the grid, in row-major order, as points of a new sample."""
+        spatial = np.broadcast_to(np.asarray(spatial), (tensor.ndim - 1,))
+        for cell in itertools.product(*[range(n) for n in tensor.shape[:-1]]):
+            where = [c + int(o) for c, o in zip(cell, offset)]
+            if not (np.abs(tensor[cell]) > threshold).any():
+                continue
+            if any(w < 0 or w >= int(s) for w, s in zip(where, spatial)):
+                continue
+            self.set(tuple(where) + (sample,), tensor[cell], False)
+
+    def locations(self):
+        return np.array(sorted(self.rows, key=self.rows.get), np.int64).reshape(len(self.rows), -1)
+
+    def features(self):
+        return np.array(self.vectors, np.float32)
+
+
 def submanifold_triples(loc, dim, size):
     """Set of (k, in_site, out_site) as coordinate tuples: in = out + tap - size//2, same sample."""
     size = np.broadcast_to(np.asarray(size), (dim,))

@@ -132,6 +132,96 @@ def check_bl_input_layer(make, dim, mode, seed, batch=3, length=70, spatial=9, p
     assert_close(out.reshape(-1, 4), back, "batch-by-length output, mode %d" % mode)
 
 
+def check_input_batch(make, dim, seed, spatial=9, planes=4):
+    """The point-at-a-time route (sparseconvnet/inputBatch.py) against a dictionary: calls with
+    and without a sample column, repeated sites inside and across calls with and without
+    overwrite, single points, samples that stay empty, a batch that grows through the sample
+    column, and a sample taken from a dense block that hangs over the edge of the grid."""
+    rng = np.random.default_rng(seed)
+    p = make(dim)
+    p.batch_begin(spatial)
+    table = bf.PointTable()
+
+    def put(locations, overwrite, sample=None):
+        vectors = rng.normal(size=(len(locations), planes)).astype(np.float32)
+        p.batch_set_locations(locations, vectors, overwrite)
+        for l, v in zip(locations, vectors):
+            table.set(tuple(l) if sample is None else tuple(l) + (sample,), v, overwrite)
+
+    def sites(n):  # repeats are likely: 9^dim cells at most
+        return rng.integers(0, spatial, size=(n, dim)).astype(np.int64)
+
+    p.batch_add_sample()                       # sample 0
+    a = sites(60)
+    put(a, False, 0)
+    put(np.concatenate([a[:20], sites(15)]), True, 0)
+    put(a[10:30], False, 0)                    # known sites, no overwrite: nothing changes
+    p.batch_add_sample()                       # sample 1 stays empty
+    p.batch_add_sample()                       # sample 2
+    put(sites(40), False, 2)
+    for _ in range(5):
+        put(sites(1), bool(rng.integers(0, 2)), 2)
+    # (the reference's pointer to the current sample does not survive a batch that grows through
+    # the sample column or a dense block: after those, only calls that name the sample, until
+    # the next add_sample)
+    with_sample = np.concatenate([sites(50), rng.choice([0, 2, 4], size=(50, 1))], 1).astype(np.int64)
+    put(with_sample, False)                    # the batch grows to 5 samples
+    again = np.concatenate([with_sample[:25], with_sample[:10], with_sample[40:]])
+    put(again, True)                           # repeats inside one overwriting call: the last one stays
+    p.batch_add_sample()                       # sample 5
+    put(sites(30), True, 5)
+    block = rng.normal(size=(4,) * dim + (planes,)).astype(np.float32)
+    block[np.abs(block).max(-1) < 0.9] *= 0.1  # some cells below the threshold
+    offset = np.array([spatial - 2] + [-1] * (dim - 1), np.int64)
+    p.batch_add_sample_from_tensor(block, offset, 0.5)   # sample 6
+    table.dense_block(block, offset, spatial, 6, 0.5)
+    put(np.concatenate([sites(10), np.full((10, 1), 6)], 1).astype(np.int64), True)
+    p.batch_end()
+
+    assert p.nactive(spatial) == len(table.rows)
+    assert p.batch_size(spatial) == 7
+    assert (p.spatial_locations(spatial) == table.locations()).all()   # rows: order of first appearance
+    feats = p.batch_features()
+    assert feats.shape == (len(table.rows), planes) and (feats == table.features()).all()
+    # the level is an ordinary one: its rulebooks come out as for any other input route
+    loc = p.spatial_locations(spatial)
+    rules = p.submanifold_rules(spatial, 3)
+    assert bf.triples_of(canon_rules(rules, loc, loc)) == bf.submanifold_triples(loc, dim, 3)
+
+
+def check_generate_rulebooks(make, dim, size, spatial, seed, n=400, batch=2):
+    """Rulebooks built ahead of their use (InputBatch.precompute_metadata): every level down to
+    the first whose extent does not halve exists afterwards, none beyond it, and the
+    rulebooks are the ones an explicit request gives."""
+    rng = np.random.default_rng(seed)
+    spatial = np.broadcast_to(np.asarray(spatial, np.int64), (dim,))
+    coords = np.concatenate([np.stack([rng.integers(0, s, n) for s in spatial], 1),
+                             rng.integers(0, batch, size=(n, 1))], 1).astype(np.int64)
+    p, q = make(dim), make(dim)
+    p.input_layer(spatial, coords, 0, 3)
+    q.input_layer(spatial, coords, 0, 3)
+    p.generate_rulebooks(size)
+    levels = [spatial]
+    while all(s >= size and s % 2 == (size == 3) for s in levels[-1]):
+        levels.append(levels[-1] // 2 if size == 2 else (levels[-1] - 1) // 2)
+    assert len(levels) >= 3
+    for fine, coarse in zip(levels, levels[1:]):
+        assert p.nactive(coarse) > 0                       # built by generate_rulebooks alone
+        r_q = q.strided_rules(fine, coarse, size, 2)
+        assert p.nactive(coarse) == q.nactive(coarse)
+        lf, lc = p.spatial_locations(fine), p.spatial_locations(coarse)
+        r_p = p.strided_rules(fine, coarse, size, 2)
+        assert bf.triples_of(canon_rules(r_p, lf, lc)) == bf.strided_triples(lf, dim, size, 2, coarse)
+        assert bf.triples_of(canon_rules(r_p, lf, lc)) == bf.triples_of(
+            canon_rules(r_q, q.spatial_locations(fine), q.spatial_locations(coarse)))
+    for lvl in levels:
+        loc = p.spatial_locations(lvl)
+        assert bf.triples_of(canon_rules(p.submanifold_rules(lvl, 3), loc, loc)) == bf.submanifold_triples(loc, dim, 3)
+    beyond = levels[-1] // 2 if size == 2 else np.maximum((levels[-1] - 1) // 2, 0)
+    if not any((beyond == l).all() for l in levels):
+        assert p.nactive(beyond) == 0
+
+
 def _setup(make, dim, spatial, n, batch, seed, C):
     rng = np.random.default_rng(seed)
     coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=n // 4)

@@ -89,6 +89,62 @@ class HipPath:
         _lib.check(self.L.scn_output_layer_fwd(self.h, _ptr(xd), _ptr(out), x.shape[1], _stream()))
         return out.cpu().numpy()
 
+    # point-at-a-time input: the calls collect, batch_end hands everything to the library
+    def batch_begin(self, spatial):
+        self.input_spatial = np.broadcast_to(np.asarray(spatial, np.int64), (self.dim,)).copy()
+        self._b_coords, self._b_vectors, self._b_flags = [], [], []
+        self._b_samples, self._b_current, self._b_feats = 0, -1, None
+
+    def batch_add_sample(self):
+        self._b_samples += 1
+        self._b_current = self._b_samples - 1
+
+    def batch_set_locations(self, locations, vectors, overwrite=False):
+        locations = np.ascontiguousarray(locations, dtype=np.int64)
+        vectors = np.ascontiguousarray(vectors, dtype=np.float32)
+        if locations.shape[1] == self.dim:
+            if self._b_current < 0:
+                raise RuntimeError("no current sample")
+            locations = np.concatenate([locations, np.full((len(locations), 1), self._b_current, np.int64)], 1)
+        elif len(locations):
+            self._b_samples = max(self._b_samples, int(locations[:, -1].max()) + 1)
+        self._b_coords.append(locations)
+        self._b_vectors.append(vectors)
+        self._b_flags.append(np.full(len(locations), 1 if overwrite else 0, np.uint8))
+
+    def batch_add_sample_from_tensor(self, tensor, offset, threshold=0.0):
+        tensor = np.ascontiguousarray(tensor, dtype=np.float32)
+        offset = np.broadcast_to(np.asarray(offset, np.int64), (self.dim,))
+        self._b_samples += 1
+        cells = np.argwhere((np.abs(tensor) > threshold).any(-1))
+        where = cells + offset
+        inside = ((where >= 0) & (where < self.input_spatial)).all(1)
+        cells, where = cells[inside], where[inside]
+        self._b_coords.append(np.concatenate([where, np.full((len(where), 1), self._b_samples - 1, np.int64)], 1))
+        self._b_vectors.append(tensor[tuple(cells.T)].reshape(len(cells), tensor.shape[-1]))
+        self._b_flags.append(np.zeros(len(where), np.uint8))
+
+    def batch_end(self):
+        coords = np.concatenate(self._b_coords) if self._b_coords else np.zeros((0, self.dim + 1), np.int64)
+        planes = self._b_vectors[0].shape[1] if self._b_vectors else 0
+        vectors = np.concatenate(self._b_vectors) if self._b_vectors else np.zeros((0, planes), np.float32)
+        flags = np.concatenate(self._b_flags) if self._b_flags else np.zeros(0, np.uint8)
+        c, v = _dev(coords, torch.int64), _dev(vectors, torch.float32)
+        f = _dev(flags, torch.uint8) if flags.any() else None
+        n = C.c_int64(0)
+        _lib.check(self.L.scn_md_input_batch(self.h, self._s(self.input_spatial), _ptr(c), _ptr(f), len(coords),
+                                             self.dim + 1, self._b_samples, _stream(), C.byref(n)))
+        out = torch.full((n.value, planes), float("nan"), dtype=torch.float32, device="cuda")
+        if planes:
+            _lib.check(self.L.scn_input_layer_fwd(self.h, _ptr(v), _ptr(out), planes, _stream()))
+        self._b_feats = out.cpu().numpy()
+
+    def batch_features(self):
+        return self._b_feats
+
+    def generate_rulebooks(self, size):
+        _lib.check(self.L.scn_md_generate_rulebooks(self.h, int(size), _stream()))
+
     def nactive(self, spatial):
         n = C.c_int64(0)
         _lib.check(self.L.scn_md_nactive(self.h, self._s(spatial), C.byref(n)))

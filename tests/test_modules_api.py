@@ -22,7 +22,7 @@ def test_exports():
                  "BatchNormalization", "BatchNormReLU", "BatchNormLeakyReLU", "MaxPooling", "InputLayer",
                  "OutputLayer", "SparseToDense", "Metadata", "SparseConvNetTensor", "Sequential", "ConcatTable",
                  "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor",
-                 "NetworkInNetwork", "AveragePooling", "UnPooling", "BLInputLayer", "BLOutputLayer"]:
+                 "NetworkInNetwork", "AveragePooling", "UnPooling", "BLInputLayer", "BLOutputLayer", "InputBatch"]:
         assert hasattr(scn, name), name
     assert scn.forward_pass_multiplyAdd_count == 0 and scn.forward_pass_hidden_states == 0
 
@@ -161,6 +161,36 @@ def test_checkpoint_round_trip(tmp_path):
     for (ka, va), (kb, vb) in zip(a.state_dict().items(), b.state_dict().items()):
         assert ka == kb and torch.equal(va, vb)
     assert scn.is_power2(8) and not scn.is_power2(6) and not scn.is_power2(0)
+
+
+def test_input_batch_collects_on_the_host():
+    # sparseconvnet/inputBatch.py:22-70: the calls and their old names; nothing touches the GPU
+    # until the features or the metadata are looked at
+    b = scn.InputBatch(2, [8, 6])
+    with pytest.raises(RuntimeError):
+        b.set_locations(torch.LongTensor([[1, 2]]), torch.FloatTensor([[1.0]]))
+    b.add_sample()
+    b.set_location(torch.LongTensor([1, 2]), torch.FloatTensor([1.0]))
+    with pytest.raises(AssertionError):
+        b.set_location(torch.LongTensor([1, 6]), torch.FloatTensor([1.0]))
+    with pytest.raises(AssertionError):
+        b.set_locations(torch.LongTensor([[8, 0, 0]]), torch.FloatTensor([[1.0]]))
+    b.set_locations(torch.LongTensor([[0, 0, 3], [7, 5, 1]]), torch.FloatTensor([[2.0], [3.0]]), True)
+    b.addSample()
+    b.setLocations(torch.LongTensor([[4, 4]]), torch.FloatTensor([[4.0]]))
+    t = torch.zeros(3, 3, 1)
+    t[0, 0, 0], t[2, 2, 0], t[1, 1, 0] = 5.0, -6.0, 0.5
+    b.add_sample_from_tensor(t, torch.LongTensor([5, 3]), threshold=1)
+    assert b._samples == 6
+    assert torch.cat(b._coords).tolist() == [[1, 2, 0], [0, 0, 3], [7, 5, 1], [4, 4, 4], [5, 3, 5], [7, 5, 5]]
+    assert torch.cat(b._vectors).flatten().tolist() == [1.0, 2.0, 3.0, 4.0, 5.0, -6.0]
+    assert b._overwrite == [(1, False), (2, True), (1, False), (2, False)]
+    for name in ("addSample", "setLocation", "setLocation_", "setLocations", "setLocations_",
+                 "addSampleFromTensor", "precomputeMetadata", "precompute_metadata"):
+        assert callable(getattr(b, name))
+    if not torch.cuda.is_available():
+        with pytest.raises(Exception):
+            b.features
 
 
 def test_no_cpu_fallback():

@@ -355,3 +355,61 @@ def test_build_stream_and_single_stream_agree():
     for a, b in zip(two, one):
         assert torch.equal(a, b)
     assert all(torch.isfinite(a).all() for a in two)
+
+
+def test_input_batch_network_vs_oracle(oracle_built):
+    """sparseconvnet/inputBatch.py's route into a network: points set one at a time and in
+    blocks, an overwriting call, a sample cut from a dense tensor, rulebooks precomputed; the
+    same calls on the CPU oracle, then the same module tree on both."""
+    torch.manual_seed(5)
+    rng = np.random.default_rng(5)
+    model = hello_world_model().cuda().eval()
+    randomise_bn(model, 6)
+    size = model.input_spatial_size(torch.LongTensor([10, 10]))
+    sp = size.numpy()
+    p = cpu_path.CpuPath(2, "oracle")
+    p.batch_begin(sp)
+
+    def fill(batch):
+        r = np.random.default_rng(7)
+        batch.add_sample()
+        pts = r.integers(0, sp[0], size=(300, 2))
+        vec = r.normal(size=(300, 1)).astype(np.float32)
+        for l, v in zip(pts[:20], vec[:20]):
+            batch.set_location(torch.from_numpy(l), torch.from_numpy(v), False)
+        batch.set_locations(torch.from_numpy(pts[20:]), torch.from_numpy(vec[20:]), False)
+        batch.set_locations(torch.from_numpy(pts[:50]), torch.from_numpy(vec[100:150]), True)
+        dense = torch.from_numpy(r.normal(size=(30, 40, 1)).astype(np.float32))
+        batch.add_sample_from_tensor(dense, torch.LongTensor([int(sp[0]) - 20, 3]), 1.0)
+        return pts, vec, dense.numpy()
+
+    batch = scn.InputBatch(2, size)
+    pts, vec, dense = fill(batch)
+    p.batch_add_sample()
+    p.batch_set_locations(pts, vec, False)
+    p.batch_set_locations(pts[:50], vec[100:150], True)
+    p.batch_add_sample_from_tensor(dense, [int(sp[0]) - 20, 3], 1.0)
+    batch.precompute_metadata(3)
+    p.generate_rulebooks(3)
+    assert batch.batch_size() == 2 and batch.features.is_cuda
+    assert (batch.get_spatial_locations().numpy() == p.spatial_locations(sp)).all()
+    assert (batch.features.cpu().numpy() == p.batch_features()).all()
+    with torch.no_grad():
+        got = model(batch)
+    want = oracle_model.run(model, p, oracle_model.CpuTensor(p.batch_features(), sp))
+    checks.assert_close(got.cpu().numpy(), want, "network over an InputBatch")
+    # without the precomputation the rulebooks are built on demand: same result
+    again = scn.InputBatch(2, size)
+    fill(again)
+    with torch.no_grad():
+        assert torch.equal(model(again), got)
+    # points set after a look at the batch: the next look sees them
+    extra = rng.integers(0, sp[0], size=(40, 2))
+    extra_v = rng.normal(size=(40, 1)).astype(np.float32)
+    batch.add_sample()
+    batch.set_locations(torch.from_numpy(extra), torch.from_numpy(extra_v), False)
+    p.batch_add_sample()
+    p.batch_set_locations(extra, extra_v, False)
+    assert batch.batch_size() == 3
+    assert (batch.get_spatial_locations().numpy() == p.spatial_locations(sp)).all()
+    assert (batch.features.cpu().numpy() == p.batch_features()).all()

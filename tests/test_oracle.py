@@ -45,6 +45,16 @@ def test_bl_input_layer_edge_cases(make):
     checks.check_bl_input_layer(make, 2, 1, seed=3, batch=5, length=1)
 
 
+@pytest.mark.parametrize("dim", [1, 2, 3])
+def test_input_batch(make, dim):
+    checks.check_input_batch(make, dim, seed=70 + dim)
+
+
+@pytest.mark.parametrize("dim,size,spatial", [(3, 2, 24), (3, 3, 23), (2, 2, (24, 12)), (2, 3, 47), (1, 2, 40)])
+def test_generate_rulebooks(make, dim, size, spatial):
+    checks.check_generate_rulebooks(make, dim, size, spatial, seed=80 + dim + size)
+
+
 @pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (2, (3, 1)), (3, (1, 3, 5)), (3, 2),
                                       (4, 3)])
 def test_submanifold(make, dim, size):
