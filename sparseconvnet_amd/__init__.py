@@ -24,7 +24,7 @@ from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, Bat
                      ValidConvolution)
 from .inputBatch import InputBatch  # noqa: E402
 from .metadata import Metadata  # noqa: E402
-from .networks import SparseVggNet, UNet  # noqa: E402
+from .networks import FullyConvolutionalNet, SparseResNet, SparseVggNet, UNet  # noqa: E402
 from .tensor import SparseConvNetTensor  # noqa: E402
 from .utils import (checkpoint_restore, checkpoint_save, is_power2, optionalTensor,  # noqa: E402
                     prepare_BLInput, toLongTensor)

@@ -22,7 +22,8 @@ def test_exports():
                  "BatchNormalization", "BatchNormReLU", "BatchNormLeakyReLU", "MaxPooling", "InputLayer",
                  "OutputLayer", "SparseToDense", "Metadata", "SparseConvNetTensor", "Sequential", "ConcatTable",
                  "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor",
-                 "NetworkInNetwork", "AveragePooling", "UnPooling", "BLInputLayer", "BLOutputLayer", "InputBatch"]:
+                 "NetworkInNetwork", "AveragePooling", "UnPooling", "BLInputLayer", "BLOutputLayer", "InputBatch", "SparseResNet",
+                 "FullyConvolutionalNet"]:
         assert hasattr(scn, name), name
     assert scn.forward_pass_multiplyAdd_count == 0 and scn.forward_pass_hidden_states == 0
 
@@ -191,6 +192,33 @@ def test_input_batch_collects_on_the_host():
     if not torch.cuda.is_available():
         with pytest.raises(Exception):
             b.features
+
+
+def test_remaining_builders_structure():
+    # networkArchitectures.py:33-130: ['C', a, b, c] = 3^d convolution beside branches one and two
+    # levels down; planes add up; module order inside the branches
+    m = scn.SparseVggNet(2, 3, [['C', 8, 4, 6]])
+    table, join, bn = m[0], m[1], m[2]
+    assert isinstance(table, scn.ConcatTable) and isinstance(join, scn.JoinTable) and bn.nPlanes == 18
+    kinds = [type(x).__name__ for x in table[2]]
+    assert kinds == ["Convolution", "BatchNormReLU", "SubmanifoldConvolution", "BatchNormReLU"] * 2 + [
+        "Deconvolution", "BatchNormReLU", "SubmanifoldConvolution", "BatchNormReLU", "Deconvolution"]
+    assert [type(x).__name__ for x in table[1]] == ["Convolution", "BatchNormReLU", "SubmanifoldConvolution",
+                                                    "BatchNormReLU", "Deconvolution"]
+    assert (m.input_spatial_size(torch.LongTensor([7, 7])) == 7).all()
+    # networkArchitectures.py:132-200: state-dict names of a two-stage ResNet
+    r = scn.SparseResNet(3, 4, [['basic', 8, 2, 1], ['basic', 16, 1, 2]])
+    keys = [k for k in r.state_dict() if k.endswith("weight") and "running" not in k]
+    assert keys == ['0.weight', '1.0.0.weight', '1.0.1.weight', '1.0.2.weight', '1.1.weight',
+                    '3.0.0.weight', '3.0.1.weight', '3.0.2.weight', '3.0.3.weight',
+                    '5.weight', '6.0.0.weight', '6.0.1.weight', '6.0.2.weight', '6.1.weight', '8.weight']
+    assert isinstance(r[1][1], scn.NetworkInNetwork) and isinstance(r[3][1], scn.Identity)
+    assert isinstance(r[6][1], scn.Convolution) and isinstance(r[6][0][0], scn.Convolution)
+    assert (r.input_spatial_size(torch.LongTensor([5, 5, 5])) == 11).all()
+    # networkArchitectures.py:259-312
+    f = scn.FullyConvolutionalNet(3, 1, [8, 16, 24])
+    assert isinstance(f[1][1][3], scn.UnPooling) and isinstance(f[2], scn.JoinTable)
+    assert (f.input_spatial_size(torch.LongTensor([8, 8, 8])) == 8).all()
 
 
 def test_no_cpu_fallback():

@@ -413,3 +413,50 @@ def test_input_batch_network_vs_oracle(oracle_built):
     assert batch.batch_size() == 3
     assert (batch.get_spatial_locations().numpy() == p.spatial_locations(sp)).all()
     assert (batch.features.cpu().numpy() == p.batch_features()).all()
+
+
+def _network_rows_vs_oracle(model, dim, spatial, coords, planes, seed, out_planes, what):
+    randomise_bn(model, seed)
+    rng = np.random.default_rng(seed)
+    feats = rng.uniform(-1, 1, size=(len(coords), planes)).astype(np.float32)
+    inp_layer = scn.InputLayer(dim, spatial, mode=3)
+    got, want, p = _run_both(model.eval(), inp_layer, [torch.as_tensor(coords), torch.as_tensor(feats)])
+    out_sp = got.spatial_size.numpy()
+    assert got.features.shape == (p.nactive(out_sp), out_planes), (got.features.shape, p.nactive(out_sp))
+    rows = lambda loc: cpu_path.canon_rows(loc)  # noqa: E731
+    checks.assert_close(got.features.cpu().numpy()[rows(got.get_spatial_locations().numpy())],
+                        want.features[rows(p.spatial_locations(out_sp))], what)
+
+
+def test_multiscale_vgg_vs_oracle(oracle_built):
+    """SparseVggNet's multi-scale 'C' layers (networkArchitectures.py:33-130): branches one, two
+    and three levels down by Convolution 3/2 and back up by Deconvolution 3/2, joined."""
+    torch.manual_seed(11)
+    model = scn.SparseVggNet(3, 3, [['C', 8, 4, 4, 4], 'MP', ['C', 8, 8], ['C3/2', 12]])
+    spatial = model.input_spatial_size(torch.LongTensor([7, 7, 7]))
+    assert (spatial == 31).all()
+    coords = synthetic.scene_batch(seed=11000, batch=2, target=2500, spatial=31, n_boxes=5)
+    _network_rows_vs_oracle(model, 3, 31, coords, 3, 11, 12, "multi-scale VGG")
+
+
+def test_resnet_vs_oracle(oracle_built):
+    """SparseResNet (networkArchitectures.py:132-200): identity, NetworkInNetwork and strided
+    Convolution shortcuts."""
+    torch.manual_seed(12)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, 8, 3, False)).add(
+        scn.SparseResNet(3, 8, [['basic', 8, 2, 1], ['basic', 12, 2, 1], ['basic', 16, 2, 2]]))
+    spatial = model.input_spatial_size(torch.LongTensor([15, 15, 15]))
+    assert (spatial == 31).all()
+    coords = synthetic.scene_batch(seed=12000, batch=2, target=2500, spatial=31, n_boxes=5)
+    _network_rows_vs_oracle(model, 3, 31, coords, 3, 12, 16, "ResNet")
+
+
+@pytest.mark.parametrize("residual", [False, True])
+def test_fully_convolutional_net_vs_oracle(oracle_built, residual):
+    """FullyConvolutionalNet (networkArchitectures.py:259-312): every level's features unpooled
+    to full resolution and joined."""
+    torch.manual_seed(13)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, 8, 3, False)).add(
+        scn.FullyConvolutionalNet(3, 2, [8, 12, 16], residual_blocks=residual))
+    coords = synthetic.scene_batch(seed=13000, batch=2, target=2500, spatial=32, n_boxes=5)
+    _network_rows_vs_oracle(model, 3, 32, coords, 3, 13, 36, "fully convolutional net")
