@@ -17,17 +17,21 @@ fuse_batchnorm = True
 # reference computes in fp32 throughout, which is also the default here.
 bf16_mfma = False
 
-from .containers import AddTable, ConcatTable, JoinTable, Sequential  # noqa: E402
+from .activations import (ELU, SELU, BatchNormELU, BatchwiseDropout, Dropout, LeakyReLU, ReLU,  # noqa: E402
+                          Sigmoid, Tanh)
+from .containers import AddTable, CheckpointedSequential, ConcatTable, JoinTable, Sequential  # noqa: E402
 from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, BatchNormReLU,  # noqa: E402
-                     BLInputLayer, BLOutputLayer, Convolution, Deconvolution, Identity, InputLayer, MaxPooling,
+                     BLInputLayer, BLOutputLayer, Convolution, Deconvolution, DenseToSparse, Identity, InputLayer,
+                     InputLayerInput, MaxPooling,
                      NetworkInNetwork, OutputLayer, SparseToDense, SubmanifoldConvolution, UnPooling,
                      ValidConvolution)
 from .inputBatch import InputBatch  # noqa: E402
 from .metadata import Metadata  # noqa: E402
 from .networks import FullyConvolutionalNet, SparseResNet, SparseVggNet, UNet  # noqa: E402
 from .tensor import SparseConvNetTensor  # noqa: E402
-from .utils import (checkpoint_restore, checkpoint_save, is_power2, optionalTensor,  # noqa: E402
-                    prepare_BLInput, toLongTensor)
+from .utils import (AddCoords, add_feature_planes, append_tensors, checkpoint_restore,  # noqa: E402
+                    checkpoint_save, compare_sparse, concatenate_feature_planes, is_power2,
+                    optionalTensor, prepare_BLInput, toLongTensor)
 
 
 def is_hip_build():

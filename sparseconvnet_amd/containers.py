@@ -63,6 +63,11 @@ class Sequential(torch.nn.Sequential):
         return self
 
 
+class CheckpointedSequential(Sequential):
+    """sequential.py:66-73 trades memory for recomputation in the backward pass; there is no
+    backward pass here, so this is Sequential under the reference's other name."""
+
+
 class _Table(torch.nn.Sequential):
     def __init__(self, *args):
         torch.nn.Sequential.__init__(self, *args)

@@ -509,3 +509,55 @@ class Identity(Module):
 
     def input_spatial_size(self, out_size):
         return out_size
+
+
+class DenseToSparse(Module):
+    """denseToSparse.py:13-67 over Metadata::createMetadataForDenseToSparse
+    (Metadata/Metadata.cpp:177-214): a dense [batch, planes, spatial...] tensor becomes a
+    sparse one whose sites are the cells with a non-zero plane, rows in (sample, row-major
+    cell) order.  Here: the non-zero cells' coordinates go through the input-layer construction
+    in mode 0 (rows = points)."""
+
+    def __init__(self, dimension):
+        Module.__init__(self)
+        self.dimension = dimension
+
+    def forward(self, input):
+        d = self.dimension
+        assert input.dim() == d + 2
+        if not input.is_cuda:
+            input = input.cuda()
+        output = SparseConvNetTensor(metadata=_md.Metadata(d), spatial_size=torch.LongTensor(list(input.shape[2:])))
+        cells = input.detach().permute(0, *range(2, 2 + d), 1)      # [batch, spatial..., planes]
+        nz = (cells.abs().sum(-1) != 0).nonzero()                    # [n, 1 + d]: sample first
+        coords = torch.cat([nz[:, 1:], nz[:, :1]], 1).contiguous()   # the library's column order
+        md, sz, batch = output.metadata, output.spatial_size, input.size(0)
+
+        def gather(x):
+            rows = x.permute(0, *range(2, 2 + d), 1)[tuple(nz.t())].float().contiguous()
+            return md.inputLayer(sz, coords, rows, batch, 0)
+        output.features = _run(gather, input)
+        return output
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+    def __repr__(self):
+        return 'DenseToSparse(' + str(self.dimension) + ')'
+
+
+class InputLayerInput(object):
+    """ioLayers.py:285-294: the (coords, features) pair an InputLayer takes, with .cuda()."""
+
+    def __init__(self, coords, features):
+        self.x = [coords, features]
+
+    def __getitem__(self, n):
+        return self.x[n]
+
+    def __len__(self):
+        return 2
+
+    def cuda(self):
+        self.x[1] = self.x[1].cuda()
+        return self

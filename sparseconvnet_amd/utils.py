@@ -83,3 +83,74 @@ def checkpoint_save(model, exp_name, name2, epoch, use_cuda=True):
     f = exp_name + '-%09d-' % epoch + name2 + '.pth'
     if os.path.isfile(f) and not is_power2(epoch):
         os.remove(f)
+
+
+def concatenate_feature_planes(input):
+    """utils.py:53-58: tensors over the same sites, planes side by side."""
+    from .tensor import SparseConvNetTensor
+    return SparseConvNetTensor(torch.cat([i.features for i in input], 1), input[0].metadata, input[0].spatial_size)
+
+
+def add_feature_planes(input):
+    """utils.py:61-66: tensors over the same sites, summed."""
+    from .tensor import SparseConvNetTensor
+    total = input[0].features
+    for i in input[1:]:
+        total = total + i.features
+    return SparseConvNetTensor(total, input[0].metadata, input[0].spatial_size)
+
+
+def append_tensors(tensors):
+    """utils.py:68-77 over Metadata::appendMetadata (Metadata/Metadata.cpp:248-262): the samples
+    of every tensor after those of the ones before it, rows in the same order.  The new
+    Metadata is built from the tensors' site lists (mode 0: rows = points)."""
+    from .metadata import Metadata
+    from .tensor import SparseConvNetTensor
+    spatial_size = tensors[0].spatial_size
+    dimension = len(spatial_size)
+    locations, first_sample = [], 0
+    for t in tensors:
+        loc = t.get_spatial_locations().clone()
+        loc[:, -1] += first_sample
+        locations.append(loc)
+        first_sample += t.batch_size()
+    features = torch.cat([t.features for t in tensors], 0)
+    md = Metadata(dimension)
+    rows = md.inputLayer(spatial_size, torch.cat(locations), features, first_sample, 0)
+    return SparseConvNetTensor(rows, md, spatial_size)
+
+
+class AddCoords(torch.nn.Module):
+    """utils.py:79-92: appends every site's coordinates, scaled to [-1, 1], as extra planes."""
+
+    def forward(self, input):
+        from .tensor import SparseConvNetTensor
+        features = input.features
+        if features.numel():
+            with torch.no_grad():
+                coords = input.get_spatial_locations()[:, :-1].to(features)
+                half = (input.spatial_size.to(features) - 1) / 2
+                coords = coords / half[None, :] - 1
+            features = torch.cat([features, coords], 1)
+        return SparseConvNetTensor(features, input.metadata, input.spatial_size)
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+
+def compare_sparse(x, y):
+    """utils.py:94-108 over Metadata::compareSparseHelper (Metadata/Metadata.cpp:585-616): mean
+    over the union of the two tensors' sites of the squared feature difference, a site missing
+    on one side counting with its squared features."""
+    dev = x.features.device
+    lx, ly = x.get_spatial_locations().to(dev), y.get_spatial_locations().to(dev)
+    both = torch.cat([lx, ly])
+    _, site = torch.unique(both, dim=0, return_inverse=True)
+    n = int(site.max()) + 1 if site.numel() else 0
+    planes = max(x.features.size(1) if x.features.dim() == 2 else 0, y.features.size(1) if y.features.dim() == 2 else 0)
+    diff = torch.zeros((n, planes), dtype=x.features.dtype, device=dev)
+    if lx.size(0):
+        diff.index_add_(0, site[:lx.size(0)], x.features)
+    if ly.size(0):
+        diff.index_add_(0, site[lx.size(0):], -y.features)
+    return diff.pow(2).sum() / n

@@ -23,7 +23,10 @@ def test_exports():
                  "OutputLayer", "SparseToDense", "Metadata", "SparseConvNetTensor", "Sequential", "ConcatTable",
                  "JoinTable", "AddTable", "Identity", "SparseVggNet", "UNet", "toLongTensor", "optionalTensor",
                  "NetworkInNetwork", "AveragePooling", "UnPooling", "BLInputLayer", "BLOutputLayer", "InputBatch", "SparseResNet",
-                 "FullyConvolutionalNet"]:
+                 "FullyConvolutionalNet", "DenseToSparse", "InputLayerInput", "ReLU", "LeakyReLU", "Tanh",
+                 "Sigmoid", "ELU", "SELU", "BatchNormELU", "Dropout", "BatchwiseDropout", "AddCoords",
+                 "append_tensors", "compare_sparse", "concatenate_feature_planes", "add_feature_planes",
+                 "CheckpointedSequential"]:
         assert hasattr(scn, name), name
     assert scn.forward_pass_multiplyAdd_count == 0 and scn.forward_pass_hidden_states == 0
 

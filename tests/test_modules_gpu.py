@@ -460,3 +460,102 @@ def test_fully_convolutional_net_vs_oracle(oracle_built, residual):
         scn.FullyConvolutionalNet(3, 2, [8, 12, 16], residual_blocks=residual))
     coords = synthetic.scene_batch(seed=13000, batch=2, target=2500, spatial=32, n_boxes=5)
     _network_rows_vs_oracle(model, 3, 32, coords, 3, 13, 36, "fully convolutional net")
+
+
+def test_dense_to_sparse_round_trip():
+    """DenseToSparse (denseToSparse.py:13-67): rows are the non-zero cells in (sample, row-major)
+    order; SparseToDense brings the dense tensor back; a convolution over the result agrees
+    with the dense one at the active sites."""
+    rng = np.random.default_rng(21)
+    dense = rng.normal(size=(3, 4, 9, 7)).astype(np.float32)
+    dense[rng.random((3, 1, 9, 7)).repeat(4, 1) < 0.6] = 0
+    dense[2] = 0                                   # a sample without sites still counts
+    x = scn.DenseToSparse(2)(torch.from_numpy(dense).cuda())
+    cells = np.argwhere(np.abs(dense).sum(1) != 0)   # [n, 3]: sample, y, x
+    assert x.batch_size() == 3 and (x.spatial_size == torch.LongTensor([9, 7])).all()
+    assert (x.get_spatial_locations().numpy() == cells[:, [1, 2, 0]]).all()
+    assert (x.features.cpu().numpy() == dense[cells[:, 0], :, cells[:, 1], cells[:, 2]]).all()
+    assert (scn.SparseToDense(2, 4)(x).cpu().numpy() == dense).all()
+    torch.manual_seed(21)
+    conv = scn.SubmanifoldConvolution(2, 4, 5, 3, True).cuda()
+    with torch.no_grad():
+        y = conv(x)
+    import bruteforce as bf
+    loc = x.get_spatial_locations().numpy()
+    want = bf.dense_subm_conv(loc, x.features.cpu().numpy(), conv.weight.detach().cpu().numpy(), (9, 7), 3, 3,
+                              conv.bias.detach().cpu().numpy())
+    checks.assert_close(y.features.cpu().numpy(), want, "convolution after DenseToSparse")
+
+
+def test_pointwise_modules_and_dropout():
+    torch.manual_seed(22)
+    coords = torch.LongTensor([[1, 2, 0], [3, 3, 0], [0, 1, 1], [4, 4, 1]])
+    feats = torch.randn(4, 6)
+    x = scn.InputLayer(2, 6, mode=0)([coords, feats.cuda()])
+    F = torch.nn.functional
+    for module, fn in [(scn.ReLU(), F.relu), (scn.LeakyReLU(), lambda t: F.leaky_relu(t, 1 / 3)),
+                       (scn.LeakyReLU(0.1), lambda t: F.leaky_relu(t, 0.1)), (scn.Tanh(), torch.tanh),
+                       (scn.Sigmoid(), torch.sigmoid), (scn.ELU(), F.elu), (scn.SELU(), F.selu),
+                       (scn.Dropout(0.25).eval(), lambda t: t * 0.75),
+                       (scn.BatchwiseDropout(0.4).eval(), lambda t: t * 0.6)]:
+        y = module(x)
+        assert y.metadata is x.metadata and (y.spatial_size == x.spatial_size).all()
+        assert torch.allclose(y.features.cpu(), fn(feats), rtol=1e-6, atol=1e-7), module
+        assert (module.input_spatial_size(torch.LongTensor([5, 5])) == 5).all()
+    kept = scn.Dropout(0.5).train()(x).features.cpu()
+    assert ((kept == 0) | (kept == feats)).all()
+    cols = scn.BatchwiseDropout(0.5).train()(x).features.cpu()
+    assert all((cols[:, c] == 0).all() or (cols[:, c] == feats[:, c]).all() for c in range(6))
+    bn_elu = scn.BatchNormELU(6).cuda().eval()
+    randomise_bn(bn_elu, 22)
+    with torch.no_grad():
+        got = bn_elu(x).features.cpu()
+    bn = bn_elu[0]
+    want = F.elu((feats - bn.running_mean.cpu()) / torch.sqrt(bn.running_var.cpu() + bn.eps) * bn.weight.detach().cpu()
+                 + bn.bias.detach().cpu())
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+
+
+def test_tensor_utilities():
+    """append_tensors, compare_sparse, AddCoords, concatenate / add_feature_planes
+    (utils.py:53-108)."""
+    rng = np.random.default_rng(23)
+
+    def tensor(seed, batch, n):
+        r = np.random.default_rng(seed)
+        c = np.unique(np.concatenate([r.integers(0, 8, (n, 3)), r.integers(0, batch, (n, 1))], 1), axis=0)
+        c = c[r.permutation(len(c))]
+        f = r.normal(size=(len(c), 4)).astype(np.float32)
+        return scn.InputLayer(3, 8, mode=0)([torch.from_numpy(c), torch.from_numpy(f).cuda()]), c, f
+
+    a, ca, fa = tensor(1, 2, 150)
+    b, cb, fb = tensor(2, 3, 100)
+    ab = scn.append_tensors([a, b])
+    assert ab.batch_size() == 5
+    shifted = cb.copy()
+    shifted[:, -1] += 2
+    assert (ab.get_spatial_locations().numpy() == np.concatenate([ca, shifted])).all()
+    assert (ab.features.cpu().numpy() == np.concatenate([fa, fb])).all()
+    torch.manual_seed(23)
+    conv = scn.SubmanifoldConvolution(3, 4, 6, 3, False).cuda()
+    with torch.no_grad():   # samples do not see each other: the appended batch convolves like its parts
+        assert torch.allclose(conv(ab).features, torch.cat([conv(a).features, conv(b).features]), rtol=1e-5,
+                              atol=1e-6)
+    # compare_sparse against a dictionary
+    c, cc, fc = tensor(3, 2, 150)
+    da = {tuple(k): v for k, v in zip(ca, fa.astype(np.float64))}
+    dc = {tuple(k): v for k, v in zip(cc, fc.astype(np.float64))}
+    assert set(da) & set(dc) and set(da) - set(dc) and set(dc) - set(da)
+    err = sum((((da.get(k, 0) - dc.get(k, 0)) ** 2).sum() for k in set(da) | set(dc))) / len(set(da) | set(dc))
+    assert abs(float(scn.compare_sparse(a, c)) - err) < 1e-4 * err
+    assert float(scn.compare_sparse(a, a)) == 0
+    # AddCoords: coordinates scaled to [-1, 1]
+    with_coords = scn.AddCoords()(a)
+    assert with_coords.features.shape == (len(ca), 7)
+    assert np.allclose(with_coords.features.cpu().numpy()[:, 4:], ca[:, :3] / 3.5 - 1, atol=1e-6)
+    assert (with_coords.features.cpu().numpy()[:, :4] == fa).all()
+    # planes side by side / summed
+    two = scn.concatenate_feature_planes([a, with_coords])
+    assert two.features.shape == (len(ca), 11) and two.metadata is a.metadata
+    assert torch.equal(scn.add_feature_planes([a, a, a]).features, a.features * 3)
+    assert rng is not None
