@@ -19,6 +19,8 @@ template class Metadata<1>;
 template class Metadata<2>;
 template class Metadata<3>;
 template class Metadata<4>;
+template class Metadata<5>;
+template class Metadata<6>;
 
 #include "CPU/BatchNormalization.cpp"
 #include "CPU/Convolution.cpp"
@@ -75,6 +77,8 @@ RuleBook &rb_get(Metadata<D> &m, int kind, const int64_t *a, const int64_t *b, c
   case 2: { constexpr Int D = 2; auto &m = *(Metadata<2> *)((Handle *)h)->m; __VA_ARGS__; } break; \
   case 3: { constexpr Int D = 3; auto &m = *(Metadata<3> *)((Handle *)h)->m; __VA_ARGS__; } break; \
   case 4: { constexpr Int D = 4; auto &m = *(Metadata<4> *)((Handle *)h)->m; __VA_ARGS__; } break; \
+  case 5: { constexpr Int D = 5; auto &m = *(Metadata<5> *)((Handle *)h)->m; __VA_ARGS__; } break; \
+  case 6: { constexpr Int D = 6; auto &m = *(Metadata<6> *)((Handle *)h)->m; __VA_ARGS__; } break; \
   }
 
 extern "C" {
@@ -86,6 +90,8 @@ void *ref_md_create(int dim) {
   case 2: h->m = new Metadata<2>(); break;
   case 3: h->m = new Metadata<3>(); break;
   case 4: h->m = new Metadata<4>(); break;
+  case 5: h->m = new Metadata<5>(); break;
+  case 6: h->m = new Metadata<6>(); break;
   default: delete h; return nullptr;
   }
   return h;

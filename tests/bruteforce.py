@@ -184,6 +184,33 @@ def triple_conv(triples, loc_in, loc_out, feats, w, bias=None):
     return y
 
 
+def rule_rows(triples, loc_in, loc_out):
+    """(k, in site, out site) triples as rows (k, in row, out row) of the two site lists."""
+    dim = loc_in.shape[1] - 1
+    row_in = {tuple(c): r for r, c in enumerate(loc_in.tolist())}
+    row_out = {tuple(c): r for r, c in enumerate(loc_out.tolist())}
+    return [(t[0], row_in[t[1:2 + dim]], row_out[t[2 + dim:]]) for t in triples]
+
+
+def rows_strided_ops(rows, x, y, w, w2, n_in, n_out, K, bias=None):
+    """Every op of a strided rulebook as loops over its rules, for dimensions beyond torch's
+    dense routines: convolution, max pooling (from zero), average pooling, and from the coarse
+    rows y back to the fine level unpooling and transposed convolution."""
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    conv = np.zeros((n_out, w.shape[3])) + (0 if bias is None else bias)
+    mp = np.zeros((n_out, x.shape[1]))
+    ap = np.zeros((n_out, x.shape[1]))
+    up = np.zeros((n_in, y.shape[1]))
+    dz = np.zeros((n_in, w2.shape[3]))
+    for k, i, j in rows:
+        conv[j] += x64[i] @ w[k, 0].astype(np.float64)
+        mp[j] = np.maximum(mp[j], x64[i])
+        ap[j] += x64[i] / K
+        up[i] += y64[j]
+        dz[i] += y64[j] @ w2[k, 0].astype(np.float64)
+    return conv, mp, ap, up, dz
+
+
 def dense_subm_conv(loc, feats, w, spatial, size, batch, bias=None):
     dim = loc.shape[1] - 1
     if dim not in _CONV:

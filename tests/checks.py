@@ -295,8 +295,25 @@ def check_strided(make, dim, size, stride, seed, out_spatial=4, n=150, batch=2, 
     b = rng.normal(size=cout).astype(np.float32) if bias else None
     y, macs = p.conv(in_sp, out_sp, size, stride, x, w, b)
     assert macs == len(expect) * cin * cout
-    dense = bf.dense_strided_conv(loc, x, w, in_sp, size, stride, batch, b)
-    assert_close(y, bf.sample_dense(dense, loc_out), "strided conv")
+    dense_ok = dim <= 3   # torch has dense convolutions and pooling up to three dimensions
+    rows = None if dense_ok else bf.rule_rows(expect, loc, loc_out)
+    want = {}
+    if dense_ok:
+        want["conv"] = bf.sample_dense(bf.dense_strided_conv(loc, x, w, in_sp, size, stride, batch, b), loc_out)
+    else:
+        want["conv"] = bf.rows_strided_ops(rows, x, np.zeros((len(loc_out), 1), np.float32), w,
+                                           np.zeros((K, 1, 1, 1), np.float32), len(loc), len(loc_out), K, b)[0]
+    assert_close(y, want["conv"], "strided conv")
+    if not dense_ok:
+        w2 = (rng.normal(size=(K, 1, cout, cin)) * 0.3).astype(np.float32)
+        _, want_mp, want_ap, want_up, want_dz = bf.rows_strided_ops(rows, x, y, w, w2, len(loc), len(loc_out), K)
+        assert_close(p.maxpool(in_sp, out_sp, size, stride, x), want_mp, "max pooling")
+        assert_close(p.avgpool(in_sp, out_sp, size, stride, x), want_ap, "average pooling")
+        assert_close(p.unpool(out_sp, in_sp, size, stride, y), want_up, "unpooling")
+        z, macs2 = p.deconv(out_sp, in_sp, size, stride, y, w2)
+        assert macs2 == len(expect) * cin * cout
+        assert_close(z, want_dz, "deconvolution")
+        return p
     # max pooling over the same rulebook: zero-initialised, so max(0, active inputs)
     mp = p.maxpool(in_sp, out_sp, size, stride, x)
     dmp = bf.dense_maxpool(loc, x, in_sp, size, stride, batch)

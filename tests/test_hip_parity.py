@@ -54,6 +54,16 @@ def test_generate_rulebooks(make, dim, size, spatial):
     checks.check_generate_rulebooks(make, dim, size, spatial, seed=80 + dim + size)
 
 
+@pytest.mark.parametrize("dim", [5, 6])
+def test_high_dimensions(make, dim):
+    # sparseconvnet_cpu.cpp:14-20 instantiates dimensions 1..6
+    checks.check_input_layer(make, dim, 4, seed=90 + dim, spatial=3, n=250)
+    checks.check_submanifold(make, dim, 3 if dim == 5 else (3, 1, 3, 1, 3, 1), seed=91 + dim, spatial=3, n=150)
+    checks.check_strided(make, dim, 2, 2, seed=92 + dim, out_spatial=2, n=150)
+    checks.check_s2d(make, dim, seed=93 + dim, spatial=3, n=80)
+    checks.check_input_batch(make, dim, seed=94 + dim, spatial=4)
+
+
 @pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (2, (3, 1)), (3, (1, 3, 5)), (3, 2),
                                       (4, 3)])
 def test_submanifold(make, dim, size):
