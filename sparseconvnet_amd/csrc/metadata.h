@@ -50,6 +50,7 @@ struct Level {
 // (Metadata::pending_macs), which is why it is held by shared_ptr.
 struct Counts {
   int K = 0;
+  int slots = 1;  // the device holds this many partial copies of the K counts, one after the other
   DevBuf<long long> dev;
   std::vector<int64_t> host;
   bool ready = false;  // host is valid
@@ -59,7 +60,7 @@ struct Counts {
     return s;
   }
 };
-void ensure_counts(Counts &c, hipStream_t s);  // fetches dev into host (one stream synchronisation)
+void ensure_counts(Counts &c, hipStream_t s);  // fetches dev into host, summed over the copies (one stream synchronisation)
 
 struct Table {
   int K = 0;
@@ -128,6 +129,16 @@ __device__ inline int listed_point(const int *sorted_idx, int st, int len, int m
 }
 
 struct Metadata {
+  Metadata() = default;
+  Metadata(const Metadata &) = delete;
+  Metadata &operator=(const Metadata &) = delete;
+  ~Metadata() {
+    if (pinned) (void)hipHostFree(pinned);
+  }
+  // Pinned host words that the constructions copy their sizes and flags into: a copy into
+  // pageable memory would be staged and waited for by the runtime, one round trip per copy.
+  static constexpr int PINNED_WORDS = 2048;
+  int *pinned = nullptr;
   int dim = 0;
   std::map<SizeKey, Level> levels;
   InputRules input;

@@ -110,6 +110,45 @@ void fill32(void *p, uint32_t v, int64_t n, hipStream_t s) {
   LAUNCH_CHECK();
 }
 
+// Three fills in one launch (a strided rulebook starts from two empty tables and zeroed
+// counts; at the deep levels of a network every launch saved is time saved).  blockIdx.y
+// picks the buffer; sizes in words, all multiples of four on 16-byte aligned buffers, else
+// three separate fills.
+struct Fill3 {
+  uint4 *p[3];
+  uint32_t v[3];
+  int64_t n4[3];
+};
+__global__ void k_fill3(Fill3 f) {
+  const int b = blockIdx.y;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const uint4 vv = make_uint4(f.v[b], f.v[b], f.v[b], f.v[b]);
+  for (; i < f.n4[b]; i += stride) f.p[b][i] = vv;
+}
+static void fill3(void *p0, uint32_t v0, int64_t n0, void *p1, uint32_t v1, int64_t n1, void *p2, uint32_t v2,
+                  int64_t n2, hipStream_t s) {
+  void *p[3] = {p0, p1, p2};
+  const uint32_t v[3] = {v0, v1, v2};
+  const int64_t n[3] = {n0, n1, n2};
+  bool wide = true;
+  for (int b = 0; b < 3; b++) wide = wide && n[b] > 0 && n[b] % 4 == 0 && (uintptr_t)p[b] % 16 == 0;
+  if (!wide) {
+    for (int b = 0; b < 3; b++) fill32(p[b], v[b], n[b], s);
+    return;
+  }
+  Fill3 f;
+  int64_t most = 0;
+  for (int b = 0; b < 3; b++) {
+    f.p[b] = (uint4 *)p[b];
+    f.v[b] = v[b];
+    f.n4[b] = n[b] / 4;
+    most = std::max(most, f.n4[b]);
+  }
+  k_fill3<<<dim3((unsigned)std::min<int64_t>(ceil_div(most, TB), 256 * 32), 3), TB, 0, s>>>(f);
+  LAUNCH_CHECK();
+}
+
 static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout,
                        const int *vin, int *vout, int64_t n, hipStream_t s, int end_bit = 64) {
   size_t bytes = 0;
@@ -122,6 +161,16 @@ static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipS
   HIP_CHECK(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, in, out, (int)n, s));
   m.tmp.reserve(bytes + 16);
   HIP_CHECK(hipcub::DeviceScan::ExclusiveSum(m.tmp.p, bytes, in, out, (int)n, s));
+}
+// Copies `words` ints from the device into the handle's pinned words and waits for them: the
+// one host round trip of a construction step.
+static const int *fetch_words(Metadata &m, const int *dev, int words, hipStream_t s) {
+  if (words > Metadata::PINNED_WORDS) throw Error("internal: read-back larger than the pinned words");
+  if (!m.pinned)
+    HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&m.pinned), Metadata::PINNED_WORDS * sizeof(int), hipHostMallocDefault));
+  HIP_CHECK(hipMemcpyAsync(m.pinned, dev, words * sizeof(int), hipMemcpyDeviceToHost, s));
+  HIP_CHECK(hipStreamSynchronize(s));
+  return m.pinned;
 }
 template <class T> static T read_back(const T *dev, hipStream_t s) {
   T h;
@@ -147,7 +196,7 @@ static void alloc_level(Level &l, const Geom &g, int64_t n, int batch) {
 // apart), and only when it can raise the slot (the plain read may be stale, which costs an
 // atomic that changes nothing).  20 000 same-address atomics cost ~130 us on a 1.3 M-point
 // input, this costs ~10.  Every thread of the workgroup must call it; values <= floor are
-// not reported.  The host takes the maximum over the slots (max_slots).
+// not reported.  The host takes the maximum over the slots.
 static const int MAX_SLOTS = 64, MAX_SLOT_STRIDE = 16;
 __device__ inline void grid_max(int v, int floor, int *slots) {
   __shared__ int block_max;
@@ -158,14 +207,6 @@ __device__ inline void grid_max(int v, int floor, int *slots) {
   __syncthreads();
   int *slot = slots + MAX_SLOT_STRIDE * (blockIdx.x & (MAX_SLOTS - 1));
   if (threadIdx.x == 0 && block_max > floor && block_max > __builtin_nontemporal_load(slot)) atomicMax(slot, block_max);
-}
-static int max_slots(const int *slots, hipStream_t s) {  // one stream synchronisation
-  int h[MAX_SLOTS * MAX_SLOT_STRIDE];
-  HIP_CHECK(hipMemcpyAsync(h, slots, sizeof h, hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipStreamSynchronize(s));
-  int v = 0;
-  for (int i = 0; i < MAX_SLOTS; i++) v = std::max(v, h[i * MAX_SLOT_STRIDE]);
-  return v;
 }
 
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
@@ -225,6 +266,7 @@ __global__ void k_input_rows_identity(Geom g, const int64_t *coords, int64_t n, 
 __global__ void k_group_heads(const unsigned long long *skeys, const int *sidx, int64_t n, int64_t n_valid,
                               int *head, int *is_first) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p == n) head[p] = 0;  // one element past the end, so that a scan of n + 1 ends with the total
   if (p >= n) return;
   int h = (p < n_valid && (p == 0 || skeys[p] != skeys[p - 1])) ? 1 : 0;
   head[p] = h;
@@ -322,9 +364,8 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   fill32(m.dflags.p, 0, n_flags, s);
   k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, bl_length, m.k0.p, m.v0.p, m.dflags.p);
   LAUNCH_CHECK();
-  std::vector<int> hflags(n_flags);
-  HIP_CHECK(hipMemcpyAsync(hflags.data(), m.dflags.p, n_flags * sizeof(int), hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipStreamSynchronize(s));
+  const int *fetched = fetch_words(m, m.dflags.p, n_flags, s);
+  const std::vector<int> hflags(fetched, fetched + n_flags);
   if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
   if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");
   int top_batch = 0;
@@ -354,19 +395,15 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
     return;
   }
 
-  m.f0.reserve(n);  // head
+  m.f0.reserve(n + 1);  // head
   m.f1.reserve(n);  // is_first
   m.s0.reserve(n + 1);  // head_scan
   m.s1.reserve(n + 1);  // first_scan
-  k_group_heads<<<grid_for(n), TB, 0, s>>>(m.k1.p, m.v1.p, n, nv, m.f0.p, m.f1.p);
+  k_group_heads<<<grid_for(n + 1), TB, 0, s>>>(m.k1.p, m.v1.p, n, nv, m.f0.p, m.f1.p);
   LAUNCH_CHECK();
-  exclusive_scan(m, m.f0.p, m.s0.p, n, s);
+  exclusive_scan(m, m.f0.p, m.s0.p, n + 1, s);  // head[n] = 0: the scan's last element is the number of groups
   exclusive_scan(m, m.f1.p, m.s1.p, n, s);
-  int last[2];
-  HIP_CHECK(hipMemcpyAsync(&last[0], m.s0.p + (n - 1), sizeof(int), hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipMemcpyAsync(&last[1], m.f0.p + (n - 1), sizeof(int), hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipStreamSynchronize(s));
-  int64_t N = (int64_t)last[0] + last[1];
+  const int64_t N = fetch_words(m, m.s0.p + n, 1, s)[0];
   alloc_level(L, g, N, batch);
   L.sched.reserve(N);
   L.identity_sched = false;
@@ -395,9 +432,13 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
                                               R.row_of_input.p, R.run_start.p, R.run_len.p,
                                               m.dflags.p + 8);
   LAUNCH_CHECK();
-  int ma = std::max(1, max_slots(m.dflags.p + 8, s));  // runs of one never touch the slots
-  // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2.
-  R.max_active = (mode == 3 || mode == 4) ? ma : 1;
+  // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2, the longest run for the
+  // summing modes (runs of one never touch the slots).
+  R.max_active = 1;
+  if (mode == 3 || mode == 4) {
+    const int *h = fetch_words(m, m.dflags.p + 8, MAX_SLOTS * MAX_SLOT_STRIDE, s);
+    for (int i = 0; i < MAX_SLOTS; i++) R.max_active = std::max(R.max_active, h[i * MAX_SLOT_STRIDE]);
+  }
 }
 
 // Reference layout of the rule rows (Metadata/IOLayersRules.h:96-119).
@@ -841,26 +882,21 @@ static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const
 
 // Rule counts are tallied per workgroup in LDS and flushed with one atomic per tap into one of
 // COUNT_SLOTS copies of the counter array (a million-site level has 15 000 workgroups; all of
-// them adding to the same K addresses cost 160 us of a 700 us rulebook build).  fold_counts
-// then sums the copies into the first one, which is the one everybody reads.
-static void start_counts(Table &t, hipStream_t s) {
+// them adding to the same K addresses cost 160 us of a 700 us rulebook build).  Whoever reads
+// the counts on the host sums the copies there (ensure_counts, take_macs).
+static void start_counts(Table &t, hipStream_t s, bool clear = true) {
   t.cnt = std::make_shared<Counts>();
   t.cnt->K = t.K;
+  t.cnt->slots = COUNT_SLOTS;
   const int64_t words = (int64_t)COUNT_SLOTS * std::max(t.K, 1);
   t.cnt->dev.reserve(words);
-  fill32(t.cnt->dev.p, 0, 2 * words, s);
+  if (clear) fill32(t.cnt->dev.p, 0, 2 * words, s);
 }
-__global__ void k_fold_counts(unsigned long long *counts, int K) {
-  const int k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= K) return;
-  unsigned long long v = 0;
-  for (int sl = 1; sl < COUNT_SLOTS; sl++) v += counts[(size_t)sl * K + k];
-  counts[k] += v;
-}
-static void fold_counts(Table &t, hipStream_t s) {
-  if (t.K <= 0) return;
-  k_fold_counts<<<grid_for(t.K), TB, 0, s>>>((unsigned long long *)t.cnt->dev.p, t.K);
-  LAUNCH_CHECK();
+static void fold_on_host(Counts &c, const long long *copies) {
+  c.host.assign(c.K, 0);
+  for (int sl = 0; sl < c.slots; sl++)
+    for (int k = 0; k < c.K; k++) c.host[k] += copies[(size_t)sl * c.K + k];
+  c.ready = true;
 }
 static void zero_counts(Table &t) {  // a table without rules
   t.cnt = std::make_shared<Counts>();
@@ -870,13 +906,12 @@ static void zero_counts(Table &t) {  // a table without rules
 }
 void ensure_counts(Counts &c, hipStream_t s) {
   if (c.ready) return;
-  std::vector<unsigned long long> h(c.K);
+  std::vector<long long> h((size_t)c.K * c.slots);
   if (c.K && c.dev.p) {
-    HIP_CHECK(hipMemcpyAsync(h.data(), c.dev.p, c.K * sizeof(long long), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipMemcpyAsync(h.data(), c.dev.p, h.size() * sizeof(long long), hipMemcpyDeviceToHost, s));
     HIP_CHECK(hipStreamSynchronize(s));
   }
-  c.host.assign(h.begin(), h.end());
-  c.ready = true;
+  fold_on_host(c, h.data());
 }
 // A forward call over table t did per_rule multiply-adds per rule.  With macs != NULL the
 // caller wants the number now; otherwise it is remembered and summed up by take_macs().
@@ -894,7 +929,7 @@ void note_macs(Metadata &m, Table &t, double per_rule, double *macs, hipStream_t
 // are asynchronous, with one synchronisation per staging buffer's worth (in practice one).
 double take_macs(Metadata &m, hipStream_t s) {
   static thread_local long long *stage = nullptr;
-  constexpr size_t STAGE = 8192;  // entries
+  constexpr size_t STAGE = 32768;  // entries: about thirty 27-tap rulebooks with all their copies
   if (!stage) HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&stage), STAGE * sizeof(long long), hipHostMallocDefault));
   std::vector<Counts *> batch;
   size_t used = 0;
@@ -903,9 +938,8 @@ double take_macs(Metadata &m, hipStream_t s) {
     HIP_CHECK(hipStreamSynchronize(s));
     size_t off = 0;
     for (Counts *c : batch) {
-      c->host.assign(stage + off, stage + off + c->K);
-      c->ready = true;
-      off += c->K;
+      fold_on_host(*c, stage + off);
+      off += (size_t)c->K * c->slots;
     }
     batch.clear();
     used = 0;
@@ -913,13 +947,14 @@ double take_macs(Metadata &m, hipStream_t s) {
   for (auto &pm : m.pending_macs) {
     Counts &c = *pm.first;
     if (c.ready || std::find(batch.begin(), batch.end(), &c) != batch.end()) continue;
-    if (!c.K || !c.dev.p || (size_t)c.K > STAGE) {  // nothing on the device (or absurdly many taps): the slow way
+    const size_t words = (size_t)c.K * c.slots;
+    if (!c.K || !c.dev.p || words > STAGE) {  // nothing on the device (or absurdly many taps): the slow way
       ensure_counts(c, s);
       continue;
     }
-    if (used + c.K > STAGE) flush();
-    HIP_CHECK(hipMemcpyAsync(stage + used, c.dev.p, c.K * sizeof(long long), hipMemcpyDeviceToHost, s));
-    used += c.K;
+    if (used + words > STAGE) flush();
+    HIP_CHECK(hipMemcpyAsync(stage + used, c.dev.p, words * sizeof(long long), hipMemcpyDeviceToHost, s));
+    used += words;
     batch.push_back(&c);
   }
   flush();
@@ -965,7 +1000,6 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
                                                            L.gridp.p, L.urow_ptr(), t.nbr.p,
                                                            (unsigned long long *)t.cnt->dev.p);
     LAUNCH_CHECK();
-    fold_counts(t, s);
     finalize_table(m, t, L.sched_ptr(), s);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
@@ -975,7 +1009,6 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
       L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p, L.gridp.p, L.urow_ptr(), t.nbr.p,
       (unsigned long long *)t.cnt->dev.p, parts);
   LAUNCH_CHECK();
-  fold_counts(t, s);
   finalize_table(m, t, L.sched_ptr(), s);
   return m.subm.emplace(key, std::move(t)).first->second;
 }
@@ -1014,6 +1047,7 @@ __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, c
 
 __global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p == n) head[p] = 0;  // one element past the end, so that a scan of n + 1 ends with the total
   if (p >= n) return;
   head[p] = (skeys[p] != SCN_EMPTY_KEY && (p == 0 || skeys[p] != skeys[p - 1])) ? 1 : 0;
 }
@@ -1101,7 +1135,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   m.k1.reserve(nc);
   m.v0.reserve(nc);
   m.v1.reserve(nc);
-  m.f0.reserve(nc);
+  m.f0.reserve(nc + 1);
   m.s0.reserve(nc + 1);
   k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), n, LI.npad,
                                                    m.k0.p, m.v0.p);
@@ -1119,14 +1153,10 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
     sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
   }
-  k_strided_heads<<<grid_for(nc), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
+  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
   LAUNCH_CHECK();
-  exclusive_scan(m, m.f0.p, m.s0.p, nc, s);
-  int last[2];
-  HIP_CHECK(hipMemcpyAsync(&last[0], m.s0.p + (nc - 1), sizeof(int), hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipMemcpyAsync(&last[1], m.f0.p + (nc - 1), sizeof(int), hipMemcpyDeviceToHost, s));
-  HIP_CHECK(hipStreamSynchronize(s));
-  int64_t n_out = (int64_t)last[0] + last[1];
+  exclusive_scan(m, m.f0.p, m.s0.p, nc + 1, s);
+  const int64_t n_out = fetch_words(m, m.s0.p + nc, 1, s)[0];
   alloc_level(LO, go, n_out, batch);
   R.by_out.n = n_out;
   R.by_out.npad = LO.npad;
@@ -1134,14 +1164,14 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   R.by_in.npad = LI.npad;
   R.by_out.nbr.reserve((size_t)f.K * LO.npad);
   R.by_in.nbr.reserve((size_t)f.K * LI.npad);
-  fill32(R.by_out.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LO.npad, s);
-  fill32(R.by_in.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LI.npad, s);
-  start_counts(R.by_out, s);
+  start_counts(R.by_out, s, false);
+  // both tables start empty and the counts at zero, in one launch
+  fill3(R.by_out.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LO.npad, R.by_in.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LI.npad,
+        R.by_out.cnt->dev.p, 0u, 2 * (int64_t)COUNT_SLOTS * std::max(f.K, 1), s);
   k_strided_emit<<<grid_for(nc), TB, f.K * sizeof(int), s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), LI.npad, m.k1.p, m.v1.p,
                                              m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
                                              LO.coords.p, LO.keys.p, (unsigned long long *)R.by_out.cnt->dev.p);
   LAUNCH_CHECK();
-  fold_counts(R.by_out, s);
   R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
   finalize_table(m, R.by_out, nullptr, s);
   return m.strided.emplace(key, std::move(R)).first->second;
