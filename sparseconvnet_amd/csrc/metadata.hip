@@ -12,6 +12,7 @@
 //   * rules are stored output-stationary as a table nbr[tap][position] instead of
 //     per-tap pair lists; pair lists are produced on demand by ballot/prefix compaction.
 #include <hipcub/hipcub.hpp>
+#include <rocprim/rocprim.hpp>
 
 #include <algorithm>
 
@@ -149,9 +150,27 @@ static void fill3(void *p0, uint32_t v0, int64_t n0, void *p1, uint32_t v1, int6
   LAUNCH_CHECK();
 }
 
+// Stable sort of (key, value) pairs by the low end_bit bits of the key.  The library's default
+// takes a merge sort up to a million items, whatever the number of key bits: log2(n / block)
+// passes.  The tables sorted here have few key bits (a tap pattern and a window number), so
+// from a few ten thousand rows on the radix sort's end_bit / 8 passes are fewer, and it is
+// chosen by hand.
+using RadixAlways = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                               rocprim::default_config, 4096>;
 static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout,
                        const int *vin, int *vout, int64_t n, hipStream_t s, int end_bit = 64) {
+  int merge_passes = 1;
+  while (((int64_t)2048 << merge_passes) < n) merge_passes++;
+  const bool radix = n > 32768 && (end_bit + 7) / 8 + 1 < merge_passes;
   size_t bytes = 0;
+  if (radix) {
+    HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                                     (unsigned)end_bit, s));
+    m.tmp.reserve(bytes + 16);
+    HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(m.tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                                     (unsigned)end_bit, s));
+    return;
+  }
   HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
   m.tmp.reserve(bytes + 16);
   HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
