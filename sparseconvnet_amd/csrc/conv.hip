@@ -1361,7 +1361,7 @@ static bool try_resident(Metadata &m, const Table &t, const float *in, float *ou
   return true;
 }
 
-// Mid-width layers (32 < nOut <= 128): row-owner kernel with 128-row workgroups (measured
+// Mid-width layers (32 < nOut <= 128): row-owner kernel with 128- or 64-row workgroups (measured
 // best on room scenes: small workgroups, five or more per CU, even out the work between
 // barriers better than 256- or 512-row ones).  Above 128 outputs the accumulators of a
 // granule no longer leave room for this layout's operands and k_conv_mfma is as fast.
@@ -1370,12 +1370,19 @@ static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *o
                           Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
   const int ncb = (int)ceil_div(n_out, 16);
   const bool narrow = n_in <= 16;
+  // 64-row workgroups where 128-row ones would leave a CU with one or two of them (a level of
+  // 60 k sites is 480 such workgroups for 256 CUs: one wavefront per SIMD, nothing to run while
+  // it waits for its gathers).  Measured: 13-18 % faster at 62 k sites, 5 % at 15 k and 250 k,
+  // equal at 1 M except for 64 output planes, which gain 2 % there too.
+  if (!narrow && ncb > 2 && (t.n < 300000 || ncb <= 4)) {
+    if (ncb <= 4) return launch_rows<4, 1, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+    if (ncb <= 6) return launch_rows<6, 1, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+    if (ncb <= 8) return launch_rows<8, 1, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+  }
   if (ncb <= 2)
     return narrow ? launch_rows<2, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
                   : launch_rows<2, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-  if (ncb <= 4)
-    return narrow ? launch_rows<4, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
-                  : launch_rows<4, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+  if (ncb <= 4) return launch_rows<4, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);  // narrow
   if (ncb <= 6)
     return narrow ? launch_rows<6, 2, 1, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s)
                   : launch_rows<6, 2, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
