@@ -88,7 +88,7 @@ def cpu_baseline(sample_sites, seed):
                       % (len(coords), R, t_rules)}
 
 
-def unet_scene(sites, seed, reps=3, residual=False, batch=1):
+def unet_scene(sites, seed, reps=7, residual=False, batch=1):
     """3D U-Net forward of examples/ScanNet/unet.py:25-38 with m=32, block_reps=2 (7 levels,
     [32..224] planes), InputLayer mode 4 on a room scene with ~30% duplicated points, eval,
     random-init weights, batch 1.  cold = new Metadata per scene, as a user runs it (input layer,
