@@ -248,6 +248,54 @@ def other_ops(sites, seed):
                    gflops=round(2.0 * n * 64 * 32 / (ms * 1e-3) / 1e9, 1)))
     ms = timed(lambda: md.maxPooling(sz, half, two, two, x32, 0))
     out.append(row("MaxPooling 2^3 / stride 2, 32 planes", ms, n * 32 * 4 + 8 * n + nc * 32 * 4))
+    ms = timed(lambda: md.averagePooling(sz, half, two, two, x32, 0))
+    out.append(row("AveragePooling 2^3 / stride 2, 32 planes", ms, n * 32 * 4 + 8 * n + nc * 32 * 4))
+    xc32 = torch.randn((nc, 32), device="cuda", generator=g)
+    ms = timed(lambda: md.unPooling(half, sz, two, two, xc32, 0))
+    out.append(row("UnPooling 2^3 / stride 2, 32 planes", ms, nc * 32 * 4 + 8 * n + n * 32 * 4))
+
+    # the other two input routes on the same points: batch-by-length (one sample, every position
+    # filled) and the point-at-a-time batch with a third of its points overwriting
+    cbl = cd[:, :3].reshape(1, npts, 3).contiguous()
+    fbl = feats.reshape(1, npts, 3)
+
+    def bl_layer():
+        m3 = M.Metadata(3)
+        m3.blInputLayer(sz, cbl, fbl, 4)
+        return m3
+    ms = host_timed(bl_layer)
+    out.append(row("BLInputLayer mode 4: rules + level + forward (%d points)" % npts, ms,
+                   npts * 24 + n * 24 + npts * 8 + npts * 12 + n * 12, points_per_s=round(npts / (ms * 1e-3))))
+    flags = (torch.arange(npts, device="cuda") % 3 == 0).to(torch.uint8)
+
+    def input_batch():
+        m3 = M.Metadata(3)
+        m3.inputBatch(sz, cd, feats, flags, 1)
+        return m3
+    ms = host_timed(input_batch)
+    out.append(row("InputBatch (a third of the points overwrite): level + features (%d points)" % npts, ms,
+                   npts * 33 + n * 24 + npts * 8 + npts * 12 + n * 12, points_per_s=round(npts / (ms * 1e-3))))
+
+    def chain():
+        m3 = M.Metadata(3)
+        m3.inputLayer(sz, cd, feats, 0, 4)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        m3.generateRuleBooks2s2()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3, m3
+    t = []
+    for _ in range(4):
+        dt, m3 = chain()
+        t.append(dt)
+        levels = [m3.getNActive(torch.LongTensor([4096 >> l] * 3)) for l in range(13)]
+        del m3
+    ms = float(np.median(t[1:]))
+    total = sum(levels)
+    # per level: keys read, 27-tap table written, the strided pair of tables and the next level written
+    out.append(row("precompute_metadata(2): 3^3 and 2^3/stride-2 rulebooks of all %d levels (%d sites in all)"
+                   % (sum(1 for v in levels if v), total), ms, total * (8 + 27 * 4 + 24 + 2 * 8 * 4),
+                   sites_per_s=round(total / (ms * 1e-3))))
     # sparse to dense on a grid that can be dense: the same scene generator at 128^3, 16 planes
     c2 = synthetic.room_scene(seed=seed + 1, target=200000, spatial=128)
     md2 = M.Metadata(3)
