@@ -77,7 +77,7 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
 //         table of a strided rulebook that is the copy of the one coarse row above each site).
 enum { POOL_MAX = 0, POOL_AVERAGE = 1, POOL_UNPOOL = 2 };
 template <int V, int MODE>
-__global__ void k_pool(const int *nbr, const int *rowmap, int K, int64_t n_out, int64_t npad,
+__global__ void k_pool(const int *nbr, const int *rowmap, const unsigned *gmask, int K, int64_t n_out, int64_t npad,
                        const float *in, int in_stride, float *out, int planes) {
   const int groups = planes / V;
   const float volume = (float)K;
@@ -89,7 +89,11 @@ __global__ void k_pool(const int *nbr, const int *rowmap, int K, int64_t n_out, 
     const int p = (int)(i - o * groups) * V;
     float acc[V];
     for (int v = 0; v < V; v++) acc[v] = 0.0f;
+    // taps that no row of this 16-row granule has are skipped without a look at the table (the
+    // fine side of a filter = stride rulebook has one tap per row, and the rows are sorted by it)
+    const unsigned present = gmask ? gmask[o >> 4] : 0xFFFFFFFFu;
     for (int k = 0; k < K; k++) {
+      if (gmask && !((present >> k) & 1u)) continue;
       const int j = nbr[(int64_t)k * npad + o];
       if (j >= 0) {
         const float *src = in + (int64_t)j * in_stride + p;
@@ -125,11 +129,12 @@ static void pool_launch(const Table &t, const float *in, int in_stride, float *o
                    ((uintptr_t)out % 16 == 0);
   int64_t total = t.n * (vec ? planes / 4 : planes);
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  const unsigned *gm = t.K <= 32 ? t.gmask.p : nullptr;  // null when the table kept no granule masks
   if (vec)
-    k_pool<4, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+    k_pool<4, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in + drop,
                                                           in_stride, out, planes);
   else
-    k_pool<1, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in + drop,
+    k_pool<1, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in + drop,
                                                           in_stride, out, planes);
   LAUNCH_CHECK();
 }
