@@ -160,6 +160,22 @@ int scn_rules_export(scn_metadata *md, int kind, const int64_t *a, const int64_t
  * after a network has been enqueued, it keeps the GPU busy in between.  The reference has no
  * counterpart; its Python layer sums the per-call values (sparseconvnet/__init__.py:7). */
 int scn_md_take_macs(scn_metadata *md, void *stream, double *macs);
+/* A handle that is destroyed or cleared while it still owes such a total does not wait for the
+ * GPU: its rule counts are copied to pinned memory behind the work already enqueued.  This call
+ * waits for those copies and returns (and resets) the multiply-adds of all handles that are
+ * gone.  No counterpart in the reference. */
+int scn_take_released_macs(double *macs);
+
+/* The library's own device buffers (rulebooks, levels, scratch) come from a process-wide cache
+ * of blocks that outlive the handle that used them, so that a stream of scenes does no
+ * hipMalloc / hipFree.  scn_release_cache waits for the device and gives every idle block back
+ * to the driver (call it when another allocator in the process runs out of memory);
+ * scn_cache_stats reports bytes in use by live handles, idle bytes held, the high-water mark of
+ * their sum and the number of hipMalloc calls made so far (any pointer may be NULL).  No
+ * counterpart in the reference, whose rulebooks live in host memory. */
+int scn_release_cache(void);
+int scn_cache_stats(int64_t *live_bytes, int64_t *idle_bytes, int64_t *peak_bytes,
+                    int64_t *device_allocations);
 
 /* InputLayer_updateOutput after the rules exist (pybind.cpp:155-159, CPU/IOLayers.cpp:49-72):
  * in [nInputRows, planes] -> out [nActive, planes]. */

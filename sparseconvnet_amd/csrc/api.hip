@@ -16,11 +16,20 @@ static thread_local std::string g_error;
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <unordered_map>
 
 namespace scn {
 namespace {
 std::mutex g_pool_mutex;
-std::multimap<std::tuple<int, int, size_t>, void *> g_pool;  // (device, cache, size class) -> free blocks
+// An idle block remembers the stream its last user enqueued on: handed to a call that runs on
+// another stream, that stream is first made to wait for everything the old one holds.
+struct IdleBlock {
+  void *p;
+  hipStream_t last;
+};
+std::multimap<std::tuple<int, int, size_t>, IdleBlock> g_pool;  // (device, cache, bytes) -> idle blocks
+std::unordered_map<void *, size_t> g_block_bytes;                // every block the cache has handed out or holds
+int64_t g_idle_bytes = 0, g_live_bytes = 0, g_peak_bytes = 0, g_mallocs = 0;
 
 int current_device() {
   int d = 0;
@@ -35,34 +44,89 @@ size_t size_class(size_t bytes) {
   size_t step = p2 / 8;
   return (bytes + step - 1) / step * step;
 }
+
+// The streams the calling thread is enqueueing on right now, per cache (set by the entry
+// points and by BuildScope); `known` is false outside any call.
+struct ThreadStreams {
+  hipStream_t s[2] = {nullptr, nullptr};
+  bool known[2] = {false, false};
+};
+ThreadStreams &thread_streams() {
+  static thread_local ThreadStreams t;
+  return t;
+}
+
+// Orders `to` behind everything enqueued on `from` so far.  Streams the caller has destroyed
+// since cannot be recorded on: then the whole device is waited for.
+void order_streams(hipStream_t from, hipStream_t to) {
+  if (from == to) return;
+  hipEvent_t ev = nullptr;
+  if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess && hipEventRecord(ev, from) == hipSuccess &&
+      hipStreamWaitEvent(to, ev, 0) == hipSuccess) {
+    (void)hipEventDestroy(ev);
+    return;
+  }
+  if (ev) (void)hipEventDestroy(ev);
+  (void)hipGetLastError();
+  (void)hipDeviceSynchronize();
+}
+
+void release_idle_locked() {
+  for (auto &kv : g_pool) {
+    g_block_bytes.erase(kv.second.p);
+    (void)hipFree(kv.second.p);
+  }
+  g_pool.clear();
+  g_idle_bytes = 0;
+}
 }  // namespace
 
 int &pool_scope() {
   static thread_local int scope = POOL_COMPUTE;
   return scope;
 }
+void pool_set_stream(int pool, hipStream_t s) {
+  thread_streams().s[pool] = s;
+  thread_streams().known[pool] = true;
+}
 
 void *pool_alloc(size_t bytes, int pool) {
   const size_t cls = size_class(bytes ? bytes : 1);
+  const int dev = current_device();
   {
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
-    auto it = g_pool.find(std::make_tuple(current_device(), pool, cls));
-    if (it != g_pool.end()) {
-      void *p = it->second;
+    std::unique_lock<std::mutex> lock(g_pool_mutex);
+    // the smallest idle block that fits, unless it would waste more than half of the request
+    auto it = g_pool.lower_bound(std::make_tuple(dev, pool, cls));
+    if (it != g_pool.end() && std::get<0>(it->first) == dev && std::get<1>(it->first) == pool &&
+        std::get<2>(it->first) <= cls + cls / 2) {
+      const IdleBlock b = it->second;
+      const size_t got = std::get<2>(it->first);
       g_pool.erase(it);
-      return p;
+      g_idle_bytes -= (int64_t)got;
+      g_live_bytes += (int64_t)got;
+      lock.unlock();
+      const ThreadStreams &t = thread_streams();
+      if (t.known[pool] && t.s[pool] != b.last) order_streams(b.last, t.s[pool]);
+      return b.p;
     }
   }
   void *p = nullptr;
   hipError_t e = hipMalloc(&p, cls);
   if (e != hipSuccess) {
-    // give cached blocks back to the driver and try once more
-    std::lock_guard<std::mutex> lock(g_pool_mutex);
-    for (auto &kv : g_pool) (void)hipFree(kv.second);
-    g_pool.clear();
+    // give idle blocks back to the driver and try once more
     (void)hipGetLastError();
+    (void)hipDeviceSynchronize();
+    {
+      std::lock_guard<std::mutex> lock(g_pool_mutex);
+      release_idle_locked();
+    }
     HIP_CHECK(hipMalloc(&p, cls));
   }
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  g_block_bytes[p] = cls;
+  g_live_bytes += (int64_t)cls;
+  g_mallocs++;
+  g_peak_bytes = std::max(g_peak_bytes, g_live_bytes + g_idle_bytes);
   return p;
 }
 
@@ -71,7 +135,11 @@ void pool_free(void *p, size_t bytes, int pool) {
   std::lock_guard<std::mutex> lock(g_pool_mutex);
   hipPointerAttribute_t attr;
   int dev = hipPointerGetAttributes(&attr, p) == hipSuccess ? attr.device : current_device();
-  g_pool.emplace(std::make_tuple(dev, pool, size_class(bytes ? bytes : 1)), p);
+  auto it = g_block_bytes.find(p);
+  const size_t got = it != g_block_bytes.end() ? it->second : size_class(bytes ? bytes : 1);
+  g_live_bytes -= (int64_t)got;
+  g_idle_bytes += (int64_t)got;
+  g_pool.emplace(std::make_tuple(dev, pool, got), IdleBlock{p, thread_streams().s[pool]});
 }
 }  // namespace scn
 
@@ -92,7 +160,12 @@ static Metadata &md(scn_metadata *h) {
   if (!h) throw Error("null metadata handle");
   return h->m;
 }
-static hipStream_t st(void *s) { return (hipStream_t)s; }
+// The stream argument of an entry point; whatever the call takes from or returns to the block
+// cache is accounted to it.
+static hipStream_t st(void *s) {
+  pool_set_stream(POOL_COMPUTE, (hipStream_t)s);
+  return (hipStream_t)s;
+}
 
 // ---- two streams -------------------------------------------------------------------------------
 // Rulebooks depend on coordinates only, never on features.  They are built on a stream of the
@@ -144,6 +217,7 @@ struct BuildScope {
       : m(m_), caller(st(stream)), bs(use_build_stream() ? device_build_stream() : st(stream)),
         builds0(m_.builds), pool0(pool_scope()) {
     pool_scope() = POOL_BUILD;
+    pool_set_stream(POOL_BUILD, bs);
     if (bs != caller && reads_caller_data) {
       hipEvent_t ev;
       HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
@@ -184,7 +258,132 @@ static void consume(Metadata &m, hipStream_t s) {
   m.consumer_waited = true;
 }
 
+// ---- pinned host blocks ------------------------------------------------------------------------
+// hipHostMalloc / hipHostFree cost tens of microseconds each and every new handle needs a few
+// pinned words: blocks go back to a process-wide list instead of to the driver.
+namespace scn {
+namespace {
+std::mutex g_pinned_mutex;
+std::multimap<size_t, void *> g_pinned_idle;
+}  // namespace
+void *pinned_acquire(size_t bytes) {
+  {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    auto it = g_pinned_idle.find(bytes);
+    if (it != g_pinned_idle.end()) {
+      void *p = it->second;
+      g_pinned_idle.erase(it);
+      return p;
+    }
+  }
+  void *p = nullptr;
+  HIP_CHECK(hipHostMalloc(&p, bytes, hipHostMallocDefault));
+  return p;
+}
+void pinned_release(void *p, size_t bytes) {
+  if (!p) return;
+  std::lock_guard<std::mutex> lock(g_pinned_mutex);
+  g_pinned_idle.emplace(bytes, p);
+}
+}  // namespace scn
+
+// ---- multiply-add counts of handles that are gone ---------------------------------------------
+// A handle that is destroyed or cleared may still owe the caller the multiply-add counts of
+// convolutions that did not ask for theirs (their rule counts are on the device).  Waiting for
+// them there would stall the host on the whole forward pass each time a scene's metadata dies:
+// instead the counts are copied to pinned memory behind the work already enqueued, an event
+// marks the copy, and scn_take_released_macs folds whatever has been left behind.
+namespace {
+struct ReleasedMacs {
+  hipEvent_t ev = nullptr;
+  long long *stage = nullptr;
+  size_t stage_bytes = 0;
+  struct Item {
+    size_t off;
+    int K, slots;
+    double per_rule;
+  };
+  std::vector<Item> items;
+};
+std::mutex g_released_mutex;
+std::vector<ReleasedMacs> g_released;
+double g_released_settled = 0;
+
+void release_macs(Metadata &m) {
+  double settled = m.macs_settled;
+  m.macs_settled = 0;
+  ReleasedMacs r;
+  size_t words = 0;
+  for (auto &pm : m.pending_macs) {
+    Counts &c = *pm.first;
+    if (c.ready || !c.K || !c.dev.p)
+      settled += (c.ready ? (double)c.total() : 0.0) * pm.second;
+    else
+      words += (size_t)c.K * c.slots;
+  }
+  if (words) {
+    try {
+      // the stream the convolutions ran on; the rule counts are final before anything on it runs
+      hipStream_t s = m.consumer_known ? m.consumer : nullptr;
+      if (m.last_ready) HIP_CHECK(hipStreamWaitEvent(s, m.last_ready, 0));
+      r.stage_bytes = round_up((int64_t)(words * sizeof(long long)), 1 << 16);
+      r.stage = static_cast<long long *>(pinned_acquire(r.stage_bytes));
+      size_t off = 0;
+      for (auto &pm : m.pending_macs) {
+        Counts &c = *pm.first;
+        if (c.ready || !c.K || !c.dev.p) continue;
+        const size_t w = (size_t)c.K * c.slots;
+        HIP_CHECK(hipMemcpyAsync(r.stage + off, c.dev.p, w * sizeof(long long), hipMemcpyDeviceToHost, s));
+        r.items.push_back({off, c.K, c.slots, pm.second});
+        off += w;
+      }
+      HIP_CHECK(hipEventCreateWithFlags(&r.ev, hipEventDisableTiming));
+      HIP_CHECK(hipEventRecord(r.ev, s));
+    } catch (...) {  // a lost device: the counts are not worth an error in a destructor
+      if (r.ev) (void)hipEventDestroy(r.ev);
+      r.ev = nullptr;
+      (void)hipGetLastError();
+      (void)hipDeviceSynchronize();
+      pinned_release(r.stage, r.stage_bytes);
+      r = ReleasedMacs();
+    }
+  }
+  m.pending_macs.clear();
+  std::lock_guard<std::mutex> lock(g_released_mutex);
+  g_released_settled += settled;
+  if (r.ev) g_released.push_back(std::move(r));
+}
+
+double take_released_macs() {
+  std::vector<ReleasedMacs> todo;
+  double total;
+  {
+    std::lock_guard<std::mutex> lock(g_released_mutex);
+    todo.swap(g_released);
+    total = g_released_settled;
+    g_released_settled = 0;
+  }
+  for (ReleasedMacs &r : todo) {
+    if (hipEventSynchronize(r.ev) == hipSuccess) {
+      for (const auto &it : r.items) {
+        long long rules = 0;
+        for (size_t i = 0; i < (size_t)it.K * it.slots; i++) rules += r.stage[it.off + i];
+        total += (double)rules * it.per_rule;
+      }
+    } else {
+      (void)hipGetLastError();
+    }
+    (void)hipEventDestroy(r.ev);
+    pinned_release(r.stage, r.stage_bytes);
+  }
+  return total;
+}
+}  // namespace
+
 static void retire(Metadata &m) {  // before the handle's buffers go back to the caches
+  // the blocks were last used on the streams this handle was driven from
+  if (m.consumer_known) pool_set_stream(POOL_COMPUTE, m.consumer);
+  if (m.build_stream) pool_set_stream(POOL_BUILD, m.build_stream);
   if (m.build_stream) {
     try {
       wait_for_consumers(m, m.build_stream);
@@ -244,6 +443,23 @@ template <class F> static void on_build_stream(Metadata &m, void *stream, F f) {
   consume(m, st(stream));
 }
 
+// The three input routes: a construction that fails (coordinates outside the grid, a bad sample
+// index, a full key) leaves the handle as it was before the call, ready for another attempt.
+template <class F> static void build_input(Metadata &m, void *stream, F build) {
+  try {
+    BuildScope b(m, stream, true);
+    build(b.s());
+  } catch (...) {
+    if (!m.input_size.empty()) m.levels.erase(m.input_size);
+    m.input = InputRules();
+    m.input_size.clear();
+    throw;
+  }
+  // the construction's last kernels may still be reading the caller's buffers: whatever the
+  // caller does with them next on its stream (free, reuse) is ordered behind them
+  consume(m, st(stream));
+}
+
 static Level *find_level(Metadata &m, const int64_t *spatial) {
   auto it = m.levels.find(mk(m.dim, spatial));
   return it == m.levels.end() ? nullptr : &it->second;
@@ -270,6 +486,7 @@ scn_metadata *scn_md_create(int dim) {
 }
 void scn_md_destroy(scn_metadata *h) {
   if (!h) return;
+  release_macs(h->m);
   retire(h->m);
   const int scope = pool_scope();
   delete h;
@@ -278,14 +495,14 @@ void scn_md_destroy(scn_metadata *h) {
 int scn_md_clear(scn_metadata *h) {
   return guarded([&] {
     Metadata &m = md(h);
+    release_macs(m);  // what the convolutions run so far still owe: scn_take_released_macs
     retire(m);
-    int dim = m.dim;
     m.levels.clear();
     m.subm.clear();
     m.strided.clear();
+    m.ident.clear();
     m.input = InputRules();
     m.input_size.clear();
-    m.dim = dim;
   });
 }
 
@@ -303,13 +520,7 @@ int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *c
     Metadata &m = md(h);
     if (n < 0) throw Error("negative point count");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
-    {
-      BuildScope b(m, stream, true);
-      build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, b.s());
-    }
-    // the construction's last kernels may still be reading `coords`: whatever the caller does
-    // with that buffer next on its stream (free it, reuse it) is ordered behind them
-    consume(m, st(stream));
+    build_input(m, stream, [&](hipStream_t s) { build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, s); });
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -320,11 +531,9 @@ int scn_md_input_batch(scn_metadata *h, const int64_t *spatial, const int64_t *c
     Metadata &m = md(h);
     if (n < 0) throw Error("negative point count");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
-    {
-      BuildScope b(m, stream, true);
-      build_input_layer(m, spatial, coords, n, ncols, min_batch, 5, b.s(), 0, overwrite);
-    }
-    consume(m, st(stream));  // as in scn_md_input_layer; `overwrite` was copied on the build stream too
+    build_input(m, stream, [&](hipStream_t s) {
+      build_input_layer(m, spatial, coords, n, ncols, min_batch, 5, s, 0, overwrite);  // `overwrite` is copied
+    });
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -352,11 +561,9 @@ int scn_md_bl_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t
     if (batch < 0 || length < 0) throw Error("negative batch size or length");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
     if (batch * length == 0) length = 1, batch = 0;
-    {
-      BuildScope b(m, stream, true);
-      build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, b.s(), length);
-    }
-    consume(m, st(stream));  // as in scn_md_input_layer
+    build_input(m, stream, [&](hipStream_t s) {
+      build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, s, length);
+    });
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -431,6 +638,25 @@ int scn_md_take_macs(scn_metadata *h, void *stream, double *macs) {
     Metadata &m = md(h);
     consume(m, st(stream));
     *macs = take_macs(m, st(stream));
+  });
+}
+int scn_take_released_macs(double *macs) {
+  return guarded([&] { *macs = take_released_macs(); });
+}
+int scn_release_cache(void) {
+  return guarded([&] {
+    HIP_CHECK(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    release_idle_locked();
+  });
+}
+int scn_cache_stats(int64_t *live_bytes, int64_t *idle_bytes, int64_t *peak_bytes, int64_t *device_allocations) {
+  return guarded([&] {
+    std::lock_guard<std::mutex> lock(g_pool_mutex);
+    if (live_bytes) *live_bytes = g_live_bytes;
+    if (idle_bytes) *idle_bytes = g_idle_bytes;
+    if (peak_bytes) *peak_bytes = g_peak_bytes;
+    if (device_allocations) *device_allocations = g_mallocs;
   });
 }
 int scn_rules_sizes(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,

@@ -37,10 +37,14 @@ inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 // library enqueues on two streams, the caller's (convolutions and the other feature passes)
 // and its own build stream (rulebook construction, see api.hip), so there are two caches and
 // a block never moves from one to the other: whatever a thread allocates while it builds
-// rulebooks (pool_scope() == POOL_BUILD) comes from and returns to the build cache.  Callers
-// that drive one process from several streams of their own must order those themselves.
+// rulebooks (pool_scope() == POOL_BUILD) comes from and returns to the build cache.  An idle
+// block remembers the stream of the call that returned it; a call on another stream that takes
+// it first waits for that stream (callers may drive different handles from different streams;
+// one handle is driven from one stream at a time).  A request takes the smallest idle block
+// that fits if that wastes at most half of the request.
 enum { POOL_COMPUTE = 0, POOL_BUILD = 1 };
 int &pool_scope();  // the calling thread's current cache
+void pool_set_stream(int pool, hipStream_t s);  // the stream the calling thread enqueues on for that cache
 void *pool_alloc(size_t bytes, int pool);
 void pool_free(void *p, size_t bytes, int pool);
 

@@ -128,13 +128,15 @@ __device__ inline int listed_point(const int *sorted_idx, int st, int len, int m
   return sorted_idx[st];
 }
 
+// Pinned host blocks from a process-wide list (api.hip).
+void *pinned_acquire(size_t bytes);
+void pinned_release(void *p, size_t bytes);
+
 struct Metadata {
   Metadata() = default;
   Metadata(const Metadata &) = delete;
   Metadata &operator=(const Metadata &) = delete;
-  ~Metadata() {
-    if (pinned) (void)hipHostFree(pinned);
-  }
+  ~Metadata() { pinned_release(pinned, PINNED_WORDS * sizeof(int)); }
   // Pinned host words that the constructions copy their sizes and flags into: a copy into
   // pageable memory would be staged and waited for by the runtime, one round trip per copy.
   static constexpr int PINNED_WORDS = 2048;

@@ -185,8 +185,7 @@ static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipS
 // one host round trip of a construction step.
 static const int *fetch_words(Metadata &m, const int *dev, int words, hipStream_t s) {
   if (words > Metadata::PINNED_WORDS) throw Error("internal: read-back larger than the pinned words");
-  if (!m.pinned)
-    HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&m.pinned), Metadata::PINNED_WORDS * sizeof(int), hipHostMallocDefault));
+  if (!m.pinned) m.pinned = static_cast<int *>(pinned_acquire(Metadata::PINNED_WORDS * sizeof(int)));
   HIP_CHECK(hipMemcpyAsync(m.pinned, dev, words * sizeof(int), hipMemcpyDeviceToHost, s));
   HIP_CHECK(hipStreamSynchronize(s));
   return m.pinned;

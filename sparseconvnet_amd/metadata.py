@@ -38,14 +38,23 @@ class MacCounter:
         self.base = 0.0
         self.live = weakref.WeakSet()
 
+    def _released(self):
+        """What Metadata objects that are gone still owed (the library settles those counts
+        without stalling when a Metadata dies; this waits for them)."""
+        macs = C.c_double(0)
+        _lib.check(_lib.lib().scn_take_released_macs(C.byref(macs)))
+        return macs.value
+
     def read(self):
         for md in list(self.live):
             self.base += md.takeMacs()
+        self.base += self._released()
         return self.base
 
     def reset(self, value):
         for md in list(self.live):
             md.takeMacs()
+        self._released()
         self.base = value
 
 
@@ -72,12 +81,8 @@ class Metadata:
     def __del__(self):
         h = getattr(self, "_h", None)
         if h:
-            try:
-                mac_counter.base += self.takeMacs()
-            except Exception:  # interpreter shutdown, lost device: the count is not worth an error
-                pass
             self._h = None
-            self._L.scn_md_destroy(h)
+            self._L.scn_md_destroy(h)  # does not wait for the GPU; the counts it owes are kept (MacCounter)
 
     def takeMacs(self):
         """Multiply-adds of the convolutions run on this Metadata since the last call whose

@@ -426,3 +426,72 @@ def test_error_paths_leave_the_handle_usable(make):
     # the handle still works
     y, macs = p.subm_conv(8, 3, x, np.ones((27, 1, 4, 2), np.float32))
     assert y.shape == (2, 2) and macs == 2 * 4 * 2 and (y == 4).all()
+
+
+def test_failed_input_layer_leaves_no_level_behind(make):
+    """A construction that fails is undone: the handle takes the next input layer without a
+    scn_md_clear in between."""
+    from sparseconvnet_amd._lib import ScnError
+    p = make(3)
+    with pytest.raises(ScnError, match="outside"):
+        p.input_layer(8, np.array([[1, 2, 9, 0]], np.int64), 0, 3)
+    assert p.nactive(8) == 0
+    with pytest.raises(ScnError, match="not been built"):
+        p.input_rules()
+    good = np.array([[1, 2, 3, 0], [4, 5, 6, 1], [1, 2, 3, 0]], np.int64)
+    assert p.input_layer(8, good, 0, 3) == 2
+    y, macs = p.subm_conv(8, 3, np.ones((2, 4), np.float32), np.ones((27, 1, 4, 2), np.float32))
+    assert (y == 4).all() and macs == 2 * 4 * 2
+
+
+def test_block_cache_across_streams_and_release():
+    """Handles driven from different streams hand their blocks to each other through the
+    library's cache (a block freed by one stream's handle is waited for before another stream's
+    handle writes it): results stay those of the single-stream run.  scn_release_cache gives the
+    idle blocks back; a destroyed handle's multiply-add counts are collected without a wait at
+    destruction."""
+    import ctypes as C
+    import torch
+    from sparseconvnet_amd import _lib
+    L = _lib.lib()
+    coords = [torch.as_tensor(synthetic.room_scene(seed=6100 + i, target=40000, spatial=512)).cuda() for i in range(2)]
+    g = torch.Generator(device="cuda").manual_seed(6)
+    w = torch.randn((27, 1, 32, 32), device="cuda", generator=g) * 0.05
+    xs = [torch.randn((len(c), 32), device="cuda", generator=g) for c in coords]
+    sp, fs = _lib.sizes(3, 512), _lib.sizes(3, 3)
+
+    def run(stream, i):
+        with torch.cuda.stream(stream):
+            sv = C.c_void_p(stream.cuda_stream)
+            h = L.scn_md_create(3)
+            n = C.c_int64(0)
+            _lib.check(L.scn_md_input_layer(h, sp, C.c_void_p(coords[i].data_ptr()), len(coords[i]), 4, 0, 0, sv, C.byref(n)))
+            y = torch.empty((n.value, 32), device="cuda")
+            _lib.check(L.scn_subm_conv_fwd(h, sp, fs, C.c_void_p(xs[i].data_ptr()), C.c_void_p(y.data_ptr()),
+                                           C.c_void_p(w.data_ptr()), None, 32, 32, 1, sv, None))
+            L.scn_md_destroy(h)  # its blocks go back while the convolution may still be running
+        return y
+    torch.cuda.synchronize()
+    main = torch.cuda.current_stream()
+    want = [run(main, i) for i in range(2)]
+    torch.cuda.synchronize()
+    released = C.c_double(0)
+    _lib.check(L.scn_take_released_macs(C.byref(released)))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got = []
+    for rep in range(6):
+        got.append((rep % 2, run(s1 if rep % 2 == 0 else s2, rep % 2)))
+    torch.cuda.synchronize()
+    for i, y in got:
+        assert torch.equal(y, want[i])
+    _lib.check(L.scn_take_released_macs(C.byref(released)))
+    assert released.value > 0 and released.value % (32 * 32) == 0
+    live, idle, peak, mallocs = (C.c_int64(0) for _ in range(4))
+    _lib.check(L.scn_cache_stats(C.byref(live), C.byref(idle), C.byref(peak), C.byref(mallocs)))
+    assert idle.value > 0 and peak.value >= idle.value + live.value
+    _lib.check(L.scn_release_cache())
+    _lib.check(L.scn_cache_stats(C.byref(live), C.byref(idle), None, None))
+    assert idle.value == 0
+    y = run(main, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(y, want[0])
