@@ -191,6 +191,22 @@ int scn_output_layer_fwd(scn_metadata *md, const float *in, float *out, int plan
 int scn_subm_conv_fwd(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
                       const float *in, float *out, const float *weight, const float *bias,
                       int n_in, int n_out, int groups, void *stream, double *macs);
+/* scn_subm_conv_fwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and result as scn_subm_conv_fwd with groups = 1 (the result may
+ * differ in the order of fp32 additions: small levels split their taps over fewer workgroups
+ * when the partial sums would not fit), but the call performs no hipMalloc / hipFree: the
+ * kernels' scratch (weights in MFMA operand order, work counters, partial tiles) lives in a
+ * static 16 MiB device array that every GPU the library runs on holds until the process ends.
+ * Limits: the rulebook of (spatial, filter) must exist already (scn_md_submanifold_rules, or an
+ * earlier convolution); the packed weights, filter volume x ceil(n_in/16)*16 x ceil(n_out/16)*16
+ * x 4 bytes, must fit in 8 MiB (27 taps of 256 x 256 do), else the call fails with a message.
+ * All such calls on one GPU share the array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered.  The multiply-add count is added to the
+ * handle's running total (scn_md_take_macs). */
+int scn_subm_conv_fwd_noalloc(scn_metadata *md, const int64_t *spatial, const int64_t *filter,
+                              const float *in, float *out, const float *weight, const float *bias,
+                              int n_in, int n_out, void *stream);
 /* Convolution_updateOutput (pybind.cpp:55-60, CPU/Convolution.cpp:45-79).
  * in [nActive(in_size), nIn] -> out [nActive(out_size), nOut]. */
 int scn_conv_fwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,

@@ -751,6 +751,25 @@ int scn_subm_conv_fwd(scn_metadata *h, const int64_t *spatial, const int64_t *fi
     subm_conv(h, spatial, filter, in, out, weight, bias, n_in, n_out, groups, nullptr, nullptr, stream, macs);
   });
 }
+int scn_subm_conv_fwd_noalloc(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in,
+                              float *out, const float *weight, const float *bias, int n_in, int n_out,
+                              void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    auto it = m.subm.find(mk(m.dim, spatial, filter));
+    if (it == m.subm.end())
+      throw Error("allocation-free convolution: build the rulebook first (scn_md_submanifold_rules)");
+    Table &t = it->second;
+    consume(m, st(stream));  // waits on an event that exists already; creates nothing
+    struct Fixed {  // the kernels' scratch is the static array for the length of this call
+      Metadata &m;
+      Fixed(Metadata &m_) : m(m_) { m.fixed_scratch = noalloc_scratch(); }
+      ~Fixed() { m.fixed_scratch = nullptr; }
+    } fixed(m);
+    conv_forward(m, t, in, level_rows(m, spatial), out, weight, bias, n_in, n_out, 1, nullptr, nullptr, st(stream));
+    note_macs(m, t, (double)n_in * n_out, nullptr, st(stream));
+  });
+}
 int scn_conv_fwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
                  const int64_t *stride, const float *in, float *out, const float *weight,
                  const float *bias, int n_in, int n_out, int groups, void *stream, double *macs) {

@@ -18,9 +18,68 @@
 // leaky ReLU of the layer in front / behind, applied to the gathered / stored values.
 #include "metadata.h"
 
+#include <map>
+#include <mutex>
 #include <type_traits>
 
 namespace scn {
+
+// ---- scratch of a convolution -------------------------------------------------------------------
+// The kernels below need device memory beyond their inputs and outputs: the weights in MFMA
+// operand order, the set counters of the resident-weights kernel, and partial tiles when a small
+// level's taps are split over workgroups.  Normally these are buffers of the handle, grown on
+// demand from the block cache.  The allocation-free entry point (scn_subm_conv_fwd_noalloc) may
+// not allocate: it takes them from this array instead, one copy per GPU, held until the process
+// ends and shared by every such call on that GPU (overlapping calls on one GPU race).
+constexpr size_t NOALLOC_QUEUE_BYTES = 4096;              // set counters (8 x 128 bytes used)
+constexpr size_t NOALLOC_WPACK_BYTES = (size_t)8 << 20;   // packed weights: 27 taps of 256 x 256 are 7.1 MB
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)16 << 20;
+constexpr size_t NOALLOC_PARTIAL_BYTES = NOALLOC_SCRATCH_BYTES - NOALLOC_WPACK_BYTES - NOALLOC_QUEUE_BYTES;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+// The array's address on the current device.  In host code the array's name is only a handle
+// for the runtime; the address kernels can use comes from hipGetSymbolAddress, once per device.
+unsigned char *noalloc_scratch() {
+  static std::mutex mu;
+  static std::map<int, unsigned char *> ptrs;
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = ptrs.find(dev);
+  if (it != ptrs.end()) return it->second;
+  void *p = nullptr;
+  HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  if (!p) throw Error("the scratch array has no address on this device");
+  return ptrs[dev] = static_cast<unsigned char *>(p);
+}
+
+static float *scratch_wpack(Metadata &m, size_t floats) {
+  if (m.fixed_scratch) {
+    if (floats * sizeof(float) > NOALLOC_WPACK_BYTES)
+      throw Error("allocation-free convolution: the packed weights (taps x input planes x output planes x 4 bytes, "
+                  "padded to 16 x 16 blocks) exceed the 8 MiB the static scratch holds");
+    return reinterpret_cast<float *>(m.fixed_scratch + NOALLOC_QUEUE_BYTES);
+  }
+  m.wpack.reserve(floats);
+  return m.wpack.p;
+}
+static int *scratch_queue(Metadata &m) {
+  if (m.fixed_scratch) return reinterpret_cast<int *>(m.fixed_scratch);
+  m.queue.reserve(8 * 32);
+  return m.queue.p;
+}
+// Partial tiles for n_split workgroups per tile; with the static scratch n_split shrinks until
+// they fit (1: no partial tiles at all).
+static float *scratch_partial(Metadata &m, int &n_split, int64_t split_stride_floats) {
+  if (m.fixed_scratch) {
+    const int64_t fit = (int64_t)(NOALLOC_PARTIAL_BYTES / sizeof(float)) / std::max<int64_t>(split_stride_floats, 1);
+    n_split = (int)std::max<int64_t>(1, std::min<int64_t>(n_split, fit));
+    return n_split > 1 ? reinterpret_cast<float *>(m.fixed_scratch + NOALLOC_QUEUE_BYTES + NOALLOC_WPACK_BYTES) : nullptr;
+  }
+  if (n_split <= 1) return nullptr;
+  m.partial.reserve((size_t)n_split * split_stride_floats);
+  return m.partial.p;
+}
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 // Four bf16 values in two registers: the A / B operand of v_mfma_f32_16x16x16_bf16, which
@@ -517,8 +576,8 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   const int cin16 = (int)ceil_div(n_in, 16);
   const int n_slab = (int)ceil_div(cin16, SS);
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
-  m.wpack.reserve(packed);
-  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
+  float *wpack = scratch_wpack(m, packed);
+  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE, take_jobs(m), BF16);
   LAUNCH_CHECK();
   auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE, BUF, BF16>;
@@ -533,14 +592,10 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   // Few tiles: deal the taps of every tile over several workgroups (about two per CU in all).
   int n_split = 1;
   if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
-  float *partial = nullptr;
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
-  if (n_split > 1) {
-    m.partial.reserve((size_t)n_split * split_stride);
-    partial = m.partial.p;
-  }
+  float *partial = scratch_partial(m, n_split, split_stride);
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), 256, lds_bytes, s>>>(
-      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, epi, n_in, n_out, n_slab, tiles_per_xcd,
+      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
       n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
   if (n_split > 1) {
@@ -871,8 +926,8 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   const int cin16 = (int)ceil_div(n_in, 16);
   const int n_slab = (int)ceil_div(cin16, SS);
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
-  m.wpack.reserve(packed);
-  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, n_slab,
+  float *wpack = scratch_wpack(m, packed);
+  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, n_slab,
                                                                       SS, NCB, SLAB_STRIDE, take_jobs(m), BF16);
   LAUNCH_CHECK();
   auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE, BUF, BF16>;
@@ -886,14 +941,10 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   const int tiles_per_xcd = (int)ceil_div(n_tiles, 8);
   int n_split = 1;
   if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
-  float *partial = nullptr;
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
-  if (n_split > 1) {
-    m.partial.reserve((size_t)n_split * split_stride);
-    partial = m.partial.p;
-  }
+  float *partial = scratch_partial(m, n_split, split_stride);
   kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), NT, lds_bytes, s>>>(
-      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, m.wpack.p, epi, n_in, n_out, n_slab, tiles_per_xcd,
+      t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
       n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
   if (n_split > 1) {
@@ -1242,8 +1293,8 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
   const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
   kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
-                                                   out, m.wpack.p, epi, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                   accumulate, m.queue.p, (unsigned)in_bytes, (unsigned)nbr_bytes);
+                                                   out, scratch_wpack(m, 0), epi, n_in_part, n_out, n_sets, sets_per_xcd,
+                                                   accumulate, scratch_queue(m), (unsigned)in_bytes, (unsigned)nbr_bytes);
   LAUNCH_CHECK();
   }
 }
@@ -1263,13 +1314,13 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
                                  int n_out, int accumulate, hipStream_t s) {
   constexpr int RG = 2;  // 32 rows per set: measured faster than 64 (more wavefronts in flight)
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
-  m.wpack.reserve(packed);
-  m.queue.reserve(8 * 32);
+  float *wpack = scratch_wpack(m, packed);
+  int *queue = scratch_queue(m);
   if constexpr (SS == 2 && VEC4) {
     // bf16 operands (when asked for): a whole 32-channel part, buffer gathers
     if (m.bf16 && n_in_part == 32 && resident_buffer_gathers(m, t, in, in_stride)) {
       k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(
-          w, m.wpack.p, t.K, w_in_stride_rows, n_in_part, n_out, SS, NCB, m.queue.p, take_jobs(m), true);
+          w, wpack, t.K, w_in_stride_rows, n_in_part, n_out, SS, NCB, queue, take_jobs(m), true);
       LAUNCH_CHECK();
       const size_t lds16 = (size_t)packed * 2;  // 2-byte elements
       const int per_cu16 = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds16));
@@ -1283,8 +1334,8 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
     }
   }
   // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
-  k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, w_in_stride_rows,
-                                                                           n_in_part, n_out, SS, NCB, m.queue.p,
+  k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, w_in_stride_rows,
+                                                                           n_in_part, n_out, SS, NCB, queue,
                                                                            take_jobs(m));
   LAUNCH_CHECK();
   const size_t lds_bytes = (size_t)packed * sizeof(float);
@@ -1303,10 +1354,9 @@ template <int NCB>
 static void launch_resident_c4(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                                Epi epi, int n_in, int n_out, hipStream_t s) {
   const int packed = t.K * NCB * 64;
-  m.wpack.reserve(packed);
-  m.queue.reserve(8 * 32);
-  k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, m.wpack.p, t.K, n_in, n_out, NCB,
-                                                                        m.queue.p, take_jobs(m));
+  float *wpack = scratch_wpack(m, packed);
+  k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, NCB,
+                                                                        scratch_queue(m), take_jobs(m));
   LAUNCH_CHECK();
   launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, epi, n_in, n_out, 0,
                                                     (size_t)packed * sizeof(float), 3, s);
@@ -1430,6 +1480,8 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
+  if (m.fixed_scratch && (bn || post || groups != 1))
+    throw Error("allocation-free convolution: plain convolutions with groups = 1 only");
   Epi epi;
   epi.bias = bias;
   m.jobs = CoefJobs();

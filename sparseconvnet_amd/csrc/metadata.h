@@ -156,6 +156,9 @@ struct Metadata {
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
   DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
+  // Non-null while an allocation-free convolution runs: the three buffers above are then fixed
+  // regions of a static device array (conv.hip) and nothing may be reserved.
+  unsigned char *fixed_scratch = nullptr;
   // Multiply-add counts of forward calls that did not ask for theirs (macs == NULL): settled
   // ones summed, the others as (counts, multiply-adds per rule) until take_macs() fetches them.
   double macs_settled = 0;
@@ -212,6 +215,7 @@ int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *p
                          hipStream_t s);
 
 // ops.hip / conv.hip
+unsigned char *noalloc_scratch();  // the static scratch array's address on the current device
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);
 struct BnArgs {  // eval batch norm + leaky ReLU in front of a convolution (device pointers)
   const float *mean, *var, *gamma, *beta;
