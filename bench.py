@@ -9,7 +9,8 @@ counted as the reference counts them (sum over filter taps of rules * nIn * nOut
 
 Prints ONE JSON line.  `roofline` describes the kernel that takes the largest share of the
 step; `sweep` lists every channel pair with its own roofline; `cpu_baseline` times the
-reference's CPU path (oracle/_ref, else the oracle port) on a bounded sample."""
+reference's CPU path (oracle/_ref, else the oracle port) on a bounded sample; `configs` holds
+the other benchmark configurations at their own shapes."""
 import argparse
 import ctypes as C
 import json
@@ -25,10 +26,43 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_FP32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PAIRS = [(3, 32), (32, 32), (64, 64), (128, 128), (256, 256)]
-# HBM-side bytes per launch on the default workload (1,000,000 sites, seed 3000, shuffled), from
-# rocprofv3 FETCH_SIZE / WRITE_SIZE passes scaled by a 1 GiB copy kernel (x2.000 / x1.000):
-# profiles/conv256_sweep1M_pmc.txt.  Only reported when the run is that workload.
-MEASURED_TRAFFIC = {(256, 256): 7.70e9, (128, 128): 1.62e9, (64, 64): 0.782e9, (32, 32): 0.430e9, (3, 32): 0.501e9}
+TRAFFIC_FILE = os.path.join("profiles", "conv_sweep1M_pmc.txt")
+
+
+def measured_traffic():
+    """HBM-side bytes per launch of the sweep's kernels on the default workload, read from the
+    committed counter summary (rocprofv3 FETCH_SIZE / WRITE_SIZE passes scaled by a plain copy
+    of known size; the file gives the commands).  Lines `nIn nOut kernel GB` after the line
+    `traffic_per_launch`.  Nothing is typed in here: without the file the field is null."""
+    out = {}
+    path = os.path.join(ROOT, TRAFFIC_FILE)
+    if not os.path.exists(path):
+        return out
+    seen = False
+    for line in open(path):
+        if line.startswith("traffic_per_launch"):
+            seen = True
+            continue
+        f = line.split()
+        if seen and len(f) == 4 and f[0].isdigit() and f[1].isdigit():
+            out[(int(f[0]), int(f[1]))] = (float(f[3]) * 1e9, f[2])
+    return out
+
+
+def hbm_roofline(byts, ms):
+    ach = byts / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(ach / HBM_PEAK_GBS, 4), "algorithmic_MB": round(byts / 1e6, 1)}
+
+
+def subm_rulebook_bytes(N, K, R):
+    """Submanifold rulebook build: packed keys read, table written and read back (12 bytes per
+    entry at load 0.5), one 12-byte probe per neighbour, 8 bytes per rule out."""
+    return N * 8 + 2 * N * 12 / 0.5 + K * N * 12 + 8 * R
+
+
+def strided_rulebook_bytes(N, N_out, R):
+    return N * 8 + (N + N_out) * 12 / 0.5 + 8 * R + N_out * 8
 
 
 def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
@@ -38,54 +72,68 @@ def conv_bytes(R, n_out_rows, K, cin, cout, s=4):
 
 
 def roofline_for(cin, cout, R, n, K, ms, traffic=None):
+    """traffic: (bytes, kernel name) from the committed counter summary, or None."""
     flops = 2.0 * R * cin * cout
     byts = conv_bytes(R, n, K, cin, cout)
     t_mfma = flops / (MFMA_FP32_TFLOPS * 1e12)
     t_hbm = byts / (HBM_PEAK_GBS * 1e9)
+    tr = {"traffic": traffic[0] if traffic else None}
+    if traffic:
+        tr["traffic_source"] = {"file": TRAFFIC_FILE, "kernel": traffic[1]}
     if t_mfma >= t_hbm:
         ach = flops / (ms * 1e-3) / 1e12
-        return {"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_FP32_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(ach / MFMA_FP32_TFLOPS, 4), "traffic": traffic}
+        return dict({"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_FP32_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(ach / MFMA_FP32_TFLOPS, 4)}, **tr)
     ach = byts / (ms * 1e-3) / 1e9
-    return {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic}
+    return dict({"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                 "frac": round(ach / HBM_PEAK_GBS, 4)}, **tr)
 
 
-def cpu_baseline(sample_sites, seed):
-    """Reference CPU path (compiled reference if oracle/_ref is there, else the oracle port) on
-    a smaller scene of the same generator: the same five convolutions, once each."""
+def cpu_baseline(kind, sample_sites, seed, passes=3):
+    """The CPU path on the GPU box's host cores: the same five convolutions on a room scene of
+    the same generator, one warm-up pass and the median of `passes`; the rulebook build is timed
+    by itself.  kind "reference": the reference's own CPU sources compiled behind
+    oracle/ref_harness.cpp (oracle/_ref); "port": this repository's restatement (oracle/)."""
     from oracle import cpu_path
     from sparseconvnet_amd import synthetic
-    kind = "reference" if cpu_path.available("ref") else "port"
     flavour = "ref" if kind == "reference" else "oracle"
-    if flavour == "oracle" and not cpu_path.available("oracle"):
+    if not cpu_path.available(flavour):
         return None
     coords = synthetic.room_scene(seed=seed, target=sample_sites, spatial=4096)
-    p = cpu_path.CpuPath(3, flavour)
-    p.input_layer(4096, coords, 0, 0)
-    t0 = time.time()
-    rules = p.submanifold_rules(4096, 3)
-    t_rules = time.time() - t0
+    t_rules = []
+    for _ in range(2):  # the second build is the warmed one
+        p = cpu_path.CpuPath(3, flavour)
+        p.input_layer(4096, coords, 0, 0)
+        t0 = time.time()
+        rules = p.submanifold_rules(4096, 3)
+        t_rules.append(time.time() - t0)
     R = sum(len(r) for r in rules)
     rng = np.random.default_rng(0)
-    flops = 0.0
-    secs = 0.0
+    work = []
     for cin, cout in PAIRS:
         x = rng.normal(size=(len(coords), cin)).astype(np.float32)
         w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
+        work.append((x, w))
+    secs, flops = [], 0.0
+    for rep in range(passes + 1):
         t0 = time.time()
-        _, macs = p.subm_conv(4096, 3, x, w)
-        secs += time.time() - t0
-        flops += 2.0 * macs
+        flops = 0.0
+        for x, w in work:
+            _, macs = p.subm_conv(4096, 3, x, w)
+            flops += 2.0 * macs
+        if rep:
+            secs.append(time.time() - t0)
+    sec = float(np.median(secs))
     try:
         import torch
         cores = torch.get_num_threads() if kind == "reference" else int(os.environ.get("OMP_NUM_THREADS", os.cpu_count()))
     except Exception:
         cores = os.cpu_count()
-    return {"value": round(flops / secs / 1e9, 2), "unit": "GFLOP/s", "cores": int(cores), "kind": kind,
-            "sample": "same sweep of 5 SubmanifoldConvolution 3^3 forwards, once each, on a %d-site room "
-                      "scene (%d rules); rulebook build %.2f s single-threaded, not included"
-                      % (len(coords), R, t_rules)}
+    return {"value": round(flops / sec / 1e9, 2), "unit": "GFLOP/s", "cores": int(cores), "kind": kind,
+            "rulebook_s": round(t_rules[-1], 3), "rulebook_cores": 1, "seconds_per_pass": round(sec, 3),
+            "sample": "the sweep's 5 SubmanifoldConvolution 3^3 forwards on a %d-site room scene (%d rules), "
+                      "1 warm-up pass + median of %d; rulebook build (one sample: single-threaded in the "
+                      "reference) timed by itself, second of two builds" % (len(coords), R, passes)}
 
 
 def unet_scene(sites, seed, reps=7, residual=False, batch=1):
@@ -111,12 +159,13 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
         coords = synthetic.scene_batch(seed=seed, batch=batch, target=sites, spatial=4096, duplicate_fraction=0.3)
     g = torch.Generator(device="cuda").manual_seed(1)
     feats = torch.rand((len(coords), 3), device="cuda", generator=g) * 2 - 1
-    cd = torch.as_tensor(coords).cuda()
+    host_coords = torch.as_tensor(coords)  # a CPU LongTensor: what the reference's InputLayer is handed (ioLayers.py:51-65)
+    cd = host_coords.cuda()
     inp_layer = scn.InputLayer(3, 4096, mode=4)
-    cold, warm = [], []
+    cold, warm, cold_host = [], [], []
+    scn.forward_pass_multiplyAdd_count = 0
     with torch.no_grad():
         for r in range(reps + 1):
-            scn.forward_pass_multiplyAdd_count = 0
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             x = inp_layer([cd, feats])
@@ -126,22 +175,182 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
             y = linear(model(x))
             torch.cuda.synchronize()
             t2 = time.perf_counter()
+            x = inp_layer([host_coords, feats])  # the previous scene's Metadata dies here, unsynchronised
+            y = linear(model(x))
+            torch.cuda.synchronize()
+            t3 = time.perf_counter()
             if r:  # first pass warms allocators and code objects
                 cold.append((t1 - t0) * 1e3)
                 warm.append((t2 - t1) * 1e3)
-            macs = scn.forward_pass_multiplyAdd_count / 2
+                cold_host.append((t3 - t2) * 1e3)
+    macs = scn.forward_pass_multiplyAdd_count / (3 * (reps + 1))
+    med = lambda v: round(float(np.median(v)), 3)
     if batch > 1:
-        return {"unet_batch%d_ms_per_batch" % batch: round(float(np.median(cold)), 3),
-                "unet_batch%d_warm_ms_per_batch" % batch: round(float(np.median(warm)), 3),
+        return {"unet_batch%d_ms_per_batch" % batch: med(cold), "unet_batch%d_warm_ms_per_batch" % batch: med(warm),
+                "unet_batch%d_from_host_coords_ms_per_batch" % batch: med(cold_host),
                 "unet_batch%d_active_sites" % batch: int(x.features.shape[0])}
     if residual:
-        return {"unet_residual_ms_per_scene": round(float(np.median(cold)), 3),
-                "unet_residual_warm_ms": round(float(np.median(warm)), 3),
+        return {"unet_residual_ms_per_scene": med(cold), "unet_residual_warm_ms": med(warm),
                 "unet_residual_gflop": round(2 * macs / 1e9, 2)}
-    return {"unet_ms_per_scene": round(float(np.median(cold)), 3), "unet_warm_ms": round(float(np.median(warm)), 3),
-            "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
+    return {"unet_ms_per_scene": med(cold), "unet_ms_per_scene_from_host_coords": med(cold_host),
+            "unet_warm_ms": med(warm), "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
             "unet_gflop": round(2 * macs / 1e9, 2),
-            "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1)}
+            "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1),
+            "unet_warm_frac_mfma_fp32": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e12 / MFMA_FP32_TFLOPS, 4),
+            "note": "ms_per_scene: new Metadata per scene (input layer, every rulebook, all layers), coordinates "
+                    "resident in HBM; from_host_coords: the same with the coordinates handed over as a CPU "
+                    "LongTensor (host-to-device copy inside the timed region); warm: rulebooks cached"}
+
+
+def _timed(torch, fn, reps=5):
+    fn()
+    ms = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms.append(e0.elapsed_time(e1))
+    return float(np.median(ms))
+
+
+def _host_timed(torch, fn, reps=4):
+    """fn() -> (milliseconds measured inside, object to keep alive until timing ends)."""
+    t = []
+    for _ in range(reps + 1):
+        dt, keep = fn()
+        t.append(dt)
+        del keep
+    return float(np.median(t[1:]))
+
+
+def config_rows():
+    """The other benchmark configurations at their own shapes: configuration 1 (the reference's
+    CPU-runnable single layer), configuration 2 (2-D VGG inference, batch 100) and configuration
+    4 (the strided tree at 4094^3).  Rulebook builds are timed from the host and listed apart
+    from the feature passes (HIP events on the launch stream)."""
+    import torch
+    import sparseconvnet_amd as scn
+    from sparseconvnet_amd import metadata as M
+    from sparseconvnet_amd import synthetic
+    L, stream = M._lib.lib(), C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    g = torch.Generator(device="cuda").manual_seed(4)
+    rows = {}
+
+    def sync_ms(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
+    # configuration 1: batch 2, 128^3, ~40k sites per sample, SubmanifoldConvolution 16 -> 16
+    coords = synthetic.config1()
+    cd = torch.as_tensor(coords).cuda()
+    s128, three = torch.LongTensor([128] * 3), torch.LongTensor([3] * 3)
+    x = torch.randn((len(coords), 16), device="cuda", generator=g)
+    w = torch.randn((27, 1, 16, 16), device="cuda", generator=g) * (2.0 / (16 * 27)) ** 0.5
+
+    def build1():
+        md = M.Metadata(3)
+        md.inputLayer(s128, cd, x, 0, 0)
+        return sync_ms(lambda: M._lib.check(L.scn_md_submanifold_rules(md._h, md._s(s128), md._s(three), stream))), md
+    rb_ms = _host_timed(torch, build1)
+    _, md = build1()
+    _, macs = md.submanifoldConvolution(s128, three, x, w, None)
+    R, n = macs / 256, len(coords)
+    ms = _timed(torch, lambda: md.submanifoldConvolution(s128, three, x, w, None, want_macs=False))
+    rows["config1"] = {"workload": "SubmanifoldConvolution 3^3 16->16, batch 2, 128^3, %d sites, %d rules" % (n, R),
+                       "ms": round(ms, 4), "gflops": round(2 * macs / (ms * 1e-3) / 1e9, 1),
+                       "sites_per_s": round(n / (ms * 1e-3)), "roofline": roofline_for(16, 16, R, n, 27, ms),
+                       "rulebook_ms": round(rb_ms, 4),
+                       "rulebook_roofline": hbm_roofline(subm_rulebook_bytes(n, 27, R), rb_ms)}
+    del md
+
+    # configuration 2: 2-D VGG (examples/hello-world.py:19-30), 100 samples of pen strokes in a 64x64
+    # canvas; the three MaxPooling 3/2 need an input extent of 8k + 7: spatial size 71, output 100x32x8x8
+    torch.manual_seed(2)
+    model = scn.Sequential().add(scn.SparseVggNet(2, 1, [['C', 8], ['C', 8], ['MP', 3, 2], ['C', 16], ['C', 16],
+                                                         ['MP', 3, 2], ['C', 24], ['C', 24], ['MP', 3, 2]])).add(
+        scn.SubmanifoldConvolution(2, 24, 32, 3, False)).add(scn.BatchNormReLU(32)).add(
+        scn.SparseToDense(2, 32)).cuda().eval()
+    c2 = synthetic.strokes2d(seed=2000, batch=100, canvas=64, spatial=71)
+    c2d = torch.as_tensor(c2).cuda()
+    f2 = torch.ones((len(c2), 1), device="cuda")
+    layer = scn.InputLayer(2, 71, mode=3)
+    with torch.no_grad():
+        def cold2():
+            out = []
+            ms = sync_ms(lambda: out.append(model(layer([c2d, f2]))))
+            return ms, out
+        cold_ms = _host_timed(torch, cold2, reps=6)
+        xin = layer([c2d, f2])
+        model(xin)
+        warm_ms = float(np.median([sync_ms(lambda: model(xin)) for _ in range(7)]))
+    rows["config2"] = {"workload": "2-D SparseVggNet C8,C8,MP3/2,C16,C16,MP3/2,C24,C24,MP3/2 + SubmanifoldConvolution "
+                                   "24->32 + BatchNormReLU + SparseToDense, batch 100, spatial 71 (64x64 canvas), "
+                                   "%d active sites" % len(c2),
+                       "ms_per_batch": round(cold_ms, 3), "warm_ms_per_batch": round(warm_ms, 3),
+                       "samples_per_s": round(100 / (cold_ms * 1e-3))}
+    del xin
+
+    # configuration 4 as a tree at 4094^3: h = Convolution 2^3/2 32->64; MaxPooling(3, 2)(h);
+    # BatchNormReLU(Deconvolution 2^3/2 64->32 (h))
+    coords = synthetic.room_scene(seed=4000, target=1000000, spatial=4094)
+    cd = torch.as_tensor(coords).cuda()
+    n = len(coords)
+    sz = [torch.LongTensor([v] * 3) for v in (4094, 2047, 1023)]
+    two, thr = torch.LongTensor([2] * 3), torch.LongTensor([3] * 3)
+    x = torch.randn((n, 32), device="cuda", generator=g)
+    w1 = torch.randn((8, 1, 32, 64), device="cuda", generator=g) * 0.1
+    w2 = torch.randn((8, 1, 64, 32), device="cuda", generator=g) * 0.1
+    bn = (torch.zeros(32, device="cuda"), torch.ones(32, device="cuda"), None, None, 1e-4, 0.0)
+
+    def build4():
+        md = M.Metadata(3)
+        md.inputLayer(sz[0], cd, x, 0, 0)
+        a = sync_ms(lambda: M._lib.check(L.scn_md_strided_rules(md._h, md._s(sz[0]), md._s(sz[1]), md._s(two),
+                                                                  md._s(two), stream)))
+        b = sync_ms(lambda: M._lib.check(L.scn_md_strided_rules(md._h, md._s(sz[1]), md._s(sz[2]), md._s(thr),
+                                                                  md._s(two), stream)))
+        return (a, b), md
+    t = []
+    for _ in range(5):
+        ab, md = build4()
+        t.append(ab)
+        if len(t) < 5:
+            del md
+    rb1, rb2 = (float(np.median([v[i] for v in t[1:]])) for i in range(2))
+    n1, n2 = md.getNActive(sz[1]), md.getNActive(sz[2])
+    h, _ = md.convolution(sz[0], sz[1], two, two, x, w1, None)
+    sizes = (C.c_int64 * 27)()
+    M._lib.check(L.scn_rules_sizes(md._h, 1, md._s(sz[1]), md._s(sz[2]), md._s(thr), md._s(two), stream, sizes))
+    R2 = int(sum(sizes))
+    ms_conv = _timed(torch, lambda: md.convolution(sz[0], sz[1], two, two, x, w1, None, want_macs=False))
+    ms_mp = _timed(torch, lambda: md.maxPooling(sz[1], sz[2], thr, two, h, 0))
+    ms_dc = _timed(torch, lambda: md.deconvolution(sz[1], sz[0], two, two, h, w2, None, post=bn, want_macs=False))
+
+    def tree():
+        hh, _ = md.convolution(sz[0], sz[1], two, two, x, w1, None, want_macs=False)
+        md.maxPooling(sz[1], sz[2], thr, two, hh, 0)
+        md.deconvolution(sz[1], sz[0], two, two, hh, w2, None, post=bn, want_macs=False)
+    ms_tree = _timed(torch, tree)
+    rows["config4"] = {
+        "workload": "strided tree on a %d-site room scene in 4094^3: Convolution 2^3/2 32->64 (-> %d sites), "
+                    "MaxPooling(3, 2) (-> %d sites), Deconvolution 2^3/2 64->32 + BatchNormReLU(32)" % (n, n1, n2),
+        "tree_ms": round(ms_tree, 4),
+        "rulebook_2s2_ms": round(rb1, 4),
+        "rulebook_2s2_roofline": hbm_roofline(strided_rulebook_bytes(n, n1, n), rb1),
+        "rulebook_3s2_ms": round(rb2, 4),
+        "rulebook_3s2_roofline": hbm_roofline(strided_rulebook_bytes(n1, n2, R2), rb2),
+        "convolution_ms": round(ms_conv, 4),
+        "convolution_roofline": hbm_roofline(conv_bytes(n, n1, 8, 32, 64), ms_conv),
+        "maxpooling_3s2_ms": round(ms_mp, 4),
+        "maxpooling_3s2_roofline": hbm_roofline(R2 * 64 * 4 + 8 * R2 + n2 * 64 * 4, ms_mp),
+        "deconvolution_bn_ms": round(ms_dc, 4),
+        "deconvolution_bn_roofline": hbm_roofline(conv_bytes(n, n, 8, 64, 32), ms_dc)}
+    return rows
 
 
 def other_ops(sites, seed):
@@ -200,9 +409,9 @@ def other_ops(sites, seed):
     md = M.Metadata(3)
     x3 = md.inputLayer(sz, cd, feats, 0, 4)
     n = x3.shape[0]
-    # coordinates read (4 int64 per point), level written (4 int32 + key per site), rules (2 int32 per point)
-    out.append(row("InputLayer mode 4: rules + level (%d points -> %d sites)" % (npts, n), ms,
-                   npts * 32 + n * 24 + npts * 8, points_per_s=round(npts / (ms * 1e-3))))
+    # int64 coordinates and features of every point read, the sites' features written
+    out.append(row("InputLayer mode 4: rules + level + forward, 3 planes (%d points -> %d sites)" % (npts, n), ms,
+                   npts * 4 * 8 + npts * 3 * 4 + n * 3 * 4, points_per_s=round(npts / (ms * 1e-3))))
     L, stream = md._L, C.c_void_p(torch.cuda.current_stream().cuda_stream)
     y3 = torch.empty((n, 3), device="cuda")
     ms = timed(lambda: M._lib.check(L.scn_input_layer_fwd(md._h, M._ptr(feats), M._ptr(y3), 3, stream)))
@@ -213,7 +422,7 @@ def other_ops(sites, seed):
     out.append(row("OutputLayer forward, 32 planes", ms, npts * 4 + npts * 128 + n * 128))
     mean, var = torch.zeros(64, device="cuda"), torch.ones(64, device="cuda")
     ms = timed(lambda: M.batchNormEval(x64, mean, var, None, None, 1e-4, 0.0))
-    out.append(row("BatchNormReLU eval (stand-alone pass), 64 planes", ms, 2 * n * 64 * 4))
+    out.append(row("BatchNormReLU eval (stand-alone pass), 64 planes", ms, 2 * n * 64 * 4 + 16 * 64))
 
     def strided():
         m2 = M.Metadata(3)
@@ -233,9 +442,8 @@ def other_ops(sites, seed):
     w_up = torch.randn((8, 1, 64, 32), device="cuda", generator=g) * 0.1
     yc, _ = md.convolution(sz, half, two, two, x32, w_dn, None)
     nc = yc.shape[0]
-    # input keys read, output level written, both rule tables written (8 taps)
     out.append(row("strided rulebook 2^3 / stride 2 + output level (%d -> %d sites)" % (n, nc), ms,
-                   n * 8 + nc * 24 + 8 * 4 * (n + nc) + 8 * n, sites_per_s=round(n / (ms * 1e-3))))
+                   strided_rulebook_bytes(n, nc, n), sites_per_s=round(n / (ms * 1e-3))))
     ms = timed(lambda: md.convolution(sz, half, two, two, x32, w_dn, None, want_macs=False))
     out.append(row("Convolution 2^3 / stride 2, 32 -> 64", ms, n * 32 * 4 + 8 * n + nc * 64 * 4 + 8 * 32 * 64 * 4,
                    gflops=round(2.0 * n * 32 * 64 / (ms * 1e-3) / 1e9, 1)))
@@ -289,13 +497,23 @@ def other_ops(sites, seed):
         dt, m3 = chain()
         t.append(dt)
         levels = [m3.getNActive(torch.LongTensor([4096 >> l] * 3)) for l in range(13)]
-        del m3
+        if len(t) < 4:
+            del m3
     ms = float(np.median(t[1:]))
     total = sum(levels)
-    # per level: keys read, 27-tap table written, the strided pair of tables and the next level written
+    # every level's submanifold rulebook and the strided one to the next level, by the same formulas
+    byts = 0.0
+    cnt = (C.c_int64 * 27)()
+    for l, nl in enumerate(levels):
+        if not nl:
+            continue
+        M._lib.check(L.scn_rules_sizes(m3._h, 0, m3._s([4096 >> l] * 3), m3._s(3), None, None, stream, cnt))
+        byts += subm_rulebook_bytes(nl, 27, sum(cnt))
+        if l + 1 < len(levels):
+            byts += strided_rulebook_bytes(nl, levels[l + 1], nl)
+    del m3
     out.append(row("precompute_metadata(2): 3^3 and 2^3/stride-2 rulebooks of all %d levels (%d sites in all)"
-                   % (sum(1 for v in levels if v), total), ms, total * (8 + 27 * 4 + 24 + 2 * 8 * 4),
-                   sites_per_s=round(total / (ms * 1e-3))))
+                   % (sum(1 for v in levels if v), total), ms, byts, sites_per_s=round(total / (ms * 1e-3))))
     # sparse to dense on a grid that can be dense: the same scene generator at 128^3, 16 planes
     c2 = synthetic.room_scene(seed=seed + 1, target=200000, spatial=128)
     md2 = M.Metadata(3)
@@ -316,7 +534,9 @@ def main():
     ap.add_argument("--seed", type=int, default=3000)
     ap.add_argument("--order", default="shuffled", choices=["shuffled", "scan"])
     ap.add_argument("--cpu-sites", type=int, default=1000000)
+    ap.add_argument("--cpu-port-sites", type=int, default=60000)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-configs", action="store_true")
     ap.add_argument("--pairs", default="")
     ap.add_argument("--no-unet", action="store_true")
     ap.add_argument("--no-ops", action="store_true")
@@ -400,13 +620,13 @@ def main():
     value = total_flops / (ms_per_step * 1e-3) / 1e9
 
     default_workload = args.sites == 1000000 and args.seed == 3000 and args.order == "shuffled"
+    traffic = measured_traffic() if default_workload else {}
     sweep = []
     for (cin, cout), ms in zip(pairs, per_pair_ms):
         sweep.append({"nIn": cin, "nOut": cout, "ms": round(ms, 4),
                       "gflops": round(2.0 * R * cin * cout / (ms * 1e-3) / 1e9, 1),
                       "sites_per_s": round(n / (ms * 1e-3)),
-                      "roofline": roofline_for(cin, cout, R, n, 27, ms,
-                                               MEASURED_TRAFFIC.get((cin, cout)) if default_workload else None)})
+                      "roofline": roofline_for(cin, cout, R, n, 27, ms, traffic.get((cin, cout)))})
     dom = int(np.argmax(per_pair_ms))
     roof = dict(sweep[dom]["roofline"])
     roof["kernel"] = "submanifold conv %d->%d" % pairs[dom]
@@ -422,6 +642,7 @@ def main():
                    "active_sites": n, "rules": R},
         "rulebook_ms": round(rulebook_ms, 3),
         "rulebook_sites_per_s": round(n / (rulebook_ms * 1e-3)),
+        "rulebook_roofline": hbm_roofline(subm_rulebook_bytes(n, 27, R), rulebook_ms),
         "roofline": roof, "sweep": sweep,
     }
     if not args.no_bf16:
@@ -457,6 +678,8 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
+    if not args.no_configs:
+        out["configs"] = config_rows()
     if not args.no_ops:
         out["other_ops"] = other_ops(args.unet_sites, 5000)
     if not args.no_unet:
@@ -471,7 +694,13 @@ def main():
             scn.bf16_mfma = False
             out["unet"].update({"unet_bf16_ms_per_scene": u["unet_ms_per_scene"], "unet_bf16_warm_ms": u["unet_warm_ms"]})
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_sites, args.seed)
+        # the reference's own CPU sources where oracle/_ref was built, else this repository's port;
+        # the port is listed as well (naive inner loops: a smaller scene keeps it bounded)
+        ref = cpu_baseline("reference", args.cpu_sites, args.seed)
+        port = cpu_baseline("port", args.cpu_port_sites, args.seed)
+        out["cpu_baseline"] = ref if ref is not None else port
+        if ref is not None and port is not None:
+            out["cpu_baseline_port"] = port
     print(json.dumps(out))
 
 
