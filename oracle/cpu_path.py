@@ -78,6 +78,27 @@ def _load(flavour):
         "input_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
         "output_fwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
         "s2d": (None, [C.c_void_p, _i64p, _f32p, _f32p, C.c_int]),
+        # backward pass
+        "subm_conv_bwd": (None, [C.c_void_p, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
+                                 C.c_int, C.c_int, C.c_int]),
+        "conv_bwd": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
+                            C.c_int, C.c_int, C.c_int]),
+        "deconv_bwd": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
+                              C.c_int, C.c_int, C.c_int]),
+        "nin_bwd": (None, [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]),
+        "bn_train": (None, [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p, _f32p, _f32p, _f32p,
+                            _f32p, C.c_float, C.c_float, C.c_float]),
+        "bn_bwd": (None, [_f32p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p, _f32p,
+                          _f32p, _f32p, C.c_float]),
+        "maxpool_bwd": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, _f32p, C.c_int, _f32p, _f32p,
+                               C.c_int, C.c_int]),
+        "avgpool_bwd": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p, C.c_int, C.c_int]),
+        "unpool_bwd": (None, [C.c_void_p, _i64p, _i64p, _i64p, _i64p, _f32p, C.c_int, _f32p, C.c_int, C.c_int]),
+        "input_bwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "output_bwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "bl_input_bwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "bl_output_bwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
+        "s2d_bwd": (None, [C.c_void_p, _i64p, _f32p, _f32p, C.c_int]),
     }
     fns = {}
     for name, (res, args) in sig.items():
@@ -107,7 +128,7 @@ def _f32(a):
 
 
 class CpuPath:
-    """One Metadata object of the CPU path plus the forward ops that use it."""
+    """One Metadata object of the CPU path plus the forward and backward ops that use it."""
 
     def __init__(self, dim, flavour="oracle"):
         self.f = _load(flavour)
@@ -338,6 +359,125 @@ class CpuPath:
                        np.float32)
         self.f["s2d"](self.h, _p64(s), _pf(x), _pf(out), x.shape[1])
         return out
+
+
+    # -- backward ops: each returns the gradients the reference's backward call fills ----------
+    def _conv_bwd(self, name, sizes, n_in_rows, x, d_out, w, with_bias):
+        x, d_out, w = _f32(x), _f32(d_out), _f32(w)
+        groups = w.shape[1]
+        n_in, n_out = w.shape[2] * groups, w.shape[3] * groups
+        d_in = np.zeros((n_in_rows, n_in), np.float32)
+        d_w = np.zeros_like(w)
+        d_b = np.zeros(n_out, np.float32) if with_bias else None
+        self.f[name](self.h, *[_p64(s) for s in sizes], _pf(x), _pf(d_in), _pf(d_out), _pf(w), _pf(d_w), _pf(d_b),
+                     n_in, n_out, groups)
+        return d_in, d_w, d_b
+
+    def subm_conv_bwd(self, spatial, filter_size, x, d_out, w, with_bias=False):
+        """(d_input, d_weight, d_bias or None) of subm_conv."""
+        self.submanifold_rules(spatial, filter_size)
+        sizes = (_sz(self.dim, spatial), _sz(self.dim, filter_size))
+        return self._conv_bwd("subm_conv_bwd", sizes, self.nactive(spatial), x, d_out, w, with_bias)
+
+    def conv_bwd(self, in_size, out_size, filter_size, stride, x, d_out, w, with_bias=False):
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, filter_size, stride)]
+        return self._conv_bwd("conv_bwd", sizes, self.nactive(in_size), x, d_out, w, with_bias)
+
+    def deconv_bwd(self, in_size, out_size, filter_size, stride, x, d_out, w, with_bias=False):
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, filter_size, stride)]
+        return self._conv_bwd("deconv_bwd", sizes, self.nactive(in_size), x, d_out, w, with_bias)
+
+    def nin_bwd(self, x, d_out, w, with_bias=False):
+        x, d_out, w = _f32(x), _f32(d_out), _f32(w)
+        d_in, d_w = np.zeros_like(x), np.zeros_like(w)
+        d_b = np.zeros(w.shape[1], np.float32) if with_bias else None
+        self.f["nin_bwd"](_pf(x), _pf(d_in), _pf(d_out), _pf(w), _pf(d_w), _pf(d_b), x.shape[0], w.shape[0], w.shape[1])
+        return d_in, d_w, d_b
+
+    def bn_train(self, x, running_mean, running_var, weight=None, bias=None, eps=1e-4, momentum=0.99,
+                 leakiness=1.0):
+        """Training-mode forward: (out, save_mean, save_invstd, new running_mean, new running_var)."""
+        x = _f32(x)
+        out = np.zeros_like(x)
+        C_ = x.shape[1]
+        sm, si = np.zeros(C_, np.float32), np.zeros(C_, np.float32)
+        rm, rv = _f32(running_mean).copy(), _f32(running_var).copy()
+        weight, bias = _f32(weight), _f32(bias)
+        self.f["bn_train"](_pf(x), _pf(out), x.shape[0], C_, C_, C_, _pf(sm), _pf(si), _pf(rm), _pf(rv),
+                           _pf(weight), _pf(bias), eps, momentum, leakiness)
+        return out, sm, si, rm, rv
+
+    def bn_bwd(self, x, out, d_out, save_mean, save_invstd, weight=None, leakiness=1.0, affine=True):
+        """(d_input, d_weight, d_bias) of the batch norm whose forward saved mean / invstd."""
+        x, out, d_out = _f32(x), _f32(out), _f32(d_out)
+        C_ = x.shape[1]
+        d_in = np.zeros_like(x)
+        d_w = np.zeros(C_, np.float32) if affine else None
+        d_b = np.zeros(C_, np.float32) if affine else None
+        self.f["bn_bwd"](_pf(x), _pf(d_in), _pf(out), _pf(d_out), x.shape[0], C_, C_, C_, _pf(_f32(save_mean)),
+                         _pf(_f32(save_invstd)), _pf(_f32(weight)), _pf(d_w), _pf(d_b), leakiness)
+        return d_in, d_w, d_b
+
+    def maxpool_bwd(self, in_size, out_size, size, stride, x, out, d_out, n_features_to_drop=0):
+        x, out, d_out = _f32(x), _f32(out), _f32(d_out)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, size, stride)]
+        d_in = np.zeros_like(x)
+        self.f["maxpool_bwd"](self.h, *[_p64(s) for s in sizes], _pf(x), _pf(d_in), x.shape[1], _pf(out), _pf(d_out),
+                              out.shape[1], n_features_to_drop)
+        return d_in
+
+    def avgpool_bwd(self, in_size, out_size, size, stride, in_planes, d_out, n_features_to_drop=0):
+        d_out = _f32(d_out)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, size, stride)]
+        d_in = np.zeros((self.nactive(in_size), in_planes), np.float32)
+        self.f["avgpool_bwd"](self.h, *[_p64(s) for s in sizes], _pf(d_in), in_planes, _pf(d_out), d_out.shape[1],
+                              n_features_to_drop)
+        return d_in
+
+    def unpool_bwd(self, in_size, out_size, size, stride, in_planes, d_out, n_features_to_drop=0):
+        """in_size: the coarse level the unpooling's input lives on."""
+        d_out = _f32(d_out)
+        sizes = [_sz(self.dim, v) for v in (in_size, out_size, size, stride)]
+        d_in = np.zeros((self.nactive(in_size), in_planes), np.float32)
+        self.f["unpool_bwd"](self.h, *[_p64(s) for s in sizes], _pf(d_in), in_planes, _pf(d_out), d_out.shape[1],
+                             n_features_to_drop)
+        return d_in
+
+    def input_bwd(self, d_out):
+        d_out = _f32(d_out)
+        hdr, _ = self.input_rules()
+        d_in = np.zeros((int(hdr[2]), d_out.shape[1]), np.float32)
+        self.f["input_bwd"](self.h, _pf(d_in), _pf(d_out), d_out.shape[1])
+        return d_in
+
+    def output_bwd(self, d_out):
+        d_out = _f32(d_out)
+        hdr, _ = self.input_rules()
+        d_in = np.zeros((int(hdr[3]), d_out.shape[1]), np.float32)
+        self.f["output_bwd"](self.h, _pf(d_in), _pf(d_out), d_out.shape[1])
+        return d_in
+
+    def bl_input_bwd(self, d_out):
+        d_out = _f32(d_out)
+        hdr, _ = self.bl_rules()
+        d_in = np.zeros((int(hdr[2]), int(hdr[3]), d_out.shape[1]), np.float32)
+        self.f["bl_input_bwd"](self.h, _pf(d_in), _pf(d_out), d_out.shape[1])
+        return d_in
+
+    def bl_output_bwd(self, d_out):
+        d_out = _f32(d_out)
+        hdr, _ = self.bl_rules()
+        flat = np.ascontiguousarray(d_out.reshape(-1, d_out.shape[-1]))
+        d_in = np.zeros((int(hdr[4]), d_out.shape[-1]), np.float32)
+        self.f["bl_output_bwd"](self.h, _pf(d_in), _pf(flat), d_out.shape[-1])
+        return d_in
+
+    def s2d_bwd(self, spatial, d_out):
+        d_out = _f32(d_out)
+        s = _sz(self.dim, spatial)
+        d_in = np.zeros((self.nactive(spatial), d_out.shape[1]), np.float32)
+        self.f["s2d_bwd"](self.h, _p64(s), _pf(d_in), _pf(d_out), d_out.shape[1])
+        return d_in
 
 
 def canon_rules(rules, loc_in, loc_out):

@@ -321,4 +321,135 @@ void ref_generate_rulebooks(void *h, int size) {
   DISPATCH(h, (void)D; if (size == 2) m.generateRuleBooks2s2(); else m.generateRuleBooks3s2());
 }
 
+// ---- backward pass: the reference's own functions behind the oracle's signatures --------------
+
+void ref_subm_conv_bwd(void *h, const int64_t *spatial, const int64_t *filter, const float *in, float *d_in,
+                       const float *d_out, const float *w, float *d_w, float *d_bias, int nIn, int nOut,
+                       int groups) {
+  DISPATCH(h, auto S = lt(spatial, D); auto F = lt(filter, D); Int n = m.getNActive(S);
+           int64_t K = F.prod().item<int64_t>();
+           auto I = ft(in, {n, nIn}); auto DI = torch::empty({0}, at::kFloat);
+           auto DO = ft(d_out, {n, nOut}).clone();
+           auto W = ft(w, {K, groups, nIn / groups, nOut / groups});
+           auto DW = torch::zeros({K, groups, nIn / groups, nOut / groups}, at::kFloat);
+           auto DB = d_bias ? torch::zeros({nOut}, at::kFloat) : torch::empty({0}, at::kFloat);
+           cpu_SubmanifoldConvolution_backward<float, D>(S, F, m, I, DI, DO, W, DW, DB);
+           copy_out(DI, d_in); copy_out(DW, d_w); if (d_bias) copy_out(DB, d_bias));
+}
+void ref_conv_bwd(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                  const int64_t *stride, const float *in, float *d_in, const float *d_out, const float *w,
+                  float *d_w, float *d_bias, int nIn, int nOut, int groups) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(filter, D); auto St = lt(stride, D);
+           Int n = m.getNActive(IS); Int no = m.getNActive(OS); int64_t K = F.prod().item<int64_t>();
+           auto I = ft(in, {n, nIn}); auto DI = torch::empty({0}, at::kFloat);
+           auto DO = ft(d_out, {no, nOut}).clone();
+           auto W = ft(w, {K, groups, nIn / groups, nOut / groups});
+           auto DW = torch::zeros({K, groups, nIn / groups, nOut / groups}, at::kFloat);
+           auto DB = d_bias ? torch::zeros({nOut}, at::kFloat) : torch::empty({0}, at::kFloat);
+           cpu_Convolution_backward<float, D>(IS, OS, F, St, m, I, DI, DO, W, DW, DB);
+           copy_out(DI, d_in); copy_out(DW, d_w); if (d_bias) copy_out(DB, d_bias));
+}
+void ref_deconv_bwd(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                    const int64_t *stride, const float *in, float *d_in, const float *d_out, const float *w,
+                    float *d_w, float *d_bias, int nIn, int nOut, int groups) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(filter, D); auto St = lt(stride, D);
+           Int n = m.getNActive(IS); Int no = m.getNActive(OS); int64_t K = F.prod().item<int64_t>();
+           auto I = ft(in, {n, nIn}); auto DI = torch::empty({0}, at::kFloat);
+           auto DO = ft(d_out, {no, nOut}).clone();
+           auto W = ft(w, {K, groups, nIn / groups, nOut / groups});
+           auto DW = torch::zeros({K, groups, nIn / groups, nOut / groups}, at::kFloat);
+           auto DB = d_bias ? torch::zeros({nOut}, at::kFloat) : torch::empty({0}, at::kFloat);
+           cpu_Deconvolution_backward<float, D>(IS, OS, F, St, m, I, DI, DO, W, DW, DB);
+           copy_out(DI, d_in); copy_out(DW, d_w); if (d_bias) copy_out(DB, d_bias));
+}
+void ref_nin_bwd(const float *in, float *d_in, const float *d_out, const float *w, float *d_w, float *d_bias,
+                 int nActive, int nIn, int nOut) {
+  auto I = ft(in, {nActive, nIn});
+  auto DO = ft(d_out, {nActive, nOut}).clone();
+  auto W = ft(w, {nIn, nOut});
+  auto DI = torch::empty({0}, at::kFloat);
+  auto DW = torch::zeros({nIn, nOut}, at::kFloat);
+  auto DB = d_bias ? torch::zeros({nOut}, at::kFloat) : torch::empty({0}, at::kFloat);
+  cpu_NetworkInNetwork_updateGradInput<float>(DI, DO, W);
+  cpu_NetworkInNetwork_accGradParameters<float>(I, DO, DW, DB);
+  copy_out(DI, d_in);
+  copy_out(DW, d_w);
+  if (d_bias) copy_out(DB, d_bias);
+}
+void ref_bn_train(const float *in, float *out, int nActive, int nPlanes, int inStride, int outStride,
+                  float *saveMean, float *saveInvStd, float *runningMean, float *runningVar,
+                  const float *weight, const float *bias, float eps, float momentum, float leakiness) {
+  BatchNormalization_ForwardPass<float>((float *)in, out, nPlanes, inStride, outStride, nActive, saveMean,
+                                        saveInvStd, runningMean, runningVar, (float *)weight, (float *)bias, eps,
+                                        momentum, true, leakiness);
+}
+void ref_bn_bwd(const float *in, float *d_in, const float *out, const float *d_out, int nActive, int nPlanes,
+                int inStride, int outStride, const float *saveMean, const float *saveInvStd,
+                const float *weight, float *d_weight, float *d_bias, float leakiness) {
+  std::vector<float> d((size_t)nActive * outStride);  // the reference scales d_out in place
+  std::memcpy(d.data(), d_out, d.size() * sizeof(float));
+  BatchNormalization_BackwardPass<float>((float *)in, d_in, (float *)out, d.data(), nPlanes, inStride, outStride,
+                                         nActive, (float *)saveMean, (float *)saveInvStd, nullptr, nullptr,
+                                         (float *)weight, nullptr, d_weight, d_bias, leakiness);
+}
+void ref_maxpool_bwd(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                     const int64_t *stride, const float *in, float *d_in, int inStride, const float *out,
+                     const float *d_out, int nPlanes, int nFeaturesToDrop) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(size, D); auto St = lt(stride, D);
+           Int n = m.getNActive(IS); Int no = m.getNActive(OS);
+           auto I = ft(in, {n, inStride}); auto DI = torch::empty({0}, at::kFloat);
+           auto O = ft(out, {no, nPlanes}); auto DO = ft(d_out, {no, nPlanes});
+           cpu_MaxPooling_updateGradInput<float, D>(IS, OS, F, St, m, I, DI, O, DO, nFeaturesToDrop);
+           copy_out(DI, d_in));
+}
+void ref_avgpool_bwd(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                     const int64_t *stride, float *d_in, int inStride, const float *d_out, int nPlanes,
+                     int nFeaturesToDrop) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(size, D); auto St = lt(stride, D);
+           Int n = m.getNActive(IS); Int no = m.getNActive(OS);
+           auto I = torch::zeros({n, inStride}, at::kFloat); auto DI = torch::empty({0}, at::kFloat);
+           auto DO = ft(d_out, {no, nPlanes});
+           cpu_AveragePooling_updateGradInput<float, D>(IS, OS, F, St, m, I, DI, DO, nFeaturesToDrop);
+           copy_out(DI, d_in));
+}
+void ref_unpool_bwd(void *h, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                    const int64_t *stride, float *d_in, int inStride, const float *d_out, int nPlanes,
+                    int nFeaturesToDrop) {
+  DISPATCH(h, auto IS = lt(inSz, D); auto OS = lt(outSz, D); auto F = lt(size, D); auto St = lt(stride, D);
+           Int n = m.getNActive(IS); Int no = m.getNActive(OS);
+           auto DI = torch::zeros({n, inStride}, at::kFloat);  // sparseconvnet/unPooling.py:49
+           auto DO = ft(d_out, {no, nPlanes});
+           cpu_UnPooling_updateGradInput<float, D>(IS, OS, F, St, m, DI, DO, nFeaturesToDrop);
+           copy_out(DI, d_in));
+}
+void ref_input_bwd(void *h, float *d_in, const float *d_out, int nPlanes) {
+  DISPATCH(h, auto &rules = m.inputLayerRuleBook; Int mode = rules[0][0];
+           auto DO = ft(d_out, {(int64_t)(mode == 0 ? rules[0][2] : rules[0][3]), nPlanes});
+           auto DI = torch::empty({0}, at::kFloat);
+           cpu_InputLayer_updateGradInput<float, D>(m, DI, DO); copy_out(DI, d_in));
+}
+void ref_output_bwd(void *h, float *d_in, const float *d_out, int nPlanes) {
+  DISPATCH(h, auto DO = ft(d_out, {(int64_t)m.inputLayerRuleBook[0][2], nPlanes});
+           auto DI = torch::empty({0}, at::kFloat);
+           cpu_OutputLayer_updateGradInput<float, D>(m, DI, DO); copy_out(DI, d_in));
+}
+void ref_bl_input_bwd(void *h, float *d_in, const float *d_out, int nPlanes) {
+  DISPATCH(h, auto DO = ft(d_out, {(int64_t)m.blLayerRuleBook[0][4], nPlanes});
+           auto DI = torch::empty({0}, at::kFloat);
+           cpu_BLInputLayer_updateGradInput<float, D>(m, DI, DO); copy_out(DI, d_in));
+}
+void ref_bl_output_bwd(void *h, float *d_in, const float *d_out, int nPlanes) {
+  DISPATCH(h, auto DO = ft(d_out, {(int64_t)m.blLayerRuleBook[0][2], (int64_t)m.blLayerRuleBook[0][3], nPlanes});
+           auto DI = torch::empty({0}, at::kFloat);
+           cpu_BLOutputLayer_updateGradInput<float, D>(m, DI, DO); copy_out(DI, d_in));
+}
+void ref_s2d_bwd(void *h, const int64_t *spatial, float *d_in, const float *d_out, int nPlanes) {
+  DISPATCH(h, auto S = lt(spatial, D); Int n = m.getNActive(S);
+           auto I = torch::zeros({n, nPlanes}, at::kFloat); auto DI = torch::empty({0}, at::kFloat);
+           std::vector<int64_t> shape{(int64_t)m.getBatchSize(S), nPlanes};
+           for (int i = 0; i < D; i++) shape.push_back(spatial[i]);
+           auto DO = ft(d_out, shape);
+           cpu_SparseToDense_updateGradInput<float, D>(S, m, I, DI, DO); copy_out(DI, d_in));
+}
+
 }  // extern "C"

@@ -1,4 +1,4 @@
-// CPU oracle for the sparse-convolution forward path.
+// CPU oracle for the sparse-convolution path (forward and backward).
 //
 // TEST INFRASTRUCTURE ONLY.  This file restates, on the CPU, the algorithm of
 // the reference implementation (facebookresearch/SparseConvNet, directory
@@ -960,6 +960,282 @@ void orc_generate_rulebooks(void *md, int size) {
     }
     getRuleBook(m, inS, outS, sz, str);
     for (int d = 0; d < m.dim; d++) inS[d] = outS[d];
+  }
+}
+
+// ---- backward pass -------------------------------------------------------------------------
+
+// The loop shared by CPU/Convolution.cpp:81-115 (strided), :152-185 (submanifold) and
+// CPU/Deconvolution.cpp:43-77 (columns swapped).  d_in is zero-filled (:94-95), d_bias is the
+// column sum of d_out when the input level has rows (:98-99); per offset with rules:
+// d_w[k] = in_rows^T * d_out_rows (matmul_out, :109) and d_in_rows = d_out_rows * w[k]^T
+// scatter-added (:110-111).  Offsets without rules leave d_w[k] as the caller made it; the
+// Python side hands over zeros (submanifoldConvolution.py:101), and so does this function.
+static void conv_backward_loop(const RuleBook &rules, int inCol, int outCol, const float *in, float *d_in,
+                               Int nInRows, const float *d_out, Int nOutRows, const float *w, float *d_w,
+                               float *d_bias, Int nIn, Int nOut, Int groups) {
+  Int ip = nIn / groups, op = nOut / groups;
+  std::memset(d_in, 0, sizeof(float) * (size_t)nInRows * nIn);
+  std::memset(d_w, 0, sizeof(float) * rules.size() * (size_t)groups * ip * op);
+  if (d_bias) {
+    for (Int c = 0; c < nOut; c++) d_bias[c] = 0.f;
+    if (nInRows)
+      for (Int r = 0; r < nOutRows; r++)
+        for (Int c = 0; c < nOut; c++) d_bias[c] += d_out[(size_t)r * nOut + c];
+  }
+  for (size_t k = 0; k < rules.size(); k++) {
+    const auto &r = rules[k];
+    Int nRules = (Int)(r.size() / 2);
+    if (!nRules) continue;
+    for (Int g = 0; g < groups; g++) {
+      const float *wk = w + (((size_t)k * groups + g) * ip) * op;
+      float *dwk = d_w + (((size_t)k * groups + g) * ip) * op;
+      for (Int i = 0; i < nRules; i++) {
+        const float *a = in + ((size_t)r[2 * i + inCol] * groups + g) * ip;
+        const float *d = d_out + ((size_t)r[2 * i + outCol] * groups + g) * op;
+        float *di = d_in + ((size_t)r[2 * i + inCol] * groups + g) * ip;
+        for (Int c = 0; c < ip; c++) {
+          float acc = 0.f;
+          for (Int o = 0; o < op; o++) {
+            dwk[(size_t)c * op + o] += a[c] * d[o];
+            acc += d[o] * wk[(size_t)c * op + o];
+          }
+          di[c] += acc;
+        }
+      }
+    }
+  }
+}
+// CPU/Convolution.cpp:152-185
+void orc_subm_conv_bwd(void *md, const int64_t *spatial, const int64_t *filter, const float *in, float *d_in,
+                       const float *d_out, const float *w, float *d_w, float *d_bias, int nIn, int nOut,
+                       int groups) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getSubmanifoldRuleBook(m, spatial, filter);
+  Int n = m.nActive[mkkey(m.dim, spatial)];
+  conv_backward_loop(rb, 0, 1, in, d_in, n, d_out, n, w, d_w, d_bias, nIn, nOut, groups);
+}
+// CPU/Convolution.cpp:81-115
+void orc_conv_bwd(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                  const int64_t *stride, const float *in, float *d_in, const float *d_out, const float *w,
+                  float *d_w, float *d_bias, int nIn, int nOut, int groups) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, inSz, outSz, filter, stride);
+  conv_backward_loop(rb, 0, 1, in, d_in, m.nActive[mkkey(m.dim, inSz)], d_out, m.nActive[mkkey(m.dim, outSz)], w,
+                     d_w, d_bias, nIn, nOut, groups);
+}
+// CPU/Deconvolution.cpp:43-77: the rulebook of (outSz -> inSz); input rows are column 1.
+void orc_deconv_bwd(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *filter,
+                    const int64_t *stride, const float *in, float *d_in, const float *d_out, const float *w,
+                    float *d_w, float *d_bias, int nIn, int nOut, int groups) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, outSz, inSz, filter, stride);
+  conv_backward_loop(rb, 1, 0, in, d_in, m.nActive[mkkey(m.dim, inSz)], d_out, m.nActive[mkkey(m.dim, outSz)], w,
+                     d_w, d_bias, nIn, nOut, groups);
+}
+// CPU/NetworkInNetwork.cpp:24-47: d_in = d_out * w^T; d_w = in^T * d_out; d_bias = column sums.
+void orc_nin_bwd(const float *in, float *d_in, const float *d_out, const float *w, float *d_w, float *d_bias,
+                 int nActive, int nIn, int nOut) {
+  std::memset(d_in, 0, sizeof(float) * (size_t)nActive * nIn);
+  std::memset(d_w, 0, sizeof(float) * (size_t)nIn * nOut);
+  if (d_bias)
+    for (int o = 0; o < nOut; o++) d_bias[o] = 0.f;
+  for (int r = 0; r < nActive; r++) {
+    const float *a = in + (size_t)r * nIn, *d = d_out + (size_t)r * nOut;
+    for (int o = 0; o < nOut && d_bias; o++) d_bias[o] += d[o];
+    for (int c = 0; c < nIn; c++) {
+      float acc = 0.f;
+      for (int o = 0; o < nOut; o++) {
+        d_w[(size_t)c * nOut + o] += a[c] * d[o];
+        acc += d[o] * w[(size_t)c * nOut + o];
+      }
+      d_in[(size_t)r * nIn + c] = acc;
+    }
+  }
+}
+// CPU/BatchNormalization.cpp:13-61 with train = true: batch statistics into saveMean /
+// saveInvStd (sums of x and x*x in row order, :20-31), running statistics updated with
+// `momentum` weighting the OLD value (:33-38, unbiased variance), then the affine map and the
+// leaky ReLU as in eval mode.
+void orc_bn_train(const float *in, float *out, int nActive, int nPlanes, int inStride, int outStride,
+                  float *saveMean, float *saveInvStd, float *runningMean, float *runningVar,
+                  const float *weight, const float *bias, float eps, float momentum, float leakiness) {
+  std::memset(saveMean, 0, nPlanes * sizeof(float));
+  std::memset(saveInvStd, 0, nPlanes * sizeof(float));
+  for (int row = 0; row < nActive; row++)
+    for (int p = 0; p < nPlanes; p++) {
+      float v = in[(size_t)row * inStride + p];
+      saveMean[p] += v;
+      saveInvStd[p] += v * v;
+    }
+  for (int p = 0; p < nPlanes; p++) {
+    saveMean[p] /= nActive;
+    runningMean[p] = momentum * runningMean[p] + (1 - momentum) * saveMean[p];
+    saveInvStd[p] -= saveMean[p] * saveMean[p] * nActive;
+    runningVar[p] = momentum * runningVar[p] + (1 - momentum) * saveInvStd[p] / (nActive - 1);
+    saveInvStd[p] = powf(saveInvStd[p] / nActive + eps, -0.5f);
+  }
+  for (int row = 0; row < nActive; row++)
+    for (int p = 0; p < nPlanes; p++) {
+      float wv = saveInvStd[p] * (weight ? weight[p] : 1.f);
+      float bv = -saveMean[p] * wv + (bias ? bias[p] : 0.f);
+      float v = in[(size_t)row * inStride + p] * wv + bv;
+      out[(size_t)row * outStride + p] = v * ((v > 0) ? 1.f : leakiness);
+    }
+}
+// CPU/BatchNormalization.cpp:63-107.  The reference scales d_out in place by the leaky slope
+// (:79-81); here d_out is left alone and the scaled value is recomputed.
+void orc_bn_bwd(const float *in, float *d_in, const float *out, const float *d_out, int nActive, int nPlanes,
+                int inStride, int outStride, const float *saveMean, const float *saveInvStd,
+                const float *weight, float *d_weight, float *d_bias, float leakiness) {
+  std::vector<float> gradMean(nPlanes, 0.f), dotp(nPlanes, 0.f), k(nPlanes, 0.f);
+  for (int row = 0; row < nActive; row++)
+    for (int p = 0; p < nPlanes; p++) {
+      float d = d_out[(size_t)row * outStride + p];
+      d *= (out[(size_t)row * outStride + p] > 0) ? 1.f : leakiness;
+      gradMean[p] += d;
+      dotp[p] += (in[(size_t)row * inStride + p] - saveMean[p]) * d;
+    }
+  for (int p = 0; p < nPlanes; p++) {
+    if (d_bias) d_bias[p] = gradMean[p];
+    gradMean[p] /= nActive;
+    k[p] = dotp[p] * saveInvStd[p] * saveInvStd[p] / nActive;
+  }
+  for (int row = 0; row < nActive; row++)
+    for (int p = 0; p < nPlanes; p++) {
+      float d = d_out[(size_t)row * outStride + p];
+      d *= (out[(size_t)row * outStride + p] > 0) ? 1.f : leakiness;
+      d_in[(size_t)row * inStride + p] = (d - gradMean[p] - (in[(size_t)row * inStride + p] - saveMean[p]) * k[p]) *
+                                         saveInvStd[p] * (weight ? weight[p] : 1.f);
+    }
+  if (d_weight)
+    for (int p = 0; p < nPlanes; p++) d_weight[p] = dotp[p] * saveInvStd[p];
+}
+// CPU/MaxPooling.cpp:21-35,61-87.  d_in is [rows(inSz), inStride], zero-filled.  As in the
+// reference, the comparison reads the input planes WITHOUT the nFeaturesToDrop offset the
+// forward pass applies (:77 against :55): with dropped features the gradient lands on the
+// first nPlanes planes wherever they happen to equal the output.
+void orc_maxpool_bwd(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                     const int64_t *stride, const float *in, float *d_in, int inStride, const float *out,
+                     const float *d_out, int nPlanes, int nFeaturesToDrop) {
+  (void)nFeaturesToDrop;
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, inSz, outSz, size, stride);
+  std::memset(d_in, 0, sizeof(float) * (size_t)m.nActive[mkkey(m.dim, inSz)] * inStride);
+  for (auto &r : rb)
+    for (Int s = 0; s < (Int)(r.size() / 2); s++) {
+      size_t i = (size_t)r[2 * s] * inStride, o = (size_t)r[2 * s + 1] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++)
+        if (out[o + p] == in[i + p]) d_in[i + p] += d_out[o + p];
+    }
+}
+// CPU/AveragePooling.cpp:21-35,62-86: d_in (zero-filled) [+ nFeaturesToDrop] += d_out / filterVolume.
+void orc_avgpool_bwd(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                     const int64_t *stride, float *d_in, int inStride, const float *d_out, int nPlanes,
+                     int nFeaturesToDrop) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, inSz, outSz, size, stride);
+  std::memset(d_in, 0, sizeof(float) * (size_t)m.nActive[mkkey(m.dim, inSz)] * inStride);
+  const Int filterVolume = (Int)rb.size();
+  for (auto &r : rb)
+    for (Int s = 0; s < (Int)(r.size() / 2); s++) {
+      float *i = d_in + nFeaturesToDrop + (size_t)r[2 * s] * inStride;
+      const float *o = d_out + (size_t)r[2 * s + 1] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) i[p] += o[p] / filterVolume;
+    }
+}
+// CPU/UnPooling.cpp:21-32,58-78: the rulebook of (outSz -> inSz); d_in lives on the coarse
+// level inSz and is zero-filled by the caller (sparseconvnet/unPooling.py:49); here too.
+void orc_unpool_bwd(void *md, const int64_t *inSz, const int64_t *outSz, const int64_t *size,
+                    const int64_t *stride, float *d_in, int inStride, const float *d_out, int nPlanes,
+                    int nFeaturesToDrop) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getRuleBook(m, outSz, inSz, size, stride);
+  std::memset(d_in, 0, sizeof(float) * (size_t)m.nActive[mkkey(m.dim, inSz)] * inStride);
+  for (auto &r : rb)
+    for (Int s = 0; s < (Int)(r.size() / 2); s++) {
+      float *i = d_in + nFeaturesToDrop + (size_t)r[2 * s + 1] * inStride;
+      const float *o = d_out + (size_t)r[2 * s] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) i[p] += o[p];
+    }
+}
+// CPU/IOLayers.cpp:31-47 with the layer's own `average`: the gradient of every listed point.
+static void input_backward_pass_avg(float *points, const float *rows, Int nRows, Int maxActive, int nPlanes,
+                                    const Int *R, bool average) {
+  for (Int row = 0; row < nRows; row++) {
+    const Int *r = R + (size_t)row * (1 + maxActive);
+    const float mult = (average && r[0] > 0) ? 1.f / r[0] : 1.f;
+    const float *f = rows + (size_t)row * nPlanes;
+    for (Int i = 1; i <= r[0]; ++i) {
+      float *o = points + (size_t)r[i] * nPlanes;
+      for (Int p = 0; p < nPlanes; p++) o[p] += mult * f[p];
+    }
+  }
+}
+// CPU/IOLayers.cpp:73-93.  d_in is [nInputRows, nPlanes].
+void orc_input_bwd(void *md, float *d_in, const float *d_out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.inputLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][3];
+  if (mode == 0) {
+    std::memcpy(d_in, d_out, sizeof(float) * (size_t)rules[0][2] * nPlanes);
+    return;
+  }
+  std::memset(d_in, 0, sizeof(float) * (size_t)rules[0][2] * nPlanes);
+  input_backward_pass_avg(d_in, d_out, nRows, maxActive, nPlanes, rules[1].data(), mode == 4);
+}
+// CPU/IOLayers.cpp:116-135: InputLayer_ForwardPass with average = false.  d_in is [nActive, nPlanes].
+void orc_output_bwd(void *md, float *d_in, const float *d_out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.inputLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][3];
+  if (mode == 0) {
+    std::memcpy(d_in, d_out, sizeof(float) * (size_t)rules[0][2] * nPlanes);
+    return;
+  }
+  std::memset(d_in, 0, sizeof(float) * (size_t)nRows * nPlanes);
+  input_forward_pass(d_out, d_in, nRows, maxActive, nPlanes, rules[1].data(), false);
+}
+// CPU/IOLayers.cpp:161-184.  d_in is [batchSize * length, nPlanes].
+void orc_bl_input_bwd(void *md, float *d_in, const float *d_out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.blLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][4];
+  size_t nPoints = (size_t)rules[0][2] * rules[0][3];
+  if (mode == 0) {
+    std::memcpy(d_in, d_out, sizeof(float) * nPoints * nPlanes);
+    return;
+  }
+  std::memset(d_in, 0, sizeof(float) * nPoints * nPlanes);
+  input_backward_pass_avg(d_in, d_out, nRows, maxActive, nPlanes, rules[1].data(), mode == 4);
+}
+// CPU/IOLayers.cpp:207-229.  d_in is [nActive, nPlanes].
+void orc_bl_output_bwd(void *md, float *d_in, const float *d_out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  auto &rules = m.blLayerRuleBook;
+  Int mode = rules[0][0], maxActive = rules[0][1], nRows = rules[0][4];
+  if (mode == 0) {
+    std::memcpy(d_in, d_out, sizeof(float) * (size_t)nRows * nPlanes);
+    return;
+  }
+  std::memset(d_in, 0, sizeof(float) * (size_t)nRows * nPlanes);
+  input_forward_pass(d_out, d_in, nRows, maxActive, nPlanes, rules[1].data(), false);
+}
+// CPU/SparseToDense.cpp:21-33,66-90: d_in [nActive, nPlanes] = the dense gradient at every site.
+void orc_s2d_bwd(void *md, const int64_t *spatial, float *d_in, const float *d_out, int nPlanes) {
+  Metadata &m = *(Metadata *)md;
+  RuleBook &rb = getSparseToDenseRuleBook(m, spatial);
+  int64_t vol = 1;
+  for (int i = 0; i < m.dim; i++) vol *= spatial[i];
+  std::memset(d_in, 0, sizeof(float) * (size_t)m.nActive[mkkey(m.dim, spatial)] * nPlanes);
+  const float *oF = d_out;
+  for (auto &r : rb) {
+    for (Int s = 0; s < (Int)(r.size() / 2); s++) {
+      float *i = d_in + (size_t)r[2 * s] * nPlanes;
+      const float *o = oF + r[2 * s + 1];
+      for (Int p = 0; p < nPlanes; p++) i[p] = o[(size_t)p * vol];
+    }
+    oF += (size_t)nPlanes * vol;
   }
 }
 

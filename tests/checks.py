@@ -481,3 +481,272 @@ def check_empty(make, dim=3):
     assert sum(len(r) for r in rules) == 0
     y, macs = p.subm_conv(8, 3, np.zeros((0, 3), np.float32), np.ones((27, 1, 3, 2), np.float32))
     assert y.shape == (0, 2) and macs == 0
+
+
+# ---- backward pass ------------------------------------------------------------------------------
+# Independent statement: torch.autograd through the dense equivalents (conv / conv_transpose /
+# pooling / batch_norm on a zero-filled dense tensor), in float64; for dimensions torch has no
+# dense routines for, loops over the brute-force rule set.
+
+def _t64(a, grad=False):
+    import torch
+    return torch.tensor(np.asarray(a, np.float64), dtype=torch.float64, requires_grad=grad)
+
+
+def _dense_t(loc, feats_t, spatial, batch):
+    """Differentiable bf.to_dense."""
+    import torch
+    dim = loc.shape[1] - 1
+    spatial = [int(s) for s in np.broadcast_to(np.asarray(spatial), (dim,))]
+    d = torch.zeros([batch, feats_t.shape[1]] + spatial, dtype=torch.float64)
+    return _index_put(d, loc, feats_t)
+
+
+def _index_put(d, loc, feats_t):
+    import torch
+    dim = loc.shape[1] - 1
+    d = d.movedim(1, -1).clone()  # [B, spatial..., C]
+    idx = (torch.as_tensor(loc[:, -1]),) + tuple(torch.as_tensor(loc[:, i]) for i in range(dim))
+    d = d.index_put(idx, feats_t)
+    return d.movedim(-1, 1)
+
+
+def _sample_t(dense, loc):
+    import torch
+    dim = loc.shape[1] - 1
+    idx = (torch.as_tensor(loc[:, -1]),) + tuple(torch.as_tensor(loc[:, i]) for i in range(dim))
+    return dense.movedim(1, -1)[idx]
+
+
+def _grads(loss, *leaves):
+    loss.backward()
+    return [None if v is None else v.grad.numpy() for v in leaves]
+
+
+def _triple_grads(rows, x, d_out, w, n_in_rows):
+    """d_in, d_w by loops over (k, in row, out row) rules."""
+    d_in = np.zeros((n_in_rows, w.shape[2]))
+    d_w = np.zeros(w.shape, np.float64)
+    for k, i, j in rows:
+        d_in[i] += d_out[j].astype(np.float64) @ w[k, 0].astype(np.float64).T
+        d_w[k, 0] += np.outer(x[i].astype(np.float64), d_out[j].astype(np.float64))
+    return d_in, d_w
+
+
+def check_conv_backward(make, dim, size, seed, spatial=8, n=200, batch=2, cin=5, cout=4, bias=True):
+    """SubmanifoldConvolution backward (CPU/Convolution.cpp:152-185)."""
+    import torch
+    rng, p, loc, x = _setup(make, dim, spatial, n, batch, seed, cin)
+    K = int(np.prod(np.broadcast_to(np.asarray(size), (dim,))))
+    w = (rng.normal(size=(K, 1, cin, cout)) * 0.3).astype(np.float32)
+    d_out = rng.normal(size=(len(loc), cout)).astype(np.float32)
+    d_in, d_w, d_b = p.subm_conv_bwd(spatial, size, x, d_out, w, with_bias=bias)
+    if dim in bf._CONV:
+        xt, wt = _t64(x, True), _t64(w, True)
+        bt = _t64(np.zeros(cout), True)
+        sz = [int(s) for s in np.broadcast_to(np.asarray(size), (dim,))]
+        pads = []
+        for s in reversed(sz):
+            pads += [s // 2, s - 1 - s // 2]
+        y = bf._CONV[dim](torch.nn.functional.pad(_dense_t(loc, xt, spatial, batch), pads),
+                          bf.dense_weight(wt, dim, sz), bt)
+        gx, gw, gb = _grads((_sample_t(y, loc) * _t64(d_out)).sum(), xt, wt, bt)
+    else:
+        rows = bf.rule_rows(bf.submanifold_triples(loc, dim, size), loc, loc)
+        gx, gw = _triple_grads(rows, x, d_out, w, len(loc))
+        gb = d_out.astype(np.float64).sum(0)
+    assert_close(d_in, gx, "submanifold d_input")
+    assert_close(d_w, gw, "submanifold d_weight")
+    if bias:
+        assert_close(d_b, gb, "submanifold d_bias")
+    else:
+        assert d_b is None
+    return p
+
+
+def check_strided_backward(make, dim, size, stride, seed, out_spatial=4, n=150, batch=2, cin=5, cout=4):
+    """Convolution, Deconvolution, MaxPooling, AveragePooling and UnPooling backward over one
+    strided rulebook (CPU/Convolution.cpp:81-115, CPU/Deconvolution.cpp:43-77,
+    CPU/MaxPooling.cpp:21-35,61-87, CPU/AveragePooling.cpp:21-35,62-86, CPU/UnPooling.cpp:21-32,58-78)."""
+    import torch
+    F = torch.nn.functional
+    size_a = np.broadcast_to(np.asarray(size), (dim,))
+    stride_a = np.broadcast_to(np.asarray(stride), (dim,))
+    out_sp = np.broadcast_to(np.asarray(out_spatial), (dim,))
+    in_sp = (out_sp - 1) * stride_a + size_a
+    rng = np.random.default_rng(seed)
+    pts = np.stack([rng.integers(0, s, n) for s in in_sp], 1)
+    coords = np.concatenate([pts, rng.integers(0, batch, (n, 1))], 1).astype(np.int64)
+    p = make(dim)
+    p.input_layer(in_sp, coords, 0, 4)
+    loc = p.spatial_locations(in_sp)
+    x = p.input_fwd(rng.normal(size=(n, cin)).astype(np.float32))
+    p.strided_rules(in_sp, out_sp, size, stride)
+    loc_out = p.spatial_locations(out_sp)
+    K = int(size_a.prod())
+    st = [int(s) for s in stride_a]
+    sz = [int(s) for s in size_a]
+    w = (rng.normal(size=(K, 1, cin, cout)) * 0.3).astype(np.float32)
+    d_y = rng.normal(size=(len(loc_out), cout)).astype(np.float32)
+    d_in, d_w, d_b = p.conv_bwd(in_sp, out_sp, size, stride, x, d_y, w, with_bias=True)
+    xt, wt, bt = _t64(x, True), _t64(w, True), _t64(np.zeros(cout), True)
+    y = bf._CONV[dim](_dense_t(loc, xt, in_sp, batch), bf.dense_weight(wt, dim, sz), bt, stride=st)
+    gx, gw, gb = _grads((_sample_t(y, loc_out) * _t64(d_y)).sum(), xt, wt, bt)
+    assert_close(d_in, gx, "strided d_input")
+    assert_close(d_w, gw, "strided d_weight")
+    assert_close(d_b, gb, "strided d_bias")
+    # transposed convolution: coarse rows in, fine rows out
+    yc = rng.normal(size=(len(loc_out), cout)).astype(np.float32)
+    w2 = (rng.normal(size=(K, 1, cout, cin)) * 0.3).astype(np.float32)
+    d_z = rng.normal(size=(len(loc), cin)).astype(np.float32)
+    d_in, d_w, d_b = p.deconv_bwd(out_sp, in_sp, size, stride, yc, d_z, w2, with_bias=True)
+    yt, wt, bt = _t64(yc, True), _t64(w2, True), _t64(np.zeros(cin), True)
+    wd = bf.dense_weight(wt, dim, sz).transpose(0, 1).contiguous()
+    z = bf._CONVT[dim](_dense_t(loc_out, yt, out_sp, batch), wd, bt, stride=st)
+    gy, gw, gb = _grads((_sample_t(z, loc) * _t64(d_z)).sum(), yt, wt, bt)
+    assert_close(d_in, gy, "transposed d_input")
+    assert_close(d_w, gw, "transposed d_weight")
+    assert_close(d_b, gb, "transposed d_bias")
+    # max pooling (from zero: a window of negative values passes no gradient)
+    mp = p.maxpool(in_sp, out_sp, size, stride, x)
+    d_mp = rng.normal(size=mp.shape).astype(np.float32)
+    got = p.maxpool_bwd(in_sp, out_sp, size, stride, x, mp, d_mp)
+    xt = _t64(x, True)
+    dense = bf._POOL[dim](_dense_t(loc, xt, in_sp, batch), sz, st).clamp(min=0)
+    (gx,) = _grads((_sample_t(dense, loc_out) * _t64(d_mp)).sum(), xt)
+    assert_close(got, gx, "max pooling d_input")
+    # average pooling
+    got = p.avgpool_bwd(in_sp, out_sp, size, stride, cin, d_mp)
+    xt = _t64(x, True)
+    dense = bf._AVG[dim](_dense_t(loc, xt, in_sp, batch), sz, st)
+    (gx,) = _grads((_sample_t(dense, loc_out) * _t64(d_mp)).sum(), xt)
+    assert_close(got, gx, "average pooling d_input")
+    got2 = p.avgpool_bwd(in_sp, out_sp, size, stride, cin, d_mp[:, 2:], 2)
+    assert (got2[:, :2] == 0).all()
+    assert_close(got2[:, 2:], gx[:, 2:], "average pooling d_input, nFeaturesToDrop")
+    # unpooling: the transposed convolution whose taps are identity matrices
+    d_up = rng.normal(size=(len(loc), cout)).astype(np.float32)
+    got = p.unpool_bwd(out_sp, in_sp, size, stride, cout, d_up)
+    yt = _t64(yc, True)
+    eye = _t64(np.broadcast_to(np.eye(cout), (K, 1, cout, cout)).copy())
+    up = bf._CONVT[dim](_dense_t(loc_out, yt, out_sp, batch), bf.dense_weight(eye, dim, sz).transpose(0, 1).contiguous(),
+                        stride=st)
+    (gy,) = _grads((_sample_t(up, loc) * _t64(d_up)).sum(), yt)
+    assert_close(got, gy, "unpooling d_input")
+    return p
+
+
+def check_bn_train(make, seed, n=257, C=13):
+    """Training-mode batch norm forward and backward (CPU/BatchNormalization.cpp:13-107)."""
+    import torch
+    F = torch.nn.functional
+    rng = np.random.default_rng(seed)
+    p = make(2)
+    for leak, affine in ((0.0, True), (0.333, True), (1.0, False)):
+        x = (rng.normal(size=(n, C)) * 2 + 1).astype(np.float32)
+        g = rng.uniform(0.5, 1.5, C).astype(np.float32) if affine else None
+        b = rng.normal(size=C).astype(np.float32) if affine else None
+        rm, rv = rng.normal(size=C).astype(np.float32), rng.uniform(0.5, 1.5, C).astype(np.float32)
+        out, sm, si, rm2, rv2 = p.bn_train(x, rm, rv, g, b, 1e-4, 0.9, leak)
+        xt = _t64(x, True)
+        gt = _t64(g, True) if affine else None
+        bt = _t64(b, True) if affine else None
+        trm, trv = _t64(rm), _t64(rv)
+        y = F.batch_norm(xt, trm, trv, gt, bt, True, 1 - 0.9, 1e-4)
+        y = torch.where(y > 0, y, y * leak)
+        assert_close(out, y.detach().numpy(), "batch norm (training) output")
+        assert_close(sm, x.astype(np.float64).mean(0), "saved mean")
+        assert_close(si, 1 / np.sqrt(x.astype(np.float64).var(0) + 1e-4), "saved inverse std")
+        assert_close(rm2, trm.numpy(), "running mean")
+        assert_close(rv2, trv.numpy(), "running variance")
+        d_out = rng.normal(size=(n, C)).astype(np.float32)
+        d_in, d_g, d_b = p.bn_bwd(x, out, d_out, sm, si, g, leak, affine)
+        gx, gg, gb = _grads((y * _t64(d_out)).sum(), xt, gt, bt)
+        assert_close(d_in, gx, "batch norm d_input")
+        if affine:
+            assert_close(d_g, gg, "batch norm d_weight")
+            assert_close(d_b, gb, "batch norm d_bias")
+
+
+def check_io_backward(make, dim, mode, seed, n=300, spatial=9, batch=3, planes=4):
+    """InputLayer / OutputLayer backward (CPU/IOLayers.cpp:73-93,116-135) against the rule rows."""
+    rng = np.random.default_rng(seed)
+    coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=0 if mode == 0 else n // 2)
+    if mode == 0:
+        coords = np.unique(coords, axis=0)
+    p = make(dim)
+    n_out = p.input_layer(spatial, coords, 0, mode)
+    row_of, _ = bf.first_occurrence_rows(coords)
+    d_out = rng.normal(size=(n_out, planes)).astype(np.float32)
+    got = p.input_bwd(d_out)
+    groups = {}
+    for i, r in enumerate(row_of):
+        groups.setdefault(int(r), []).append(i)
+    want = np.zeros((len(coords), planes))
+    for r, pts in groups.items():
+        if mode in (0, 3):
+            want[pts] = d_out[r]
+        elif mode == 4:
+            want[pts] = d_out[r].astype(np.float64) * np.float32(1.0 / len(pts))
+        elif mode == 1:
+            want[pts[0]] = d_out[r]
+        else:
+            want[pts[-1]] = d_out[r]
+    assert_close(got, want, "input layer d_input, mode %d" % mode)
+    d_pts = rng.normal(size=(len(coords), planes)).astype(np.float32)
+    got = p.output_bwd(d_pts)
+    want = np.zeros((n_out, planes))
+    for r, pts in groups.items():
+        listed = pts if mode in (0, 3, 4) else ([pts[0]] if mode == 1 else [pts[-1]])
+        want[r] = d_pts[listed].astype(np.float64).sum(0)
+    assert_close(got, want, "output layer d_input, mode %d" % mode)
+
+
+def check_bl_backward(make, dim, mode, seed, batch=3, length=70, spatial=9, planes=5):
+    """BLInputLayer / BLOutputLayer backward (CPU/IOLayers.cpp:161-184,207-229)."""
+    rng = np.random.default_rng(seed)
+    coords = rng.integers(0, spatial, (batch, length, dim)).astype(np.int64)
+    if mode != 0:
+        coords[rng.random((batch, length)) < 0.2] = -1
+    p = make(dim)
+    n_out = p.bl_input_layer(spatial, coords, mode)
+    hdr, rows = p.bl_rules()
+    d_out = rng.normal(size=(n_out, planes)).astype(np.float32)
+    got = p.bl_input_bwd(d_out)
+    want = np.zeros((batch * length, planes))
+    if mode == 0:
+        want[:] = d_out
+    else:
+        for r in range(n_out):
+            cnt = rows[r, 0]
+            for i in rows[r, 1:1 + cnt]:
+                want[i] += d_out[r].astype(np.float64) * (np.float32(1.0 / cnt) if mode == 4 else 1.0)
+    assert_close(got.reshape(-1, planes), want, "batch-by-length input d_input, mode %d" % mode)
+    d_pts = rng.normal(size=(batch, length, planes)).astype(np.float32)
+    got = p.bl_output_bwd(d_pts)
+    flat = d_pts.reshape(-1, planes)
+    want = np.zeros((n_out, planes))
+    if mode == 0:
+        want[:] = flat
+    else:
+        for r in range(n_out):
+            want[r] = flat[rows[r, 1:1 + rows[r, 0]]].astype(np.float64).sum(0)
+    assert_close(got, want, "batch-by-length output d_input, mode %d" % mode)
+
+
+def check_misc_backward(make, seed):
+    """SparseToDense and NetworkInNetwork backward (CPU/SparseToDense.cpp:21-33,66-90,
+    CPU/NetworkInNetwork.cpp:24-47)."""
+    rng, p, loc, x = _setup(make, 2, 6, 60, 3, seed, 4)
+    d_dense = rng.normal(size=(3, 4, 6, 6)).astype(np.float32)
+    got = p.s2d_bwd(6, d_dense)
+    assert_close(got, bf.sample_dense(_t64(d_dense), loc), "sparse to dense d_input")
+    for rows, cin, cout in ((257, 13, 7), (64, 32, 32), (300, 64, 96)):
+        a = rng.normal(size=(rows, cin)).astype(np.float32)
+        w = (rng.normal(size=(cin, cout)) * 0.3).astype(np.float32)
+        d = rng.normal(size=(rows, cout)).astype(np.float32)
+        d_in, d_w, d_b = p.nin_bwd(a, d, w, with_bias=True)
+        a64, w64, d64 = a.astype(np.float64), w.astype(np.float64), d.astype(np.float64)
+        assert_close(d_in, d64 @ w64.T, "network in network d_input")
+        assert_close(d_w, a64.T @ d64, "network in network d_weight")
+        assert_close(d_b, d64.sum(0), "network in network d_bias")

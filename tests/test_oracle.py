@@ -101,3 +101,29 @@ def test_special_values(make):
 
 def test_empty(make):
     checks.check_empty(make)
+
+
+# ---- backward pass: the same independent checks on the oracle and on the compiled reference ----
+
+@pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (3, 2), (2, (3, 1)), (4, 3)])
+def test_conv_backward(make, dim, size):
+    checks.check_conv_backward(make, dim, size, seed=30 + dim, spatial=8 if dim < 4 else 5, bias=(dim != 2))
+
+
+@pytest.mark.parametrize("dim,size,stride", [(3, 2, 2), (3, 3, 2), (2, 3, 2), (2, 2, 2), (1, 3, 2), (2, (3, 2), (2, 1))])
+def test_strided_backward(make, dim, size, stride):
+    checks.check_strided_backward(make, dim, size, stride, seed=40 + dim)
+
+
+def test_bn_train(make):
+    checks.check_bn_train(make, seed=50)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+def test_io_backward(make, mode):
+    checks.check_io_backward(make, 3, mode, seed=60 + mode)
+    checks.check_bl_backward(make, 2, mode, seed=65 + mode)
+
+
+def test_misc_backward(make):
+    checks.check_misc_backward(make, seed=70)
