@@ -1,5 +1,5 @@
-/* C ABI of libscn_hip.so: the MI355X (gfx950) forward path of submanifold
- * sparse convolutional networks.
+/* C ABI of libscn_hip.so: the MI355X (gfx950) path of submanifold sparse
+ * convolutional networks (forward pass, and the backward pass of the same ops).
  *
  * The library replaces what the reference binds through its pybind11 module
  * `sparseconvnet.SCN` for the forward pass (reference paths are relative to
@@ -279,6 +279,74 @@ int scn_bn_eval_fwd(const float *in, float *out, int64_t rows, int planes, int64
  * in [nActive, planes] -> out [batch, planes, spatial...], zero-filled first. */
 int scn_s2d_fwd(scn_metadata *md, const int64_t *spatial, const float *in, float *out,
                 int planes, void *stream);
+
+/* ---- backward pass ----------------------------------------------------------------------------
+ * Gradients are device fp32 arrays allocated by the caller and written in full (the reference's
+ * Python side hands zero-filled tensors to calls that accumulate into them); d_bias may be NULL.
+ * d_out is never modified. */
+
+/* SubmanifoldConvolution_backward (pybind.cpp:140-146, CPU/Convolution.cpp:152-185):
+ * d_in [nActive, nIn], d_weight as weight, d_bias [nOut] = column sums of d_out. */
+int scn_subm_conv_bwd(scn_metadata *md, const int64_t *spatial, const int64_t *filter, const float *in,
+                      float *d_in, const float *d_out, const float *weight, float *d_weight,
+                      float *d_bias, int n_in, int n_out, int groups, void *stream);
+/* Convolution_backward (pybind.cpp:61-66, CPU/Convolution.cpp:81-115). */
+int scn_conv_bwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                 const int64_t *filter, const int64_t *stride, const float *in, float *d_in,
+                 const float *d_out, const float *weight, float *d_weight, float *d_bias, int n_in,
+                 int n_out, int groups, void *stream);
+/* Deconvolution_backward (pybind.cpp:85-90, CPU/Deconvolution.cpp:43-77). */
+int scn_deconv_bwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                   const int64_t *filter, const int64_t *stride, const float *in, float *d_in,
+                   const float *d_out, const float *weight, float *d_weight, float *d_bias, int n_in,
+                   int n_out, int groups, void *stream);
+/* NetworkInNetwork_updateGradInput + NetworkInNetwork_accGradParameters (pybind.cpp:226-229,
+ * CPU/NetworkInNetwork.cpp:24-47); the handle as for scn_nin_fwd. */
+int scn_nin_bwd(scn_metadata *md, const float *in, float *d_in, const float *d_out, const float *weight,
+                float *d_weight, float *d_bias, int64_t rows, int n_in, int n_out, void *stream);
+/* BatchNormalization_updateOutput with train=true (pybind.cpp:220, CPU/BatchNormalization.cpp:13-61):
+ * batch mean and 1/sqrt(biased variance + eps) into save_mean / save_invstd [planes]; running_mean /
+ * running_var updated in place as momentum * old + (1 - momentum) * batch value (unbiased
+ * variance); out = leaky(x * w + b) with the batch statistics.  The reference call takes no
+ * metadata; here the handle owns the scratch of the column reductions (any handle will do; the
+ * caller has the tensor's at hand). */
+int scn_bn_train_fwd(scn_metadata *md, const float *in, float *out, int64_t rows, int planes,
+                     int64_t in_stride, int64_t out_stride, float *save_mean, float *save_invstd,
+                     float *running_mean, float *running_var, const float *gamma, const float *beta,
+                     float eps, float momentum, float leakiness, void *stream);
+/* BatchNormalization_backward (pybind.cpp:222, CPU/BatchNormalization.cpp:63-107,132-158), from
+ * the statistics the forward pass saved.  d_gamma / d_beta may be NULL. */
+int scn_bn_bwd(scn_metadata *md, const float *in, float *d_in, const float *out, const float *d_out,
+               int64_t rows, int planes, int64_t in_stride, int64_t out_stride, const float *save_mean,
+               const float *save_invstd, const float *gamma, float *d_gamma, float *d_beta,
+               float leakiness, void *stream);
+/* MaxPooling_updateGradInput (pybind.cpp:108-113, CPU/MaxPooling.cpp:21-35,61-87): d_in
+ * [nActive(in_size), in_stride]; every input that equals its window's output receives that
+ * window's gradient.  As in the reference, the comparison reads input planes [0, planes), without
+ * the n_features_to_drop offset of the forward pass. */
+int scn_maxpool_bwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                    const int64_t *size, const int64_t *stride, const float *in, float *d_in,
+                    int in_stride, const float *out, const float *d_out, int planes,
+                    int n_features_to_drop, void *stream);
+/* AveragePooling_updateGradInput (pybind.cpp:49-54, CPU/AveragePooling.cpp:21-35,62-86). */
+int scn_avgpool_bwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                    const int64_t *size, const int64_t *stride, float *d_in, int in_stride,
+                    const float *d_out, int planes, int n_features_to_drop, void *stream);
+/* UnPooling_updateGradInput (pybind.cpp:194-198, CPU/UnPooling.cpp:21-32,58-78): in_size is the
+ * coarse level the unpooling's input lives on; d_in [nActive(in_size), in_stride]. */
+int scn_unpool_bwd(scn_metadata *md, const int64_t *in_size, const int64_t *out_size,
+                   const int64_t *size, const int64_t *stride, float *d_in, int in_stride,
+                   const float *d_out, int planes, int n_features_to_drop, void *stream);
+/* InputLayer_updateGradInput / BLInputLayer_updateGradInput (pybind.cpp:160-163,177-180,
+ * CPU/IOLayers.cpp:73-93,161-184): d_out [nActive, planes] -> d_in [nInputRows, planes]. */
+int scn_input_layer_bwd(scn_metadata *md, float *d_in, const float *d_out, int planes, void *stream);
+/* OutputLayer_updateGradInput / BLOutputLayer_updateGradInput (pybind.cpp:168-171,185-188,
+ * CPU/IOLayers.cpp:116-135,207-229): d_out [nInputRows, planes] -> d_in [nActive, planes]. */
+int scn_output_layer_bwd(scn_metadata *md, float *d_in, const float *d_out, int planes, void *stream);
+/* SparseToDense_updateGradInput (pybind.cpp:130-134, CPU/SparseToDense.cpp:21-33,66-90):
+ * d_out [batch, planes, spatial...] -> d_in [nActive, planes]. */
+int scn_s2d_bwd(scn_metadata *md, const int64_t *spatial, float *d_in, const float *d_out, int planes,
+                void *stream);
 
 #ifdef __cplusplus
 }

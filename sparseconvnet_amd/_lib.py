@@ -68,6 +68,23 @@ SIGNATURES = {
     "scn_bn_eval_fwd": (C.c_int, [_vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp,
                                   C.c_float, C.c_float, _vp]),
     "scn_s2d_fwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, _vp]),
+    # backward pass
+    "scn_subm_conv_bwd": (C.c_int, [_vp, _i64p, _i64p, _vp, _vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, _vp]),
+    "scn_conv_bwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
+                               C.c_int, _vp]),
+    "scn_deconv_bwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int,
+                                 C.c_int, _vp]),
+    "scn_nin_bwd": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, C.c_int, _vp]),
+    "scn_bn_train_fwd": (C.c_int, [_vp, _vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp, _vp,
+                                   _vp, C.c_float, C.c_float, C.c_float, _vp]),
+    "scn_bn_bwd": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, _vp, _vp, _vp, _vp,
+                             _vp, C.c_float, _vp]),
+    "scn_maxpool_bwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, C.c_int, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "scn_avgpool_bwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int, _vp]),
+    "scn_unpool_bwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, C.c_int, _vp, C.c_int, C.c_int, _vp]),
+    "scn_input_layer_bwd": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp]),
+    "scn_output_layer_bwd": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp]),
+    "scn_s2d_bwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, _vp]),
 }
 
 _lib = None

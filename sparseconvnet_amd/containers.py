@@ -64,8 +64,9 @@ class Sequential(torch.nn.Sequential):
 
 
 class CheckpointedSequential(Sequential):
-    """sequential.py:66-73 trades memory for recomputation in the backward pass; there is no
-    backward pass here, so this is Sequential under the reference's other name."""
+    """sequential.py:66-73 trades memory for recomputation in the backward pass
+    (torch.utils.checkpoint over the module chain); here it runs as Sequential, keeping its
+    activations: the reference's other name for the same function."""
 
 
 class _Table(torch.nn.Sequential):

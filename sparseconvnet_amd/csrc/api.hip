@@ -875,4 +875,119 @@ int scn_s2d_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float 
   });
 }
 
+// ---- backward pass -----------------------------------------------------------------------------
+
+int scn_subm_conv_bwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in, float *d_in,
+                      const float *d_out, const float *weight, float *d_weight, float *d_bias, int n_in,
+                      int n_out, int groups, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    Table &t = subm_table(m, spatial, filter, stream);
+    subm_conv_backward(m, t, filter, in, d_in, d_out, weight, d_weight, d_bias, n_in, n_out, groups, st(stream));
+  });
+}
+int scn_conv_bwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                 const int64_t *stride, const float *in, float *d_in, const float *d_out, const float *weight,
+                 float *d_weight, float *d_bias, int n_in, int n_out, int groups, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    StridedRules &r = strided_table_fine(m, in_size, out_size, filter, stride, stream);
+    strided_conv_backward(m, r.by_out, r.by_in, level_rows(m, in_size), level_rows(m, out_size), in, d_in, d_out,
+                          weight, d_weight, d_bias, n_in, n_out, groups, st(stream));
+  });
+}
+int scn_deconv_bwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *filter,
+                   const int64_t *stride, const float *in, float *d_in, const float *d_out, const float *weight,
+                   float *d_weight, float *d_bias, int n_in, int n_out, int groups, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    // CPU/Deconvolution.cpp:56-57: the rulebook of (out_size -> in_size)
+    StridedRules &r = strided_table_fine(m, out_size, in_size, filter, stride, stream);
+    strided_conv_backward(m, r.by_in, r.by_out, level_rows(m, in_size), level_rows(m, out_size), in, d_in, d_out,
+                          weight, d_weight, d_bias, n_in, n_out, groups, st(stream));
+  });
+}
+int scn_nin_bwd(scn_metadata *h, const float *in, float *d_in, const float *d_out, const float *weight,
+                float *d_weight, float *d_bias, int64_t rows, int n_in, int n_out, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (rows < 0 || rows >= ((int64_t)1 << 31)) throw Error("network in network: row count out of range");
+    Table *tp;
+    {
+      BuildScope b(m, stream);
+      tp = &identity_table(m, rows, b.s());
+    }
+    consume(m, st(stream));
+    nin_backward(m, *tp, in, d_in, d_out, weight, d_weight, d_bias, n_in, n_out, st(stream));
+  });
+}
+int scn_bn_train_fwd(scn_metadata *h, const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                     int64_t out_stride, float *save_mean, float *save_invstd, float *running_mean,
+                     float *running_var, const float *gamma, const float *beta, float eps, float momentum,
+                     float leakiness, void *stream) {
+  return guarded([&] {
+    bn_train_forward(&md(h), in, out, rows, planes, in_stride, out_stride, save_mean, save_invstd, running_mean,
+                     running_var, gamma, beta, eps, momentum, leakiness, st(stream));
+  });
+}
+int scn_bn_bwd(scn_metadata *h, const float *in, float *d_in, const float *out, const float *d_out, int64_t rows,
+               int planes, int64_t in_stride, int64_t out_stride, const float *save_mean, const float *save_invstd,
+               const float *gamma, float *d_gamma, float *d_beta, float leakiness, void *stream) {
+  return guarded([&] {
+    bn_backward(&md(h), in, d_in, out, d_out, rows, planes, in_stride, out_stride, save_mean, save_invstd, gamma,
+                d_gamma, d_beta, leakiness, st(stream));
+  });
+}
+int scn_maxpool_bwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
+                    const int64_t *stride, const float *in, float *d_in, int in_stride, const float *out,
+                    const float *d_out, int planes, int n_features_to_drop, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
+    StridedRules &r = strided_table_fine(m, in_size, out_size, size, stride, stream);
+    pool_backward(0, r.by_in, in, d_in, in_stride, out, d_out, planes, n_features_to_drop, st(stream));
+  });
+}
+int scn_avgpool_bwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
+                    const int64_t *stride, float *d_in, int in_stride, const float *d_out, int planes,
+                    int n_features_to_drop, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
+    StridedRules &r = strided_table_fine(m, in_size, out_size, size, stride, stream);
+    pool_backward(1, r.by_in, nullptr, d_in, in_stride, nullptr, d_out, planes, n_features_to_drop, st(stream));
+  });
+}
+int scn_unpool_bwd(scn_metadata *h, const int64_t *in_size, const int64_t *out_size, const int64_t *size,
+                   const int64_t *stride, float *d_in, int in_stride, const float *d_out, int planes,
+                   int n_features_to_drop, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (planes != in_stride - n_features_to_drop) throw Error("planes must equal in_stride - n_features_to_drop");
+    // CPU/UnPooling.cpp:68-69: the rulebook of (out_size -> in_size); the gradient is gathered from the coarse side
+    StridedRules &r = strided_table(m, out_size, in_size, size, stride, stream);
+    pool_backward(2, r.by_out, nullptr, d_in, in_stride, nullptr, d_out, planes, n_features_to_drop, st(stream));
+  });
+}
+int scn_input_layer_bwd(scn_metadata *h, float *d_in, const float *d_out, int planes, void *stream) {
+  return guarded([&] {
+    consume(md(h), st(stream));
+    input_backward(md(h).input, d_in, d_out, planes, st(stream));
+  });
+}
+int scn_output_layer_bwd(scn_metadata *h, float *d_in, const float *d_out, int planes, void *stream) {
+  return guarded([&] {
+    consume(md(h), st(stream));
+    output_backward(md(h).input, d_in, d_out, planes, st(stream));
+  });
+}
+int scn_s2d_bwd(scn_metadata *h, const int64_t *spatial, float *d_in, const float *d_out, int planes, void *stream) {
+  return guarded([&] {
+    Level *l = find_level(md(h), spatial);
+    if (!l) throw Error("sparse to dense: unknown spatial size");
+    consume(md(h), st(stream));
+    s2d_backward(*l, d_in, d_out, planes, st(stream));
+  });
+}
+
 }  // extern "C"

@@ -1,0 +1,591 @@
+// Backward pass: gradients of the convolutions (with respect to input rows, weights and bias),
+// of NetworkInNetwork, of batch normalisation in training mode (plus its training-mode forward),
+// of the pooling layers, the input / output layers and sparse-to-dense.
+//
+// The reference computes these on the host per filter offset: gather rows, two GEMMs, scatter-add
+// (CPU/Convolution.cpp:81-115,152-185, CPU/Deconvolution.cpp:43-77).  Here:
+//   * the gradient of the input rows is itself an output-stationary convolution over a neighbour
+//     table, with every tap's weight slice transposed: for a strided rulebook the table indexed
+//     from the other side (the two tables of StridedRules list the same rules), for a
+//     submanifold rulebook the same table with the taps mirrored (rule (k, i -> j) is rule
+//     (K-1-k, j -> i)), so it runs through the forward kernels of conv.hip: no atomics,
+//     deterministic;
+//   * the gradient of the weights is, per tap, a [nIn x positions] x [positions x nOut] product
+//     over the positions that have the tap: MFMA tiles over chunks of positions, partial sums per
+//     chunk, then a reduction in fixed order (no float atomics, deterministic);
+//   * column sums (bias gradients, batch-norm statistics) are two-stage reductions in fixed order.
+#include "metadata.h"
+
+namespace scn {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+static const int TB = 256;
+static inline dim3 grid_for(int64_t n, int tb = TB) { return dim3((unsigned)std::max<int64_t>(1, ceil_div(n, tb))); }
+
+// ---- transposed weights ------------------------------------------------------------------------
+// wt[k'][g][o][c] = w[k][g][c][o], k' = K-1-k with mirror, else k.
+__global__ void k_transpose_weights(const float *w, float *wt, int K, int groups, int ip, int op, int mirror) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t per = (int64_t)groups * ip * op;
+  if (i >= K * per) return;
+  const int k = (int)(i / per);
+  int64_t r = i - k * per;
+  const int g = (int)(r / ((int64_t)ip * op));
+  r -= (int64_t)g * ip * op;
+  const int o = (int)(r / ip), c = (int)(r - (int64_t)o * ip);
+  const int ks = mirror ? K - 1 - k : k;
+  wt[i] = w[(((int64_t)ks * groups + g) * ip + c) * op + o];
+}
+
+// ---- column sums -------------------------------------------------------------------------------
+// partial[b][q][c] for row block b: q = 0: sum of a(row, c), q = 1: sum of b(row, c), where
+//   MODE 0  a = x                                   (bias gradient; one quantity)
+//   MODE 1  a = x, b = x * x                        (batch-norm statistics)
+//   MODE 2  a = d * r, b = (x - mean[c]) * d * r    with r = out > 0 ? 1 : leak  (batch-norm backward)
+// A workgroup of 256 threads covers CW columns by 256 / CW rows at a time.
+template <int MODE>
+__global__ void k_colsum(const float *x, int64_t x_stride, const float *d, const float *out, int64_t o_stride,
+                         const float *mean, float leak, int64_t rows, int planes, int CW, int64_t rows_per_block,
+                         float *partial) {
+  __shared__ float red[2][256];
+  const int tx = threadIdx.x % CW, ty = threadIdx.x / CW, RW = 256 / CW;
+  const int c = blockIdx.y * CW + tx;
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_block, r1 = min(rows, r0 + rows_per_block);
+  float a = 0.f, b = 0.f;
+  if (c < planes) {
+    const float mu = MODE == 2 ? mean[c] : 0.f;
+    for (int64_t r = r0 + ty; r < r1; r += RW) {
+      if (MODE == 0) {
+        a += x[r * x_stride + c];
+      } else if (MODE == 1) {
+        const float v = x[r * x_stride + c];
+        a += v;
+        b += v * v;
+      } else {
+        float g = d[r * o_stride + c];
+        g *= out[r * o_stride + c] > 0.f ? 1.f : leak;
+        a += g;
+        b += (x[r * x_stride + c] - mu) * g;
+      }
+    }
+  }
+  red[0][threadIdx.x] = a;
+  red[1][threadIdx.x] = b;
+  __syncthreads();
+  if (ty == 0 && c < planes) {
+    for (int q = 1; q < RW; q++) {
+      a += red[0][q * CW + tx];
+      b += red[1][q * CW + tx];
+    }
+    float *p = partial + (size_t)blockIdx.x * 2 * planes;
+    p[c] = a;
+    p[planes + c] = b;
+  }
+}
+struct ColsumPlan {
+  int CW, blocks;
+  int64_t rows_per_block;
+};
+static ColsumPlan colsum_plan(int64_t rows, int planes) {
+  ColsumPlan p;
+  p.CW = planes <= 16 ? 16 : planes <= 32 ? 32 : 64;
+  const int col_blocks = (int)ceil_div(planes, p.CW);
+  // about four workgroups per CU in all, at least 256 rows each
+  int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(rows, 256), 1024 / col_blocks));
+  p.rows_per_block = round_up(ceil_div(rows, blocks), 256 / p.CW);
+  p.blocks = (int)ceil_div(rows, p.rows_per_block);
+  return p;
+}
+// out[c] = sum over row blocks, in block order, accumulated in double.
+__global__ void k_colsum_finish(const float *partial, int blocks, int planes, float *out) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= planes) return;
+  double s = 0;
+  for (int b = 0; b < blocks; b++) s += partial[(size_t)b * 2 * planes + c];
+  out[c] = (float)s;
+}
+static void column_sums(Metadata &m, const float *x, int64_t rows, int planes, float *out, hipStream_t s) {
+  if (planes <= 0) return;
+  if (rows <= 0) {
+    fill32(out, 0, planes, s);
+    return;
+  }
+  const ColsumPlan p = colsum_plan(rows, planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes);
+  k_colsum<0><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(x, planes, nullptr, nullptr, 0, nullptr, 0.f,
+                                                                                 rows, planes, p.CW, p.rows_per_block,
+                                                                                 m.partial.p);
+  LAUNCH_CHECK();
+  k_colsum_finish<<<grid_for(planes), TB, 0, s>>>(m.partial.p, p.blocks, planes, out);
+  LAUNCH_CHECK();
+}
+
+// ---- weight gradient ---------------------------------------------------------------------------
+// dW[k][c][o] = sum over positions t with nbr[k][t] >= 0 of a[nbr[k][t]][c] * b[row(t)][o].
+// One workgroup (4 wavefronts): tap k, positions [chunk * chunk_len, ...), channel tile 64 x 64.
+// Per step of 32 positions the gathered rows of a and the rows of b go through LDS as
+// [position][channel]; wavefront (wr, wc) owns the 32 x 32 quadrant and feeds
+// v_mfma_f32_16x16x4_f32 with the channel along the matrix rows / columns and four positions
+// along the contraction.  Steps none of whose positions has the tap are skipped by the table's
+// granule masks.  The next step's rows are fetched into registers while the current one runs.
+constexpr int DW_T = 64, DW_PS = 32, DW_LD = DW_T + 16;
+template <bool VEC4>
+__global__ __launch_bounds__(256) void k_conv_dw(const int *__restrict__ nbr, const int *__restrict__ rowmap,
+                                                 const unsigned *__restrict__ gmask, int K, int64_t n, int64_t npad,
+                                                 const float *__restrict__ a, int n_a, const float *__restrict__ b,
+                                                 int n_b, int64_t chunk_len, float *__restrict__ partial) {
+  __shared__ __attribute__((aligned(16))) float la[DW_PS * DW_LD], lb[DW_PS * DW_LD];
+  const int k = blockIdx.y;
+  const int tiles_o = (n_b + DW_T - 1) / DW_T;
+  const int ct = blockIdx.z / tiles_o, ot = blockIdx.z % tiles_o;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int wr = wave >> 1, wc = wave & 1;
+  const int64_t p0 = (int64_t)blockIdx.x * chunk_len, p1 = min(n, p0 + chunk_len);
+  // staging role of this thread: position lp of the step, channels [4 * lc, 4 * lc + 4) of each tile
+  const int lp = threadIdx.x >> 4, lc = threadIdx.x & 15;  // two positions per thread: lp and lp + 16
+  v4f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  auto step_has_tap = [&](int64_t t0) {
+    if (gmask == nullptr) return true;
+    const int64_t g0 = t0 >> 4, gl = (n - 1) >> 4;
+    return (((gmask[min(g0, gl)] | gmask[min(g0 + 1, gl)]) >> k) & 1u) != 0u;
+  };
+  auto load4 = [&](const float *base, int64_t row, int width, int c0) {
+    v4f v = (v4f){0.f, 0.f, 0.f, 0.f};
+    if (row < 0) return v;
+    const float *src = base + row * width;
+    if (VEC4) {
+      if (c0 < width) v = *reinterpret_cast<const v4f *>(src + c0);
+    } else {
+      if (c0 + 0 < width) v.x = src[c0 + 0];
+      if (c0 + 1 < width) v.y = src[c0 + 1];
+      if (c0 + 2 < width) v.z = src[c0 + 2];
+      if (c0 + 3 < width) v.w = src[c0 + 3];
+    }
+    return v;
+  };
+  v4f ra[2], rb[2];
+  auto fetch = [&](int64_t t0) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int64_t t = t0 + lp + 16 * h;
+      int64_t ja = -1, jb = -1;
+      if (t < p1) {
+        ja = nbr[(int64_t)k * npad + t];
+        jb = ja >= 0 ? (rowmap ? rowmap[t] : t) : -1;
+      }
+      ra[h] = load4(a, ja, n_a, ct * DW_T + 4 * lc);
+      rb[h] = load4(b, jb, n_b, ot * DW_T + 4 * lc);
+    }
+  };
+  // first step of the chunk that has the tap
+  int64_t t_cur = p0;
+  while (t_cur < p1 && !step_has_tap(t_cur)) t_cur += DW_PS;
+  if (t_cur < p1) fetch(t_cur);
+  while (t_cur < p1) {
+    __syncthreads();  // the previous step's MFMAs have read LDS
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      *reinterpret_cast<v4f *>(&la[(lp + 16 * h) * DW_LD + 4 * lc]) = ra[h];
+      *reinterpret_cast<v4f *>(&lb[(lp + 16 * h) * DW_LD + 4 * lc]) = rb[h];
+    }
+    __syncthreads();
+    int64_t t_nxt = t_cur + DW_PS;
+    while (t_nxt < p1 && !step_has_tap(t_nxt)) t_nxt += DW_PS;
+    if (t_nxt < p1) fetch(t_nxt);
+#pragma unroll
+    for (int kk = 0; kk < DW_PS / 4; kk++) {
+      float av[2], bv[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) av[i] = la[(4 * kk + g) * DW_LD + (2 * wr + i) * 16 + r16];
+#pragma unroll
+      for (int j = 0; j < 2; j++) bv[j] = lb[(4 * kk + g) * DW_LD + (2 * wc + j) * 16 + r16];
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+    t_cur = t_nxt;
+  }
+  // acc[i][j][r] = dW[k][ct*64 + (2wr+i)*16 + 4g + r][ot*64 + (2wc+j)*16 + r16] of this chunk
+  float *pk = partial + ((size_t)blockIdx.x * K + k) * (size_t)n_a * n_b;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int c = ct * DW_T + (2 * wr + i) * 16 + 4 * g + r, o = ot * DW_T + (2 * wc + j) * 16 + r16;
+        if (c < n_a && o < n_b) pk[(size_t)c * n_b + o] = acc[i][j][r];
+      }
+}
+// dw[i] = sum over chunks, in chunk order
+__global__ void k_dw_reduce(const float *partial, int chunks, int64_t per_chunk, float *dw) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= per_chunk) return;
+  float s = 0.f;
+  for (int c = 0; c < chunks; c++) s += partial[(size_t)c * per_chunk + i];
+  dw[i] = s;
+}
+// Any groups, any shapes: one thread per weight, positions in order.  The correctness path for
+// grouped convolutions, which the MFMA kernel does not cover.
+__global__ void k_conv_dw_generic(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad, const float *a,
+                                  int n_a, const float *b, int n_b, int groups, float *dw) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int ip = n_a / groups, op = n_b / groups;
+  if (i >= (int64_t)K * groups * ip * op) return;
+  const int o = (int)(i % op), c = (int)((i / op) % ip), g = (int)((i / ((int64_t)op * ip)) % groups);
+  const int k = (int)(i / ((int64_t)op * ip * groups));
+  float s = 0.f;
+  for (int64_t t = 0; t < n; t++) {
+    const int j = nbr[(int64_t)k * npad + t];
+    if (j < 0) continue;
+    const int64_t row = rowmap ? rowmap[t] : t;
+    s += a[(int64_t)j * n_a + g * ip + c] * b[row * n_b + g * op + o];
+  }
+  dw[i] = s;
+}
+
+static void weight_gradient(Metadata &m, const Table &t, const float *a, int n_a, const float *b, int n_b, int groups,
+                            float *dw, hipStream_t s) {
+  const int64_t per_chunk = (int64_t)t.K * (n_a / groups) * (n_b / groups) * groups;
+  if (t.n == 0) {
+    fill32(dw, 0, per_chunk, s);
+    return;
+  }
+  if (groups != 1) {
+    k_conv_dw_generic<<<grid_for(per_chunk), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, a, n_a, b, n_b,
+                                                         groups, dw);
+    LAUNCH_CHECK();
+    return;
+  }
+  const int tiles = (int)(ceil_div(n_a, DW_T) * ceil_div(n_b, DW_T));
+  if (t.K > 65535 || tiles > 65535) throw Error("weight gradient: filter volume or channel count too large");
+  // chunks: enough workgroups to fill the chip, partial sums bounded to about 256 MB
+  int64_t chunks = ceil_div(2048, (int64_t)t.K * tiles);
+  chunks = std::min<int64_t>(chunks, std::max<int64_t>(1, ((int64_t)64 << 20) / per_chunk));
+  chunks = std::max<int64_t>(1, std::min<int64_t>(chunks, ceil_div(t.n, 4 * DW_PS)));
+  const int64_t chunk_len = round_up(ceil_div(t.n, chunks), DW_PS);
+  chunks = ceil_div(t.n, chunk_len);
+  m.partial.reserve((size_t)chunks * per_chunk);
+  const bool vec4 = n_a % 4 == 0 && n_b % 4 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0;
+  const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
+  const dim3 grid((unsigned)chunks, (unsigned)t.K, (unsigned)tiles);
+  if (vec4)
+    k_conv_dw<true><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a, b, n_b, chunk_len,
+                                         m.partial.p);
+  else
+    k_conv_dw<false><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a, b, n_b, chunk_len,
+                                          m.partial.p);
+  LAUNCH_CHECK();
+  k_dw_reduce<<<grid_for(per_chunk), TB, 0, s>>>(m.partial.p, (int)chunks, per_chunk, dw);
+  LAUNCH_CHECK();
+}
+
+// ---- input gradient when the rules cannot be read from the other side ----------------------------
+// d_in[nbr[k][t]] += d_out[row(t)] * w[k]^T by scatter with atomics: submanifold rulebooks whose
+// taps have no mirror image (even filter sizes) or whose level holds repeated points.  Correct
+// for any table; the order of the additions, and so the last bits of the result, may vary.
+__global__ void k_conv_dinput_scatter(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad,
+                                      const float *d_out, const float *w, int n_in, int n_out, int groups,
+                                      float *d_in) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * n_in) return;
+  const int64_t t = i / n_in;
+  const int c = (int)(i - t * n_in);
+  const int ip = n_in / groups, op = n_out / groups, g = c / ip, cg = c - g * ip;
+  const int64_t row = rowmap ? rowmap[t] : t;
+  const float *d = d_out + row * n_out + g * op;
+  for (int k = 0; k < K; k++) {
+    const int j = nbr[(int64_t)k * npad + t];
+    if (j < 0) continue;
+    const float *wk = w + (((int64_t)k * groups + g) * ip + cg) * op;
+    float acc = 0.f;
+    for (int o = 0; o < op; o++) acc += d[o] * wk[o];
+    atomicAdd(&d_in[(int64_t)j * n_in + c], acc);
+  }
+}
+// flag[0] = 1 unless every position's centre tap names its own row (a level without repeated points)
+__global__ void k_centre_is_identity(const int *nbr_centre, const int *rowmap, int64_t n, int *flag) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n && nbr_centre[t] != (rowmap ? rowmap[t] : (int)t)) flag[0] = 1;
+}
+
+// Whether rule (k, i -> j) of a submanifold table implies rule (K-1-k, j -> i): odd filter sizes
+// on a level without repeated points.  Checked once per table (one host round trip).
+static bool taps_mirror(Metadata &m, Table &t, const int64_t *filter, hipStream_t s) {
+  if (t.mirror_known) return t.mirror;
+  bool odd = true;
+  for (int d = 0; d < m.dim; d++) odd = odd && (filter[d] % 2 == 1);
+  t.mirror = odd;
+  if (odd && t.n > 0) {
+    m.dflags.reserve(16);
+    fill32(m.dflags.p, 0, 1, s);
+    k_centre_is_identity<<<grid_for(t.n), TB, 0, s>>>(t.nbr.p + (int64_t)(t.K / 2) * t.npad, t.rowmap_ptr(), t.n,
+                                                      m.dflags.p);
+    LAUNCH_CHECK();
+    int flag = 0;
+    HIP_CHECK(hipMemcpyAsync(&flag, m.dflags.p, sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    t.mirror = flag == 0;
+  }
+  t.mirror_known = true;
+  return t.mirror;
+}
+
+// d_in = (table read from the output side) convolution of d_out with transposed weights.
+static void input_gradient(Metadata &m, const Table &t, const float *d_out, int64_t d_out_rows, float *d_in,
+                           const float *w, int n_in, int n_out, int groups, bool mirror, hipStream_t s) {
+  const int64_t wn = (int64_t)t.K * (n_in / groups) * (n_out / groups) * groups;
+  m.wt.reserve(wn);
+  k_transpose_weights<<<grid_for(wn), TB, 0, s>>>(w, m.wt.p, t.K, groups, n_in / groups, n_out / groups, mirror ? 1 : 0);
+  LAUNCH_CHECK();
+  conv_forward(m, t, d_out, d_out_rows, d_in, m.wt.p, nullptr, n_out, n_in, groups, nullptr, nullptr, s);
+}
+
+// CPU/Convolution.cpp:152-185.  d_bias may be null.
+void subm_conv_backward(Metadata &m, Table &t, const int64_t *filter, const float *in, float *d_in,
+                        const float *d_out, const float *w, float *d_w, float *d_bias, int n_in, int n_out,
+                        int groups, hipStream_t s) {
+  if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
+    throw Error("channel counts must be positive multiples of groups");
+  if (d_bias) column_sums(m, d_out, t.n, n_out, d_bias, s);
+  weight_gradient(m, t, in, n_in, d_out, n_out, groups, d_w, s);
+  if (t.n == 0) return;
+  if (taps_mirror(m, t, filter, s)) {
+    input_gradient(m, t, d_out, t.n, d_in, w, n_in, n_out, groups, true, s);
+  } else {
+    fill32(d_in, 0, t.n * n_in, s);
+    k_conv_dinput_scatter<<<grid_for(t.n * n_in), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, d_out, w, n_in,
+                                                               n_out, groups, d_in);
+    LAUNCH_CHECK();
+  }
+}
+// CPU/Convolution.cpp:81-115 (fwd: the table read from the coarse side, other: from the fine side)
+// and CPU/Deconvolution.cpp:43-77 (fwd: from the fine side, other: from the coarse side).
+// in_rows / out_rows: rows of the op's input and output levels.
+void strided_conv_backward(Metadata &m, const Table &fwd, const Table &other, int64_t in_rows, int64_t out_rows,
+                           const float *in, float *d_in, const float *d_out, const float *w, float *d_w, float *d_bias,
+                           int n_in, int n_out, int groups, hipStream_t s) {
+  if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
+    throw Error("channel counts must be positive multiples of groups");
+  if (d_bias) {
+    if (in_rows > 0)  // CPU/Convolution.cpp:98: only when the input level has rows
+      column_sums(m, d_out, out_rows, n_out, d_bias, s);
+    else
+      fill32(d_bias, 0, n_out, s);
+  }
+  weight_gradient(m, fwd, in, n_in, d_out, n_out, groups, d_w, s);
+  if (in_rows == 0) return;
+  if (other.n != in_rows) throw Error("internal: the rulebook's other side does not match the input level");
+  input_gradient(m, other, d_out, out_rows, d_in, w, n_in, n_out, groups, false, s);
+}
+
+// ---- batch normalisation, training mode ----------------------------------------------------------
+// CPU/BatchNormalization.cpp:19-40: batch mean and biased variance into save_mean / save_invstd,
+// running statistics updated with `momentum` weighting the old value and the unbiased variance;
+// coef = scale | shift for the affine pass.
+__global__ void k_bn_train_finish(const float *partial, int blocks, int planes, int64_t rows, float *save_mean,
+                                  float *save_invstd, float *running_mean, float *running_var, const float *gamma,
+                                  const float *beta, float eps, float momentum, float *coef) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= planes) return;
+  double s1 = 0, s2 = 0;
+  for (int b = 0; b < blocks; b++) {
+    s1 += partial[(size_t)b * 2 * planes + c];
+    s2 += partial[(size_t)b * 2 * planes + planes + c];
+  }
+  const double mean = s1 / (double)rows;
+  double ss = s2 - mean * mean * (double)rows;  // sum of squared deviations
+  if (ss < 0) ss = 0;
+  save_mean[c] = (float)mean;
+  running_mean[c] = momentum * running_mean[c] + (1 - momentum) * (float)mean;
+  running_var[c] = momentum * running_var[c] + (1 - momentum) * (float)(ss / (double)(rows - 1));
+  const float invstd = powf((float)(ss / (double)rows) + eps, -0.5f);
+  save_invstd[c] = invstd;
+  const float w = invstd * (gamma ? gamma[c] : 1.f);
+  coef[c] = w;
+  coef[planes + c] = -(float)mean * w + (beta ? beta[c] : 0.f);
+}
+// out = leaky(x * sc + sh), one thread per element (rows x planes), any strides
+__global__ void k_affine_leaky(const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                               int64_t out_stride, const float *coef, float leak) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = rows * planes, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / planes;
+    const int c = (int)(i - r * planes);
+    const float y = in[r * in_stride + c] * coef[c] + coef[planes + c];
+    out[r * out_stride + c] = y * (y > 0 ? 1.f : leak);
+  }
+}
+void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                      int64_t out_stride, float *save_mean, float *save_invstd, float *running_mean,
+                      float *running_var, const float *gamma, const float *beta, float eps, float momentum,
+                      float leak, hipStream_t s) {
+  if (rows <= 0 || planes <= 0) return;
+  Metadata &m = *scratch;
+  const ColsumPlan p = colsum_plan(rows, planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes);
+  m.prebuf.reserve(2 * (size_t)planes);
+  k_colsum<1><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(in, in_stride, nullptr, nullptr, 0, nullptr,
+                                                                                 0.f, rows, planes, p.CW, p.rows_per_block,
+                                                                                 m.partial.p);
+  LAUNCH_CHECK();
+  k_bn_train_finish<<<grid_for(planes), TB, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_mean, save_invstd,
+                                                    running_mean, running_var, gamma, beta, eps, momentum, m.prebuf.p);
+  LAUNCH_CHECK();
+  const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
+  k_affine_leaky<<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, m.prebuf.p, leak);
+  LAUNCH_CHECK();
+}
+// CPU/BatchNormalization.cpp:84-106: coef = gradMean | k | invstd * gamma
+__global__ void k_bn_bwd_finish(const float *partial, int blocks, int planes, int64_t rows, const float *save_invstd,
+                                const float *gamma, float *d_gamma, float *d_beta, float *coef) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= planes) return;
+  double sd = 0, dotp = 0;
+  for (int b = 0; b < blocks; b++) {
+    sd += partial[(size_t)b * 2 * planes + c];
+    dotp += partial[(size_t)b * 2 * planes + planes + c];
+  }
+  const float invstd = save_invstd[c];
+  if (d_beta) d_beta[c] = (float)sd;
+  if (d_gamma) d_gamma[c] = (float)dotp * invstd;
+  coef[c] = (float)(sd / (double)rows);
+  coef[planes + c] = (float)dotp * invstd * invstd / (float)rows;
+  coef[2 * planes + c] = invstd * (gamma ? gamma[c] : 1.f);
+}
+__global__ void k_bn_bwd_apply(const float *in, float *d_in, const float *out, const float *d_out, int64_t rows,
+                               int planes, int64_t in_stride, int64_t out_stride, const float *save_mean,
+                               const float *coef, float leak) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = rows * planes, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / planes;
+    const int c = (int)(i - r * planes);
+    float d = d_out[r * out_stride + c];
+    d *= out[r * out_stride + c] > 0.f ? 1.f : leak;
+    d_in[r * in_stride + c] =
+        (d - coef[c] - (in[r * in_stride + c] - save_mean[c]) * coef[planes + c]) * coef[2 * planes + c];
+  }
+}
+// CPU/BatchNormalization.cpp:63-107.  d_out is not modified (the reference scales it in place).
+void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *out, const float *d_out, int64_t rows,
+                 int planes, int64_t in_stride, int64_t out_stride, const float *save_mean, const float *save_invstd,
+                 const float *gamma, float *d_gamma, float *d_beta, float leak, hipStream_t s) {
+  if (planes <= 0) return;
+  if (rows <= 0) {
+    if (d_gamma) fill32(d_gamma, 0, planes, s);
+    if (d_beta) fill32(d_beta, 0, planes, s);
+    return;
+  }
+  Metadata &m = *scratch;
+  const ColsumPlan p = colsum_plan(rows, planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes);
+  m.prebuf.reserve(3 * (size_t)planes);
+  k_colsum<2><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(in, in_stride, d_out, out, out_stride,
+                                                                                 save_mean, leak, rows, planes, p.CW,
+                                                                                 p.rows_per_block, m.partial.p);
+  LAUNCH_CHECK();
+  k_bn_bwd_finish<<<grid_for(planes), TB, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_invstd, gamma, d_gamma, d_beta,
+                                                  m.prebuf.p);
+  LAUNCH_CHECK();
+  const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
+  k_bn_bwd_apply<<<dim3((unsigned)blocks), TB, 0, s>>>(in, d_in, out, d_out, rows, planes, in_stride, out_stride, save_mean,
+                                                       m.prebuf.p, leak);
+  LAUNCH_CHECK();
+}
+
+// ---- pooling -------------------------------------------------------------------------------------
+// Gathers over the table read from the side of the gradient that is being written, one thread per
+// (position, plane); taps in ascending order, as the reference walks its rule lists.
+// MAX      CPU/MaxPooling.cpp:21-35,61-87: table = fine side; d_in[i][p] = sum over the windows o
+//          that hold i of (out[o][p] == in[i][p] ? d_out[o][p] : 0).  The reference compares with
+//          the input planes WITHOUT the nFeaturesToDrop offset its forward pass applies; so does this.
+// AVERAGE  CPU/AveragePooling.cpp:21-35,62-86: table = fine side; d_in[i][drop + p] = sum of d_out[o][p] / K.
+// UNPOOL   CPU/UnPooling.cpp:21-32,58-78: table = coarse side; d_in[o][drop + p] = sum of d_out[i][p].
+// The columns of d_in the rules do not reach are zeroed.
+enum { PB_MAX = 0, PB_AVERAGE = 1, PB_UNPOOL = 2 };
+template <int MODE>
+__global__ void k_pool_bwd(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad, const float *in,
+                           float *d_in, int in_stride, const float *out, const float *d_out, int planes, int drop) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = n * in_stride, step = (int64_t)gridDim.x * blockDim.x;
+  const int off = MODE == PB_MAX ? 0 : drop;
+  for (; i < total; i += step) {
+    const int64_t t = i / in_stride;
+    const int col = (int)(i - t * in_stride);
+    const int64_t row = rowmap ? rowmap[t] : t;
+    const int p = col - off;
+    float acc = 0.f;
+    if (p >= 0 && p < planes) {
+      const float x = MODE == PB_MAX ? in[row * in_stride + col] : 0.f;
+      for (int k = 0; k < K; k++) {
+        const int o = nbr[(int64_t)k * npad + t];
+        if (o < 0) continue;
+        const float d = d_out[(int64_t)o * planes + p];
+        if (MODE == PB_MAX)
+          acc += out[(int64_t)o * planes + p] == x ? d : 0.f;
+        else if (MODE == PB_AVERAGE)
+          acc += d / (float)K;
+        else
+          acc += d;
+      }
+    }
+    d_in[row * in_stride + col] = acc;
+  }
+}
+void pool_backward(int mode, const Table &t, const float *in, float *d_in, int in_stride, const float *out,
+                   const float *d_out, int planes, int drop, hipStream_t s) {
+  if (t.n == 0 || in_stride <= 0) return;
+  const int64_t blocks = std::min<int64_t>(ceil_div(t.n * in_stride, TB), 256 * 64);
+  const dim3 g((unsigned)blocks);
+  if (mode == PB_MAX)
+    k_pool_bwd<PB_MAX><<<g, TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, d_in, in_stride, out, d_out, planes, drop);
+  else if (mode == PB_AVERAGE)
+    k_pool_bwd<PB_AVERAGE><<<g, TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, d_in, in_stride, out, d_out, planes, drop);
+  else
+    k_pool_bwd<PB_UNPOOL><<<g, TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, d_in, in_stride, out, d_out, planes, drop);
+  LAUNCH_CHECK();
+}
+
+// ---- sparse to dense -------------------------------------------------------------------------------
+// CPU/SparseToDense.cpp:21-33,66-90: d_in[row][p] = d_out[sample][p][offset(site)].
+__global__ void k_s2d_bwd(Geom g, const int *soa, int64_t n, int64_t npad, float *d_in, const float *d_out, int planes,
+                          int64_t vol) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = n * planes, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / planes;
+    const int p = (int)(i - r * planes);
+    int64_t off = 0;
+    for (int d = 0; d < g.dim; d++) off = off * g.size[d] + soa[d * npad + r];
+    const int b = soa[g.dim * npad + r];
+    d_in[i] = d_out[((int64_t)b * planes + p) * vol + off];
+  }
+}
+void s2d_backward(const Level &l, float *d_in, const float *d_out, int planes, hipStream_t s) {
+  if (l.n == 0 || planes <= 0) return;
+  int64_t vol = 1;
+  for (int d = 0; d < l.g.dim; d++) vol *= l.g.size[d];
+  const int64_t blocks = std::min<int64_t>(ceil_div(l.n * planes, TB), 256 * 64);
+  k_s2d_bwd<<<dim3((unsigned)blocks), TB, 0, s>>>(l.g, l.coords.p, l.n, l.npad, d_in, d_out, planes, vol);
+  LAUNCH_CHECK();
+}
+
+// CPU/NetworkInNetwork.cpp:24-47 over the one-tap identity table.
+void nin_backward(Metadata &m, const Table &t, const float *in, float *d_in, const float *d_out, const float *w,
+                  float *d_w, float *d_bias, int n_in, int n_out, hipStream_t s) {
+  if (d_bias) column_sums(m, d_out, t.n, n_out, d_bias, s);
+  weight_gradient(m, t, in, n_in, d_out, n_out, 1, d_w, s);
+  if (t.n == 0) return;
+  input_gradient(m, t, d_out, t.n, d_in, w, n_in, n_out, 1, false, s);
+}
+
+}  // namespace scn

@@ -70,6 +70,9 @@ struct Table {
   DevBuf<unsigned> gmask;  // K <= 32 and pattern-sorted: bit k of gmask[i] = some position of granule i (16 positions) has tap k
   bool identity_rows = false;  // rowmap[t] == t: kernels skip the indirection
   const int *rowmap_ptr() const { return identity_rows ? nullptr : rowmap.p; }
+  // Submanifold tables, decided on first use by a backward pass: does rule (k, i -> j) imply
+  // rule (K-1-k, j -> i)?  (Odd filter sizes on a level without repeated points.)
+  bool mirror_known = false, mirror = false;
   std::shared_ptr<Counts> cnt;  // never null once the table has been built
   const std::vector<int64_t> &counts(hipStream_t s) {
     ensure_counts(*cnt, s);
@@ -154,7 +157,8 @@ struct Metadata {
   DevBuf<int> v0, v1, f0, f1, s0, s1;
   DevBuf<int> dflags;
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
-  DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups
+  DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups; partial sums of reductions
+  DevBuf<float> wt;       // transposed weights of the input-gradient convolution of a backward pass
   DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
   // Non-null while an allocation-free convolution runs: the three buffers above are then fixed
   // regions of a static device array (conv.hip) and nothing may be reserved.
@@ -238,5 +242,28 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
 void input_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s);
 void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s);
 void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStream_t s);
+
+// backward.hip
+void subm_conv_backward(Metadata &m, Table &t, const int64_t *filter, const float *in, float *d_in,
+                        const float *d_out, const float *w, float *d_w, float *d_bias, int n_in, int n_out,
+                        int groups, hipStream_t s);
+void strided_conv_backward(Metadata &m, const Table &fwd, const Table &other, int64_t in_rows, int64_t out_rows,
+                           const float *in, float *d_in, const float *d_out, const float *w, float *d_w, float *d_bias,
+                           int n_in, int n_out, int groups, hipStream_t s);
+void nin_backward(Metadata &m, const Table &t, const float *in, float *d_in, const float *d_out, const float *w,
+                  float *d_w, float *d_bias, int n_in, int n_out, hipStream_t s);
+void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
+                      int64_t out_stride, float *save_mean, float *save_invstd, float *running_mean,
+                      float *running_var, const float *gamma, const float *beta, float eps, float momentum,
+                      float leak, hipStream_t s);
+void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *out, const float *d_out, int64_t rows,
+                 int planes, int64_t in_stride, int64_t out_stride, const float *save_mean, const float *save_invstd,
+                 const float *gamma, float *d_gamma, float *d_beta, float leak, hipStream_t s);
+// mode 0: max pooling (table read from the fine side), 1: average pooling (fine side), 2: unpooling (coarse side)
+void pool_backward(int mode, const Table &t, const float *in, float *d_in, int in_stride, const float *out,
+                   const float *d_out, int planes, int drop, hipStream_t s);
+void s2d_backward(const Level &l, float *d_in, const float *d_out, int planes, hipStream_t s);
+void input_backward(const InputRules &r, float *d_in, const float *d_out, int planes, hipStream_t s);
+void output_backward(const InputRules &r, float *d_in, const float *d_out, int planes, hipStream_t s);
 
 }  // namespace scn

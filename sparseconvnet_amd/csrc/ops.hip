@@ -157,7 +157,7 @@ void unpool_forward(const Table &t, const float *in, int in_stride, float *out, 
 // the site lists.
 __global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const int *run_len,
                             const unsigned char *overwrite, int64_t n_out, int mode, const float *in, float *out,
-                            int planes) {
+                            int planes, int average) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = n_out * planes;
   int64_t step = (int64_t)gridDim.x * blockDim.x;
@@ -169,7 +169,7 @@ __global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const i
     if (mode == 1 || mode == 2 || mode == 5) {
       acc += in[(int64_t)listed_point(sorted_idx, st, len, mode, overwrite) * planes + p];
     } else {
-      float mult = (mode == 4 && len > 0) ? 1.0f / (float)len : 1.0f;
+      float mult = (average && len > 0) ? 1.0f / (float)len : 1.0f;
       for (int q = 0; q < len; q++) acc += mult * in[(int64_t)sorted_idx[st + q] * planes + p];
     }
     out[i] = acc;
@@ -187,17 +187,36 @@ void input_forward(const InputRules &r, const float *in, float *out, int planes,
   int64_t total = r.n_out * planes;
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p,
-                                                    r.n_out, r.mode, in, out, planes);
+                                                    r.n_out, r.mode, in, out, planes, r.mode == 4 ? 1 : 0);
+  LAUNCH_CHECK();
+}
+// CPU/IOLayers.cpp:116-135 (and :207-229): the gradient of the output layer's input is
+// InputLayer_ForwardPass without averaging: every site sums the gradients of the points it lists.
+void output_backward(const InputRules &r, float *d_in, const float *d_out, int planes, hipStream_t s) {
+  if (r.mode < 0) throw Error("input layer rules have not been built");
+  if (planes <= 0) return;
+  if (r.mode == 0) {
+    if (r.n_in)
+      HIP_CHECK(hipMemcpyAsync(d_in, d_out, sizeof(float) * r.n_in * planes, hipMemcpyDeviceToDevice, s));
+    return;
+  }
+  if (r.n_out == 0) return;
+  int64_t total = r.n_out * planes;
+  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p,
+                                                    r.n_out, r.mode, d_out, d_in, planes, 0);
   LAUNCH_CHECK();
 }
 
 // CPU/IOLayers.cpp:95-115 (InputLayer_BackwardPass :31-47 without averaging): every input
 // point listed in its site's rule receives the site's row; as a gather per input point.
 // Modes 1 / 2 / 5 list a single point per site, the others get zeros.
+// average != 0: the row is scaled by 1 / (number of points of the site), which makes this the
+// gradient of the mode-4 input layer (CPU/IOLayers.cpp:31-47 with average = true).
 template <int V>
 __global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, const int *run_start,
                              const int *run_len, const unsigned char *overwrite, int64_t n_in, int mode,
-                             const float *in, float *out, int planes) {
+                             const float *in, float *out, int planes, int average) {
   // thread -> (input point, group of V planes)
   const int groups = planes / V;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -210,16 +229,20 @@ __global__ void k_output_fwd(const int *row_of_input, const int *sorted_idx, con
     bool listed = row >= 0;  // empty positions of a batch-by-length input get zeros
     if (listed && (mode == 1 || mode == 2 || mode == 5))
       listed = listed_point(sorted_idx, run_start[row], run_len[row], mode, overwrite) == (int)pt;
+    const float mult = (average && listed) ? 1.0f / (float)run_len[row] : 1.0f;
     if (V == 4) {
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       if (listed) v = *reinterpret_cast<const float4 *>(in + (int64_t)row * planes + p);
+      if (average) v = make_float4(mult * v.x, mult * v.y, mult * v.z, mult * v.w);
       *reinterpret_cast<float4 *>(out + pt * planes + p) = v;
     } else {
-      out[pt * planes + p] = listed ? in[(int64_t)row * planes + p] : 0.0f;
+      const float v = listed ? in[(int64_t)row * planes + p] : 0.0f;
+      out[pt * planes + p] = average ? mult * v : v;
     }
   }
 }
-void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s) {
+static void output_forward_impl(const InputRules &r, const float *in, float *out, int planes, int average,
+                                hipStream_t s) {
   if (r.mode < 0) throw Error("input layer rules have not been built");
   if (planes <= 0 || r.n_in == 0) return;
   if (r.mode == 0) {
@@ -235,11 +258,21 @@ void output_forward(const InputRules &r, const float *in, float *out, int planes
   const int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   if (vec)
     k_output_fwd<4><<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
-                                                          r.run_len.p, r.overwrite.p, r.n_in, r.mode, in, out, planes);
+                                                          r.run_len.p, r.overwrite.p, r.n_in, r.mode, in, out, planes,
+                                                          average);
   else
     k_output_fwd<1><<<dim3((unsigned)blocks), TB, 0, s>>>(r.row_of_input.p, r.sorted_idx.p, r.run_start.p,
-                                                          r.run_len.p, r.overwrite.p, r.n_in, r.mode, in, out, planes);
+                                                          r.run_len.p, r.overwrite.p, r.n_in, r.mode, in, out, planes,
+                                                          average);
   LAUNCH_CHECK();
+}
+void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s) {
+  output_forward_impl(r, in, out, planes, 0, s);
+}
+// CPU/IOLayers.cpp:73-93 (and :161-184): every listed point receives its site's gradient, scaled
+// by 1 / count in mode 4; points a site does not list, and empty positions, get zeros.
+void input_backward(const InputRules &r, float *d_in, const float *d_out, int planes, hipStream_t s) {
+  output_forward_impl(r, d_out, d_in, planes, r.mode == 4 ? 1 : 0, s);
 }
 
 // ---- sparse to dense --------------------------------------------------------------------

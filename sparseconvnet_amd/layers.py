@@ -1,8 +1,8 @@
-"""The forward-pass modules, with the constructor signatures, attribute names, parameter
+"""The modules of the path, with the constructor signatures, attribute names, parameter
 shapes, initialisation, spatial-size arithmetic and repr of the reference's Python modules
 (cited per class; paths relative to the reference's sparseconvnet/ directory).  Each forward
-calls the HIP library through sparseconvnet_amd.metadata; there is no backward: this build
-covers inference, and differentiating through a module raises."""
+and each backward calls the HIP library through sparseconvnet_amd.metadata; the
+torch.autograd.Function classes mirror the reference's *Function classes."""
 import torch
 from torch.autograd import Function
 from torch.nn import Module, Parameter
@@ -14,22 +14,141 @@ from .tensor import SparseConvNetTensor
 from .utils import optionalTensor, toLongTensor
 
 
-class _ForwardOnly(Function):
-    """Runs `fn(*tensors)` outside autograd; backward is not part of this build."""
+def _opt(t):
+    """None for the empty tensor that stands for "no bias" (utils.py:21-22)."""
+    return t if t is not None and t.numel() else None
+
+
+class _ConvFunction(Function):
+    """submanifoldConvolution.py:63-113, convolution.py:72-130, deconvolution.py:49-128: kind 0 /
+    1 / 2.  pre / post: eval-mode batch norms applied inside the convolution (inference only)."""
 
     @staticmethod
-    def forward(ctx, fn, *tensors):
-        return fn(*tensors)
+    def forward(ctx, features, weight, bias, md, kind, sizes, pre, post):
+        ctx.md, ctx.kind, ctx.sizes, ctx.fused = md, kind, sizes, pre is not None or post is not None
+        ctx.has_bias = bias.numel() > 0
+        ctx.save_for_backward(features, weight)
+        fn = (md.submanifoldConvolution, md.convolution, md.deconvolution)[kind]
+        out, _ = fn(*sizes, features, weight, bias, pre, post, want_macs=False)
+        _count(out)
+        return out
 
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("sparseconvnet_amd implements the forward (inference) pass only")
+    def backward(ctx, grad_output):
+        # batchNormalization.py:147: the reference refuses to differentiate an eval-mode batch norm
+        assert not ctx.fused, "backward through an eval-mode batch normalisation; call .train() on the model"
+        features, weight = ctx.saved_tensors
+        fn = (ctx.md.submanifoldConvolutionBackward, ctx.md.convolutionBackward, ctx.md.deconvolutionBackward)[ctx.kind]
+        d_in, d_w, d_b = fn(*ctx.sizes, features, grad_output.contiguous(), weight, ctx.has_bias)
+        return d_in, d_w, d_b, None, None, None, None, None
 
 
-def _run(fn, *tensors):
-    if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors):
-        return _ForwardOnly.apply(fn, *tensors)
-    return fn(*tensors)
+class _NetworkInNetworkFunction(Function):
+    """networkInNetwork.py:13-56."""
+
+    @staticmethod
+    def forward(ctx, features, weight, bias, md):
+        ctx.md, ctx.has_bias = md, bias.numel() > 0
+        ctx.save_for_backward(features, weight)
+        out, _ = md.networkInNetwork(features, weight, bias, want_macs=False)
+        _count(out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        features, weight = ctx.saved_tensors
+        d_in, d_w, d_b = ctx.md.networkInNetworkBackward(features, grad_output.contiguous(), weight, ctx.has_bias)
+        return d_in, d_w, d_b, None
+
+
+class _BatchNormalizationFunction(Function):
+    """batchNormalization.py:93-160."""
+
+    @staticmethod
+    def forward(ctx, features, weight, bias, running_mean, running_var, eps, momentum, train, leakiness, md):
+        ctx.md, ctx.train, ctx.leakiness, ctx.affine = md, train, leakiness, weight.numel() > 0
+        if train:
+            out, save_mean, save_invstd = md.batchNormTrain(features, running_mean, running_var, _opt(weight),
+                                                            _opt(bias), eps, momentum, leakiness)
+            ctx.save_for_backward(features, out, weight, save_mean, save_invstd)
+        else:
+            out = _md.batchNormEval(features, running_mean, running_var, _opt(weight), _opt(bias), eps, leakiness)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert ctx.train, "backward through an eval-mode batch normalisation; call .train() on the model"
+        features, out, weight, save_mean, save_invstd = ctx.saved_tensors
+        d_in, d_w, d_b = ctx.md.batchNormBackward(features, out, grad_output.contiguous(), save_mean, save_invstd,
+                                                  _opt(weight), ctx.leakiness, ctx.affine)
+        return d_in, d_w, d_b, None, None, None, None, None, None, None
+
+
+class _PoolingFunction(Function):
+    """maxPooling.py:14-72, averagePooling.py:13-66, unPooling.py:14-57: which = 'max', 'average',
+    'un'.  sizes = (input level, output level, pool size, pool stride) of the op."""
+
+    @staticmethod
+    def forward(ctx, features, md, which, sizes, drop):
+        ctx.md, ctx.which, ctx.sizes, ctx.drop, ctx.shape = md, which, sizes, drop, tuple(features.shape)
+        fn = {"max": md.maxPooling, "average": md.averagePooling, "un": md.unPooling}[which]
+        out = fn(*sizes, features, drop)
+        if which == "max":
+            ctx.save_for_backward(features, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        g = grad_output.contiguous()
+        if ctx.which == "max":
+            features, out = ctx.saved_tensors
+            d_in = ctx.md.maxPoolingBackward(*ctx.sizes, features, out, g, ctx.drop)
+        elif ctx.which == "average":
+            d_in = ctx.md.averagePoolingBackward(*ctx.sizes, ctx.shape, g, ctx.drop)
+        else:
+            d_in = ctx.md.unPoolingBackward(*ctx.sizes, ctx.shape, g, ctx.drop)
+        return d_in, None, None, None, None
+
+
+class _InputLayerFunction(Function):
+    """ioLayers.py:163-196 and :216-248 (bl)."""
+
+    @staticmethod
+    def forward(ctx, features, md, spatial_size, coords, batch_size, mode, bl):
+        ctx.md, ctx.bl = md, bl
+        if bl:
+            return md.blInputLayer(spatial_size, coords, features, mode)
+        return md.inputLayer(spatial_size, coords, features, batch_size, mode)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return ctx.md.inputLayerBackward(grad_output.contiguous(), ctx.bl), None, None, None, None, None, None
+
+
+class _OutputLayerFunction(Function):
+    """ioLayers.py:198-213 and :250-283 (bl)."""
+
+    @staticmethod
+    def forward(ctx, features, md, bl):
+        ctx.md, ctx.rows = md, features.size(0)
+        return md.blOutputLayer(features) if bl else md.outputLayer(features)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return ctx.md.outputLayerBackward(grad_output.contiguous(), ctx.rows), None, None
+
+
+class _SparseToDenseFunction(Function):
+    """sparseToDense.py:25-54."""
+
+    @staticmethod
+    def forward(ctx, features, md, spatial_size, planes):
+        ctx.md, ctx.spatial_size, ctx.rows = md, spatial_size, features.size(0)
+        return md.sparseToDense(spatial_size, features, planes)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return ctx.md.sparseToDenseBackward(ctx.spatial_size, grad_output.contiguous(), ctx.rows), None, None, None
 
 
 def _size_repr(prefix, size, stride=None):
@@ -121,13 +240,8 @@ class SubmanifoldConvolution(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
-        md, sz, fs, bn, post = input.metadata, input.spatial_size, self.filter_size, _bn_args(pre_bn), _bn_args(post_bn)
-
-        def fn(x, w, b):
-            y, _ = md.submanifoldConvolution(sz, fs, x, w, b, bn, post, want_macs=False)
-            _count(y)
-            return y
-        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 0,
+                                              (input.spatial_size, self.filter_size), _bn_args(pre_bn), _bn_args(post_bn))
         return output
 
     def __repr__(self):
@@ -165,14 +279,9 @@ class Convolution(Module):
             self.filter_stride, rounding_mode='trunc') + 1
         assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
             input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
-        md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
-        bn, post = _bn_args(pre_bn), _bn_args(post_bn)
-
-        def fn(x, w, b):
-            y, _ = md.convolution(*a, x, w, b, bn, post, want_macs=False)
-            _count(y)
-            return y
-        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 1,
+                                              a, _bn_args(pre_bn), _bn_args(post_bn))
         return output
 
     def __repr__(self):
@@ -204,14 +313,9 @@ class Deconvolution(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
-        md, a = input.metadata, (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
-        bn, post = _bn_args(pre_bn), _bn_args(post_bn)
-
-        def fn(x, w, b):
-            y, _ = md.deconvolution(*a, x, w, b, bn, post, want_macs=False)
-            _count(y)
-            return y
-        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 2,
+                                              a, _bn_args(pre_bn), _bn_args(post_bn))
         return output
 
     def __repr__(self):
@@ -242,13 +346,8 @@ class NetworkInNetwork(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
-        md = input.metadata
-
-        def fn(x, w, b):
-            y, _ = md.networkInNetwork(x, w, b, want_macs=False)
-            _count(y)
-            return y
-        output.features = _run(fn, input.features, self.weight, optionalTensor(self, 'bias'))
+        output.features = _NetworkInNetworkFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'),
+                                                          input.metadata)
         return output
 
     def __repr__(self):
@@ -260,7 +359,8 @@ class NetworkInNetwork(Module):
 
 class BatchNormalization(Module):
     """batchNormalization.py:13-71.  leakiness: 0 = ReLU, (0,1) = leaky ReLU, 1 = none.
-    Only eval mode is implemented: the running statistics are used as they are."""
+    Training mode normalises with the batch statistics and updates the running ones
+    (momentum weights the old value); eval mode uses the running statistics as they are."""
 
     def __init__(self, nPlanes, eps=1e-4, momentum=0.99, affine=True, leakiness=1):
         Module.__init__(self)
@@ -279,15 +379,12 @@ class BatchNormalization(Module):
         if input.features.nelement() == 0:
             return input
         assert input.features.size(1) == self.nPlanes, (self.nPlanes, input.features.shape)
-        if self.training:
-            raise NotImplementedError("sparseconvnet_amd batch normalisation runs in eval mode only; "
-                                      "call .eval() on the model")
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
-        eps, leak, mean, var = self.eps, self.leakiness, self.running_mean, self.running_var
-        output.features = _run(lambda x, w, b: _md.batchNormEval(x, mean, var, w, b, eps, leak),
-                               input.features, optionalTensor(self, 'weight'), optionalTensor(self, 'bias'))
+        output.features = _BatchNormalizationFunction.apply(
+            input.features, optionalTensor(self, 'weight'), optionalTensor(self, 'bias'), self.running_mean,
+            self.running_var, self.eps, self.momentum, self.training, self.leakiness, input.metadata)
         return output
 
     def input_spatial_size(self, out_size):
@@ -339,9 +436,8 @@ class MaxPooling(Module):
         output.spatial_size = (input.spatial_size - self.pool_size).div(
             self.pool_stride, rounding_mode='trunc') + 1
         assert ((output.spatial_size - 1) * self.pool_stride + self.pool_size == input.spatial_size).all()
-        md, a, drop = input.metadata, (input.spatial_size, output.spatial_size, self.pool_size,
-                                       self.pool_stride), self.nFeaturesToDrop
-        output.features = _run(lambda x: md.maxPooling(*a, x, drop), input.features)
+        a = (input.spatial_size, output.spatial_size, self.pool_size, self.pool_stride)
+        output.features = _PoolingFunction.apply(input.features, input.metadata, "max", a, self.nFeaturesToDrop)
         return output
 
     def input_spatial_size(self, out_size):
@@ -363,9 +459,8 @@ class AveragePooling(MaxPooling):
         output.spatial_size = (input.spatial_size - self.pool_size).div(
             self.pool_stride, rounding_mode='trunc') + 1
         assert ((output.spatial_size - 1) * self.pool_stride + self.pool_size == input.spatial_size).all()
-        md, a, drop = input.metadata, (input.spatial_size, output.spatial_size, self.pool_size,
-                                       self.pool_stride), self.nFeaturesToDrop
-        output.features = _run(lambda x: md.averagePooling(*a, x, drop), input.features)
+        a = (input.spatial_size, output.spatial_size, self.pool_size, self.pool_stride)
+        output.features = _PoolingFunction.apply(input.features, input.metadata, "average", a, self.nFeaturesToDrop)
         return output
 
     def __repr__(self):
@@ -387,9 +482,8 @@ class UnPooling(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.pool_stride + self.pool_size
-        md, a, drop = input.metadata, (input.spatial_size, output.spatial_size, self.pool_size,
-                                       self.pool_stride), self.nFeaturesToDrop
-        output.features = _run(lambda x: md.unPooling(*a, x, drop), input.features)
+        a = (input.spatial_size, output.spatial_size, self.pool_size, self.pool_stride)
+        output.features = _PoolingFunction.apply(input.features, input.metadata, "un", a, self.nFeaturesToDrop)
         return output
 
     def input_spatial_size(self, out_size):
@@ -425,9 +519,9 @@ class InputLayer(Module):
         feats = input[1].to(self.device) if self.device else input[1]
         if not feats.is_cuda:
             feats = feats.cuda()
-        md, sz, coords, mode = output.metadata, self.spatial_size, input[0], self.mode
         batch_size = 0 if len(input) == 2 else input[2]
-        output.features = _run(lambda f: md.inputLayer(sz, coords, f, batch_size, mode), feats.float())
+        output.features = _InputLayerFunction.apply(feats.float(), output.metadata, self.spatial_size, input[0], batch_size,
+                                                    self.mode, False)
         return output
 
 
@@ -439,8 +533,7 @@ class OutputLayer(Module):
         self.dimension = dimension
 
     def forward(self, input):
-        md = input.metadata
-        return _run(lambda x: md.outputLayer(x), input.features)
+        return _OutputLayerFunction.apply(input.features, input.metadata, False)
 
 
 class BLInputLayer(Module):
@@ -465,8 +558,8 @@ class BLInputLayer(Module):
         feats = input[1].to(self.device) if self.device else input[1]
         if not feats.is_cuda:
             feats = feats.cuda()
-        md, sz, coords, mode = output.metadata, self.spatial_size, input[0], self.mode
-        output.features = _run(lambda f: md.blInputLayer(sz, coords, f, mode), feats.float())
+        output.features = _InputLayerFunction.apply(feats.float(), output.metadata, self.spatial_size, input[0], 0,
+                                                    self.mode, True)
         return output
 
 
@@ -478,8 +571,7 @@ class BLOutputLayer(Module):
         self.dimension = dimension
 
     def forward(self, input):
-        md = input.metadata
-        return _run(lambda x: md.blOutputLayer(x), input.features)
+        return _OutputLayerFunction.apply(input.features, input.metadata, True)
 
 
 class SparseToDense(Module):
@@ -491,8 +583,7 @@ class SparseToDense(Module):
         self.nPlanes = nPlanes
 
     def forward(self, input):
-        md, sz, planes = input.metadata, input.spatial_size, self.nPlanes
-        return _run(lambda x: md.sparseToDense(sz, x, planes), input.features)
+        return _SparseToDenseFunction.apply(input.features, input.metadata, input.spatial_size, self.nPlanes)
 
     def input_spatial_size(self, out_size):
         return out_size
@@ -536,7 +627,8 @@ class DenseToSparse(Module):
         def gather(x):
             rows = x.permute(0, *range(2, 2 + d), 1)[tuple(nz.t())].float().contiguous()
             return md.inputLayer(sz, coords, rows, batch, 0)
-        output.features = _run(gather, input)
+        with torch.no_grad():
+            output.features = gather(input)
         return output
 
     def input_spatial_size(self, out_size):

@@ -290,6 +290,135 @@ class Metadata:
         return out
 
 
+    # ---- backward ops: each returns the gradients the reference's backward call fills ----------
+    def _convBackward(self, fn, size_args, features, grad_output, weight, with_bias):
+        features = _features(features, "features")
+        grad_output = _features(grad_output, "grad_output")
+        weight = _features(weight, "weight")
+        K, groups, ip, op = weight.shape
+        d_in = torch.empty_like(features)
+        d_w = torch.empty_like(weight)
+        d_b = torch.empty((groups * op,), dtype=torch.float32, device=features.device) if with_bias else None
+        _lib.check(fn(self._h, *size_args, _ptr(features), _ptr(d_in), _ptr(grad_output), _ptr(weight), _ptr(d_w),
+                      _ptr(d_b), groups * ip, groups * op, groups, _stream()))
+        return d_in, d_w, d_b
+
+    def submanifoldConvolutionBackward(self, spatial_size, filter_size, features, grad_output, weight, with_bias):
+        return self._convBackward(self._L.scn_subm_conv_bwd, (self._s(spatial_size), self._s(filter_size)), features,
+                                  grad_output, weight, with_bias)
+
+    def convolutionBackward(self, in_size, out_size, filter_size, stride, features, grad_output, weight, with_bias):
+        a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        return self._convBackward(self._L.scn_conv_bwd, a, features, grad_output, weight, with_bias)
+
+    def deconvolutionBackward(self, in_size, out_size, filter_size, stride, features, grad_output, weight, with_bias):
+        a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        return self._convBackward(self._L.scn_deconv_bwd, a, features, grad_output, weight, with_bias)
+
+    def networkInNetworkBackward(self, features, grad_output, weight, with_bias):
+        features = _features(features, "features")
+        grad_output = _features(grad_output, "grad_output")
+        weight = _features(weight, "weight")
+        n_in, n_out = weight.shape
+        d_in, d_w = torch.empty_like(features), torch.empty_like(weight)
+        d_b = torch.empty((n_out,), dtype=torch.float32, device=features.device) if with_bias else None
+        _lib.check(self._L.scn_nin_bwd(self._h, _ptr(features), _ptr(d_in), _ptr(grad_output), _ptr(weight), _ptr(d_w),
+                                       _ptr(d_b), features.size(0), n_in, n_out, _stream()))
+        return d_in, d_w, d_b
+
+    def batchNormTrain(self, features, running_mean, running_var, weight, bias, eps, momentum, leakiness):
+        """Training-mode forward: (output, saved mean, saved 1/std); running statistics updated in place."""
+        features = _features(features, "features")
+        out = torch.empty_like(features)
+        planes = features.size(1)
+        save_mean = torch.empty(planes, dtype=torch.float32, device=features.device)
+        save_invstd = torch.empty(planes, dtype=torch.float32, device=features.device)
+        w = weight if weight is not None and weight.numel() else None
+        b = bias if bias is not None and bias.numel() else None
+        _lib.check(self._L.scn_bn_train_fwd(self._h, _ptr(features), _ptr(out), features.size(0), planes,
+                                            features.stride(0), out.stride(0), _ptr(save_mean), _ptr(save_invstd),
+                                            _ptr(running_mean), _ptr(running_var), _ptr(w), _ptr(b), float(eps),
+                                            float(momentum), float(leakiness), _stream()))
+        return out, save_mean, save_invstd
+
+    def batchNormBackward(self, features, output, grad_output, save_mean, save_invstd, weight, leakiness, affine):
+        features = _features(features, "features")
+        grad_output = _features(grad_output, "grad_output")
+        planes = features.size(1)
+        d_in = torch.empty_like(features)
+        d_w = torch.empty(planes, dtype=torch.float32, device=features.device) if affine else None
+        d_b = torch.empty(planes, dtype=torch.float32, device=features.device) if affine else None
+        w = weight if weight is not None and weight.numel() else None
+        _lib.check(self._L.scn_bn_bwd(self._h, _ptr(features), _ptr(d_in), _ptr(output), _ptr(grad_output),
+                                      features.size(0), planes, features.stride(0), output.stride(0), _ptr(save_mean),
+                                      _ptr(save_invstd), _ptr(w), _ptr(d_w), _ptr(d_b), float(leakiness), _stream()))
+        return d_in, d_w, d_b
+
+    def maxPoolingBackward(self, in_size, out_size, pool_size, pool_stride, features, output, grad_output,
+                           n_features_to_drop):
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        features = _features(features, "features")
+        grad_output = _features(grad_output, "grad_output")
+        d_in = torch.empty_like(features)
+        if features.size(0):
+            _lib.check(self._L.scn_maxpool_bwd(self._h, *a, _ptr(features), _ptr(d_in), features.size(1), _ptr(output),
+                                               _ptr(grad_output), output.size(1), n_features_to_drop, _stream()))
+        return d_in
+
+    def averagePoolingBackward(self, in_size, out_size, pool_size, pool_stride, input_shape, grad_output,
+                               n_features_to_drop):
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        grad_output = _features(grad_output, "grad_output")
+        d_in = torch.empty(tuple(input_shape), dtype=torch.float32, device=grad_output.device)
+        if d_in.size(0):
+            _lib.check(self._L.scn_avgpool_bwd(self._h, *a, _ptr(d_in), d_in.size(1), _ptr(grad_output),
+                                               grad_output.size(1), n_features_to_drop, _stream()))
+        return d_in
+
+    def unPoolingBackward(self, in_size, out_size, pool_size, pool_stride, input_shape, grad_output,
+                          n_features_to_drop):
+        a = [self._s(v) for v in (in_size, out_size, pool_size, pool_stride)]
+        grad_output = _features(grad_output, "grad_output")
+        d_in = torch.empty(tuple(input_shape), dtype=torch.float32, device=grad_output.device)
+        if d_in.size(0):
+            _lib.check(self._L.scn_unpool_bwd(self._h, *a, _ptr(d_in), d_in.size(1), _ptr(grad_output),
+                                              grad_output.size(1), n_features_to_drop, _stream()))
+        return d_in
+
+    def inputLayerBackward(self, grad_output, bl=False):
+        """d(features of the points) from d(features of the sites); bl: [batch, length, planes]."""
+        grad_output = _features(grad_output, "grad_output")
+        planes = grad_output.size(1)
+        if bl:
+            hdr = (C.c_int32 * 5)()
+            _lib.check(self._L.scn_md_bl_rules_header(self._h, hdr))
+            d_in = torch.empty((hdr[2], hdr[3], planes), dtype=torch.float32, device=grad_output.device)
+        else:
+            hdr = (C.c_int32 * 4)()
+            _lib.check(self._L.scn_md_input_rules_header(self._h, hdr))
+            d_in = torch.empty((hdr[2], planes), dtype=torch.float32, device=grad_output.device)
+        if d_in.numel():
+            _lib.check(self._L.scn_input_layer_bwd(self._h, _ptr(d_in), _ptr(grad_output), planes, _stream()))
+        return d_in
+
+    def outputLayerBackward(self, grad_output, n_active):
+        """d(features of the sites) from d(features of the points) ([points, planes] or [batch, length, planes])."""
+        grad_output = _features(grad_output, "grad_output")
+        planes = grad_output.size(-1)
+        d_in = torch.empty((n_active, planes), dtype=torch.float32, device=grad_output.device)
+        if d_in.numel():
+            _lib.check(self._L.scn_output_layer_bwd(self._h, _ptr(d_in), _ptr(grad_output), planes, _stream()))
+        return d_in
+
+    def sparseToDenseBackward(self, spatial_size, grad_output, n_active):
+        grad_output = _features(grad_output, "grad_output")
+        d_in = torch.empty((n_active, grad_output.size(1)), dtype=torch.float32, device=grad_output.device)
+        if d_in.numel():
+            _lib.check(self._L.scn_s2d_bwd(self._h, self._s(spatial_size), _ptr(d_in), _ptr(grad_output),
+                                           grad_output.size(1), _stream()))
+        return d_in
+
+
 def batchNormEval(features, running_mean, running_var, weight, bias, eps, leakiness):
     features = _features(features, "features")
     out = torch.empty_like(features)

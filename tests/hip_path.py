@@ -309,3 +309,116 @@ class HipPath:
         _lib.check(self.L.scn_s2d_fwd(self.h, self._s(spatial), _ptr(xd), _ptr(out), x.shape[1],
                                       _stream()))
         return out.cpu().numpy()
+
+    # -- backward ops (same interface as oracle.cpu_path.CpuPath) ------------------------------
+    def _conv_bwd(self, fn, sizes, n_in_rows, x, d_out, w, with_bias):
+        groups = w.shape[1]
+        n_in, n_out = w.shape[2] * groups, w.shape[3] * groups
+        xd, dd, wd = _dev(x, torch.float32), _dev(d_out, torch.float32), _dev(w, torch.float32)
+        d_in = torch.full((n_in_rows, n_in), float("nan"), dtype=torch.float32, device="cuda")
+        d_w = torch.full_like(wd, float("nan"))
+        d_b = torch.full((n_out,), float("nan"), dtype=torch.float32, device="cuda") if with_bias else None
+        _lib.check(fn(self.h, *sizes, _ptr(xd), _ptr(d_in), _ptr(dd), _ptr(wd), _ptr(d_w), _ptr(d_b), n_in, n_out,
+                      groups, _stream()))
+        return d_in.cpu().numpy(), d_w.cpu().numpy(), (d_b.cpu().numpy() if with_bias else None)
+
+    def subm_conv_bwd(self, spatial, filter_size, x, d_out, w, with_bias=False):
+        sizes = (self._s(spatial), self._s(filter_size))
+        return self._conv_bwd(self.L.scn_subm_conv_bwd, sizes, self.nactive(spatial), x, d_out, w, with_bias)
+
+    def conv_bwd(self, in_size, out_size, filter_size, stride, x, d_out, w, with_bias=False):
+        sizes = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        return self._conv_bwd(self.L.scn_conv_bwd, sizes, self.nactive(in_size), x, d_out, w, with_bias)
+
+    def deconv_bwd(self, in_size, out_size, filter_size, stride, x, d_out, w, with_bias=False):
+        sizes = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
+        return self._conv_bwd(self.L.scn_deconv_bwd, sizes, self.nactive(in_size), x, d_out, w, with_bias)
+
+    def nin_bwd(self, x, d_out, w, with_bias=False):
+        xd, dd, wd = _dev(x, torch.float32), _dev(d_out, torch.float32), _dev(w, torch.float32)
+        d_in, d_w = torch.full_like(xd, float("nan")), torch.full_like(wd, float("nan"))
+        d_b = torch.full((w.shape[1],), float("nan"), dtype=torch.float32, device="cuda") if with_bias else None
+        _lib.check(self.L.scn_nin_bwd(self.h, _ptr(xd), _ptr(d_in), _ptr(dd), _ptr(wd), _ptr(d_w), _ptr(d_b), x.shape[0],
+                                      w.shape[0], w.shape[1], _stream()))
+        return d_in.cpu().numpy(), d_w.cpu().numpy(), (d_b.cpu().numpy() if with_bias else None)
+
+    def bn_train(self, x, running_mean, running_var, weight=None, bias=None, eps=1e-4, momentum=0.99, leakiness=1.0):
+        xd = _dev(x, torch.float32)
+        out = torch.full_like(xd, float("nan"))
+        C_ = x.shape[1]
+        sm, si = torch.zeros(C_, device="cuda"), torch.zeros(C_, device="cuda")
+        rm, rv = _dev(running_mean, torch.float32).clone(), _dev(running_var, torch.float32).clone()
+        gd = _dev(weight, torch.float32) if weight is not None else None
+        bd = _dev(bias, torch.float32) if bias is not None else None
+        _lib.check(self.L.scn_bn_train_fwd(self.h, _ptr(xd), _ptr(out), x.shape[0], C_, C_, C_, _ptr(sm), _ptr(si), _ptr(rm),
+                                           _ptr(rv), _ptr(gd), _ptr(bd), eps, momentum, leakiness, _stream()))
+        return tuple(t.cpu().numpy() for t in (out, sm, si, rm, rv))
+
+    def bn_bwd(self, x, out, d_out, save_mean, save_invstd, weight=None, leakiness=1.0, affine=True):
+        xd, od, dd = _dev(x, torch.float32), _dev(out, torch.float32), _dev(d_out, torch.float32)
+        C_ = x.shape[1]
+        d_in = torch.full_like(xd, float("nan"))
+        d_w = torch.full((C_,), float("nan"), device="cuda") if affine else None
+        d_b = torch.full((C_,), float("nan"), device="cuda") if affine else None
+        gd = _dev(weight, torch.float32) if weight is not None else None
+        sm, si = _dev(save_mean, torch.float32), _dev(save_invstd, torch.float32)
+        _lib.check(self.L.scn_bn_bwd(self.h, _ptr(xd), _ptr(d_in), _ptr(od), _ptr(dd), x.shape[0], C_, C_, C_, _ptr(sm),
+                                     _ptr(si), _ptr(gd), _ptr(d_w), _ptr(d_b), leakiness, _stream()))
+        return d_in.cpu().numpy(), (d_w.cpu().numpy() if affine else None), (d_b.cpu().numpy() if affine else None)
+
+    def maxpool_bwd(self, in_size, out_size, size, stride, x, out, d_out, n_features_to_drop=0):
+        sizes = [self._s(v) for v in (in_size, out_size, size, stride)]
+        xd, od, dd = _dev(x, torch.float32), _dev(out, torch.float32), _dev(d_out, torch.float32)
+        d_in = torch.full_like(xd, float("nan"))
+        _lib.check(self.L.scn_maxpool_bwd(self.h, *sizes, _ptr(xd), _ptr(d_in), x.shape[1], _ptr(od), _ptr(dd),
+                                          out.shape[1], n_features_to_drop, _stream()))
+        return d_in.cpu().numpy()
+
+    def _pool_bwd(self, fn, in_size, out_size, size, stride, in_planes, d_out, n_features_to_drop):
+        sizes = [self._s(v) for v in (in_size, out_size, size, stride)]
+        dd = _dev(d_out, torch.float32)
+        d_in = torch.full((self.nactive(in_size), in_planes), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(fn(self.h, *sizes, _ptr(d_in), in_planes, _ptr(dd), d_out.shape[1], n_features_to_drop, _stream()))
+        return d_in.cpu().numpy()
+
+    def avgpool_bwd(self, in_size, out_size, size, stride, in_planes, d_out, n_features_to_drop=0):
+        return self._pool_bwd(self.L.scn_avgpool_bwd, in_size, out_size, size, stride, in_planes, d_out,
+                              n_features_to_drop)
+
+    def unpool_bwd(self, in_size, out_size, size, stride, in_planes, d_out, n_features_to_drop=0):
+        return self._pool_bwd(self.L.scn_unpool_bwd, in_size, out_size, size, stride, in_planes, d_out,
+                              n_features_to_drop)
+
+    def input_bwd(self, d_out):
+        hdr = self._hdr()
+        dd = _dev(d_out, torch.float32)
+        d_in = torch.full((hdr[2], d_out.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_input_layer_bwd(self.h, _ptr(d_in), _ptr(dd), d_out.shape[1], _stream()))
+        return d_in.cpu().numpy()
+
+    def output_bwd(self, d_out):
+        hdr = self._hdr()
+        dd = _dev(d_out, torch.float32)
+        d_in = torch.full((hdr[3], d_out.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_output_layer_bwd(self.h, _ptr(d_in), _ptr(dd), d_out.shape[1], _stream()))
+        return d_in.cpu().numpy()
+
+    def bl_input_bwd(self, d_out):
+        hdr, _ = self.bl_rules()
+        dd = _dev(d_out, torch.float32)
+        d_in = torch.full((int(hdr[2]), int(hdr[3]), d_out.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_input_layer_bwd(self.h, _ptr(d_in), _ptr(dd), d_out.shape[1], _stream()))
+        return d_in.cpu().numpy()
+
+    def bl_output_bwd(self, d_out):
+        hdr, _ = self.bl_rules()
+        dd = _dev(np.ascontiguousarray(d_out.reshape(-1, d_out.shape[-1])), torch.float32)
+        d_in = torch.full((int(hdr[4]), d_out.shape[-1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_output_layer_bwd(self.h, _ptr(d_in), _ptr(dd), d_out.shape[-1], _stream()))
+        return d_in.cpu().numpy()
+
+    def s2d_bwd(self, spatial, d_out):
+        dd = _dev(d_out, torch.float32)
+        d_in = torch.full((self.nactive(spatial), d_out.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_s2d_bwd(self.h, self._s(spatial), _ptr(d_in), _ptr(dd), d_out.shape[1], _stream()))
+        return d_in.cpu().numpy()

@@ -1,0 +1,117 @@
+"""Backward pass of the HIP library through its C ABI: the independent checks of tests/checks.py
+(torch.autograd through the dense equivalents) and the CPU oracle on the same seeded inputs over
+every kernel family's channel range.  Gradients within 1e-4 relative / 1e-5 absolute (fp32)."""
+import numpy as np
+import pytest
+
+import checks
+from oracle import cpu_path
+from oracle.cpu_path import canon_rows
+from sparseconvnet_amd import synthetic
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def make():
+    import torch
+    assert torch.cuda.is_available()
+    from hip_path import HipPath
+    return lambda dim: HipPath(dim)
+
+
+@pytest.mark.parametrize("dim,size", [(1, 3), (2, 3), (3, 3), (3, 2), (2, (3, 1)), (4, 3)])
+def test_conv_backward(make, dim, size):
+    checks.check_conv_backward(make, dim, size, seed=30 + dim, spatial=8 if dim < 4 else 5, bias=(dim != 2))
+
+
+@pytest.mark.parametrize("dim,size,stride", [(3, 2, 2), (3, 3, 2), (2, 3, 2), (2, 2, 2), (1, 3, 2), (2, (3, 2), (2, 1))])
+def test_strided_backward(make, dim, size, stride):
+    checks.check_strided_backward(make, dim, size, stride, seed=40 + dim)
+
+
+def test_bn_train(make):
+    checks.check_bn_train(make, seed=50)
+    checks.check_bn_train(make, seed=51, n=5000, C=96)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+def test_io_backward(make, mode):
+    checks.check_io_backward(make, 3, mode, seed=60 + mode)
+    checks.check_bl_backward(make, 2, mode, seed=65 + mode)
+
+
+def test_misc_backward(make):
+    checks.check_misc_backward(make, seed=70)
+
+
+@pytest.mark.parametrize("cin,cout,groups", [(3, 32, 1), (32, 32, 1), (16, 16, 1), (64, 64, 1), (96, 128, 1),
+                                             (128, 160, 1), (256, 256, 1), (30, 50, 1), (8, 12, 2), (64, 32, 1)])
+def test_conv_gradients_vs_oracle(oracle_built, cin, cout, groups):
+    """Submanifold, strided and transposed convolution gradients on a 20,000-site room scene
+    against the oracle, over the channel ranges of every forward kernel family (the input
+    gradient runs through them) and of the weight-gradient kernel's tiles."""
+    from hip_path import HipPath
+    g, o = HipPath(3), cpu_path.CpuPath(3, "oracle")
+    coords = synthetic.room_scene(seed=4200, target=20000, spatial=126, duplicate_fraction=0.0)
+    rng = np.random.default_rng(cin * 1000 + cout)
+    x = rng.normal(size=(len(coords), cin)).astype(np.float32)
+    for p in (g, o):
+        assert p.input_layer(126, coords, 0, 3) == len(coords)
+        p.strided_rules(126, 63, 2, 2)
+    lg, lo = g.spatial_locations(63), o.spatial_locations(63)
+    rg, ro = canon_rows(lg), canon_rows(lo)
+
+    def w(k, a, b):
+        return (rng.normal(size=(k, groups, a // groups, b // groups)) * (2.0 / (a * k)) ** 0.5).astype(np.float32)
+    w_s, w_d, w_u = w(27, cin, cout), w(8, cin, cout), w(8, cout, cin)
+    d_y = rng.normal(size=(len(coords), cout)).astype(np.float32)
+    got, want = g.subm_conv_bwd(126, 3, x, d_y, w_s, True), o.subm_conv_bwd(126, 3, x, d_y, w_s, True)
+    for a, b, what in zip(got, want, ("d_input", "d_weight", "d_bias")):
+        checks.assert_close(a, b, "submanifold " + what)
+    # strided: the coarse level's rows are numbered differently on the two sides
+    d_c = rng.normal(size=(len(lo), cout)).astype(np.float32)
+    d_cg = np.empty_like(d_c)
+    d_cg[rg] = d_c[ro]
+    got, want = g.conv_bwd(126, 63, 2, 2, x, d_cg, w_d, True), o.conv_bwd(126, 63, 2, 2, x, d_c, w_d, True)
+    for a, b, what in zip(got, want, ("d_input", "d_weight", "d_bias")):
+        checks.assert_close(a, b, "strided " + what)
+    xc = rng.normal(size=(len(lo), cout)).astype(np.float32)
+    xg = np.empty_like(xc)
+    xg[rg] = xc[ro]
+    d_f = rng.normal(size=(len(coords), cin)).astype(np.float32)
+    got, want = g.deconv_bwd(63, 126, 2, 2, xg, d_f, w_u, True), o.deconv_bwd(63, 126, 2, 2, xc, d_f, w_u, True)
+    checks.assert_close(got[0][rg], want[0][ro], "transposed d_input")
+    checks.assert_close(got[1], want[1], "transposed d_weight")
+    checks.assert_close(got[2], want[2], "transposed d_bias")
+
+
+def test_pooling_and_nin_gradients_vs_oracle(oracle_built):
+    from hip_path import HipPath
+    g, o = HipPath(3), cpu_path.CpuPath(3, "oracle")
+    coords = synthetic.room_scene(seed=4300, target=30000, spatial=127, duplicate_fraction=0.2)
+    rng = np.random.default_rng(43)
+    f = rng.normal(size=(len(coords), 32)).astype(np.float32)
+    res = []
+    for p in (g, o):
+        p.input_layer(127, coords, 0, 4)
+        x = p.input_fwd(f)
+        p.strided_rules(127, 63, 3, 2)
+        l1 = p.spatial_locations(63)
+        r1 = canon_rows(l1)
+        mp = p.maxpool(127, 63, 3, 2, x)
+        d = np.empty_like(mp)
+        d[r1] = np.random.default_rng(44).normal(size=mp.shape).astype(np.float32)
+        res.append(dict(x=x, mp=mp[r1], d_max=p.maxpool_bwd(127, 63, 3, 2, x, mp, d),
+                        d_avg=p.avgpool_bwd(127, 63, 3, 2, 32, d), d_avg4=p.avgpool_bwd(127, 63, 3, 2, 36, d, 4),
+                        d_in=p.input_bwd(x), d_outl=p.output_bwd(f)))
+        up_d = np.random.default_rng(45).normal(size=(len(x), 32)).astype(np.float32)
+        res[-1]["d_un"] = p.unpool_bwd(63, 127, 3, 2, 32, up_d)[r1]
+    for k in res[0]:
+        checks.assert_close(res[0][k], res[1][k], k)
+    for rows, cin, cout in ((70000, 64, 32), (5000, 256, 256), (777, 33, 17)):
+        a = rng.normal(size=(rows, cin)).astype(np.float32)
+        w = (rng.normal(size=(cin, cout)) * 0.1).astype(np.float32)
+        d = rng.normal(size=(rows, cout)).astype(np.float32)
+        for u, v, what in zip(g.nin_bwd(a, d, w, True), o.nin_bwd(a, d, w, True), ("d_input", "d_weight", "d_bias")):
+            checks.assert_close(u, v, "network in network %s %dx%d" % (what, cin, cout))

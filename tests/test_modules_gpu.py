@@ -165,16 +165,126 @@ def test_vgg2d_vs_oracle(oracle_built):
     checks.assert_close(got.cpu().numpy(), want, "2-D VGG dense output")
 
 
-def test_training_mode_and_backward_are_refused():
-    bn = scn.BatchNormReLU(4).cuda()
-    t = scn.InputLayer(2, 8)([torch.LongTensor([[1, 1, 0]]), torch.ones(1, 4).cuda()])
-    with pytest.raises(NotImplementedError):
-        bn(t)  # training mode
-    conv = scn.SubmanifoldConvolution(2, 4, 4, 3, False).cuda()
-    y = conv(t).features
-    assert y.requires_grad
-    with pytest.raises((NotImplementedError, RuntimeError)):
-        y.sum().backward()
+def test_eval_mode_batch_norm_refuses_backward():
+    """batchNormalization.py:147 asserts ctx.train in backward; so does this build, also when the
+    eval-mode batch norm was applied inside a convolution."""
+    bn = scn.BatchNormReLU(4).cuda().eval()
+    feats = torch.ones(3, 4).cuda().requires_grad_()
+    t = scn.InputLayer(2, 8)([torch.LongTensor([[1, 1, 0], [2, 2, 0], [5, 5, 0]]), feats])
+    with pytest.raises(AssertionError):
+        bn(t).features.sum().backward()
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(2, 4, 4, 3, False)).add(scn.BatchNormReLU(4)).cuda().eval()
+    with pytest.raises(AssertionError):
+        model(t).features.sum().backward()
+
+
+def test_module_chain_gradients_vs_oracle(oracle_built):
+    """A chain of every differentiable module in training mode (InputLayer mode 4, submanifold
+    convolution with bias, BatchNormReLU, strided convolution, BatchNormLeakyReLU, max and average
+    pooling side branches, transposed convolution, NetworkInNetwork, OutputLayer): the gradients
+    torch.autograd collects through this build's Functions against the same chain walked backwards
+    by hand with the oracle's backward calls."""
+    torch.manual_seed(31)
+    rng = np.random.default_rng(31)
+    coords = synthetic.room_scene(seed=3100, target=3000, spatial=30, duplicate_fraction=0.3)
+    feats = rng.normal(size=(len(coords), 3)).astype(np.float32)
+    conv1 = scn.SubmanifoldConvolution(3, 3, 8, 3, True).cuda()
+    bn1 = scn.BatchNormReLU(8).cuda()
+    down = scn.Convolution(3, 8, 12, 2, 2, False).cuda()
+    bn2 = scn.BatchNormLeakyReLU(12, leakiness=0.2).cuda()
+    up = scn.Deconvolution(3, 12, 8, 2, 2, True).cuda()
+    nin = scn.NetworkInNetwork(8, 5, True).cuda()
+    mp, ap, unp = scn.MaxPooling(3, 2, 2).cuda(), scn.AveragePooling(3, 2, 2).cuda(), scn.UnPooling(3, 2, 2).cuda()
+    with torch.no_grad():
+        conv1.bias.normal_()
+        up.bias.normal_()
+        nin.bias.normal_()
+        for b in (bn1, bn2):
+            b.weight.uniform_(0.5, 1.5)
+            b.bias.normal_()
+    mods = [conv1, bn1, down, bn2, up, nin]
+    for m in mods:
+        m.train()
+    f = torch.as_tensor(feats).cuda().requires_grad_()
+    x0 = scn.InputLayer(3, 30, mode=4)([torch.as_tensor(coords), f])
+    h1 = bn1(conv1(x0))
+    h2 = bn2(down(h1))
+    pooled = scn.AddTable()([mp(h1), ap(h1), scn.Identity()(mp(h1))])  # max pooling counted twice
+    side = unp(pooled)
+    y = nin(scn.AddTable()([up(h2), side]))
+    out = scn.OutputLayer(3)(y)
+    g_out = torch.as_tensor(rng.normal(size=tuple(out.shape)).astype(np.float32)).cuda()
+    (out * g_out).sum().backward()
+
+    # the same chain on the oracle, forwards and then backwards by hand
+    o = cpu_path.CpuPath(3, "oracle")
+    P = lambda t: t.detach().cpu().numpy()
+    o.input_layer(30, coords, 0, 4)
+    a0 = o.input_fwd(feats)
+    a1, _ = o.subm_conv(30, 3, a0, P(conv1.weight), P(conv1.bias))
+    b1, sm1, si1, _, _ = o.bn_train(a1, np.zeros(8), np.ones(8), P(bn1.weight), P(bn1.bias), 1e-4, 0.99, 0.0)
+    a2, _ = o.conv(30, 15, 2, 2, b1, P(down.weight))
+    b2, sm2, si2, _, _ = o.bn_train(a2, np.zeros(12), np.ones(12), P(bn2.weight), P(bn2.bias), 1e-4, 0.99, 0.2)
+    m1, v1 = o.maxpool(30, 15, 2, 2, b1), o.avgpool(30, 15, 2, 2, b1)
+    pooled_o = m1 + v1 + m1
+    side_o = o.unpool(15, 30, 2, 2, pooled_o)
+    a3, _ = o.deconv(15, 30, 2, 2, b2, P(up.weight), P(up.bias))
+    s3 = a3 + side_o
+    yo, _ = o.nin(s3, P(nin.weight), P(nin.bias))
+    checks.assert_close(P(out), o.output_fwd(yo), "forward of the chain")
+    d_y = o.output_bwd(P(g_out))
+    d_s3, d_wn, d_bn = o.nin_bwd(s3, d_y, P(nin.weight), True)
+    d_b2, d_wu, d_bu = o.deconv_bwd(15, 30, 2, 2, b2, d_s3, P(up.weight), True)
+    d_pooled = o.unpool_bwd(15, 30, 2, 2, 8, d_s3)
+    d_b1 = 2 * o.maxpool_bwd(30, 15, 2, 2, b1, m1, d_pooled) + o.avgpool_bwd(30, 15, 2, 2, 8, d_pooled)
+    d_a2, d_g2, d_be2 = o.bn_bwd(a2, b2, d_b2, sm2, si2, P(bn2.weight), 0.2)
+    d_b1c, d_wd, _ = o.conv_bwd(30, 15, 2, 2, b1, d_a2, P(down.weight))
+    d_b1 = d_b1 + d_b1c
+    d_a1, d_g1, d_be1 = o.bn_bwd(a1, b1, d_b1, sm1, si1, P(bn1.weight), 0.0)
+    d_a0, d_w1, d_bias1 = o.subm_conv_bwd(30, 3, a0, d_a1, P(conv1.weight), True)
+    d_f = o.input_bwd(d_a0)
+    # (the gradients compared below do not depend on how either side numbers the coarse rows)
+    for got, want, what in ((f.grad, d_f, "input features"), (conv1.weight.grad, d_w1, "conv1 weight"),
+                            (bn1.weight.grad, d_g1, "bn1 weight"),
+                            (bn1.bias.grad, d_be1, "bn1 bias"), (down.weight.grad, d_wd, "strided weight"),
+                            (bn2.weight.grad, d_g2, "bn2 weight"), (bn2.bias.grad, d_be2, "bn2 bias"),
+                            (up.weight.grad, d_wu, "transposed weight"), (up.bias.grad, d_bu, "transposed bias"),
+                            (nin.weight.grad, d_wn, "nin weight"), (nin.bias.grad, d_bn, "nin bias")):
+        checks.assert_close(P(got), want, "gradient of " + what)
+    # a bias in front of a training-mode batch norm has gradient zero: both sides hold the rounding
+    # noise of a column sum that cancels, so the bound is relative to the summands
+    assert (np.abs(P(conv1.bias.grad) - d_bias1) <= 1e-6 * np.abs(d_a1).sum(0)).all()
+    assert (np.abs(d_bias1) <= 1e-6 * np.abs(d_a1).sum(0)).all()
+    # running statistics moved towards the batch's (momentum 0.99 weights the old value)
+    checks.assert_close(P(bn1.running_mean), 0.01 * a1.astype(np.float64).mean(0), "running mean")
+
+
+def test_unet_trains():
+    """A small U-Net (residual blocks, training-mode batch norms, JoinTable / AddTable through
+    torch) fits a toy per-point regression target: gradients reach every parameter and the loss
+    falls under plain SGD."""
+    torch.manual_seed(32)
+    m = 8
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 1, [m, 2 * m, 3 * m], True)).add(scn.BatchNormReLU(m)).add(scn.OutputLayer(3)).cuda().train()
+    head = torch.nn.Linear(m, 1).cuda()
+    coords = synthetic.room_scene(seed=3200, target=4000, spatial=64, duplicate_fraction=0.2)
+    feats = torch.rand((len(coords), 3), device="cuda")
+    target = (torch.as_tensor(coords[:, 2:3]).float().cuda() / 64.0)
+    params = list(model.parameters()) + list(head.parameters())
+    opt = torch.optim.SGD(params, lr=0.05, momentum=0.9)
+    layer = scn.InputLayer(3, 64, mode=4)
+    losses = []
+    for step in range(12):
+        opt.zero_grad()
+        pred = head(model(layer([torch.as_tensor(coords), feats])))
+        loss = ((pred - target) ** 2).mean()
+        loss.backward()
+        if step == 0:
+            assert all(p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().sum() > 0 for p in params)
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < 0.5 * losses[0], losses
 
 
 def test_empty_input_passes_through():
