@@ -113,38 +113,6 @@ template <bool PRE> __device__ inline v4f pre_act(v4f v, v4f sc, v4f sh, float l
   y.w *= (y.w > 0.f ? 1.f : leak);
   return y;
 }
-// What happens to an accumulated output value before it is stored: + bias, then optionally the
-// eval batch norm + leaky ReLU of the layer that follows (folded to scale / shift per output
-// channel), so that layer needs no pass of its own.
-struct Epi {
-  const float *bias = nullptr;               // [nOut] or null
-  const float *sc = nullptr, *sh = nullptr;  // [nOut] each, or nulls
-  float leak = 1.0f;
-};
-__device__ inline float epi_act(float v, float sc, float sh, float leak) {
-  const float y = v * sc + sh;
-  return y > 0.f ? y : y * leak;
-}
-// Folding a batch norm to scale / shift (sc[c] = gamma / sqrt(var + eps), sh[c] = beta -
-// mean * sc, zeros from n to n_pad) is a few hundred values: the weight-packing launch that
-// precedes every MFMA convolution does it on the side (its first workgroup), so it costs no
-// launch of its own.  CoefJobs lives in metadata.h.
-__device__ inline void coef_job(const CoefJob &j) {
-  for (int c = threadIdx.x; c < j.n_pad; c += blockDim.x) {
-    float w = 0.f, b = 0.f;
-    if (c < j.n) {
-      w = (1.0f / sqrtf(j.var[c] + j.eps)) * (j.gamma ? j.gamma[c] : 1.0f);
-      b = -j.mean[c] * w + (j.beta ? j.beta[c] : 0.0f);
-    }
-    j.sc[c] = w;
-    j.sh[c] = b;
-  }
-}
-__device__ inline void coef_jobs(const CoefJobs &jobs) {
-  if (blockIdx.x != 0) return;
-  if (jobs.pre.n_pad) coef_job(jobs.pre);
-  if (jobs.post.n_pad) coef_job(jobs.post);
-}
 __global__ void k_coefs(CoefJobs jobs) { coef_jobs(jobs); }
 // Hands the pending jobs to the launch being prepared (and forgets them).
 static CoefJobs take_jobs(Metadata &m) {
@@ -1353,6 +1321,11 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
 template <int NCB>
 static void launch_resident_c4(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                                Epi epi, int n_in, int n_out, hipStream_t s) {
+  if (in == m.cur_in_base && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
+    // epi.sc / epi.sh point at arrays nobody fills on this path: the kernel folds the batch norm itself
+    conv_first_forward(t, in, m.cur_in_rows, out, w, epi.bias, take_jobs(m).post, epi.leak, n_in, n_out, s);
+    return;
+  }
   const int packed = t.K * NCB * 64;
   float *wpack = scratch_wpack(m, packed);
   k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, NCB,

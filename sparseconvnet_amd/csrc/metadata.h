@@ -218,6 +218,45 @@ std::vector<int64_t> s2d_sizes(Metadata &m, const int64_t *spatial, hipStream_t 
 int64_t export_s2d_pairs(Metadata &m, const int64_t *spatial, int sample, int *pairs,
                          hipStream_t s);
 
+// What happens to an accumulated output value before it is stored: + bias, then optionally the
+// eval batch norm + leaky ReLU of the layer that follows (folded to scale / shift per output
+// channel), so that layer needs no pass of its own.
+struct Epi {
+  const float *bias = nullptr;               // [nOut] or null
+  const float *sc = nullptr, *sh = nullptr;  // [nOut] each, or nulls
+  float leak = 1.0f;
+};
+__device__ inline float epi_act(float v, float sc, float sh, float leak) {
+  const float y = v * sc + sh;
+  return y > 0.f ? y : y * leak;
+}
+// Folding a batch norm to scale / shift (sc[c] = gamma / sqrt(var + eps), sh[c] = beta -
+// mean * sc, zeros from n to n_pad) is a few hundred values: the weight-packing launch that
+// precedes every MFMA convolution does it on the side (its first workgroup), so it costs no
+// launch of its own.  CoefJobs lives in metadata.h.
+__device__ inline void coef_job(const CoefJob &j) {
+  for (int c = threadIdx.x; c < j.n_pad; c += blockDim.x) {
+    float w = 0.f, b = 0.f;
+    if (c < j.n) {
+      w = (1.0f / sqrtf(j.var[c] + j.eps)) * (j.gamma ? j.gamma[c] : 1.0f);
+      b = -j.mean[c] * w + (j.beta ? j.beta[c] : 0.0f);
+    }
+    j.sc[c] = w;
+    j.sh[c] = b;
+  }
+}
+__device__ inline void coef_jobs(const CoefJobs &jobs) {
+  if (blockIdx.x != 0) return;
+  if (jobs.pre.n_pad) coef_job(jobs.pre);
+  if (jobs.post.n_pad) coef_job(jobs.post);
+}
+// conv_first.hip: the convolution kernel for nIn <= 4, nOut <= 32 and up to 32 taps; it reads the
+// weights as the caller holds them and folds the batch norm behind the convolution itself
+// (bn.n == 0: none), so it needs no scratch.  in_rows: rows of the input matrix that starts at `in`.
+bool conv_first_serves(const Table &t, int64_t in_rows, int n_in, int n_out);
+void conv_first_forward(const Table &t, const float *in, int64_t in_rows, float *out, const float *w, const float *bias,
+                        CoefJob bn, float leak, int n_in, int n_out, hipStream_t s);
+
 // ops.hip / conv.hip
 unsigned char *noalloc_scratch();  // the static scratch array's address on the current device
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);
