@@ -177,6 +177,13 @@ int scn_release_cache(void);
 int scn_cache_stats(int64_t *live_bytes, int64_t *idle_bytes, int64_t *peak_bytes,
                     int64_t *device_allocations);
 
+/* The sort the rulebook builders use, by itself (for tests and measurement): a stable sort of
+ * n (64-bit key, 32-bit value) pairs, device arrays, by the low end_bit bits of the key; the
+ * input arrays are not written, scratch comes from the handle.  The reference keeps its sites
+ * in hash maps and has no such step (Metadata/Metadata.h:22-33). */
+int scn_sort_pairs(scn_metadata *md, const unsigned long long *keys_in, unsigned long long *keys_out,
+                   const int *values_in, int *values_out, int64_t n, int end_bit, void *stream);
+
 /* InputLayer_updateOutput after the rules exist (pybind.cpp:155-159, CPU/IOLayers.cpp:49-72):
  * in [nInputRows, planes] -> out [nActive, planes]. */
 int scn_input_layer_fwd(scn_metadata *md, const float *in, float *out, int planes, void *stream);

@@ -659,6 +659,14 @@ int scn_cache_stats(int64_t *live_bytes, int64_t *idle_bytes, int64_t *peak_byte
     if (device_allocations) *device_allocations = g_mallocs;
   });
 }
+int scn_sort_pairs(scn_metadata *h, const unsigned long long *keys_in, unsigned long long *keys_out, const int *values_in,
+                   int *values_out, int64_t n, int end_bit, void *stream) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (n < 0 || end_bit < 1 || end_bit > 64) throw Error("sort: n must not be negative, end_bit in 1..64");
+    radix_sort_pairs(m, keys_in, keys_out, values_in, values_out, n, end_bit, static_cast<hipStream_t>(stream));
+  });
+}
 int scn_rules_sizes(scn_metadata *h, int kind, const int64_t *a, const int64_t *b, const int64_t *c,
                     const int64_t *d, void *stream, int64_t *sizes) {
   return guarded([&] {

@@ -257,6 +257,11 @@ bool conv_first_serves(const Table &t, int64_t in_rows, int n_in, int n_out);
 void conv_first_forward(const Table &t, const float *in, int64_t in_rows, float *out, const float *w, const float *bias,
                         CoefJob bn, float leak, int n_in, int n_out, hipStream_t s);
 
+// sort.hip: stable radix sort of (key, value) pairs by the low end_bit bits of the key; the input
+// arrays are left as they are, scratch comes from m.tmp.
+void radix_sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout, const int *vin, int *vout,
+                      int64_t n, int end_bit, hipStream_t s);
+
 // ops.hip / conv.hip
 unsigned char *noalloc_scratch();  // the static scratch array's address on the current device
 void fill32(void *p, uint32_t v, int64_t n, hipStream_t s);

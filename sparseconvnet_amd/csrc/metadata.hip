@@ -150,30 +150,31 @@ static void fill3(void *p0, uint32_t v0, int64_t n0, void *p1, uint32_t v1, int6
   LAUNCH_CHECK();
 }
 
-// Stable sort of (key, value) pairs by the low end_bit bits of the key.  The library's default
-// takes a merge sort up to a million items, whatever the number of key bits: log2(n / block)
-// passes.  The tables sorted here have few key bits (a tap pattern and a window number), so
-// from a few ten thousand rows on the radix sort's end_bit / 8 passes are fewer, and it is
-// chosen by hand.
+// Stable sort of (key, value) pairs by the low end_bit bits of the key.  From 32 k to 1.5 million pairs
+// this repository's own sort (sort.hip: three short launches per digit, measured 95-145 us for a
+// million pairs of 35 bits against the library's 175 us, 50-80 us against 100-150 us at 15 k to
+// 250 k pairs); above, the library's radix sort, whose tiles stage their pairs through LDS and
+// write long runs (measured faster from about two million pairs on).
 using RadixAlways = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
                                                rocprim::default_config, 4096>;
 static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout,
                        const int *vin, int *vout, int64_t n, hipStream_t s, int end_bit = 64) {
-  int merge_passes = 1;
-  while (((int64_t)2048 << merge_passes) < n) merge_passes++;
-  const bool radix = n > 32768 && (end_bit + 7) / 8 + 1 < merge_passes;
-  size_t bytes = 0;
-  if (radix) {
-    HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u,
-                                                     (unsigned)end_bit, s));
-    m.tmp.reserve(bytes + 16);
-    HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(m.tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u,
-                                                     (unsigned)end_bit, s));
+  if (n > 32768 && n <= 1500000) {
+    radix_sort_pairs(m, kin, kout, vin, vout, n, end_bit, s);
     return;
   }
-  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
+  size_t bytes = 0;
+  if (n <= 32768) {  // the library's choice at this size, a merge sort of a few passes, is the fastest measured
+    HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
+    m.tmp.reserve(bytes + 16);
+    HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
+    return;
+  }
+  HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                                   (unsigned)end_bit, s));
   m.tmp.reserve(bytes + 16);
-  HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
+  HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(m.tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                                   (unsigned)end_bit, s));
 }
 static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipStream_t s) {
   size_t bytes = 0;
@@ -719,20 +720,34 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
 // (by 20-30% for 64..256 channels) and one global sort (which loses the locality).
 static const int PATTERN_WINDOWS = 8;
 
-// Sort key of a position: window, then (when the bits allow) the number of absent taps, then
-// the tap mask.  Inside a window the positions with the most taps come first and the
-// cheapest last, which shortens the tail of kernels that hand positions out in order.
-__global__ void k_table_masks(int64_t window, int pc_bits, const int *nbr, int K, int64_t n, int64_t npad,
-                              unsigned long long *keys, int *idx) {
+// Sort key of a position: window, then the number of absent taps (shifted right by pc_shift
+// when the key bits are short), then the tap mask, or, when the mask has more than code_bits
+// bits, a hash of it (positions with the same taps still end up next to each other, but
+// patterns that share a hash value interleave and similar patterns are no longer neighbours:
+// measured 2 % slower convolutions on a 27-tap table, so only filters of more than 27 taps get
+// one).  Inside a window the positions with the most taps come first and the cheapest last,
+// which shortens the tail of kernels that hand positions out in order.
+// masks[t] (K <= 32): the tap mask itself, for the granule masks.
+struct PatternKey {  // how finalize_table's sort key is put together
+  int64_t window;
+  int pc_bits, pc_shift, code_bits, K;
+};
+__device__ inline unsigned long long pattern_key(const PatternKey &p, int64_t t, unsigned long long mask) {
+  unsigned long long hi = (unsigned long long)(t / p.window);
+  if (p.pc_bits) hi = (hi << p.pc_bits) | (unsigned long long)((p.K - __popcll(mask)) >> p.pc_shift);
+  const unsigned long long code = p.code_bits < p.K ? (mask * 0x9E3779B97F4A7C15ull) >> (64 - p.code_bits) : mask;
+  return (hi << p.code_bits) | code;
+}
+__global__ void k_table_masks(int64_t window, int pc_bits, int pc_shift, int code_bits, const int *nbr, int K, int64_t n,
+                              int64_t npad, unsigned long long *keys, int *idx, unsigned *masks) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n) return;
   unsigned long long mask = 0;
   for (int k = 0; k < K; k++)
     if (nbr[(int64_t)k * npad + t] >= 0) mask |= 1ull << k;
-  unsigned long long hi = (unsigned long long)(t / window);
-  if (pc_bits) hi = (hi << pc_bits) | (unsigned long long)(K - __popcll(mask));
-  keys[t] = (hi << K) | mask;
+  keys[t] = pattern_key(PatternKey{window, pc_bits, pc_shift, code_bits, K}, t, mask);
   idx[t] = (int)t;
+  if (masks) masks[t] = (unsigned)mask;
 }
 __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, const int *perm,
                                 const int *base, int *nbr2, int *rowmap) {
@@ -744,17 +759,16 @@ __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, 
   nbr2[(int64_t)k * npad + t] = nbr[(int64_t)k * npad + src];
   if (k == 0) rowmap[t] = base ? base[src] : src;
 }
-// sorted keys carry each position's tap mask in their low K bits (K <= 32)
-__global__ void k_granule_masks(const unsigned long long *skeys, int K, int64_t n, int64_t n_granules,
-                                unsigned *gmask) {
+// gmask[i] = OR of the tap masks of granule i's 16 positions; perm[t] = the position's place before the sort
+__global__ void k_granule_masks(const unsigned *masks, const int *perm, int64_t n, int64_t n_granules, unsigned *gmask) {
   int64_t gi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gi >= n_granules) return;
-  unsigned long long m = 0;
+  unsigned m = 0;
   for (int r = 0; r < 16; r++) {
     const int64_t t = gi * 16 + r;
-    if (t < n) m |= skeys[t];
+    if (t < n) m |= masks[perm[t]];
   }
-  gmask[gi] = (unsigned)(m & ((1ull << K) - 1ull));
+  gmask[gi] = m;
 }
 __global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -763,16 +777,42 @@ __global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
 
 // t.nbr is indexed by the level's schedule (base[t] = row, or t itself when base is null).
 // Re-sort positions by neighbour pattern inside windows and record the position -> row map.
-static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s) {
+// The sort key's layout for a table of n positions and K taps (K <= 62).
+static PatternKey pattern_plan(int64_t n, int K, int &key_bits) {
+  PatternKey p;
+  p.K = K;
+  p.window = std::max<int64_t>(256, round_up(ceil_div(n, PATTERN_WINDOWS), 256));
+  int block_bits = 0;
+  while (((int64_t)1 << block_bits) < ceil_div(n, p.window)) block_bits++;
+  int pc_bits = 1;
+  while ((1 << pc_bits) <= K) pc_bits++;
+  // Up to 40 key bits (four sort passes; a 27-tap table needs 35): beyond that the count of
+  // absent taps gives way first, then the mask (hashed).  Measured on 27-tap tables of a
+  // million rows: a coarser count (33 bits, three passes) gains nothing, a 14-bit hash of the
+  // mask saves 40 us of sorting and costs 4-7 % in every convolution.
+  const int budget = 40;
+  p.pc_shift = std::max(0, std::min(pc_bits, block_bits + pc_bits + K - budget));
+  p.pc_bits = pc_bits - p.pc_shift;
+  p.code_bits = std::min(K, budget - block_bits - p.pc_bits);
+  key_bits = p.code_bits + p.pc_bits + block_bits;
+  return p;
+}
+// Buffers the keyed form of finalize_table expects to be filled: m.k0 keys, m.v0 positions, m.f1 masks.
+static void reserve_pattern_buffers(Metadata &m, const Table &t) {
+  m.k0.reserve(t.n);
+  m.k1.reserve(t.n);
+  m.v0.reserve(t.n);
+  m.v1.reserve(t.n);
+  if (t.K <= 32) m.f1.reserve(t.n);
+}
+// keyed: the kernel that wrote t.nbr has written the sort keys, positions and masks as well.
+static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s, bool keyed = false) {
   if (t.n == 0) {
     t.identity_rows = true;
     return;
   }
   t.rowmap.reserve(t.npad);
-  const int64_t window = std::max<int64_t>(256, round_up(ceil_div(t.n, PATTERN_WINDOWS), 256));
-  int block_bits = 1;
-  while (((int64_t)1 << block_bits) <= t.n / window) block_bits++;
-  if (t.K + block_bits > 62) {  // the pattern does not fit the sort key: keep schedule order
+  if (t.K > 62) {  // the pattern does not fit a machine word: keep schedule order
     t.identity_rows = base == nullptr;
     if (base) {
       k_copy_rowmap<<<grid_for(t.n), TB, 0, s>>>(base, t.n, t.rowmap.p);
@@ -780,16 +820,16 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
     }
     return;
   }
-  m.k0.reserve(t.n);
-  m.k1.reserve(t.n);
-  m.v0.reserve(t.n);
-  m.v1.reserve(t.n);
-  int pc_bits = 1;
-  while ((1 << pc_bits) <= t.K) pc_bits++;
-  if (t.K + pc_bits + block_bits > 62) pc_bits = 0;
-  k_table_masks<<<grid_for(t.n), TB, 0, s>>>(window, pc_bits, t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p);
-  LAUNCH_CHECK();
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, t.K + pc_bits + block_bits);
+  int key_bits = 0;
+  const PatternKey pk = pattern_plan(t.n, t.K, key_bits);
+  reserve_pattern_buffers(m, t);
+  unsigned *masks = t.K <= 32 ? reinterpret_cast<unsigned *>(m.f1.p) : nullptr;
+  if (!keyed) {
+    k_table_masks<<<grid_for(t.n), TB, 0, s>>>(pk.window, pk.pc_bits, pk.pc_shift, pk.code_bits, t.nbr.p, t.K, t.n, t.npad,
+                                               m.k0.p, m.v0.p, masks);
+    LAUNCH_CHECK();
+  }
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, key_bits);
   DevBuf<int> nbr2;
   nbr2.reserve((size_t)t.K * t.npad);
   k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
@@ -800,7 +840,7 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   if (t.K <= 32) {
     const int64_t n_granules = ceil_div(t.n, 16);
     t.gmask.reserve(n_granules);
-    k_granule_masks<<<grid_for(n_granules), TB, 0, s>>>(m.k1.p, t.K, t.n, n_granules, t.gmask.p);
+    k_granule_masks<<<grid_for(n_granules), TB, 0, s>>>(masks, m.v1.p, t.n, n_granules, t.gmask.p);
     LAUNCH_CHECK();
   }
 }
@@ -812,12 +852,15 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
 template <int DIM>
 __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_t n, int64_t npad,
                                 const BlockEntry *table, const unsigned long long *mask_p, const int *urow,
-                                int *nbr, unsigned long long *counts) {
+                                int *nbr, unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
+                                int *pidx, unsigned *pmasks) {
   const unsigned long long mask = *mask_p;
   constexpr int K = DIM == 3 ? 27 : 9;
   constexpr int PER = K / 3;
   __shared__ int lcount[K];
+  __shared__ unsigned lmask[64];  // tap mask of each of the block's positions, collected from the three wavefronts
   if (threadIdx.x < K) lcount[threadIdx.x] = 0;
+  if (threadIdx.x < 64) lmask[threadIdx.x] = 0;
   __syncthreads();
   const int part = threadIdx.x >> 6;  // offset -1, 0, +1 along the first dimension
   int64_t t = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63);
@@ -840,6 +883,7 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
   const unsigned long long bpart = (unsigned long long)soa[DIM * npad + row] << (DIM * g.bits);
   unsigned long long last_bkey = SCN_EMPTY_KEY, last_mask = 0;
   int last_base = 0;
+  unsigned my_mask = 0;
 #pragma unroll
   for (int kk = 0; kk < PER; kk++) {
     const int k = part * PER + kk;
@@ -870,12 +914,21 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
       }
     }
     if (live) nbr[(int64_t)k * npad + t] = j;
+    if (j >= 0) my_mask |= 1u << k;
     const unsigned long long hits = __ballot(live && j >= 0);
     if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&lcount[k], __popcll(hits));
   }
+  atomicOr(&lmask[threadIdx.x & 63], my_mask);
   __syncthreads();
   unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * K;
   if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&slot[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
+  // what the pattern sort of finalize_table starts from (k_table_masks would re-read the table for it)
+  if (threadIdx.x < 64 && live) {
+    const unsigned mk = lmask[threadIdx.x];
+    pkeys[t] = pattern_key(pk, t, mk);
+    pidx[t] = (int)t;
+    pmasks[t] = mk;
+  }
 }
 
 static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const int64_t *out_size) {
@@ -1009,16 +1062,20 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   bool all3 = true;
   for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
   if (all3 && (m.dim == 2 || m.dim == 3)) {
+    int key_bits = 0;
+    const PatternKey pk = pattern_plan(t.n, t.K, key_bits);
+    reserve_pattern_buffers(m, t);
+    unsigned *masks = reinterpret_cast<unsigned *>(m.f1.p);
     if (m.dim == 3)
       k_subm_rules_s3<3><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
                                                            L.gridp.p, L.urow_ptr(), t.nbr.p,
-                                                           (unsigned long long *)t.cnt->dev.p);
+                                                           (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks);
     else
       k_subm_rules_s3<2><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
                                                            L.gridp.p, L.urow_ptr(), t.nbr.p,
-                                                           (unsigned long long *)t.cnt->dev.p);
+                                                           (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks);
     LAUNCH_CHECK();
-    finalize_table(m, t, L.sched_ptr(), s);
+    finalize_table(m, t, L.sched_ptr(), s, true);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
   // one wavefront per slice of the first filter dimension when that divides the taps evenly

@@ -1,0 +1,198 @@
+// Stable least-significant-digit radix sort of (64-bit key, 32-bit value) pairs by the low
+// `end_bit` bits of the key: what the rulebook builders sort by (site keys of an input layer,
+// candidate output sites of a strided rulebook, tap patterns of a neighbour table).  These are
+// tens of thousands to a few million pairs with 16 to 48 significant key bits: small enough
+// that a general-purpose library sort spends its time in launches (a histogram pass, then per
+// digit a look-back scan with two state fills in front), which is what this file avoids.
+//
+// Per digit (up to 9 bits) three launches, none of which waits on another workgroup:
+//   k_rs_hist     per tile of TILE pairs, the count of every digit value   hist[digit][tile]
+//   k_rs_colscan  per digit value, the exclusive prefix over tiles (in place) and the total
+//   k_rs_scatter  per tile: rank every pair among the tile's pairs of the same digit value
+//                 (stable), add the tile's prefix and the digit value's base (exclusive scan of
+//                 the totals, recomputed by every workgroup), write the pair there.
+// Ranking inside a tile: wavefront w owns a contiguous quarter of the tile and walks it 64 pairs
+// at a time; the lanes of a round that hold the same digit value find each other with one
+// ballot per digit bit, the first of them reads and bumps the wavefront's running count of that value in LDS
+// (only this wavefront touches its counts, so no barrier), which gives every pair its rank
+// inside the wavefront's quarter; a prefix over the four wavefronts' counts then orders the
+// quarters.  (Below a few ten thousand pairs the library's merge sort is faster and the callers use it.)
+// The input arrays are not written: passes alternate between the output arrays and scratch.
+#include "metadata.h"
+
+namespace scn {
+
+typedef unsigned long long u64;
+constexpr int RS_THREADS = 256, RS_WAVES = 4, RS_ITEMS = 8, RS_TILE = RS_THREADS * RS_ITEMS;  // 2048 pairs per tile
+constexpr int RS_MAX_BITS = 9, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured: four
+// digits of 9 bits beat three of 11 and five of 7 on a million pairs of 35 bits)
+
+__global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const u64 *__restrict__ keys, int64_t n, int shift, int bits,
+                                                        int tiles, int *__restrict__ hist) {
+  __shared__ int h[RS_MAX_BINS];
+  const int bins = 1 << bits;
+  for (int d = threadIdx.x; d < bins; d += RS_THREADS) h[d] = 0;
+  __syncthreads();
+  const unsigned mask = (unsigned)bins - 1u;
+  const int64_t base = (int64_t)blockIdx.x * RS_TILE;
+#pragma unroll
+  for (int r = 0; r < RS_ITEMS; r++) {
+    const int64_t i = base + r * RS_THREADS + threadIdx.x;
+    if (i < n) atomicAdd(&h[(unsigned)(keys[i] >> shift) & mask], 1);
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < bins; d += RS_THREADS) hist[(size_t)d * tiles + blockIdx.x] = h[d];
+}
+
+// One workgroup (64 threads) per digit value: hist[d][*] becomes its exclusive prefix over tiles,
+// tot[d] the sum.
+__global__ __launch_bounds__(64) void k_rs_colscan(int *__restrict__ hist, int tiles, int *__restrict__ tot) {
+  int *col = hist + (size_t)blockIdx.x * tiles;
+  const int lane = threadIdx.x;
+  const int per = (tiles + 63) / 64;
+  const int t0 = min(tiles, lane * per), t1 = min(tiles, t0 + per);
+  int sum = 0;
+  for (int t = t0; t < t1; t++) sum += col[t];
+  int incl = sum;  // inclusive scan over the 64 lanes
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  int run = incl - sum;
+  for (int t = t0; t < t1; t++) {
+    const int c = col[t];
+    col[t] = run;
+    run += c;
+  }
+  if (lane == 63) tot[blockIdx.x] = incl;
+}
+
+// Rank of each of a wavefront's ITEMS x 64 pairs (round r, lane) among the pairs of its quarter
+// with the same digit value, in round-major order; cnt[0 .. 2^bits) (this wavefront's, zero on entry)
+// ends as the quarter's count of every value.
+template <int ITEMS>
+__device__ inline void rank_quarter(const unsigned (&digit)[ITEMS], const bool (&valid)[ITEMS], int bits, int *cnt,
+                                    int lane, int (&rank)[ITEMS]) {
+  const u64 below = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int r = 0; r < ITEMS; r++) {
+    u64 peers = __ballot(valid[r]);
+    for (int b = 0; b < bits; b++) {
+      const u64 has = __ballot((digit[r] >> b) & 1u);
+      peers &= ((digit[r] >> b) & 1u) ? has : ~has;
+    }
+    const int before = __popcll(peers & below);
+    int old = 0;
+    if (valid[r]) old = cnt[digit[r]];  // every lane of the group reads the count before its first lane bumps it
+    if (valid[r] && before == 0) cnt[digit[r]] = old + __popcll(peers);
+    rank[r] = old + before;
+  }
+}
+
+__global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict__ kin, const int *__restrict__ vin,
+                                                           u64 *__restrict__ kout, int *__restrict__ vout, int64_t n,
+                                                           int shift, int bits, int tiles, const int *__restrict__ offs,
+                                                           const int *__restrict__ tot) {
+  __shared__ int cnt[RS_WAVES][RS_MAX_BINS];
+  __shared__ int base[RS_MAX_BINS];  // where the tile's first pair of each digit value goes
+  __shared__ int wsum[RS_WAVES];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int bins = 1 << bits;
+  const unsigned mask = (unsigned)bins - 1u;
+  // exclusive scan of the digit values' totals (thread t: values [t * per, (t + 1) * per)) + this tile's prefix
+  {
+    const int per = (bins + RS_THREADS - 1) / RS_THREADS;  // 1 or 2
+    const int d0 = threadIdx.x * per;
+    int mine = 0;
+    for (int j = 0; j < per; j++)
+      if (d0 + j < bins) mine += tot[d0 + j];
+    int incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) wsum[wave] = incl;
+    for (int d = threadIdx.x; d < bins; d += RS_THREADS) {
+#pragma unroll
+      for (int w = 0; w < RS_WAVES; w++) cnt[w][d] = 0;
+    }
+    __syncthreads();
+    int run = incl - mine;
+    for (int w = 0; w < wave; w++) run += wsum[w];
+    for (int j = 0; j < per; j++)
+      if (d0 + j < bins) {
+        base[d0 + j] = run + offs[(size_t)(d0 + j) * tiles + blockIdx.x];
+        run += tot[d0 + j];
+      }
+  }
+  // this wavefront's quarter: pairs [q0, q0 + ITEMS * 64)
+  const int64_t q0 = (int64_t)blockIdx.x * RS_TILE + (int64_t)wave * (RS_ITEMS * 64);
+  u64 key[RS_ITEMS];
+  int val[RS_ITEMS];
+  unsigned digit[RS_ITEMS];
+  bool valid[RS_ITEMS];
+  int rank[RS_ITEMS];
+#pragma unroll
+  for (int r = 0; r < RS_ITEMS; r++) {
+    const int64_t i = q0 + r * 64 + lane;
+    valid[r] = i < n;
+    key[r] = valid[r] ? kin[i] : 0ull;
+    val[r] = valid[r] ? vin[i] : 0;
+    digit[r] = (unsigned)(key[r] >> shift) & mask;
+  }
+  rank_quarter<RS_ITEMS>(digit, valid, bits, cnt[wave], lane, rank);
+  __syncthreads();  // all four quarters counted, base[] written
+#pragma unroll
+  for (int r = 0; r < RS_ITEMS; r++) {
+    if (!valid[r]) continue;
+    int at = base[digit[r]] + rank[r];
+    for (int w = 0; w < wave; w++) at += cnt[w][digit[r]];
+    kout[at] = key[r];
+    vout[at] = val[r];
+  }
+}
+
+void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, int *vout, int64_t n, int end_bit,
+                      hipStream_t s) {
+  if (n <= 0) return;
+  end_bit = std::max(1, std::min(64, end_bit));
+  if (n >= ((int64_t)1 << 31)) throw Error("sort: too many pairs");
+  // as few digits as 9 bits each allow, of equal width
+  const int passes = (end_bit + RS_MAX_BITS - 1) / RS_MAX_BITS;
+  const int width = (end_bit + passes - 1) / passes;
+  const int tiles = (int)ceil_div(n, RS_TILE);
+  // scratch: a second pair of arrays (when there is more than one pass), the tile counts, the totals
+  const size_t kbytes = round_up((size_t)n * sizeof(u64), 256), vbytes = round_up((size_t)n * sizeof(int), 256);
+  const size_t hbytes = round_up(((size_t)1 << width) * tiles * sizeof(int), 256);
+  m.tmp.reserve((passes > 1 ? kbytes + vbytes : 0) + hbytes + ((size_t)1 << width) * sizeof(int));
+  unsigned char *p = m.tmp.p;
+  u64 *ktmp = nullptr;
+  int *vtmp = nullptr;
+  if (passes > 1) {
+    ktmp = reinterpret_cast<u64 *>(p);
+    vtmp = reinterpret_cast<int *>(p + kbytes);
+    p += kbytes + vbytes;
+  }
+  int *hist = reinterpret_cast<int *>(p), *tot = reinterpret_cast<int *>(p + hbytes);
+  const u64 *ksrc = kin;
+  const int *vsrc = vin;
+  for (int pass = 0; pass < passes; pass++) {
+    // the last pass writes the output arrays; the ones before alternate so that it can
+    const bool to_out = (passes - 1 - pass) % 2 == 0;
+    u64 *kdst = to_out ? kout : ktmp;
+    int *vdst = to_out ? vout : vtmp;
+    const int shift = width * pass, bits = std::min(width, end_bit - shift);
+    k_rs_hist<<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist);
+    LAUNCH_CHECK();
+    k_rs_colscan<<<dim3(1 << bits), 64, 0, s>>>(hist, tiles, tot);
+    LAUNCH_CHECK();
+    k_rs_scatter<<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot);
+    LAUNCH_CHECK();
+    ksrc = kdst;
+    vsrc = vdst;
+  }
+}
+
+}  // namespace scn
