@@ -185,6 +185,31 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
                 cold_host.append((t3 - t2) * 1e3)
     macs = scn.forward_pass_multiplyAdd_count / (3 * (reps + 1))
     med = lambda v: round(float(np.median(v)), 3)
+    graph_ms = None
+    if batch == 1 and not residual:
+        # The warm forward pass captured once as a HIP graph and replayed: the same kernels without
+        # the host's per-call work between them (what a serving loop over a fixed scene would run).
+        side = torch.cuda.Stream()
+        with torch.no_grad():
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                linear(model(x))
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                yg = linear(model(x))
+            reps_ms = []
+            for _ in range(reps):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                graph.replay()
+                torch.cuda.synchronize()
+                reps_ms.append((time.perf_counter() - t0) * 1e3)
+            same = bool(torch.equal(yg, linear(model(x))))
+            torch.cuda.synchronize()
+        graph_ms = med(reps_ms) if same else None
+        del graph
     if batch > 1:
         return {"unet_batch%d_ms_per_batch" % batch: med(cold), "unet_batch%d_warm_ms_per_batch" % batch: med(warm),
                 "unet_batch%d_from_host_coords_ms_per_batch" % batch: med(cold_host),
@@ -193,13 +218,14 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
         return {"unet_residual_ms_per_scene": med(cold), "unet_residual_warm_ms": med(warm),
                 "unet_residual_gflop": round(2 * macs / 1e9, 2)}
     return {"unet_ms_per_scene": med(cold), "unet_ms_per_scene_from_host_coords": med(cold_host),
-            "unet_warm_ms": med(warm), "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
+            "unet_warm_ms": med(warm), "unet_warm_graph_replay_ms": graph_ms, "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
             "unet_gflop": round(2 * macs / 1e9, 2),
             "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1),
             "unet_warm_frac_mfma_fp32": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e12 / MFMA_FP32_TFLOPS, 4),
             "note": "ms_per_scene: new Metadata per scene (input layer, every rulebook, all layers), coordinates "
                     "resident in HBM; from_host_coords: the same with the coordinates handed over as a CPU "
-                    "LongTensor (host-to-device copy inside the timed region); warm: rulebooks cached"}
+                    "LongTensor (host-to-device copy inside the timed region); warm: rulebooks cached; "
+                    "warm_graph_replay: the warm pass replayed as one HIP graph (null if the replay's result differed)"}
 
 
 def _timed(torch, fn, reps=5):

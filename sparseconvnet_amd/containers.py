@@ -21,11 +21,19 @@ class Sequential(torch.nn.Sequential):
 
     def forward(self, input):
         # Same chain as sequential.py:10-35, except that eval-mode batch normalisations next
-        # to a convolution are applied inside that convolution (layers.fuse_plan).
-        from .layers import fuse_plan
+        # to a convolution are applied inside that convolution (layers.fuse_plan) and one behind a
+        # JoinTable while the parts are joined (layers.join_batchnorm).
+        from .layers import fuse_plan, join_batchnorm
         mods = self._chain()
         i = 0
         while i < len(mods):
+            if type(mods[i]) is JoinTable and i + 1 < len(mods) and isinstance(input, (list, tuple)) \
+                    and not mods[i]._forward_hooks and not mods[i]._forward_pre_hooks:
+                joined = join_batchnorm(input, mods[i + 1])
+                if joined is not None:
+                    input = joined
+                    i += 2
+                    continue
             plan = fuse_plan(mods[i:i + 3], input) if isinstance(input, SparseConvNetTensor) else None
             if plan is None:
                 input = mods[i](input)

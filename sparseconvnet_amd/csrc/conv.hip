@@ -691,7 +691,25 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   typedef int v4i_t __attribute__((ext_vector_type(4)));
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
-  const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
+  // COAL (see k_conv_resident): gathers are issued with the four lanes of a quad reading 64
+  // consecutive bytes of one row; the values move to the MFMA's operand lanes when they are staged.
+  // Only the bf16 variant, which is bound by its gathers (measured at a million sites: 64 -> 64
+  // 0.46 -> 0.38 ms, 128 -> 128 0.89 -> 0.77 ms); the fp32 variant is bound by MFMA issue and
+  // loses 2-6 % to the extra permutes.
+  constexpr bool COAL = BUF && BF16;
+  const int ld_row = COAL ? lane >> 2 : r16, ld_g = COAL ? lane & 3 : g;
+  const int perm_src = (4 * r16 + g) * 4;
+  auto to_operand_lanes = [&](v4f v) {
+    if constexpr (COAL) {
+      const float x = v.x, y = v.y, z = v.z, w = v.w;
+      v.x = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, x)));
+      v.y = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, y)));
+      v.z = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, z)));
+      v.w = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, w)));
+    }
+    return v;
+  };
+  const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)ld_g;
   int nx_ti = 0, nx_sl = 0;  // (tap index, slab) of the next iteration to issue; issue() runs in sequence
   auto issue = [&](int) {
     const int sl = nx_sl;
@@ -708,8 +726,8 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     if (PRE) {
 #pragma unroll
       for (int s = 0; s < SS; s++) {
-        psc[s] = *reinterpret_cast<const v4f *>(pre_sc + (sl * SS + s) * 16 + 4 * g);
-        psh[s] = *reinterpret_cast<const v4f *>(pre_sh + (sl * SS + s) * 16 + 4 * g);
+        psc[s] = *reinterpret_cast<const v4f *>(pre_sc + (sl * SS + s) * 16 + 4 * ld_g);
+        psh[s] = *reinterpret_cast<const v4f *>(pre_sh + (sl * SS + s) * 16 + 4 * ld_g);
       }
     }
     const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
@@ -720,7 +738,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     }
 #pragma unroll
     for (int q = 0; q < RG; q++) {
-      const int j = jtab[((wave * RG + q) * K + k) * 16 + r16];
+      const int j = jtab[((wave * RG + q) * K + k) * 16 + ld_row];
       if constexpr (BUF) {
         // Buffer loads return zeros past the end of the buffer: an absent row becomes an
         // offset of 2 GiB (the launcher only takes this path for smaller inputs, whole slabs
@@ -770,19 +788,19 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
             v0 = ok ? v0 : (v4f){0.f, 0.f, 0.f, 0.f};
             v1 = ok ? v1 : (v4f){0.f, 0.f, 0.f, 0.f};
           }
-          a_cur[q][s / 2] = __builtin_bit_cast(v4f, to_bf16x8(v0, v1));
+          a_cur[q][s / 2] = to_operand_lanes(__builtin_bit_cast(v4f, to_bf16x8(v0, v1)));
         }
         continue;
       }
 #pragma unroll
       for (int s = 0; s < SS; s++) {
         if constexpr (BUF && !PRE && !BF16) {
-          a_cur[q][s] = a_nxt[q][s];
+          a_cur[q][s] = to_operand_lanes(a_nxt[q][s]);
           continue;
         }
         if constexpr (BUF && PRE && !BF16) {
           const v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
-          a_cur[q][s] = ok ? v : (v4f){0.f, 0.f, 0.f, 0.f};
+          a_cur[q][s] = to_operand_lanes(ok ? v : (v4f){0.f, 0.f, 0.f, 0.f});
           continue;
         }
         if constexpr (!BUF) {
@@ -1054,17 +1072,36 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
       j[0] = nbr[(int64_t)it.k * npad + t];
     }
   };
+  // COAL: a gather instruction reads 16 rows x 64 bytes.  In the MFMA's operand layout (lane
+  // g * 16 + r: bytes [16 g, 16 g + 16) of row r) neighbouring lanes read different rows, 64
+  // separate accesses for the texture unit; read as lane 4 r + g instead, the four lanes of a
+  // quad read 64 consecutive bytes, one access, and the values change lanes afterwards (an
+  // LDS-crossbar permute per register, at use).
+  constexpr bool COAL = BUF && VEC4 && !C4;
+  const int ld_row = COAL ? lane >> 2 : r16;                 // row of a granule this lane loads
+  const unsigned ld_off = COAL ? 16u * (unsigned)(lane & 3) : lane_off;
+  const int perm_src = (4 * r16 + g) * 4;                    // byte address of the lane that loaded this lane's operand
+  auto to_operand_lanes = [&](v4f v) {
+    if constexpr (COAL) {
+      const float x = v.x, y = v.y, z = v.z, w = v.w;  // (element references do not survive a bit cast)
+      v.x = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, x)));
+      v.y = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, y)));
+      v.z = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, z)));
+      v.w = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(perm_src, __builtin_bit_cast(int, w)));
+    }
+    return v;
+  };
   auto issue_a = [&](const Item &it, const int *jset, AV (*a)[SS], unsigned &okbits) {
     okbits = 0;
     int j[RG];
 #pragma unroll
-    for (int q = 0; q < RG; q++) j[q] = __shfl(jset[0], q * 16 + r16, 64);
+    for (int q = 0; q < RG; q++) j[q] = __shfl(jset[0], q * 16 + ld_row, 64);
 #pragma unroll
     for (int q = 0; q < RG; q++) {
-      const bool ok = j[q] >= 0 && (int64_t)it.set * (RG * 16) + q * 16 + r16 < n;
+      const bool ok = j[q] >= 0 && (int64_t)it.set * (RG * 16) + q * 16 + ld_row < n;
       okbits |= ok ? 1u << q : 0u;
       if constexpr (BUF) {
-        const unsigned voff = ok ? (__umul24((unsigned)j[q], row_bytes) + lane_off) : 0x80000000u;
+        const unsigned voff = ok ? (__umul24((unsigned)j[q], row_bytes) + ld_off) : 0x80000000u;
 #pragma unroll
         for (int s = 0; s < SS; s++) {
           if constexpr (C4)
@@ -1140,7 +1177,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
         for (int q = 0; q < RG; q++) {
           const bool ok = (okb >> q) & 1u;
           if (__ballot(ok) == 0ull) continue;  // uniform: no row of this granule has the tap
-          const v8s av = to_bf16x8(ar[S][q][0], ar[S][q][1]);
+          v8s av = to_bf16x8(ar[S][q][0], ar[S][q][1]);
+          if constexpr (COAL) av = __builtin_bit_cast(v8s, to_operand_lanes(__builtin_bit_cast(v4f, av)));
 #pragma unroll
           for (int cb = 0; cb < NCB; cb++) acc[q][cb] = mfma_bf16(av, __builtin_bit_cast(v8s, b[cb]), acc[q][cb]);
         }
@@ -1157,7 +1195,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
 #pragma unroll
           for (int s = 0; s < SS; s++) {
             const int c0 = s * 16 + 4 * g;
-            v4f av = ar[S][q][s];
+            v4f av = to_operand_lanes(ar[S][q][s]);
             if (BUF) {
             } else if (VEC4) {
               if (!(ok && c0 < n_in)) av = (v4f){0.f, 0.f, 0.f, 0.f};

@@ -84,6 +84,49 @@ class _BatchNormalizationFunction(Function):
         return d_in, d_w, d_b, None, None, None, None, None, None, None
 
 
+class _JoinBatchNormFunction(Function):
+    """JoinTable followed by an eval-mode batch normalisation (tables.py:35-48,
+    batchNormalization.py:93-117) in one pass per part: each part is normalised with its range
+    of the planes straight into its columns of the joined matrix, which costs what the
+    concatenation alone costs and spares the convolution behind it the normalisation."""
+
+    @staticmethod
+    def forward(ctx, running_mean, running_var, weight, bias, eps, leakiness, *parts):
+        rows = parts[0].size(0)
+        out = parts[0].new_empty((rows, sum(p.size(1) for p in parts)))
+        off = 0
+        for p in parts:
+            c = p.size(1)
+            _md.batchNormEval(p, running_mean[off:off + c], running_var[off:off + c],
+                              weight[off:off + c] if weight.numel() else None,
+                              bias[off:off + c] if bias.numel() else None, eps, leakiness, out=out[:, off:off + c])
+            off += c
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        # batchNormalization.py:147
+        assert False, "backward through an eval-mode batch normalisation; call .train() on the model"
+
+
+def join_batchnorm(parts, bn):
+    """JoinTable()(parts) followed by the eval-mode batch normalisation `bn`, or None when the
+    two have to run one after the other (plane counts that do not add up, empty tensors)."""
+    if not _pkg.fuse_batchnorm or not _is_bn(bn) or len(parts) < 2:
+        return None
+    feats = [p.features for p in parts]
+    if any(f.dim() != 2 or f.nelement() == 0 or f.size(0) != feats[0].size(0) for f in feats):
+        return None
+    if sum(f.size(1) for f in feats) != bn.nPlanes:
+        return None
+    output = SparseConvNetTensor()
+    output.metadata = parts[0].metadata
+    output.spatial_size = parts[0].spatial_size
+    output.features = _JoinBatchNormFunction.apply(bn.running_mean, bn.running_var, optionalTensor(bn, 'weight').detach(),
+                                                   optionalTensor(bn, 'bias').detach(), bn.eps, bn.leakiness, *feats)
+    return output
+
+
 class _PoolingFunction(Function):
     """maxPooling.py:14-72, averagePooling.py:13-66, unPooling.py:14-57: which = 'max', 'average',
     'un'.  sizes = (input level, output level, pool size, pool stride) of the op."""

@@ -419,9 +419,13 @@ class Metadata:
         return d_in
 
 
-def batchNormEval(features, running_mean, running_var, weight, bias, eps, leakiness):
+def batchNormEval(features, running_mean, running_var, weight, bias, eps, leakiness, out=None):
+    """out: where the result goes, rows of features.size(1) floats at any row stride (a column
+    range of a wider matrix); a new tensor when None."""
     features = _features(features, "features")
-    out = torch.empty_like(features)
+    if out is None:
+        out = torch.empty_like(features)
+    assert out.shape == features.shape and out.stride(1) == 1 and out.dtype == torch.float32 and out.is_cuda
     w = weight if weight is not None and weight.numel() else None
     b = bias if bias is not None and bias.numel() else None
     _lib.check(_lib.lib().scn_bn_eval_fwd(_ptr(features), _ptr(out), features.size(0), features.size(1),
