@@ -381,24 +381,27 @@ def config_rows():
 
 def other_ops(sites, seed):
     """The rest of the path on the same kind of scene, each op by itself with inputs resident
-    in HBM: ms (median of 5, HIP events on the launch stream) and the algorithmic bytes it has
-    to move, against the 8 TB/s of HBM.  Rulebook builds are timed from the host (they
+    in HBM: ms per call (median of 5 timings of 8 calls back to back, HIP events on the launch
+    stream) and the algorithmic bytes it has to move, against the 8 TB/s of HBM.  Rulebook builds are timed from the host (they
     synchronise)."""
     import torch
     import sparseconvnet_amd as scn
     from sparseconvnet_amd import metadata as M
     from sparseconvnet_amd import synthetic
 
-    def timed(fn, reps=5):
+    def timed(fn, reps=5, inner=8):
+        # `inner` calls back to back between one pair of events: these ops last 25-100 us, and a
+        # single call between two events measures the launch as much as the kernel
         fn()
         ms = []
         for _ in range(reps):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            fn()
+            for _ in range(inner):
+                fn()
             e1.record()
             torch.cuda.synchronize()
-            ms.append(e0.elapsed_time(e1))
+            ms.append(e0.elapsed_time(e1) / inner)
         return float(np.median(ms))
 
     def host_timed(fn, reps=4):
@@ -567,6 +570,7 @@ def main():
     ap.add_argument("--no-unet", action="store_true")
     ap.add_argument("--no-ops", action="store_true")
     ap.add_argument("--no-bf16", action="store_true")
+    ap.add_argument("--no-backward", action="store_true")
     ap.add_argument("--no-residual", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 3 times, to scale profiler byte counters")
@@ -671,6 +675,27 @@ def main():
         "rulebook_roofline": hbm_roofline(subm_rulebook_bytes(n, 27, R), rulebook_ms),
         "roofline": roof, "sweep": sweep,
     }
+    if not args.no_backward:
+        # Backward pass of the same layers on the same scene (gradients of input rows, weights and
+        # bias): R.nIn.nOut multiply-adds for the input gradient and as many for the weight
+        # gradient, twice the forward pass's count.
+        bw = []
+        for cin, cout, x, w, y in work:
+            if cin * cout > 128 * 128:
+                continue  # the widest layer: nothing the narrower ones do not show, 25 ms per call
+            d_y = torch.randn((n, cout), device="cuda", generator=g)
+            d_x, d_w, d_b = torch.empty_like(x), torch.empty_like(w), torch.empty(cout, device="cuda")
+
+            def bwd():
+                _lib.check(L.scn_subm_conv_bwd(h, sp, fs, C.c_void_p(x.data_ptr()), C.c_void_p(d_x.data_ptr()),
+                                               C.c_void_p(d_y.data_ptr()), C.c_void_p(w.data_ptr()),
+                                               C.c_void_p(d_w.data_ptr()), C.c_void_p(d_b.data_ptr()), cin, cout, 1, stream))
+            ms = _timed(torch, bwd, reps=3)
+            bw.append({"nIn": cin, "nOut": cout, "ms": round(ms, 4),
+                       "gflops": round(4.0 * R * cin * cout / (ms * 1e-3) / 1e9, 1),
+                       "frac_mfma_fp32": round(4.0 * R * cin * cout / (ms * 1e-3) / 1e12 / MFMA_FP32_TFLOPS, 4)})
+            del d_y, d_x, d_w, d_b
+        out["sweep_backward"] = bw
     if not args.no_bf16:
         # Optional reduced-precision path (bf16 operands, fp32 accumulation), same work, listed
         # beside the fp32 sweep; `value` and `roofline` above are fp32 only.

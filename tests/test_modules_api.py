@@ -234,3 +234,24 @@ def test_no_cpu_fallback():
         layer([coords, torch.ones(2, 1)])
     with pytest.raises(ScnError):
         scn.metadata.batchNormEval(torch.ones(2, 3), torch.zeros(3), torch.ones(3), None, None, 1e-4, 0)
+
+
+def test_reference_state_dict_loads_strictly():
+    """tests/golden/unet_state_dict.pth was written by the reference's own Python modules
+    (tests/golden/make_state_dict_golden.py): the same constructor calls on this package give a
+    model whose state dict has exactly those keys, in that order, with those shapes, and
+    load_state_dict(strict=True) accepts the file (what sparseconvnet/utils.py:138-177 does with a
+    checkpoint)."""
+    import os
+    import torch
+    sys_path_root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    state = torch.load(os.path.join(sys_path_root, "tests", "golden", "unet_state_dict.pth"), weights_only=True)
+    m = 8
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 1, [m, 2 * m, 3 * m], True)).add(scn.BatchNormReLU(m)).add(scn.OutputLayer(3))
+    own = model.state_dict()
+    assert list(own) == list(state)
+    assert [tuple(v.shape) for v in own.values()] == [tuple(v.shape) for v in state.values()]
+    assert all(v.dtype == state[k].dtype for k, v in own.items())
+    result = model.load_state_dict(state, strict=True)
+    assert not result.missing_keys and not result.unexpected_keys

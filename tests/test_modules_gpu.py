@@ -669,3 +669,30 @@ def test_tensor_utilities():
     assert two.features.shape == (len(ca), 11) and two.metadata is a.metadata
     assert torch.equal(scn.add_feature_planes([a, a, a]).features, a.features * 3)
     assert rng is not None
+
+
+def test_reference_state_dict_reproduces_reference_output():
+    """A state dict written by the reference's Python modules, loaded into the same network built
+    from this package, gives the output the reference's CPU path computed for the fixture's input
+    (tests/golden/make_state_dict_golden.py wrote both): checkpoints of the reference carry over."""
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    state = torch.load(os.path.join(here, "golden", "unet_state_dict.pth"), weights_only=True)
+    io = np.load(os.path.join(here, "golden", "unet_state_dict_io.npz"))
+    m = 8
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 1, [m, 2 * m, 3 * m], True)).add(scn.BatchNormReLU(m)).add(scn.OutputLayer(3))
+    model.load_state_dict(state, strict=True)
+    model = model.cuda().eval()
+    with torch.no_grad():
+        x = scn.InputLayer(3, 32, mode=4)([torch.as_tensor(io["coords"]), torch.as_tensor(io["feats"]).cuda()])
+        got = model(x).cpu().numpy()
+    checks.assert_close(got, io["out"], "output of the reference's checkpoint")
+    for fuse in (False,):  # and with every batch norm as a pass of its own
+        scn.fuse_batchnorm = fuse
+        try:
+            with torch.no_grad():
+                x = scn.InputLayer(3, 32, mode=4)([torch.as_tensor(io["coords"]), torch.as_tensor(io["feats"]).cuda()])
+                checks.assert_close(model(x).cpu().numpy(), io["out"], "unfused, output of the reference's checkpoint")
+        finally:
+            scn.fuse_batchnorm = True
