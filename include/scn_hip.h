@@ -287,6 +287,17 @@ int scn_bn_eval_fwd(const float *in, float *out, int64_t rows, int planes, int64
 int scn_s2d_fwd(scn_metadata *md, const int64_t *spatial, const float *in, float *out,
                 int planes, void *stream);
 
+/* ActivePooling_updateOutput / ActivePooling_updateGradInput (pybind.cpp:34-43,
+ * CPU/ActivePooling.cpp:8-83): out [batchSize, planes] = per sample the sum of its active rows, times
+ * 1 / count when average != 0; d_in [nActive, planes] = the sample's gradient for each of its rows
+ * (same factor).  The reference's rule builder (Metadata/ActivePoolingRules.h:16-34) does not return
+ * for a sample with more than one site (its padding loop tests a constant); what is built here is the
+ * rule matrix its header comment specifies, and agrees with the reference where that returns. */
+int scn_active_pooling_fwd(scn_metadata *md, const int64_t *spatial, const float *in, float *out,
+                           int planes, int average, void *stream);
+int scn_active_pooling_bwd(scn_metadata *md, const int64_t *spatial, float *d_in, const float *d_out,
+                           int planes, int average, void *stream);
+
 /* ---- backward pass ----------------------------------------------------------------------------
  * Gradients are device fp32 arrays allocated by the caller and written in full (the reference's
  * Python side hands zero-filled tensors to calls that accumulate into them); d_bias may be NULL.

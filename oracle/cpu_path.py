@@ -99,6 +99,8 @@ def _load(flavour):
         "bl_input_bwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
         "bl_output_bwd": (None, [C.c_void_p, _f32p, _f32p, C.c_int]),
         "s2d_bwd": (None, [C.c_void_p, _i64p, _f32p, _f32p, C.c_int]),
+        "active_pooling": (C.c_int, [C.c_void_p, _i64p, _f32p, _f32p, C.c_int, C.c_int]),
+        "active_pooling_bwd": (C.c_int, [C.c_void_p, _i64p, _f32p, _f32p, C.c_int, C.c_int]),
     }
     fns = {}
     for name, (res, args) in sig.items():
@@ -471,6 +473,21 @@ class CpuPath:
         d_in = np.zeros((int(hdr[4]), d_out.shape[-1]), np.float32)
         self.f["bl_output_bwd"](self.h, _pf(d_in), _pf(flat), d_out.shape[-1])
         return d_in
+
+    def active_pooling(self, spatial, x, average=False):
+        """[batch, planes], or None from the compiled reference where its rule builder
+        (Metadata/ActivePoolingRules.h:29) would not return: a sample with other than one site."""
+        x = _f32(x)
+        out = np.zeros((self.batch_size(spatial), x.shape[1]), np.float32)
+        ok = self.f["active_pooling"](self.h, _p64(_sz(self.dim, spatial)), _pf(x), _pf(out), x.shape[1], int(average))
+        return out if ok else None
+
+    def active_pooling_bwd(self, spatial, d_out, average=False):
+        d_out = _f32(d_out)
+        d_in = np.zeros((self.nactive(spatial), d_out.shape[1]), np.float32)
+        ok = self.f["active_pooling_bwd"](self.h, _p64(_sz(self.dim, spatial)), _pf(d_in), _pf(d_out), d_out.shape[1],
+                                          int(average))
+        return d_in if ok else None
 
     def s2d_bwd(self, spatial, d_out):
         d_out = _f32(d_out)

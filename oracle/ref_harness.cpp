@@ -31,6 +31,7 @@ template class Metadata<6>;
 #include "CPU/UnPooling.cpp"
 #include "CPU/NetworkInNetwork.cpp"
 #include "CPU/SparseToDense.cpp"
+#include "CPU/ActivePooling.cpp"
 
 #include <cstring>
 
@@ -452,4 +453,27 @@ void ref_s2d_bwd(void *h, const int64_t *spatial, float *d_in, const float *d_ou
            cpu_SparseToDense_updateGradInput<float, D>(S, m, I, DI, DO); copy_out(DI, d_in));
 }
 
+// ActivePooling_updateOutput / _updateGradInput (pybind.cpp:34-43).  The reference's rule builder
+// (Metadata/ActivePoolingRules.h:29) only returns when no sample holds more than one site; for
+// anything else these return 0 without calling it.
+static int active_pooling_terminates(void *h, const int64_t *spatial) {
+  int ok = 1;
+  DISPATCH(h, auto S = lt(spatial, D); auto &SGs = m.getSparseGrid(S); for (auto &sg : SGs) if (sg.mp.size() != 1) ok = 0);
+  return ok;
+}
+int ref_active_pooling(void *h, const int64_t *spatial, const float *in, float *out, int nPlanes, int average) {
+  if (!active_pooling_terminates(h, spatial)) return 0;
+  DISPATCH(h, auto S = lt(spatial, D); Int n = m.getNActive(S); auto I = ft(in, {n, nPlanes});
+           auto O = torch::empty({0}, at::kFloat);
+           cpu_ActivePooling_updateOutput<float, D>(S, m, I, O, average != 0); copy_out(O, out));
+  return 1;
+}
+int ref_active_pooling_bwd(void *h, const int64_t *spatial, float *d_in, const float *d_out, int nPlanes, int average) {
+  if (!active_pooling_terminates(h, spatial)) return 0;
+  DISPATCH(h, auto S = lt(spatial, D); Int n = m.getNActive(S); auto I = torch::zeros({n, nPlanes}, at::kFloat);
+           auto DI = torch::empty({0}, at::kFloat);
+           auto DO = ft(d_out, {(int64_t)m.getSparseGrid(S).size(), nPlanes});
+           cpu_ActivePooling_updateGradInput<float, D>(S, m, I, DI, DO, average != 0); copy_out(DI, d_in));
+  return 1;
+}
 }  // extern "C"

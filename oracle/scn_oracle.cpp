@@ -1239,4 +1239,66 @@ void orc_s2d_bwd(void *md, const int64_t *spatial, float *d_in, const float *d_o
   }
 }
 
+// Metadata/ActivePoolingRules.h:16-34 as its header comment describes it: rules[0] is a
+// batchSize x (maxActive + 1) matrix, first column the number of active sites of the sample,
+// then its rows (sg.ctr + value, in the grid's iteration order), zero padded.  (As written the
+// reference pads with `while (rules.size() % (maxActive + 1) != 0)`, where rules.size() is the
+// constant 2: that loop ends only when no sample has more than one site.  For such inputs this
+// function and the reference agree; beyond, this is the matrix the comment specifies.)
+static void active_pooling_rules(const Grids &SGs, std::vector<Int> &r, Int &maxActive) {
+  maxActive = 0;
+  for (auto &sg : SGs) maxActive = std::max(maxActive, (Int)sg.count);
+  r.clear();
+  for (auto &sg : SGs) {
+    const size_t row0 = r.size();
+    r.push_back((Int)sg.count);
+    for (size_t b = 0; b < sg.used.size(); b++)
+      if (sg.used[b]) r.push_back(sg.ctr + sg.vals[b]);
+    r.resize(row0 + (size_t)maxActive + 1, 0);  // padding
+  }
+}
+// CPU/ActivePooling.cpp:8-25,47-63: out [batchSize, nPlanes] = per sample the sum of its rows,
+// times 1 / count with average.
+// Returns 1 (the compiled reference's entry returns 0 where its rule builder would not return).
+int orc_active_pooling(void *md, const int64_t *spatial, const float *in, float *out, int nPlanes, int average) {
+  Metadata &m = *(Metadata *)md;
+  const Grids &SGs = m.grids[mkkey(m.dim, spatial)];
+  std::vector<Int> rules;
+  Int maxActive = 0;
+  active_pooling_rules(SGs, rules, maxActive);
+  const Int batchSize = (Int)SGs.size();
+  std::memset(out, 0, sizeof(float) * (size_t)batchSize * nPlanes);
+  for (Int o = 0; o < batchSize; o++) {
+    const Int *r = &rules[(size_t)o * (maxActive + 1)];
+    Int nActive = *r++;
+    const float mult = (average && nActive > 0) ? 1.0f / nActive : 1.0f;
+    while (nActive-- > 0) {
+      const float *inp = in + (size_t)(*r++) * nPlanes;
+      for (int p = 0; p < nPlanes; p++) out[(size_t)o * nPlanes + p] += inp[p] * mult;
+    }
+  }
+  return 1;
+}
+// CPU/ActivePooling.cpp:26-44,65-83: d_in [nActive, nPlanes]: every row receives its sample's
+// gradient (times 1 / count with average).
+int orc_active_pooling_bwd(void *md, const int64_t *spatial, float *d_in, const float *d_out, int nPlanes,
+                           int average) {
+  Metadata &m = *(Metadata *)md;
+  const Grids &SGs = m.grids[mkkey(m.dim, spatial)];
+  std::vector<Int> rules;
+  Int maxActive = 0;
+  active_pooling_rules(SGs, rules, maxActive);
+  std::memset(d_in, 0, sizeof(float) * (size_t)m.nActive[mkkey(m.dim, spatial)] * nPlanes);
+  for (Int o = 0; o < (Int)SGs.size(); o++) {
+    const Int *r = &rules[(size_t)o * (maxActive + 1)];
+    Int nActive = *r++;
+    const float mult = (average && nActive > 0) ? 1.0f / nActive : 1.0f;
+    while (nActive-- > 0) {
+      float *inp = d_in + (size_t)(*r++) * nPlanes;
+      for (int p = 0; p < nPlanes; p++) inp[p] = d_out[(size_t)o * nPlanes + p] * mult;
+    }
+  }
+  return 1;
+}
+
 }  // extern "C"

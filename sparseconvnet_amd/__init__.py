@@ -20,7 +20,7 @@ bf16_mfma = False
 from .activations import (ELU, SELU, BatchNormELU, BatchwiseDropout, Dropout, LeakyReLU, ReLU,  # noqa: E402
                           Sigmoid, Tanh)
 from .containers import AddTable, CheckpointedSequential, ConcatTable, JoinTable, Sequential  # noqa: E402
-from .layers import (AveragePooling, BatchNormalization, BatchNormLeakyReLU, BatchNormReLU,  # noqa: E402
+from .layers import (ActivePooling, AveragePooling, BatchNormalization, BatchNormLeakyReLU, BatchNormReLU,  # noqa: E402
                      BLInputLayer, BLOutputLayer, Convolution, Deconvolution, DenseToSparse, Identity, InputLayer,
                      InputLayerInput, MaxPooling,
                      NetworkInNetwork, OutputLayer, SparseToDense, SubmanifoldConvolution, UnPooling,

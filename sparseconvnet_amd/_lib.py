@@ -51,6 +51,8 @@ SIGNATURES = {
     "scn_subm_conv_fwd_noalloc": (C.c_int, [_vp, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_take_released_macs": (C.c_int, [C.POINTER(C.c_double)]),
     "scn_release_cache": (C.c_int, []),
+    "scn_active_pooling_fwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "scn_active_pooling_bwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_sort_pairs": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, _vp]),
     "scn_cache_stats": (C.c_int, [_i64p, _i64p, _i64p, _i64p]),
     "scn_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,

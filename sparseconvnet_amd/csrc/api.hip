@@ -883,6 +883,25 @@ int scn_s2d_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float 
   });
 }
 
+int scn_active_pooling_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float *out, int planes,
+                           int average, void *stream) {
+  return guarded([&] {
+    Level *l = find_level(md(h), spatial);
+    if (!l) throw Error("active pooling: unknown spatial size");
+    consume(md(h), st(stream));
+    active_pool_forward(md(h), *l, in, out, planes, average, st(stream));
+  });
+}
+int scn_active_pooling_bwd(scn_metadata *h, const int64_t *spatial, float *d_in, const float *d_out, int planes,
+                           int average, void *stream) {
+  return guarded([&] {
+    Level *l = find_level(md(h), spatial);
+    if (!l) throw Error("active pooling: unknown spatial size");
+    consume(md(h), st(stream));
+    active_pool_backward(md(h), *l, d_in, d_out, planes, average, st(stream));
+  });
+}
+
 // ---- backward pass -----------------------------------------------------------------------------
 
 int scn_subm_conv_bwd(scn_metadata *h, const int64_t *spatial, const int64_t *filter, const float *in, float *d_in,

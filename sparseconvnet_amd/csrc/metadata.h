@@ -286,6 +286,9 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
 void input_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s);
 void output_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s);
 void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStream_t s);
+void active_pool_forward(Metadata &m, const Level &l, const float *in, float *out, int planes, int average, hipStream_t s);
+void active_pool_backward(Metadata &m, const Level &l, float *d_in, const float *d_out, int planes, int average,
+                          hipStream_t s);
 
 // backward.hip
 void subm_conv_backward(Metadata &m, Table &t, const int64_t *filter, const float *in, float *d_in,

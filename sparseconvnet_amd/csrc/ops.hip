@@ -303,4 +303,101 @@ void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStr
   LAUNCH_CHECK();
 }
 
+// ---- active pooling ------------------------------------------------------------------------
+// CPU/ActivePooling.cpp:8-25,47-63: out[sample] = sum of the sample's rows (times 1 / count with
+// average), out is [batch, planes].  The level's schedule lists rows by ascending site key and
+// the sample index is the key's top part, so every sample is one contiguous range of schedule
+// positions: start[b] .. start[b + 1].  Sums are taken in that order, in a fixed number of chunks
+// per sample, then over the chunks: the same bits on every run.
+__global__ void k_sample_starts(const int *soa, const int *sched, int dim, int64_t n, int64_t npad, int batch,
+                                int *start) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int *sample = soa + (int64_t)dim * npad;
+  const int b = sample[sched ? sched[t] : t];
+  const int before = t > 0 ? sample[sched ? sched[t - 1] : t - 1] : -1;
+  for (int q = before + 1; q <= b; q++) start[q] = (int)t;  // samples without sites begin where the next one does
+  if (t == n - 1)
+    for (int q = b + 1; q <= batch; q++) start[q] = (int)n;
+}
+// grid (sample * chunks + chunk, column tile of CW): partial[(sample * chunks + chunk) * planes + c]
+__global__ void k_active_pool_partial(const int *sched, const int *start, int chunks, const float *in, int planes,
+                                      int CW, float *partial) {
+  __shared__ float red[256];
+  const int b = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
+  const int tx = threadIdx.x % CW, ty = threadIdx.x / CW, RW = 256 / CW;
+  const int c = blockIdx.y * CW + tx;
+  const int lo = start[b], hi = start[b + 1];
+  const int per = (hi - lo + chunks - 1) / chunks;
+  const int t0 = min(hi, lo + chunk * per), t1 = min(hi, t0 + per);
+  float acc = 0.f;
+  if (c < planes)
+    for (int t = t0 + ty; t < t1; t += RW) acc += in[(int64_t)(sched ? sched[t] : t) * planes + c];
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  if (ty == 0 && c < planes) {
+    for (int q = 1; q < RW; q++) acc += red[q * CW + tx];
+    partial[(size_t)blockIdx.x * planes + c] = acc;
+  }
+}
+__global__ void k_active_pool_finish(const float *partial, const int *start, int chunks, int batch, int planes,
+                                     int average, float *out) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= batch * planes) return;
+  const int b = i / planes, c = i - b * planes;
+  float s = 0.f;
+  for (int q = 0; q < chunks; q++) s += partial[((size_t)b * chunks + q) * planes + c];
+  const int count = start[b + 1] - start[b];
+  out[i] = (average && count > 0) ? s * (1.0f / (float)count) : s;
+}
+// CPU/ActivePooling.cpp:26-44,65-83: every row receives its sample's gradient.
+__global__ void k_active_pool_bwd(const int *soa, int dim, int64_t n, int64_t npad, const int *start, int planes,
+                                  int average, const float *d_out, float *d_in) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = n * planes, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / planes;
+    const int c = (int)(i - r * planes);
+    const int b = soa[(int64_t)dim * npad + r];
+    const int count = start[b + 1] - start[b];
+    const float mult = (average && count > 0) ? 1.0f / (float)count : 1.0f;
+    d_in[i] = d_out[(int64_t)b * planes + c] * mult;
+  }
+}
+static const int *sample_starts(Metadata &m, const Level &l, hipStream_t s) {
+  m.s0.reserve(l.batch + 1);
+  k_sample_starts<<<dim3((unsigned)ceil_div(l.n, TB)), TB, 0, s>>>(l.coords.p, l.sched_ptr(), l.g.dim, l.n, l.npad,
+                                                                 l.batch, m.s0.p);
+  LAUNCH_CHECK();
+  return m.s0.p;
+}
+void active_pool_forward(Metadata &m, const Level &l, const float *in, float *out, int planes, int average,
+                         hipStream_t s) {
+  if (l.batch <= 0 || planes <= 0) return;
+  if (l.n == 0) {
+    fill32(out, 0, (int64_t)l.batch * planes, s);
+    return;
+  }
+  const int *start = sample_starts(m, l, s);
+  // about a thousand workgroups over the batch, at least 256 rows each on average
+  int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(1024, l.batch), ceil_div(l.n, (int64_t)256 * l.batch)));
+  const int CW = planes <= 16 ? 16 : planes <= 32 ? 32 : 64;
+  m.partial.reserve((size_t)l.batch * chunks * planes);
+  k_active_pool_partial<<<dim3((unsigned)(l.batch * chunks), (unsigned)ceil_div(planes, CW)), 256, 0, s>>>(
+      l.sched_ptr(), start, chunks, in, planes, CW, m.partial.p);
+  LAUNCH_CHECK();
+  k_active_pool_finish<<<dim3((unsigned)ceil_div((int64_t)l.batch * planes, TB)), TB, 0, s>>>(m.partial.p, start, chunks,
+                                                                                            l.batch, planes, average, out);
+  LAUNCH_CHECK();
+}
+void active_pool_backward(Metadata &m, const Level &l, float *d_in, const float *d_out, int planes, int average,
+                          hipStream_t s) {
+  if (l.n == 0 || planes <= 0) return;
+  const int *start = sample_starts(m, l, s);
+  const int64_t blocks = std::min<int64_t>(ceil_div(l.n * planes, TB), 256 * 64);
+  k_active_pool_bwd<<<dim3((unsigned)blocks), TB, 0, s>>>(l.coords.p, l.g.dim, l.n, l.npad, start, planes, average, d_out,
+                                                          d_in);
+  LAUNCH_CHECK();
+}
+
 }  // namespace scn

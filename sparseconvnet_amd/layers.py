@@ -127,6 +127,20 @@ def join_batchnorm(parts, bn):
     return output
 
 
+class _ActivePoolingFunction(Function):
+    """The calls pybind.cpp:34-43 binds (the reference's Python package has no module over them)."""
+
+    @staticmethod
+    def forward(ctx, features, md, spatial_size, average):
+        ctx.md, ctx.spatial_size, ctx.average, ctx.shape = md, spatial_size, average, tuple(features.shape)
+        return md.activePooling(spatial_size, features, average)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return ctx.md.activePoolingBackward(ctx.spatial_size, ctx.shape, grad_output.contiguous(), ctx.average), \
+            None, None, None
+
+
 class _PoolingFunction(Function):
     """maxPooling.py:14-72, averagePooling.py:13-66, unPooling.py:14-57: which = 'max', 'average',
     'un'.  sizes = (input level, output level, pool size, pool stride) of the op."""
@@ -615,6 +629,27 @@ class BLOutputLayer(Module):
 
     def forward(self, input):
         return _OutputLayerFunction.apply(input.features, input.metadata, True)
+
+
+class ActivePooling(Module):
+    """Sums (average=True: averages) the active rows of every sample: a dense [batchSize, nPlanes]
+    tensor, whatever the spatial size (SCN/CPU/ActivePooling.cpp:47-63, bound by pybind.cpp:34-43;
+    sparseToDense.py:9 names it as the other way out of a sparse network.  The reference ships no
+    Python class for it; the constructor follows its pooling modules)."""
+
+    def __init__(self, dimension, average=False):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.average = average
+
+    def forward(self, input):
+        return _ActivePoolingFunction.apply(input.features, input.metadata, input.spatial_size, self.average)
+
+    def input_spatial_size(self, out_size):
+        return out_size
+
+    def __repr__(self):
+        return 'ActivePooling(average)' if self.average else 'ActivePooling'
 
 
 class SparseToDense(Module):

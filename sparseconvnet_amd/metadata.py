@@ -289,6 +289,24 @@ class Metadata:
                                        _stream()))
         return out
 
+    def activePooling(self, spatial_size, features, average):
+        """ActivePooling_updateOutput (pybind.cpp:34-38): [batchSize, planes], per sample the sum
+        (average: the mean) of its active rows."""
+        features = _features(features, "features")
+        out = torch.empty((self.getBatchSize(spatial_size), features.size(1)), dtype=torch.float32,
+                          device=features.device)
+        _lib.check(self._L.scn_active_pooling_fwd(self._h, self._s(spatial_size), _ptr(features), _ptr(out),
+                                                  features.size(1), int(bool(average)), _stream()))
+        return out
+
+    def activePoolingBackward(self, spatial_size, shape, grad_output, average):
+        """ActivePooling_updateGradInput (pybind.cpp:39-43): shape = that of the op's input."""
+        grad_output = _features(grad_output, "grad_output")
+        d_in = torch.empty(shape, dtype=torch.float32, device=grad_output.device)
+        if d_in.numel():
+            _lib.check(self._L.scn_active_pooling_bwd(self._h, self._s(spatial_size), _ptr(d_in), _ptr(grad_output),
+                                                      shape[1], int(bool(average)), _stream()))
+        return d_in
 
     # ---- backward ops: each returns the gradients the reference's backward call fills ----------
     def _convBackward(self, fn, size_args, features, grad_output, weight, with_bias):

@@ -392,6 +392,42 @@ def check_s2d(make, dim, seed, spatial=6, n=80, batch=3, C=4):
     assert sum(len(r) for r in rules) == len(loc)
 
 
+def check_active_pooling(make, dim, seed, spatial=6, n=90, batch=4, C=5):
+    """ActivePooling forward and backward (CPU/ActivePooling.cpp:8-83) against the closed form: per
+    sample the sum / mean of its rows, and that sample's gradient (times 1 / count) back to each of
+    its rows.  Two inputs: samples of many sites, one of them empty (where the compiled reference's
+    rule builder does not return and its adapter answers None), and samples of exactly one site
+    each (where it returns: the one input on which the reference itself can be asked)."""
+    rng = np.random.default_rng(seed)
+    for single in (False, True):
+        if single:
+            coords = np.concatenate([rng.integers(0, spatial, size=(batch, dim)), np.arange(batch)[:, None]], 1)
+        else:
+            coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=n // 4)
+            coords = coords[coords[:, -1] != 1]  # sample 1 stays empty
+        feats = rng.normal(size=(len(coords), C)).astype(np.float32)
+        p = make(dim)
+        p.input_layer(spatial, coords, batch, 3)
+        loc = p.spatial_locations(spatial)
+        x = p.input_fwd(feats)
+        d_out = rng.normal(size=(batch, C)).astype(np.float32)
+        for average in (False, True):
+            got = p.active_pooling(spatial, x, average)
+            got_b = p.active_pooling_bwd(spatial, d_out, average)
+            if got is None:  # the compiled reference on an input its rule builder cannot handle
+                assert not single and got_b is None
+                continue
+            want = np.zeros((batch, C))
+            count = np.bincount(loc[:, -1], minlength=batch)
+            np.add.at(want, loc[:, -1], x.astype(np.float64))
+            mult = np.where(count > 0, 1.0 / np.maximum(count, 1), 1.0) if average else np.ones(batch)
+            assert got.shape == (batch, C)
+            assert_close(got, want * mult[:, None], "active pooling, average=%s" % average)
+            assert_close(got_b, (d_out * mult[:, None])[loc[:, -1]], "active pooling gradient, average=%s" % average)
+        if single:
+            assert got is not None
+
+
 def check_level_replacement(make, seed=11):
     """What happens to a level that is built twice, as the reference does it
     (Metadata/ConvolutionRules.h:68-70, Metadata/Metadata.cpp:492-518, CPU/Deconvolution.cpp:15-18):

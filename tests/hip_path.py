@@ -417,6 +417,20 @@ class HipPath:
         _lib.check(self.L.scn_output_layer_bwd(self.h, _ptr(d_in), _ptr(dd), d_out.shape[-1], _stream()))
         return d_in.cpu().numpy()
 
+    def active_pooling(self, spatial, x, average=False):
+        xd = _dev(x, torch.float32)
+        out = torch.full((self.batch_size(spatial), x.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_active_pooling_fwd(self.h, self._s(spatial), _ptr(xd), _ptr(out), x.shape[1], int(average),
+                                                 _stream()))
+        return out.cpu().numpy()
+
+    def active_pooling_bwd(self, spatial, d_out, average=False):
+        dd = _dev(d_out, torch.float32)
+        d_in = torch.full((self.nactive(spatial), d_out.shape[1]), float("nan"), dtype=torch.float32, device="cuda")
+        _lib.check(self.L.scn_active_pooling_bwd(self.h, self._s(spatial), _ptr(d_in), _ptr(dd), d_out.shape[1],
+                                                 int(average), _stream()))
+        return d_in.cpu().numpy()
+
     def s2d_bwd(self, spatial, d_out):
         dd = _dev(d_out, torch.float32)
         d_in = torch.full((self.nactive(spatial), d_out.shape[1]), float("nan"), dtype=torch.float32, device="cuda")

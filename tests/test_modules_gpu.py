@@ -696,3 +696,28 @@ def test_reference_state_dict_reproduces_reference_output():
                 checks.assert_close(model(x).cpu().numpy(), io["out"], "unfused, output of the reference's checkpoint")
         finally:
             scn.fuse_batchnorm = True
+
+
+def test_active_pooling_module():
+    """ActivePooling at the end of a network: per-sample sums / means of the rows, and autograd
+    through it (each row receives its sample's gradient, scaled by 1 / count when averaging)."""
+    coords = synthetic.scene_batch(seed=5200, batch=3, target=2000, spatial=48, n_boxes=4, duplicate_fraction=0.0)
+    feats = torch.randn((len(coords), 6), device="cuda", requires_grad=True)
+    x = scn.InputLayer(3, 48, mode=3)([torch.as_tensor(coords), feats])
+    sample = x.metadata.getSpatialLocations(x.spatial_size)[:, -1].cuda()
+    for average in (False, True):
+        y = scn.ActivePooling(3, average)(x)
+        want = torch.zeros((3, 6), device="cuda").index_add_(0, sample, x.features.detach())
+        count = torch.bincount(sample, minlength=3).float()
+        if average:
+            want = want / count[:, None]
+        assert y.shape == (3, 6)
+        checks.assert_close(y.detach().cpu().numpy(), want.cpu().numpy(), "active pooling module")
+        g = torch.randn((3, 6), device="cuda")
+        feats.grad = None
+        (y * g).sum().backward()
+        # mode 3 without repeated points: input rows are the level's rows
+        expect = g[sample] / (count[sample][:, None] if average else 1.0)
+        rows = x.metadata.getSpatialLocations(x.spatial_size)
+        assert len(rows) == len(coords)
+        checks.assert_close(feats.grad.cpu().numpy(), expect.cpu().numpy(), "active pooling module gradient")

@@ -91,6 +91,11 @@ def test_s2d(make, dim):
     checks.check_s2d(make, dim, seed=2 + dim)
 
 
+@pytest.mark.parametrize("dim", [1, 2, 3, 4])
+def test_active_pooling(make, dim):
+    checks.check_active_pooling(make, dim, seed=70 + dim)
+
+
 def test_level_replacement(make):
     checks.check_level_replacement(make)
 
