@@ -287,6 +287,22 @@ int scn_bn_eval_fwd(const float *in, float *out, int64_t rows, int planes, int64
 int scn_s2d_fwd(scn_metadata *md, const int64_t *spatial, const float *in, float *out,
                 int planes, void *stream);
 
+/* Parameters that do not change between calls (inference).  A convolution call derives two things
+ * from its parameters before it can run: the weights in the operand order of the matrix
+ * instructions, and each fused batch norm folded to scale / shift; by default on every call.  A
+ * scn_params object keeps them: scn_md_use_params(md, p) makes the NEXT convolution call on md
+ * (scn_subm_conv_fwd, scn_conv_fwd, scn_deconv_fwd, scn_conv_bn_fwd, scn_nin_fwd) take what p holds
+ * and add what it lacks.  The caller promises that the weight, bias and batch-norm arrays passed
+ * with p are the same arrays with the same contents every time, until scn_params_clear(p) (after
+ * an optimiser step, a load_state_dict) or scn_params_destroy(p); one object per convolution
+ * module.  Results are bit-identical with and without.  No counterpart in the reference, whose
+ * kernels read the weights as stored (CUDA/Convolution.cu:444-521). */
+typedef struct scn_params scn_params;
+scn_params *scn_params_create(void);
+void scn_params_destroy(scn_params *p);
+int scn_params_clear(scn_params *p);
+int scn_md_use_params(scn_metadata *md, scn_params *p);
+
 /* ActivePooling_updateOutput / ActivePooling_updateGradInput (pybind.cpp:34-43,
  * CPU/ActivePooling.cpp:8-83): out [batchSize, planes] = per sample the sum of its active rows, times
  * 1 / count when average != 0; d_in [nActive, planes] = the sample's gradient for each of its rows

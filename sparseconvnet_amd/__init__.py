@@ -12,6 +12,18 @@ forward_pass_hidden_states = 0
 # convolution to that convolution (one pass over the rows instead of two).  False: run
 # every module as a pass of its own.
 fuse_batchnorm = True
+# Eval-mode convolution modules keep what they derive from their parameters (weights in the matrix
+# instructions' operand order, folded batch norms) between calls, keyed on every parameter tensor's
+# address and version counter.  parameters_changed() drops all of it (needed only after writes that
+# bypass the version counter, i.e. through tensor.data).
+frozen_parameters = True
+_parameter_epoch = 0
+
+
+def parameters_changed():
+    global _parameter_epoch
+    _parameter_epoch += 1
+
 # True: every Metadata created from now on runs its wide convolutions (more than 32 output
 # planes, or 128 and more input planes) with bf16 operands and fp32 accumulation.  The
 # reference computes in fp32 throughout, which is also the default here.

@@ -51,6 +51,10 @@ SIGNATURES = {
     "scn_subm_conv_fwd_noalloc": (C.c_int, [_vp, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_take_released_macs": (C.c_int, [C.POINTER(C.c_double)]),
     "scn_release_cache": (C.c_int, []),
+    "scn_params_create": (_vp, []),
+    "scn_params_destroy": (None, [_vp]),
+    "scn_params_clear": (C.c_int, [_vp]),
+    "scn_md_use_params": (C.c_int, [_vp, _vp]),
     "scn_active_pooling_fwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_active_pooling_bwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_sort_pairs": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, _vp]),

@@ -8,6 +8,9 @@ using namespace scn;
 struct scn_metadata {
   Metadata m;
 };
+struct scn_params {
+  FrozenParams p;
+};
 
 static thread_local std::string g_error;
 
@@ -883,6 +886,24 @@ int scn_s2d_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float 
   });
 }
 
+scn_params *scn_params_create(void) {
+  try {
+    return new scn_params();
+  } catch (const std::exception &e) {
+    g_error = e.what();
+    return nullptr;
+  }
+}
+void scn_params_destroy(scn_params *p) { delete p; }
+int scn_params_clear(scn_params *p) {
+  return guarded([&] {
+    if (!p) throw Error("null parameter set");
+    p->p.clear();
+  });
+}
+int scn_md_use_params(scn_metadata *h, scn_params *p) {
+  return guarded([&] { md(h).frozen = p ? &p->p : nullptr; });
+}
 int scn_active_pooling_fwd(scn_metadata *h, const int64_t *spatial, const float *in, float *out, int planes,
                            int average, void *stream) {
   return guarded([&] {

@@ -345,6 +345,7 @@ static void input_gradient(Metadata &m, const Table &t, const float *d_out, int6
   m.wt.reserve(wn);
   k_transpose_weights<<<grid_for(wn), TB, 0, s>>>(w, m.wt.p, t.K, groups, n_in / groups, n_out / groups, mirror ? 1 : 0);
   LAUNCH_CHECK();
+  m.frozen = nullptr;  // the transposed weights are scratch of this call
   conv_forward(m, t, d_out, d_out_rows, d_in, m.wt.p, nullptr, n_out, n_in, groups, nullptr, nullptr, s);
 }
 

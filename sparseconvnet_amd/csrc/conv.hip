@@ -63,10 +63,35 @@ static float *scratch_wpack(Metadata &m, size_t floats) {
   m.wpack.reserve(floats);
   return m.wpack.p;
 }
-static int *scratch_queue(Metadata &m) {
+// Nine counters 128 bytes apart: one per XCD for the sets handed out, one for the workgroups that
+// have finished.  They are zero between launches: static device memory starts as zeros, the
+// handle's buffer is cleared when it is allocated, and the last workgroup of every launch clears
+// them again.
+static int *scratch_queue(Metadata &m, hipStream_t s) {
   if (m.fixed_scratch) return reinterpret_cast<int *>(m.fixed_scratch);
-  m.queue.reserve(8 * 32);
+  if (!m.queue_zeroed) {
+    m.queue.reserve(9 * 32);
+    fill32(m.queue.p, 0, 9 * 32, s);
+    m.queue_zeroed = true;
+  }
   return m.queue.p;
+}
+// The weights of the running convolution in the layout `key` names, `floats` long: from the
+// caller's frozen set when there is one (packed by `pack(dst)` the first time), else packed into
+// the handle's scratch on every call.
+template <class F>
+static float *packed_weights(Metadata &m, std::vector<int64_t> key, size_t floats, F pack) {
+  if (m.frozen && !m.fixed_scratch) {
+    auto it = m.frozen->packed.find(key);
+    if (it != m.frozen->packed.end() && it->second.cap >= floats) return it->second.p;
+    DevBuf<float> &b = m.frozen->packed[key];
+    b.reserve(floats);
+    pack(b.p);
+    return b.p;
+  }
+  float *dst = scratch_wpack(m, floats);
+  pack(dst);
+  return dst;
 }
 // Partial tiles for n_split workgroups per tile; with the static scratch n_split shrinks until
 // they fit (1: no partial tiles at all).
@@ -544,10 +569,11 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   const int cin16 = (int)ceil_div(n_in, 16);
   const int n_slab = (int)ceil_div(cin16, SS);
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
-  float *wpack = scratch_wpack(m, packed);
-  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m), BF16);
-  LAUNCH_CHECK();
+  float *wpack = packed_weights(m, {0, (int64_t)(uintptr_t)w, t.K, n_in, n_out, SS, NCB, BF16}, packed, [&](float *dst) {
+    k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, dst, t.K, n_in, n_out, n_slab, SS, NCB,
+                                                                        SLAB_STRIDE, take_jobs(m), BF16);
+    LAUNCH_CHECK();
+  });
   auto kern = k_conv_mfma<NCBW, WC, GW, SS, VEC4, PRE, BUF, BF16>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -912,10 +938,11 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   const int cin16 = (int)ceil_div(n_in, 16);
   const int n_slab = (int)ceil_div(cin16, SS);
   const int64_t packed = (int64_t)t.K * n_slab * SLAB_STRIDE;
-  float *wpack = scratch_wpack(m, packed);
-  k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, n_slab,
-                                                                      SS, NCB, SLAB_STRIDE, take_jobs(m), BF16);
-  LAUNCH_CHECK();
+  float *wpack = packed_weights(m, {0, (int64_t)(uintptr_t)w, t.K, n_in, n_out, SS, NCB, BF16}, packed, [&](float *dst) {
+    k_pack_weights<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, dst, t.K, n_in, n_out, n_slab, SS, NCB,
+                                                                        SLAB_STRIDE, take_jobs(m), BF16);
+    LAUNCH_CHECK();
+  });
   auto kern = k_conv_rows<NCB, RG, SS, VEC4, NW, PRE, BUF, BF16>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -1254,6 +1281,15 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     if (!I0.valid) break;
     step(std::integral_constant<int, 2>{});
   }
+  // The last workgroup to get here leaves the counters at zero for the next launch (every
+  // workgroup has taken its last set by now: nobody adds to them any more).
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    if (atomicAdd(queue + 8 * 32, 1) == (int)gridDim.x - 1) {
+      for (int i = 0; i < 9; i++) queue[i * 32] = 0;
+    }
+  }
 }
 
 // B operands of the four-channel layout: wp[(k * NCB + cb) * 64 + lane] = w[k][lane / 16][16 cb + lane % 16].
@@ -1271,8 +1307,8 @@ __global__ void k_pack_weights_c4(const float *w, float *wp, int K, int n_in, in
 
 template <int NCB, int RG, int SS, bool VEC4, int WAVES, bool C4, bool BUF = false, bool BF16 = false>
 static void launch_resident_kernel(Metadata &m, const Table &t, const float *in, int in_stride, float *out,
-                                   Epi epi, int n_in_part, int n_out, int accumulate, size_t lds_bytes,
-                                   int per_cu, hipStream_t s) {
+                                   const float *wpack, Epi epi, int n_in_part, int n_out, int accumulate,
+                                   size_t lds_bytes, int per_cu, hipStream_t s) {
   // bytes from `in` (which may point at a channel offset inside the first row) to the end
   const int64_t in_bytes = (m.cur_in_rows * in_stride - (in - m.cur_in_base)) * 4;
   const int64_t nbr_bytes = (int64_t)t.K * t.npad * 4;
@@ -1280,7 +1316,7 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
     const bool whole = C4 || n_in_part == 16 * SS;
     if (whole && m.cur_in_rows > 0 && m.cur_in_rows < (1 << 24) && in_stride * 4 < (1 << 24) && in_bytes > 0 &&
         in_bytes < ((int64_t)1 << 31) && nbr_bytes < ((int64_t)1 << 31)) {
-      launch_resident_kernel<NCB, RG, SS, VEC4, WAVES, C4, true, BF16>(m, t, in, in_stride, out, epi, n_in_part,
+      launch_resident_kernel<NCB, RG, SS, VEC4, WAVES, C4, true, BF16>(m, t, in, in_stride, out, wpack, epi, n_in_part,
                                                                        n_out, accumulate, lds_bytes, per_cu, s);
       return;
     }
@@ -1299,8 +1335,8 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
   const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
   kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
-                                                   out, scratch_wpack(m, 0), epi, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                   accumulate, scratch_queue(m), (unsigned)in_bytes, (unsigned)nbr_bytes);
+                                                   out, wpack, epi, n_in_part, n_out, n_sets, sets_per_xcd,
+                                                   accumulate, scratch_queue(m, s), (unsigned)in_bytes, (unsigned)nbr_bytes);
   LAUNCH_CHECK();
   }
 }
@@ -1320,38 +1356,38 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
                                  int n_out, int accumulate, hipStream_t s) {
   constexpr int RG = 2;  // 32 rows per set: measured faster than 64 (more wavefronts in flight)
   const int64_t packed = (int64_t)t.K * SS * NCB * 256;
-  float *wpack = scratch_wpack(m, packed);
-  int *queue = scratch_queue(m);
+  int *queue = scratch_queue(m, s);
+  bool bf16 = false;
+  if constexpr (SS == 2 && VEC4)  // bf16 operands (when asked for): a whole 32-channel part, buffer gathers
+    bf16 = m.bf16 && n_in_part == 32 && resident_buffer_gathers(m, t, in, in_stride);
+  // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
+  const float *wpack = packed_weights(m, {1, (int64_t)(uintptr_t)w, t.K, w_in_stride_rows, n_in_part, n_out, SS, NCB, bf16},
+                                      packed, [&](float *dst) {
+    k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, dst, t.K, w_in_stride_rows, n_in_part,
+                                                                             n_out, SS, NCB, queue, take_jobs(m), bf16);
+    LAUNCH_CHECK();
+  });
   if constexpr (SS == 2 && VEC4) {
-    // bf16 operands (when asked for): a whole 32-channel part, buffer gathers
-    if (m.bf16 && n_in_part == 32 && resident_buffer_gathers(m, t, in, in_stride)) {
-      k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(
-          w, wpack, t.K, w_in_stride_rows, n_in_part, n_out, SS, NCB, queue, take_jobs(m), true);
-      LAUNCH_CHECK();
+    if (bf16) {
       const size_t lds16 = (size_t)packed * 2;  // 2-byte elements
       const int per_cu16 = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds16));
       if (lds16 > 80 * 1024)
-        launch_resident_kernel<NCB, RG, SS, VEC4, 16, false, true, true>(m, t, in, in_stride, out, epi, n_in_part, n_out,
-                                                                         accumulate, lds16, 1, s);
+        launch_resident_kernel<NCB, RG, SS, VEC4, 16, false, true, true>(m, t, in, in_stride, out, wpack, epi, n_in_part,
+                                                                         n_out, accumulate, lds16, 1, s);
       else
-        launch_resident_kernel<NCB, RG, SS, VEC4, 8, false, true, true>(m, t, in, in_stride, out, epi, n_in_part, n_out,
-                                                                        accumulate, lds16, per_cu16, s);
+        launch_resident_kernel<NCB, RG, SS, VEC4, 8, false, true, true>(m, t, in, in_stride, out, wpack, epi, n_in_part,
+                                                                        n_out, accumulate, lds16, per_cu16, s);
       return;
     }
   }
-  // weights of this channel range: rows [c_lo, c_lo + n_in_part) of every tap's [nIn x nOut] slice
-  k_pack_weights_part<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, w_in_stride_rows,
-                                                                           n_in_part, n_out, SS, NCB, queue,
-                                                                           take_jobs(m));
-  LAUNCH_CHECK();
   const size_t lds_bytes = (size_t)packed * sizeof(float);
   if (lds_bytes > 80 * 1024) {
-    launch_resident_kernel<NCB, RG, SS, VEC4, 16, false>(m, t, in, in_stride, out, epi, n_in_part, n_out, accumulate,
-                                                         lds_bytes, 1, s);
+    launch_resident_kernel<NCB, RG, SS, VEC4, 16, false>(m, t, in, in_stride, out, wpack, epi, n_in_part, n_out,
+                                                         accumulate, lds_bytes, 1, s);
   } else {
     const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / std::max<size_t>(lds_bytes, 1)));
-    launch_resident_kernel<NCB, RG, SS, VEC4, 8, false>(m, t, in, in_stride, out, epi, n_in_part, n_out, accumulate,
-                                                        lds_bytes, per_cu, s);
+    launch_resident_kernel<NCB, RG, SS, VEC4, 8, false>(m, t, in, in_stride, out, wpack, epi, n_in_part, n_out,
+                                                        accumulate, lds_bytes, per_cu, s);
   }
 }
 
@@ -1361,15 +1397,18 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
                                Epi epi, int n_in, int n_out, hipStream_t s) {
   if (in == m.cur_in_base && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
     // epi.sc / epi.sh point at arrays nobody fills on this path: the kernel folds the batch norm itself
-    conv_first_forward(t, in, m.cur_in_rows, out, w, epi.bias, take_jobs(m).post, epi.leak, n_in, n_out, s);
+    take_jobs(m);
+    conv_first_forward(t, in, m.cur_in_rows, out, w, epi.bias, m.post_raw, epi.leak, n_in, n_out, s);
     return;
   }
   const int packed = t.K * NCB * 64;
-  float *wpack = scratch_wpack(m, packed);
-  k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, wpack, t.K, n_in, n_out, NCB,
-                                                                        scratch_queue(m), take_jobs(m));
-  LAUNCH_CHECK();
-  launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, epi, n_in, n_out, 0,
+  int *queue = scratch_queue(m, s);
+  const float *wpack = packed_weights(m, {2, (int64_t)(uintptr_t)w, t.K, n_in, n_out, NCB}, packed, [&](float *dst) {
+    k_pack_weights_c4<<<dim3((unsigned)ceil_div(packed, 256)), 256, 0, s>>>(w, dst, t.K, n_in, n_out, NCB, queue,
+                                                                          take_jobs(m));
+    LAUNCH_CHECK();
+  });
+  launch_resident_kernel<NCB, 4, 1, false, 8, true>(m, t, in, n_in, out, wpack, epi, n_in, n_out, 0,
                                                     (size_t)packed * sizeof(float), 3, s);
 }
 
@@ -1488,6 +1527,10 @@ static bool conv_mfma_paths(Metadata &m, const Table &t, const float *in, float 
 void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
                   const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, const BnArgs *post,
                   hipStream_t s) {
+  struct FrozenReset {  // a frozen set serves one call
+    Metadata &m;
+    ~FrozenReset() { m.frozen = nullptr; }
+  } frozen_reset{m};
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (t.n == 0) return;
@@ -1498,23 +1541,41 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   m.jobs = CoefJobs();
   m.cur_in_rows = n_in_rows;
   m.cur_in_base = in;
+  FrozenParams *frozen = m.fixed_scratch ? nullptr : m.frozen;
+  m.post_raw = CoefJob();
   if (post) {
-    m.postbuf.reserve(2 * (size_t)n_out);
-    m.jobs.post = CoefJob{post->mean, post->var, post->gamma, post->beta, post->eps, n_out, n_out, m.postbuf.p,
-                          m.postbuf.p + n_out};
-    epi.sc = m.postbuf.p;
-    epi.sh = m.postbuf.p + n_out;
+    DevBuf<float> &buf = frozen ? frozen->post : m.postbuf;
+    buf.reserve(2 * (size_t)n_out);
+    m.jobs.post = CoefJob{post->mean, post->var, post->gamma, post->beta, post->eps, n_out, n_out, buf.p, buf.p + n_out};
+    m.post_raw = m.jobs.post;
+    epi.sc = buf.p;
+    epi.sh = buf.p + n_out;
     epi.leak = post->leak;
   }
-  if (bn && groups == 1 && !resident_fits(m, t, n_in, n_out, true)) {
+  const bool pre_fused = bn && groups == 1 && !resident_fits(m, t, n_in, n_out, true);
+  PreArgs pre;
+  if (pre_fused) {
     const int n_pad = (int)round_up(n_in, 64) + 64;
-    m.prebuf.reserve(2 * (size_t)n_pad);
-    m.jobs.pre = CoefJob{bn->mean, bn->var, bn->gamma, bn->beta, bn->eps, n_in, n_pad, m.prebuf.p,
-                         m.prebuf.p + n_pad};
-    PreArgs pre;
-    pre.sc = m.prebuf.p;
-    pre.sh = m.prebuf.p + n_pad;
+    DevBuf<float> &buf = frozen ? frozen->pre : m.prebuf;
+    buf.reserve(2 * (size_t)n_pad);
+    m.jobs.pre = CoefJob{bn->mean, bn->var, bn->gamma, bn->beta, bn->eps, n_in, n_pad, buf.p, buf.p + n_pad};
+    pre.sc = buf.p;
+    pre.sh = buf.p + n_pad;
     pre.leak = bn->leak;
+  }
+  if (frozen) {
+    // folded once, by a launch of their own (the packing launches that normally fold them on the
+    // side do not run when the packed weights are found)
+    if (frozen->post_done) m.jobs.post = CoefJob();
+    if (frozen->pre_done) m.jobs.pre = CoefJob();
+    if (m.jobs.post.n_pad || m.jobs.pre.n_pad) {
+      k_coefs<<<dim3(1), 256, 0, s>>>(take_jobs(m));
+      LAUNCH_CHECK();
+    }
+    frozen->post_done = frozen->post_done || post != nullptr;
+    frozen->pre_done = frozen->pre_done || pre_fused;
+  }
+  if (pre_fused) {
     if (conv_mfma_paths<true>(m, t, in, out, w, epi, n_in, n_out, pre, s)) return;
     m.jobs.pre = CoefJob();
   }

@@ -105,6 +105,23 @@ struct CoefJobs {
   CoefJob pre, post;
 };
 
+// What a convolution derives from its parameters before it can run: the weights in MFMA operand
+// order (one buffer per layout: the kernel taken depends on the level's size and on the bf16
+// switch) and batch-norm statistics folded to scale / shift.  Normally derived on every call into
+// the handle's scratch; a caller that knows its parameters unchanged between calls (inference)
+// hands the convolution one of these objects to keep them in (scn_params_create).
+struct FrozenParams {
+  std::map<std::vector<int64_t>, DevBuf<float>> packed;
+  DevBuf<float> pre, post;   // scale | shift arrays, as conv_forward lays them out
+  bool pre_done = false, post_done = false;
+  void clear() {
+    packed.clear();
+    pre.release();
+    post.release();
+    pre_done = post_done = false;
+  }
+};
+
 struct InputRules {
   int mode = -1;      // 1: the first point of a site is listed, 2: the last, 3 / 4: all (sum / mean),
                       // 5: the first, unless later points of the site carry an overwrite flag: then the last of those
@@ -160,6 +177,10 @@ struct Metadata {
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups; partial sums of reductions
   DevBuf<float> wt;       // transposed weights of the input-gradient convolution of a backward pass
   DevBuf<int> queue;      // set counters of the resident-weights convolution kernel
+  // The next convolution keeps its packed weights and folded batch norms here and takes what it
+  // finds (scn_md_use_params; reset by every convolution call).
+  FrozenParams *frozen = nullptr;
+  bool queue_zeroed = false;  // `queue` has been cleared once (the kernel that uses it leaves it cleared)
   // Non-null while an allocation-free convolution runs: the three buffers above are then fixed
   // regions of a static device array (conv.hip) and nothing may be reserved.
   unsigned char *fixed_scratch = nullptr;
@@ -170,6 +191,7 @@ struct Metadata {
   int64_t cur_in_rows = 0;  // rows and start of the input matrix of the convolution being launched
   const float *cur_in_base = nullptr;
   CoefJobs jobs;          // coefficient arrays the next weight-packing launch has to fill
+  CoefJob post_raw;       // the running convolution's batch norm behind it, for the kernel that folds it itself
   DevBuf<float> postbuf;  // scale / shift of a batch norm fused into the running convolution's stores
   DevBuf<float> prebuf;   // scale / shift of a batch norm fused into the running convolution
   DevBuf<float> bntmp;    // normalised input when a fused batch norm has no fused kernel

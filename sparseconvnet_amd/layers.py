@@ -19,6 +19,57 @@ def _opt(t):
     return t if t is not None and t.numel() else None
 
 
+class _FrozenParams:
+    """What a convolution module keeps between eval-mode calls: a scn_params object of the library
+    (packed weights, folded batch norms) and the state of the tensors it was derived from.  The
+    state is (address, version counter) per tensor: optimiser steps, load_state_dict, .cuda() and
+    every other in-place write or replacement change it, and the object is cleared.  Writes
+    through `tensor.data` do not move the version counter: after such a write in eval mode call
+    sparseconvnet_amd.parameters_changed(), or switch sparseconvnet_amd.frozen_parameters off."""
+
+    def __init__(self):
+        self.handle, self.state, self.epoch = None, None, -1
+
+    def use(self, md, tensors):
+        if not _pkg.frozen_parameters:
+            return
+        L = _md._lib.lib()
+        state = tuple((t.data_ptr(), t._version) for t in tensors if t is not None)
+        if self.handle is None:
+            self.handle = L.scn_params_create()
+        if state != self.state or self.epoch != _pkg._parameter_epoch:
+            _md._lib.check(L.scn_params_clear(self.handle))
+            self.state, self.epoch = state, _pkg._parameter_epoch
+        _md._lib.check(L.scn_md_use_params(md._h, self.handle))
+
+    def __deepcopy__(self, memo):  # a copied or unpickled module starts with nothing kept
+        return _FrozenParams()
+
+    def __reduce__(self):
+        return (_FrozenParams, ())
+
+    def __del__(self):
+        try:
+            if self.handle is not None:
+                _md._lib.lib().scn_params_destroy(self.handle)
+        except Exception:
+            pass
+
+
+def _use_frozen(module, md, weight, bias, pre=None, post=None):
+    """Eval mode: the module's convolution may keep what it derives from its parameters."""
+    if module.training:
+        return
+    f = module.__dict__.get('_frozen')
+    if f is None:
+        f = module.__dict__['_frozen'] = _FrozenParams()
+    tensors = [weight, bias]
+    for bn in (pre, post):
+        if bn is not None:
+            tensors += list(bn[:4])
+    f.use(md, tensors)
+
+
 class _ConvFunction(Function):
     """submanifoldConvolution.py:63-113, convolution.py:72-130, deconvolution.py:49-128: kind 0 /
     1 / 2.  pre / post: eval-mode batch norms applied inside the convolution (inference only)."""
@@ -297,8 +348,10 @@ class SubmanifoldConvolution(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
+        pre, post = _bn_args(pre_bn), _bn_args(post_bn)
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 0,
-                                              (input.spatial_size, self.filter_size), _bn_args(pre_bn), _bn_args(post_bn))
+                                              (input.spatial_size, self.filter_size), pre, post)
         return output
 
     def __repr__(self):
@@ -337,8 +390,10 @@ class Convolution(Module):
         assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
             input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        pre, post = _bn_args(pre_bn), _bn_args(post_bn)
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 1,
-                                              a, _bn_args(pre_bn), _bn_args(post_bn))
+                                              a, pre, post)
         return output
 
     def __repr__(self):
@@ -371,8 +426,10 @@ class Deconvolution(Module):
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
         a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        pre, post = _bn_args(pre_bn), _bn_args(post_bn)
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 2,
-                                              a, _bn_args(pre_bn), _bn_args(post_bn))
+                                              a, pre, post)
         return output
 
     def __repr__(self):
@@ -403,6 +460,7 @@ class NetworkInNetwork(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'))
         output.features = _NetworkInNetworkFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'),
                                                           input.metadata)
         return output

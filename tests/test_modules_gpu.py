@@ -721,3 +721,57 @@ def test_active_pooling_module():
         rows = x.metadata.getSpatialLocations(x.spatial_size)
         assert len(rows) == len(coords)
         checks.assert_close(feats.grad.cpu().numpy(), expect.cpu().numpy(), "active pooling module gradient")
+
+
+def test_frozen_parameters_agree_and_follow_changes():
+    """Eval-mode modules keep their packed weights and folded batch norms between calls: results
+    are bit-identical with the cache on and off, a second call (which packs nothing) repeats the
+    first, and a changed weight or statistic (in-place write, load_state_dict) is seen."""
+    torch.manual_seed(12)
+    m = 16
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 1, [m, 2 * m, 3 * m], True)).add(scn.BatchNormReLU(m)).add(scn.OutputLayer(3)).cuda().eval()
+    randomise_bn(model, 12)
+    coords = synthetic.room_scene(seed=9300, target=20000, spatial=256, duplicate_fraction=0.2)
+    feats = torch.rand((len(coords), 3), device="cuda")
+    layer = scn.InputLayer(3, 256, mode=4)
+
+    def run():
+        with torch.no_grad():
+            return model(layer([torch.as_tensor(coords), feats])).clone()
+
+    scn.frozen_parameters = False
+    try:
+        plain = run()
+    finally:
+        scn.frozen_parameters = True
+    first, second = run(), run()
+    assert torch.equal(first, plain) and torch.equal(second, plain)
+    conv = [mod for mod in model.modules() if isinstance(mod, scn.SubmanifoldConvolution)][3]
+    bn = [mod for mod in model.modules() if isinstance(mod, scn.BatchNormalization)][2]
+    with torch.no_grad():
+        conv.weight.mul_(1.5)
+        bn.running_var.add_(0.25)
+    changed = run()
+    assert not torch.equal(changed, plain)
+    scn.frozen_parameters = False
+    try:
+        assert torch.equal(run(), changed)
+    finally:
+        scn.frozen_parameters = True
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    with torch.no_grad():
+        for p in model.parameters():
+            p.mul_(0.5)
+    assert not torch.equal(run(), changed)
+    model.load_state_dict(state)
+    assert torch.equal(run(), changed)
+    with torch.no_grad():
+        conv.weight.data.mul_(2.0)   # a write the version counter does not see ...
+    scn.parameters_changed()         # ... announced by hand
+    scn.frozen_parameters = False
+    try:
+        want = run()
+    finally:
+        scn.frozen_parameters = True
+    assert torch.equal(run(), want) and not torch.equal(want, changed)
