@@ -33,6 +33,10 @@ struct Level {
   DevBuf<int> urow;
   bool grid_built = false;
   bool dups = false;
+  // Active-site counts of the levels that successive filter 2 / stride 2 rulebooks make of this
+  // one (size halved once, twice, ...), when somebody has computed them (metadata.hip:
+  // halving_sizes): a strided build that finds its output size here needs no read-back.
+  std::vector<int64_t> halvings;
   const int *urow_ptr() const { return dups ? urow.p : sched_ptr(); }
   const int *sched_ptr() const { return identity_sched ? nullptr : sched.p; }
 };

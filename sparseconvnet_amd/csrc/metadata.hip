@@ -1106,8 +1106,11 @@ __device__ inline bool candidate(const Geom &gi, const Filt &f, const int *p, in
   return true;
 }
 
+// zero: 16 x 64 counters that the launch behind this one (k_strided_heads) adds to, or null.
 __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, const int *sched,
-                                     int64_t n, int64_t npad, unsigned long long *keys, int *payload) {
+                                     int64_t n, int64_t npad, unsigned long long *keys, int *payload, int *zero) {
+  if (zero && blockIdx.x == 0)
+    for (int i = threadIdx.x; i < 16 * 64; i += blockDim.x) zero[i] = 0;
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n * f.M) return;
   int64_t t = e / f.M;
@@ -1120,11 +1123,39 @@ __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, c
   payload[e] = (int)e;
 }
 
-__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head) {
+// head[p] = 1 where a new output site begins in the sorted candidate keys.
+// counts (optional; filter = stride = 2 over exactly halving sizes, Morton keys): the sizes of the
+// levels that further halvings will make.  Two sites fall into the same site j halvings further
+// down iff their keys agree above the low dim * j bits (a Morton key drops one bit per coordinate
+// per halving; the sample index sits above), so in ascending key order a position starts a new
+// site on every level up to (highest bit in which it differs from its predecessor) / dim, and one
+// pass counts the sites of all levels: counts[j], j = 0 .. levels.  The whole chain of levels
+// then costs one read-back instead of one per level.
+__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head, int dim, int levels,
+                                int *counts) {
+  __shared__ int hist[64];
+  if (counts) {
+    if (threadIdx.x < 64) hist[threadIdx.x] = 0;
+    __syncthreads();
+  }
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p == n) head[p] = 0;  // one element past the end, so that a scan of n + 1 ends with the total
-  if (p >= n) return;
-  head[p] = (skeys[p] != SCN_EMPTY_KEY && (p == 0 || skeys[p] != skeys[p - 1])) ? 1 : 0;
+  int top = -1;  // a new site on levels 0 .. top
+  if (p < n) {
+    const unsigned long long k = skeys[p], d = p ? k ^ skeys[p - 1] : ~0ull;
+    head[p] = (k != SCN_EMPTY_KEY && d != 0ull) ? 1 : 0;
+    if (counts && k != SCN_EMPTY_KEY && d != 0ull) top = p ? min(levels, (63 - __clzll((long long)d)) / dim) : levels;
+  }
+  if (!counts) return;
+  for (int l = 0; l <= levels; l++) {
+    const unsigned long long b = __ballot(top >= l);
+    if ((threadIdx.x & 63) == 0 && b) atomicAdd(&hist[l], __popcll(b));
+  }
+  __syncthreads();
+  // one of 16 copies of the counters (thousands of workgroups adding to the same few addresses take
+  // longer than the rest of the kernel); the host adds the copies up
+  if (threadIdx.x <= levels && hist[threadIdx.x])
+    atomicAdd(&counts[(blockIdx.x & 15) * 64 + threadIdx.x], hist[threadIdx.x]);
 }
 
 // One thread per sorted candidate: output row = number of heads before it; the filter tap
@@ -1212,15 +1243,27 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   m.v1.reserve(nc);
   m.f0.reserve(nc + 1);
   m.s0.reserve(nc + 1);
-  k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), n, LI.npad,
-                                                   m.k0.p, m.v0.p);
-  LAUNCH_CHECK();
   // Filter = stride = 2 in every dimension over exactly fitting sizes (the U-Net's and most
   // networks' downsampling): each site has one candidate, the Morton key of its coordinates
   // halved, which ascends with the site's own key, so the schedule order is already sorted.
   bool presorted = m.dim <= 3 && f.M == 1;
   for (int d = 0; d < m.dim; d++)
     presorted = presorted && filter[d] == 2 && stride[d] == 2 && in_size[d] == 2 * out_size[d];
+  // The caller has to learn the new level's size: a read-back per rulebook, except along a chain
+  // of exact halvings, whose sizes the first rulebook of the chain counts all at once
+  // (k_strided_heads) and hands down from level to level.
+  int chain = 0;  // further exact halvings of the output size, when this call has to count
+  if (presorted && LI.halvings.empty()) {
+    for (bool even = true; even && chain < 60 / m.dim - 1;) {
+      for (int d = 0; d < m.dim; d++) even = even && (out_size[d] >> chain) % 2 == 0 && (out_size[d] >> chain) >= 2;
+      if (even) chain++;
+    }
+    m.dflags.reserve(16 * 64);
+  }
+  const bool count = presorted && LI.halvings.empty();
+  k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), n, LI.npad,
+                                                   m.k0.p, m.v0.p, count ? m.dflags.p : nullptr);
+  LAUNCH_CHECK();
   if (presorted) {
     std::swap(m.k0, m.k1);
     std::swap(m.v0, m.v1);
@@ -1228,11 +1271,23 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
     sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
   }
-  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
+  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p, m.dim, chain, count ? m.dflags.p : nullptr);
   LAUNCH_CHECK();
   exclusive_scan(m, m.f0.p, m.s0.p, nc + 1, s);
-  const int64_t n_out = fetch_words(m, m.s0.p + nc, 1, s)[0];
+  int64_t n_out = -1;
+  if (count) {
+    const int *c = fetch_words(m, m.dflags.p, 16 * 64, s);
+    LI.halvings.assign(chain + 1, 0);
+    for (int copy = 0; copy < 16; copy++)
+      for (int l = 0; l <= chain; l++) LI.halvings[l] += c[copy * 64 + l];
+  }
+  if (presorted) {
+    n_out = LI.halvings[0];
+  } else {
+    n_out = fetch_words(m, m.s0.p + nc, 1, s)[0];
+  }
   alloc_level(LO, go, n_out, batch);
+  if (presorted) LO.halvings.assign(LI.halvings.begin() + 1, LI.halvings.end());
   R.by_out.n = n_out;
   R.by_out.npad = LO.npad;
   R.by_in.n = n;
