@@ -19,6 +19,7 @@
 namespace scn {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 static const int TB = 256;
 static inline dim3 grid_for(int64_t n, int tb = TB) { return dim3((unsigned)std::max<int64_t>(1, ceil_div(n, tb))); }
 
@@ -96,13 +97,37 @@ static ColsumPlan colsum_plan(int64_t rows, int planes) {
   p.blocks = (int)ceil_div(rows, p.rows_per_block);
   return p;
 }
-// out[c] = sum over row blocks, in block order, accumulated in double.
-__global__ void k_colsum_finish(const float *partial, int blocks, int planes, float *out) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= planes) return;
-  double s = 0;
-  for (int b = 0; b < blocks; b++) s += partial[(size_t)b * 2 * planes + c];
-  out[c] = (float)s;
+// out[i] = sum over blocks b of partial[b * stride + i], i < count.  A workgroup of 16 wavefronts
+// takes 64 consecutive outputs: wavefront w adds up its contiguous share of the blocks in order,
+// wavefront 0 then adds the 16 shares in order (a fixed order: the result is the same on every
+// run).  ACC is the accumulator type, OUT the type the sums are written in.
+template <typename ACC, typename OUT>
+__global__ __launch_bounds__(1024) void k_sum_blocks(const float *__restrict__ partial, int blocks, int64_t stride,
+                                                     int64_t count, OUT *__restrict__ out) {
+  __shared__ ACC part[16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + lane;
+  const int per = (blocks + 15) / 16;
+  const int b0 = min(blocks, wave * per), b1 = min(blocks, b0 + per);
+  ACC s = 0;
+  if (i < count)
+    for (int b = b0; b < b1; b++) s += (ACC)partial[(size_t)b * stride + i];
+  part[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && i < count) {
+    ACC tot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++) tot += part[w][lane];
+    out[i] = (OUT)tot;
+  }
+}
+// The two column sums of a batch-normalisation pass in double, behind the blocks' partial sums.
+static double *sum_pairs(Metadata &m, int blocks, int planes, hipStream_t s) {
+  double *sums = reinterpret_cast<double *>(m.partial.p + (size_t)blocks * 2 * planes);
+  k_sum_blocks<double, double><<<dim3((unsigned)ceil_div(2 * planes, 64)), 1024, 0, s>>>(m.partial.p, blocks, (int64_t)2 * planes,
+                                                                                        (int64_t)2 * planes, sums);
+  LAUNCH_CHECK();
+  return sums;
 }
 static void column_sums(Metadata &m, const float *x, int64_t rows, int planes, float *out, hipStream_t s) {
   if (planes <= 0) return;
@@ -116,7 +141,7 @@ static void column_sums(Metadata &m, const float *x, int64_t rows, int planes, f
                                                                                  rows, planes, p.CW, p.rows_per_block,
                                                                                  m.partial.p);
   LAUNCH_CHECK();
-  k_colsum_finish<<<grid_for(planes), TB, 0, s>>>(m.partial.p, p.blocks, planes, out);
+  k_sum_blocks<double, float><<<dim3((unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, p.blocks, (int64_t)2 * planes, planes, out);
   LAUNCH_CHECK();
 }
 
@@ -224,14 +249,135 @@ __global__ __launch_bounds__(256) void k_conv_dw(const int *__restrict__ nbr, co
         if (c < n_a && o < n_b) pk[(size_t)c * n_b + o] = acc[i][j][r];
       }
 }
-// dw[i] = sum over chunks, in chunk order
-__global__ void k_dw_reduce(const float *partial, int chunks, int64_t per_chunk, float *dw) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= per_chunk) return;
-  float s = 0.f;
-  for (int c = 0; c < chunks; c++) s += partial[(size_t)c * per_chunk + i];
-  dw[i] = s;
+// The same sums for narrow layers (both channel counts <= 64), where the kernel above spends its
+// time re-reading: one workgroup per tap reads the rows of b once per tap, 27 times in all.  Here
+// a workgroup of eight wavefronts takes a share of the positions and a 32 x 32 channel tile for
+// ALL taps: wavefront w keeps the accumulators of taps w, w + 8, w + 16, w + 24 (16 registers
+// each) and walks its share 16 positions (one granule of the tap masks) at a time, skipping the
+// taps the granule does not have.  Nothing goes through LDS: the MFMA contracts over four positions,
+// lane (r, g) supplies position 4 g + kk of the granule and, of that position's row, the two
+// channels 2 r and 2 r + 1 as one 8-byte load (16 lanes read 128 consecutive bytes); instruction
+// i of a pair takes component i, so that it computes the gradient's rows 2 * (MFMA row) + i, and
+// likewise for the columns.  The rows of b are loaded once per granule and serve all its taps.
+constexpr int DT_NW = 8, DT_T = 32, DT_SLOTS = 4, DT_BLOCK = 8;  // DT_BLOCK granules of 16 positions per turn
+template <bool VEC2>
+__global__ __launch_bounds__(DT_NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_dw_taps(const int *__restrict__ nbr, const int *__restrict__ rowmap,
+                                                             const unsigned *__restrict__ gmask, int K, int64_t n,
+                                                             int64_t npad, const float *__restrict__ a, int n_a,
+                                                             unsigned a_bytes, const float *__restrict__ b, int n_b,
+                                                             unsigned b_bytes, float *__restrict__ partial) {
+  const int tiles_o = (n_b + DT_T - 1) / DT_T;
+  const int ct = blockIdx.y / tiles_o, ot = blockIdx.y % tiles_o;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  v4f acc[DT_SLOTS][2][2];
+#pragma unroll
+  for (int sl = 0; sl < DT_SLOTS; sl++)
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) acc[sl][i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int ca = ct * DT_T + 2 * r16, cb = ot * DT_T + 2 * r16;
+  // rows of a come through a buffer resource: an offset of 2^31 or more reads zeros, which serves
+  // absent rules (negative row) and channels beyond the last
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a), 0, (int)a_bytes, 0x00020000);
+  const unsigned nowhere = 0x80000000u, a_row_bytes = (unsigned)n_a * 4u;
+  const unsigned ca0 = ca < n_a ? (unsigned)ca * 4u : nowhere, ca1 = ca + 1 < n_a ? (unsigned)ca * 4u + 4u : nowhere;
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(b), 0, (int)b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t nbr_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(nbr), 0, (int)((unsigned)K * (unsigned)npad * 4u), 0x00020000);
+  const unsigned b_row_bytes = (unsigned)n_b * 4u;
+  const unsigned cb0 = cb < n_b ? (unsigned)cb * 4u : nowhere, cb1 = cb + 1 < n_b ? (unsigned)cb * 4u + 4u : nowhere;
+  // two channels of row j (negative: zeros); every row offset there is lies below 2^31
+  auto pair_of = [&](const __amdgpu_buffer_rsrc_t &rsrc, int j, unsigned row_bytes, unsigned c0, unsigned c1) {
+    const unsigned row = (unsigned)j * row_bytes;
+    if (VEC2) return __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rsrc, j < 0 ? nowhere : row + c0, 0, 0));
+    v2f v;
+    v.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, j < 0 ? nowhere : row + c0, 0, 0));
+    v.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, j < 0 ? nowhere : row + c1, 0, 0));
+    return v;
+  };
+  unsigned own = 0u;  // the taps this wavefront accumulates
+#pragma unroll
+  for (int sl = 0; sl < DT_SLOTS; sl++)
+    if (wave + sl * DT_NW < K) own |= 1u << (wave + sl * DT_NW);
+  // Workgroup x takes the blocks of DT_BLOCK granules x, x + gridDim.x, ...: every workgroup sees
+  // every part of the pattern-sorted table, so that they all carry about the same number of rules.
+  const int n_granules = (int)((n + 15) >> 4), n32 = (int)n;  // the host checks that 4 K npad < 2^31
+  for (int gb = blockIdx.x * DT_BLOCK; gb < n_granules; gb += gridDim.x * DT_BLOCK) {
+    const int ge = min(n_granules, gb + DT_BLOCK);
+    for (int gi = gb; gi < ge; gi++) {
+      const unsigned present = gmask[gi] & own;
+      if (present == 0u) continue;  // uniform over the wavefront
+      const int t0 = gi << 4;
+      // this lane's four positions of the granule: t0 + 4 g + kk; first the index quads of the
+      // wavefront's taps, then all gathers, then the MFMAs: two memory latencies per granule
+      // (fetching the next granule's quads meanwhile costs more registers than there are at
+      // four wavefronts per SIMD, and measured slower with fewer)
+      int4 j4[DT_SLOTS];
+      const unsigned toff = (unsigned)(t0 + 4 * g) * 4u;
+#pragma unroll
+      for (int sl = 0; sl < DT_SLOTS; sl++) {
+        const int k = wave + sl * DT_NW;
+        // a tap the granule does not have: an offset past the table, which reads zeros; made -1 below
+        j4[sl] = __builtin_bit_cast(int4, __builtin_amdgcn_raw_buffer_load_b128(
+                                              nbr_rsrc, ((present >> k) & 1u) ? toff : nowhere, (unsigned)k * (unsigned)npad * 4u, 0));
+      }
+      v2f bv[4];
+      if (rowmap) {
+        const int4 r4 = *reinterpret_cast<const int4 *>(rowmap + t0 + 4 * g);
+        const int r[4] = {r4.x, r4.y, r4.z, r4.w};
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) bv[kk] = pair_of(b_rsrc, t0 + 4 * g + kk < n32 ? r[kk] : -1, b_row_bytes, cb0, cb1);
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+          const int t = t0 + 4 * g + kk;
+          bv[kk] = pair_of(b_rsrc, t < n32 ? t : -1, b_row_bytes, cb0, cb1);
+        }
+      }
+      v2f av[DT_SLOTS][4];
+#pragma unroll
+      for (int sl = 0; sl < DT_SLOTS; sl++) {
+        const int k = wave + sl * DT_NW;
+        const bool has = (present >> k) & 1u;
+        const int j[4] = {j4[sl].x, j4[sl].y, j4[sl].z, j4[sl].w};
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) av[sl][kk] = pair_of(a_rsrc, has ? j[kk] : -1, a_row_bytes, ca0, ca1);
+      }
+#pragma unroll
+      for (int sl = 0; sl < DT_SLOTS; sl++) {
+        const int k = wave + sl * DT_NW;
+        if (!((present >> k) & 1u)) continue;  // uniform over the wavefront
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+          for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int jx = 0; jx < 2; jx++)
+              acc[sl][i][jx] =
+                  __builtin_amdgcn_mfma_f32_16x16x4f32(av[sl][kk][i], bv[kk][jx], acc[sl][i][jx], 0, 0, 0);
+      }
+    }
+  }
+  // acc[sl][i][jx][r] = dW[k][ct*32 + 2 (4 g + r) + i][ot*32 + 2 r16 + jx] of this chunk
+#pragma unroll
+  for (int sl = 0; sl < DT_SLOTS; sl++) {
+    const int k = wave + sl * DT_NW;
+    if (k >= K) continue;
+    float *pk = partial + ((size_t)blockIdx.x * K + k) * (size_t)n_a * n_b;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int c = ct * DT_T + 2 * (4 * g + r) + i;
+        if (c >= n_a) continue;
+        if (cb + 0 < n_b) pk[(size_t)c * n_b + cb + 0] = acc[sl][i][0][r];
+        if (cb + 1 < n_b) pk[(size_t)c * n_b + cb + 1] = acc[sl][i][1][r];
+      }
+  }
 }
+
 // Any groups, any shapes: one thread per weight, positions in order.  The correctness path for
 // grouped convolutions, which the MFMA kernel does not cover.
 __global__ void k_conv_dw_generic(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad, const float *a,
@@ -251,7 +397,8 @@ __global__ void k_conv_dw_generic(const int *nbr, const int *rowmap, int K, int6
   dw[i] = s;
 }
 
-static void weight_gradient(Metadata &m, const Table &t, const float *a, int n_a, const float *b, int n_b, int groups,
+static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t a_rows, int n_a, const float *b,
+                            int64_t b_rows, int n_b, int groups,
                             float *dw, hipStream_t s) {
   const int64_t per_chunk = (int64_t)t.K * (n_a / groups) * (n_b / groups) * groups;
   if (t.n == 0) {
@@ -264,6 +411,30 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int n_a
     LAUNCH_CHECK();
     return;
   }
+  const bool vec4 = n_a % 4 == 0 && n_b % 4 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0;
+  if (t.K <= DT_NW * DT_SLOTS && t.gmask.p && n_a <= 64 && n_b <= 64 && t.npad % 4 == 0 &&
+      a_rows * n_a * 4 < ((int64_t)1 << 31) && b_rows * n_b * 4 < ((int64_t)1 << 31) &&
+      (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31)) {
+    // narrow layers: all taps per workgroup
+    const int tiles = (int)(ceil_div(n_a, DT_T) * ceil_div(n_b, DT_T));
+    // one resident round: two workgroups per compute unit, shared between the channel tiles
+    const int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(t.n, 16 * DT_BLOCK), 512 / tiles));
+    m.partial.reserve((size_t)chunks * per_chunk);
+    const dim3 grid((unsigned)chunks, (unsigned)tiles);
+    const bool vec2 = n_a % 2 == 0 && n_b % 2 == 0 && (uintptr_t)a % 8 == 0 && (uintptr_t)b % 8 == 0;
+    if (vec2)
+      k_conv_dw_taps<true><<<grid, DT_NW * 64, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, a, n_a,
+                                                       (unsigned)(a_rows * n_a * 4), b, n_b,
+                                                       (unsigned)(b_rows * n_b * 4), m.partial.p);
+    else
+      k_conv_dw_taps<false><<<grid, DT_NW * 64, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, a, n_a,
+                                                        (unsigned)(a_rows * n_a * 4), b, n_b,
+                                                       (unsigned)(b_rows * n_b * 4), m.partial.p);
+    LAUNCH_CHECK();
+    k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
+    LAUNCH_CHECK();
+    return;
+  }
   const int tiles = (int)(ceil_div(n_a, DW_T) * ceil_div(n_b, DW_T));
   if (t.K > 65535 || tiles > 65535) throw Error("weight gradient: filter volume or channel count too large");
   // chunks: enough workgroups to fill the chip, partial sums bounded to about 256 MB
@@ -273,7 +444,6 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int n_a
   const int64_t chunk_len = round_up(ceil_div(t.n, chunks), DW_PS);
   chunks = ceil_div(t.n, chunk_len);
   m.partial.reserve((size_t)chunks * per_chunk);
-  const bool vec4 = n_a % 4 == 0 && n_b % 4 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0;
   const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
   const dim3 grid((unsigned)chunks, (unsigned)t.K, (unsigned)tiles);
   if (vec4)
@@ -283,7 +453,7 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int n_a
     k_conv_dw<false><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a, b, n_b, chunk_len,
                                           m.partial.p);
   LAUNCH_CHECK();
-  k_dw_reduce<<<grid_for(per_chunk), TB, 0, s>>>(m.partial.p, (int)chunks, per_chunk, dw);
+  k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
   LAUNCH_CHECK();
 }
 
@@ -356,7 +526,7 @@ void subm_conv_backward(Metadata &m, Table &t, const int64_t *filter, const floa
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
   if (d_bias) column_sums(m, d_out, t.n, n_out, d_bias, s);
-  weight_gradient(m, t, in, n_in, d_out, n_out, groups, d_w, s);
+  weight_gradient(m, t, in, t.n, n_in, d_out, t.n, n_out, groups, d_w, s);
   if (t.n == 0) return;
   if (taps_mirror(m, t, filter, s)) {
     input_gradient(m, t, d_out, t.n, d_in, w, n_in, n_out, groups, true, s);
@@ -381,7 +551,7 @@ void strided_conv_backward(Metadata &m, const Table &fwd, const Table &other, in
     else
       fill32(d_bias, 0, n_out, s);
   }
-  weight_gradient(m, fwd, in, n_in, d_out, n_out, groups, d_w, s);
+  weight_gradient(m, fwd, in, in_rows, n_in, d_out, out_rows, n_out, groups, d_w, s);
   if (in_rows == 0) return;
   if (other.n != in_rows) throw Error("internal: the rulebook's other side does not match the input level");
   input_gradient(m, other, d_out, out_rows, d_in, w, n_in, n_out, groups, false, s);
@@ -391,16 +561,12 @@ void strided_conv_backward(Metadata &m, const Table &fwd, const Table &other, in
 // CPU/BatchNormalization.cpp:19-40: batch mean and biased variance into save_mean / save_invstd,
 // running statistics updated with `momentum` weighting the old value and the unbiased variance;
 // coef = scale | shift for the affine pass.
-__global__ void k_bn_train_finish(const float *partial, int blocks, int planes, int64_t rows, float *save_mean,
+__global__ void k_bn_train_finish(const double *sums, int planes, int64_t rows, float *save_mean,
                                   float *save_invstd, float *running_mean, float *running_var, const float *gamma,
                                   const float *beta, float eps, float momentum, float *coef) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= planes) return;
-  double s1 = 0, s2 = 0;
-  for (int b = 0; b < blocks; b++) {
-    s1 += partial[(size_t)b * 2 * planes + c];
-    s2 += partial[(size_t)b * 2 * planes + planes + c];
-  }
+  const double s1 = sums[c], s2 = sums[planes + c];
   const double mean = s1 / (double)rows;
   double ss = s2 - mean * mean * (double)rows;  // sum of squared deviations
   if (ss < 0) ss = 0;
@@ -432,13 +598,14 @@ void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t ro
   if (rows <= 0 || planes <= 0) return;
   Metadata &m = *scratch;
   const ColsumPlan p = colsum_plan(rows, planes);
-  m.partial.reserve((size_t)p.blocks * 2 * planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes + 4 * (size_t)planes);
   m.prebuf.reserve(2 * (size_t)planes);
   k_colsum<1><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(in, in_stride, nullptr, nullptr, 0, nullptr,
                                                                                  0.f, rows, planes, p.CW, p.rows_per_block,
                                                                                  m.partial.p);
   LAUNCH_CHECK();
-  k_bn_train_finish<<<grid_for(planes), TB, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_mean, save_invstd,
+  const double *sums = sum_pairs(m, p.blocks, planes, s);
+  k_bn_train_finish<<<grid_for(planes), TB, 0, s>>>(sums, planes, rows, save_mean, save_invstd,
                                                     running_mean, running_var, gamma, beta, eps, momentum, m.prebuf.p);
   LAUNCH_CHECK();
   const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
@@ -446,15 +613,11 @@ void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t ro
   LAUNCH_CHECK();
 }
 // CPU/BatchNormalization.cpp:84-106: coef = gradMean | k | invstd * gamma
-__global__ void k_bn_bwd_finish(const float *partial, int blocks, int planes, int64_t rows, const float *save_invstd,
+__global__ void k_bn_bwd_finish(const double *sums, int planes, int64_t rows, const float *save_invstd,
                                 const float *gamma, float *d_gamma, float *d_beta, float *coef) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= planes) return;
-  double sd = 0, dotp = 0;
-  for (int b = 0; b < blocks; b++) {
-    sd += partial[(size_t)b * 2 * planes + c];
-    dotp += partial[(size_t)b * 2 * planes + planes + c];
-  }
+  const double sd = sums[c], dotp = sums[planes + c];
   const float invstd = save_invstd[c];
   if (d_beta) d_beta[c] = (float)sd;
   if (d_gamma) d_gamma[c] = (float)dotp * invstd;
@@ -488,13 +651,14 @@ void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *o
   }
   Metadata &m = *scratch;
   const ColsumPlan p = colsum_plan(rows, planes);
-  m.partial.reserve((size_t)p.blocks * 2 * planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes + 4 * (size_t)planes);
   m.prebuf.reserve(3 * (size_t)planes);
   k_colsum<2><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(in, in_stride, d_out, out, out_stride,
                                                                                  save_mean, leak, rows, planes, p.CW,
                                                                                  p.rows_per_block, m.partial.p);
   LAUNCH_CHECK();
-  k_bn_bwd_finish<<<grid_for(planes), TB, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_invstd, gamma, d_gamma, d_beta,
+  const double *sums = sum_pairs(m, p.blocks, planes, s);
+  k_bn_bwd_finish<<<grid_for(planes), TB, 0, s>>>(sums, planes, rows, save_invstd, gamma, d_gamma, d_beta,
                                                   m.prebuf.p);
   LAUNCH_CHECK();
   const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
@@ -584,7 +748,7 @@ void s2d_backward(const Level &l, float *d_in, const float *d_out, int planes, h
 void nin_backward(Metadata &m, const Table &t, const float *in, float *d_in, const float *d_out, const float *w,
                   float *d_w, float *d_bias, int n_in, int n_out, hipStream_t s) {
   if (d_bias) column_sums(m, d_out, t.n, n_out, d_bias, s);
-  weight_gradient(m, t, in, n_in, d_out, n_out, 1, d_w, s);
+  weight_gradient(m, t, in, t.n, n_in, d_out, t.n, n_out, 1, d_w, s);
   if (t.n == 0) return;
   input_gradient(m, t, d_out, t.n, d_in, w, n_in, n_out, 1, false, s);
 }

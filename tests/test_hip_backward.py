@@ -86,6 +86,24 @@ def test_conv_gradients_vs_oracle(oracle_built, cin, cout, groups):
     checks.assert_close(got[2], want[2], "transposed d_bias")
 
 
+@pytest.mark.parametrize("cin,cout", [(3, 32), (32, 32), (48, 64)])
+def test_weight_gradient_over_many_blocks(oracle_built, cin, cout):
+    """150,000 sites: more blocks of positions than the narrow layers' weight-gradient kernel has
+    workgroups, so that each of them takes several turns."""
+    from hip_path import HipPath
+    g, o = HipPath(3), cpu_path.CpuPath(3, "oracle")
+    coords = synthetic.room_scene(seed=4400, target=150000, spatial=400, duplicate_fraction=0.0)
+    rng = np.random.default_rng(cin * 77 + cout)
+    x = rng.normal(size=(len(coords), cin)).astype(np.float32)
+    d_y = rng.normal(size=(len(coords), cout)).astype(np.float32)
+    w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
+    for p in (g, o):
+        assert p.input_layer(400, coords, 0, 3) == len(coords)
+    got, want = g.subm_conv_bwd(400, 3, x, d_y, w, True), o.subm_conv_bwd(400, 3, x, d_y, w, True)
+    for a, b, what in zip(got, want, ("d_input", "d_weight", "d_bias")):
+        checks.assert_close(a, b, "submanifold " + what)
+
+
 def test_pooling_and_nin_gradients_vs_oracle(oracle_built):
     from hip_path import HipPath
     g, o = HipPath(3), cpu_path.CpuPath(3, "oracle")
