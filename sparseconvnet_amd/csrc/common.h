@@ -169,4 +169,24 @@ __device__ inline int64_t block_find(const BlockEntry *table, uint64_t mask, uin
   return -1;
 }
 
+// Occupancy bits and first row of the block with key bkey (false: no such block).  A slot's key
+// and bits come with one 16-byte load, the row only when the key matches.
+__device__ inline bool block_lookup(const BlockEntry *table, uint64_t mask, uint64_t bkey, unsigned long long &bits,
+                                    int &base) {
+  uint64_t b = hash64(bkey) & mask;
+  for (uint64_t i = 0; i <= mask; i++) {
+    const ulonglong2 km = *reinterpret_cast<const ulonglong2 *>(&table[b]);
+    if (km.x == bkey) {
+      bits = km.y;
+      base = table[b].base;
+      return true;
+    }
+    if (km.x == SCN_EMPTY_KEY) break;
+    b = (b + 1) & mask;
+  }
+  bits = 0ull;
+  base = 0;
+  return false;
+}
+
 }  // namespace scn

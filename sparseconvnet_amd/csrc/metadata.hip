@@ -869,9 +869,11 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
   const int row = sched ? sched[t] : (int)t;
   unsigned long long sp[DIM][3];
   bool okc[DIM][3];
+  int cd[DIM];
 #pragma unroll
   for (int d = 0; d < DIM; d++) {
     const int c = soa[d * npad + row];
+    cd[d] = c;
 #pragma unroll
     for (int o = 0; o < 3; o++) {
       const int v = c + o - 1;
@@ -881,8 +883,63 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
     }
   }
   const unsigned long long bpart = (unsigned long long)soa[DIM * npad + row] << (DIM * g.bits);
-  unsigned long long last_bkey = SCN_EMPTY_KEY, last_mask = 0;
-  int last_base = 0;
+  // The lane's taps (first-dimension offset fixed by its wavefront) lie in at most two blocks
+  // along each remaining dimension: the blocks of the lowest and of the highest in-range
+  // coordinate.  All of them (two, or two by two) are looked up at once, whole 32-byte entries,
+  // so that a lane waits for memory once instead of once per block it meets on its way through
+  // the taps; entry e = 2 * (high block along dimension 1) + (high block along the last).
+  constexpr int NE = DIM == 3 ? 4 : 2;
+  constexpr int SH = DIM == 3 ? 2 : 3;  // a block is 4 x 4 x 4 sites, or 8 x 8
+  bool hi_of[DIM][3];  // [d][o]: tap offset o along d lies in the high block (always false when there is only one)
+  unsigned long long lo_sp[DIM], hi_sp[DIM];
+  bool split[DIM];
+#pragma unroll
+  for (int d = 1; d < DIM; d++) {
+    const int lo = max(cd[d] - 1, 0), hi = min(cd[d] + 1, g.size[d] - 1);
+    split[d] = (lo >> SH) != (hi >> SH);
+    lo_sp[d] = okc[d][0] ? sp[d][0] : sp[d][1];
+    hi_sp[d] = okc[d][2] ? sp[d][2] : sp[d][1];
+#pragma unroll
+    for (int o = 0; o < 3; o++) hi_of[d][o] = ((cd[d] + o - 1) >> SH) != (lo >> SH);
+  }
+  unsigned long long ebits[NE];
+  int ebase[NE];
+  {
+    unsigned long long want[NE], at[NE];
+    ulonglong2 km[NE];
+    bool need[NE];
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+      unsigned long long key;
+      if (DIM == 3) {
+        key = bpart | sp[0][part] | ((e & 2) ? hi_sp[1] : lo_sp[1]) | ((e & 1) ? hi_sp[2] : lo_sp[2]);
+        need[e] = okc[0][part] && (!(e & 2) || split[1]) && (!(e & 1) || split[2]);
+      } else {
+        key = bpart | sp[0][part] | ((e & 1) ? hi_sp[1] : lo_sp[1]);
+        need[e] = okc[0][part] && (!(e & 1) || split[1]);
+      }
+      want[e] = key >> 6;
+      at[e] = hash64(want[e]) & mask;
+    }
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+      km[e] = make_ulonglong2(SCN_EMPTY_KEY, 0ull);
+      ebase[e] = 0;
+      if (need[e]) {
+        km[e] = *reinterpret_cast<const ulonglong2 *>(&table[at[e]]);
+        ebase[e] = table[at[e]].base;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < NE; e++) {
+      ebits[e] = km[e].y;
+      if (km[e].x != want[e]) {
+        ebits[e] = 0ull;
+        // not in its first slot: absent (empty slot), or further along the probe sequence
+        if (km[e].x != SCN_EMPTY_KEY) block_lookup(table, mask, want[e], ebits[e], ebase[e]);
+      }
+    }
+  }
   unsigned my_mask = 0;
 #pragma unroll
   for (int kk = 0; kk < PER; kk++) {
@@ -891,25 +948,26 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
     const int o1 = DIM == 3 ? kk / 3 : kk, o2 = kk % 3;
     bool inside;
     unsigned long long key;
+    int e;
     if (DIM == 3) {
       inside = okc[0][part] && okc[1][o1] && okc[2][o2];
       key = bpart | sp[0][part] | sp[1][o1] | sp[2][o2];
+      e = (hi_of[1][o1] ? 2 : 0) + (hi_of[2][o2] ? 1 : 0);
     } else {
       inside = okc[0][part] && okc[1][o1];
       key = bpart | sp[0][part] | sp[1][o1];
+      e = hi_of[1][o1] ? 1 : 0;
     }
     int j = -1;
     if (inside) {
-      const unsigned long long bkey = key >> 6;
-      if (bkey != last_bkey) {
-        last_bkey = bkey;
-        const int64_t slot = block_find(table, mask, bkey);
-        last_mask = slot >= 0 ? table[slot].mask : 0ull;
-        last_base = slot >= 0 ? table[slot].base : 0;
-      }
+      unsigned long long bits = ebits[0];
+      int base = ebase[0];
+#pragma unroll
+      for (int x = 1; x < NE; x++)
+        if (e == x) bits = ebits[x], base = ebase[x];
       const unsigned long long bit = 1ull << (key & 63);
-      if (last_mask & bit) {
-        const int r = last_base + __popcll(last_mask & (bit - 1));
+      if (bits & bit) {
+        const int r = base + __popcll(bits & (bit - 1));
         j = urow ? urow[r] : r;
       }
     }
