@@ -43,45 +43,93 @@ __global__ void k_transpose_weights(const float *w, float *wt, int K, int groups
 //   MODE 0  a = x                                   (bias gradient; one quantity)
 //   MODE 1  a = x, b = x * x                        (batch-norm statistics)
 //   MODE 2  a = d * r, b = (x - mean[c]) * d * r    with r = out > 0 ? 1 : leak  (batch-norm backward)
-// A workgroup of 256 threads covers CW columns by 256 / CW rows at a time.
-template <int MODE>
-__global__ void k_colsum(const float *x, int64_t x_stride, const float *d, const float *out, int64_t o_stride,
-                         const float *mean, float leak, int64_t rows, int planes, int CW, int64_t rows_per_block,
-                         float *partial) {
-  __shared__ float red[2][256];
-  const int tx = threadIdx.x % CW, ty = threadIdx.x / CW, RW = 256 / CW;
-  const int c = blockIdx.y * CW + tx;
+// A workgroup of 256 threads covers CW columns by 256 * V / CW rows at a time; a thread owns V
+// consecutive columns (V = 4: 16-byte loads, when the plane count and the row strides are
+// multiples of four and the arrays 16-byte aligned) and has four rows in flight.
+template <int MODE, int V>
+__global__ __launch_bounds__(256) void k_colsum(const float *__restrict__ x, int64_t x_stride, const float *__restrict__ d,
+                                                const float *__restrict__ out, int64_t o_stride,
+                                                const float *__restrict__ mean, float leak, int64_t rows, int planes, int CW,
+                                                int64_t rows_per_block, float *__restrict__ partial) {
+  __shared__ float red[2][256 * V];
+  const int TPR = CW / V;  // threads per row
+  const int tx = threadIdx.x % TPR, ty = threadIdx.x / TPR, RW = 256 / TPR;
+  const int c = blockIdx.y * CW + tx * V;
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_block, r1 = min(rows, r0 + rows_per_block);
-  float a = 0.f, b = 0.f;
-  if (c < planes) {
-    const float mu = MODE == 2 ? mean[c] : 0.f;
-    for (int64_t r = r0 + ty; r < r1; r += RW) {
-      if (MODE == 0) {
-        a += x[r * x_stride + c];
-      } else if (MODE == 1) {
-        const float v = x[r * x_stride + c];
-        a += v;
-        b += v * v;
-      } else {
-        float g = d[r * o_stride + c];
-        g *= out[r * o_stride + c] > 0.f ? 1.f : leak;
-        a += g;
-        b += (x[r * x_stride + c] - mu) * g;
-      }
+  float a[V], b[V];
+#pragma unroll
+  for (int v = 0; v < V; v++) a[v] = b[v] = 0.f;
+  auto load = [&](const float *base, int64_t off, float (&dst)[V]) {
+    if constexpr (V == 4) {
+      const v4f t = *reinterpret_cast<const v4f *>(base + off);
+      dst[0] = t.x, dst[1] = t.y, dst[2] = t.z, dst[3] = t.w;
+    } else {
+      dst[0] = base[off];
     }
+  };
+  if (c < planes) {
+    float mu[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) mu[v] = MODE == 2 ? mean[c + v] : 0.f;
+    auto row = [&](int64_t r) {
+      float xv[V], dv[V], ov[V];
+      if (MODE != 2) {
+        load(x, r * x_stride + c, xv);
+#pragma unroll
+        for (int v = 0; v < V; v++) {
+          a[v] += xv[v];
+          if (MODE == 1) b[v] += xv[v] * xv[v];
+        }
+      } else {
+        load(d, r * o_stride + c, dv);
+        load(out, r * o_stride + c, ov);
+        load(x, r * x_stride + c, xv);
+#pragma unroll
+        for (int v = 0; v < V; v++) {
+          const float g = dv[v] * (ov[v] > 0.f ? 1.f : leak);
+          a[v] += g;
+          b[v] += (xv[v] - mu[v]) * g;
+        }
+      }
+    };
+    int64_t r = r0 + ty;
+    for (; r + 3 * RW < r1; r += 4 * RW) {  // four independent rows per trip
+      row(r);
+      row(r + RW);
+      row(r + 2 * RW);
+      row(r + 3 * RW);
+    }
+    for (; r < r1; r += RW) row(r);
   }
-  red[0][threadIdx.x] = a;
-  red[1][threadIdx.x] = b;
+#pragma unroll
+  for (int v = 0; v < V; v++) {
+    red[0][threadIdx.x * V + v] = a[v];
+    red[1][threadIdx.x * V + v] = b[v];
+  }
   __syncthreads();
-  if (ty == 0 && c < planes) {
-    for (int q = 1; q < RW; q++) {
-      a += red[0][q * CW + tx];
-      b += red[1][q * CW + tx];
+  // red[q][(ty * TPR + tx) * V + v] = column tx * V + v of row group ty: thread t < CW adds up column t
+  if (threadIdx.x < CW && blockIdx.y * CW + threadIdx.x < planes) {
+    float sa = 0.f, sb = 0.f;
+    for (int q = 0; q < RW; q++) {
+      sa += red[0][q * CW + threadIdx.x];
+      sb += red[1][q * CW + threadIdx.x];
     }
     float *p = partial + (size_t)blockIdx.x * 2 * planes;
-    p[c] = a;
-    p[planes + c] = b;
+    p[blockIdx.y * CW + threadIdx.x] = sa;
+    p[planes + blockIdx.y * CW + threadIdx.x] = sb;
   }
+}
+// Launches k_colsum<MODE, 4> when every operand allows 16-byte loads, else <MODE, 1>.
+template <int MODE>
+static void launch_colsum(dim3 grid, hipStream_t s, const float *x, int64_t x_stride, const float *d, const float *out,
+                          int64_t o_stride, const float *mean, float leak, int64_t rows, int planes, int CW,
+                          int64_t rows_per_block, float *partial) {
+  auto ok = [](const float *p, int64_t stride) { return p == nullptr || ((uintptr_t)p % 16 == 0 && stride % 4 == 0); };
+  if (planes % 4 == 0 && ok(x, x_stride) && ok(d, o_stride) && ok(out, o_stride))
+    k_colsum<MODE, 4><<<grid, 256, 0, s>>>(x, x_stride, d, out, o_stride, mean, leak, rows, planes, CW, rows_per_block, partial);
+  else
+    k_colsum<MODE, 1><<<grid, 256, 0, s>>>(x, x_stride, d, out, o_stride, mean, leak, rows, planes, CW, rows_per_block, partial);
+  LAUNCH_CHECK();
 }
 struct ColsumPlan {
   int CW, blocks;
@@ -137,10 +185,9 @@ static void column_sums(Metadata &m, const float *x, int64_t rows, int planes, f
   }
   const ColsumPlan p = colsum_plan(rows, planes);
   m.partial.reserve((size_t)p.blocks * 2 * planes);
-  k_colsum<0><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(x, planes, nullptr, nullptr, 0, nullptr, 0.f,
+  launch_colsum<0>(dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), s, x, planes, nullptr, nullptr, 0, nullptr, 0.f,
                                                                                  rows, planes, p.CW, p.rows_per_block,
                                                                                  m.partial.p);
-  LAUNCH_CHECK();
   k_sum_blocks<double, float><<<dim3((unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, p.blocks, (int64_t)2 * planes, planes, out);
   LAUNCH_CHECK();
 }
@@ -600,10 +647,9 @@ void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t ro
   const ColsumPlan p = colsum_plan(rows, planes);
   m.partial.reserve((size_t)p.blocks * 2 * planes + 4 * (size_t)planes);
   m.prebuf.reserve(2 * (size_t)planes);
-  k_colsum<1><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(in, in_stride, nullptr, nullptr, 0, nullptr,
+  launch_colsum<1>(dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), s, in, in_stride, nullptr, nullptr, 0, nullptr,
                                                                                  0.f, rows, planes, p.CW, p.rows_per_block,
                                                                                  m.partial.p);
-  LAUNCH_CHECK();
   const double *sums = sum_pairs(m, p.blocks, planes, s);
   k_bn_train_finish<<<grid_for(planes), TB, 0, s>>>(sums, planes, rows, save_mean, save_invstd,
                                                     running_mean, running_var, gamma, beta, eps, momentum, m.prebuf.p);
@@ -653,10 +699,9 @@ void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *o
   const ColsumPlan p = colsum_plan(rows, planes);
   m.partial.reserve((size_t)p.blocks * 2 * planes + 4 * (size_t)planes);
   m.prebuf.reserve(3 * (size_t)planes);
-  k_colsum<2><<<dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), 256, 0, s>>>(in, in_stride, d_out, out, out_stride,
+  launch_colsum<2>(dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), s, in, in_stride, d_out, out, out_stride,
                                                                                  save_mean, leak, rows, planes, p.CW,
                                                                                  p.rows_per_block, m.partial.p);
-  LAUNCH_CHECK();
   const double *sums = sum_pairs(m, p.blocks, planes, s);
   k_bn_bwd_finish<<<grid_for(planes), TB, 0, s>>>(sums, planes, rows, save_invstd, gamma, d_gamma, d_beta,
                                                   m.prebuf.p);
