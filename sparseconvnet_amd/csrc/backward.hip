@@ -425,6 +425,153 @@ __global__ __launch_bounds__(DT_NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   }
 }
 
+// Wider layers: a wavefront per (tap, 64 x 64 channel tile, share of the positions), no LDS; a
+// workgroup holds the 2 x 2 tiles of a 128 x 128 block and keeps them in step with a barrier
+// per granule, so that of the two wavefronts that need the same quads the second reads L1 (the
+// kernel is bound by the traffic between L2 and the compute units: 512 bytes per position and
+// tile for 64 MFMAs).
+// As in k_conv_dw_taps the MFMA contracts over four positions and the operands come straight
+// from the rows: lane (r, g) loads the four channels 4 r .. 4 r + 3 of position 4 g + kk (16
+// lanes read 256 consecutive bytes); the sixteen instructions of a position quad pair component
+// i of the a-side with component j of the b-side, so instruction (i, j) computes rows
+// 4 * (MFMA row) + i and columns 4 * (MFMA column) + j of the tile.
+// Granules without the tap are skipped by the granule masks (when the table has them).  A tap
+// with few rules gets few shares (tap_shares, from the table's rule counts) so that every
+// wavefront carries about the same number of rules; blocks of DT_BLOCK granules are dealt
+// round-robin over a tap's shares.  The loop runs two granules ahead: while the MFMAs of one
+// granule issue, the rows of the next are on their way and the indices of the one after.
+constexpr int DWV_T = 64;
+struct TapShares {
+  unsigned short n[32];  // K <= 32: shares of tap k that have work; the rest only write zeros
+};
+template <bool VEC4>
+__global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nbr, const int *__restrict__ rowmap,
+                                                      const unsigned *__restrict__ gmask, int K, int64_t n, int64_t npad,
+                                                      const float *__restrict__ a, int n_a, unsigned a_bytes,
+                                                      const float *__restrict__ b, int n_b, unsigned b_bytes, int shares,
+                                                      TapShares tap_shares, float *__restrict__ partial) {
+  const int k = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int share = blockIdx.y;
+  // the four wavefronts of a workgroup: the 2 x 2 tiles of a 128 x 128 block, in step (see the barrier below)
+  const int mt_o = (n_b + 2 * DWV_T - 1) / (2 * DWV_T);
+  const int ct = 2 * (blockIdx.z / mt_o) + (wave >> 1), ot = 2 * (blockIdx.z % mt_o) + (wave & 1);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int ca = ct * DWV_T + 4 * r16, cb = ot * DWV_T + 4 * r16;
+  const unsigned nowhere = 0x80000000u;  // offsets from here on read zeros
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a), 0, (int)a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(b), 0, (int)b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t nbr_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(nbr), 0, (int)((unsigned)K * (unsigned)npad * 4u), 0x00020000);
+  const __amdgpu_buffer_rsrc_t map_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(rowmap ? rowmap : nbr), 0, (int)((unsigned)npad * 4u), 0x00020000);
+  const unsigned a_row_bytes = (unsigned)n_a * 4u, b_row_bytes = (unsigned)n_b * 4u;
+  // four channels of row j from column c0 on (negative row, or columns past the last: zeros)
+  auto quad_of = [&](const __amdgpu_buffer_rsrc_t &rsrc, int j, unsigned row_bytes, int c0, int width) {
+    const unsigned row = (unsigned)j * row_bytes;
+    if (VEC4) {
+      const unsigned off = (j < 0 || c0 >= width) ? nowhere : row + (unsigned)c0 * 4u;
+      return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
+    }
+    float e[4];
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+      const unsigned off = (j < 0 || c0 + x >= width) ? nowhere : row + (unsigned)(c0 + x) * 4u;
+      e[x] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0));
+    }
+    return (v4f){e[0], e[1], e[2], e[3]};
+  };
+  v4f acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int n_granules = (int)((n + 15) >> 4), n32 = (int)n;
+  const bool idle = ct * DWV_T >= n_a || ot * DWV_T >= n_b;  // a tile past the last channel: only keeps the barrier count
+  const int mine = K <= 32 ? (int)tap_shares.n[k] : shares;    // shares of this tap that have work
+  // This share's granules: blocks share, share + mine, ... of DT_BLOCK granules, those with the tap.
+  auto next_granule = [&](int gi) {  // the one after gi (n_granules: none)
+    for (;;) {
+      gi++;
+      if (gi % DT_BLOCK == 0) gi += (mine - 1) * DT_BLOCK;
+      if (gi >= n_granules) return n_granules;
+      if (!gmask || ((gmask[gi] >> k) & 1u)) return gi;
+    }
+  };
+  struct Quads {
+    v4f a[4], b[4];
+  };
+  int4 jq, rq;  // neighbour rows and rows of b of the lane's four positions, for the granule whose rows are requested next
+  auto load_indices = [&](int gi) {
+    const unsigned toff = gi < n_granules ? (unsigned)(gi * 16 + 4 * g) * 4u : nowhere;
+    jq = __builtin_bit_cast(int4, __builtin_amdgcn_raw_buffer_load_b128(nbr_rsrc, toff, (unsigned)k * (unsigned)npad * 4u, 0));
+    const int t = gi * 16 + 4 * g;
+    rq = make_int4(t, t + 1, t + 2, t + 3);
+    if (rowmap) rq = __builtin_bit_cast(int4, __builtin_amdgcn_raw_buffer_load_b128(map_rsrc, toff, 0, 0));
+  };
+  auto load_rows = [&](int gi, Quads &q) {
+    const int j[4] = {jq.x, jq.y, jq.z, jq.w}, r[4] = {rq.x, rq.y, rq.z, rq.w};
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+      const bool live = gi < n_granules && gi * 16 + 4 * g + kk < n32;
+      q.a[kk] = quad_of(a_rsrc, live ? j[kk] : -1, a_row_bytes, ca, n_a);
+      q.b[kk] = quad_of(b_rsrc, live ? r[kk] : -1, b_row_bytes, cb, n_b);
+    }
+  };
+  auto multiply = [&](const Quads &q) {
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int jx = 0; jx < 4; jx++)
+          acc[i][jx] = __builtin_amdgcn_mfma_f32_16x16x4f32(q.a[kk][i], q.b[kk][jx], acc[i][jx], 0, 0, 0);
+  };
+  if (share < mine) {  // uniform over the workgroup
+    Quads X, Y;
+    int g0 = share * DT_BLOCK;
+    if (g0 >= n_granules) g0 = n_granules;
+    else if (gmask && !((gmask[g0] >> k) & 1u)) g0 = next_granule(g0);
+    int g1 = next_granule(g0);
+    if (!idle) {
+      load_indices(g0);
+      load_rows(g0, X);
+      load_indices(g1);
+    }
+    while (g0 < n_granules) {
+      // X: rows of g0 (requested), jq / rq: indices of g1 (requested).  The barriers keep the four
+      // wavefronts on the same granule, so that of two that load the same quads one reads L1.
+      const int g2 = next_granule(g1), g3 = next_granule(g2);
+      __syncthreads();
+      if (!idle) {
+        load_rows(g1, Y);
+        load_indices(g2);
+        multiply(X);
+      }
+      __syncthreads();
+      if (!idle) {
+        load_rows(g2, X);
+        load_indices(g3);
+        if (g1 < n_granules) multiply(Y);
+      }
+      g0 = g2;
+      g1 = g3;
+    }
+  }
+  // acc[i][jx][r] = dW[k][ct*64 + 4 (4 g + r) + i][ot*64 + 4 r16 + jx] of this share (zeros for a share without work)
+  float *pk = partial + ((size_t)share * K + k) * (size_t)n_a * n_b;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int c = ct * DWV_T + 4 * (4 * g + r) + i;
+      if (c >= n_a) continue;
+#pragma unroll
+      for (int jx = 0; jx < 4; jx++)
+        if (cb + jx < n_b) pk[(size_t)c * n_b + cb + jx] = acc[i][jx][r];
+    }
+}
+
 // Any groups, any shapes: one thread per weight, positions in order.  The correctness path for
 // grouped convolutions, which the MFMA kernel does not cover.
 __global__ void k_conv_dw_generic(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad, const float *a,
@@ -481,6 +628,48 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
     LAUNCH_CHECK();
     return;
+  }
+  if (t.npad % 4 == 0 && a_rows * n_a * 4 < ((int64_t)1 << 31) && b_rows * n_b * 4 < ((int64_t)1 << 31) &&
+      (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31) && t.K <= 65535) {
+    // wider layers: a wavefront per (tap, 64 x 64 tile, share of the positions)
+    const int tiles = (int)(ceil_div(n_a, 2 * DWV_T) * ceil_div(n_b, 2 * DWV_T));  // blocks of 2 x 2 tiles
+    // Shares of the positions per tap in proportion to the tap's rules (the table's counts; the
+    // first call on a table fetches them), about three workgroups per compute unit in all;
+    // partial sums bounded to 256 MB, at least a block of granules per share.
+    TapShares ts{};
+    int64_t shares = ceil_div(768, (int64_t)t.K * tiles);
+    if (t.K <= 32 && t.K > 1) {
+      ensure_counts(*t.cnt, s);
+      int64_t most = 1, all = 0;
+      for (int k = 0; k < t.K; k++) most = std::max(most, t.cnt->host[k]), all += t.cnt->host[k];
+      shares = ceil_div((int64_t)768 * most, std::max<int64_t>(1, all) * tiles);  // of the heaviest tap
+    }
+    shares = std::min<int64_t>(shares, std::max<int64_t>(1, ((int64_t)64 << 20) / per_chunk));
+    shares = std::max<int64_t>(1, std::min<int64_t>(shares, ceil_div(t.n, 16 * DT_BLOCK)));
+    if (t.K <= 32) {
+      int64_t most = 1;
+      for (int k = 0; k < t.K && t.K > 1; k++) most = std::max(most, t.cnt->host[k]);
+      for (int k = 0; k < t.K; k++)
+        ts.n[k] = (unsigned short)(t.K > 1 ? std::max<int64_t>(1, ceil_div(shares * t.cnt->host[k], most)) : shares);
+    }
+    if (tiles <= 65535 && shares <= 65535) {
+      m.partial.reserve((size_t)shares * per_chunk);
+      const dim3 grid((unsigned)t.K, (unsigned)shares, (unsigned)tiles);
+      const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
+      if (vec4)
+        k_conv_dw_wave<true><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,
+                                                  (unsigned)(a_rows * n_a * 4), b, n_b, (unsigned)(b_rows * n_b * 4),
+                                                  (int)shares, ts, m.partial.p);
+      else
+        k_conv_dw_wave<false><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,
+                                                   (unsigned)(a_rows * n_a * 4), b, n_b, (unsigned)(b_rows * n_b * 4),
+                                                   (int)shares, ts, m.partial.p);
+      LAUNCH_CHECK();
+      k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)shares, per_chunk,
+                                                                                      per_chunk, dw);
+      LAUNCH_CHECK();
+      return;
+    }
   }
   const int tiles = (int)(ceil_div(n_a, DW_T) * ceil_div(n_b, DW_T));
   if (t.K > 65535 || tiles > 65535) throw Error("weight gradient: filter volume or channel count too large");
