@@ -115,6 +115,25 @@ __host__ __device__ inline uint64_t spread3(uint64_t v) {  // 21 bits -> every 3
   return v;
 }
 
+__host__ __device__ inline uint32_t compact2(uint64_t v) {  // every 2nd bit -> 32 bits (inverse of spread2)
+  v &= 0x5555555555555555ull;
+  v = (v | (v >> 1)) & 0x3333333333333333ull;
+  v = (v | (v >> 2)) & 0x0F0F0F0F0F0F0F0Full;
+  v = (v | (v >> 4)) & 0x00FF00FF00FF00FFull;
+  v = (v | (v >> 8)) & 0x0000FFFF0000FFFFull;
+  v = (v | (v >> 16)) & 0x00000000FFFFFFFFull;
+  return (uint32_t)v;
+}
+__host__ __device__ inline uint32_t compact3(uint64_t v) {  // every 3rd bit -> 21 bits (inverse of spread3)
+  v &= 0x1249249249249249ull;
+  v = (v | (v >> 2)) & 0x10C30C30C30C30C3ull;
+  v = (v | (v >> 4)) & 0x100F00F00F00F00Full;
+  v = (v | (v >> 8)) & 0x001F0000FF0000FFull;
+  v = (v | (v >> 16)) & 0x001F00000000FFFFull;
+  v = (v | (v >> 32)) & 0x00000000001FFFFFull;
+  return (uint32_t)v;
+}
+
 // c: dim coordinates, all inside [0, size).  The last coordinate varies fastest.
 __host__ __device__ inline uint64_t site_key(const Geom &g, const int *c, int batch) {
   switch (g.dim) {

@@ -31,6 +31,7 @@ struct Level {
   DevBuf<BlockEntry> table;
   DevBuf<unsigned long long> gridp;
   DevBuf<int> urow;
+  DevBuf<unsigned long long> skeys;  // [n + 1] site key of every schedule position (ascending), kept with the grid
   bool grid_built = false;
   bool dups = false;
   // Active-site counts of the levels that successive filter 2 / stride 2 rulebooks make of this
@@ -176,6 +177,7 @@ struct Metadata {
   DevBuf<unsigned char> tmp;
   DevBuf<unsigned long long> k0, k1;
   DevBuf<int> v0, v1, f0, f1, s0, s1;
+  DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups; partial sums of reductions

@@ -587,7 +587,7 @@ __global__ void k_block_insert(const unsigned long long *ukey, const int *head, 
 static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   if (L.grid_built) return;
   const int64_t n = L.n;
-  m.k0.reserve(n + 1);
+  L.skeys.reserve(n + 1);
   m.k1.reserve(n + 1);
   m.f0.reserve(n + 1);
   m.s0.reserve(n + 1);
@@ -597,20 +597,20 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   uint64_t cap_alloc = 64;
   while (cap_alloc < (uint64_t)n * 2) cap_alloc <<= 1;
   L.table.reserve(cap_alloc);
-  const unsigned long long *ukey = m.k0.p;
+  const unsigned long long *ukey = L.skeys.p;
   const int *n_sites_dev = nullptr;
   if (n) {
     if (L.dups) {
       // distinct sites first: ukey / urow by compaction; their number stays on the device
-      k_sorted_keys<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, m.k0.p);
+      k_sorted_keys<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, L.skeys.p);
       LAUNCH_CHECK();
       m.f1.reserve(n + 1);
       m.s1.reserve(n + 1);
       L.urow.reserve(n);
-      k_run_tails<<<grid_for(n), TB, 0, s>>>(m.k0.p, n, m.f1.p);
+      k_run_tails<<<grid_for(n), TB, 0, s>>>(L.skeys.p, n, m.f1.p);
       LAUNCH_CHECK();
       exclusive_scan(m, m.f1.p, m.s1.p, n, s);
-      k_compact_sites<<<grid_for(n), TB, 0, s>>>(m.k0.p, L.sched_ptr(), m.f1.p, m.s1.p, n, m.k1.p, L.urow.p);
+      k_compact_sites<<<grid_for(n), TB, 0, s>>>(L.skeys.p, L.sched_ptr(), m.f1.p, m.s1.p, n, m.k1.p, L.urow.p);
       LAUNCH_CHECK();
       n_sites_dev = m.s1.p + (n - 1);  // index of the last distinct site (the last position ends a run)
       ukey = m.k1.p;
@@ -618,7 +618,7 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
       k_block_heads<<<grid_for(n), TB, 0, s>>>(ukey, n, m.f0.p);
       LAUNCH_CHECK();
     } else {
-      k_grid_heads<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, m.k0.p, m.f0.p);
+      k_grid_heads<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, L.skeys.p, m.f0.p);
       LAUNCH_CHECK();
     }
     exclusive_scan(m, m.f0.p, m.s0.p, n, s);
@@ -759,6 +759,33 @@ __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, 
   nbr2[(int64_t)k * npad + t] = nbr[(int64_t)k * npad + src];
   if (k == 0) rowmap[t] = base ? base[src] : src;
 }
+// The same from a site-major table rows[src][ROWW]: a workgroup moves 64 positions, reading
+// each one's row in 16-byte pieces and writing 256 contiguous bytes per tap.
+template <int ROWW>
+__global__ __launch_bounds__(256) void k_table_rows_permute(const int *__restrict__ rows, int K, int64_t n, int64_t npad,
+                                                            const int *__restrict__ perm, const int *__restrict__ base,
+                                                            int *__restrict__ nbr2, int *__restrict__ rowmap) {
+  __shared__ int tile[64][ROWW + 1];
+  const int64_t t0 = (int64_t)blockIdx.x * 64;
+  for (int e = threadIdx.x; e < 64 * (ROWW / 4); e += 256) {
+    const int r = e / (ROWW / 4), c = 4 * (e % (ROWW / 4));
+    if (t0 + r >= n) break;
+    const int4 v = *reinterpret_cast<const int4 *>(rows + (int64_t)perm[t0 + r] * ROWW + c);
+    tile[r][c + 0] = v.x;
+    tile[r][c + 1] = v.y;
+    tile[r][c + 2] = v.z;
+    tile[r][c + 3] = v.w;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < K * 64; e += 256) {
+    const int k = e >> 6, r = e & 63;
+    if (t0 + r < n) nbr2[(int64_t)k * npad + t0 + r] = tile[r][k];
+  }
+  if (threadIdx.x < 64 && t0 + threadIdx.x < n) {
+    const int src = perm[t0 + threadIdx.x];
+    rowmap[t0 + threadIdx.x] = base ? base[src] : src;
+  }
+}
 // gmask[i] = OR of the tap masks of granule i's 16 positions; perm[t] = the position's place before the sort
 __global__ void k_granule_masks(const unsigned *masks, const int *perm, int64_t n, int64_t n_granules, unsigned *gmask) {
   int64_t gi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -805,8 +832,11 @@ static void reserve_pattern_buffers(Metadata &m, const Table &t) {
   m.v1.reserve(t.n);
   if (t.K <= 32) m.f1.reserve(t.n);
 }
-// keyed: the kernel that wrote t.nbr has written the sort keys, positions and masks as well.
-static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s, bool keyed = false) {
+// keyed: the kernel that wrote the table has written the sort keys, positions and masks as well.
+// rows (with keyed): that kernel wrote the table site-major, roww ints per site, into `rows`
+// and t.nbr is still empty.
+static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s, bool keyed = false,
+                           const int *rows = nullptr, int roww = 0) {
   if (t.n == 0) {
     t.identity_rows = true;
     return;
@@ -832,8 +862,13 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, key_bits);
   DevBuf<int> nbr2;
   nbr2.reserve((size_t)t.K * t.npad);
-  k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
-                                                     t.rowmap.p);
+  if (rows && roww == 32)
+    k_table_rows_permute<32><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p);
+  else if (rows && roww == 12)
+    k_table_rows_permute<12><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p);
+  else
+    k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
+                                                       t.rowmap.p);
   LAUNCH_CHECK();
   t.nbr = std::move(nbr2);
   t.identity_rows = false;
@@ -849,30 +884,45 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
 // is the OR of per-coordinate spread values, so each coordinate is spread three times per
 // site (for c-1, c, c+1) instead of once per tap, and the tap loop is fully unrolled.
 // One wavefront per slice of the first filter dimension, as in k_subm_rules.
+#define S3_ROW_INTS(dim) ((dim) == 3 ? 32 : 12)  // ints per site of the site-major table: 27 or 9 taps, padded to 16 bytes
 template <int DIM>
-__global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_t n, int64_t npad,
+__global__ void k_subm_rules_s3(Geom g, const unsigned long long *skeys, int64_t n, int64_t npad,
                                 const BlockEntry *table, const unsigned long long *mask_p, const int *urow,
-                                int *nbr, unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
+                                int *rows, unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
                                 int *pidx, unsigned *pmasks) {
   const unsigned long long mask = *mask_p;
   constexpr int K = DIM == 3 ? 27 : 9;
   constexpr int PER = K / 3;
+  constexpr int ROWW = S3_ROW_INTS(DIM);
+  // The table leaves this kernel site-major, rows[t][ROWW] (taps K .. ROWW-1 = -1): the
+  // pattern sort moves whole sites, and k_table_rows_permute then reads one contiguous row per
+  // site where a tap-major table would be read four bytes per sector.
+  __shared__ int tile[64][ROWW + 1];
   __shared__ int lcount[K];
   __shared__ unsigned lmask[64];  // tap mask of each of the block's positions, collected from the three wavefronts
   if (threadIdx.x < K) lcount[threadIdx.x] = 0;
   if (threadIdx.x < 64) lmask[threadIdx.x] = 0;
   __syncthreads();
   const int part = threadIdx.x >> 6;  // offset -1, 0, +1 along the first dimension
-  int64_t t = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63);
+  // Workgroups are dealt to the eight XCDs in turn; XCD x takes the x-th eighth of the positions
+  // (a compact piece of the curve), so that the block entries it looks up, an eighth of the
+  // table, stay in its own L2.
+  const int per_xcd = gridDim.x / 8;  // the grid is a multiple of eight workgroups
+  const int wg = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if ((int64_t)wg * 64 >= n) return;  // the whole workgroup: padding of the grid
+  int64_t t = (int64_t)wg * 64 + (threadIdx.x & 63);
   const bool live = t < n;
   if (!live) t = n - 1;
-  const int row = sched ? sched[t] : (int)t;
+  // The site of position t from its key (the positions' keys are one coalesced read; the
+  // coordinates by row would be four gathers through the schedule, per wavefront).
+  const unsigned long long skey = skeys[t];
   unsigned long long sp[DIM][3];
   bool okc[DIM][3];
   int cd[DIM];
 #pragma unroll
   for (int d = 0; d < DIM; d++) {
-    const int c = soa[d * npad + row];
+    const int c = DIM == 3 ? (int)compact3(skey >> (DIM - 1 - d)) & ((1 << g.bits) - 1)
+                           : (int)compact2(skey >> (DIM - 1 - d)) & ((1 << g.bits) - 1);
     cd[d] = c;
 #pragma unroll
     for (int o = 0; o < 3; o++) {
@@ -882,7 +932,7 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
       sp[d][o] = s << (DIM - 1 - d);
     }
   }
-  const unsigned long long bpart = (unsigned long long)soa[DIM * npad + row] << (DIM * g.bits);
+  const unsigned long long bpart = (skey >> (DIM * g.bits)) << (DIM * g.bits);  // the sample index, in place
   // The lane's taps (first-dimension offset fixed by its wavefront) lie in at most two blocks
   // along each remaining dimension: the blocks of the lowest and of the highest in-range
   // coordinate.  All of them (two, or two by two) are looked up at once, whole 32-byte entries,
@@ -971,13 +1021,25 @@ __global__ void k_subm_rules_s3(Geom g, const int *soa, const int *sched, int64_
         j = urow ? urow[r] : r;
       }
     }
-    if (live) nbr[(int64_t)k * npad + t] = j;
+    tile[threadIdx.x & 63][k] = j;
     if (j >= 0) my_mask |= 1u << k;
     const unsigned long long hits = __ballot(live && j >= 0);
     if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&lcount[k], __popcll(hits));
   }
   atomicOr(&lmask[threadIdx.x & 63], my_mask);
   __syncthreads();
+  // the workgroup's 64 rows are one contiguous piece of the table
+  for (int e = threadIdx.x; e < 64 * (ROWW / 4); e += 192) {
+    const int r = e / (ROWW / 4), c = 4 * (e % (ROWW / 4));
+    const int64_t tr = (int64_t)wg * 64 + r;
+    if (tr >= n) break;
+    int4 v;
+    v.x = c + 0 < K ? tile[r][c + 0] : -1;
+    v.y = c + 1 < K ? tile[r][c + 1] : -1;
+    v.z = c + 2 < K ? tile[r][c + 2] : -1;
+    v.w = c + 3 < K ? tile[r][c + 3] : -1;
+    *reinterpret_cast<int4 *>(rows + tr * ROWW + c) = v;
+  }
   unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * K;
   if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&slot[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
   // what the pattern sort of finalize_table starts from (k_table_masks would re-read the table for it)
@@ -1115,27 +1177,29 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   ensure_grid(m, L, s);
   t.n = L.n;
   t.npad = L.npad;
-  t.nbr.reserve((size_t)f.K * t.npad);
   start_counts(t, s);
   bool all3 = true;
   for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
-  if (all3 && (m.dim == 2 || m.dim == 3)) {
+  if (all3 && (m.dim == 2 || m.dim == 3) && t.n > 0) {
     int key_bits = 0;
     const PatternKey pk = pattern_plan(t.n, t.K, key_bits);
     reserve_pattern_buffers(m, t);
     unsigned *masks = reinterpret_cast<unsigned *>(m.f1.p);
+    const int roww = S3_ROW_INTS(m.dim);
+    m.rowtab.reserve((size_t)t.npad * roww);
     if (m.dim == 3)
-      k_subm_rules_s3<3><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
-                                                           L.gridp.p, L.urow_ptr(), t.nbr.p,
+      k_subm_rules_s3<3><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.skeys.p, L.n, L.npad, L.table.p,
+                                                           L.gridp.p, L.urow_ptr(), m.rowtab.p,
                                                            (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks);
     else
-      k_subm_rules_s3<2><<<grid_for(L.n, 64), 192, 0, s>>>(L.g, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p,
-                                                           L.gridp.p, L.urow_ptr(), t.nbr.p,
+      k_subm_rules_s3<2><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.skeys.p, L.n, L.npad, L.table.p,
+                                                           L.gridp.p, L.urow_ptr(), m.rowtab.p,
                                                            (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks);
     LAUNCH_CHECK();
-    finalize_table(m, t, L.sched_ptr(), s, true);
+    finalize_table(m, t, L.sched_ptr(), s, true, m.rowtab.p, roww);
     return m.subm.emplace(key, std::move(t)).first->second;
   }
+  t.nbr.reserve((size_t)f.K * t.npad);
   // one wavefront per slice of the first filter dimension when that divides the taps evenly
   const int parts = (m.dim >= 2 && f.size[0] <= 4) ? f.size[0] : 1;
   k_subm_rules<<<grid_for(L.n, 64), 64 * parts, f.K * sizeof(int), s>>>(
