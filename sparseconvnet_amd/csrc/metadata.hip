@@ -764,7 +764,8 @@ __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, 
 template <int ROWW>
 __global__ __launch_bounds__(256) void k_table_rows_permute(const int *__restrict__ rows, int K, int64_t n, int64_t npad,
                                                             const int *__restrict__ perm, const int *__restrict__ base,
-                                                            int *__restrict__ nbr2, int *__restrict__ rowmap) {
+                                                            int *__restrict__ nbr2, int *__restrict__ rowmap,
+                                                            unsigned *__restrict__ gmask) {
   __shared__ int tile[64][ROWW + 1];
   const int64_t t0 = (int64_t)blockIdx.x * 64;
   for (int e = threadIdx.x; e < 64 * (ROWW / 4); e += 256) {
@@ -781,9 +782,19 @@ __global__ __launch_bounds__(256) void k_table_rows_permute(const int *__restric
     const int k = e >> 6, r = e & 63;
     if (t0 + r < n) nbr2[(int64_t)k * npad + t0 + r] = tile[r][k];
   }
-  if (threadIdx.x < 64 && t0 + threadIdx.x < n) {
-    const int src = perm[t0 + threadIdx.x];
-    rowmap[t0 + threadIdx.x] = base ? base[src] : src;
+  if (threadIdx.x < 64) {  // the first wavefront
+    const bool live = t0 + threadIdx.x < n;
+    if (live) {
+      const int src = perm[t0 + threadIdx.x];
+      rowmap[t0 + threadIdx.x] = base ? base[src] : src;
+    }
+    // gmask of the workgroup's four granules: OR of the tap masks of 16 positions each
+    unsigned mk = 0;
+    if (live)
+      for (int k = 0; k < K; k++) mk |= tile[threadIdx.x][k] >= 0 ? 1u << k : 0u;
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) mk |= __shfl_xor(mk, o, 64);
+    if ((threadIdx.x & 15) == 0 && t0 + threadIdx.x < n) gmask[(t0 + threadIdx.x) >> 4] = mk;
   }
 }
 // gmask[i] = OR of the tap masks of granule i's 16 positions; perm[t] = the position's place before the sort
@@ -862,17 +873,21 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, key_bits);
   DevBuf<int> nbr2;
   nbr2.reserve((size_t)t.K * t.npad);
+  const bool from_rows = rows && (roww == 32 || roww == 12);  // these also write the granule masks (K <= 32)
+  if (from_rows) t.gmask.reserve(ceil_div(t.n, 16));
   if (rows && roww == 32)
-    k_table_rows_permute<32><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p);
+    k_table_rows_permute<32><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p,
+                                                               t.gmask.p);
   else if (rows && roww == 12)
-    k_table_rows_permute<12><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p);
+    k_table_rows_permute<12><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p,
+                                                               t.gmask.p);
   else
     k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
                                                        t.rowmap.p);
   LAUNCH_CHECK();
   t.nbr = std::move(nbr2);
   t.identity_rows = false;
-  if (t.K <= 32) {
+  if (t.K <= 32 && !from_rows) {
     const int64_t n_granules = ceil_div(t.n, 16);
     t.gmask.reserve(n_granules);
     k_granule_masks<<<grid_for(n_granules), TB, 0, s>>>(masks, m.v1.p, t.n, n_granules, t.gmask.p);
