@@ -188,6 +188,22 @@ __device__ inline int64_t block_find(const BlockEntry *table, uint64_t mask, uin
   return -1;
 }
 
+// Coordinates and sample index back from a site key; dimensions 1 to 3 (above, keys are linear indices).
+__host__ __device__ inline void site_of_key(const Geom &g, uint64_t key, int *c, int &batch) {
+  const uint64_t low = (1ull << g.bits) - 1ull;
+  if (g.dim == 1) {
+    c[0] = (int)(key & low);
+  } else if (g.dim == 2) {
+    c[0] = (int)(compact2(key >> 1) & low);
+    c[1] = (int)(compact2(key) & low);
+  } else {
+    c[0] = (int)(compact3(key >> 2) & low);
+    c[1] = (int)(compact3(key >> 1) & low);
+    c[2] = (int)(compact3(key) & low);
+  }
+  batch = (int)(key >> (g.dim * g.bits));
+}
+
 // Occupancy bits and first row of the block with key bkey (false: no such block).  A slot's key
 // and bits come with one 16-byte load, the row only when the key matches.
 __device__ inline bool block_lookup(const BlockEntry *table, uint64_t mask, uint64_t bkey, unsigned long long &bits,

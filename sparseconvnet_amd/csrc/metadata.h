@@ -31,7 +31,8 @@ struct Level {
   DevBuf<BlockEntry> table;
   DevBuf<unsigned long long> gridp;
   DevBuf<int> urow;
-  DevBuf<unsigned long long> skeys;  // [n + 1] site key of every schedule position (ascending), kept with the grid
+  DevBuf<unsigned long long> skeys;  // [n + 1] site key of every schedule position (ascending); filled on first use
+  bool skeys_ready = false;
   bool grid_built = false;
   bool dups = false;
   // Active-site counts of the levels that successive filter 2 / stride 2 rulebooks make of this

@@ -584,6 +584,17 @@ __global__ void k_block_insert(const unsigned long long *ukey, const int *head, 
   }
 }
 
+// skeys[t] = key of the site at schedule position t (ascending), computed once per level.
+static const unsigned long long *position_keys(Level &L, hipStream_t s) {
+  if (!L.skeys_ready && L.n) {
+    L.skeys.reserve(L.n + 1);
+    k_sorted_keys<<<grid_for(L.n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), L.n, L.skeys.p);
+    LAUNCH_CHECK();
+    L.skeys_ready = true;
+  }
+  return L.skeys.p;
+}
+
 static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   if (L.grid_built) return;
   const int64_t n = L.n;
@@ -631,6 +642,7 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
     LAUNCH_CHECK();
   }
   L.grid_built = true;
+  L.skeys_ready = n > 0;
 }
 
 // ---- submanifold rules -----------------------------------------------------------------
@@ -1244,18 +1256,26 @@ __device__ inline bool candidate(const Geom &gi, const Filt &f, const int *p, in
 }
 
 // zero: 16 x 64 counters that the launch behind this one (k_strided_heads) adds to, or null.
+// pos_keys (optional, dimensions up to 3): the site key of every schedule position; the site is
+// then decoded from one coalesced read instead of gathered by row through the schedule.
 __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, const int *sched,
-                                     int64_t n, int64_t npad, unsigned long long *keys, int *payload, int *zero) {
+                                     const unsigned long long *pos_keys, int64_t n, int64_t npad,
+                                     unsigned long long *keys, int *payload, int *zero) {
   if (zero && blockIdx.x == 0)
     for (int i = threadIdx.x; i < 16 * 64; i += blockDim.x) zero[i] = 0;
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n * f.M) return;
   int64_t t = e / f.M;
   int m = (int)(e - t * f.M);
-  int row = sched ? sched[t] : (int)t;
   int p[SCN_MAXD], j[SCN_MAXD];
-  for (int d = 0; d < f.dim; d++) p[d] = soa[d * npad + row];
-  int b = soa[f.dim * npad + row];
+  int b;
+  if (pos_keys) {
+    site_of_key(gi, pos_keys[t], p, b);
+  } else {
+    const int row = sched ? sched[t] : (int)t;
+    for (int d = 0; d < f.dim; d++) p[d] = soa[d * npad + row];
+    b = soa[f.dim * npad + row];
+  }
   keys[e] = candidate(gi, f, p, m, j) ? site_key(go, j, b) : SCN_EMPTY_KEY;
   payload[e] = (int)e;
 }
@@ -1298,8 +1318,8 @@ __global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int 
 // One thread per sorted candidate: output row = number of heads before it; the filter tap
 // is the input site's offset inside the output's input box (Metadata/ConvolutionRules.h:19-31,
 // Metadata/RectangularRegions.h:30-38,95-105).
-__global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched, int64_t npad_in,
-                               const unsigned long long *skeys, const int *spayload, const int *head,
+__global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched, const unsigned long long *pos_keys,
+                               int64_t npad_in, const unsigned long long *skeys, const int *spayload, const int *head,
                                const int *head_scan, int64_t n_cand, int64_t npad_out, int *by_out,
                                int *by_in, int *out_soa, unsigned long long *out_keys,
                                unsigned long long *counts) {
@@ -1313,7 +1333,13 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
     int t = e / f.M, m = e - t * f.M;
     int row = sched ? sched[t] : t;
     int pc[SCN_MAXD], j[SCN_MAXD];
-    for (int d = 0; d < f.dim; d++) pc[d] = soa[d * npad_in + row];
+    int b;
+    if (pos_keys) {
+      site_of_key(gi, pos_keys[t], pc, b);
+    } else {
+      for (int d = 0; d < f.dim; d++) pc[d] = soa[d * npad_in + row];
+      b = soa[f.dim * npad_in + row];
+    }
     candidate(gi, f, pc, m, j);
     int k = 0;
     for (int d = 0; d < f.dim; d++) k = k * f.size[d] + (pc[d] - j[d] * f.stride[d]);
@@ -1323,7 +1349,7 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
     atomicAdd(&lcount[k], 1);
     if (head[p]) {
       for (int d = 0; d < f.dim; d++) out_soa[d * npad_out + o] = j[d];
-      out_soa[f.dim * npad_out + o] = soa[f.dim * npad_in + row];
+      out_soa[f.dim * npad_out + o] = b;
       out_keys[o] = key;
     }
   }
@@ -1398,7 +1424,9 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     m.dflags.reserve(16 * 64);
   }
   const bool count = presorted && LI.halvings.empty();
-  k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), n, LI.npad,
+  // a level with a schedule of its own (the input layer's): sites from the positions' keys
+  const unsigned long long *pos_keys = (m.dim <= 3 && !LI.identity_sched) ? position_keys(LI, s) : nullptr;
+  k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
                                                    m.k0.p, m.v0.p, count ? m.dflags.p : nullptr);
   LAUNCH_CHECK();
   if (presorted) {
@@ -1435,7 +1463,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   // both tables start empty and the counts at zero, in one launch
   fill3(R.by_out.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LO.npad, R.by_in.nbr.p, 0xFFFFFFFFu, (int64_t)f.K * LI.npad,
         R.by_out.cnt->dev.p, 0u, 2 * (int64_t)COUNT_SLOTS * std::max(f.K, 1), s);
-  k_strided_emit<<<grid_for(nc), TB, f.K * sizeof(int), s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), LI.npad, m.k1.p, m.v1.p,
+  k_strided_emit<<<grid_for(nc), TB, f.K * sizeof(int), s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), pos_keys, LI.npad, m.k1.p, m.v1.p,
                                              m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
                                              LO.coords.p, LO.keys.p, (unsigned long long *)R.by_out.cnt->dev.p);
   LAUNCH_CHECK();
