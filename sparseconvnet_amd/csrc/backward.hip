@@ -296,7 +296,7 @@ __global__ __launch_bounds__(256) void k_conv_dw(const int *__restrict__ nbr, co
         if (c < n_a && o < n_b) pk[(size_t)c * n_b + o] = acc[i][j][r];
       }
 }
-// The same sums for narrow layers (both channel counts <= 64), where the kernel above spends its
+// The same sums for narrow layers (both channel counts <= 32), where the kernel above spends its
 // time re-reading: one workgroup per tap reads the rows of b once per tap, 27 times in all.  Here
 // a workgroup of eight wavefronts takes a share of the positions and a 32 x 32 channel tile for
 // ALL taps: wavefront w keeps the accumulators of taps w, w + 8, w + 16, w + 24 (16 registers
@@ -452,10 +452,14 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
                                                       TapShares tap_shares, float *__restrict__ partial) {
   const int k = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int share = blockIdx.y;
-  // the four wavefronts of a workgroup: the 2 x 2 tiles of a 128 x 128 block, in step (see the barrier below)
+  // The four wavefronts of a workgroup: the 2 x 2 tiles of a 128 x 128 block, in step (see the
+  // barriers below); with at most 64 channels on both sides there is one tile, and the four take
+  // four shares of the positions instead, each on its own.
+  const bool single = n_a <= DWV_T && n_b <= DWV_T;
+  const int share = single ? blockIdx.y * 4 + wave : blockIdx.y;
   const int mt_o = (n_b + 2 * DWV_T - 1) / (2 * DWV_T);
-  const int ct = 2 * (blockIdx.z / mt_o) + (wave >> 1), ot = 2 * (blockIdx.z % mt_o) + (wave & 1);
+  const int ct = single ? 0 : 2 * (blockIdx.z / mt_o) + (wave >> 1), ot = single ? 0 : 2 * (blockIdx.z % mt_o) + (wave & 1);
+  if (share >= shares) return;  // (single only: its wavefronts meet at no barrier)
   const int r16 = lane & 15, g = lane >> 4;
   const int ca = ct * DWV_T + 4 * r16, cb = ot * DWV_T + 4 * r16;
   const unsigned nowhere = 0x80000000u;  // offsets from here on read zeros
@@ -527,7 +531,7 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
         for (int jx = 0; jx < 4; jx++)
           acc[i][jx] = __builtin_amdgcn_mfma_f32_16x16x4f32(q.a[kk][i], q.b[kk][jx], acc[i][jx], 0, 0, 0);
   };
-  if (share < mine) {  // uniform over the workgroup
+  if (share < mine) {  // uniform over the workgroup (over the wavefront when single)
     Quads X, Y;
     int g0 = share * DT_BLOCK;
     if (g0 >= n_granules) g0 = n_granules;
@@ -542,13 +546,13 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
       // X: rows of g0 (requested), jq / rq: indices of g1 (requested).  The barriers keep the four
       // wavefronts on the same granule, so that of two that load the same quads one reads L1.
       const int g2 = next_granule(g1), g3 = next_granule(g2);
-      __syncthreads();
+      if (!single) __syncthreads();
       if (!idle) {
         load_rows(g1, Y);
         load_indices(g2);
         multiply(X);
       }
-      __syncthreads();
+      if (!single) __syncthreads();
       if (!idle) {
         load_rows(g2, X);
         load_indices(g3);
@@ -606,7 +610,9 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     return;
   }
   const bool vec4 = n_a % 4 == 0 && n_b % 4 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0;
-  if (t.K <= DT_NW * DT_SLOTS && t.gmask.p && n_a <= 64 && n_b <= 64 && t.npad % 4 == 0 &&
+  // up to 32 channels on both sides; from there on the per-wavefront kernel below is faster
+  // (64 -> 64 at 1 M sites: 1.97 against 1.3 ms)
+  if (t.K <= DT_NW * DT_SLOTS && t.gmask.p && n_a <= DT_T && n_b <= DT_T && t.npad % 4 == 0 &&
       a_rows * n_a * 4 < ((int64_t)1 << 31) && b_rows * n_b * 4 < ((int64_t)1 << 31) &&
       (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31)) {
     // narrow layers: all taps per workgroup
@@ -637,12 +643,14 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     // first call on a table fetches them), about three workgroups per compute unit in all;
     // partial sums bounded to 256 MB, at least a block of granules per share.
     TapShares ts{};
-    int64_t shares = ceil_div(768, (int64_t)t.K * tiles);
+    const bool single = n_a <= DWV_T && n_b <= DWV_T;   // one tile: a workgroup's wavefronts take four shares
+    const int64_t groups_wanted = single ? 3072 : 768;  // wavefronts, or workgroups of four tiles
+    int64_t shares = ceil_div(groups_wanted, (int64_t)t.K * tiles);
     if (t.K <= 32 && t.K > 1) {
       ensure_counts(*t.cnt, s);
       int64_t most = 1, all = 0;
       for (int k = 0; k < t.K; k++) most = std::max(most, t.cnt->host[k]), all += t.cnt->host[k];
-      shares = ceil_div((int64_t)768 * most, std::max<int64_t>(1, all) * tiles);  // of the heaviest tap
+      shares = ceil_div(groups_wanted * most, std::max<int64_t>(1, all) * tiles);  // of the heaviest tap
     }
     shares = std::min<int64_t>(shares, std::max<int64_t>(1, ((int64_t)64 << 20) / per_chunk));
     shares = std::max<int64_t>(1, std::min<int64_t>(shares, ceil_div(t.n, 16 * DT_BLOCK)));
@@ -654,7 +662,7 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     }
     if (tiles <= 65535 && shares <= 65535) {
       m.partial.reserve((size_t)shares * per_chunk);
-      const dim3 grid((unsigned)t.K, (unsigned)shares, (unsigned)tiles);
+      const dim3 grid((unsigned)t.K, (unsigned)(single ? ceil_div(shares, 4) : shares), (unsigned)tiles);
       const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
       if (vec4)
         k_conv_dw_wave<true><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,
