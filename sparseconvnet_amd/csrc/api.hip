@@ -552,7 +552,7 @@ int scn_md_input_rules_header(scn_metadata *h, int32_t hdr[4]) {
     Metadata &m = md(h);
     if (m.input.mode < 0) throw Error("input layer rules have not been built");
     hdr[0] = m.input.user_mode;
-    hdr[1] = m.input.max_active;
+    hdr[1] = input_max_active(m);
     hdr[2] = (int32_t)m.input.n_in;
     hdr[3] = (int32_t)m.input.n_out;
   });
@@ -575,7 +575,7 @@ int scn_md_bl_rules_header(scn_metadata *h, int32_t hdr[5]) {
     Metadata &m = md(h);
     if (m.input.mode < 0 || m.input.bl_length == 0) throw Error("batch-by-length input rules have not been built");
     hdr[0] = m.input.user_mode;
-    hdr[1] = m.input.max_active;
+    hdr[1] = input_max_active(m);
     hdr[2] = (int32_t)m.input.bl_batch;
     hdr[3] = (int32_t)m.input.bl_length;
     hdr[4] = (int32_t)m.input.n_out;

@@ -132,7 +132,10 @@ struct InputRules {
   int mode = -1;      // 1: the first point of a site is listed, 2: the last, 3 / 4: all (sum / mean),
                       // 5: the first, unless later points of the site carry an overwrite flag: then the last of those
   int user_mode = -1; // the mode the caller gave (the batch-by-length layer numbers 1 and 2 the other way round)
-  int max_active = 0;
+  int max_active = 0;        // valid when max_known; read through input_max_active()
+  bool max_known = true;     // false: the longest run is still in max_slots on the device (modes 3 and 4)
+  DevBuf<int> max_slots;     // slotted maxima of the run lengths, written by the construction
+  hipStream_t built_on = nullptr;  // the stream the construction was enqueued on
   int64_t n_in = 0, n_out = 0;
   int64_t bl_batch = 0, bl_length = 0;  // batch-by-length input (BLInputLayer); 0: plain input layer
   DevBuf<int> row_of_input;  // [n_in]; -1: an empty position of a batch-by-length input
@@ -234,6 +237,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
                        const unsigned char *overwrite = nullptr);
 void generate_rulebooks(Metadata &m, int size, hipStream_t s);
 void export_input_rules(Metadata &m, int *rows, hipStream_t s);
+int input_max_active(Metadata &m);  // longest run of points on one site (modes 3 and 4), fetched from the device on first use
 void spatial_locations(Metadata &m, const int64_t *spatial, int64_t *out, hipStream_t s);
 Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *filter, hipStream_t s);
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,

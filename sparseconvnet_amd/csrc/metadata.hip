@@ -440,7 +440,8 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   if (N == 0) return;
   m.v0.reserve(std::max<int64_t>(n, 2 * N + 2));  // reused: row_of_group | head_pos
   int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
-  fill32(m.dflags.p, 0, n_flags, s);
+  R.max_slots.reserve(MAX_SLOTS * MAX_SLOT_STRIDE);
+  fill32(R.max_slots.p, 0, MAX_SLOTS * MAX_SLOT_STRIDE, s);
   k_assign_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, m.s1.p, nv, L.sched.p, row_of_group, head_pos);
   LAUNCH_CHECK();
   k_assign_coords<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, bl_length, m.f1.p, m.s1.p, n, L.npad, L.coords.p,
@@ -449,15 +450,23 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   // the groups end where the empty positions begin
   k_finish_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, row_of_group, head_pos, nv, (int)N,
                                               R.row_of_input.p, R.run_start.p, R.run_len.p,
-                                              m.dflags.p + 8);
+                                              R.max_slots.p);
   LAUNCH_CHECK();
   // Metadata/IOLayersRules.h:92,111: maxActive is 1 for modes 1 and 2, the longest run for the
-  // summing modes (runs of one never touch the slots).
+  // summing modes (runs of one never touch the slots).  Only the rule export asks for it, so
+  // it stays on the device until then (input_max_active): one host round trip less per scene.
   R.max_active = 1;
-  if (mode == 3 || mode == 4) {
-    const int *h = fetch_words(m, m.dflags.p + 8, MAX_SLOTS * MAX_SLOT_STRIDE, s);
+  R.max_known = !(mode == 3 || mode == 4);
+  R.built_on = s;
+}
+int input_max_active(Metadata &m) {
+  InputRules &R = m.input;
+  if (!R.max_known) {
+    const int *h = fetch_words(m, R.max_slots.p, MAX_SLOTS * MAX_SLOT_STRIDE, R.built_on);
     for (int i = 0; i < MAX_SLOTS; i++) R.max_active = std::max(R.max_active, h[i * MAX_SLOT_STRIDE]);
+    R.max_known = true;
   }
+  return R.max_active;
 }
 
 // Reference layout of the rule rows (Metadata/IOLayersRules.h:96-119).
@@ -480,7 +489,7 @@ void export_input_rules(Metadata &m, int *rows, hipStream_t s) {
   InputRules &R = m.input;
   if (R.mode <= 0 || R.n_out == 0) return;
   k_export_input_rules<<<grid_for(R.n_out), TB, 0, s>>>(R.sorted_idx.p, R.run_start.p, R.run_len.p,
-                                                        R.overwrite.p, R.n_out, R.mode, R.max_active, rows);
+                                                        R.overwrite.p, R.n_out, R.mode, input_max_active(m), rows);
   LAUNCH_CHECK();
 }
 
