@@ -296,12 +296,14 @@ __global__ void k_group_heads(const unsigned long long *skeys, const int *sidx, 
 // Two passes so that every array is written in ascending order (stream compaction) instead of
 // being scattered: one over the sorted points for what is indexed by group (key order) ...
 __global__ void k_assign_groups(const int *sidx, const int *head, const int *head_scan, const int *first_scan,
-                                int64_t n, int *sched, int *row_of_group, int *head_pos) {
+                                const unsigned long long *sorted_keys, int64_t n, int *sched, int *row_of_group,
+                                int *head_pos, unsigned long long *pos_keys) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n || !head[p]) return;
   const int row = first_scan[sidx[p]];
   const int u = head_scan[p];
   sched[u] = row;
+  pos_keys[u] = sorted_keys[p];  // the level's keys by schedule position (Level::skeys)
   row_of_group[u] = row;
   head_pos[u] = (int)p;
 }
@@ -442,7 +444,10 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   int *row_of_group = m.v0.p, *head_pos = m.v0.p + N;
   R.max_slots.reserve(MAX_SLOTS * MAX_SLOT_STRIDE);
   fill32(R.max_slots.p, 0, MAX_SLOTS * MAX_SLOT_STRIDE, s);
-  k_assign_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, m.s1.p, nv, L.sched.p, row_of_group, head_pos);
+  L.skeys.reserve(N + 1);
+  k_assign_groups<<<grid_for(nv), TB, 0, s>>>(m.v1.p, m.f0.p, m.s0.p, m.s1.p, m.k1.p, nv, L.sched.p, row_of_group, head_pos,
+                                              L.skeys.p);
+  L.skeys_ready = true;
   LAUNCH_CHECK();
   k_assign_coords<<<grid_for(n), TB, 0, s>>>(g, coords, ncols, bl_length, m.f1.p, m.s1.p, n, L.npad, L.coords.p,
                                              L.keys.p);
@@ -636,6 +641,9 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
       ukey = m.k1.p;
       // positions past the last distinct site hold stale keys: heads there are never read
       k_block_heads<<<grid_for(n), TB, 0, s>>>(ukey, n, m.f0.p);
+      LAUNCH_CHECK();
+    } else if (L.skeys_ready) {  // the input layer left the positions' keys
+      k_block_heads<<<grid_for(n), TB, 0, s>>>(L.skeys.p, n, m.f0.p);
       LAUNCH_CHECK();
     } else {
       k_grid_heads<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, L.skeys.p, m.f0.p);
