@@ -5,7 +5,7 @@
 // that a general-purpose library sort spends its time in launches (a histogram pass, then per
 // digit a look-back scan with two state fills in front), which is what this file avoids.
 //
-// Per digit (up to 9 bits) three launches, none of which waits on another workgroup:
+// Per digit (up to 10 bits) three launches, none of which waits on another workgroup:
 //   k_rs_hist     per tile of TILE pairs, the count of every digit value   hist[digit][tile]
 //   k_rs_colscan  per digit value, the exclusive prefix over tiles (in place) and the total
 //   k_rs_scatter  per tile: rank every pair among the tile's pairs of the same digit value
@@ -24,8 +24,8 @@ namespace scn {
 
 typedef unsigned long long u64;
 constexpr int RS_THREADS = 256, RS_WAVES = 4, RS_ITEMS = 8, RS_TILE = RS_THREADS * RS_ITEMS;  // 2048 pairs per tile
-constexpr int RS_MAX_BITS = 9, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured: four
-// digits of 9 bits beat three of 11 and five of 7 on a million pairs of 35 bits)
+constexpr int RS_MAX_BITS = 10, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured on a million
+// pairs of 35 bits: four digits of 9 bits beat three of 11 and five of 7; 40 bits sort in four digits of 10)
 
 __global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const u64 *__restrict__ keys, int64_t n, int shift, int bits,
                                                         int tiles, int *__restrict__ hist) {
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict
   const unsigned mask = (unsigned)bins - 1u;
   // exclusive scan of the digit values' totals (thread t: values [t * per, (t + 1) * per)) + this tile's prefix
   {
-    const int per = (bins + RS_THREADS - 1) / RS_THREADS;  // 1 or 2
+    const int per = (bins + RS_THREADS - 1) / RS_THREADS;  // 1 to 4
     const int d0 = threadIdx.x * per;
     int mine = 0;
     for (int j = 0; j < per; j++)
@@ -159,7 +159,7 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
   if (n <= 0) return;
   end_bit = std::max(1, std::min(64, end_bit));
   if (n >= ((int64_t)1 << 31)) throw Error("sort: too many pairs");
-  // as few digits as 9 bits each allow, of equal width
+  // as few digits as RS_MAX_BITS bits each allow, of equal width
   const int passes = (end_bit + RS_MAX_BITS - 1) / RS_MAX_BITS;
   const int width = (end_bit + passes - 1) / passes;
   const int tiles = (int)ceil_div(n, RS_TILE);
