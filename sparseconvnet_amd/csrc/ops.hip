@@ -175,6 +175,33 @@ __global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const i
     out[i] = acc;
   }
 }
+// The same for one to four planes (coordinates-and-colour inputs): one thread per row, so that
+// a row's run and point indices are read once instead of once per plane.
+template <int P>
+__global__ void k_input_fwd_row(const int *__restrict__ sorted_idx, const int *__restrict__ run_start,
+                                const int *__restrict__ run_len, const unsigned char *__restrict__ overwrite, int64_t n_out,
+                                int mode, const float *__restrict__ in, float *__restrict__ out, int average) {
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_out) return;
+  const int st = run_start[r], len = run_len[r];
+  float acc[P];
+#pragma unroll
+  for (int p = 0; p < P; p++) acc[p] = 0.0f;
+  if (mode == 1 || mode == 2 || mode == 5) {
+    const float *src = in + (int64_t)listed_point(sorted_idx, st, len, mode, overwrite) * P;
+#pragma unroll
+    for (int p = 0; p < P; p++) acc[p] += src[p];
+  } else {
+    const float mult = (average && len > 0) ? 1.0f / (float)len : 1.0f;
+    for (int q = 0; q < len; q++) {
+      const float *src = in + (int64_t)sorted_idx[st + q] * P;
+#pragma unroll
+      for (int p = 0; p < P; p++) acc[p] += mult * src[p];
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < P; p++) out[r * P + p] = acc[p];
+}
 void input_forward(const InputRules &r, const float *in, float *out, int planes, hipStream_t s) {
   if (r.mode < 0) throw Error("input layer rules have not been built");
   if (planes <= 0) return;
@@ -184,10 +211,24 @@ void input_forward(const InputRules &r, const float *in, float *out, int planes,
     return;
   }
   if (r.n_out == 0) return;
+  const int average = r.mode == 4 ? 1 : 0;
+  if (planes <= 4) {
+    const dim3 grid((unsigned)ceil_div(r.n_out, TB));
+#define SCN_ROW(P)                                                                                                  \
+  k_input_fwd_row<P><<<grid, TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p, r.n_out, r.mode, in, \
+                                         out, average)
+    if (planes == 1) SCN_ROW(1);
+    else if (planes == 2) SCN_ROW(2);
+    else if (planes == 3) SCN_ROW(3);
+    else SCN_ROW(4);
+#undef SCN_ROW
+    LAUNCH_CHECK();
+    return;
+  }
   int64_t total = r.n_out * planes;
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p,
-                                                    r.n_out, r.mode, in, out, planes, r.mode == 4 ? 1 : 0);
+                                                    r.n_out, r.mode, in, out, planes, average);
   LAUNCH_CHECK();
 }
 // CPU/IOLayers.cpp:116-135 (and :207-229): the gradient of the output layer's input is
