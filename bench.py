@@ -210,16 +210,22 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
             torch.cuda.synchronize()
         graph_ms = med(reps_ms) if same else None
         del graph
+    # device memory the library itself holds (rulebooks of the live handles, scratch, idle blocks of
+    # its cache; features and weights are torch's): high-water mark since the process started
+    import ctypes
+    peak = ctypes.c_int64(0)
+    scn.metadata._lib.lib().scn_cache_stats(None, None, ctypes.byref(peak), None)
     if batch > 1:
         return {"unet_batch%d_ms_per_batch" % batch: med(cold), "unet_batch%d_warm_ms_per_batch" % batch: med(warm),
                 "unet_batch%d_from_host_coords_ms_per_batch" % batch: med(cold_host),
-                "unet_batch%d_active_sites" % batch: int(x.features.shape[0])}
+                "unet_batch%d_active_sites" % batch: int(x.features.shape[0]),
+                "library_peak_MiB_after_batch%d" % batch: round(peak.value / 2 ** 20)}
     if residual:
         return {"unet_residual_ms_per_scene": med(cold), "unet_residual_warm_ms": med(warm),
                 "unet_residual_gflop": round(2 * macs / 1e9, 2)}
     return {"unet_ms_per_scene": med(cold), "unet_ms_per_scene_from_host_coords": med(cold_host),
             "unet_warm_ms": med(warm), "unet_warm_graph_replay_ms": graph_ms, "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
-            "unet_gflop": round(2 * macs / 1e9, 2),
+            "unet_gflop": round(2 * macs / 1e9, 2), "library_peak_MiB": round(peak.value / 2 ** 20),
             "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1),
             "unet_warm_frac_mfma_fp32": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e12 / MFMA_FP32_TFLOPS, 4),
             "note": "ms_per_scene: new Metadata per scene (input layer, every rulebook, all layers), coordinates "
