@@ -1415,9 +1415,8 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
 // Narrow layers: nOut <= 32, any nIn, K <= 32.  nIn is processed in parts of up to 32
 // channels so that every part's weights fit in LDS; parts after the first accumulate.
 // The resident kernel serves nOut <= 32 with up to 32 taps.  It takes the input channels in
-// parts of 32 and has no fused batch norm, so from 128 input channels on, or from 64 when a
-// batch norm comes with the call or the filter has few taps, the row-owner kernel is at
-// least as fast (measured).
+// parts of 32 (every part after the first re-reads and re-writes the output) and has no fused
+// batch norm, so from 64 input channels on the row-owner kernel is faster (measured).
 static bool resident_fits(const Metadata &m, const Table &t, int n_in, int n_out, bool with_bn) {
   if (!(t.K <= 32 && n_out <= 32 && t.gmask.p != nullptr)) return false;
   // the resident kernel computes in fp32 only; from two parts on the row-owner kernel's bf16
@@ -1426,7 +1425,8 @@ static bool resident_fits(const Metadata &m, const Table &t, int n_in, int n_out
   // several parts re-read and re-write the output once per part: with few taps (strided and
   // transposed convolutions) that costs more than the convolution itself
   if (n_in > 32 && t.K <= 8) return false;
-  return n_in < (with_bn ? 64 : 128);
+  (void)with_bn;
+  return n_in < 64;  // two parts and more: the row-owner kernel is 3 % (64 -> 32) to 10 % (96 -> 32) faster at 1 M sites
 }
 
 // No fused batch norm here: this kernel's time goes into the vector instructions around its
