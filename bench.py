@@ -234,6 +234,40 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
                     "warm_graph_replay: the warm pass replayed as one HIP graph (null if the replay's result differed)"}
 
 
+def unet_train_step(sites, seed, reps=3):
+    """One training step of the same U-Net (train mode: batch norms take batch statistics) on one
+    room scene: InputLayer, forward, a scalar loss, backward through every layer down to the
+    input features and every parameter.  New Metadata per step, as a training loop runs."""
+    import torch
+    import sparseconvnet_amd as scn
+    from sparseconvnet_amd import synthetic
+    m = 32
+    torch.manual_seed(0)
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m, 4 * m, 5 * m, 6 * m, 7 * m], False)).add(
+        scn.BatchNormReLU(m)).add(scn.OutputLayer(3)).cuda().train()
+    linear = torch.nn.Linear(m, 20).cuda()
+    coords = synthetic.room_scene(seed=seed, target=sites, spatial=4096, duplicate_fraction=0.3)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    feats = (torch.rand((len(coords), 3), device="cuda", generator=g) * 2 - 1).requires_grad_(True)
+    cd = torch.as_tensor(coords).cuda()
+    inp_layer = scn.InputLayer(3, 4096, mode=4)
+    ms = []
+    for r in range(reps + 1):
+        for p in list(model.parameters()) + list(linear.parameters()):
+            p.grad = None
+        feats.grad = None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        y = linear(model(inp_layer([cd, feats])))
+        y.square().mean().backward()
+        torch.cuda.synchronize()
+        ms.append((time.perf_counter() - t0) * 1e3)
+    return {"unet_train_step_ms": round(float(np.median(ms[1:])), 3),
+            "unet_train_step_note": "forward in train mode + backward of one %d-point scene, new Metadata per step, "
+                                    "optimizer step not included" % len(coords)}
+
+
 def _timed(torch, fn, reps=5):
     fn()
     ms = []
@@ -744,6 +778,8 @@ def main():
         if not args.no_residual:
             out["unet"].update(unet_scene(args.unet_sites, 5000, residual=True))
             out["unet"].update(unet_scene(args.unet_sites, 7000, reps=2, batch=4))
+        if not args.no_backward:
+            out["unet"].update(unet_train_step(args.unet_sites, 5000))
         if not args.no_bf16:
             import sparseconvnet_amd as scn
             scn.bf16_mfma = True

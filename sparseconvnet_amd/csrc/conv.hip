@@ -519,7 +519,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       const int64_t pos = tbase + (wr * GW + q) * 16 + 4 * g + r;
       if (pos >= n) continue;
       const int64_t row = rowmap ? rowmap[pos] : pos;
-      float *o = out + row * n_out;
+      float *o = out + row * (epi.out_stride ? epi.out_stride : n_out);
 #pragma unroll
       for (int c = 0; c < NCBW; c++) {
         const int col = 16 * (wc * NCBW + c) + r16;
@@ -542,7 +542,7 @@ __global__ void k_conv_reduce(const float *partial, int n_split, int64_t split_s
   for (int sp = 0; sp < n_split; sp++) acc += partial[sp * split_stride + pos * ld + col];
   if (epi.sc) acc = epi_act(acc, epi.sc[col], epi.sh[col], epi.leak);
   int64_t row = rowmap ? rowmap[pos] : pos;
-  out[row * n_out + col] = acc;
+  out[row * (epi.out_stride ? epi.out_stride : n_out) + col] = acc;
 }
 
 struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
@@ -902,7 +902,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
       const int64_t pos = tbase + (wave * RG + q) * 16 + 4 * g + r;
       if (pos >= n) continue;
       const int64_t row = rowmap ? rowmap[pos] : pos;
-      float *o = out + row * n_out;
+      float *o = out + row * (epi.out_stride ? epi.out_stride : n_out);
 #pragma unroll
       for (int cb = 0; cb < NCB; cb++) {
         const int col = 16 * cb + r16;
@@ -1520,6 +1520,15 @@ static bool conv_mfma_paths(Metadata &m, const Table &t, const float *in, float 
   return false;
 }
 
+// dst[r][c] = w[r][c0 + c], c < wc: one column range of a [rows x n_out] weight matrix, contiguous.
+__global__ void k_take_columns(const float *w, int64_t rows, int n_out, int c0, int wc, float *dst) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * wc) return;
+  const int64_t r = i / wc;
+  const int c = (int)(i - r * wc);
+  dst[i] = w[r * n_out + c0 + c];
+}
+
 // bn: optional eval batch norm + leaky ReLU applied to the input rows before the convolution
 // (what a BatchNormalization module in front of the convolution computes), fused into the
 // gather; post: the same for a BatchNormalization module behind the convolution, applied to
@@ -1588,6 +1597,28 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     m.cur_in_base = src;
   }
   if (groups == 1 && conv_mfma_paths<false>(m, t, src, out, w, epi, n_in, n_out, PreArgs(), s)) return;
+  if (groups == 1 && n_out > 256 && t.n > 0) {
+    // More output planes than the MFMA kernels hold accumulators for (the input gradient of a
+    // convolution behind a JoinTable is one): ranges of at most 256 columns, each a convolution
+    // of its own over that range's weights, written into its columns of `out`.
+    const int ranges = (int)ceil_div(n_out, 256);
+    const int width = (int)round_up(ceil_div(n_out, ranges), 16);
+    const int64_t rows_w = (int64_t)t.K * n_in;
+    m.wcols.reserve((size_t)rows_w * n_out);
+    bool ok = true;
+    for (int c0 = 0; c0 < n_out && ok; c0 += width) {
+      const int wc = std::min(width, n_out - c0);
+      float *dst = m.wcols.p + rows_w * c0;
+      k_take_columns<<<dim3((unsigned)ceil_div(rows_w * wc, 256)), 256, 0, s>>>(w, rows_w, n_out, c0, wc, dst);
+      LAUNCH_CHECK();
+      Epi e = epi;
+      if (e.bias) e.bias += c0;
+      if (e.sc) e.sc += c0, e.sh += c0;
+      e.out_stride = n_out;
+      ok = conv_mfma_paths<false>(m, t, src, out + c0, dst, e, n_in, wc, PreArgs(), s);
+    }
+    if (ok) return;
+  }
   if (m.jobs.post.n_pad) {  // no packing launch on this path: fold the coefficients by themselves
     k_coefs<<<dim3(1), 256, 0, s>>>(take_jobs(m));
     LAUNCH_CHECK();

@@ -181,6 +181,7 @@ struct Metadata {
   DevBuf<unsigned char> tmp;
   DevBuf<unsigned long long> k0, k1;
   DevBuf<int> v0, v1, f0, f1, s0, s1;
+  DevBuf<float> wcols;  // column ranges of a wide layer's weights, one contiguous block per range (conv_forward)
   DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
@@ -258,6 +259,7 @@ struct Epi {
   const float *bias = nullptr;               // [nOut] or null
   const float *sc = nullptr, *sh = nullptr;  // [nOut] each, or nulls
   float leak = 1.0f;
+  int out_stride = 0;  // floats between output rows; 0: nOut (k_conv_mfma, k_conv_rows, k_conv_reduce honour it)
 };
 __device__ inline float epi_act(float v, float sc, float sh, float leak) {
   const float y = v * sc + sh;
