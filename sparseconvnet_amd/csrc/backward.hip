@@ -453,12 +453,17 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
   const int k = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // The four wavefronts of a workgroup: the 2 x 2 tiles of a 128 x 128 block, in step (see the
-  // barriers below); with at most 64 channels on both sides there is one tile, and the four take
-  // four shares of the positions instead, each on its own.
-  const bool single = n_a <= DWV_T && n_b <= DWV_T;
-  const int share = single ? blockIdx.y * 4 + wave : blockIdx.y;
+  // barriers below).  A layer of fewer than four tiles (at most 64 channels on one side and 128 on
+  // the other) would leave wavefronts idle that way: there the workgroup's four wavefronts are
+  // four (share, tile) pairs in a row, each on its own.
+  const int tiles_a = (n_a + DWV_T - 1) / DWV_T, tiles_b = (n_b + DWV_T - 1) / DWV_T;
+  const bool single = tiles_a * tiles_b < 4;
+  const int slot = blockIdx.y * 4 + wave;
+  const int share = single ? slot / (tiles_a * tiles_b) : blockIdx.y;
+  const int tile = slot % (tiles_a * tiles_b);
   const int mt_o = (n_b + 2 * DWV_T - 1) / (2 * DWV_T);
-  const int ct = single ? 0 : 2 * (blockIdx.z / mt_o) + (wave >> 1), ot = single ? 0 : 2 * (blockIdx.z % mt_o) + (wave & 1);
+  const int ct = single ? tile / tiles_b : 2 * (blockIdx.z / mt_o) + (wave >> 1);
+  const int ot = single ? tile % tiles_b : 2 * (blockIdx.z % mt_o) + (wave & 1);
   if (share >= shares) return;  // (single only: its wavefronts meet at no barrier)
   const int r16 = lane & 15, g = lane >> 4;
   const int ca = ct * DWV_T + 4 * r16, cb = ot * DWV_T + 4 * r16;
@@ -638,13 +643,14 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
   if (t.npad % 4 == 0 && a_rows * n_a * 4 < ((int64_t)1 << 31) && b_rows * n_b * 4 < ((int64_t)1 << 31) &&
       (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31) && t.K <= 65535) {
     // wider layers: a wavefront per (tap, 64 x 64 tile, share of the positions)
-    const int tiles = (int)(ceil_div(n_a, 2 * DWV_T) * ceil_div(n_b, 2 * DWV_T));  // blocks of 2 x 2 tiles
+    const int tiles64 = (int)(ceil_div(n_a, DWV_T) * ceil_div(n_b, DWV_T));
+    const bool single = tiles64 < 4;  // fewer than four tiles: a workgroup's wavefronts are (share, tile) pairs
+    const int tiles = single ? 1 : (int)(ceil_div(n_a, 2 * DWV_T) * ceil_div(n_b, 2 * DWV_T));  // blocks of 2 x 2 tiles
     // Shares of the positions per tap in proportion to the tap's rules (the table's counts; the
     // first call on a table fetches them), about three workgroups per compute unit in all;
     // partial sums bounded to 256 MB, at least a block of granules per share.
     TapShares ts{};
-    const bool single = n_a <= DWV_T && n_b <= DWV_T;   // one tile: a workgroup's wavefronts take four shares
-    const int64_t groups_wanted = single ? 3072 : 768;  // wavefronts, or workgroups of four tiles
+    const int64_t groups_wanted = single ? 3072 / tiles64 : 768;  // shares of wavefronts, or workgroups of four tiles
     int64_t shares = ceil_div(groups_wanted, (int64_t)t.K * tiles);
     if (t.K <= 32 && t.K > 1) {
       ensure_counts(*t.cnt, s);
@@ -662,7 +668,7 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     }
     if (tiles <= 65535 && shares <= 65535) {
       m.partial.reserve((size_t)shares * per_chunk);
-      const dim3 grid((unsigned)t.K, (unsigned)(single ? ceil_div(shares, 4) : shares), (unsigned)tiles);
+      const dim3 grid((unsigned)t.K, (unsigned)(single ? ceil_div(shares * tiles64, 4) : shares), (unsigned)tiles);
       const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
       if (vec4)
         k_conv_dw_wave<true><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,
