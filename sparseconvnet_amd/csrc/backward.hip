@@ -169,13 +169,29 @@ __global__ __launch_bounds__(1024) void k_sum_blocks(const float *__restrict__ p
     out[i] = (OUT)tot;
   }
 }
-// The two column sums of a batch-normalisation pass in double, behind the blocks' partial sums.
-static double *sum_pairs(Metadata &m, int blocks, int planes, hipStream_t s) {
-  double *sums = reinterpret_cast<double *>(m.partial.p + (size_t)blocks * 2 * planes);
-  k_sum_blocks<double, double><<<dim3((unsigned)ceil_div(2 * planes, 64)), 1024, 0, s>>>(m.partial.p, blocks, (int64_t)2 * planes,
-                                                                                        (int64_t)2 * planes, sums);
-  LAUNCH_CHECK();
-  return sums;
+// The two column sums of a batch-normalisation pass, in double, for the 64 columns of workgroup
+// blockIdx.x (1024 threads): partial[b][q][c] summed over the row blocks b in the fixed order of
+// k_sum_blocks.  Every thread of wavefront 0 returns with the sums of column blockIdx.x * 64 + lane.
+__device__ inline void pair_sums64(const float *__restrict__ partial, int blocks, int planes, double &s1, double &s2) {
+  __shared__ double part[2][16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const int per = (blocks + 15) / 16;
+  const int b0 = min(blocks, wave * per), b1 = min(blocks, b0 + per);
+  double a = 0, b = 0;
+  if (c < planes)
+    for (int i = b0; i < b1; i++) {
+      a += (double)partial[(size_t)i * 2 * planes + c];
+      b += (double)partial[(size_t)i * 2 * planes + planes + c];
+    }
+  part[0][wave][lane] = a;
+  part[1][wave][lane] = b;
+  __syncthreads();
+  s1 = s2 = 0;
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 0; w < 16; w++) s1 += part[0][w][lane], s2 += part[1][w][lane];
+  }
 }
 static void column_sums(Metadata &m, const float *x, int64_t rows, int planes, float *out, hipStream_t s) {
   if (planes <= 0) return;
@@ -811,12 +827,14 @@ void strided_conv_backward(Metadata &m, const Table &fwd, const Table &other, in
 // CPU/BatchNormalization.cpp:19-40: batch mean and biased variance into save_mean / save_invstd,
 // running statistics updated with `momentum` weighting the old value and the unbiased variance;
 // coef = scale | shift for the affine pass.
-__global__ void k_bn_train_finish(const double *sums, int planes, int64_t rows, float *save_mean,
-                                  float *save_invstd, float *running_mean, float *running_var, const float *gamma,
-                                  const float *beta, float eps, float momentum, float *coef) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= planes) return;
-  const double s1 = sums[c], s2 = sums[planes + c];
+__global__ __launch_bounds__(1024) void k_bn_train_finish(const float *partial, int blocks, int planes, int64_t rows,
+                                                          float *save_mean, float *save_invstd, float *running_mean,
+                                                          float *running_var, const float *gamma, const float *beta,
+                                                          float eps, float momentum, float *coef) {
+  double s1, s2;
+  pair_sums64(partial, blocks, planes, s1, s2);
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  if (threadIdx.x >= 64 || c >= planes) return;
   const double mean = s1 / (double)rows;
   double ss = s2 - mean * mean * (double)rows;  // sum of squared deviations
   if (ss < 0) ss = 0;
@@ -848,25 +866,27 @@ void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t ro
   if (rows <= 0 || planes <= 0) return;
   Metadata &m = *scratch;
   const ColsumPlan p = colsum_plan(rows, planes);
-  m.partial.reserve((size_t)p.blocks * 2 * planes + 4 * (size_t)planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes);
   m.prebuf.reserve(2 * (size_t)planes);
   launch_colsum<1>(dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), s, in, in_stride, nullptr, nullptr, 0, nullptr,
                                                                                  0.f, rows, planes, p.CW, p.rows_per_block,
                                                                                  m.partial.p);
-  const double *sums = sum_pairs(m, p.blocks, planes, s);
-  k_bn_train_finish<<<grid_for(planes), TB, 0, s>>>(sums, planes, rows, save_mean, save_invstd,
-                                                    running_mean, running_var, gamma, beta, eps, momentum, m.prebuf.p);
+  k_bn_train_finish<<<dim3((unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_mean,
+                                                                          save_invstd, running_mean, running_var, gamma,
+                                                                          beta, eps, momentum, m.prebuf.p);
   LAUNCH_CHECK();
   const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
   k_affine_leaky<<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, m.prebuf.p, leak);
   LAUNCH_CHECK();
 }
 // CPU/BatchNormalization.cpp:84-106: coef = gradMean | k | invstd * gamma
-__global__ void k_bn_bwd_finish(const double *sums, int planes, int64_t rows, const float *save_invstd,
-                                const float *gamma, float *d_gamma, float *d_beta, float *coef) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= planes) return;
-  const double sd = sums[c], dotp = sums[planes + c];
+__global__ __launch_bounds__(1024) void k_bn_bwd_finish(const float *partial, int blocks, int planes, int64_t rows,
+                                                        const float *save_invstd, const float *gamma, float *d_gamma,
+                                                        float *d_beta, float *coef) {
+  double sd, dotp;
+  pair_sums64(partial, blocks, planes, sd, dotp);
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  if (threadIdx.x >= 64 || c >= planes) return;
   const float invstd = save_invstd[c];
   if (d_beta) d_beta[c] = (float)sd;
   if (d_gamma) d_gamma[c] = (float)dotp * invstd;
@@ -900,14 +920,13 @@ void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *o
   }
   Metadata &m = *scratch;
   const ColsumPlan p = colsum_plan(rows, planes);
-  m.partial.reserve((size_t)p.blocks * 2 * planes + 4 * (size_t)planes);
+  m.partial.reserve((size_t)p.blocks * 2 * planes);
   m.prebuf.reserve(3 * (size_t)planes);
   launch_colsum<2>(dim3(p.blocks, (unsigned)ceil_div(planes, p.CW)), s, in, in_stride, d_out, out, out_stride,
                                                                                  save_mean, leak, rows, planes, p.CW,
                                                                                  p.rows_per_block, m.partial.p);
-  const double *sums = sum_pairs(m, p.blocks, planes, s);
-  k_bn_bwd_finish<<<grid_for(planes), TB, 0, s>>>(sums, planes, rows, save_invstd, gamma, d_gamma, d_beta,
-                                                  m.prebuf.p);
+  k_bn_bwd_finish<<<dim3((unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_invstd,
+                                                                        gamma, d_gamma, d_beta, m.prebuf.p);
   LAUNCH_CHECK();
   const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
   k_bn_bwd_apply<<<dim3((unsigned)blocks), TB, 0, s>>>(in, d_in, out, d_out, rows, planes, in_stride, out_stride, save_mean,

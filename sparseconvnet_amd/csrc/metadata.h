@@ -135,7 +135,6 @@ struct InputRules {
   int max_active = 0;        // valid when max_known; read through input_max_active()
   bool max_known = true;     // false: the longest run is still in max_slots on the device (modes 3 and 4)
   DevBuf<int> max_slots;     // slotted maxima of the run lengths, written by the construction
-  hipStream_t built_on = nullptr;  // the stream the construction was enqueued on
   int64_t n_in = 0, n_out = 0;
   int64_t bl_batch = 0, bl_length = 0;  // batch-by-length input (BLInputLayer); 0: plain input layer
   DevBuf<int> row_of_input;  // [n_in]; -1: an empty position of a batch-by-length input

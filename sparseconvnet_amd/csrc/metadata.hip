@@ -462,12 +462,14 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   // it stays on the device until then (input_max_active): one host round trip less per scene.
   R.max_active = 1;
   R.max_known = !(mode == 3 || mode == 4);
-  R.built_on = s;
 }
 int input_max_active(Metadata &m) {
   InputRules &R = m.input;
   if (!R.max_known) {
-    const int *h = fetch_words(m, R.max_slots.p, MAX_SLOTS * MAX_SLOT_STRIDE, R.built_on);
+    // a rare call (rule export): wait for the whole device rather than keep the construction's stream alive
+    std::vector<int> h((size_t)MAX_SLOTS * MAX_SLOT_STRIDE);
+    HIP_CHECK(hipDeviceSynchronize());
+    HIP_CHECK(hipMemcpy(h.data(), R.max_slots.p, h.size() * sizeof(int), hipMemcpyDeviceToHost));
     for (int i = 0; i < MAX_SLOTS; i++) R.max_active = std::max(R.max_active, h[i * MAX_SLOT_STRIDE]);
     R.max_known = true;
   }
