@@ -175,7 +175,8 @@ def test_strided_tree_vs_oracle(oracle_built):
 
 
 @pytest.mark.parametrize("cin,cout,groups", [(3, 32, 1), (32, 32, 1), (40, 16, 1), (48, 64, 1), (64, 96, 1),
-                                             (96, 128, 1), (128, 160, 1), (30, 50, 1), (64, 32, 1), (8, 12, 2)])
+                                             (96, 128, 1), (128, 160, 1), (30, 50, 1), (64, 32, 1), (8, 12, 2),
+                                             (48, 320, 1)])
 def test_fused_bn_conv_vs_oracle(oracle_built, cin, cout, groups):
     """The fused entry point (eval batch norm + leaky ReLU in front of the convolution applied
     in its gather, the one behind it applied to its stores) against the oracle's separate
