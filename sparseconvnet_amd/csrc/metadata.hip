@@ -573,27 +573,36 @@ __global__ void k_block_clear(BlockEntry *table, int64_t cap_alloc, const int *h
     table[b].base = 0;
   }
 }
-// The first site of every block collects the occupancy bits of its block (its run of at most
-// 64 consecutive distinct keys), claims a slot and stores key, mask and its own rank.
+// One lane per distinct site (ascending keys).  The sites of a block are neighbours in that order,
+// so a wavefront ORs the occupancy bits of each run of equal block keys it holds with six
+// shuffle steps; the first lane of a run claims the block's slot (or finds it, when the run began
+// in the wavefront before and that one was faster) and ORs the run's bits in; the lane that
+// starts the block (head) also stores its rank.  k_block_clear has zeroed the bits.
 __global__ void k_block_insert(const unsigned long long *ukey, const int *head, int64_t n_sites,
                                const int *n_sites_dev, BlockEntry *table, const unsigned long long *mask_p) {
-  int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t U = n_sites_dev ? (int64_t)*n_sites_dev + 1 : n_sites;
-  if (u >= U || !head[u]) return;
-  const unsigned long long mask = *mask_p;
-  const unsigned long long bkey = ukey[u] >> 6;
-  unsigned long long bits = 0;
-  for (int64_t v = u; v < U && v < u + 64; v++) {
-    const unsigned long long k = ukey[v];
-    if ((k >> 6) != bkey) break;
-    bits |= 1ull << (k & 63);
+  const int lane = threadIdx.x & 63;
+  const bool live = u < U;
+  const unsigned long long k = live ? ukey[u] : 0ull;
+  // dead lanes (behind the last site) get a block key no live lane has
+  const unsigned long long bkey = live ? k >> 6 : SCN_EMPTY_KEY;
+  unsigned long long bits = live ? 1ull << (k & 63) : 0ull;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const unsigned long long other_bits = __shfl_down(bits, o, 64);
+    const unsigned long long other_key = __shfl_down(bkey, o, 64);
+    if (lane + o < 64 && other_key == bkey) bits |= other_bits;
   }
+  const unsigned long long before = __shfl_up(bkey, 1, 64);
+  if (!live || (lane > 0 && before == bkey)) return;  // not the first lane of its run
+  const unsigned long long mask = *mask_p;
   unsigned long long b = hash64(bkey) & mask;
   for (unsigned long long i = 0; i <= mask; i++) {
-    unsigned long long old = atomicCAS(&table[b].key, SCN_EMPTY_KEY, bkey);
-    if (old == SCN_EMPTY_KEY) {
-      table[b].mask = bits;
-      table[b].base = (int)u;
+    const unsigned long long old = atomicCAS(&table[b].key, SCN_EMPTY_KEY, bkey);
+    if (old == SCN_EMPTY_KEY || old == bkey) {
+      atomicOr(&table[b].mask, bits);
+      if (head[u]) table[b].base = (int)u;
       return;
     }
     b = (b + 1) & mask;
