@@ -583,6 +583,14 @@ def other_ops(sites, seed):
     del m3
     out.append(row("precompute_metadata(2): 3^3 and 2^3/stride-2 rulebooks of all %d levels (%d sites in all)"
                    % (sum(1 for v in levels if v), total), ms, byts, sites_per_s=round(total / (ms * 1e-3))))
+    # per-sample mean of the active rows (one sample here: a column mean over every row), on the
+    # level a stride-2 convolution made (rows in site order) and on the input level (rows in the
+    # caller's point order: the sums walk the samples' site ranges, a gather there)
+    ms = timed(lambda: md.activePooling(half, yc, True))
+    out.append(row("ActivePooling (mean), 64 planes, %d sites (level of a stride-2 convolution)" % yc.shape[0], ms,
+                   yc.shape[0] * 64 * 4 + 64 * 4))
+    ms = timed(lambda: md.activePooling(sz, x32, True))
+    out.append(row("ActivePooling (mean), 32 planes, input level", ms, n * 32 * 4 + 32 * 4))
     # sparse to dense on a grid that can be dense: the same scene generator at 128^3, 16 planes
     c2 = synthetic.room_scene(seed=seed + 1, target=200000, spatial=128)
     md2 = M.Metadata(3)

@@ -362,34 +362,73 @@ __global__ void k_sample_starts(const int *soa, const int *sched, int dim, int64
     for (int q = b + 1; q <= batch; q++) start[q] = (int)n;
 }
 // grid (sample * chunks + chunk, column tile of CW): partial[(sample * chunks + chunk) * planes + c]
-__global__ void k_active_pool_partial(const int *sched, const int *start, int chunks, const float *in, int planes,
-                                      int CW, float *partial) {
-  __shared__ float red[256];
+template <int V>
+__global__ __launch_bounds__(256) void k_active_pool_partial(const int *__restrict__ sched, const int *__restrict__ start,
+                                                             int chunks, const float *__restrict__ in, int planes, int CW,
+                                                             float *__restrict__ partial) {
+  // A thread owns V consecutive planes (V = 4: 16-byte loads) and has four rows in flight.
+  __shared__ float red[256 * V];
   const int b = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
-  const int tx = threadIdx.x % CW, ty = threadIdx.x / CW, RW = 256 / CW;
-  const int c = blockIdx.y * CW + tx;
+  const int TPR = CW / V;
+  const int tx = threadIdx.x % TPR, ty = threadIdx.x / TPR, RW = 256 / TPR;
+  const int c = blockIdx.y * CW + tx * V;
   const int lo = start[b], hi = start[b + 1];
   const int per = (hi - lo + chunks - 1) / chunks;
   const int t0 = min(hi, lo + chunk * per), t1 = min(hi, t0 + per);
-  float acc = 0.f;
-  if (c < planes)
-    for (int t = t0 + ty; t < t1; t += RW) acc += in[(int64_t)(sched ? sched[t] : t) * planes + c];
-  red[threadIdx.x] = acc;
+  float acc[V];
+#pragma unroll
+  for (int v = 0; v < V; v++) acc[v] = 0.f;
+  if (c < planes) {
+    auto add_row = [&](int t) {
+      const float *src = in + (int64_t)(sched ? sched[t] : t) * planes + c;
+      if constexpr (V == 4) {
+        const float4 x = *reinterpret_cast<const float4 *>(src);
+        acc[0] += x.x, acc[1] += x.y, acc[2] += x.z, acc[3] += x.w;
+      } else {
+        acc[0] += src[0];
+      }
+    };
+    int t = t0 + ty;
+    for (; t + 3 * RW < t1; t += 4 * RW) {
+      add_row(t);
+      add_row(t + RW);
+      add_row(t + 2 * RW);
+      add_row(t + 3 * RW);
+    }
+    for (; t < t1; t += RW) add_row(t);
+  }
+#pragma unroll
+  for (int v = 0; v < V; v++) red[threadIdx.x * V + v] = acc[v];
   __syncthreads();
-  if (ty == 0 && c < planes) {
-    for (int q = 1; q < RW; q++) acc += red[q * CW + tx];
-    partial[(size_t)blockIdx.x * planes + c] = acc;
+  // red[(ty * TPR + tx) * V + v] = plane tx * V + v of row group ty: thread i < CW adds up plane i
+  if (threadIdx.x < CW && blockIdx.y * CW + threadIdx.x < planes) {
+    float sum = 0.f;
+    for (int q = 0; q < RW; q++) sum += red[q * CW + threadIdx.x];
+    partial[(size_t)blockIdx.x * planes + blockIdx.y * CW + threadIdx.x] = sum;
   }
 }
-__global__ void k_active_pool_finish(const float *partial, const int *start, int chunks, int batch, int planes,
-                                     int average, float *out) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= batch * planes) return;
-  const int b = i / planes, c = i - b * planes;
+// grid (sample, tile of 64 planes), 1024 threads: wavefront w adds up its contiguous share of the
+// sample's chunks in order, wavefront 0 then the 16 shares in order (a fixed order).
+__global__ __launch_bounds__(1024) void k_active_pool_finish(const float *__restrict__ partial, const int *__restrict__ start,
+                                                             int chunks, int batch, int planes, int average,
+                                                             float *__restrict__ out) {
+  __shared__ float part[16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.x, c = blockIdx.y * 64 + lane;
+  const int per = (chunks + 15) / 16;
+  const int q0 = min(chunks, wave * per), q1 = min(chunks, q0 + per);
   float s = 0.f;
-  for (int q = 0; q < chunks; q++) s += partial[((size_t)b * chunks + q) * planes + c];
-  const int count = start[b + 1] - start[b];
-  out[i] = (average && count > 0) ? s * (1.0f / (float)count) : s;
+  if (c < planes)
+    for (int q = q0; q < q1; q++) s += partial[((size_t)b * chunks + q) * planes + c];
+  part[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && c < planes) {
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) tot += part[w][lane];
+    const int count = start[b + 1] - start[b];
+    out[(size_t)b * planes + c] = (average && count > 0) ? tot * (1.0f / (float)count) : tot;
+  }
 }
 // CPU/ActivePooling.cpp:26-44,65-83: every row receives its sample's gradient.
 __global__ void k_active_pool_bwd(const int *soa, int dim, int64_t n, int64_t npad, const int *start, int planes,
@@ -424,11 +463,14 @@ void active_pool_forward(Metadata &m, const Level &l, const float *in, float *ou
   int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(1024, l.batch), ceil_div(l.n, (int64_t)256 * l.batch)));
   const int CW = planes <= 16 ? 16 : planes <= 32 ? 32 : 64;
   m.partial.reserve((size_t)l.batch * chunks * planes);
-  k_active_pool_partial<<<dim3((unsigned)(l.batch * chunks), (unsigned)ceil_div(planes, CW)), 256, 0, s>>>(
-      l.sched_ptr(), start, chunks, in, planes, CW, m.partial.p);
+  const dim3 grid((unsigned)(l.batch * chunks), (unsigned)ceil_div(planes, CW));
+  if (planes % 4 == 0 && (uintptr_t)in % 16 == 0)
+    k_active_pool_partial<4><<<grid, 256, 0, s>>>(l.sched_ptr(), start, chunks, in, planes, CW, m.partial.p);
+  else
+    k_active_pool_partial<1><<<grid, 256, 0, s>>>(l.sched_ptr(), start, chunks, in, planes, CW, m.partial.p);
   LAUNCH_CHECK();
-  k_active_pool_finish<<<dim3((unsigned)ceil_div((int64_t)l.batch * planes, TB)), TB, 0, s>>>(m.partial.p, start, chunks,
-                                                                                            l.batch, planes, average, out);
+  k_active_pool_finish<<<dim3((unsigned)l.batch, (unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, start, chunks,
+                                                                                              l.batch, planes, average, out);
   LAUNCH_CHECK();
 }
 void active_pool_backward(Metadata &m, const Level &l, float *d_in, const float *d_out, int planes, int average,
