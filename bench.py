@@ -419,7 +419,7 @@ def config_rows():
     return rows
 
 
-def other_ops(sites, seed):
+def other_ops(sites, seed, backward=True):
     """The rest of the path on the same kind of scene, each op by itself with inputs resident
     in HBM: ms per call (median of 5 timings of 8 calls back to back, HIP events on the launch
     stream) and the algorithmic bytes it has to move, against the 8 TB/s of HBM.  Rulebook builds are timed from the host (they
@@ -530,6 +530,42 @@ def other_ops(sites, seed):
     xc32 = torch.randn((nc, 32), device="cuda", generator=g)
     ms = timed(lambda: md.unPooling(half, sz, two, two, xc32, 0))
     out.append(row("UnPooling 2^3 / stride 2, 32 planes", ms, nc * 32 * 4 + 8 * n + n * 32 * 4))
+
+    if backward:
+        # gradients of the same operators on the same scene (bytes: every array each reads or writes, once)
+        d64, d32 = torch.randn_like(x64), torch.randn_like(x32)
+        dc64, dc32 = torch.randn_like(yc), torch.randn_like(xc32)
+        mp = md.maxPooling(sz, half, two, two, x32, 0)
+        rm, rv = torch.zeros(64, device="cuda"), torch.ones(64, device="cuda")
+        gam, bet = torch.ones(64, device="cuda"), torch.zeros(64, device="cuda")
+        ms = timed(lambda: md.batchNormTrain(x64, rm, rv, gam, bet, 1e-4, 0.9, 0.0))
+        out.append(row("BatchNormReLU training forward, 64 planes", ms, 3 * n * 64 * 4))
+        y_bn, sm, si = md.batchNormTrain(x64, rm, rv, gam, bet, 1e-4, 0.9, 0.0)
+        ms = timed(lambda: md.batchNormBackward(x64, y_bn, d64, sm, si, gam, 0.0, True))
+        out.append(row("BatchNormReLU backward, 64 planes", ms, 7 * n * 64 * 4))
+        ms = timed(lambda: md.convolutionBackward(sz, half, two, two, x32, dc64, w_dn, False))
+        out.append(row("Convolution 2^3 / stride 2 backward, 32 -> 64", ms, 2 * (n * 32 * 4 + nc * 64 * 4) + 16 * n,
+                       gflops=round(4.0 * n * 32 * 64 / (ms * 1e-3) / 1e9, 1)))
+        ms = timed(lambda: md.deconvolutionBackward(half, sz, two, two, yc, d32, w_up, False))
+        out.append(row("Deconvolution 2^3 / stride 2 backward, 64 -> 32", ms, 2 * (nc * 64 * 4 + n * 32 * 4) + 16 * n,
+                       gflops=round(4.0 * n * 64 * 32 / (ms * 1e-3) / 1e9, 1)))
+        ms = timed(lambda: md.networkInNetworkBackward(x64, d32, w_nin, False))
+        out.append(row("NetworkInNetwork backward, 64 -> 32", ms, 2 * n * 64 * 4 + 2 * n * 32 * 4,
+                       gflops=round(4.0 * n * 64 * 32 / (ms * 1e-3) / 1e9, 1)))
+        ms = timed(lambda: md.maxPoolingBackward(sz, half, two, two, x32, mp, dc32, 0))
+        out.append(row("MaxPooling 2^3 / stride 2 backward, 32 planes", ms, 2 * n * 32 * 4 + 8 * n + 2 * nc * 32 * 4))
+        ms = timed(lambda: md.averagePoolingBackward(sz, half, two, two, x32.shape, dc32, 0))
+        out.append(row("AveragePooling 2^3 / stride 2 backward, 32 planes", ms, n * 32 * 4 + 8 * n + nc * 32 * 4))
+        ms = timed(lambda: md.unPoolingBackward(half, sz, two, two, xc32.shape, d32, 0))
+        out.append(row("UnPooling 2^3 / stride 2 backward, 32 planes", ms, nc * 32 * 4 + 8 * n + n * 32 * 4))
+        ms = timed(lambda: md.inputLayerBackward(x3))
+        out.append(row("InputLayer backward, 3 planes", ms, npts * 12 + npts * 4 + n * 12))
+        dpts = torch.randn((npts, 32), device="cuda", generator=g)
+        ms = timed(lambda: md.outputLayerBackward(dpts, n))
+        out.append(row("OutputLayer backward, 32 planes", ms, npts * 32 * 4 + npts * 4 + n * 32 * 4 + n * 8))
+        ms = timed(lambda: md.activePoolingBackward(half, yc.shape, torch.randn((1, 64), device="cuda"), True))
+        out.append(row("ActivePooling backward, 64 planes, %d sites" % nc, ms, nc * 64 * 4))
+        del d64, d32, dc64, dc32, mp, y_bn, dpts
 
     # the other two input routes on the same points: batch-by-length (one sample, every position
     # filled) and the point-at-a-time batch with a third of its points overwriting
@@ -780,7 +816,7 @@ def main():
     if not args.no_configs:
         out["configs"] = config_rows()
     if not args.no_ops:
-        out["other_ops"] = other_ops(args.unet_sites, 5000)
+        out["other_ops"] = other_ops(args.unet_sites, 5000, backward=not args.no_backward)
     if not args.no_unet:
         out["unet"] = unet_scene(args.unet_sites, 5000)
         if not args.no_residual:

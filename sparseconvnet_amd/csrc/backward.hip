@@ -859,6 +859,25 @@ __global__ void k_affine_leaky(const float *in, float *out, int64_t rows, int pl
     out[r * out_stride + c] = y * (y > 0 ? 1.f : leak);
   }
 }
+// The same, four planes per thread (plane count and strides multiples of four, 16-byte aligned).
+__global__ void k_affine_leaky4(const float *__restrict__ in, float *__restrict__ out, int64_t rows, int planes,
+                                int64_t in_stride, int64_t out_stride, const float *__restrict__ coef, float leak) {
+  const int quads = planes >> 2;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = rows * quads, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / quads;
+    const int c = 4 * (int)(i - r * quads);
+    const v4f x = *reinterpret_cast<const v4f *>(in + r * in_stride + c);
+    const v4f sc = *reinterpret_cast<const v4f *>(coef + c), sh = *reinterpret_cast<const v4f *>(coef + planes + c);
+    v4f y = x * sc + sh;
+    y.x *= y.x > 0 ? 1.f : leak;
+    y.y *= y.y > 0 ? 1.f : leak;
+    y.z *= y.z > 0 ? 1.f : leak;
+    y.w *= y.w > 0 ? 1.f : leak;
+    *reinterpret_cast<v4f *>(out + r * out_stride + c) = y;
+  }
+}
 void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t rows, int planes, int64_t in_stride,
                       int64_t out_stride, float *save_mean, float *save_invstd, float *running_mean,
                       float *running_var, const float *gamma, const float *beta, float eps, float momentum,
@@ -875,6 +894,12 @@ void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t ro
                                                                           save_invstd, running_mean, running_var, gamma,
                                                                           beta, eps, momentum, m.prebuf.p);
   LAUNCH_CHECK();
+  if (planes % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const int64_t blocks4 = std::min<int64_t>(ceil_div(rows * (planes / 4), TB), 256 * 64);
+    k_affine_leaky4<<<dim3((unsigned)blocks4), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, m.prebuf.p, leak);
+    LAUNCH_CHECK();
+    return;
+  }
   const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
   k_affine_leaky<<<dim3((unsigned)blocks), TB, 0, s>>>(in, out, rows, planes, in_stride, out_stride, m.prebuf.p, leak);
   LAUNCH_CHECK();
@@ -973,9 +998,61 @@ __global__ void k_pool_bwd(const int *nbr, const int *rowmap, int K, int64_t n, 
     d_in[row * in_stride + col] = acc;
   }
 }
+// The same with nothing dropped and plane counts that are multiples of four: one thread per
+// (position, four planes), 16-byte accesses, and only the taps the position's granule has
+// (gmask; a fine row of a size = stride pooling has one) are looked at.
+template <int MODE>
+__global__ void k_pool_bwd4(const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask,
+                            int K, int64_t n, int64_t npad, const float *__restrict__ in, float *__restrict__ d_in,
+                            const float *__restrict__ out, const float *__restrict__ d_out, int planes) {
+  const int quads = planes >> 2;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = n * quads, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t t = i / quads;
+    const int c = 4 * (int)(i - t * quads);
+    const int64_t row = rowmap ? rowmap[t] : t;
+    v4f x = (v4f){0.f, 0.f, 0.f, 0.f}, acc = x;
+    if (MODE == PB_MAX) x = *reinterpret_cast<const v4f *>(in + row * planes + c);
+    unsigned taps = gmask ? gmask[t >> 4] : (K >= 32 ? 0xFFFFFFFFu : (1u << K) - 1u);
+    while (taps) {
+      const int k = __ffs((int)taps) - 1;
+      taps &= taps - 1u;
+      const int o = nbr[(int64_t)k * npad + t];
+      if (o < 0) continue;
+      const v4f d = *reinterpret_cast<const v4f *>(d_out + (int64_t)o * planes + c);
+      if (MODE == PB_MAX) {
+        const v4f y = *reinterpret_cast<const v4f *>(out + (int64_t)o * planes + c);
+        acc.x += y.x == x.x ? d.x : 0.f;
+        acc.y += y.y == x.y ? d.y : 0.f;
+        acc.z += y.z == x.z ? d.z : 0.f;
+        acc.w += y.w == x.w ? d.w : 0.f;
+      } else if (MODE == PB_AVERAGE) {
+        acc.x += d.x / (float)K, acc.y += d.y / (float)K, acc.z += d.z / (float)K, acc.w += d.w / (float)K;
+      } else {
+        acc += d;
+      }
+    }
+    *reinterpret_cast<v4f *>(d_in + row * planes + c) = acc;
+  }
+}
 void pool_backward(int mode, const Table &t, const float *in, float *d_in, int in_stride, const float *out,
                    const float *d_out, int planes, int drop, hipStream_t s) {
   if (t.n == 0 || in_stride <= 0) return;
+  auto al = [](const float *p) { return p == nullptr || (uintptr_t)p % 16 == 0; };
+  if (drop == 0 && in_stride == planes && planes % 4 == 0 && t.K <= 32 && al(in) && al(d_in) && al(out) && al(d_out)) {
+    const int64_t blocks4 = std::min<int64_t>(ceil_div(t.n * (planes / 4), TB), 256 * 64);
+    const dim3 g4((unsigned)blocks4);
+    const unsigned *gm = t.gmask.p;
+    if (mode == PB_MAX)
+      k_pool_bwd4<PB_MAX><<<g4, TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in, d_in, out, d_out, planes);
+    else if (mode == PB_AVERAGE)
+      k_pool_bwd4<PB_AVERAGE><<<g4, TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in, d_in, out, d_out, planes);
+    else
+      k_pool_bwd4<PB_UNPOOL><<<g4, TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in, d_in, out, d_out, planes);
+    LAUNCH_CHECK();
+    return;
+  }
   const int64_t blocks = std::min<int64_t>(ceil_div(t.n * in_stride, TB), 256 * 64);
   const dim3 g((unsigned)blocks);
   if (mode == PB_MAX)

@@ -175,6 +175,32 @@ __global__ void k_input_fwd(const int *sorted_idx, const int *run_start, const i
     out[i] = acc;
   }
 }
+// The same for plane counts that are multiples of four: one thread per (row, four planes), 16-byte
+// accesses; a row's run and point indices are read once per four planes.
+__global__ void k_input_fwd4(const int *__restrict__ sorted_idx, const int *__restrict__ run_start,
+                             const int *__restrict__ run_len, const unsigned char *__restrict__ overwrite, int64_t n_out,
+                             int mode, const float *__restrict__ in, float *__restrict__ out, int planes, int average) {
+  const int quads = planes >> 2;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = n_out * quads, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / quads;
+    const int c = 4 * (int)(i - r * quads);
+    const int st = run_start[r], len = run_len[r];
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (mode == 1 || mode == 2 || mode == 5) {
+      const float4 x = *reinterpret_cast<const float4 *>(in + (int64_t)listed_point(sorted_idx, st, len, mode, overwrite) * planes + c);
+      acc.x += x.x, acc.y += x.y, acc.z += x.z, acc.w += x.w;
+    } else {
+      const float mult = (average && len > 0) ? 1.0f / (float)len : 1.0f;
+      for (int q = 0; q < len; q++) {
+        const float4 x = *reinterpret_cast<const float4 *>(in + (int64_t)sorted_idx[st + q] * planes + c);
+        acc.x += mult * x.x, acc.y += mult * x.y, acc.z += mult * x.z, acc.w += mult * x.w;
+      }
+    }
+    *reinterpret_cast<float4 *>(out + r * planes + c) = acc;
+  }
+}
 // The same for one to four planes (coordinates-and-colour inputs): one thread per row, so that
 // a row's run and point indices are read once instead of once per plane.
 template <int P>
@@ -225,6 +251,13 @@ void input_forward(const InputRules &r, const float *in, float *out, int planes,
     LAUNCH_CHECK();
     return;
   }
+  if (planes % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const int64_t blocks4 = std::min<int64_t>(ceil_div(r.n_out * (planes / 4), TB), 256 * 64);
+    k_input_fwd4<<<dim3((unsigned)blocks4), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p, r.n_out,
+                                                        r.mode, in, out, planes, average);
+    LAUNCH_CHECK();
+    return;
+  }
   int64_t total = r.n_out * planes;
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p,
@@ -242,6 +275,13 @@ void output_backward(const InputRules &r, float *d_in, const float *d_out, int p
     return;
   }
   if (r.n_out == 0) return;
+  if (planes % 4 == 0 && (uintptr_t)d_out % 16 == 0 && (uintptr_t)d_in % 16 == 0) {
+    const int64_t blocks4 = std::min<int64_t>(ceil_div(r.n_out * (planes / 4), TB), 256 * 64);
+    k_input_fwd4<<<dim3((unsigned)blocks4), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p, r.n_out,
+                                                        r.mode, d_out, d_in, planes, 0);
+    LAUNCH_CHECK();
+    return;
+  }
   int64_t total = r.n_out * planes;
   int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
   k_input_fwd<<<dim3((unsigned)blocks), TB, 0, s>>>(r.sorted_idx.p, r.run_start.p, r.run_len.p, r.overwrite.p,
