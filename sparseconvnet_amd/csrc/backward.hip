@@ -460,7 +460,10 @@ constexpr int DWV_T = 64;
 struct TapShares {
   unsigned short n[32];  // K <= 32: shares of tap k that have work; the rest only write zeros
 };
-template <bool VEC4>
+// NA, NB: channels per lane on the a- and the b-side (4, or 2 for a side of at most 32 channels: a
+// tile is 16 NA x 16 NB channels, so that a narrow side does not fill half its MFMAs with zeros).
+// VEC: a lane's channels come as one 16- or 8-byte load (plane counts multiples of NA / NB, arrays aligned).
+template <bool VEC, int NA, int NB>
 __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nbr, const int *__restrict__ rowmap,
                                                       const unsigned *__restrict__ gmask, int K, int64_t n, int64_t npad,
                                                       const float *__restrict__ a, int n_a, unsigned a_bytes,
@@ -472,17 +475,18 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
   // barriers below).  A layer of fewer than four tiles (at most 64 channels on one side and 128 on
   // the other) would leave wavefronts idle that way: there the workgroup's four wavefronts are
   // four (share, tile) pairs in a row, each on its own.
-  const int tiles_a = (n_a + DWV_T - 1) / DWV_T, tiles_b = (n_b + DWV_T - 1) / DWV_T;
+  constexpr int TA = 16 * NA, TB_ = 16 * NB;  // tile: TA channels of a by TB_ channels of b
+  const int tiles_a = (n_a + TA - 1) / TA, tiles_b = (n_b + TB_ - 1) / TB_;
   const bool single = tiles_a * tiles_b < 4;
   const int slot = blockIdx.y * 4 + wave;
   const int share = single ? slot / (tiles_a * tiles_b) : blockIdx.y;
   const int tile = slot % (tiles_a * tiles_b);
-  const int mt_o = (n_b + 2 * DWV_T - 1) / (2 * DWV_T);
+  const int mt_o = (n_b + 2 * TB_ - 1) / (2 * TB_);
   const int ct = single ? tile / tiles_b : 2 * (blockIdx.z / mt_o) + (wave >> 1);
   const int ot = single ? tile % tiles_b : 2 * (blockIdx.z % mt_o) + (wave & 1);
   if (share >= shares) return;  // (single only: its wavefronts meet at no barrier)
   const int r16 = lane & 15, g = lane >> 4;
-  const int ca = ct * DWV_T + 4 * r16, cb = ot * DWV_T + 4 * r16;
+  const int ca = ct * TA + NA * r16, cb = ot * TB_ + NB * r16;
   const unsigned nowhere = 0x80000000u;  // offsets from here on read zeros
   const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a), 0, (int)a_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(b), 0, (int)b_bytes, 0x00020000);
@@ -491,28 +495,34 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
   const __amdgpu_buffer_rsrc_t map_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(rowmap ? rowmap : nbr), 0, (int)((unsigned)npad * 4u), 0x00020000);
   const unsigned a_row_bytes = (unsigned)n_a * 4u, b_row_bytes = (unsigned)n_b * 4u;
-  // four channels of row j from column c0 on (negative row, or columns past the last: zeros)
-  auto quad_of = [&](const __amdgpu_buffer_rsrc_t &rsrc, int j, unsigned row_bytes, int c0, int width) {
+  // N channels of row j from column c0 on (negative row, or columns past the last: zeros)
+  auto comps_of = [&](auto n_tag, const __amdgpu_buffer_rsrc_t &rsrc, int j, unsigned row_bytes, int c0, int width,
+                      float *e) {
+    constexpr int N = decltype(n_tag)::value;
     const unsigned row = (unsigned)j * row_bytes;
-    if (VEC4) {
+    if constexpr (VEC && N == 4) {
       const unsigned off = (j < 0 || c0 >= width) ? nowhere : row + (unsigned)c0 * 4u;
-      return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
-    }
-    float e[4];
+      const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
+      e[0] = v.x, e[1] = v.y, e[2] = v.z, e[3] = v.w;
+    } else if constexpr (VEC && N == 2) {
+      const unsigned off = (j < 0 || c0 >= width) ? nowhere : row + (unsigned)c0 * 4u;
+      const v2f v = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0));
+      e[0] = v.x, e[1] = v.y;
+    } else {
 #pragma unroll
-    for (int x = 0; x < 4; x++) {
-      const unsigned off = (j < 0 || c0 + x >= width) ? nowhere : row + (unsigned)(c0 + x) * 4u;
-      e[x] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0));
+      for (int x = 0; x < N; x++) {
+        const unsigned off = (j < 0 || c0 + x >= width) ? nowhere : row + (unsigned)(c0 + x) * 4u;
+        e[x] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0));
+      }
     }
-    return (v4f){e[0], e[1], e[2], e[3]};
   };
-  v4f acc[4][4];
+  v4f acc[NA][NB];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < NA; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NB; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
   const int n_granules = (int)((n + 15) >> 4), n32 = (int)n;
-  const bool idle = ct * DWV_T >= n_a || ot * DWV_T >= n_b;  // a tile past the last channel: only keeps the barrier count
+  const bool idle = ct * TA >= n_a || ot * TB_ >= n_b;  // a tile past the last channel: only keeps the barrier count
   const int mine = K <= 32 ? (int)tap_shares.n[k] : shares;    // shares of this tap that have work
   // This share's granules: blocks share, share + mine, ... of DT_BLOCK granules, those with the tap.
   auto next_granule = [&](int gi) {  // the one after gi (n_granules: none)
@@ -524,7 +534,7 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
     }
   };
   struct Quads {
-    v4f a[4], b[4];
+    float a[4][NA], b[4][NB];
   };
   int4 jq, rq;  // neighbour rows and rows of b of the lane's four positions, for the granule whose rows are requested next
   auto load_indices = [&](int gi) {
@@ -539,17 +549,17 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) {
       const bool live = gi < n_granules && gi * 16 + 4 * g + kk < n32;
-      q.a[kk] = quad_of(a_rsrc, live ? j[kk] : -1, a_row_bytes, ca, n_a);
-      q.b[kk] = quad_of(b_rsrc, live ? r[kk] : -1, b_row_bytes, cb, n_b);
+      comps_of(std::integral_constant<int, NA>(), a_rsrc, live ? j[kk] : -1, a_row_bytes, ca, n_a, q.a[kk]);
+      comps_of(std::integral_constant<int, NB>(), b_rsrc, live ? r[kk] : -1, b_row_bytes, cb, n_b, q.b[kk]);
     }
   };
   auto multiply = [&](const Quads &q) {
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+      for (int i = 0; i < NA; i++)
 #pragma unroll
-        for (int jx = 0; jx < 4; jx++)
+        for (int jx = 0; jx < NB; jx++)
           acc[i][jx] = __builtin_amdgcn_mfma_f32_16x16x4f32(q.a[kk][i], q.b[kk][jx], acc[i][jx], 0, 0, 0);
   };
   if (share < mine) {  // uniform over the workgroup (over the wavefront when single)
@@ -583,16 +593,16 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
       g1 = g3;
     }
   }
-  // acc[i][jx][r] = dW[k][ct*64 + 4 (4 g + r) + i][ot*64 + 4 r16 + jx] of this share (zeros for a share without work)
+  // acc[i][jx][r] = dW[k][ct*TA + NA (4 g + r) + i][ot*TB_ + NB r16 + jx] of this share (zeros for a share without work)
   float *pk = partial + ((size_t)share * K + k) * (size_t)n_a * n_b;
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < NA; i++)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      const int c = ct * DWV_T + 4 * (4 * g + r) + i;
+      const int c = ct * TA + NA * (4 * g + r) + i;
       if (c >= n_a) continue;
 #pragma unroll
-      for (int jx = 0; jx < 4; jx++)
+      for (int jx = 0; jx < NB; jx++)
         if (cb + jx < n_b) pk[(size_t)c * n_b + cb + jx] = acc[i][jx][r];
     }
 }
@@ -659,9 +669,12 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
   if (t.npad % 4 == 0 && a_rows * n_a * 4 < ((int64_t)1 << 31) && b_rows * n_b * 4 < ((int64_t)1 << 31) &&
       (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31) && t.K <= 65535) {
     // wider layers: a wavefront per (tap, 64 x 64 tile, share of the positions)
-    const int tiles64 = (int)(ceil_div(n_a, DWV_T) * ceil_div(n_b, DWV_T));
+    // a side of at most 32 channels gives a lane two channels of it instead of four: tiles of 32 there
+    const int na = n_a <= 32 ? 2 : 4, nb = n_b <= 32 ? 2 : 4;
+    const int tile_a = 16 * na, tile_b = 16 * nb;
+    const int tiles64 = (int)(ceil_div(n_a, tile_a) * ceil_div(n_b, tile_b));
     const bool single = tiles64 < 4;  // fewer than four tiles: a workgroup's wavefronts are (share, tile) pairs
-    const int tiles = single ? 1 : (int)(ceil_div(n_a, 2 * DWV_T) * ceil_div(n_b, 2 * DWV_T));  // blocks of 2 x 2 tiles
+    const int tiles = single ? 1 : (int)(ceil_div(n_a, 2 * tile_a) * ceil_div(n_b, 2 * tile_b));  // blocks of 2 x 2 tiles
     // Shares of the positions per tap in proportion to the tap's rules (the table's counts; the
     // first call on a table fetches them), about three workgroups per compute unit in all;
     // partial sums bounded to 256 MB, at least a block of granules per share.
@@ -686,14 +699,24 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
       m.partial.reserve((size_t)shares * per_chunk);
       const dim3 grid((unsigned)t.K, (unsigned)(single ? ceil_div(shares * tiles64, 4) : shares), (unsigned)tiles);
       const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
-      if (vec4)
-        k_conv_dw_wave<true><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,
-                                                  (unsigned)(a_rows * n_a * 4), b, n_b, (unsigned)(b_rows * n_b * 4),
-                                                  (int)shares, ts, m.partial.p);
-      else
-        k_conv_dw_wave<false><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,
-                                                   (unsigned)(a_rows * n_a * 4), b, n_b, (unsigned)(b_rows * n_b * 4),
-                                                   (int)shares, ts, m.partial.p);
+      // one load per lane and side when the plane counts are multiples of the lane's channels and the arrays aligned
+      const bool vec = n_a % na == 0 && n_b % nb == 0 && (uintptr_t)a % (4 * na) == 0 && (uintptr_t)b % (4 * nb) == 0;
+#define SCN_DWV(V, A, B)                                                                                              \
+  k_conv_dw_wave<V, A, B><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,                 \
+                                               (unsigned)(a_rows * n_a * 4), b, n_b, (unsigned)(b_rows * n_b * 4),    \
+                                               (int)shares, ts, m.partial.p)
+      if (vec) {
+        if (na == 4 && nb == 4) SCN_DWV(true, 4, 4);
+        else if (na == 4) SCN_DWV(true, 4, 2);
+        else if (nb == 4) SCN_DWV(true, 2, 4);
+        else SCN_DWV(true, 2, 2);
+      } else {
+        if (na == 4 && nb == 4) SCN_DWV(false, 4, 4);
+        else if (na == 4) SCN_DWV(false, 4, 2);
+        else if (nb == 4) SCN_DWV(false, 2, 4);
+        else SCN_DWV(false, 2, 2);
+      }
+#undef SCN_DWV
       LAUNCH_CHECK();
       k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)shares, per_chunk,
                                                                                       per_chunk, dw);
