@@ -956,6 +956,35 @@ __global__ void k_bn_bwd_apply(const float *in, float *d_in, const float *out, c
         (d - coef[c] - (in[r * in_stride + c] - save_mean[c]) * coef[planes + c]) * coef[2 * planes + c];
   }
 }
+// The same, four planes per thread (plane count and strides multiples of four, arrays 16-byte aligned).
+__global__ void k_bn_bwd_apply4(const float *__restrict__ in, float *__restrict__ d_in, const float *__restrict__ out,
+                                const float *__restrict__ d_out, int64_t rows, int planes, int64_t in_stride,
+                                int64_t out_stride, const float *__restrict__ save_mean, const float *__restrict__ coef,
+                                float leak) {
+  const int quads = planes >> 2;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = rows * quads, step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const int64_t r = i / quads;
+    const int c = 4 * (int)(i - r * quads);
+    const v4f d = *reinterpret_cast<const v4f *>(d_out + r * out_stride + c);
+    const v4f y = *reinterpret_cast<const v4f *>(out + r * out_stride + c);
+    const v4f x = *reinterpret_cast<const v4f *>(in + r * in_stride + c);
+    const v4f mu = *reinterpret_cast<const v4f *>(save_mean + c), c0 = *reinterpret_cast<const v4f *>(coef + c),
+              c1 = *reinterpret_cast<const v4f *>(coef + planes + c), c2 = *reinterpret_cast<const v4f *>(coef + 2 * planes + c);
+    v4f g;
+    g.x = d.x * (y.x > 0.f ? 1.f : leak);
+    g.y = d.y * (y.y > 0.f ? 1.f : leak);
+    g.z = d.z * (y.z > 0.f ? 1.f : leak);
+    g.w = d.w * (y.w > 0.f ? 1.f : leak);
+    v4f o;
+    o.x = (g.x - c0.x - (x.x - mu.x) * c1.x) * c2.x;
+    o.y = (g.y - c0.y - (x.y - mu.y) * c1.y) * c2.y;
+    o.z = (g.z - c0.z - (x.z - mu.z) * c1.z) * c2.z;
+    o.w = (g.w - c0.w - (x.w - mu.w) * c1.w) * c2.w;
+    *reinterpret_cast<v4f *>(d_in + r * in_stride + c) = o;
+  }
+}
 // CPU/BatchNormalization.cpp:63-107.  d_out is not modified (the reference scales it in place).
 void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *out, const float *d_out, int64_t rows,
                  int planes, int64_t in_stride, int64_t out_stride, const float *save_mean, const float *save_invstd,
@@ -976,6 +1005,15 @@ void bn_backward(Metadata *scratch, const float *in, float *d_in, const float *o
   k_bn_bwd_finish<<<dim3((unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, p.blocks, planes, rows, save_invstd,
                                                                         gamma, d_gamma, d_beta, m.prebuf.p);
   LAUNCH_CHECK();
+  auto al = [](const float *p) { return (uintptr_t)p % 16 == 0; };
+  if (planes % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 && al(in) && al(d_in) && al(out) && al(d_out) &&
+      al(save_mean)) {
+    const int64_t blocks4 = std::min<int64_t>(ceil_div(rows * (planes / 4), TB), 256 * 64);
+    k_bn_bwd_apply4<<<dim3((unsigned)blocks4), TB, 0, s>>>(in, d_in, out, d_out, rows, planes, in_stride, out_stride,
+                                                           save_mean, m.prebuf.p, leak);
+    LAUNCH_CHECK();
+    return;
+  }
   const int64_t blocks = std::min<int64_t>(ceil_div(rows * planes, TB), 256 * 64);
   k_bn_bwd_apply<<<dim3((unsigned)blocks), TB, 0, s>>>(in, d_in, out, d_out, rows, planes, in_stride, out_stride, save_mean,
                                                        m.prebuf.p, leak);
