@@ -99,6 +99,13 @@ def test_active_pooling(make, dim):
     checks.check_active_pooling(make, dim, seed=70 + dim)
 
 
+@pytest.mark.parametrize("planes,n", [(96, 3000), (64, 20000), (7, 5000)])
+def test_active_pooling_wide(make, planes, n):
+    """More planes than one 64-plane tile of the kernels, plane counts that do and do not allow
+    16-byte loads, and samples of thousands of sites (several chunks of rows per sample)."""
+    checks.check_active_pooling(make, 3, seed=90 + planes, spatial=40, n=n, batch=3, C=planes)
+
+
 def test_level_replacement(make):
     checks.check_level_replacement(make)
 
