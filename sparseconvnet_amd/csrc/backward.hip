@@ -145,17 +145,18 @@ static ColsumPlan colsum_plan(int64_t rows, int planes) {
   p.blocks = (int)ceil_div(rows, p.rows_per_block);
   return p;
 }
-// out[i] = sum over blocks b of partial[b * stride + i], i < count.  A workgroup of 16 wavefronts
-// takes 64 consecutive outputs: wavefront w adds up its contiguous share of the blocks in order,
-// wavefront 0 then adds the 16 shares in order (a fixed order: the result is the same on every
-// run).  ACC is the accumulator type, OUT the type the sums are written in.
+// out[i] = sum over blocks b of partial[b * stride + i], i < count.  A workgroup of 1, 4 or 16
+// wavefronts (blockDim.x / 64) takes 64 consecutive outputs: wavefront w adds up its contiguous
+// share of the blocks in order, wavefront 0 then adds the shares in order (a fixed order: the
+// result is the same on every run).  ACC is the accumulator type, OUT the type the sums are written in.
 template <typename ACC, typename OUT>
 __global__ __launch_bounds__(1024) void k_sum_blocks(const float *__restrict__ partial, int blocks, int64_t stride,
                                                      int64_t count, OUT *__restrict__ out) {
   __shared__ ACC part[16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t i = (int64_t)blockIdx.x * 64 + lane;
-  const int per = (blocks + 15) / 16;
+  const int waves = blockDim.x >> 6;
+  const int per = (blocks + waves - 1) / waves;
   const int b0 = min(blocks, wave * per), b1 = min(blocks, b0 + per);
   ACC s = 0;
   if (i < count)
@@ -164,11 +165,12 @@ __global__ __launch_bounds__(1024) void k_sum_blocks(const float *__restrict__ p
   __syncthreads();
   if (wave == 0 && i < count) {
     ACC tot = 0;
-#pragma unroll
-    for (int w = 0; w < 16; w++) tot += part[w][lane];
+    for (int w = 0; w < waves; w++) tot += part[w][lane];
     out[i] = (OUT)tot;
   }
 }
+// Wavefronts per workgroup of k_sum_blocks: every wavefront gets at least four blocks to add.
+static inline unsigned sum_threads(int64_t blocks) { return blocks >= 64 ? 1024 : blocks >= 16 ? 256 : 64; }
 // The two column sums of a batch-normalisation pass, in double, for the 64 columns of workgroup
 // blockIdx.x (1024 threads): partial[b][q][c] summed over the row blocks b in the fixed order of
 // k_sum_blocks.  Every thread of wavefront 0 returns with the sums of column blockIdx.x * 64 + lane.
@@ -662,7 +664,7 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
                                                         (unsigned)(a_rows * n_a * 4), b, n_b,
                                                        (unsigned)(b_rows * n_b * 4), m.partial.p);
     LAUNCH_CHECK();
-    k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
+    k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), sum_threads(chunks), 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
     LAUNCH_CHECK();
     return;
   }
@@ -718,7 +720,7 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
       }
 #undef SCN_DWV
       LAUNCH_CHECK();
-      k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)shares, per_chunk,
+      k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), sum_threads(shares), 0, s>>>(m.partial.p, (int)shares, per_chunk,
                                                                                       per_chunk, dw);
       LAUNCH_CHECK();
       return;
@@ -742,7 +744,7 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     k_conv_dw<false><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a, b, n_b, chunk_len,
                                           m.partial.p);
   LAUNCH_CHECK();
-  k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), 1024, 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
+  k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), sum_threads(chunks), 0, s>>>(m.partial.p, (int)chunks, per_chunk, per_chunk, dw);
   LAUNCH_CHECK();
 }
 
