@@ -159,8 +159,10 @@ __global__ __launch_bounds__(1024) void k_sum_blocks(const float *__restrict__ p
   const int per = (blocks + waves - 1) / waves;
   const int b0 = min(blocks, wave * per), b1 = min(blocks, b0 + per);
   ACC s = 0;
-  if (i < count)
+  if (i < count) {
+#pragma unroll 4
     for (int b = b0; b < b1; b++) s += (ACC)partial[(size_t)b * stride + i];
+  }
   part[wave][lane] = s;
   __syncthreads();
   if (wave == 0 && i < count) {
@@ -182,6 +184,7 @@ __device__ inline void pair_sums64(const float *__restrict__ partial, int blocks
   const int b0 = min(blocks, wave * per), b1 = min(blocks, b0 + per);
   double a = 0, b = 0;
   if (c < planes)
+#pragma unroll 4
     for (int i = b0; i < b1; i++) {
       a += (double)partial[(size_t)i * 2 * planes + c];
       b += (double)partial[(size_t)i * 2 * planes + planes + c];
