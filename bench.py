@@ -730,14 +730,26 @@ def main():
     ms_per_step = wall / args.steps * 1e3
     per_pair_ms = [float(np.mean([ev[s][i][0].elapsed_time(ev[s][i][1]) for s in range(args.steps)]))
                    for i in range(len(work))]
+    # every pair once more on its own, back to back: a short launch right behind the long 256->256 one of
+    # the step above runs slower than among launches of its own kind
+    alone_ms = []
+    for wk in work:
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        conv(*wk)
+        a.record()
+        for _ in range(args.steps):
+            conv(*wk)
+        b.record()
+        torch.cuda.synchronize()
+        alone_ms.append(a.elapsed_time(b) / args.steps)
     total_flops = sum(2.0 * R * cin * cout for cin, cout in pairs)
     value = total_flops / (ms_per_step * 1e-3) / 1e9
 
     default_workload = args.sites == 1000000 and args.seed == 3000 and args.order == "shuffled"
     traffic = measured_traffic() if default_workload else {}
     sweep = []
-    for (cin, cout), ms in zip(pairs, per_pair_ms):
-        sweep.append({"nIn": cin, "nOut": cout, "ms": round(ms, 4),
+    for (cin, cout), ms, alone in zip(pairs, per_pair_ms, alone_ms):
+        sweep.append({"nIn": cin, "nOut": cout, "ms": round(ms, 4), "ms_back_to_back": round(alone, 4),
                       "gflops": round(2.0 * R * cin * cout / (ms * 1e-3) / 1e9, 1),
                       "sites_per_s": round(n / (ms * 1e-3)),
                       "roofline": roofline_for(cin, cout, R, n, 27, ms, traffic.get((cin, cout)))})
