@@ -61,7 +61,7 @@ template <int NIN> __device__ inline float plane_of(const typename RowOf<NIN>::t
 }
 
 template <int NIN, int NCB>
-__global__ __launch_bounds__(256) void k_conv_first(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))) void k_conv_first(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
     int64_t n, int64_t npad, const float *__restrict__ in, float *__restrict__ out,
     const float *__restrict__ w, const float *__restrict__ bias, CoefJob bn, float leak, int n_out, int n_sets,
