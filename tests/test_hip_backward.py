@@ -105,6 +105,51 @@ def test_weight_gradient_over_many_blocks(oracle_built, cin, cout):
         checks.assert_close(a, b, "submanifold " + what)
 
 
+def test_full_size_gradient_identities():
+    """The bench scene at its full size (1,000,000 sites), where the oracle takes too long: the
+    convolution is bilinear in (input, weights), so for any d_y
+        <d_y, conv(x, w)> = <d_input, x> = <d_weight, w>   and   d_bias = column sums of d_y.
+    A dropped tap, a share of positions counted twice or not at all, or a transposed operand breaks
+    one of the equalities.  Inner products in float64 on the host; 2e-4 relative (fp32 sums of
+    10^7..10^9 products on the GPU side)."""
+    from hip_path import HipPath
+    g = HipPath(3)
+    coords = synthetic.room_scene(seed=3000, target=1000000, spatial=4096)
+    n = len(coords)
+    assert g.input_layer(4096, coords, 0, 0) == n
+    rng = np.random.default_rng(31)
+    for cin, cout in ((3, 32), (32, 32), (64, 64), (128, 128)):
+        x = rng.normal(size=(n, cin)).astype(np.float32)
+        d_y = rng.normal(size=(n, cout)).astype(np.float32)
+        w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
+        y, _ = g.subm_conv(4096, 3, x, w)
+        d_x, d_w, d_b = g.subm_conv_bwd(4096, 3, x, d_y, w, True)
+        dot = lambda a, b: float(np.einsum("ij,ij->", a.reshape(len(a), -1), b.reshape(len(b), -1), dtype=np.float64))
+        ref = dot(d_y, y)
+        scale = np.sqrt(dot(d_y, d_y) * dot(y, y))  # the size a sum of that many products could have
+        assert abs(dot(d_x, x) - ref) <= 2e-4 * scale, (cin, cout, "d_input", dot(d_x, x), ref)
+        assert abs(dot(d_w, w) - ref) <= 2e-4 * scale, (cin, cout, "d_weight", dot(d_w, w), ref)
+        checks.assert_close(d_b, d_y.sum(0, dtype=np.float64).astype(np.float32), "d_bias at 1 M sites")
+        # the weight gradient of one tap by hand: centre tap pairs every site with itself
+        want = (x.astype(np.float64).T @ d_y.astype(np.float64)).astype(np.float32)
+        checks.assert_close(d_w[13, 0], want, "centre-tap d_weight at 1 M sites")
+    # the same identities for the 2^3 / stride-2 convolution and its transpose between 4096^3 and 2048^3
+    g.strided_rules(4096, 2048, 2, 2)
+    n_c = len(g.spatial_locations(2048))
+    for kind, fwd, bwd, rows_in, rows_out in (("strided", g.conv, g.conv_bwd, n, n_c), ("transposed", g.deconv, g.deconv_bwd, n_c, n)):
+        sizes = (4096, 2048, 2, 2) if kind == "strided" else (2048, 4096, 2, 2)
+        x = rng.normal(size=(rows_in, 32)).astype(np.float32)
+        d_y = rng.normal(size=(rows_out, 64)).astype(np.float32)
+        w = (rng.normal(size=(8, 1, 32, 64)) * 0.1).astype(np.float32)
+        y, _ = fwd(*sizes, x, w)
+        d_x, d_w, d_b = bwd(*sizes, x, d_y, w, True)
+        ref = dot(d_y, y)
+        scale = np.sqrt(dot(d_y, d_y) * dot(y, y))
+        assert abs(dot(d_x, x) - ref) <= 2e-4 * scale, (kind, "d_input", dot(d_x, x), ref)
+        assert abs(dot(d_w, w) - ref) <= 2e-4 * scale, (kind, "d_weight", dot(d_w, w), ref)
+        checks.assert_close(d_b, d_y.sum(0, dtype=np.float64).astype(np.float32), kind + " d_bias at 1 M sites")
+
+
 def test_pooling_and_nin_gradients_vs_oracle(oracle_built):
     from hip_path import HipPath
     g, o = HipPath(3), cpu_path.CpuPath(3, "oracle")
