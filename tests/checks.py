@@ -696,6 +696,9 @@ def check_bn_train(make, seed, n=257, C=13):
         assert_close(rm2, trm.numpy(), "running mean")
         assert_close(rv2, trv.numpy(), "running variance")
         d_out = rng.normal(size=(n, C)).astype(np.float32)
+        # an output within rounding of zero may be on either side of the leaky ReLU's kink in fp32:
+        # such values get no gradient, so that their side does not matter
+        d_out[np.abs(y.detach().numpy()) < 1e-5] = 0
         d_in, d_g, d_b = p.bn_bwd(x, out, d_out, sm, si, g, leak, affine)
         gx, gg, gb = _grads((y * _t64(d_out)).sum(), xt, gt, bt)
         assert_close(d_in, gx, "batch norm d_input")

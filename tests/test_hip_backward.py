@@ -35,6 +35,12 @@ def test_bn_train(make):
     checks.check_bn_train(make, seed=51, n=5000, C=96)
 
 
+def test_bn_train_full_size(make):
+    """1,000,000 rows: every workgroup of the column-sum passes has work, the partial sums go
+    through all sixteen wavefronts of the finishing kernels."""
+    checks.check_bn_train(make, seed=52, n=1000000, C=32)
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
 def test_io_backward(make, mode):
     checks.check_io_backward(make, 3, mode, seed=60 + mode)
