@@ -156,6 +156,61 @@ def test_full_size_gradient_identities():
         checks.assert_close(d_b, d_y.sum(0, dtype=np.float64).astype(np.float32), kind + " d_bias at 1 M sites")
 
 
+def test_full_size_linear_ops_are_adjoint():
+    """The bench's U-Net scene (1,300,000 points, 1,000,000 sites): every linear operator's backward
+    pass is its transpose, <d_out, A f> = <A^T d_out, f> - input layer (mean of the points of a
+    site), output layer, average pooling, unpooling, ActivePooling, sparse to dense at a coarse
+    level; max pooling hands every gradient to the row that held the maximum, so the gradients
+    of the outputs above zero all arrive and nothing else does."""
+    from hip_path import HipPath
+    g = HipPath(3)
+    coords = synthetic.room_scene(seed=5000, target=1000000, spatial=4096, duplicate_fraction=0.3)
+    n_sites = g.input_layer(4096, coords, 0, 4)
+    assert len(coords) > 1200000 and 900000 < n_sites < len(coords)
+    rng = np.random.default_rng(53)
+    dot = lambda a, b: float(np.einsum("i,i->", a.reshape(-1), b.reshape(-1), dtype=np.float64))
+
+    def adjoint(what, f, y, d_out, d_in):
+        ref, got = dot(d_out, y), dot(d_in, f)
+        assert abs(got - ref) <= 2e-4 * np.sqrt(dot(d_out, d_out) * dot(y, y)), (what, got, ref)
+
+    f = rng.normal(size=(len(coords), 8)).astype(np.float32)
+    x = g.input_fwd(f)
+    assert x.shape == (n_sites, 8)
+    d = rng.normal(size=x.shape).astype(np.float32)
+    adjoint("input layer", f, x, d, g.input_bwd(d))
+    back = g.output_fwd(x)
+    d = rng.normal(size=back.shape).astype(np.float32)
+    adjoint("output layer", x, back, d, g.output_bwd(d))
+    g.strided_rules(4096, 2047, 3, 2)
+    n_c = g.nactive(2047)
+    avg = g.avgpool(4096, 2047, 3, 2, x)
+    d = rng.normal(size=avg.shape).astype(np.float32)
+    adjoint("average pooling", x, avg, d, g.avgpool_bwd(4096, 2047, 3, 2, 8, d))
+    c = rng.normal(size=(n_c, 8)).astype(np.float32)
+    up = g.unpool(2047, 4096, 3, 2, c)
+    d = rng.normal(size=up.shape).astype(np.float32)
+    adjoint("unpooling", c, up, d, g.unpool_bwd(2047, 4096, 3, 2, 8, d))
+    mp = g.maxpool(4096, 2047, 3, 2, x)
+    d = rng.normal(size=mp.shape).astype(np.float32)
+    d_x = g.maxpool_bwd(4096, 2047, 3, 2, x, mp, d)
+    want = np.where(mp > 0, d, 0).sum(0, dtype=np.float64)
+    checks.assert_close(d_x.sum(0, dtype=np.float64), want, "max pooling: gradients that arrive")
+    assert ((d_x != 0) <= (x > 0)).all()  # only a positive input can have been a maximum above zero
+    ap = g.active_pooling(4096, x, True)
+    d = rng.normal(size=ap.shape).astype(np.float32)
+    adjoint("ActivePooling", x, ap, d, g.active_pooling_bwd(4096, d, True))
+    # sparse to dense at 64^3 (dense blocks of 4096^3 do not exist): five more halvings
+    size = 2047
+    while size > 63:
+        g.strided_rules(size, size // 2, 3, 2)
+        size //= 2
+    c = rng.normal(size=(g.nactive(size), 8)).astype(np.float32)
+    dense = g.s2d(size, c)
+    d = rng.normal(size=dense.shape).astype(np.float32)
+    adjoint("sparse to dense", c, dense, d, g.s2d_bwd(size, d))
+
+
 def test_pooling_and_nin_gradients_vs_oracle(oracle_built):
     from hip_path import HipPath
     g, o = HipPath(3), cpu_path.CpuPath(3, "oracle")
