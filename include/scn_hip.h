@@ -207,7 +207,8 @@ int scn_subm_conv_fwd(scn_metadata *md, const int64_t *spatial, const int64_t *f
  * static 16 MiB device array that every GPU the library runs on holds until the process ends.
  * Limits: the rulebook of (spatial, filter) must exist already (scn_md_submanifold_rules, or an
  * earlier convolution); the packed weights, filter volume x ceil(n_in/16)*16 x ceil(n_out/16)*16
- * x 4 bytes, must fit in 8 MiB (27 taps of 256 x 256 do), else the call fails with a message.
+ * x 4 bytes, must fit in 8 MiB (27 taps of 256 x 256 do), and n_out may be at most 256 (wider
+ * layers would need an allocated copy of their weights), else the call fails with a message.
  * All such calls on one GPU share the array: calls that overlap on one GPU (two streams, two
  * threads) race; calls on one stream are ordered.  The multiply-add count is added to the
  * handle's running total (scn_md_take_macs). */

@@ -16,16 +16,22 @@ def sources():
     return sorted(glob.glob(os.path.join(HERE, "csrc", "*.hip")))
 
 
-def build_library(verbose=False):
+def build_library(verbose=False, incremental=False):
+    """incremental: translation units whose object file is newer than the source and every header
+    are not compiled again (for work on one kernel file; the default compiles everything)."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     srcs = sources()
     objs = []
     procs = []
     objdir = os.path.join(HERE, "csrc", "build")
     os.makedirs(objdir, exist_ok=True)
+    headers = glob.glob(os.path.join(HERE, "csrc", "*.h")) + glob.glob(os.path.join(HERE, "..", "include", "*.h"))
+    newest_header = max(os.path.getmtime(h) for h in headers)
     for s in srcs:  # one hipcc per translation unit, in parallel
         o = os.path.join(objdir, os.path.basename(s)[:-4] + ".o")
         objs.append(o)
+        if incremental and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(s), newest_header):
+            continue
         cmd = [hipcc] + [f for f in FLAGS if f != "-shared"] + ["-c", s, "-o", o]
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
     for cmd, p in procs:
@@ -40,4 +46,5 @@ def build_library(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build_library())
+    import sys
+    print(build_library(incremental="--incremental" in sys.argv))

@@ -11,7 +11,8 @@
 //     filter box mostly re-use the entry of the previous tap;
 //   * rules are stored output-stationary as a table nbr[tap][position] instead of
 //     per-tap pair lists; pair lists are produced on demand by ballot/prefix compaction.
-#include <hipcub/hipcub.hpp>
+#include <cstring>
+
 #include <rocprim/rocprim.hpp>
 
 #include <algorithm>
@@ -164,10 +165,10 @@ static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long
     return;
   }
   size_t bytes = 0;
-  if (n <= 32768) {  // the library's choice at this size, a merge sort of a few passes, is the fastest measured
-    HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
+  if (n <= 32768) {  // rocPRIM's own choice at this size (a merge sort of a few passes) is the fastest measured
+    HIP_CHECK(rocprim::radix_sort_pairs(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u, (unsigned)end_bit, s));
     m.tmp.reserve(bytes + 16);
-    HIP_CHECK(hipcub::DeviceRadixSort::SortPairs(m.tmp.p, bytes, kin, kout, vin, vout, (int)n, 0, end_bit, s));
+    HIP_CHECK(rocprim::radix_sort_pairs(m.tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u, (unsigned)end_bit, s));
     return;
   }
   HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u,
@@ -178,9 +179,9 @@ static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long
 }
 static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipStream_t s) {
   size_t bytes = 0;
-  HIP_CHECK(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, in, out, (int)n, s));
+  HIP_CHECK(rocprim::exclusive_scan(nullptr, bytes, in, out, 0, (size_t)n, rocprim::plus<int>(), s));
   m.tmp.reserve(bytes + 16);
-  HIP_CHECK(hipcub::DeviceScan::ExclusiveSum(m.tmp.p, bytes, in, out, (int)n, s));
+  HIP_CHECK(rocprim::exclusive_scan(m.tmp.p, bytes, in, out, 0, (size_t)n, rocprim::plus<int>(), s));
 }
 // Copies `words` ints from the device into the handle's pinned words and waits for them: the
 // one host round trip of a construction step.

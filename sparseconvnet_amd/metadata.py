@@ -20,6 +20,15 @@ def _ptr(t):
     return C.c_void_p(t.data_ptr()) if t is not None and t.numel() else C.c_void_p(0)
 
 
+def _mark_written(t):
+    """Moves the version counter of a tensor the library has written to behind torch's back."""
+    try:
+        torch.autograd.graph.increment_version(t)
+    except AttributeError:  # older torch: drop everything that is keyed on version counters instead
+        import sparseconvnet_amd
+        sparseconvnet_amd.parameters_changed()
+
+
 def _features(t, what):
     if not t.is_cuda:
         raise _lib.ScnError("%s must be a CUDA tensor: this library has no CPU path" % what)
@@ -357,6 +366,11 @@ class Metadata:
                                             features.stride(0), out.stride(0), _ptr(save_mean), _ptr(save_invstd),
                                             _ptr(running_mean), _ptr(running_var), _ptr(w), _ptr(b), float(eps),
                                             float(momentum), float(leakiness), _stream()))
+        # The library wrote the running statistics through raw pointers: tell torch, so that whatever is
+        # keyed on their version counters (the folded batch norms eval-mode convolutions keep) notices.
+        for t in (running_mean, running_var):
+            if t is not None:
+                _mark_written(t)
         return out, save_mean, save_invstd
 
     def batchNormBackward(self, features, output, grad_output, save_mean, save_invstd, weight, leakiness, affine):

@@ -75,6 +75,52 @@ def check_input_layer(make, dim, mode, seed, n=300, spatial=9, batch=3, with_bat
         assert (out[~picked] == 0).all()
 
 
+def check_mode0_repeated_points(make, dim, seed, n=300, spatial=9, batch=2, cin=3, cout=4):
+    """InputLayer mode 0 with a quarter of the points repeated (Metadata/IOLayersRules.h:28-58:
+    `mp[p] = i` for every point in turn, so the last point of a site wins).  Every point keeps a
+    row of its own (nActive = n, rows in input order, features copied), but only the winner of a
+    site is in the grid: the rules of a 3^d convolution connect winners only, and the rows of
+    shadowed points receive the bias alone.
+    getSpatialLocations: the reference walks the grids (Metadata.cpp:149-170) and leaves the rows
+    of shadowed points at zero; the HIP library keeps every point's coordinates.  Both are
+    accepted for those rows, the winners' rows must hold their coordinates."""
+    rng = np.random.default_rng(seed)
+    coords = bf.random_sites(rng, dim, spatial, n, batch, duplicates=n // 4)
+    feats = rng.normal(size=(len(coords), cin)).astype(np.float32)
+    p = make(dim)
+    assert p.input_layer(spatial, coords, 0, 0) == len(coords)
+    x = p.input_fwd(feats)
+    assert_close(x, feats)
+    last = {}
+    for i, c in enumerate(map(tuple, coords.tolist())):
+        last[c] = i
+    winner = np.zeros(len(coords), bool)
+    winner[list(last.values())] = True
+    assert 0 < (~winner).sum() < len(coords)
+    loc = p.spatial_locations(spatial)
+    assert loc.shape == coords.shape and (loc[winner] == coords[winner]).all()
+    assert (loc[~winner] == 0).all() or (loc[~winner] == coords[~winner]).all()
+    rules = p.submanifold_rules(spatial, 3)
+    got = set((k, int(i), int(j)) for k, r in enumerate(rules) for i, j in np.asarray(r).reshape(-1, 2).tolist())
+    sites = np.array(sorted(last), np.int64)
+    want_rules = set((t[0], last[t[1:2 + dim]], last[t[2 + dim:]]) for t in bf.submanifold_triples(sites, dim, 3))
+    assert got == want_rules
+    assert sum(len(r) for r in rules) == len(got)
+    K = 3 ** dim
+    w = (rng.normal(size=(K, 1, cin, cout)) * 0.3).astype(np.float32)
+    b = rng.normal(size=cout).astype(np.float32)
+    y, macs = p.subm_conv(spatial, 3, x, w, b)
+    assert macs == len(got) * cin * cout
+    want = np.tile(b.astype(np.float64), (len(coords), 1))
+    for k, i, j in want_rules:
+        want[j] += feats[i].astype(np.float64) @ w[k, 0].astype(np.float64)
+    assert_close(y, want.astype(np.float32), "convolution over a mode-0 level with repeated points")
+    assert (y[~winner] == b).all()
+    # the output layer hands every point its own row back
+    assert_close(p.output_fwd(y), y)
+    return coords, feats, w, b, y, rules
+
+
 def check_bl_input_layer(make, dim, mode, seed, batch=3, length=70, spatial=9, planes=5, empties=True):
     """BLInputLayer / BLOutputLayer against a per-sample dictionary: row numbering, rule table,
     merged features (mode 1 = last point of a site, 2 = first, 3 = sum, 4 = mean) and the way

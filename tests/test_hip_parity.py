@@ -32,6 +32,13 @@ def test_input_layer_no_batch_column(make):
     checks.check_input_layer(make, 2, 0, seed=6, with_batch_col=False)
 
 
+@pytest.mark.parametrize("dim", [1, 2, 3])
+def test_input_layer_mode0_repeated_points(make, dim):
+    checks.check_mode0_repeated_points(make, dim, seed=40 + dim)
+    if dim == 3:  # many workgroups, MFMA convolution kernel
+        checks.check_mode0_repeated_points(make, dim, seed=44, n=20000, spatial=48, cin=16, cout=16)
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("dim", [2, 3])
 def test_bl_input_layer(make, dim, mode):
@@ -263,8 +270,9 @@ def _neighbour_counts(coords, spatial):
 @pytest.mark.parametrize("cin,cout", [(32, 32), (32, 16), (64, 64), (64, 32), (128, 128), (96, 160), (256, 256), (128, 32)])
 def test_bf16_path_vs_oracle(oracle_built, cin, cout):
     """The optional bf16-operand path: submanifold convolution (with and without a batch norm
-    in front), strided convolution and deconvolution against the fp32 oracle, within 1e-2 of
-    the output scale; the fp32 path on the same handle stays within its own tolerance."""
+    in front), strided convolution and deconvolution against the fp32 oracle, every element within
+    1e-2 relative + 4e-3 of the largest output; the fp32 path on the same handle stays within its own
+    tolerance."""
     hp, op = _both(3, oracle_built)
     hp.set_bf16(True)
     rng = np.random.default_rng(cin * 7 + cout)
@@ -276,10 +284,15 @@ def test_bf16_path_vs_oracle(oracle_built, cin, cout):
     ro, rh = canon_rows(op.spatial_locations(64)), canon_rows(hp.spatial_locations(64))
 
     def close(got, want, what):
+        # 1e-2 relative per element, plus an absolute term for elements that are small through
+        # cancellation: operands rounded to 8 significant bits put an error of about 2e-3 of the
+        # output's root mean square on every sum, whatever the sum's own size (4e-3 of the largest
+        # output is a few times that).
         scale = float(np.abs(want).max())
-        err = float(np.abs(got - want).max())
-        assert err <= 1e-2 * scale, "%s: max err %g against scale %g" % (what, err, scale)
-        assert err > 0  # the reduced-precision kernels did run
+        err = np.abs(got.astype(np.float64) - want)
+        bad = err > 4e-3 * scale + 1e-2 * np.abs(want)
+        assert not bad.any(), "%s: %d/%d off, max err %g against scale %g" % (what, bad.sum(), bad.size, err.max(), scale)
+        assert err.max() > 0  # the reduced-precision kernels did run
 
     w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
     yo, _ = op.subm_conv(64, 3, xo, w)

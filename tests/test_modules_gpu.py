@@ -96,6 +96,31 @@ def test_unet_vs_oracle(oracle_built):
     assert logits.shape == (len(coords), 20)
 
 
+@pytest.mark.parametrize("batch,target,seed", [(1, 120000, 5100), (2, 40000, 5101)])
+def test_unet_full_width_vs_oracle(oracle_built, batch, target, seed):
+    """Configuration 5 at its full width (examples/ScanNet/unet.py:25-38): m = 32, 7 levels with
+    32 ... 224 planes (joins up to 448), two blocks per level, InputLayer mode 4 with 30 %
+    repeated points, in a 4096^3 grid; only the scene is smaller than the benchmark's (levels of
+    120 k, 29 k, 7 k, ... sites, which takes every convolution kernel family and the small-level
+    paths).  GPU against the oracle over the same module tree, 1e-4 relative / 1e-5 absolute."""
+    torch.manual_seed(seed)
+    m = 32
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m * (i + 1) for i in range(7)], False)).add(scn.OutputLayer(3)).eval()
+    randomise_bn(model, seed)
+    if batch == 1:
+        coords = synthetic.room_scene(seed=seed, target=target, spatial=4096, duplicate_fraction=0.3)
+    else:
+        coords = synthetic.scene_batch(seed=seed, batch=batch, target=target, spatial=4096, duplicate_fraction=0.3)
+    rng = np.random.default_rng(seed)
+    feats = rng.uniform(-1, 1, size=(len(coords), 3)).astype(np.float32)
+    inp_layer = scn.InputLayer(3, 4096, mode=4)
+    got, want, p = _run_both(model, inp_layer, [torch.as_tensor(coords), torch.as_tensor(feats)])
+    assert got.shape == (len(coords), m)
+    assert len(p.spatial_locations(64)) > 0  # all seven levels are populated
+    checks.assert_close(got.cpu().numpy(), want, "full-width U-Net output rows (batch %d)" % batch)
+
+
 def test_residual_unet_vs_oracle(oracle_built):
     """The ScanNet example's residual variant at reduced width: blocks of two BN + convolution
     pairs added to the block input, through a NetworkInNetwork where the plane count changes."""
@@ -775,3 +800,38 @@ def test_frozen_parameters_agree_and_follow_changes():
     finally:
         scn.frozen_parameters = True
     assert torch.equal(run(), want) and not torch.equal(want, changed)
+
+
+@pytest.mark.gpu
+def test_frozen_parameters_follow_training_mode_batch_norm():
+    """A training-mode forward updates the running statistics inside the library, through raw
+    pointers.  The folded batch norms that eval-mode convolutions keep must notice: an eval pass,
+    a train-mode forward without any optimiser step, and an eval pass again, which has to equal
+    the result computed with nothing kept."""
+    torch.manual_seed(13)
+    m = 16
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 1, [m, 2 * m, 3 * m], False)).add(scn.BatchNormReLU(m)).add(scn.OutputLayer(3)).cuda().eval()
+    randomise_bn(model, 13)
+    for p in model.parameters():
+        p.requires_grad_(False)  # a frozen backbone: no weight's version counter will move either
+    coords = synthetic.room_scene(seed=9400, target=15000, spatial=256, duplicate_fraction=0.2)
+    feats = torch.rand((len(coords), 3), device="cuda")
+    layer = scn.InputLayer(3, 256, mode=4)
+
+    def run():
+        with torch.no_grad():
+            return model(layer([torch.as_tensor(coords), feats])).clone()
+
+    before = run()
+    model.train()
+    run()            # batch statistics; running_mean / running_var move
+    model.eval()
+    after = run()
+    assert not torch.equal(after, before)
+    scn.frozen_parameters = False
+    try:
+        want = run()
+    finally:
+        scn.frozen_parameters = True
+    assert torch.equal(after, want)

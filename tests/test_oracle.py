@@ -33,6 +33,11 @@ def test_input_layer_no_batch_column(make):
     checks.check_input_layer(make, 2, 0, seed=6, with_batch_col=False)
 
 
+@pytest.mark.parametrize("dim", [1, 2, 3])
+def test_input_layer_mode0_repeated_points(make, dim):
+    checks.check_mode0_repeated_points(make, dim, seed=40 + dim)
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("dim", [2, 3])
 def test_bl_input_layer(make, dim, mode):

@@ -83,6 +83,38 @@ def test_noalloc_matches_the_allocating_entry_point():
         y = torch.empty((n, 256), device="cuda")
         assert L.scn_subm_conv_fwd_noalloc(h, sp, fs, _ptr(x), _ptr(y), _ptr(w), None, 512, 256, stream) != 0
         assert b"8 MiB" in L.scn_last_error()
+        # more than 256 output planes would need an allocated copy of the weights: refused as well
+        x = torch.randn((n, 64), device="cuda", generator=g)
+        w = torch.randn((27, 1, 64, 320), device="cuda", generator=g)
+        y = torch.empty((n, 320), device="cuda")
+        assert L.scn_subm_conv_fwd_noalloc(h, sp, fs, _ptr(x), _ptr(y), _ptr(w), None, 64, 320, stream) != 0
+        assert b"256 output planes" in L.scn_last_error()
+        # A handle that has only had its rulebook built (no allocating convolution has warmed any of
+        # its buffers): the allocation counter must not move over calls of every kernel family.
+        coords = synthetic.room_scene(seed=7102, target=20000, spatial=256)
+        cd = torch.as_tensor(coords).cuda()
+        hf = L.scn_md_create(3)
+        scenes.append((hf, None, None, 0, cd))
+        nf = C.c_int64(0)
+        spf = _lib.sizes(3, 256)
+        _lib.check(L.scn_md_input_layer(hf, spf, _ptr(cd), len(coords), 4, 0, 0, stream, C.byref(nf)))
+        _lib.check(L.scn_md_submanifold_rules(hf, spf, fs, stream))
+        fresh = []
+        for cin, cout in pairs:
+            x = torch.randn((nf.value, cin), device="cuda", generator=g)
+            w = torch.randn((27, 1, cin, cout), device="cuda", generator=g) * (2.0 / (cin * 27)) ** 0.5
+            fresh.append((x, w, torch.empty((nf.value, cout), device="cuda"), torch.empty((nf.value, cout), device="cuda"), cin, cout))
+        torch.cuda.synchronize()
+        _lib.check(L.scn_cache_stats(None, None, None, C.byref(before)))
+        for x, w, got, _, cin, cout in fresh:
+            _lib.check(L.scn_subm_conv_fwd_noalloc(hf, spf, fs, _ptr(x), _ptr(got), _ptr(w), None, cin, cout, stream))
+        _lib.check(L.scn_cache_stats(None, None, None, C.byref(after)))
+        assert after.value == before.value, "the allocation-free entry point allocated device memory on a fresh handle"
+        for x, w, got, want, cin, cout in fresh:
+            _lib.check(L.scn_subm_conv_fwd(hf, spf, fs, _ptr(x), _ptr(want), _ptr(w), None, cin, cout, 1, stream, None))
+        torch.cuda.synchronize()
+        for x, w, got, want, cin, cout in fresh:
+            checks.assert_close(got.cpu().numpy(), want.cpu().numpy(), "fresh handle %d -> %d" % (cin, cout))
     finally:
         for h, *_ in scenes:
             L.scn_md_destroy(h)
