@@ -32,7 +32,7 @@ def build_library(verbose=False, incremental=False):
         objs.append(o)
         if incremental and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(s), newest_header):
             continue
-        cmd = [hipcc] + [f for f in FLAGS if f != "-shared"] + ["-c", s, "-o", o]
+        cmd = [hipcc] + [f for f in FLAGS if f != "-shared"] + os.environ.get("SCN_EXTRA_FLAGS", "").split() + ["-c", s, "-o", o]
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
     for cmd, p in procs:
         out = p.communicate()[0].decode()

@@ -84,6 +84,60 @@ struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
   float leak = 1.0f;
 };
 
+// What a tile's workgroup (NT threads, G granules of 16 positions from position tbase on) sets up
+// before its tap loop: the tile's neighbour rows in LDS, jtab[(granule * K + tap) * 16 + row], the
+// granules that have each tap, gmask[tap], and the list of the taps any of its rows has (of those
+// this workgroup is to take when the taps of a tile are dealt over n_split workgroups: tap k
+// belongs to workgroup k % n_split).  Every thread of the workgroup calls it; it ends with a
+// barrier and returns the length of the list.
+// The table is read tap by tap, 16 * G consecutive entries each, and all of a thread's loads
+// (up to eight) are in flight together: a loop of load - store - ballot steps paid one memory
+// latency per step, 5 us for 27 taps where the whole convolution of a small level takes 20.
+template <int NT, int G>
+__device__ inline int tile_setup(const int *__restrict__ nbr, int K, int64_t n, int64_t npad, int64_t tbase, int n_split,
+                                 int split, int *jtab, unsigned *gmask, int *taplist, int *ntaps_p) {
+  constexpr int PER_TAP = G * 16;          // entries of one tap
+  static_assert(NT % PER_TAP == 0 || PER_TAP % NT == 0, "threads and tile rows must divide one another");
+  for (int k = threadIdx.x; k < K; k += NT) gmask[k] = 0u;
+  __syncthreads();
+  const int total = K * PER_TAP;
+  constexpr int BATCH = 8;
+  for (int e0 = 0; e0 < total; e0 += BATCH * NT) {
+    int jv[BATCH];
+#pragma unroll
+    for (int i = 0; i < BATCH; i++) {
+      const int e = e0 + i * NT + (int)threadIdx.x;
+      const int k = e / PER_TAP, p = e % PER_TAP;
+      jv[i] = -1;
+      if (e < total && tbase + p < n) jv[i] = nbr[(int64_t)k * npad + tbase + p];
+    }
+#pragma unroll
+    for (int i = 0; i < BATCH; i++) {
+      const int e = e0 + i * NT + (int)threadIdx.x;
+      const int k = e / PER_TAP, p = e % PER_TAP;
+      if (e < total) jtab[((p >> 4) * K + k) * 16 + (p & 15)] = jv[i];
+      // sixteen consecutive lanes hold one granule's rows of one tap
+      const unsigned long long bal = __ballot(jv[i] >= 0);
+      const int lane = threadIdx.x & 63;
+      if ((lane & 15) == 0 && e < total && ((bal >> lane) & 0xFFFFull)) atomicOr(&gmask[k], 1u << (p >> 4));
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {  // the first wavefront lists the taps, 64 at a time, in ascending order
+    int count = 0;
+    for (int k0 = 0; k0 < K; k0 += 64) {
+      const int k = k0 + (int)threadIdx.x;
+      const bool mine = k < K && gmask[k] != 0u && (n_split == 1 || k % n_split == split);
+      const unsigned long long bal = __ballot(mine);
+      if (mine) taplist[count + __popcll(bal & ((1ull << threadIdx.x) - 1ull))] = k;
+      count += __popcll(bal);
+    }
+    if (threadIdx.x == 0) *ntaps_p = count;
+  }
+  __syncthreads();
+  return *ntaps_p;
+}
+
 // Launchers of the kernels conv.hip defines for the other translation units.
 // k_pack_weights / k_pack_weights_part / k_pack_weights_c4: weights into MFMA B-operand order.
 void launch_pack_weights(const float *w, float *wp, int K, int n_in, int n_out, int n_slab, int SS, int NCB,

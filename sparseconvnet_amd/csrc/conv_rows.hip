@@ -3,6 +3,11 @@
 
 namespace scn {
 
+static int dbg_prio() {
+  static const int v = getenv("SCN_DBG_PRIO") ? atoi(getenv("SCN_DBG_PRIO")) : 0;
+  return v;
+}
+
 // ---- row-owner kernel for mid-width layers ----------------------------------------------
 // NW wavefronts, each owning RG granules of a tile of NW*RG granules.  Only the weight slab
 // goes through (double-buffered) LDS; every wavefront gathers the input rows of its own
@@ -16,7 +21,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
-    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
+    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes, int prio) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int NT = NW * 64;
@@ -37,39 +42,18 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
 
-  const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+  const int tile = tiles_per_xcd ? (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3) : blockIdx.x;
   if (tile >= n_tiles) return;
   const int64_t tbase = (int64_t)tile * TM;
 
-  for (int k = threadIdx.x; k < K; k += NT) gmask[k] = 0u;
-  __syncthreads();
-#pragma unroll
-  for (int q = 0; q < RG; q++) {
-    const int gr = wave * RG + q;
-    const int64_t t = tbase + gr * 16 + r16;
-    for (int kb = 0; kb < K; kb += 4) {
-      const int k = kb + g;
-      int j = -1;
-      if (k < K && t < n) j = nbr[(int64_t)k * npad + t];
-      if (k < K) jtab[(gr * K + k) * 16 + r16] = j;
-      const unsigned long long bal = __ballot(j >= 0);
-      if (lane == 0) {
-#pragma unroll
-        for (int gg = 0; gg < 4; gg++)
-          if ((bal >> (16 * gg)) & 0xFFFFull) atomicOr(&gmask[kb + gg], 1u << gr);
-      }
-    }
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int c = 0;
-    for (int k = 0; k < K; k++)
-      if (gmask[k] && (n_split == 1 || k % n_split == (int)blockIdx.y)) taplist[c++] = k;
-    *ntaps_p = c;
-  }
-  __syncthreads();
-  const int ntaps = *ntaps_p;
+  const int ntaps = tile_setup<NT, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
   const int total = ntaps * n_slab;
+  if (prio) {
+    const int q = ntaps * 4 / (K + 1);
+    if (q >= 3) __builtin_amdgcn_s_setprio(3);
+    else if (q == 2) __builtin_amdgcn_s_setprio(2);
+    else if (q == 1) __builtin_amdgcn_s_setprio(1);
+  }
 
   v4f acc[RG][NCB];
 #pragma unroll
@@ -319,14 +303,14 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
     attr_set = true;
   }
   const int n_tiles = (int)ceil_div(t.n, G * 16);
-  const int tiles_per_xcd = (int)ceil_div(n_tiles, 8);
+  const int tiles_per_xcd = t.spread ? 0 : (int)ceil_div(n_tiles, 8);  // 0: tile = workgroup index
   int n_split = 1;
   if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
   float *partial = scratch_partial(m, n_split, split_stride);
-  kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), NT, lds_bytes, s>>>(
+  kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), NT, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4), dbg_prio());
   LAUNCH_CHECK();
   if (n_split > 1) {
     launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
@@ -347,6 +331,16 @@ static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *o
   // 60 k sites is 480 such workgroups for 256 CUs: one wavefront per SIMD, nothing to run while
   // it waits for its gathers).  Measured: 13-18 % faster at 62 k sites, 5 % at 15 k and 250 k,
   // equal at 1 M except for 64 output planes, which gain 2 % there too.
+  if constexpr (VEC4) {
+    static const int dss = getenv("SCN_DBG_SS") ? atoi(getenv("SCN_DBG_SS")) : 0;
+    if (!narrow && ncb > 2 && (t.n < 300000 || ncb <= 4) && dss && n_in % (16 * dss) == 0) {
+#define SCN_TRY(N, S) if (ncb <= N && dss == S) return launch_rows<N, 1, S, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      SCN_TRY(4, 4) SCN_TRY(4, 3) SCN_TRY(4, 6)
+      SCN_TRY(6, 4) SCN_TRY(6, 3) SCN_TRY(6, 6)
+      SCN_TRY(8, 4) SCN_TRY(8, 3)
+#undef SCN_TRY
+    }
+  }
   if (!narrow && ncb > 2 && (t.n < 300000 || ncb <= 4)) {
     if (ncb <= 4) return launch_rows<4, 1, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     if (ncb <= 6) return launch_rows<6, 1, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);

@@ -2,6 +2,17 @@
 #include "conv_common.h"
 
 namespace scn {
+#ifdef SCN_PHASES
+__device__ unsigned long long g_phase[16 * 8];
+#define PHASE(i) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 16) g_phase[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define PHASE(i)
+#endif
+
+static int dbg_prio() {
+  static const int v = getenv("SCN_DBG_PRIO") ? atoi(getenv("SCN_DBG_PRIO")) : 0;
+  return v;
+}
 
 // ---- MFMA kernel ------------------------------------------------------------------------
 // A workgroup of 4 wavefronts owns a tile of G = GW*WR granules (16 rows each).  The
@@ -25,7 +36,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
-    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
+    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes, int prio) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int WR = 4 / WC;
@@ -52,40 +63,21 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of
   // tiles so that neighbouring tiles (which gather the same rows) share one L2.
-  const int tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+  PHASE(0);
+  const int tile = tiles_per_xcd ? (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3) : blockIdx.x;
   if (tile >= n_tiles) return;  // whole workgroup leaves: no barrier is skipped
   const int64_t tbase = (int64_t)tile * TM;
 
-  for (int k = threadIdx.x; k < K; k += 256) gmask[k] = 0u;
-  __syncthreads();
-  // Neighbour rows of the tile -> LDS, four taps per pass (one per 16-lane group).
-  for (int gr = wave; gr < G; gr += 4) {
-    const int64_t t = tbase + gr * 16 + r16;
-    for (int kb = 0; kb < K; kb += 4) {
-      const int k = kb + g;
-      int j = -1;
-      if (k < K && t < n) j = nbr[(int64_t)k * npad + t];
-      if (k < K) jtab[(gr * K + k) * 16 + r16] = j;
-      const unsigned long long bal = __ballot(j >= 0);
-      if (lane == 0) {
-#pragma unroll
-        for (int gg = 0; gg < 4; gg++)
-          if ((bal >> (16 * gg)) & 0xFFFFull) atomicOr(&gmask[kb + gg], 1u << gr);
-      }
-    }
+  const int ntaps = tile_setup<256, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
+  PHASE(1);
+  const int total = ntaps * n_slab;
+  PHASE(2);
+  if (prio) {
+    const int q = ntaps * 4 / (K + 1);
+    if (q >= 3) __builtin_amdgcn_s_setprio(3);
+    else if (q == 2) __builtin_amdgcn_s_setprio(2);
+    else if (q == 1) __builtin_amdgcn_s_setprio(1);
   }
-  __syncthreads();
-  // With n_split > 1 the taps of a tile are dealt over n_split workgroups (blockIdx.y), each
-  // of which writes a partial tile that k_conv_reduce sums: small levels have too few tiles
-  // to fill the GPU and too long a serial tap loop otherwise.
-  if (threadIdx.x == 0) {
-    int c = 0;
-    for (int k = 0; k < K; k++)
-      if (gmask[k] && (n_split == 1 || k % n_split == (int)blockIdx.y)) taplist[c++] = k;
-    *ntaps_p = c;
-  }
-  __syncthreads();
-  const int total = *ntaps_p * n_slab;
 
   v4f acc[GW][NCBW];
 #pragma unroll
@@ -112,7 +104,6 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   const __amdgpu_buffer_rsrc_t rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, BUF ? (int)in_bytes : 0, 0x00020000);
   const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)g;
-  const int ntaps = *ntaps_p;
   // Issue the loads of iteration `it`: this wavefront's weights into register set P (= it % 2)
   // and its share of the A fragments (granule, step) into areg.
   auto issue = [&](int it, auto par_c) {
@@ -238,10 +229,13 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   };
 
   if (total > 0) issue(0, std::integral_constant<int, 0>{});
+  PHASE(3);
   for (int it = 0; it < total; it += 2) {
     iterate(it, std::integral_constant<int, 0>{});
+    if (it == 0) PHASE(4);
     if (it + 1 < total) iterate(it + 1, std::integral_constant<int, 1>{});
   }
+  PHASE(5);
 
   // acc[q][c][r] = result for position tbase + 16*(wr*GW+q) + 4*g + r, column 16*(wc*NCBW+c) + r16
   if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
@@ -253,6 +247,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 #pragma unroll
         for (int c = 0; c < NCBW; c++)
           pt[(int64_t)((wr * GW + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * (wc * NCBW + c) + r16] = acc[q][c][r];
+    PHASE(6);
     return;
   }
   float bv[NCBW], es[NCBW], eh[NCBW];
@@ -313,15 +308,15 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
     attr_set = true;
   }
   const int n_tiles = (int)ceil_div(t.n, G * 16);
-  const int tiles_per_xcd = (int)ceil_div(n_tiles, 8);
+  const int tiles_per_xcd = t.spread ? 0 : (int)ceil_div(n_tiles, 8);  // 0: tile = workgroup index
   // Few tiles: deal the taps of every tile over several workgroups (about two per CU in all).
   int n_split = 1;
   if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
   float *partial = scratch_partial(m, n_split, split_stride);
-  kern<<<dim3((unsigned)(tiles_per_xcd * 8), n_split), 256, lds_bytes, s>>>(
+  kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), 256, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4), dbg_prio());
   LAUNCH_CHECK();
   if (n_split > 1) {
     launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
@@ -343,6 +338,22 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
   // Levels of a few thousand sites: 64-row tiles instead of 128-row ones give the chip twice the
   // workgroups to spread (measured: 12-23 % faster at 16 k sites, 10 % at 1 k, 30 % at 250,
   // equal at 4 k, where the tap split halves in exchange).
+  if constexpr (VEC4) {
+    static const int dss = getenv("SCN_DBG_TSS") ? atoi(getenv("SCN_DBG_TSS")) : 0;
+    if (!narrow && t.n < 30000 && ncb > 8 && (dss == 2 || dss == 4)) {
+      if (dss == 2) {
+        if (ncb <= 10) return launch_mfma<5, 2, 2, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+        if (ncb <= 12) return launch_mfma<3, 4, 4, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+        if (ncb <= 14) return launch_mfma<7, 2, 2, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+        if (ncb <= 16) return launch_mfma<4, 4, 4, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      } else {
+        if (ncb <= 10) return launch_mfma<5, 2, 2, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+        if (ncb <= 12) return launch_mfma<3, 4, 4, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+        if (ncb <= 14) return launch_mfma<7, 2, 2, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+        if (ncb <= 16) return launch_mfma<4, 4, 4, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      }
+    }
+  }
   if (!narrow && t.n < 30000 && ncb > 8) {
     if (ncb <= 10) return launch_mfma<5, 2, 2, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     if (ncb <= 12) return launch_mfma<3, 4, 4, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
@@ -373,4 +384,9 @@ bool conv_tiled_dispatch(bool vec4, bool pre_fused, Metadata &m, const Table &t,
               : dispatch_ncb<false, false>(ncb, m, t, in, out, w, epi, n_in, n_out, pre, s);
 }
 
+#ifdef SCN_PHASES
+extern "C" int scn_dbg_phases(unsigned long long *out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_phase), sizeof(g_phase));
+}
+#endif
 }  // namespace scn

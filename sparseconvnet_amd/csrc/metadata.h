@@ -75,6 +75,10 @@ struct Table {
   DevBuf<int> rowmap;
   DevBuf<unsigned> gmask;  // K <= 32 and pattern-sorted: bit k of gmask[i] = some position of granule i (16 positions) has tap k
   bool identity_rows = false;  // rowmap[t] == t: kernels skip the indirection
+  // The pattern sort ran over all positions at once (small levels): consecutive tiles descend in
+  // cost from the first to the last, so kernels deal tiles to workgroups in turn instead of giving
+  // each XCD a contiguous range.
+  bool spread = false;
   const int *rowmap_ptr() const { return identity_rows ? nullptr : rowmap.p; }
   // Submanifold tables, decided on first use by a backward pass: does rule (k, i -> j) imply
   // rule (K-1-k, j -> i)?  (Odd filter sizes on a level without repeated points.)

@@ -684,9 +684,13 @@ struct Filt {
 // One thread per schedule position t: probe the filter box around the row's site
 // (Metadata/SubmanifoldConvolutionRules.h:11-45; taps enumerate the box row-major with the
 // last dimension fastest, Metadata/RectangularRegions.h:56-71).
+// dup_keys (levels whose keys may repeat, else null): the positions' keys, ascending; of a run of
+// equal keys only the last position is a site (`mp[p] = i`, Metadata/IOLayersRules.h:41,54), the
+// others are rows no rule touches.
 __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, int64_t n,
                              int64_t npad, const BlockEntry *table, const unsigned long long *mask_p,
-                             const int *urow, int *nbr, unsigned long long *counts, int parts) {
+                             const int *urow, int *nbr, unsigned long long *counts, int parts,
+                             const unsigned long long *dup_keys) {
   const unsigned long long mask = *mask_p;
   // blockDim = 64 * parts: wavefront p of the block handles taps [p*K/parts, (p+1)*K/parts)
   // (one slice of the first filter dimension) of the block's 64 positions.
@@ -713,8 +717,9 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
     int b = soa[g.dim * npad + row];
     unsigned long long last_bkey = SCN_EMPTY_KEY, last_mask = 0;  // block of the previous tap
     int last_base = 0;
+    const bool shadowed = dup_keys && t + 1 < n && dup_keys[t + 1] == dup_keys[t];
     for (int k = k0; k < k0 + per; k++) {
-      bool inside = true;
+      bool inside = !shadowed;
       for (int d = 0; d < g.dim; d++) {
         q[d] = c[d] + tap[d] - f.size[d] / 2;
         if (q[d] < 0 || q[d] >= g.size[d]) inside = false;
@@ -860,7 +865,8 @@ __global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
 static PatternKey pattern_plan(int64_t n, int K, int &key_bits) {
   PatternKey p;
   p.K = K;
-  p.window = std::max<int64_t>(256, round_up(ceil_div(n, PATTERN_WINDOWS), 256));
+  static const int64_t gsort = getenv("SCN_DBG_GSORT") ? atoll(getenv("SCN_DBG_GSORT")) : 0;
+  p.window = std::max<int64_t>(256, round_up(ceil_div(n, n < gsort ? 1 : PATTERN_WINDOWS), 256));
   int block_bits = 0;
   while (((int64_t)1 << block_bits) < ceil_div(n, p.window)) block_bits++;
   int pc_bits = 1;
@@ -905,6 +911,7 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   }
   int key_bits = 0;
   const PatternKey pk = pattern_plan(t.n, t.K, key_bits);
+  t.spread = pk.window >= t.n;
   reserve_pattern_buffers(m, t);
   unsigned *masks = t.K <= 32 ? reinterpret_cast<unsigned *>(m.f1.p) : nullptr;
   if (!keyed) {
@@ -946,7 +953,7 @@ template <int DIM>
 __global__ void k_subm_rules_s3(Geom g, const unsigned long long *skeys, int64_t n, int64_t npad,
                                 const BlockEntry *table, const unsigned long long *mask_p, const int *urow,
                                 int *rows, unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
-                                int *pidx, unsigned *pmasks) {
+                                int *pidx, unsigned *pmasks, bool dups) {
   const unsigned long long mask = *mask_p;
   constexpr int K = DIM == 3 ? 27 : 9;
   constexpr int PER = K / 3;
@@ -973,6 +980,8 @@ __global__ void k_subm_rules_s3(Geom g, const unsigned long long *skeys, int64_t
   // The site of position t from its key (the positions' keys are one coalesced read; the
   // coordinates by row would be four gathers through the schedule, per wavefront).
   const unsigned long long skey = skeys[t];
+  // keys may repeat (dups): only the last position of a run of equal keys is a site, see k_subm_rules
+  const bool shadowed = dups && t + 1 < n && skeys[t + 1] == skey;
   unsigned long long sp[DIM][3];
   bool okc[DIM][3];
   int cd[DIM];
@@ -1057,11 +1066,11 @@ __global__ void k_subm_rules_s3(Geom g, const unsigned long long *skeys, int64_t
     unsigned long long key;
     int e;
     if (DIM == 3) {
-      inside = okc[0][part] && okc[1][o1] && okc[2][o2];
+      inside = !shadowed && okc[0][part] && okc[1][o1] && okc[2][o2];
       key = bpart | sp[0][part] | sp[1][o1] | sp[2][o2];
       e = (hi_of[1][o1] ? 2 : 0) + (hi_of[2][o2] ? 1 : 0);
     } else {
-      inside = okc[0][part] && okc[1][o1];
+      inside = !shadowed && okc[0][part] && okc[1][o1];
       key = bpart | sp[0][part] | sp[1][o1];
       e = hi_of[1][o1] ? 1 : 0;
     }
@@ -1247,11 +1256,11 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
     if (m.dim == 3)
       k_subm_rules_s3<3><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.skeys.p, L.n, L.npad, L.table.p,
                                                            L.gridp.p, L.urow_ptr(), m.rowtab.p,
-                                                           (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks);
+                                                           (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks, L.dups);
     else
       k_subm_rules_s3<2><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.skeys.p, L.n, L.npad, L.table.p,
                                                            L.gridp.p, L.urow_ptr(), m.rowtab.p,
-                                                           (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks);
+                                                           (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks, L.dups);
     LAUNCH_CHECK();
     finalize_table(m, t, L.sched_ptr(), s, true, m.rowtab.p, roww);
     return m.subm.emplace(key, std::move(t)).first->second;
@@ -1261,7 +1270,7 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   const int parts = (m.dim >= 2 && f.size[0] <= 4) ? f.size[0] : 1;
   k_subm_rules<<<grid_for(L.n, 64), 64 * parts, f.K * sizeof(int), s>>>(
       L.g, f, L.coords.p, L.sched_ptr(), L.n, L.npad, L.table.p, L.gridp.p, L.urow_ptr(), t.nbr.p,
-      (unsigned long long *)t.cnt->dev.p, parts);
+      (unsigned long long *)t.cnt->dev.p, parts, L.dups ? L.skeys.p : nullptr);
   LAUNCH_CHECK();
   finalize_table(m, t, L.sched_ptr(), s);
   return m.subm.emplace(key, std::move(t)).first->second;
@@ -1288,9 +1297,11 @@ __device__ inline bool candidate(const Geom &gi, const Filt &f, const int *p, in
 // zero: 16 x 64 counters that the launch behind this one (k_strided_heads) adds to, or null.
 // pos_keys (optional, dimensions up to 3): the site key of every schedule position; the site is
 // then decoded from one coalesced read instead of gathered by row through the schedule.
+// dup_keys (levels whose keys may repeat, else null): the positions' keys; only the last position of a
+// run of equal keys is a site (see k_subm_rules), the others have no candidates.
 __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, const int *sched,
                                      const unsigned long long *pos_keys, int64_t n, int64_t npad,
-                                     unsigned long long *keys, int *payload, int *zero) {
+                                     unsigned long long *keys, int *payload, int *zero, const unsigned long long *dup_keys) {
   if (zero && blockIdx.x == 0)
     for (int i = threadIdx.x; i < 16 * 64; i += blockDim.x) zero[i] = 0;
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1306,7 +1317,8 @@ __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, c
     for (int d = 0; d < f.dim; d++) p[d] = soa[d * npad + row];
     b = soa[f.dim * npad + row];
   }
-  keys[e] = candidate(gi, f, p, m, j) ? site_key(go, j, b) : SCN_EMPTY_KEY;
+  const bool shadowed = dup_keys && t + 1 < n && dup_keys[t + 1] == dup_keys[t];
+  keys[e] = (!shadowed && candidate(gi, f, p, m, j)) ? site_key(go, j, b) : SCN_EMPTY_KEY;
   payload[e] = (int)e;
 }
 
@@ -1439,7 +1451,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   // Filter = stride = 2 in every dimension over exactly fitting sizes (the U-Net's and most
   // networks' downsampling): each site has one candidate, the Morton key of its coordinates
   // halved, which ascends with the site's own key, so the schedule order is already sorted.
-  bool presorted = m.dim <= 3 && f.M == 1;
+  bool presorted = m.dim <= 3 && f.M == 1 && !LI.dups;  // rows without a site leave holes in the order
   for (int d = 0; d < m.dim; d++)
     presorted = presorted && filter[d] == 2 && stride[d] == 2 && in_size[d] == 2 * out_size[d];
   // The caller has to learn the new level's size: a read-back per rulebook, except along a chain
@@ -1456,8 +1468,9 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   const bool count = presorted && LI.halvings.empty();
   // a level with a schedule of its own (the input layer's): sites from the positions' keys
   const unsigned long long *pos_keys = (m.dim <= 3 && !LI.identity_sched) ? position_keys(LI, s) : nullptr;
+  const unsigned long long *dup_keys = LI.dups ? position_keys(LI, s) : nullptr;
   k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
-                                                   m.k0.p, m.v0.p, count ? m.dflags.p : nullptr);
+                                                   m.k0.p, m.v0.p, count ? m.dflags.p : nullptr, dup_keys);
   LAUNCH_CHECK();
   if (presorted) {
     std::swap(m.k0, m.k1);

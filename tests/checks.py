@@ -118,7 +118,18 @@ def check_mode0_repeated_points(make, dim, seed, n=300, spatial=9, batch=2, cin=
     assert (y[~winner] == b).all()
     # the output layer hands every point its own row back
     assert_close(p.output_fwd(y), y)
-    return coords, feats, w, b, y, rules
+    # a strided rulebook over the same level: its rules start from the winners only
+    # (Metadata/ConvolutionRules.h:61-105 walks the input grids)
+    if spatial == 9:
+        srules = p.strided_rules(9, 4, 3, 2)
+        loc_out = p.spatial_locations(4)
+        got_s = set()
+        for k, r in enumerate(srules):
+            for i, j in np.asarray(r).reshape(-1, 2).tolist():
+                got_s.add((k, int(i)) + tuple(loc_out[j].tolist()))
+        want_s = set((t[0], last[t[1:2 + dim]]) + t[2 + dim:] for t in bf.strided_triples(sites, dim, 3, 2, 4))
+        assert got_s == want_s
+        assert sum(len(r) for r in srules) == len(got_s)
 
 
 def check_bl_input_layer(make, dim, mode, seed, batch=3, length=70, spatial=9, planes=5, empties=True):
