@@ -105,7 +105,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))) voi
   const unsigned shift8 = 8u * (unsigned)g;
   const int64_t n_granules = (n + 15) >> 4;
   const int xcd = blockIdx.x & 7, blk = blockIdx.x >> 3;
-  const int set_end = min(n_sets, (xcd + 1) * sets_per_xcd);
+  // sets_per_xcd == 0 (the table's positions are pattern-sorted as a whole, most expensive first):
+  // sets are dealt to the workgroups in turn instead of one contiguous range per XCD
+  const int set_end = sets_per_xcd ? min(n_sets, (xcd + 1) * sets_per_xcd) : n_sets;
 
   // The next group of (up to) four taps out of `rest`: their numbers packed one per byte (K for
   // an unused slot), and the OR of their bits.
@@ -147,7 +149,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))) voi
   };
 
   for (int sw = 0; sw < sets_per_wave; sw++) {
-    const int set = xcd * sets_per_xcd + (blk * sets_per_wave + sw) * 4 + wave;  // wave-uniform
+    const int set = sets_per_xcd ? xcd * sets_per_xcd + (blk * sets_per_wave + sw) * 4 + wave
+                                 : ((int)blockIdx.x * sets_per_wave + sw) * 4 + wave;  // wave-uniform
     if (set >= set_end) break;
     unsigned gm[4];
 #pragma unroll
@@ -264,11 +267,11 @@ static void launch_first(const Table &t, const float *in, int64_t in_rows, float
                          CoefJob bn, float leak, int n_out, hipStream_t s) {
   const int64_t in_bytes = in_rows * NIN * 4, nbr_bytes = (int64_t)t.K * t.npad * 4, out_bytes = t.n * n_out * 4;
   const int n_sets = (int)ceil_div(t.n, 64);
-  const int sets_per_xcd = (int)ceil_div(n_sets, 8);
+  const int sets_per_xcd = t.spread ? 0 : (int)ceil_div(n_sets, 8);
   // one set per wavefront: measured best (the hardware's workgroup dispatch evens out the sets'
   // different tap counts)
   const int spw = 1;
-  const int blocks = 8 * (int)ceil_div(sets_per_xcd, 4 * spw);
+  const int blocks = sets_per_xcd ? 8 * (int)ceil_div(sets_per_xcd, 4 * spw) : (int)ceil_div(n_sets, 4 * spw);
   k_conv_first<NIN, NCB><<<dim3(blocks), 256, (size_t)(t.K + 1) * first_tap_floats(NIN, NCB) * sizeof(float), s>>>(
       t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, out, w, bias, bn, leak, n_out, n_sets, sets_per_xcd, spw,
       (unsigned)in_bytes, (unsigned)nbr_bytes, (unsigned)out_bytes);

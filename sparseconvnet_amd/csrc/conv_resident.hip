@@ -22,7 +22,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, const unsigned *__restrict__ gmask, int K,
     int64_t n, int64_t npad, const float *__restrict__ in, int in_stride, float *__restrict__ out,
     const float *__restrict__ wp, Epi epi, int n_in, int n_out, int n_sets,
-    int sets_per_xcd, int accumulate, int *__restrict__ queue, unsigned in_bytes, unsigned nbr_bytes) {
+    int sets_per_xcd, int accumulate, int *__restrict__ queue, unsigned in_bytes, unsigned nbr_bytes, int spread) {
   static_assert(!BUF || VEC4 || C4, "buffer gathers need float4 rows or the four-channel layout");
   static_assert(!C4 || SS == 1, "the four-channel layout has one slab");
   static_assert(!BF16 || (BUF && !C4 && SS == 2), "the bf16 variant: buffer gathers, one pair of steps");
@@ -66,8 +66,12 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   // wavefronts of a SIMD finish one after the other, and shares differ in their tap counts.)
   // Every counter value is handed out once, values past the range end a wavefront's stream.
   const int xcd = blockIdx.x & 7, blk = blockIdx.x >> 3, blocks_per_xcd = gridDim.x >> 3;
+  // spread (the table's positions are pattern-sorted as a whole, most expensive first): XCD x takes
+  // the sets x, x + 8, x + 16, ... instead of a contiguous range, which would hand all the expensive
+  // sets to the first XCD.  The stream below counts in the XCD's own numbering; set_of() gives the set.
   const int set_begin = xcd * sets_per_xcd;
-  const int set_end = min(n_sets, set_begin + sets_per_xcd);
+  const int set_end = spread ? set_begin + max(0, (n_sets - xcd + 7) >> 3) : min(n_sets, set_begin + sets_per_xcd);
+  auto set_of = [&](int i) { return min(spread ? (i - set_begin) * 8 + xcd : i, n_sets - 1); };
   const int first_round = blocks_per_xcd * WAVES;
   int *ctr = queue + xcd * 32;
   auto take = [&]() {
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   // generator of the item stream (wave-uniform state)
   int g_set = set_begin + blk * WAVES + wave;
   bool g_has = g_set < set_end;
-  unsigned g_rest = g_has ? set_mask(g_set) : 0u;
+  unsigned g_rest = g_has ? set_mask(set_of(g_set)) : 0u;
   int g_next = take();           // the set after g_set
   unsigned g_mask_next = 0;      // its tap mask, read two items after g_next was requested
   int g_age = 0;
@@ -87,15 +91,15 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
     bool last, valid;
   };
   auto gen = [&]() {
-    if (++g_age == 2) g_mask_next = set_mask(min(g_next, n_sets - 1));
+    if (++g_age == 2) g_mask_next = set_mask(set_of(g_next));
     Item it;
     it.valid = g_has;
-    it.set = g_has ? g_set : 0;
+    it.set = g_has ? set_of(g_set) : 0;
     it.k = g_has ? __ffs(g_rest) - 1 : 0;
     g_rest &= g_rest - 1;
     it.last = g_has && g_rest == 0u;
     if (it.last) {
-      if (g_age < 2) g_mask_next = set_mask(min(g_next, n_sets - 1));  // a set of one or two taps
+      if (g_age < 2) g_mask_next = set_mask(set_of(g_next));  // a set of one or two taps
       g_set = g_next;
       g_has = g_set < set_end;
       g_rest = g_mask_next;
@@ -358,7 +362,7 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
   const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
   kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
                                                    out, wpack, epi, n_in_part, n_out, n_sets, sets_per_xcd,
-                                                   accumulate, scratch_queue(m, s), (unsigned)in_bytes, (unsigned)nbr_bytes);
+                                                   accumulate, scratch_queue(m, s), (unsigned)in_bytes, (unsigned)nbr_bytes, t.spread ? 1 : 0);
   LAUNCH_CHECK();
   }
 }

@@ -3,11 +3,6 @@
 
 namespace scn {
 
-static int dbg_prio() {
-  static const int v = getenv("SCN_DBG_PRIO") ? atoi(getenv("SCN_DBG_PRIO")) : 0;
-  return v;
-}
-
 // ---- row-owner kernel for mid-width layers ----------------------------------------------
 // NW wavefronts, each owning RG granules of a tile of NW*RG granules.  Only the weight slab
 // goes through (double-buffered) LDS; every wavefront gathers the input rows of its own
@@ -21,7 +16,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
-    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes, int prio) {
+    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int NT = NW * 64;
@@ -48,25 +43,39 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 
   const int ntaps = tile_setup<NT, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
   const int total = ntaps * n_slab;
-  if (prio) {
-    const int q = ntaps * 4 / (K + 1);
-    if (q >= 3) __builtin_amdgcn_s_setprio(3);
-    else if (q == 2) __builtin_amdgcn_s_setprio(2);
-    else if (q == 1) __builtin_amdgcn_s_setprio(1);
+  // Filters of up to 64 taps: the tap list and the taps of this wavefront's granules as bit masks in
+  // scalar registers, so that the tap of an iteration and whether a granule has it are scalar
+  // arithmetic instead of LDS reads on the path from the barrier to the first MFMA.
+  const bool small_k = K <= 64;
+  unsigned long long tmask = 0ull, mym[RG];
+#pragma unroll
+  for (int q = 0; q < RG; q++) mym[q] = 0ull;
+  if (small_k) {
+    const unsigned gmv = lane < K ? gmask[lane] : 0u;
+    tmask = __ballot(gmv != 0u && (n_split == 1 || lane % n_split == (int)blockIdx.y));
+#pragma unroll
+    for (int q = 0; q < RG; q++) mym[q] = __ballot((gmv >> (wave * RG + q)) & 1u) & tmask;
   }
-
   v4f acc[RG][NCB];
 #pragma unroll
   for (int q = 0; q < RG; q++)
 #pragma unroll
     for (int cb = 0; cb < NCB; cb++) acc[q][cb] = (v4f){0.f, 0.f, 0.f, 0.f};
 
+  // Loads in flight: the weight slab one iteration ahead (it comes from L2), the gathered rows AD
+  // iterations ahead, in a ring of register sets (the loop below is unrolled AD times so that the
+  // set is a constant).  On a level whose rows an XCD does not keep in its L2 a gather takes longer
+  // than the MFMAs of one iteration (0.7 us at 96 output planes); measured 5 % at 60 k sites.
+  // Two granules per wavefront (the 128-row tiles of million-site levels, whose gathers mostly hit
+  // L2): one iteration of look-ahead, as the ring's registers would cost a wavefront per SIMD.
+  constexpr int AD = RG == 1 ? 3 : 1;
   v4f wreg[WPT];
-  v4f a_nxt[RG][SS];
+  v4f a_ring[AD][RG][SS];
+  unsigned gm_ring[AD] = {}, ok_ring[AD] = {};
+  int sl_ring[AD] = {};
   v4f a_cur[RG][WS];  // bf16: the eight values of a pair of steps
   v4f psc[SS], psh[SS];
-  unsigned gm_nxt = 0, gm_cur = 0, ok_nxt = 0;
-  int sl_nxt = 0;
+  unsigned gm_cur = 0;
 
   typedef int v4i_t __attribute__((ext_vector_type(4)));
   const __amdgpu_buffer_rsrc_t rsrc =
@@ -90,19 +99,46 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     return v;
   };
   const unsigned row_bytes = (unsigned)n_in * 4u, lane_off = 16u * (unsigned)ld_g;
-  int nx_ti = 0, nx_sl = 0;  // (tap index, slab) of the next iteration to issue; issue() runs in sequence
-  auto issue = [&](int) {
-    const int sl = nx_sl;
+  // Two cursors over the iterations (slab outer, tap inner: see k_conv_mfma), one for the weights
+  // and one for the rows.  Both stay on the last iteration once they reach it: the loads are
+  // issued unconditionally (a few re-read the last iteration's operands at the end of a tile), so
+  // the number of loads in flight at every wait is a constant the compiler can count on.
+  int w_ti = 0, w_sl = 0, w_left = total;
+  int a_ti = 0, a_sl = 0, a_left = total;
+  unsigned long long w_rest = tmask, a_rest = tmask;  // small_k: taps of the current slab still to come
+  // The tap at a cursor, and the cursor's step to the next iteration (it stays on the last one).
+  auto tap_at = [&](int ti, unsigned long long rest) {
+    return small_k ? (int)__builtin_ctzll(rest | (1ull << 63)) : __builtin_amdgcn_readfirstlane(taplist[ti]);
+  };
+  auto advance = [&](int &ti, int &sl, int &left, unsigned long long &rest) {
+    if (--left > 0) {
+      rest &= rest - 1ull;
+      if (++ti == ntaps) {  // slab outer, tap inner (see k_conv_mfma)
+        ti = 0;
+        sl++;
+        rest = tmask;
+      }
+    }
+  };
+  // Neighbour rows of the iteration at the rows' cursor, read from LDS one call ahead of their use.
+  int j_pre[RG];
+  auto prefetch_j = [&]() {
+    const int k = tap_at(a_ti, a_rest);
+#pragma unroll
+    for (int q = 0; q < RG; q++) j_pre[q] = jtab[((wave * RG + q) * K + k) * 16 + ld_row];
+  };
+  // (Past the end the loads ask for an offset outside their buffer, which the hardware answers with
+  // zeros without touching memory: a strided table's tiles have one or two iterations, and re-reading
+  // operands three times over would double their traffic.)
+  const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(wp), 0, (int)min((int64_t)K * n_slab * SLAB_STRIDE_F4 * 16, (int64_t)0x7FFFFFFF), 0x00020000);
+  auto issue_w = [&]() {
+    const int sl = w_sl;
+    const bool live = w_left > 0;
     // LDS values every lane reads alike: tell the compiler, so that what follows from them
     // (weight address, branches on the granule mask) is scalar work
-    const int k = __builtin_amdgcn_readfirstlane(taplist[nx_ti]);
-    if (++nx_ti == ntaps) {  // slab outer, tap inner (see k_conv_mfma)
-      nx_ti = 0;
-      nx_sl++;
-    }
-    gm_nxt = __builtin_amdgcn_readfirstlane(gmask[k]);
-    sl_nxt = sl;
-    ok_nxt = 0;
+    const int k = tap_at(w_ti, w_rest);
+    advance(w_ti, w_sl, w_left, w_rest);
     if (PRE) {
 #pragma unroll
       for (int s = 0; s < SS; s++) {
@@ -110,58 +146,84 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
         psh[s] = *reinterpret_cast<const v4f *>(pre_sh + (sl * SS + s) * 16 + 4 * ld_g);
       }
     }
-    const v4f *wsrc = reinterpret_cast<const v4f *>(wp) + ((int64_t)k * n_slab + sl) * SLAB_STRIDE_F4;
+    // The slab's byte offset goes in the scalar operand, the lane's part in the vector operand; only
+    // the vector operand is checked against the buffer's size, so that is where "past the end" goes.
+    const unsigned sbase = (unsigned)(k * n_slab + sl) * (unsigned)(SLAB_STRIDE_F4 * 16);
 #pragma unroll
     for (int i = 0; i < WPT; i++) {
       const int e = threadIdx.x + i * NT;
-      wreg[i] = wsrc[e < SLAB_F4 ? e : 0];
+      const unsigned voff = live ? (unsigned)(e < SLAB_F4 ? e : 0) * 16u : 0x80000000u;
+      wreg[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, voff, sbase, 0));
     }
+  };
+  auto issue_a = [&](auto stage_c) {
+    constexpr int S = decltype(stage_c)::value;
+    const int sl = a_sl;
+    const bool live = a_left > 0;
+    const int k = tap_at(a_ti, a_rest);
+    advance(a_ti, a_sl, a_left, a_rest);
+    // bit q: granule q of this wavefront has the tap
+    if (small_k) {
+      gm_ring[S] = 0u;
+#pragma unroll
+      for (int q = 0; q < RG; q++) gm_ring[S] |= (unsigned)((mym[q] >> k) & 1ull) << q;
+    } else {
+      gm_ring[S] = (__builtin_amdgcn_readfirstlane(gmask[k]) >> (wave * RG)) & ((1u << RG) - 1u);
+    }
+    sl_ring[S] = sl;
+    ok_ring[S] = 0;
+    int jq[RG];
+#pragma unroll
+    for (int q = 0; q < RG; q++) jq[q] = j_pre[q];
+    prefetch_j();  // for the next call
 #pragma unroll
     for (int q = 0; q < RG; q++) {
-      const int j = jtab[((wave * RG + q) * K + k) * 16 + ld_row];
+      const int j = jq[q];
       if constexpr (BUF) {
         // Buffer loads return zeros past the end of the buffer: an absent row becomes an
         // offset of 2 GiB (the launcher only takes this path for smaller inputs, whole slabs
         // and fewer than 2^24 rows), so no select is needed afterwards and the address is
         // one 24-bit multiply-add.
-        const unsigned voff = j >= 0 ? __umul24((unsigned)j, row_bytes) + lane_off : 0x80000000u;
-        if (PRE && j >= 0) ok_nxt |= 1u << q;  // zero must stay zero through the pre-activation
+        const unsigned voff = (j >= 0 && live) ? __umul24((unsigned)j, row_bytes) + lane_off : 0x80000000u;
+        if (PRE && j >= 0) ok_ring[S] |= 1u << q;  // zero must stay zero through the pre-activation
 #pragma unroll
         for (int s = 0; s < SS; s++)
-          a_nxt[q][s] = __builtin_bit_cast(
+          a_ring[S][q][s] = __builtin_bit_cast(
               v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, (sl * SS + s) * 64, 0));
         continue;
       }
-      if (j >= 0) ok_nxt |= 1u << q;
+      if (j >= 0) ok_ring[S] |= 1u << q;
       const float *src = in + (int64_t)(j < 0 ? 0 : j) * n_in;
 #pragma unroll
       for (int s = 0; s < SS; s++) {
         const int c0 = (sl * SS + s) * 16 + 4 * g;
         if (VEC4) {
           const int cc = c0 < n_in ? c0 : n_in - 4;
-          a_nxt[q][s] = *reinterpret_cast<const v4f *>(src + cc);
+          a_ring[S][q][s] = *reinterpret_cast<const v4f *>(src + cc);
         } else {
-          a_nxt[q][s].x = src[min(c0 + 0, n_in - 1)];
-          a_nxt[q][s].y = src[min(c0 + 1, n_in - 1)];
-          a_nxt[q][s].z = src[min(c0 + 2, n_in - 1)];
-          a_nxt[q][s].w = src[min(c0 + 3, n_in - 1)];
+          a_ring[S][q][s].x = src[min(c0 + 0, n_in - 1)];
+          a_ring[S][q][s].y = src[min(c0 + 1, n_in - 1)];
+          a_ring[S][q][s].z = src[min(c0 + 2, n_in - 1)];
+          a_ring[S][q][s].w = src[min(c0 + 3, n_in - 1)];
         }
       }
     }
   };
 
-  if (total > 0) issue(0);
-  for (int it = 0; it < total; it++) {
+  // One iteration: the weights of `it` go to LDS, its rows (ring set S) to the operand registers,
+  // then the loads of the iterations ahead are issued and the MFMAs run.
+  auto iterate = [&](int it, auto stage_c) {
+    constexpr int S = decltype(stage_c)::value;
     v4f *wb = wbuf + (it & 1) * LDS_SLAB_F4;
 #pragma unroll
     for (int i = 0; i < WPT; i++) wb[threadIdx.x + i * NT] = wreg[i];
 #pragma unroll
     for (int q = 0; q < RG; q++) {
-      const bool ok = (ok_nxt >> q) & 1u;
+      const bool ok = (ok_ring[S] >> q) & 1u;
       if constexpr (BF16) {
 #pragma unroll
         for (int s = 0; s < SS; s += 2) {
-          v4f v0 = a_nxt[q][s], v1 = a_nxt[q][s + 1];
+          v4f v0 = a_ring[S][q][s], v1 = a_ring[S][q][s + 1];
           if constexpr (PRE) {
             v0 = pre_act<PRE>(v0, psc[s], psh[s], pre_leak);
             v1 = pre_act<PRE>(v1, psc[s + 1], psh[s + 1], pre_leak);
@@ -175,17 +237,17 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
 #pragma unroll
       for (int s = 0; s < SS; s++) {
         if constexpr (BUF && !PRE && !BF16) {
-          a_cur[q][s] = to_operand_lanes(a_nxt[q][s]);
+          a_cur[q][s] = to_operand_lanes(a_ring[S][q][s]);
           continue;
         }
         if constexpr (BUF && PRE && !BF16) {
-          const v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
+          const v4f v = pre_act<PRE>(a_ring[S][q][s], psc[s], psh[s], pre_leak);
           a_cur[q][s] = to_operand_lanes(ok ? v : (v4f){0.f, 0.f, 0.f, 0.f});
           continue;
         }
         if constexpr (!BUF) {
-          const int c0 = (sl_nxt * SS + s) * 16 + 4 * g;
-          v4f v = pre_act<PRE>(a_nxt[q][s], psc[s], psh[s], pre_leak);
+          const int c0 = (sl_ring[S] * SS + s) * 16 + 4 * g;
+          v4f v = pre_act<PRE>(a_ring[S][q][s], psc[s], psh[s], pre_leak);
           if (VEC4) {
             if (!(ok && c0 < n_in)) v = (v4f){0.f, 0.f, 0.f, 0.f};
           } else {
@@ -198,10 +260,11 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
         }
       }
     }
-    gm_cur = gm_nxt;
+    gm_cur = gm_ring[S];
     __syncthreads();  // slab of `it` visible; every wavefront is done with the other buffer
-    if (it + 1 < total) issue(it + 1);
-    if (((gm_cur >> (wave * RG)) & ((1u << RG) - 1u)) == 0u) continue;  // none of my granules has the tap
+    issue_w();
+    issue_a(stage_c);
+    if (gm_cur == 0u) return;  // none of my granules has the tap
 #pragma unroll
     for (int s = 0; s < WS; s++) {
       v4f b[NCB];
@@ -209,7 +272,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
       for (int cb = 0; cb < NCB; cb++) b[cb] = wb[(s * NCB + cb) * 64 + lane];
 #pragma unroll
       for (int q = 0; q < RG; q++) {
-        if (!((gm_cur >> (wave * RG + q)) & 1u)) continue;  // uniform over the wavefront
+        if (!((gm_cur >> q) & 1u)) continue;  // uniform over the wavefront
         if constexpr (BF16) {
 #pragma unroll
           for (int cb = 0; cb < NCB; cb++)
@@ -227,8 +290,25 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
         }
       }
     }
-  }
+  };
 
+  static_assert(AD == 1 || AD == 3, "the loop is unrolled for a ring of one or three");
+  if (total > 0) {
+    prefetch_j();
+    issue_a(std::integral_constant<int, 0>{});
+    if constexpr (AD == 3) {
+      issue_a(std::integral_constant<int, 1>{});
+      issue_a(std::integral_constant<int, 2>{});
+    }
+    issue_w();
+  }
+  for (int it = 0; it < total; it += AD) {
+    iterate(it, std::integral_constant<int, 0>{});
+    if constexpr (AD == 3) {
+      if (it + 1 < total) iterate(it + 1, std::integral_constant<int, 1>{});
+      if (it + 2 < total) iterate(it + 2, std::integral_constant<int, 2>{});
+    }
+  }
   if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
     float *pt = partial + ((int64_t)blockIdx.y * n_tiles * TM + tbase) * (NCB * 16);
 #pragma unroll
@@ -310,11 +390,9 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   float *partial = scratch_partial(m, n_split, split_stride);
   kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), NT, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4), dbg_prio());
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
-  if (n_split > 1) {
-    launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
-  }
+  if (n_split > 1) launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
   return true;
 }
 
@@ -331,15 +409,14 @@ static bool dispatch_rows(Metadata &m, const Table &t, const float *in, float *o
   // 60 k sites is 480 such workgroups for 256 CUs: one wavefront per SIMD, nothing to run while
   // it waits for its gathers).  Measured: 13-18 % faster at 62 k sites, 5 % at 15 k and 250 k,
   // equal at 1 M except for 64 output planes, which gain 2 % there too.
+  // 128 output planes on a level of a few thousand to a few ten thousand sites: slabs of 64 input
+  // channels halve the number of iterations (and barriers) of every tile; with one or two
+  // workgroups per CU that is what counts (measured at 14 k sites: 128 -> 128 134 -> 110 us,
+  // 256 -> 128 245 -> 192 us; no gain at 60 k and 250 k sites, where the larger slab costs a
+  // resident workgroup per CU).
   if constexpr (VEC4) {
-    static const int dss = getenv("SCN_DBG_SS") ? atoi(getenv("SCN_DBG_SS")) : 0;
-    if (!narrow && ncb > 2 && (t.n < 300000 || ncb <= 4) && dss && n_in % (16 * dss) == 0) {
-#define SCN_TRY(N, S) if (ncb <= N && dss == S) return launch_rows<N, 1, S, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-      SCN_TRY(4, 4) SCN_TRY(4, 3) SCN_TRY(4, 6)
-      SCN_TRY(6, 4) SCN_TRY(6, 3) SCN_TRY(6, 6)
-      SCN_TRY(8, 4) SCN_TRY(8, 3)
-#undef SCN_TRY
-    }
+    if (!narrow && ncb > 6 && ncb <= 8 && t.n < 30000 && n_in % 64 == 0)
+      return launch_rows<8, 1, 4, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
   }
   if (!narrow && ncb > 2 && (t.n < 300000 || ncb <= 4)) {
     if (ncb <= 4) return launch_rows<4, 1, 2, VEC4, 4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);

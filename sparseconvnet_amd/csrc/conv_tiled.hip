@@ -2,17 +2,6 @@
 #include "conv_common.h"
 
 namespace scn {
-#ifdef SCN_PHASES
-__device__ unsigned long long g_phase[16 * 8];
-#define PHASE(i) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 16) g_phase[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define PHASE(i)
-#endif
-
-static int dbg_prio() {
-  static const int v = getenv("SCN_DBG_PRIO") ? atoi(getenv("SCN_DBG_PRIO")) : 0;
-  return v;
-}
 
 // ---- MFMA kernel ------------------------------------------------------------------------
 // A workgroup of 4 wavefronts owns a tile of G = GW*WR granules (16 rows each).  The
@@ -36,7 +25,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
     int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
-    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes, int prio) {
+    const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
   constexpr int WR = 4 / WC;
@@ -62,23 +51,15 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   const int wr = wave / WC, wc = wave % WC;
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of
-  // tiles so that neighbouring tiles (which gather the same rows) share one L2.
-  PHASE(0);
+  // tiles so that neighbouring tiles (which gather the same rows) share one L2.  Small levels
+  // (tiles_per_xcd == 0, Table::spread) list their tiles most expensive first: workgroup i takes
+  // tile i, so that the long tiles start first and on different CUs.
   const int tile = tiles_per_xcd ? (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3) : blockIdx.x;
   if (tile >= n_tiles) return;  // whole workgroup leaves: no barrier is skipped
   const int64_t tbase = (int64_t)tile * TM;
 
   const int ntaps = tile_setup<256, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
-  PHASE(1);
   const int total = ntaps * n_slab;
-  PHASE(2);
-  if (prio) {
-    const int q = ntaps * 4 / (K + 1);
-    if (q >= 3) __builtin_amdgcn_s_setprio(3);
-    else if (q == 2) __builtin_amdgcn_s_setprio(2);
-    else if (q == 1) __builtin_amdgcn_s_setprio(1);
-  }
-
   v4f acc[GW][NCBW];
 #pragma unroll
   for (int q = 0; q < GW; q++)
@@ -229,13 +210,10 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   };
 
   if (total > 0) issue(0, std::integral_constant<int, 0>{});
-  PHASE(3);
   for (int it = 0; it < total; it += 2) {
     iterate(it, std::integral_constant<int, 0>{});
-    if (it == 0) PHASE(4);
     if (it + 1 < total) iterate(it + 1, std::integral_constant<int, 1>{});
   }
-  PHASE(5);
 
   // acc[q][c][r] = result for position tbase + 16*(wr*GW+q) + 4*g + r, column 16*(wc*NCBW+c) + r16
   if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
@@ -247,7 +225,6 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 #pragma unroll
         for (int c = 0; c < NCBW; c++)
           pt[(int64_t)((wr * GW + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * (wc * NCBW + c) + r16] = acc[q][c][r];
-    PHASE(6);
     return;
   }
   float bv[NCBW], es[NCBW], eh[NCBW];
@@ -316,11 +293,9 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   float *partial = scratch_partial(m, n_split, split_stride);
   kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), 256, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4), dbg_prio());
+      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
-  if (n_split > 1) {
-    launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
-  }
+  if (n_split > 1) launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
   return true;
 }
 
@@ -338,22 +313,6 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
   // Levels of a few thousand sites: 64-row tiles instead of 128-row ones give the chip twice the
   // workgroups to spread (measured: 12-23 % faster at 16 k sites, 10 % at 1 k, 30 % at 250,
   // equal at 4 k, where the tap split halves in exchange).
-  if constexpr (VEC4) {
-    static const int dss = getenv("SCN_DBG_TSS") ? atoi(getenv("SCN_DBG_TSS")) : 0;
-    if (!narrow && t.n < 30000 && ncb > 8 && (dss == 2 || dss == 4)) {
-      if (dss == 2) {
-        if (ncb <= 10) return launch_mfma<5, 2, 2, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-        if (ncb <= 12) return launch_mfma<3, 4, 4, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-        if (ncb <= 14) return launch_mfma<7, 2, 2, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-        if (ncb <= 16) return launch_mfma<4, 4, 4, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-      } else {
-        if (ncb <= 10) return launch_mfma<5, 2, 2, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-        if (ncb <= 12) return launch_mfma<3, 4, 4, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-        if (ncb <= 14) return launch_mfma<7, 2, 2, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-        if (ncb <= 16) return launch_mfma<4, 4, 4, 4, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
-      }
-    }
-  }
   if (!narrow && t.n < 30000 && ncb > 8) {
     if (ncb <= 10) return launch_mfma<5, 2, 2, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     if (ncb <= 12) return launch_mfma<3, 4, 4, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
@@ -384,9 +343,4 @@ bool conv_tiled_dispatch(bool vec4, bool pre_fused, Metadata &m, const Table &t,
               : dispatch_ncb<false, false>(ncb, m, t, in, out, w, epi, n_in, n_out, pre, s);
 }
 
-#ifdef SCN_PHASES
-extern "C" int scn_dbg_phases(unsigned long long *out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_phase), sizeof(g_phase));
-}
-#endif
 }  // namespace scn

@@ -765,6 +765,14 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
 // measured on room scenes of 60k..4M sites, 8 or 16 ranges beat both 256-position blocks
 // (by 20-30% for 64..256 channels) and one global sort (which loses the locality).
 static const int PATTERN_WINDOWS = 8;
+// Below this many positions the sort runs over the whole table (Table::spread).  A level of
+// 250 k sites or fewer is a few waves of workgroups: what decides a kernel's duration there is how
+// evenly the expensive tiles (those with the most taps) are spread over the CUs and how early they
+// start, not L2 locality.  One window puts them first, kernels then deal tiles to workgroups in
+// turn; it also wastes fewer MFMAs on 16-row granules of mixed patterns (13 % -> 5 % at 60 k sites,
+// 37 % -> 17 % at 14 k).  Measured on the room scene: convolutions 9 % faster at 247 k sites, 19 %
+// at 61 k, 9 % at 14 k; at a million sites one window is slower.
+static const int64_t PATTERN_WHOLE_BELOW = 300000;
 
 // Sort key of a position: window, then the number of absent taps (shifted right by pc_shift
 // when the key bits are short), then the tap mask, or, when the mask has more than code_bits
@@ -865,8 +873,7 @@ __global__ void k_copy_rowmap(const int *base, int64_t n, int *rowmap) {
 static PatternKey pattern_plan(int64_t n, int K, int &key_bits) {
   PatternKey p;
   p.K = K;
-  static const int64_t gsort = getenv("SCN_DBG_GSORT") ? atoll(getenv("SCN_DBG_GSORT")) : 0;
-  p.window = std::max<int64_t>(256, round_up(ceil_div(n, n < gsort ? 1 : PATTERN_WINDOWS), 256));
+  p.window = std::max<int64_t>(256, round_up(ceil_div(n, n < PATTERN_WHOLE_BELOW ? 1 : PATTERN_WINDOWS), 256));
   int block_bits = 0;
   while (((int64_t)1 << block_bits) < ceil_div(n, p.window)) block_bits++;
   int pc_bits = 1;
