@@ -210,6 +210,9 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
             torch.cuda.synchronize()
         graph_ms = med(reps_ms) if same else None
         del graph
+    layers = None
+    if batch == 1 and not residual:
+        layers = unet_layer_table(torch, scn, model, x)
     # device memory the library itself holds (rulebooks of the live handles, scratch, idle blocks of
     # its cache; features and weights are torch's): high-water mark since the process started
     import ctypes
@@ -223,7 +226,8 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
     if residual:
         return {"unet_residual_ms_per_scene": med(cold), "unet_residual_warm_ms": med(warm),
                 "unet_residual_gflop": round(2 * macs / 1e9, 2)}
-    return {"unet_ms_per_scene": med(cold), "unet_ms_per_scene_from_host_coords": med(cold_host),
+    return {"unet_layers": layers, "unet_conv_ms_sum": round(sum(r["ms"] for r in layers), 4),
+            "unet_ms_per_scene": med(cold), "unet_ms_per_scene_from_host_coords": med(cold_host),
             "unet_warm_ms": med(warm), "unet_warm_graph_replay_ms": graph_ms, "unet_points": int(len(coords)), "unet_active_sites": int(x.features.shape[0]),
             "unet_gflop": round(2 * macs / 1e9, 2), "library_peak_MiB": round(peak.value / 2 ** 20),
             "unet_warm_gflops": round(2 * macs / (float(np.median(warm)) * 1e-3) / 1e9, 1),
@@ -232,6 +236,49 @@ def unet_scene(sites, seed, reps=7, residual=False, batch=1):
                     "resident in HBM; from_host_coords: the same with the coordinates handed over as a CPU "
                     "LongTensor (host-to-device copy inside the timed region); warm: rulebooks cached; "
                     "warm_graph_replay: the warm pass replayed as one HIP graph (null if the replay's result differed)"}
+
+
+def unet_layer_table(torch, scn, model, x, reps=5):
+    """Every convolution of one warm U-Net pass, in call order: HIP events on the launch stream
+    around each call (median of `reps` passes), the kernel the library chose, the layer's
+    multiply-adds as the reference counts them and its roofline (fp32 MFMA peak or HBM,
+    whichever bounds the layer)."""
+    from sparseconvnet_amd import metadata as M
+    recs = []
+    orig = M.Metadata._conv
+
+    def timed_conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out, macs = orig(self, kind, size_args, n_rows, features, weight, bias, bn, post, True)
+        e1.record()
+        kernel = self._L.scn_md_last_conv_kernel(self._h).decode()
+        recs.append((kind, features.shape[0], n_rows, weight.shape[0], weight.shape[1] * weight.shape[2],
+                     weight.shape[1] * weight.shape[3], macs, bn is not None, post is not None, kernel, e0, e1))
+        return out, (macs if want_macs else None)
+    M.Metadata._conv = timed_conv
+    passes = []
+    try:
+        with torch.no_grad():
+            for _ in range(reps + 1):
+                recs.clear()
+                model(x)
+                torch.cuda.synchronize()
+                passes.append([r[-2].elapsed_time(r[-1]) for r in recs])
+    finally:
+        M.Metadata._conv = orig
+    ms = np.median(np.array(passes[1:]), axis=0)
+    rows = []
+    for r, t in zip(recs, ms):
+        kind, n_in_rows, n_out_rows, K, cin, cout, macs, pre, post, kernel = r[:10]
+        R = macs / (cin * cout)
+        rows.append({"op": ("SubmanifoldConvolution", "Convolution", "Deconvolution")[kind],
+                     "rows_in": int(n_in_rows), "rows_out": int(n_out_rows), "taps": int(K), "rules": int(R),
+                     "nIn": int(cin), "nOut": int(cout), "bn_in_front": bool(pre), "bn_behind": bool(post),
+                     "kernel": kernel, "ms": round(float(t), 4),
+                     "tflops": round(2.0 * macs / (float(t) * 1e-3) / 1e12, 2),
+                     "roofline": roofline_for(cin, cout, R, n_out_rows, K, float(t))})
+    return rows
 
 
 def unet_train_step(sites, seed, reps=3):

@@ -65,6 +65,10 @@ int scn_set_build_stream(int enable);
  * fp32.  Results then agree with the fp32 path to about 1e-2 relative to the output scale.
  * Off by default. */
 int scn_md_set_bf16(scn_metadata *md, int enable);
+/* No counterpart in the reference: the kernel the handle's last convolution call ran, as text
+ * (family and tile shape, e.g. "rows ncb=6 rg=1 ss=2 nw=4 split=1"), for benchmark tables and
+ * profiles.  The pointer stays valid until the handle's next convolution call. */
+const char *scn_md_last_conv_kernel(scn_metadata *md);
 /* Metadata::inputLayer (Metadata/Metadata.cpp:413-425, Metadata/IOLayersRules.h:18-121).
  * coords: device int64 [n, ncols], ncols = dim (one sample) or dim+1 (last column = sample
  * index).  mode 0: rows = input order, no merging; 1: first, 2: last, 3: sum, 4: mean of the

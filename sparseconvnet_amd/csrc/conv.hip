@@ -275,6 +275,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   } frozen_reset{m};
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
+  m.last_kernel.clear();
   if (t.n == 0) return;
   if (m.fixed_scratch && (bn || post || groups != 1))
     throw Error("allocation-free convolution: plain convolutions with groups = 1 only");
@@ -352,6 +353,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
       if (e.sc) e.sc += c0, e.sh += c0;
       e.out_stride = n_out;
       ok = conv_mfma_paths<false>(m, t, src, out + c0, dst, e, n_in, wc, PreArgs(), s);
+      m.last_kernel += " +";  // the next range's kernel is appended
     }
     if (ok) return;
   }
@@ -360,6 +362,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     LAUNCH_CHECK();
   }
   int64_t total = t.n * n_out;
+  note_kernel(m, "generic", {{"groups", groups}});
   k_conv_generic<<<dim3((unsigned)ceil_div(total, 256)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, src,
                                                                        out, w, epi, n_in, n_out, groups);
   LAUNCH_CHECK();

@@ -79,6 +79,31 @@ static inline CoefJobs take_jobs(Metadata &m) {
 constexpr int packed_slab_floats(int SS, int NCB) { return (SS * NCB * 64 + 255) / 256 * 256 * 4; }
 
 
+// Profiling build (-DSCN_PHASES, see build.py's SCN_EXTRA_FLAGS): thread 0 of every 16th workgroup
+// of a tiled kernel stamps the 100 MHz wall clock at up to seven points of its life into its
+// translation unit's g_phase_stamps; slot 7 holds the tile's iteration count.  SCN_PHASE_EXPORT(name)
+// defines the extern "C" function that copies the stamps to the host.  Compiled out otherwise.
+#ifdef SCN_PHASES
+static __device__ unsigned long long g_phase_stamps[64 * 8];
+#define SCN_PHASE_SLOT() (blockIdx.y == 0 && (blockIdx.x % 16) == 0 && blockIdx.x / 16 < 64 && threadIdx.x == 0)
+#define SCN_PHASE(i) do { if (SCN_PHASE_SLOT()) g_phase_stamps[(blockIdx.x / 16) * 8 + (i)] = wall_clock64(); } while (0)
+#define SCN_PHASE_VALUE(i, v) do { if (SCN_PHASE_SLOT()) g_phase_stamps[(blockIdx.x / 16) * 8 + (i)] = (unsigned long long)(v); } while (0)
+#define SCN_PHASE_EXPORT(name) \
+  extern "C" int name(unsigned long long *out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_phase_stamps), sizeof(g_phase_stamps)); }
+#else
+#define SCN_PHASE(i)
+#define SCN_PHASE_VALUE(i, v)
+#define SCN_PHASE_EXPORT(name)
+#endif
+
+// Notes the kernel a convolution call launches (Metadata::last_kernel).
+inline void note_kernel(Metadata &m, const char *family, std::initializer_list<std::pair<const char *, int>> params) {
+  std::string t = family;
+  for (auto &p : params) t += std::string(" ") + p.first + "=" + std::to_string(p.second);
+  if (!m.last_kernel.empty() && m.last_kernel.back() == '+') m.last_kernel += " " + t;  // column ranges, channel parts
+  else m.last_kernel = t;
+}
+
 struct PreArgs {  // device pointers to the padded coefficient arrays, or nulls
   const float *sc = nullptr, *sh = nullptr;
   float leak = 1.0f;

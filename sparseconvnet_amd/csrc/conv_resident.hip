@@ -360,6 +360,7 @@ static void launch_resident_kernel(Metadata &m, const Table &t, const float *in,
   const int n_sets = (int)ceil_div(t.n, RG * 16);
   const int sets_per_xcd = (int)ceil_div(n_sets, 8);
   const int blocks = 8 * (int)std::max<int64_t>(1, std::min<int64_t>(32 * per_cu, ceil_div(sets_per_xcd, WAVES)));
+  note_kernel(m, BF16 ? "resident-bf16" : (C4 ? "resident-c4" : "resident"), {{"ncb", NCB}, {"rg", RG}, {"ss", SS}, {"waves", WAVES}});
   kern<<<dim3(blocks), WAVES * 64, lds_bytes, s>>>(t.nbr.p, t.rowmap_ptr(), t.gmask.p, t.K, t.n, t.npad, in, in_stride,
                                                    out, wpack, epi, n_in_part, n_out, n_sets, sets_per_xcd,
                                                    accumulate, scratch_queue(m, s), (unsigned)in_bytes, (unsigned)nbr_bytes, t.spread ? 1 : 0);
@@ -422,6 +423,7 @@ static void launch_resident_c4(Metadata &m, const Table &t, const float *in, flo
   if (in == m.cur_in_base && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
     // epi.sc / epi.sh point at arrays nobody fills on this path: the kernel folds the batch norm itself
     take_jobs(m);
+    note_kernel(m, "first", {{"nin", n_in}});
     conv_first_forward(t, in, m.cur_in_rows, out, w, epi.bias, m.post_raw, epi.leak, n_in, n_out, s);
     return;
   }

@@ -37,12 +37,15 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
 
+  SCN_PHASE(0);  // start
   const int tile = tiles_per_xcd ? (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3) : blockIdx.x;
   if (tile >= n_tiles) return;
   const int64_t tbase = (int64_t)tile * TM;
 
   const int ntaps = tile_setup<NT, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
   const int total = ntaps * n_slab;
+  SCN_PHASE(1);  // tile set up
+  SCN_PHASE_VALUE(7, total);
   // Filters of up to 64 taps: the tap list and the taps of this wavefront's granules as bit masks in
   // scalar registers, so that the tap of an iteration and whether a granule has it are scalar
   // arithmetic instead of LDS reads on the path from the barrier to the first MFMA.
@@ -302,13 +305,16 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     }
     issue_w();
   }
+  SCN_PHASE(2);  // first loads issued
   for (int it = 0; it < total; it += AD) {
     iterate(it, std::integral_constant<int, 0>{});
+    if (it == 0) SCN_PHASE(3);  // first iteration done
     if constexpr (AD == 3) {
       if (it + 1 < total) iterate(it + 1, std::integral_constant<int, 1>{});
       if (it + 2 < total) iterate(it + 2, std::integral_constant<int, 2>{});
     }
   }
+  SCN_PHASE(4);  // tap loop done
   if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
     float *pt = partial + ((int64_t)blockIdx.y * n_tiles * TM + tbase) * (NCB * 16);
 #pragma unroll
@@ -346,6 +352,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
       }
     }
   }
+  SCN_PHASE(5);  // rows stored
 }
 
 template <int NCB, int RG, int SS, bool VEC4, int NW, bool PRE, bool BUF = false, bool BF16 = false>
@@ -388,6 +395,7 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
   float *partial = scratch_partial(m, n_split, split_stride);
+  note_kernel(m, BF16 ? "rows-bf16" : "rows", {{"ncb", NCB}, {"rg", RG}, {"ss", SS}, {"nw", NW}, {"pre", PRE}, {"split", n_split}});
   kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), NT, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
       n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
@@ -444,5 +452,7 @@ bool conv_rows_dispatch(bool vec4, bool pre_fused, Metadata &m, const Table &t, 
   return vec4 ? dispatch_rows<true, false>(m, t, in, out, w, epi, n_in, n_out, pre, s)
               : dispatch_rows<false, false>(m, t, in, out, w, epi, n_in, n_out, pre, s);
 }
+
+SCN_PHASE_EXPORT(scn_dbg_phases_rows)
 
 }  // namespace scn

@@ -291,6 +291,7 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
   float *partial = scratch_partial(m, n_split, split_stride);
+  note_kernel(m, BF16 ? "tiled-bf16" : "tiled", {{"ncbw", NCBW}, {"wc", WC}, {"gw", GW}, {"ss", SS}, {"pre", PRE}, {"split", n_split}});
   kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), 256, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
       n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));

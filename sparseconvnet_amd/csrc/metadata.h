@@ -213,6 +213,7 @@ struct Metadata {
   // inputs) round their operands to bf16 and run the bf16 MFMA with fp32 accumulation when the
   // input consists of whole 32-channel slabs; off unless the caller asks for it.
   bool bf16 = false;
+  std::string last_kernel;  // what the last convolution call launched (scn_md_last_conv_kernel)
   // Ordering between the stream rulebooks are built on and the stream the caller's feature
   // passes run on (api.hip: BuildScope, consume).
   uint64_t builds = 0;              // bumped by every construction that enqueued work

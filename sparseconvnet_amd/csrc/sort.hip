@@ -23,10 +23,11 @@
 namespace scn {
 
 typedef unsigned long long u64;
-constexpr int RS_THREADS = 256, RS_WAVES = 4, RS_ITEMS = 8, RS_TILE = RS_THREADS * RS_ITEMS;  // 2048 pairs per tile
+constexpr int RS_THREADS = 256, RS_WAVES = 4;  // a tile is RS_THREADS * ITEMS pairs: 4096 (large inputs) or 2048
 constexpr int RS_MAX_BITS = 10, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured on a million
 // pairs of 35 bits: four digits of 9 bits beat three of 11 and five of 7; 40 bits sort in four digits of 10)
 
+template <int RS_ITEMS>
 __global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const u64 *__restrict__ keys, int64_t n, int shift, int bits,
                                                         int tiles, int *__restrict__ hist) {
   __shared__ int h[RS_MAX_BINS];
@@ -34,6 +35,7 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const u64 *__restrict__ 
   for (int d = threadIdx.x; d < bins; d += RS_THREADS) h[d] = 0;
   __syncthreads();
   const unsigned mask = (unsigned)bins - 1u;
+  constexpr int RS_TILE = RS_THREADS * RS_ITEMS;
   const int64_t base = (int64_t)blockIdx.x * RS_TILE;
 #pragma unroll
   for (int r = 0; r < RS_ITEMS; r++) {
@@ -90,20 +92,25 @@ __device__ inline void rank_quarter(const unsigned (&digit)[ITEMS], const bool (
   }
 }
 
+template <int RS_ITEMS>
 __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict__ kin, const int *__restrict__ vin,
                                                            u64 *__restrict__ kout, int *__restrict__ vout, int64_t n,
                                                            int shift, int bits, int tiles, const int *__restrict__ offs,
                                                            const int *__restrict__ tot) {
+  constexpr int RS_TILE = RS_THREADS * RS_ITEMS;
   __shared__ int cnt[RS_WAVES][RS_MAX_BINS];
-  __shared__ int base[RS_MAX_BINS];  // where the tile's first pair of each digit value goes
-  __shared__ int wsum[RS_WAVES];
+  __shared__ int base[RS_MAX_BINS];    // where the tile's first pair of each digit value goes
+  __shared__ int lstart[RS_MAX_BINS];  // the same inside the tile: pairs of smaller digit values
+  __shared__ int wsum[RS_WAVES], wsum2[RS_WAVES];
+  __shared__ u64 skey[RS_TILE];        // the tile's pairs in the order they leave in
+  __shared__ int sval[RS_TILE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int bins = 1 << bits;
   const unsigned mask = (unsigned)bins - 1u;
+  const int per = (bins + RS_THREADS - 1) / RS_THREADS;  // digit values per thread, 1 to 4
+  const int d0 = threadIdx.x * per;
   // exclusive scan of the digit values' totals (thread t: values [t * per, (t + 1) * per)) + this tile's prefix
   {
-    const int per = (bins + RS_THREADS - 1) / RS_THREADS;  // 1 to 4
-    const int d0 = threadIdx.x * per;
     int mine = 0;
     for (int j = 0; j < per; j++)
       if (d0 + j < bins) mine += tot[d0 + j];
@@ -144,13 +151,51 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict
   }
   rank_quarter<RS_ITEMS>(digit, valid, bits, cnt[wave], lane, rank);
   __syncthreads();  // all four quarters counted, base[] written
+  // The tile's own exclusive prefix over digit values: a pair leaves the tile at lstart[d] + (pairs
+  // of the same value before it), so that what goes to consecutive addresses of the output sits
+  // at consecutive places of the tile and is written by consecutive lanes (a lane writing its own
+  // pair where it belongs touched one 32-byte sector per 8- or 4-byte store).
+  {
+    int mine = 0;
+    for (int j = 0; j < per; j++)
+      if (d0 + j < bins)
+        for (int w = 0; w < RS_WAVES; w++) mine += cnt[w][d0 + j];
+    int incl = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) wsum2[wave] = incl;
+    __syncthreads();
+    int run = incl - mine;
+    for (int w = 0; w < wave; w++) run += wsum2[w];
+    for (int j = 0; j < per; j++)
+      if (d0 + j < bins) {
+        lstart[d0 + j] = run;
+        for (int w = 0; w < RS_WAVES; w++) run += cnt[w][d0 + j];
+      }
+  }
+  __syncthreads();
 #pragma unroll
   for (int r = 0; r < RS_ITEMS; r++) {
     if (!valid[r]) continue;
-    int at = base[digit[r]] + rank[r];
+    int at = lstart[digit[r]] + rank[r];
     for (int w = 0; w < wave; w++) at += cnt[w][digit[r]];
-    kout[at] = key[r];
-    vout[at] = val[r];
+    skey[at] = key[r];
+    sval[at] = val[r];
+  }
+  __syncthreads();
+  const int64_t tile_n = min((int64_t)RS_TILE, n - (int64_t)blockIdx.x * RS_TILE);
+#pragma unroll
+  for (int r = 0; r < RS_ITEMS; r++) {
+    const int pos = r * RS_THREADS + threadIdx.x;
+    if (pos >= tile_n) continue;
+    const u64 k = skey[pos];
+    const unsigned d = (unsigned)(k >> shift) & mask;
+    const int at = base[d] + (pos - lstart[d]);
+    kout[at] = k;
+    vout[at] = sval[pos];
   }
 }
 
@@ -162,7 +207,12 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
   // as few digits as RS_MAX_BITS bits each allow, of equal width
   const int passes = (end_bit + RS_MAX_BITS - 1) / RS_MAX_BITS;
   const int width = (end_bit + passes - 1) / passes;
-  const int tiles = (int)ceil_div(n, RS_TILE);
+  // Large inputs take tiles of 4096 pairs (longer runs per digit value in the scatter's stores: a
+  // million pairs of 35 bits 145 -> 122 us, eight million 800 -> 490 us); below half a million pairs
+  // there are too few of those to fill the chip and 2048-pair tiles are faster.
+  const bool big = n >= 500000;
+  const int tile = RS_THREADS * (big ? 16 : 8);
+  const int tiles = (int)ceil_div(n, tile);
   // scratch: a second pair of arrays (when there is more than one pass), the tile counts, the totals
   const size_t kbytes = round_up((size_t)n * sizeof(u64), 256), vbytes = round_up((size_t)n * sizeof(int), 256);
   const size_t hbytes = round_up(((size_t)1 << width) * tiles * sizeof(int), 256);
@@ -184,11 +234,13 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
     u64 *kdst = to_out ? kout : ktmp;
     int *vdst = to_out ? vout : vtmp;
     const int shift = width * pass, bits = std::min(width, end_bit - shift);
-    k_rs_hist<<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist);
+    if (big) k_rs_hist<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist);
+    else k_rs_hist<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist);
     LAUNCH_CHECK();
     k_rs_colscan<<<dim3(1 << bits), 64, 0, s>>>(hist, tiles, tot);
     LAUNCH_CHECK();
-    k_rs_scatter<<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot);
+    if (big) k_rs_scatter<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot);
+    else k_rs_scatter<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot);
     LAUNCH_CHECK();
     ksrc = kdst;
     vsrc = vdst;
