@@ -79,6 +79,15 @@ const char *scn_md_last_conv_kernel(scn_metadata *md);
 int scn_md_input_layer(scn_metadata *md, const int64_t *spatial, const int64_t *coords,
                        int64_t n, int ncols, int min_batch, int mode, void *stream,
                        int64_t *n_active);
+/* The same with the coordinates in host memory, as the reference's InputLayer receives them (a CPU
+ * LongTensor, sparseconvnet/ioLayers.py:51-65; Metadata/Metadata.cpp:413-425 reads it on the host).
+ * coords: host int64 [n, ncols], pageable or pinned; it has been read completely when the call
+ * returns.  A few host threads narrow the values to int16 (grids of up to 32767 cells per
+ * dimension; int32 otherwise or when a value does not fit) into pinned memory and the pieces are
+ * copied while the next ones are narrowed: a quarter of the bytes of an int64 copy cross PCIe. */
+int scn_md_input_layer_host(scn_metadata *md, const int64_t *spatial, const int64_t *host_coords,
+                            int64_t n, int ncols, int min_batch, int mode, void *stream,
+                            int64_t *n_active);
 /* The point-at-a-time input of sparseconvnet/inputBatch.py, as one pass over everything the
  * caller collected: Metadata::setInputSpatialSize / batchAddSample / setInputSpatialLocation(s)
  * (Metadata/Metadata.cpp:74-147) with addPointToSparseGridMapAndFeatures (:29-46).  coords as

@@ -30,6 +30,7 @@ SIGNATURES = {
     "scn_md_set_bf16": (C.c_int, [_vp, C.c_int]),
     "scn_md_last_conv_kernel": (C.c_char_p, [_vp]),
     "scn_md_input_layer": (C.c_int, [_vp, _i64p, _vp, C.c_int64, C.c_int, C.c_int, C.c_int, _vp, _i64p]),
+    "scn_md_input_layer_host": (C.c_int, [_vp, _i64p, _vp, C.c_int64, C.c_int, C.c_int, C.c_int, _vp, _i64p]),
     "scn_md_input_rules_header": (C.c_int, [_vp, C.POINTER(C.c_int32)]),
     "scn_md_input_rules": (C.c_int, [_vp, _vp, _vp]),
     "scn_md_bl_input_layer": (C.c_int, [_vp, _i64p, _vp, C.c_int64, C.c_int64, C.c_int, _vp, _i64p]),

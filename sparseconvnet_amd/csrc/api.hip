@@ -524,7 +524,29 @@ int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *c
     Metadata &m = md(h);
     if (n < 0) throw Error("negative point count");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
-    build_input(m, stream, [&](hipStream_t s) { build_input_layer(m, spatial, coords, n, ncols, min_batch, mode, s); });
+    build_input(m, stream, [&](hipStream_t s) { build_input_layer(m, spatial, CoordSrc{coords, 8}, n, ncols, min_batch, mode, s); });
+    if (n_active) *n_active = m.input.n_out;
+  });
+}
+int scn_md_input_layer_host(scn_metadata *h, const int64_t *spatial, const int64_t *host_coords, int64_t n,
+                            int ncols, int min_batch, int mode, void *stream, int64_t *n_active) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (n < 0) throw Error("negative point count");
+    if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
+    bool allow16 = true;
+    for (int d = 0; d < m.dim; d++) allow16 = allow16 && spatial[d] <= 32767;
+    try {
+      build_input(m, stream, [&](hipStream_t s) {
+        const CoordSrc src = stage_host_coords(m, host_coords, n * ncols, s, allow16);
+        build_input_layer(m, spatial, src, n, ncols, min_batch, mode, s);
+      });
+    } catch (...) {
+      (void)hipDeviceSynchronize();  // copies out of the pinned block may still be under way
+      release_staging(m);
+      throw;
+    }
+    release_staging(m);
     if (n_active) *n_active = m.input.n_out;
   });
 }
@@ -536,7 +558,7 @@ int scn_md_input_batch(scn_metadata *h, const int64_t *spatial, const int64_t *c
     if (n < 0) throw Error("negative point count");
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
     build_input(m, stream, [&](hipStream_t s) {
-      build_input_layer(m, spatial, coords, n, ncols, min_batch, 5, s, 0, overwrite);  // `overwrite` is copied
+      build_input_layer(m, spatial, CoordSrc{coords, 8}, n, ncols, min_batch, 5, s, 0, overwrite);  // `overwrite` is copied
     });
     if (n_active) *n_active = m.input.n_out;
   });
@@ -566,7 +588,7 @@ int scn_md_bl_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t
     if (m.input.mode >= 0) throw Error("this metadata already has an input layer; call scn_md_clear first");
     if (batch * length == 0) length = 1, batch = 0;
     build_input(m, stream, [&](hipStream_t s) {
-      build_input_layer(m, spatial, coords, batch * length, m.dim, 0, mode, s, length);
+      build_input_layer(m, spatial, CoordSrc{coords, 8}, batch * length, m.dim, 0, mode, s, length);
     });
     if (n_active) *n_active = m.input.n_out;
   });

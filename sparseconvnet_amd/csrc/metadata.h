@@ -160,6 +160,18 @@ __device__ inline int listed_point(const int *sorted_idx, int st, int len, int m
   return sorted_idx[st];
 }
 
+// Where a construction reads the caller's coordinates: int64 as the caller holds them on the
+// device, or the int16 / int32 values host_input.hip narrowed them to on their way from the host.
+struct CoordSrc {
+  const void *p;
+  int width;  // bytes per value: 8, 4 or 2
+};
+__device__ inline int64_t coord_at(const CoordSrc &c, int64_t i) {
+  if (c.width == 8) return static_cast<const int64_t *>(c.p)[i];
+  if (c.width == 4) return static_cast<const int32_t *>(c.p)[i];
+  return static_cast<const int16_t *>(c.p)[i];
+}
+
 // Pinned host blocks from a process-wide list (api.hip).
 void *pinned_acquire(size_t bytes);
 void pinned_release(void *p, size_t bytes);
@@ -168,7 +180,15 @@ struct Metadata {
   Metadata() = default;
   Metadata(const Metadata &) = delete;
   Metadata &operator=(const Metadata &) = delete;
-  ~Metadata() { pinned_release(pinned, PINNED_WORDS * sizeof(int)); }
+  ~Metadata() {
+    pinned_release(pinned, PINNED_WORDS * sizeof(int));
+    if (staging) pinned_release(staging, staging_bytes);
+  }
+  // Coordinates that arrived in host memory: their narrowed copy on the device, and the pinned
+  // block the copy was made from until the stream has been waited for (host_input.hip).
+  DevBuf<unsigned char> hostcoords;
+  void *staging = nullptr;
+  size_t staging_bytes = 0;
   // Pinned host words that the constructions copy their sizes and flags into: a copy into
   // pageable memory would be staged and waited for by the runtime, one round trip per copy.
   static constexpr int PINNED_WORDS = 2048;
@@ -237,9 +257,12 @@ Geom make_geom(int dim, const int64_t *spatial);
 // first index and positions whose first coordinate is negative are empty.
 // mode 5 (point-at-a-time input, Metadata/Metadata.cpp:29-46 as one pass): overwrite[i] != 0 marks
 // points that replace what their site holds; NULL: none does.
-void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
+void build_input_layer(Metadata &m, const int64_t *spatial, CoordSrc coords, int64_t n,
                        int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length = 0,
                        const unsigned char *overwrite = nullptr);
+// host_input.hip
+CoordSrc stage_host_coords(Metadata &m, const int64_t *host, int64_t values, hipStream_t s, bool allow16);
+void release_staging(Metadata &m);
 void generate_rulebooks(Metadata &m, int size, hipStream_t s);
 void export_input_rules(Metadata &m, int *rows, hipStream_t s);
 int input_max_active(Metadata &m);  // longest run of points on one site (modes 3 and 4), fetched from the device on first use

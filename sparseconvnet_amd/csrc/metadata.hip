@@ -232,23 +232,23 @@ __device__ inline void grid_max(int v, int floor, int *slots) {
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
 // bl_len > 0: the sample of point i is i / bl_len and a negative first coordinate marks an
 // empty position (Metadata/IOLayersRules.h:183,204,234): key EMPTY, counted in flags[4].
-__global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols, int64_t bl_len,
+__global__ void k_input_keys(Geom g, CoordSrc coords, int64_t n, int ncols, int64_t bl_len,
                              unsigned long long *keys, int *idx, int *flags) {
   // flags[0]: error bits, flags[4]: empty positions, flags[8...]: slots of the largest sample index
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int bmax = 0;
   bool empty = false;
   if (i < n) {
-    const int64_t *c = coords + i * ncols;
+    const int64_t c0 = i * ncols;
     int cc[SCN_MAXD];
     bool ok = true;
-    empty = bl_len > 0 && c[0] < 0;
+    empty = bl_len > 0 && coord_at(coords, c0) < 0;
     for (int d = 0; d < g.dim; d++) {
-      int64_t v = c[d];
+      int64_t v = coord_at(coords, c0 + d);
       if (v < 0 || v >= g.size[d]) ok = false;
       cc[d] = (int)v;
     }
-    int64_t b = bl_len > 0 ? i / bl_len : (ncols > g.dim ? c[g.dim] : 0);
+    int64_t b = bl_len > 0 ? i / bl_len : (ncols > g.dim ? coord_at(coords, c0 + g.dim) : 0);
     if (b < 0 || b >= g.max_batch) {
       atomicOr(&flags[0], 2);
       ok = false;
@@ -271,13 +271,13 @@ __global__ void k_input_keys(Geom g, const int64_t *coords, int64_t n, int ncols
 }
 
 // mode 0: row = input index.
-__global__ void k_input_rows_identity(Geom g, const int64_t *coords, int64_t n, int ncols, int64_t bl_len,
+__global__ void k_input_rows_identity(Geom g, CoordSrc coords, int64_t n, int ncols, int64_t bl_len,
                                       int64_t npad, int *soa) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const int64_t *c = coords + i * ncols;
-  for (int d = 0; d < g.dim; d++) soa[d * npad + i] = (int)c[d];
-  soa[g.dim * npad + i] = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)c[g.dim] : 0);
+  const int64_t c0 = i * ncols;
+  for (int d = 0; d < g.dim; d++) soa[d * npad + i] = (int)coord_at(coords, c0 + d);
+  soa[g.dim * npad + i] = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)coord_at(coords, c0 + g.dim) : 0);
 }
 
 // After the stable sort: head[p] marks the first point of each group of equal keys;
@@ -310,19 +310,19 @@ __global__ void k_assign_groups(const int *sidx, const int *head, const int *hea
 }
 // ... and one over the points in input order for what is indexed by row: coordinates and key
 // of every first occurrence.
-__global__ void k_assign_coords(Geom g, const int64_t *coords, int ncols, int64_t bl_len, const int *is_first,
+__global__ void k_assign_coords(Geom g, CoordSrc coords, int ncols, int64_t bl_len, const int *is_first,
                                 const int *first_scan, int64_t n, int64_t npad, int *soa,
                                 unsigned long long *level_keys) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n || !is_first[i]) return;
   const int row = first_scan[i];
-  const int64_t *c = coords + i * ncols;
+  const int64_t c0 = i * ncols;
   int cc[SCN_MAXD];
   for (int d = 0; d < g.dim; d++) {
-    cc[d] = (int)c[d];
+    cc[d] = (int)coord_at(coords, c0 + d);
     soa[d * npad + row] = cc[d];
   }
-  const int b = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)c[g.dim] : 0);
+  const int b = bl_len > 0 ? (int)(i / bl_len) : (ncols > g.dim ? (int)coord_at(coords, c0 + g.dim) : 0);
   soa[g.dim * npad + row] = b;
   level_keys[row] = site_key(g, cc, b);
 }
@@ -347,7 +347,7 @@ __global__ void k_finish_groups(const int *sidx, const int *head, const int *hea
   grid_max(len, 1, max_active);  // longest run; runs of one are the floor
 }
 
-void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coords, int64_t n,
+void build_input_layer(Metadata &m, const int64_t *spatial, CoordSrc coords, int64_t n,
                        int ncols, int min_batch, int mode, hipStream_t s, int64_t bl_length,
                        const unsigned char *overwrite) {
   const bool bl = bl_length > 0;
@@ -387,6 +387,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, const int64_t *coord
   k_input_keys<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, bl_length, m.k0.p, m.v0.p, m.dflags.p);
   LAUNCH_CHECK();
   const int *fetched = fetch_words(m, m.dflags.p, n_flags, s);
+  release_staging(m);  // coordinates from the host: their copies are behind us now
   const std::vector<int> hflags(fetched, fetched + n_flags);
   if (hflags[0] & 2) throw Error("input layer: sample index negative or too large for the site key");
   if (hflags[0] & 1) throw Error("input layer: coordinate outside [0, spatial_size)");

@@ -127,13 +127,21 @@ class Metadata:
 
     # ---- forward ops; each returns a new CUDA tensor ---------------------------------
     def inputLayer(self, spatial_size, coords, features, batch_size, mode):
-        coords = coords.to(device=features.device, dtype=torch.int64).contiguous()
         assert coords.dim() == 2 and coords.size(0) == features.size(0)
         features = _features(features, "input features")
         n = C.c_int64(0)
-        _lib.check(self._L.scn_md_input_layer(self._h, self._s(spatial_size), _ptr(coords), coords.size(0),
-                                              coords.size(1), int(batch_size), int(mode), _stream(),
-                                              C.byref(n)))
+        if coords.device.type == "cpu":
+            # the reference's calling convention (ioLayers.py:51-65): the library reads the host
+            # tensor itself, narrowing the values on their way to the device
+            coords = coords.to(dtype=torch.int64).contiguous()
+            _lib.check(self._L.scn_md_input_layer_host(self._h, self._s(spatial_size), C.c_void_p(coords.data_ptr()),
+                                                       coords.size(0), coords.size(1), int(batch_size), int(mode),
+                                                       _stream(), C.byref(n)))
+        else:
+            coords = coords.to(device=features.device, dtype=torch.int64).contiguous()
+            _lib.check(self._L.scn_md_input_layer(self._h, self._s(spatial_size), _ptr(coords), coords.size(0),
+                                                  coords.size(1), int(batch_size), int(mode), _stream(),
+                                                  C.byref(n)))
         out = torch.empty((n.value, features.size(1)), dtype=torch.float32, device=features.device)
         _lib.check(self._L.scn_input_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out

@@ -41,10 +41,17 @@ class HipPath:
         return _lib.sizes(self.dim, x) if x is not None else None
 
     # -- metadata ---------------------------------------------------------
+    host_coords = False  # True: coordinates are handed over in host memory (scn_md_input_layer_host)
+
     def input_layer(self, spatial, coords, batch_size=0, mode=3):
         coords = np.ascontiguousarray(coords, dtype=np.int64)
-        c = _dev(coords, torch.int64)
         n = C.c_int64(0)
+        if self.host_coords:
+            _lib.check(self.L.scn_md_input_layer_host(self.h, self._s(spatial), C.c_void_p(coords.ctypes.data),
+                                                      coords.shape[0], coords.shape[1], batch_size, mode, _stream(),
+                                                      C.byref(n)))
+            return n.value
+        c = _dev(coords, torch.int64)
         _lib.check(self.L.scn_md_input_layer(self.h, self._s(spatial), _ptr(c), coords.shape[0],
                                              coords.shape[1], batch_size, mode, _stream(), C.byref(n)))
         return n.value

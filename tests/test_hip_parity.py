@@ -27,6 +27,57 @@ def test_input_layer(make, dim, mode):
     checks.check_input_layer(make, dim, mode, seed=10 * dim + mode)
 
 
+@pytest.fixture(scope="module")
+def make_host(make):
+    """The same library with the coordinates handed over in host memory, as the reference's
+    InputLayer receives them (scn_md_input_layer_host)."""
+    def factory(dim):
+        p = make(dim)
+        p.host_coords = True
+        return p
+    return factory
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dim", [1, 3])
+def test_input_layer_from_host_coordinates(make_host, dim, mode):
+    checks.check_input_layer(make_host, dim, mode, seed=10 * dim + mode)
+    if mode == 4:
+        checks.check_input_layer(make_host, dim, mode, seed=7, with_batch_col=False)
+        checks.check_mode0_repeated_points(make_host, dim, seed=40 + dim)
+
+
+def test_host_coordinates_wide_values_and_sizes(make, make_host):
+    """Host coordinates are narrowed to int16 on their way to the device where the grid allows it:
+    sample indices beyond int16, grids beyond int16 and inputs of several chunks give the level
+    the device path gives; values outside the grid are still refused."""
+    from sparseconvnet_amd._lib import ScnError
+    rng = np.random.default_rng(77)
+    cases = []
+    c = rng.integers(0, 50, (3000, 4)).astype(np.int64)
+    c[:, 3] = rng.integers(0, 3, 3000) * 20000  # sample indices 0, 20000, 40000: the last needs int32
+    cases.append((50, c))
+    c = rng.integers(0, 100000, (5000, 3)).astype(np.int64)  # a grid beyond int16, no sample column
+    cases.append((100000, c))
+    c = rng.integers(0, 300, (1500000, 4)).astype(np.int64)   # several chunks, many repeated points
+    c[:, 3] = rng.integers(0, 2, len(c))
+    cases.append((300, c))
+    for spatial, coords in cases:
+        a, b = make(3), make_host(3)
+        na, nb = a.input_layer(spatial, coords, 0, 4), b.input_layer(spatial, coords, 0, 4)
+        assert na == nb > 0
+        assert (a.spatial_locations(spatial) == b.spatial_locations(spatial)).all()
+        f = rng.normal(size=(len(coords), 2)).astype(np.float32)
+        assert (a.input_fwd(f) == b.input_fwd(f)).all()
+    p = make_host(3)
+    for bad in ([[1, 2, 70000, 0]], [[1, -40000, 3, 0]], [[1, 2, 3, -1]], [[1 << 40, 2, 3, 0]]):
+        with pytest.raises(ScnError):
+            p.input_layer(64, np.array(bad, np.int64), 0, 3)
+        from sparseconvnet_amd import _lib
+        _lib.check(_lib.lib().scn_md_clear(p.h))
+    assert p.input_layer(64, np.array([[1, 2, 3, 0], [1, 2, 3, 0]], np.int64), 0, 3) == 1
+
+
 def test_input_layer_no_batch_column(make):
     checks.check_input_layer(make, 3, 4, seed=5, with_batch_col=False)
     checks.check_input_layer(make, 2, 0, seed=6, with_batch_col=False)
