@@ -15,7 +15,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     const int *__restrict__ nbr, const int *__restrict__ rowmap, int K, int64_t n, int64_t npad,
     const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp,
     Epi epi, int n_in, int n_out, int n_slab, int tiles_per_xcd, int n_tiles,
-    int n_split, float *__restrict__ partial, const float *__restrict__ pre_sc,
+    int n_split, int split_tiles, float *__restrict__ partial, const float *__restrict__ pre_sc,
     const float *__restrict__ pre_sh, float pre_leak, unsigned in_bytes) {
   static_assert(!BUF || VEC4, "buffer gathers need float4 rows");
   static_assert(!BF16 || (BUF && SS % 2 == 0), "the bf16 variant: buffer gathers, steps in pairs");
@@ -38,11 +38,25 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   const int r16 = lane & 15, g = lane >> 4;
 
   SCN_PHASE(0);  // start
-  const int tile = tiles_per_xcd ? (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+  // The taps of the first split_tiles tiles are dealt over n_split workgroups each (`split`: which of
+  // them this is, -1: the tile is this workgroup's alone).  Levels of fewer than 256 tiles split
+  // all their tiles, to fill the chip.
+  int tile, split;
+  if (tiles_per_xcd) {
+    tile = (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3);
+    split = n_split > 1 ? (int)blockIdx.y : -1;
+  } else if ((int)blockIdx.x < split_tiles * n_split) {
+    tile = blockIdx.x % split_tiles;
+    split = blockIdx.x / split_tiles;
+  } else {
+    tile = split_tiles + ((int)blockIdx.x - split_tiles * n_split);
+    split = -1;
+  }
+  const int ways = split < 0 ? 1 : n_split;
   if (tile >= n_tiles) return;
   const int64_t tbase = (int64_t)tile * TM;
 
-  const int ntaps = tile_setup<NT, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
+  const int ntaps = tile_setup<NT, G>(nbr, K, n, npad, tbase, ways, split, jtab, gmask, taplist, ntaps_p);
   const int total = ntaps * n_slab;
   SCN_PHASE(1);  // tile set up
   SCN_PHASE_VALUE(7, total);
@@ -55,7 +69,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
   for (int q = 0; q < RG; q++) mym[q] = 0ull;
   if (small_k) {
     const unsigned gmv = lane < K ? gmask[lane] : 0u;
-    tmask = __ballot(gmv != 0u && (n_split == 1 || lane % n_split == (int)blockIdx.y));
+    tmask = __ballot(gmv != 0u && (ways == 1 || lane % ways == split));
 #pragma unroll
     for (int q = 0; q < RG; q++) mym[q] = __ballot((gmv >> (wave * RG + q)) & 1u) & tmask;
   }
@@ -315,8 +329,8 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
     }
   }
   SCN_PHASE(4);  // tap loop done
-  if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
-    float *pt = partial + ((int64_t)blockIdx.y * n_tiles * TM + tbase) * (NCB * 16);
+  if (split >= 0) {  // partial tiles: [n_split][split_tiles * TM][NCB * 16]
+    float *pt = partial + ((int64_t)split * split_tiles * TM + tbase) * (NCB * 16);
 #pragma unroll
     for (int q = 0; q < RG; q++)
 #pragma unroll
@@ -391,16 +405,29 @@ static bool launch_rows(Metadata &m, const Table &t, const float *in, float *out
   }
   const int n_tiles = (int)ceil_div(t.n, G * 16);
   const int tiles_per_xcd = t.spread ? 0 : (int)ceil_div(n_tiles, 8);  // 0: tile = workgroup index
-  int n_split = 1;
-  if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
-  const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
+  // Few tiles: deal the taps of every tile over several workgroups (about two per CU in all).
+  // (Splitting only the most expensive tiles of a larger level, whose 27-tap tiles run three times
+  // the iterations of its 9-tap ones, was measured slower at 61 k sites, 179 -> 192 us: the extra
+  // workgroups no longer all fit on the chip at once.  The kernel keeps the means: split_tiles.)
+  int n_split = 1, split_tiles = 0;
+  if (n_tiles < 256) {
+    n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
+    split_tiles = n_tiles;
+  }
+  const int64_t split_stride = (int64_t)split_tiles * G * 16 * NCB * 16;
   float *partial = scratch_partial(m, n_split, split_stride);
-  note_kernel(m, BF16 ? "rows-bf16" : "rows", {{"ncb", NCB}, {"rg", RG}, {"ss", SS}, {"nw", NW}, {"pre", PRE}, {"split", n_split}});
-  kern<<<dim3((unsigned)(tiles_per_xcd ? tiles_per_xcd * 8 : n_tiles), n_split), NT, lds_bytes, s>>>(
+  if (n_split <= 1) n_split = 1, split_tiles = 0;
+  note_kernel(m, BF16 ? "rows-bf16" : "rows", {{"ncb", NCB}, {"rg", RG}, {"ss", SS}, {"nw", NW}, {"pre", PRE}, {"split", n_split},
+                                                {"split_tiles", split_tiles}});
+  const dim3 grid = tiles_per_xcd ? dim3((unsigned)(tiles_per_xcd * 8), n_split)
+                                  : dim3((unsigned)(split_tiles * n_split + (n_tiles - split_tiles)));
+  kern<<<grid, NT, lds_bytes, s>>>(
       t.nbr.p, t.rowmap_ptr(), t.K, t.n, t.npad, in, out, wpack, epi, n_in, n_out, n_slab, tiles_per_xcd,
-      n_tiles, n_split, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
+      n_tiles, n_split, split_tiles, partial, pre.sc, pre.sh, pre.leak, (unsigned)(m.cur_in_rows * n_in * 4));
   LAUNCH_CHECK();
-  if (n_split > 1) launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), t.n, epi, out, n_out, s);
+  if (n_split > 1)
+    launch_conv_reduce(partial, n_split, split_stride, NCB * 16, t.rowmap_ptr(), std::min<int64_t>(t.n, (int64_t)split_tiles * G * 16),
+                       epi, out, n_out, s);
   return true;
 }
 
