@@ -25,6 +25,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_FP32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+MFMA_BF16_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 PAIRS = [(3, 32), (32, 32), (64, 64), (128, 128), (256, 256)]
 TRAFFIC_FILE = os.path.join("profiles", "conv_sweep1M_pmc.txt")
 
@@ -89,11 +90,52 @@ def roofline_for(cin, cout, R, n, K, ms, traffic=None):
                  "frac": round(ach / HBM_PEAK_GBS, 4)}, **tr)
 
 
-def cpu_baseline(kind, sample_sites, seed, passes=3):
+def gpu_outputs(coords, work):
+    """The library's outputs for the CPU leg's own inputs: rows in the order of the points (input
+    mode 0 on distinct points), one SubmanifoldConvolution 3^3 per (x, w) of `work`."""
+    import torch
+    from sparseconvnet_amd import _lib
+    L = _lib.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sp, fs = _lib.sizes(3, 4096), _lib.sizes(3, 3)
+    cd = torch.as_tensor(coords).cuda()
+    h = L.scn_md_create(3)
+    n = C.c_int64(0)
+    _lib.check(L.scn_md_input_layer(h, sp, C.c_void_p(cd.data_ptr()), len(coords), coords.shape[1], 0, 0, stream,
+                                    C.byref(n)))
+    assert n.value == len(coords)
+    macs = C.c_double(0)
+    for x, w in work:
+        xd, wd = torch.as_tensor(x).cuda(), torch.as_tensor(w).cuda()
+        y = torch.empty((len(coords), w.shape[-1]), device="cuda")
+        _lib.check(L.scn_subm_conv_fwd(h, sp, fs, C.c_void_p(xd.data_ptr()), C.c_void_p(y.data_ptr()),
+                                       C.c_void_p(wd.data_ptr()), None, x.shape[1], w.shape[-1], 1, stream,
+                                       C.byref(macs)))
+        yield y.cpu().numpy()
+    L.scn_md_destroy(h)
+
+
+def roofline_bf16(cin, cout, R, n, K, ms):
+    """The bf16-operand path (rows and weights rounded to bf16 on the way into the MFMA, fp32 rows
+    in memory and fp32 accumulation): same algorithmic bytes as fp32, priced against the dense
+    bf16 MFMA peak or HBM, whichever bounds it."""
+    flops = 2.0 * R * cin * cout
+    byts = conv_bytes(R, n, K, cin, cout)
+    if flops / (MFMA_BF16_TFLOPS * 1e12) >= byts / (HBM_PEAK_GBS * 1e9):
+        ach = flops / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": round(ach, 3), "peak": MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach / MFMA_BF16_TFLOPS, 4), "traffic": None}
+    return dict(hbm_roofline(byts, ms), traffic=None)
+
+
+def cpu_baseline(kind, sample_sites, seed, passes=3, compare=None):
     """The CPU path on the GPU box's host cores: the same five convolutions on a room scene of
     the same generator, one warm-up pass and the median of `passes`; the rulebook build is timed
     by itself.  kind "reference": the reference's own CPU sources compiled behind
-    oracle/ref_harness.cpp (oracle/_ref); "port": this repository's restatement (oracle/)."""
+    oracle/ref_harness.cpp (oracle/_ref); "port": this repository's restatement (oracle/).
+    compare: a function (coords, work) yielding the library's output per pair; the largest
+    absolute difference from the CPU outputs of the last pass is reported per pair, beside the
+    largest absolute CPU output (fp32 sums of up to 27 x nIn products in a different order)."""
     from oracle import cpu_path
     from sparseconvnet_amd import synthetic
     flavour = "ref" if kind == "reference" else "oracle"
@@ -114,16 +156,24 @@ def cpu_baseline(kind, sample_sites, seed, passes=3):
         x = rng.normal(size=(len(coords), cin)).astype(np.float32)
         w = (rng.normal(size=(27, 1, cin, cout)) * (2.0 / (cin * 27)) ** 0.5).astype(np.float32)
         work.append((x, w))
-    secs, flops = [], 0.0
+    secs, flops, outs = [], 0.0, []
     for rep in range(passes + 1):
         t0 = time.time()
-        flops = 0.0
+        flops, outs = 0.0, []
         for x, w in work:
-            _, macs = p.subm_conv(4096, 3, x, w)
+            y, macs = p.subm_conv(4096, 3, x, w)
             flops += 2.0 * macs
+            outs.append(y if compare is not None else None)
         if rep:
             secs.append(time.time() - t0)
     sec = float(np.median(secs))
+    parity = None
+    if compare is not None:
+        parity = {}
+        for (cin, cout), want, got in zip(PAIRS, outs, compare(coords, work)):
+            parity["%dx%d" % (cin, cout)] = {"max_abs_err": float(np.abs(got - want).max()),
+                                             "max_abs_out": float(np.abs(want).max())}
+        del outs
     try:
         import torch
         cores = torch.get_num_threads() if kind == "reference" else int(os.environ.get("OMP_NUM_THREADS", os.cpu_count()))
@@ -131,6 +181,7 @@ def cpu_baseline(kind, sample_sites, seed, passes=3):
         cores = os.cpu_count()
     return {"value": round(flops / sec / 1e9, 2), "unit": "GFLOP/s", "cores": int(cores), "kind": kind,
             "rulebook_s": round(t_rules[-1], 3), "rulebook_cores": 1, "seconds_per_pass": round(sec, 3),
+            "parity_max_err": parity,
             "sample": "the sweep's 5 SubmanifoldConvolution 3^3 forwards on a %d-site room scene (%d rules), "
                       "1 warm-up pass + median of %d; rulebook build (one sample: single-threaded in the "
                       "reference) timed by itself, second of two builds" % (len(coords), R, passes)}
@@ -860,7 +911,8 @@ def main():
             ms = float(np.mean(t))
             bf.append({"nIn": wk[0], "nOut": wk[1], "ms": round(ms, 4),
                        "gflops": round(2.0 * R * wk[0] * wk[1] / (ms * 1e-3) / 1e9, 1),
-                       "speedup_vs_f32": round(per_pair_ms[i] / ms, 2)})
+                       "speedup_vs_f32": round(per_pair_ms[i] / ms, 2),
+                       "roofline": roofline_bf16(wk[0], wk[1], R, n, 27, ms)})
         out["sweep_bf16"] = bf
         _lib.check(L.scn_md_set_bf16(h, 0))
     L.scn_md_destroy(h)
@@ -892,8 +944,8 @@ def main():
     if not args.no_cpu:
         # the reference's own CPU sources where oracle/_ref was built, else this repository's port;
         # the port is listed as well (naive inner loops: a smaller scene keeps it bounded)
-        ref = cpu_baseline("reference", args.cpu_sites, args.seed)
-        port = cpu_baseline("port", args.cpu_port_sites, args.seed)
+        ref = cpu_baseline("reference", args.cpu_sites, args.seed, compare=gpu_outputs)
+        port = cpu_baseline("port", args.cpu_port_sites, args.seed, compare=gpu_outputs)
         out["cpu_baseline"] = ref if ref is not None else port
         if ref is not None and port is not None:
             out["cpu_baseline_port"] = port

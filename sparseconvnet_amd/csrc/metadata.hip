@@ -783,24 +783,43 @@ static const int64_t PATTERN_WHOLE_BELOW = 300000;
 // one).  Inside a window the positions with the most taps come first and the cheapest last,
 // which shortens the tail of kernels that hand positions out in order.
 // masks[t] (K <= 32): the tap mask itself, for the granule masks.
+// Tables of up to 8 taps (filter 2 in up to three dimensions): the code is the mask's rank in the
+// order (most taps first, then by value), 8 bits that sort like count-then-mask does, so that a
+// table of one window is sorted in a single pass.
 struct PatternKey {  // how finalize_table's sort key is put together
   int64_t window;
-  int pc_bits, pc_shift, code_bits, K;
+  int pc_bits, pc_shift, code_bits, K, ranked;
 };
+// Rank of a K-bit mask (K <= 8) among all K-bit masks ordered by falling number of set bits, then
+// rising value: the masks with more bits come first, and among those with c bits the rank is the
+// combinatorial number sum over the j-th lowest set bit at position i of C(i, j).
+__device__ inline unsigned mask_rank(unsigned mask, int K) {
+  constexpr unsigned char C[9][9] = {{1, 0, 0, 0, 0, 0, 0, 0, 0},     {1, 1, 0, 0, 0, 0, 0, 0, 0},     {1, 2, 1, 0, 0, 0, 0, 0, 0},
+                                     {1, 3, 3, 1, 0, 0, 0, 0, 0},     {1, 4, 6, 4, 1, 0, 0, 0, 0},     {1, 5, 10, 10, 5, 1, 0, 0, 0},
+                                     {1, 6, 15, 20, 15, 6, 1, 0, 0},  {1, 7, 21, 35, 35, 21, 7, 1, 0}, {1, 8, 28, 56, 70, 56, 28, 8, 1}};
+  const int c = __popc(mask);
+  unsigned r = 0;
+  for (int more = c + 1; more <= K; more++) r += C[K][more];
+  int j = 0;
+  for (int i = 0; i < K; i++)
+    if (mask >> i & 1u) r += C[i][++j];
+  return r;
+}
 __device__ inline unsigned long long pattern_key(const PatternKey &p, int64_t t, unsigned long long mask) {
   unsigned long long hi = (unsigned long long)(t / p.window);
+  if (p.ranked) return (hi << p.code_bits) | mask_rank((unsigned)mask, p.K);
   if (p.pc_bits) hi = (hi << p.pc_bits) | (unsigned long long)((p.K - __popcll(mask)) >> p.pc_shift);
   const unsigned long long code = p.code_bits < p.K ? (mask * 0x9E3779B97F4A7C15ull) >> (64 - p.code_bits) : mask;
   return (hi << p.code_bits) | code;
 }
-__global__ void k_table_masks(int64_t window, int pc_bits, int pc_shift, int code_bits, const int *nbr, int K, int64_t n,
-                              int64_t npad, unsigned long long *keys, int *idx, unsigned *masks) {
+__global__ void k_table_masks(PatternKey pk, const int *nbr, int K, int64_t n, int64_t npad, unsigned long long *keys,
+                              int *idx, unsigned *masks) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n) return;
   unsigned long long mask = 0;
   for (int k = 0; k < K; k++)
     if (nbr[(int64_t)k * npad + t] >= 0) mask |= 1ull << k;
-  keys[t] = pattern_key(PatternKey{window, pc_bits, pc_shift, code_bits, K}, t, mask);
+  keys[t] = pattern_key(pk, t, mask);
   idx[t] = (int)t;
   if (masks) masks[t] = (unsigned)mask;
 }
@@ -813,6 +832,25 @@ __global__ void k_table_permute(const int *nbr, int K, int64_t n, int64_t npad, 
   int src = perm[t];
   nbr2[(int64_t)k * npad + t] = nbr[(int64_t)k * npad + src];
   if (k == 0) rowmap[t] = base ? base[src] : src;
+}
+// Few taps (K <= 16): one thread moves a position's K entries and the granule masks come out of
+// the same launch (an OR over the 16 lanes of a granule).
+__global__ void k_table_permute_few(const int *nbr, int K, int64_t n, int64_t npad, const int *perm, const int *base,
+                                    int *nbr2, int *rowmap, unsigned *gmask) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned mk = 0;
+  if (t < n) {
+    const int src = perm[t];
+    for (int k = 0; k < K; k++) {
+      const int v = nbr[(int64_t)k * npad + src];
+      nbr2[(int64_t)k * npad + t] = v;
+      mk |= v >= 0 ? 1u << k : 0u;
+    }
+    rowmap[t] = base ? base[src] : src;
+  }
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) mk |= __shfl_xor(mk, o, 64);
+  if ((threadIdx.x & 15) == 0 && t < n) gmask[t >> 4] = mk;
 }
 // The same from a site-major table rows[src][ROWW]: a workgroup moves 64 positions, reading
 // each one's row in 16-byte pieces and writing 256 contiguous bytes per tap.
@@ -877,6 +915,13 @@ static PatternKey pattern_plan(int64_t n, int K, int &key_bits) {
   p.window = std::max<int64_t>(256, round_up(ceil_div(n, n < PATTERN_WHOLE_BELOW ? 1 : PATTERN_WINDOWS), 256));
   int block_bits = 0;
   while (((int64_t)1 << block_bits) < ceil_div(n, p.window)) block_bits++;
+  p.ranked = K <= 8;
+  if (p.ranked) {
+    p.pc_bits = p.pc_shift = 0;
+    p.code_bits = 8;
+    key_bits = 8 + block_bits;
+    return p;
+  }
   int pc_bits = 1;
   while ((1 << pc_bits) <= K) pc_bits++;
   // Up to 40 key bits (four sort passes; a 27-tap table needs 35): beyond that the count of
@@ -923,14 +968,14 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   reserve_pattern_buffers(m, t);
   unsigned *masks = t.K <= 32 ? reinterpret_cast<unsigned *>(m.f1.p) : nullptr;
   if (!keyed) {
-    k_table_masks<<<grid_for(t.n), TB, 0, s>>>(pk.window, pk.pc_bits, pk.pc_shift, pk.code_bits, t.nbr.p, t.K, t.n, t.npad,
-                                               m.k0.p, m.v0.p, masks);
+    k_table_masks<<<grid_for(t.n), TB, 0, s>>>(pk, t.nbr.p, t.K, t.n, t.npad, m.k0.p, m.v0.p, masks);
     LAUNCH_CHECK();
   }
   sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, key_bits);
   DevBuf<int> nbr2;
   nbr2.reserve((size_t)t.K * t.npad);
-  const bool from_rows = rows && (roww == 32 || roww == 12);  // these also write the granule masks (K <= 32)
+  const bool few = !rows && t.K <= 16;
+  const bool from_rows = (rows && (roww == 32 || roww == 12)) || few;  // these also write the granule masks (K <= 32)
   if (from_rows) t.gmask.reserve(ceil_div(t.n, 16));
   if (rows && roww == 32)
     k_table_rows_permute<32><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p,
@@ -938,6 +983,9 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
   else if (rows && roww == 12)
     k_table_rows_permute<12><<<grid_for(t.n, 64), 256, 0, s>>>(rows, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p,
                                                                t.gmask.p);
+  else if (few)
+    k_table_permute_few<<<grid_for(t.n), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p, t.rowmap.p,
+                                                     t.gmask.p);
   else
     k_table_permute<<<grid_for(t.n * t.K), TB, 0, s>>>(t.nbr.p, t.K, t.n, t.npad, m.v1.p, base, nbr2.p,
                                                        t.rowmap.p);
@@ -1302,16 +1350,13 @@ __device__ inline bool candidate(const Geom &gi, const Filt &f, const int *p, in
   return true;
 }
 
-// zero: 16 x 64 counters that the launch behind this one (k_strided_heads) adds to, or null.
 // pos_keys (optional, dimensions up to 3): the site key of every schedule position; the site is
 // then decoded from one coalesced read instead of gathered by row through the schedule.
 // dup_keys (levels whose keys may repeat, else null): the positions' keys; only the last position of a
 // run of equal keys is a site (see k_subm_rules), the others have no candidates.
 __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, const int *sched,
                                      const unsigned long long *pos_keys, int64_t n, int64_t npad,
-                                     unsigned long long *keys, int *payload, int *zero, const unsigned long long *dup_keys) {
-  if (zero && blockIdx.x == 0)
-    for (int i = threadIdx.x; i < 16 * 64; i += blockDim.x) zero[i] = 0;
+                                     unsigned long long *keys, int *payload, const unsigned long long *dup_keys) {
   int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n * f.M) return;
   int64_t t = e / f.M;
@@ -1331,38 +1376,13 @@ __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, c
 }
 
 // head[p] = 1 where a new output site begins in the sorted candidate keys.
-// counts (optional; filter = stride = 2 over exactly halving sizes, Morton keys): the sizes of the
-// levels that further halvings will make.  Two sites fall into the same site j halvings further
-// down iff their keys agree above the low dim * j bits (a Morton key drops one bit per coordinate
-// per halving; the sample index sits above), so in ascending key order a position starts a new
-// site on every level up to (highest bit in which it differs from its predecessor) / dim, and one
-// pass counts the sites of all levels: counts[j], j = 0 .. levels.  The whole chain of levels
-// then costs one read-back instead of one per level.
-__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head, int dim, int levels,
-                                int *counts) {
-  __shared__ int hist[64];
-  if (counts) {
-    if (threadIdx.x < 64) hist[threadIdx.x] = 0;
-    __syncthreads();
-  }
+__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p == n) head[p] = 0;  // one element past the end, so that a scan of n + 1 ends with the total
-  int top = -1;  // a new site on levels 0 .. top
   if (p < n) {
-    const unsigned long long k = skeys[p], d = p ? k ^ skeys[p - 1] : ~0ull;
-    head[p] = (k != SCN_EMPTY_KEY && d != 0ull) ? 1 : 0;
-    if (counts && k != SCN_EMPTY_KEY && d != 0ull) top = p ? min(levels, (63 - __clzll((long long)d)) / dim) : levels;
+    const unsigned long long k = skeys[p];
+    head[p] = (k != SCN_EMPTY_KEY && (p == 0 || k != skeys[p - 1])) ? 1 : 0;
   }
-  if (!counts) return;
-  for (int l = 0; l <= levels; l++) {
-    const unsigned long long b = __ballot(top >= l);
-    if ((threadIdx.x & 63) == 0 && b) atomicAdd(&hist[l], __popcll(b));
-  }
-  __syncthreads();
-  // one of 16 copies of the counters (thousands of workgroups adding to the same few addresses take
-  // longer than the rest of the kernel); the host adds the copies up
-  if (threadIdx.x <= levels && hist[threadIdx.x])
-    atomicAdd(&counts[(blockIdx.x & 15) * 64 + threadIdx.x], hist[threadIdx.x]);
 }
 
 // One thread per sorted candidate: output row = number of heads before it; the filter tap
@@ -1409,6 +1429,135 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
     if (lcount[k]) atomicAdd(&slot[k], (unsigned long long)lcount[k]);
 }
 
+// ---- filter = stride = 2 over exactly halving sizes (the U-Net's and most networks' downsampling) ----
+// Every site has one output site, that of its coordinates halved, and the Morton key of that site
+// ascends with the site's own key: in schedule order the inputs of an output site are neighbours
+// (at most 2^dim of them), the output sites are the runs of equal parent keys, and nothing needs to
+// be sorted.  Two launches make both tables, the output level and the keys of the pattern sort.
+constexpr int HB = 1024;  // positions per workgroup of the two kernels
+__device__ inline unsigned long long parent_key(const Geom &gi, const Geom &go, unsigned long long key, int *tap,
+                                                int *j, int &b) {
+  int p[SCN_MAXD];
+  site_of_key(gi, key, p, b);
+  int k = 0;
+  for (int d = 0; d < gi.dim; d++) {
+    j[d] = p[d] >> 1;
+    k = 2 * k + (p[d] & 1);  // tap = the site's offset inside its output site's 2^dim box
+  }
+  *tap = k;
+  return site_key(go, j, b);
+}
+// block_heads[w] = output sites that begin in workgroup w's HB positions.
+// counts (optional, 16 x 64 zeroed words): the sizes of the levels that `levels` further halvings
+// will make.  Two sites fall into the same site j halvings further down iff their output keys agree
+// above the low dim * j bits (a Morton key drops one bit per coordinate per halving; the sample
+// index sits above), so in ascending key order a position starts a new site on every level up to
+// (highest bit in which its output key differs from its predecessor's) / dim, and one pass counts
+// the sites of all levels: counts[j], j = 0 .. levels, in one of 16 copies that the host adds up
+// (thousands of workgroups adding to the same few addresses take longer than the rest of the
+// kernel).  The whole chain of levels then costs one read-back instead of one per level.
+// zero: words cleared for the launch behind this one.
+__global__ __launch_bounds__(HB) void k_halve_heads(Geom gi, Geom go, const unsigned long long *keys, int64_t n,
+                                                    int levels, int *block_heads, int *counts, uint32_t *zero,
+                                                    int zero_words) {
+  __shared__ int hist[64];
+  __shared__ int total;
+  for (int i = blockIdx.x * HB + threadIdx.x; i < zero_words; i += gridDim.x * HB) zero[i] = 0u;
+  if (threadIdx.x < 64) hist[threadIdx.x] = 0;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * HB + threadIdx.x;
+  int top = -1;  // a new site on levels 0 .. top
+  if (p < n) {
+    int tap, j[SCN_MAXD], b;
+    const unsigned long long ck = parent_key(gi, go, keys[p], &tap, j, b);
+    const unsigned long long d = p ? ck ^ parent_key(gi, go, keys[p - 1], &tap, j, b) : ~0ull;
+    if (d) top = p ? min(levels, (63 - __clzll((long long)d)) / gi.dim) : levels;
+  }
+  const unsigned long long heads = __ballot(top >= 0);
+  if ((threadIdx.x & 63) == 0 && heads) atomicAdd(&total, __popcll(heads));
+  if (counts)
+    for (int l = 0; l <= levels; l++) {
+      const unsigned long long bl = __ballot(top >= l);
+      if ((threadIdx.x & 63) == 0 && bl) atomicAdd(&hist[l], __popcll(bl));
+    }
+  __syncthreads();
+  if (threadIdx.x == 0) block_heads[blockIdx.x] = total;
+  if (counts && threadIdx.x <= levels && hist[threadIdx.x])
+    atomicAdd(&counts[(blockIdx.x & 15) * 64 + threadIdx.x], hist[threadIdx.x]);
+}
+// One thread per input position t: its output row o is the number of output sites that begin at or
+// before t, less one (workgroups before this one: block_heads; inside: ballots).  It writes its own
+// rule into both tables and -1 into the other taps of by_in; the first position of an output site
+// looks at the up to 2^dim - 1 positions behind it for the site's tap mask, writes -1 into the
+// absent taps of by_out, the site's coordinates and key, and its pattern-sort key
+// (Metadata/ConvolutionRules.h:19-31, Metadata/RectangularRegions.h:30-38,95-105 for this filter).
+__global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, const unsigned long long *keys, const int *sched,
+                                                   int64_t n, int64_t npad_in, int64_t npad_out, const int *block_heads,
+                                                   int *by_out, int *by_in, int *out_soa, unsigned long long *out_keys,
+                                                   unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
+                                                   int *pidx, unsigned *pmasks) {
+  const int K = 1 << gi.dim;
+  __shared__ int red[HB / 64], wave_heads[HB / 64], lcount[8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int before = 0;
+  for (int i = threadIdx.x; i < (int)blockIdx.x; i += HB) before += block_heads[i];
+#pragma unroll
+  for (int o = 32; o; o >>= 1) before += __shfl_xor(before, o, 64);
+  if (threadIdx.x < 8) lcount[threadIdx.x] = 0;
+  const int64_t p = (int64_t)blockIdx.x * HB + threadIdx.x;
+  const bool live = p < n;
+  int tap = -1, j[SCN_MAXD], b = 0;
+  unsigned long long ck = 0;
+  bool head = false;
+  if (live) {
+    ck = parent_key(gi, go, keys[p], &tap, j, b);
+    if (p) {
+      int t2, j2[SCN_MAXD], b2;
+      head = ck != parent_key(gi, go, keys[p - 1], &t2, j2, b2);
+    } else {
+      head = true;
+    }
+  }
+  const unsigned long long heads = __ballot(head);
+  if (lane == 0) {
+    red[wave] = before;
+    wave_heads[wave] = __popcll(heads);
+  }
+  __syncthreads();
+  int o = 0;
+  for (int w = 0; w < HB / 64; w++) o += red[w] + (w < wave ? wave_heads[w] : 0);
+  o += __popcll(heads & (~0ull >> (63 - lane))) - 1;  // heads at or before this lane, less one
+  if (live) {
+    const int row = sched ? sched[p] : (int)p;
+    for (int k = 0; k < K; k++) by_in[(int64_t)k * npad_in + p] = k == tap ? o : -1;
+    by_out[(int64_t)tap * npad_out + o] = row;
+    if (head) {
+      unsigned mask = 1u << tap;
+      for (int i = 1; i < K && p + i < n; i++) {
+        int t2, j2[SCN_MAXD], b2;
+        if (parent_key(gi, go, keys[p + i], &t2, j2, b2) != ck) break;
+        mask |= 1u << t2;
+      }
+      for (int k = 0; k < K; k++)
+        if (!(mask >> k & 1u)) by_out[(int64_t)k * npad_out + o] = -1;
+      for (int d = 0; d < gi.dim; d++) out_soa[d * npad_out + o] = j[d];
+      out_soa[gi.dim * npad_out + o] = b;
+      out_keys[o] = ck;
+      pkeys[o] = pattern_key(pk, o, mask);
+      pidx[o] = o;
+      pmasks[o] = mask;
+    }
+  }
+  for (int k = 0; k < K; k++) {
+    const unsigned long long bk = __ballot(tap == k);
+    if (lane == 0 && bk) atomicAdd(&lcount[k], __popcll(bk));
+  }
+  __syncthreads();
+  unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * K;
+  if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&slot[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
+}
+
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
                             const int64_t *filter, const int64_t *stride, hipStream_t s) {
   SizeKey key = mk(m.dim, in_size, filter, stride);
@@ -1450,12 +1599,6 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   Level &LI = m.levels[R.in_size];
   int64_t nc = n * f.M;
   if (nc >= ((int64_t)1 << 31) - 64) throw Error("strided rules: too many candidate pairs for int32 indices");
-  m.k0.reserve(nc);
-  m.k1.reserve(nc);
-  m.v0.reserve(nc);
-  m.v1.reserve(nc);
-  m.f0.reserve(nc + 1);
-  m.s0.reserve(nc + 1);
   // Filter = stride = 2 in every dimension over exactly fitting sizes (the U-Net's and most
   // networks' downsampling): each site has one candidate, the Morton key of its coordinates
   // halved, which ascends with the site's own key, so the schedule order is already sorted.
@@ -1464,7 +1607,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     presorted = presorted && filter[d] == 2 && stride[d] == 2 && in_size[d] == 2 * out_size[d];
   // The caller has to learn the new level's size: a read-back per rulebook, except along a chain
   // of exact halvings, whose sizes the first rulebook of the chain counts all at once
-  // (k_strided_heads) and hands down from level to level.
+  // (k_halve_heads) and hands down from level to level.
   int chain = 0;  // further exact halvings of the output size, when this call has to count
   if (presorted && LI.halvings.empty()) {
     for (bool even = true; even && chain < 60 / m.dim - 1;) {
@@ -1474,36 +1617,63 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     m.dflags.reserve(16 * 64);
   }
   const bool count = presorted && LI.halvings.empty();
+  if (presorted) {
+    // positions' keys: the level's own when its rows are in schedule order (a level made here)
+    const unsigned long long *keys = LI.identity_sched ? LI.keys.p : position_keys(LI, s);
+    const int blocks = (int)ceil_div(n, HB);
+    m.f0.reserve(blocks);
+    start_counts(R.by_out, s, false);
+    const int count_words = 2 * COUNT_SLOTS * f.K;
+    if (count) fill32(m.dflags.p, 0, 16 * 64, s);
+    k_halve_heads<<<dim3(blocks), HB, 0, s>>>(LI.g, go, keys, n, chain, m.f0.p, count ? m.dflags.p : nullptr,
+                                              reinterpret_cast<uint32_t *>(R.by_out.cnt->dev.p), count_words);
+    LAUNCH_CHECK();
+    if (count) {
+      const int *c = fetch_words(m, m.dflags.p, 16 * 64, s);
+      LI.halvings.assign(chain + 1, 0);
+      for (int copy = 0; copy < 16; copy++)
+        for (int l = 0; l <= chain; l++) LI.halvings[l] += c[copy * 64 + l];
+    }
+    const int64_t n_out = LI.halvings[0];
+    alloc_level(LO, go, n_out, batch);
+    LO.halvings.assign(LI.halvings.begin() + 1, LI.halvings.end());
+    R.by_out.n = n_out;
+    R.by_out.npad = LO.npad;
+    R.by_in.n = n;
+    R.by_in.npad = LI.npad;
+    R.by_out.nbr.reserve((size_t)f.K * LO.npad);
+    R.by_in.nbr.reserve((size_t)f.K * LI.npad);
+    int key_bits = 0;
+    const PatternKey pk = pattern_plan(n_out, f.K, key_bits);
+    reserve_pattern_buffers(m, R.by_out);
+    k_halve_emit<<<dim3(blocks), HB, 0, s>>>(LI.g, go, keys, LI.sched_ptr(), n, LI.npad, LO.npad, m.f0.p, R.by_out.nbr.p,
+                                             R.by_in.nbr.p, LO.coords.p, LO.keys.p,
+                                             (unsigned long long *)R.by_out.cnt->dev.p, pk, m.k0.p, m.v0.p,
+                                             reinterpret_cast<unsigned *>(m.f1.p));
+    LAUNCH_CHECK();
+    R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
+    finalize_table(m, R.by_out, nullptr, s, true);
+    return m.strided.emplace(key, std::move(R)).first->second;
+  }
+  m.k0.reserve(nc);
+  m.k1.reserve(nc);
+  m.v0.reserve(nc);
+  m.v1.reserve(nc);
+  m.f0.reserve(nc + 1);
+  m.s0.reserve(nc + 1);
   // a level with a schedule of its own (the input layer's): sites from the positions' keys
   const unsigned long long *pos_keys = (m.dim <= 3 && !LI.identity_sched) ? position_keys(LI, s) : nullptr;
   const unsigned long long *dup_keys = LI.dups ? position_keys(LI, s) : nullptr;
   k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
-                                                   m.k0.p, m.v0.p, count ? m.dflags.p : nullptr, dup_keys);
+                                                   m.k0.p, m.v0.p, dup_keys);
   LAUNCH_CHECK();
-  if (presorted) {
-    std::swap(m.k0, m.k1);
-    std::swap(m.v0, m.v1);
-  } else {
-    // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
-    sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
-  }
-  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p, m.dim, chain, count ? m.dflags.p : nullptr);
+  // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
+  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
   LAUNCH_CHECK();
   exclusive_scan(m, m.f0.p, m.s0.p, nc + 1, s);
-  int64_t n_out = -1;
-  if (count) {
-    const int *c = fetch_words(m, m.dflags.p, 16 * 64, s);
-    LI.halvings.assign(chain + 1, 0);
-    for (int copy = 0; copy < 16; copy++)
-      for (int l = 0; l <= chain; l++) LI.halvings[l] += c[copy * 64 + l];
-  }
-  if (presorted) {
-    n_out = LI.halvings[0];
-  } else {
-    n_out = fetch_words(m, m.s0.p + nc, 1, s)[0];
-  }
+  const int64_t n_out = fetch_words(m, m.s0.p + nc, 1, s)[0];
   alloc_level(LO, go, n_out, batch);
-  if (presorted) LO.halvings.assign(LI.halvings.begin() + 1, LI.halvings.end());
   R.by_out.n = n_out;
   R.by_out.npad = LO.npad;
   R.by_in.n = n;
