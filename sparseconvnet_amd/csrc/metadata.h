@@ -207,6 +207,7 @@ struct Metadata {
   DevBuf<float> wcols;  // column ranges of a wide layer's weights, one contiguous block per range (conv_forward)
   DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
+  DevBuf<unsigned long long> ticket;  // [0]: arrival ticket of grid_count (zero between launches), [1]: the count
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups; partial sums of reductions
   DevBuf<float> wt;       // transposed weights of the input-gradient convolution of a backward pass

@@ -160,7 +160,7 @@ using RadixAlways = rocprim::radix_sort_config<rocprim::default_config, rocprim:
                                                rocprim::default_config, 4096>;
 static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout,
                        const int *vin, int *vout, int64_t n, hipStream_t s, int end_bit = 64) {
-  if (n > 32768 && n <= 1500000) {
+  if ((n > 32768 && n <= 1500000) || n <= 4096) {  // up to 4096 pairs: one launch, one workgroup
     radix_sort_pairs(m, kin, kout, vin, vout, n, end_bit, s);
     return;
   }
@@ -227,6 +227,39 @@ __device__ inline void grid_max(int v, int floor, int *slots) {
   __syncthreads();
   int *slot = slots + MAX_SLOT_STRIDE * (blockIdx.x & (MAX_SLOTS - 1));
   if (threadIdx.x == 0 && block_max > floor && block_max > __builtin_nontemporal_load(slot)) atomicMax(slot, block_max);
+}
+
+// Adds up a count over a whole grid of workgroups with no launch in front to clear a counter and
+// none behind to add up: every workgroup adds (1 << 32 | its count) to *ticket, so the value a
+// workgroup gets back tells it how many came before and what they counted; the last one writes
+// the sum to ticket[1] and puts the ticket back to zero for the next launch.  Every thread of
+// every workgroup must call it, once.  Launches that share a ticket must not overlap (one stream).
+// Same-address atomics take about 12 ns each: grids of a few hundred workgroups (COUNT_GRID) that
+// stride over their input, not one workgroup per 256 elements.
+static const int COUNT_GRID = 256;
+__device__ inline void grid_count(int mine, unsigned long long *ticket) {
+  __shared__ int block_total;
+  if (threadIdx.x == 0) block_total = 0;
+  __syncthreads();
+#pragma unroll
+  for (int o = 32; o; o >>= 1) mine += __shfl_xor(mine, o, 64);
+  if ((threadIdx.x & 63) == 0 && mine) atomicAdd(&block_total, mine);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned long long old = atomicAdd(ticket, (1ull << 32) | (unsigned long long)(unsigned)block_total);
+    if ((old >> 32) == gridDim.x - 1) {
+      ticket[1] = (old & 0xFFFFFFFFull) + (unsigned)block_total;
+      atomicExch(ticket, 0ull);
+    }
+  }
+}
+static dim3 count_grid(int64_t n) { return dim3((unsigned)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n, TB), COUNT_GRID))); }
+static unsigned long long *count_ticket(Metadata &m, hipStream_t s) {
+  if (!m.ticket.p) {
+    m.ticket.reserve(2);
+    fill32(m.ticket.p, 0, 4, s);
+  }
+  return m.ticket.p;
 }
 
 // flags[0] |= 1: coordinate outside the grid; |= 2: sample index out of range.
@@ -399,7 +432,6 @@ void build_input_layer(Metadata &m, const int64_t *spatial, CoordSrc coords, int
   // keeps the EMPTY keys (all ones) of empty positions behind every real key
   const int bits = key_bits(g, (int64_t)top_batch + 1) + (n_empty ? 1 : 0);
   if (bits > 64) throw Error("batch-by-length input layer: grid too large for a layer with empty positions");
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s, bits);
   // Metadata/IOLayersRules.h:25,46-47,76-77: the batch is at least min_batch and grows to
   // the largest sample index + 1; without a sample column there is exactly one sample.
   // :140 batch-by-length: one grid per sample of the input, filled or not.
@@ -408,15 +440,19 @@ void build_input_layer(Metadata &m, const int64_t *spatial, CoordSrc coords, int
   if (mode == 0) {
     alloc_level(L, g, n, batch);
     L.sched.reserve(n);
+    L.skeys.reserve(n + 1);
     L.identity_sched = false;
     L.dups = true;  // mode 0 does not merge repeated points
+    // the sorted pairs are the level's schedule and its positions' keys
+    sort_pairs(m, m.k0.p, L.skeys.p, m.v0.p, L.sched.p, n, s, bits);
+    L.skeys_ready = true;
     k_input_rows_identity<<<grid_for(n), TB, 0, s>>>(g, coords, n, ncols, bl_length, L.npad, L.coords.p);
     LAUNCH_CHECK();
     HIP_CHECK(hipMemcpyAsync(L.keys.p, m.k0.p, n * sizeof(unsigned long long), hipMemcpyDeviceToDevice, s));
-    HIP_CHECK(hipMemcpyAsync(L.sched.p, m.v1.p, n * sizeof(int), hipMemcpyDeviceToDevice, s));
     R.n_out = n;
     return;
   }
+  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, n, s, bits);
 
   m.f0.reserve(n + 1);  // head
   m.f1.reserve(n);  // is_first
@@ -547,27 +583,39 @@ __device__ inline unsigned long long grid_capacity(long long nblocks) {
   while (cap < (unsigned long long)nblocks * 2ull) cap <<= 1;
   return cap;
 }
-// skey[t] = key of the row at schedule position t; head[t] = 1 where a block of 64 keys starts.
+// skey[t] = key of the row at schedule position t; head[t] = 1 where a block of 64 keys starts;
+// ticket[1] = the number of blocks (grid_count).
 __global__ void k_grid_heads(const unsigned long long *keys, const int *sched, int64_t n,
-                             unsigned long long *skey, int *head) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  const unsigned long long k = keys[sched ? sched[t] : t];
-  skey[t] = k;
-  head[t] = (t == 0 || (k >> 6) != (keys[sched ? sched[t - 1] : t - 1] >> 6)) ? 1 : 0;
+                             unsigned long long *skey, int *head, unsigned long long *ticket) {
+  int heads = 0;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x) {
+    const unsigned long long k = keys[sched ? sched[t] : t];
+    skey[t] = k;
+    const int h = (t == 0 || (k >> 6) != (keys[sched ? sched[t - 1] : t - 1] >> 6)) ? 1 : 0;
+    head[t] = h;
+    heads += h;
+  }
+  grid_count(heads, ticket);
 }
-__global__ void k_block_heads(const unsigned long long *ukey, int64_t n, int *head) {
-  int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (u < n) head[u] = (u == 0 || (ukey[u] >> 6) != (ukey[u - 1] >> 6)) ? 1 : 0;
+// n_sites_dev: the index of the last distinct site when their number is only known on the device
+// (levels with repeated keys; positions behind it hold stale keys), else null.
+__global__ void k_block_heads(const unsigned long long *ukey, int64_t n, const int *n_sites_dev, int *head,
+                              unsigned long long *ticket) {
+  const int64_t U = n_sites_dev ? (int64_t)*n_sites_dev + 1 : n;
+  int heads = 0;
+  for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < U; u += (int64_t)gridDim.x * blockDim.x) {
+    const int h = (u == 0 || (ukey[u] >> 6) != (ukey[u - 1] >> 6)) ? 1 : 0;
+    head[u] = h;
+    heads += h;
+  }
+  grid_count(heads, ticket);
 }
 // Empties the part of the table that will be used and records its mask (capacity - 1) for the
-// kernels that follow.  n_sites_dev: the number of distinct sites when it is only known on
-// the device (levels with repeated keys), else null.
-__global__ void k_block_clear(BlockEntry *table, int64_t cap_alloc, const int *head, const int *head_scan,
-                              int64_t n_sites, const int *n_sites_dev, unsigned long long *mask_out) {
+// kernels that follow.  ticket[1]: the number of blocks, as the head kernel in front left it.
+__global__ void k_block_clear(BlockEntry *table, int64_t cap_alloc, const unsigned long long *ticket,
+                              unsigned long long *mask_out) {
   int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t U = n_sites_dev ? (int64_t)*n_sites_dev + 1 : n_sites;
-  const unsigned long long cap = grid_capacity(U > 0 ? (long long)head_scan[U - 1] + head[U - 1] : 0);
+  const unsigned long long cap = grid_capacity((long long)ticket[1]);
   if (b == 0) *mask_out = cap - 1;
   if (b < cap_alloc && (unsigned long long)b < cap) {
     table[b].key = SCN_EMPTY_KEY;
@@ -637,11 +685,11 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   L.table.reserve(cap_alloc);
   const unsigned long long *ukey = L.skeys.p;
   const int *n_sites_dev = nullptr;
+  unsigned long long *ticket = count_ticket(m, s);
   if (n) {
     if (L.dups) {
       // distinct sites first: ukey / urow by compaction; their number stays on the device
-      k_sorted_keys<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, L.skeys.p);
-      LAUNCH_CHECK();
+      position_keys(L, s);
       m.f1.reserve(n + 1);
       m.s1.reserve(n + 1);
       L.urow.reserve(n);
@@ -652,20 +700,19 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
       LAUNCH_CHECK();
       n_sites_dev = m.s1.p + (n - 1);  // index of the last distinct site (the last position ends a run)
       ukey = m.k1.p;
-      // positions past the last distinct site hold stale keys: heads there are never read
-      k_block_heads<<<grid_for(n), TB, 0, s>>>(ukey, n, m.f0.p);
+      k_block_heads<<<count_grid(n), TB, 0, s>>>(ukey, n, n_sites_dev, m.f0.p, ticket);
       LAUNCH_CHECK();
     } else if (L.skeys_ready) {  // the input layer left the positions' keys
-      k_block_heads<<<grid_for(n), TB, 0, s>>>(L.skeys.p, n, m.f0.p);
+      k_block_heads<<<count_grid(n), TB, 0, s>>>(L.skeys.p, n, nullptr, m.f0.p, ticket);
       LAUNCH_CHECK();
     } else {
-      k_grid_heads<<<grid_for(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, L.skeys.p, m.f0.p);
+      k_grid_heads<<<count_grid(n), TB, 0, s>>>(L.keys.p, L.sched_ptr(), n, L.skeys.p, m.f0.p, ticket);
       LAUNCH_CHECK();
     }
-    exclusive_scan(m, m.f0.p, m.s0.p, n, s);
+  } else {
+    fill32(ticket + 1, 0, 2, s);  // no sites: no blocks
   }
-  k_block_clear<<<grid_for((int64_t)cap_alloc), TB, 0, s>>>(L.table.p, (int64_t)cap_alloc, m.f0.p, m.s0.p, n,
-                                                           n_sites_dev, L.gridp.p);
+  k_block_clear<<<grid_for((int64_t)cap_alloc), TB, 0, s>>>(L.table.p, (int64_t)cap_alloc, ticket, L.gridp.p);
   LAUNCH_CHECK();
   if (n) {
     k_block_insert<<<grid_for(n), TB, 0, s>>>(ukey, m.f0.p, n, n_sites_dev, L.table.p, L.gridp.p);
@@ -783,26 +830,34 @@ static const int64_t PATTERN_WHOLE_BELOW = 300000;
 // one).  Inside a window the positions with the most taps come first and the cheapest last,
 // which shortens the tail of kernels that hand positions out in order.
 // masks[t] (K <= 32): the tap mask itself, for the granule masks.
-// Tables of up to 8 taps (filter 2 in up to three dimensions): the code is the mask's rank in the
-// order (most taps first, then by value), 8 bits that sort like count-then-mask does, so that a
-// table of one window is sorted in a single pass.
+// Tables of up to 32 taps: the code is the mask's rank in the order (most taps first, then by
+// value), which sorts exactly like count-then-mask does in K bits instead of K + log2(K): three
+// passes instead of four for 27 taps, one instead of two for 8 or 9.
 struct PatternKey {  // how finalize_table's sort key is put together
   int64_t window;
   int pc_bits, pc_shift, code_bits, K, ranked;
 };
-// Rank of a K-bit mask (K <= 8) among all K-bit masks ordered by falling number of set bits, then
+struct Binomials {
+  unsigned v[33][33];      // v[i][j] = C(i, j)
+  unsigned above[33][33];  // above[K][c] = number of K-bit masks with more than c set bits
+  constexpr Binomials() : v{}, above{} {
+    for (int i = 0; i < 33; i++) {
+      v[i][0] = 1;
+      for (int j = 1; j <= i; j++) v[i][j] = v[i - 1][j - 1] + (j < i ? v[i - 1][j] : 0u);
+    }
+    for (int k = 0; k < 33; k++)
+      for (int c = k - 1; c >= 0; c--) above[k][c] = above[k][c + 1] + v[k][c + 1];
+  }
+};
+__constant__ const Binomials c_binom = Binomials();
+// Rank of a K-bit mask (K <= 32) among all K-bit masks ordered by falling number of set bits, then
 // rising value: the masks with more bits come first, and among those with c bits the rank is the
-// combinatorial number sum over the j-th lowest set bit at position i of C(i, j).
+// combinatorial number, the sum over the set bits of C(position, number of set bits up to and
+// including it) (one independent table read per bit).
 __device__ inline unsigned mask_rank(unsigned mask, int K) {
-  constexpr unsigned char C[9][9] = {{1, 0, 0, 0, 0, 0, 0, 0, 0},     {1, 1, 0, 0, 0, 0, 0, 0, 0},     {1, 2, 1, 0, 0, 0, 0, 0, 0},
-                                     {1, 3, 3, 1, 0, 0, 0, 0, 0},     {1, 4, 6, 4, 1, 0, 0, 0, 0},     {1, 5, 10, 10, 5, 1, 0, 0, 0},
-                                     {1, 6, 15, 20, 15, 6, 1, 0, 0},  {1, 7, 21, 35, 35, 21, 7, 1, 0}, {1, 8, 28, 56, 70, 56, 28, 8, 1}};
-  const int c = __popc(mask);
-  unsigned r = 0;
-  for (int more = c + 1; more <= K; more++) r += C[K][more];
-  int j = 0;
+  unsigned r = c_binom.above[K][__popc(mask)];
   for (int i = 0; i < K; i++)
-    if (mask >> i & 1u) r += C[i][++j];
+    if (mask >> i & 1u) r += c_binom.v[i][__popc(mask & ((2u << i) - 1u))];
   return r;
 }
 __device__ inline unsigned long long pattern_key(const PatternKey &p, int64_t t, unsigned long long mask) {
@@ -915,20 +970,19 @@ static PatternKey pattern_plan(int64_t n, int K, int &key_bits) {
   p.window = std::max<int64_t>(256, round_up(ceil_div(n, n < PATTERN_WHOLE_BELOW ? 1 : PATTERN_WINDOWS), 256));
   int block_bits = 0;
   while (((int64_t)1 << block_bits) < ceil_div(n, p.window)) block_bits++;
-  p.ranked = K <= 8;
+  p.ranked = K <= 32;
   if (p.ranked) {
     p.pc_bits = p.pc_shift = 0;
-    p.code_bits = 8;
-    key_bits = 8 + block_bits;
+    p.code_bits = K;
+    key_bits = K + block_bits;
     return p;
   }
+  // Wider filters (33 .. 62 taps): count of absent taps, then the mask.  Up to 40 key bits (four
+  // sort passes): beyond that the count gives way first, then the mask (hashed).  Measured on
+  // 27-tap tables of a million rows before those were ranked: no count at all costs 2.5-4 % in
+  // every convolution (the heaviest positions no longer come first), a 14-bit hash of the mask 4-7 %.
   int pc_bits = 1;
   while ((1 << pc_bits) <= K) pc_bits++;
-  // Up to 40 key bits (four sort passes; a 27-tap table needs 35): beyond that the count of
-  // absent taps gives way first, then the mask (hashed).  Measured on 27-tap tables of a
-  // million rows: a coarser count (33 bits) gains nothing, no count at all (30 bits, three
-  // passes of 10) saves 10 us of sorting and costs 2.5-4 % in every convolution (the heaviest
-  // positions no longer come first), a 14-bit hash of the mask saves 40 us and costs 4-7 %.
   const int budget = 40;
   p.pc_shift = std::max(0, std::min(pc_bits, block_bits + pc_bits + K - budget));
   p.pc_bits = pc_bits - p.pc_shift;
@@ -1434,15 +1488,22 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
 // ascends with the site's own key: in schedule order the inputs of an output site are neighbours
 // (at most 2^dim of them), the output sites are the runs of equal parent keys, and nothing needs to
 // be sorted.  Two launches make both tables, the output level and the keys of the pattern sort.
-constexpr int HB = 1024;  // positions per workgroup of the two kernels
-__device__ inline unsigned long long parent_key(const Geom &gi, const Geom &go, unsigned long long key, int *tap,
-                                                int *j, int &b) {
-  int p[SCN_MAXD];
+constexpr int HB = 512;  // positions per workgroup of the two kernels
+// shift: the output level's key has one bit less per coordinate (sizes that halve exactly nearly
+// always do), so the parent's key is the site's shifted down by dim bits and the tap, the site's
+// offset inside its output site's 2^dim box, is the bits that fall out.
+__device__ inline unsigned long long parent_key(const Geom &gi, const Geom &go, bool shift, unsigned long long key,
+                                                int *tap) {
+  if (shift) {
+    *tap = (int)(key & ((1u << gi.dim) - 1u));
+    return key >> gi.dim;
+  }
+  int p[SCN_MAXD], j[SCN_MAXD], b;
   site_of_key(gi, key, p, b);
   int k = 0;
   for (int d = 0; d < gi.dim; d++) {
     j[d] = p[d] >> 1;
-    k = 2 * k + (p[d] & 1);  // tap = the site's offset inside its output site's 2^dim box
+    k = 2 * k + (p[d] & 1);
   }
   *tap = k;
   return site_key(go, j, b);
@@ -1457,9 +1518,9 @@ __device__ inline unsigned long long parent_key(const Geom &gi, const Geom &go, 
 // (thousands of workgroups adding to the same few addresses take longer than the rest of the
 // kernel).  The whole chain of levels then costs one read-back instead of one per level.
 // zero: words cleared for the launch behind this one.
-__global__ __launch_bounds__(HB) void k_halve_heads(Geom gi, Geom go, const unsigned long long *keys, int64_t n,
-                                                    int levels, int *block_heads, int *counts, uint32_t *zero,
-                                                    int zero_words) {
+__global__ __launch_bounds__(HB) void k_halve_heads(Geom gi, Geom go, bool shift, const unsigned long long *keys,
+                                                    int64_t n, int levels, int *block_heads, int *counts,
+                                                    uint32_t *zero, int zero_words) {
   __shared__ int hist[64];
   __shared__ int total;
   for (int i = blockIdx.x * HB + threadIdx.x; i < zero_words; i += gridDim.x * HB) zero[i] = 0u;
@@ -1469,9 +1530,9 @@ __global__ __launch_bounds__(HB) void k_halve_heads(Geom gi, Geom go, const unsi
   const int64_t p = (int64_t)blockIdx.x * HB + threadIdx.x;
   int top = -1;  // a new site on levels 0 .. top
   if (p < n) {
-    int tap, j[SCN_MAXD], b;
-    const unsigned long long ck = parent_key(gi, go, keys[p], &tap, j, b);
-    const unsigned long long d = p ? ck ^ parent_key(gi, go, keys[p - 1], &tap, j, b) : ~0ull;
+    int tap;
+    const unsigned long long ck = parent_key(gi, go, shift, keys[p], &tap);
+    const unsigned long long d = p ? ck ^ parent_key(gi, go, shift, keys[p - 1], &tap) : ~0ull;
     if (d) top = p ? min(levels, (63 - __clzll((long long)d)) / gi.dim) : levels;
   }
   const unsigned long long heads = __ballot(top >= 0);
@@ -1492,7 +1553,7 @@ __global__ __launch_bounds__(HB) void k_halve_heads(Geom gi, Geom go, const unsi
 // looks at the up to 2^dim - 1 positions behind it for the site's tap mask, writes -1 into the
 // absent taps of by_out, the site's coordinates and key, and its pattern-sort key
 // (Metadata/ConvolutionRules.h:19-31, Metadata/RectangularRegions.h:30-38,95-105 for this filter).
-__global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, const unsigned long long *keys, const int *sched,
+__global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift, const unsigned long long *keys, const int *sched,
                                                    int64_t n, int64_t npad_in, int64_t npad_out, const int *block_heads,
                                                    int *by_out, int *by_in, int *out_soa, unsigned long long *out_keys,
                                                    unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
@@ -1507,17 +1568,13 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, const unsig
   if (threadIdx.x < 8) lcount[threadIdx.x] = 0;
   const int64_t p = (int64_t)blockIdx.x * HB + threadIdx.x;
   const bool live = p < n;
-  int tap = -1, j[SCN_MAXD], b = 0;
+  int tap = -1;
   unsigned long long ck = 0;
   bool head = false;
   if (live) {
-    ck = parent_key(gi, go, keys[p], &tap, j, b);
-    if (p) {
-      int t2, j2[SCN_MAXD], b2;
-      head = ck != parent_key(gi, go, keys[p - 1], &t2, j2, b2);
-    } else {
-      head = true;
-    }
+    ck = parent_key(gi, go, shift, keys[p], &tap);
+    int t2;
+    head = p == 0 || ck != parent_key(gi, go, shift, keys[p - 1], &t2);
   }
   const unsigned long long heads = __ballot(head);
   if (lane == 0) {
@@ -1535,10 +1592,12 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, const unsig
     if (head) {
       unsigned mask = 1u << tap;
       for (int i = 1; i < K && p + i < n; i++) {
-        int t2, j2[SCN_MAXD], b2;
-        if (parent_key(gi, go, keys[p + i], &t2, j2, b2) != ck) break;
+        int t2;
+        if (parent_key(gi, go, shift, keys[p + i], &t2) != ck) break;
         mask |= 1u << t2;
       }
+      int j[SCN_MAXD], b;
+      site_of_key(go, ck, j, b);
       for (int k = 0; k < K; k++)
         if (!(mask >> k & 1u)) by_out[(int64_t)k * npad_out + o] = -1;
       for (int d = 0; d < gi.dim; d++) out_soa[d * npad_out + o] = j[d];
@@ -1625,7 +1684,8 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     start_counts(R.by_out, s, false);
     const int count_words = 2 * COUNT_SLOTS * f.K;
     if (count) fill32(m.dflags.p, 0, 16 * 64, s);
-    k_halve_heads<<<dim3(blocks), HB, 0, s>>>(LI.g, go, keys, n, chain, m.f0.p, count ? m.dflags.p : nullptr,
+    const bool shift = go.bits == LI.g.bits - 1;
+    k_halve_heads<<<dim3(blocks), HB, 0, s>>>(LI.g, go, shift, keys, n, chain, m.f0.p, count ? m.dflags.p : nullptr,
                                               reinterpret_cast<uint32_t *>(R.by_out.cnt->dev.p), count_words);
     LAUNCH_CHECK();
     if (count) {
@@ -1646,7 +1706,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     int key_bits = 0;
     const PatternKey pk = pattern_plan(n_out, f.K, key_bits);
     reserve_pattern_buffers(m, R.by_out);
-    k_halve_emit<<<dim3(blocks), HB, 0, s>>>(LI.g, go, keys, LI.sched_ptr(), n, LI.npad, LO.npad, m.f0.p, R.by_out.nbr.p,
+    k_halve_emit<<<dim3(blocks), HB, 0, s>>>(LI.g, go, shift, keys, LI.sched_ptr(), n, LI.npad, LO.npad, m.f0.p, R.by_out.nbr.p,
                                              R.by_in.nbr.p, LO.coords.p, LO.keys.p,
                                              (unsigned long long *)R.by_out.cnt->dev.p, pk, m.k0.p, m.v0.p,
                                              reinterpret_cast<unsigned *>(m.f1.p));

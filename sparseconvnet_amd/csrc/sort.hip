@@ -80,6 +80,10 @@ __device__ inline void rank_quarter(const unsigned (&digit)[ITEMS], const bool (
 #pragma unroll
   for (int r = 0; r < ITEMS; r++) {
     u64 peers = __ballot(valid[r]);
+    if (!peers) {  // a round past the end of the input (the whole wavefront agrees)
+      rank[r] = 0;
+      continue;
+    }
     for (int b = 0; b < bits; b++) {
       const u64 has = __ballot((digit[r] >> b) & 1u);
       peers &= ((digit[r] >> b) & 1u) ? has : ~has;
@@ -199,6 +203,94 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict
   }
 }
 
+// Up to RS1_MAX pairs: one workgroup takes them through every digit without leaving LDS, one
+// launch instead of three per digit (the deep levels of a network are a few hundred to a few
+// thousand sites, and what their rulebooks cost is launches).  Sixteen wavefronts each keep a
+// contiguous 256 pairs in registers and rank them as k_rs_scatter does, with digits of up to 8 bits
+// (the prefix over 16 wavefronts' counts of every digit value is what a pass costs here, so fewer
+// values beat fewer passes); the pairs change places through LDS between digits.
+constexpr int RS1_THREADS = 1024, RS1_WAVES = 16, RS1_ITEMS = 4, RS1_MAX = RS1_THREADS * RS1_ITEMS;
+constexpr int RS1_BITS = 8, RS1_BINS = 1 << RS1_BITS;
+__global__ __launch_bounds__(RS1_THREADS) void k_rs_single(const u64 *__restrict__ kin, const int *__restrict__ vin,
+                                                           u64 *__restrict__ kout, int *__restrict__ vout, int n,
+                                                           int end_bit, int width) {
+  constexpr int ITEMS = RS1_ITEMS;
+  __shared__ int cnt[RS1_WAVES][RS1_BINS];
+  __shared__ int lstart[RS1_BINS];
+  __shared__ int wsum[RS1_BINS / 64];
+  __shared__ u64 skey[RS1_MAX];
+  __shared__ int sval[RS1_MAX];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int q0 = wave * (ITEMS * 64);
+  u64 key[ITEMS];
+  int val[ITEMS];
+  unsigned digit[ITEMS];
+  bool valid[ITEMS];
+  int rank[ITEMS];
+#pragma unroll
+  for (int r = 0; r < ITEMS; r++) {
+    const int i = q0 + r * 64 + lane;
+    valid[r] = i < n;
+    key[r] = valid[r] ? kin[i] : 0ull;
+    val[r] = valid[r] ? vin[i] : 0;
+  }
+  for (int shift = 0; shift < end_bit; shift += width) {
+    const int bits = min(width, end_bit - shift), bins = 1 << bits;
+    const unsigned mask = (unsigned)bins - 1u;
+    for (int e = threadIdx.x; e < RS1_WAVES * bins; e += RS1_THREADS) cnt[e / bins][e % bins] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) digit[r] = (unsigned)(key[r] >> shift) & mask;
+    rank_quarter<ITEMS>(digit, valid, bits, cnt[wave], lane, rank);
+    __syncthreads();
+    // thread d < bins: the counts of value d become their exclusive prefix over the wavefronts;
+    // then an exclusive scan of the totals over d (the first bins / 64 wavefronts)
+    int total = 0;
+    if (threadIdx.x < bins) {
+      for (int w = 0; w < RS1_WAVES; w++) {
+        const int c = cnt[w][threadIdx.x];
+        cnt[w][threadIdx.x] = total;
+        total += c;
+      }
+    }
+    int incl = total;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63 && wave < RS1_BINS / 64) wsum[wave] = incl;
+    __syncthreads();
+    if (threadIdx.x < bins) {
+      int run = incl - total;
+      for (int w = 0; w < wave; w++) run += wsum[w];
+      lstart[threadIdx.x] = run;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+      if (!valid[r]) continue;
+      const int at = lstart[digit[r]] + cnt[wave][digit[r]] + rank[r];
+      skey[at] = key[r];
+      sval[at] = val[r];
+    }
+    __syncthreads();
+    if (shift + width < end_bit) {  // the pairs of this wavefront's range for the next digit
+#pragma unroll
+      for (int r = 0; r < ITEMS; r++) {
+        const int i = q0 + r * 64 + lane;
+        key[r] = valid[r] ? skey[i] : 0ull;
+        val[r] = valid[r] ? sval[i] : 0;
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = threadIdx.x; i < n; i += RS1_THREADS) {
+    kout[i] = skey[i];
+    vout[i] = sval[i];
+  }
+}
+
 void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, int *vout, int64_t n, int end_bit,
                       hipStream_t s) {
   if (n <= 0) return;
@@ -207,6 +299,12 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
   // as few digits as RS_MAX_BITS bits each allow, of equal width
   const int passes = (end_bit + RS_MAX_BITS - 1) / RS_MAX_BITS;
   const int width = (end_bit + passes - 1) / passes;
+  if (n <= RS1_MAX) {
+    const int p1 = (end_bit + RS1_BITS - 1) / RS1_BITS;
+    k_rs_single<<<dim3(1), RS1_THREADS, 0, s>>>(kin, vin, kout, vout, (int)n, end_bit, (end_bit + p1 - 1) / p1);
+    LAUNCH_CHECK();
+    return;
+  }
   // Large inputs take tiles of 4096 pairs (longer runs per digit value in the scatter's stores: a
   // million pairs of 35 bits 145 -> 122 us, eight million 800 -> 490 us); below half a million pairs
   // there are too few of those to fill the chip and 2048-pair tiles are faster.

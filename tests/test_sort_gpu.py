@@ -10,7 +10,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("n,bits", [(1, 8), (63, 3), (4096, 16), (4097, 16), (2048 * 3 + 5, 24), (100003, 36),
-                                    (1 << 20, 40), (300000, 64), (70000, 1), (5000, 9), (2500000, 33)])
+                                    (1 << 20, 40), (300000, 64), (70000, 1), (5000, 9), (2500000, 33),
+                                    (1000, 27), (4095, 35), (3001, 64), (2, 1)])
 def test_sort_pairs(n, bits):
     import torch
     from sparseconvnet_amd import _lib
