@@ -69,6 +69,12 @@ int scn_md_set_bf16(scn_metadata *md, int enable);
  * (family and tile shape, e.g. "rows ncb=6 rg=1 ss=2 nw=4 split=1"), for benchmark tables and
  * profiles.  The pointer stays valid until the handle's next convolution call. */
 const char *scn_md_last_conv_kernel(scn_metadata *md);
+/* No counterpart in the reference (its JoinTable copies, sparseconvnet/tables.py:35-48): the next
+ * convolution call on this handle (scn_subm_conv_fwd, scn_conv_fwd, scn_deconv_fwd, scn_conv_bn_fwd,
+ * scn_nin_fwd) writes its output rows `stride` floats apart instead of nOut, so that a caller can
+ * have it fill a range of columns of a wider matrix (the part of a concatenation that the
+ * convolution produces).  stride >= nOut, nOut <= 256; it serves one call and 0 switches it off. */
+int scn_md_next_output_stride(scn_metadata *md, int64_t stride);
 /* Metadata::inputLayer (Metadata/Metadata.cpp:413-425, Metadata/IOLayersRules.h:18-121).
  * coords: device int64 [n, ncols], ncols = dim (one sample) or dim+1 (last column = sample
  * index).  mode 0: rows = input order, no merging; 1: first, 2: last, 3: sum, 4: mean of the

@@ -20,11 +20,17 @@ class Sequential(torch.nn.Sequential):
         return out
 
     def forward(self, input):
-        # Same chain as sequential.py:10-35, except that eval-mode batch normalisations next
-        # to a convolution are applied inside that convolution (layers.fuse_plan) and one behind a
-        # JoinTable while the parts are joined (layers.join_batchnorm).
-        from .layers import fuse_plan, join_batchnorm
-        mods = self._chain()
+        return self._run(self._chain(), input)
+
+    @staticmethod
+    def _run(mods, input, tail=None):
+        """Same chain as sequential.py:10-35, except that eval-mode batch normalisations next
+        to a convolution are applied inside that convolution (layers.fuse_plan), one behind a
+        JoinTable while the parts are joined (layers.join_batchnorm), and one behind a ConcatTable
+        and a JoinTable by whatever produces each part (layers.concat_join_batchnorm).
+        tail: (batch norm arguments, output columns) for the convolution that ends `mods`: it
+        applies that batch norm to its output and writes it into those columns."""
+        from .layers import fuse_plan, join_batchnorm, concat_join_batchnorm
         i = 0
         while i < len(mods):
             if type(mods[i]) is JoinTable and i + 1 < len(mods) and isinstance(input, (list, tuple)) \
@@ -34,13 +40,26 @@ class Sequential(torch.nn.Sequential):
                     input = joined
                     i += 2
                     continue
+            if type(mods[i]) is ConcatTable and i + 2 < len(mods) and type(mods[i + 1]) is JoinTable \
+                    and not any(m._forward_hooks or m._forward_pre_hooks for m in mods[i:i + 2]):
+                joined = concat_join_batchnorm(mods[i], mods[i + 2], input)
+                if joined is not None:
+                    input = joined
+                    i += 3
+                    continue
             plan = fuse_plan(mods[i:i + 3], input) if isinstance(input, SparseConvNetTensor) else None
             if plan is None:
-                input = mods[i](input)
+                if tail is not None and i == len(mods) - 1:
+                    input = mods[i](input, post_bn=tail[0], out=tail[1])
+                else:
+                    input = mods[i](input)
                 i += 1
             else:
                 conv, pre, post, used = plan
-                input = conv(input, pre_bn=pre, post_bn=post)
+                if tail is not None and i + used == len(mods) and post is None:
+                    input = conv(input, pre_bn=pre, post_bn=tail[0], out=tail[1])
+                else:
+                    input = conv(input, pre_bn=pre, post_bn=post)
                 i += used
         return input
 

@@ -517,6 +517,12 @@ int scn_set_build_stream(int enable) {
 int scn_md_set_bf16(scn_metadata *h, int enable) {
   return guarded([&] { md(h).bf16 = enable != 0; });
 }
+int scn_md_next_output_stride(scn_metadata *h, int64_t stride) {
+  return guarded([&] {
+    if (stride < 0) throw Error("output stride must not be negative");
+    md(h).next_out_stride = stride;
+  });
+}
 const char *scn_md_last_conv_kernel(scn_metadata *h) { return h ? h->m.last_kernel.c_str() : ""; }
 int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *coords, int64_t n,
                        int ncols, int min_batch, int mode, void *stream, int64_t *n_active) {

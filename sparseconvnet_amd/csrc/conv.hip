@@ -111,7 +111,7 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
   }
   if (epi.sc) acc = epi_act(acc, epi.sc[oc], epi.sh[oc], epi.leak);
   int64_t row = rowmap ? rowmap[t] : t;
-  out[row * n_out + oc] = acc;
+  out[row * (epi.out_stride ? epi.out_stride : n_out) + oc] = acc;
 }
 
 // ---- weight packing ---------------------------------------------------------------------
@@ -289,9 +289,12 @@ __global__ void k_take_columns(const float *w, int64_t rows, int n_out, int c0, 
 void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_rows, float *out, const float *w,
                   const float *bias, int n_in, int n_out, int groups, const BnArgs *bn, const BnArgs *post,
                   hipStream_t s) {
-  struct FrozenReset {  // a frozen set serves one call
+  struct FrozenReset {  // a frozen set and an output stride serve one call
     Metadata &m;
-    ~FrozenReset() { m.frozen = nullptr; }
+    ~FrozenReset() {
+      m.frozen = nullptr;
+      m.next_out_stride = 0;
+    }
   } frozen_reset{m};
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
     throw Error("channel counts must be positive multiples of groups");
@@ -304,6 +307,11 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     throw Error("allocation-free convolution: at most 256 output planes");
   Epi epi;
   epi.bias = bias;
+  if (m.next_out_stride) {
+    if (m.next_out_stride < n_out || m.next_out_stride > INT32_MAX) throw Error("output stride below the plane count");
+    if (n_out > 256 || m.fixed_scratch) throw Error("output stride: at most 256 output planes, not with the allocation-free entry");
+    epi.out_stride = (int)m.next_out_stride;
+  }
   m.jobs = CoefJobs();
   m.cur_in_rows = n_in_rows;
   m.cur_in_base = in;

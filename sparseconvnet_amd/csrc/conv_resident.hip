@@ -291,7 +291,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
           const int64_t pos = t0 + q * 16 + 4 * g + r;
           if (pos < n) {
             const int64_t row = rowmap ? rowmap[pos] : pos;
-            float *o = out + row * n_out;
+            float *o = out + row * (epi.out_stride ? epi.out_stride : n_out);
 #pragma unroll
             for (int cb = 0; cb < NCB; cb++) {
               const int col = 16 * cb + r16;
@@ -420,7 +420,7 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
 template <int NCB>
 static void launch_resident_c4(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                                Epi epi, int n_in, int n_out, hipStream_t s) {
-  if (in == m.cur_in_base && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
+  if (in == m.cur_in_base && !epi.out_stride && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
     // epi.sc / epi.sh point at arrays nobody fills on this path: the kernel folds the batch norm itself
     take_jobs(m);
     note_kernel(m, "first", {{"nin", n_in}});
@@ -472,6 +472,7 @@ bool try_resident(Metadata &m, const Table &t, const float *in, float *out, cons
     const float *w_p = w + (int64_t)c_lo * n_out;
     const int acc = c_lo > 0;
     Epi b;  // bias with the first part, the following layer's batch norm with the last
+    b.out_stride = epi.out_stride;
     if (!acc) b.bias = epi.bias;
     if (c_lo + 32 >= n_in) {
       b.sc = epi.sc;

@@ -207,6 +207,7 @@ struct Metadata {
   DevBuf<float> wcols;  // column ranges of a wide layer's weights, one contiguous block per range (conv_forward)
   DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
+  int64_t next_out_stride = 0;  // floats between the output rows of the next convolution call (0: its plane count); serves one call
   DevBuf<unsigned long long> ticket;  // [0]: arrival ticket of grid_count (zero between launches), [1]: the count
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
   DevBuf<float> partial;  // partial tiles of a convolution whose taps are split over workgroups; partial sums of reductions
@@ -287,7 +288,7 @@ struct Epi {
   const float *bias = nullptr;               // [nOut] or null
   const float *sc = nullptr, *sh = nullptr;  // [nOut] each, or nulls
   float leak = 1.0f;
-  int out_stride = 0;  // floats between output rows; 0: nOut (k_conv_mfma, k_conv_rows, k_conv_reduce honour it)
+  int out_stride = 0;  // floats between output rows; 0: nOut
 };
 __device__ inline float epi_act(float v, float sc, float sh, float leak) {
   const float y = v * sc + sh;

@@ -75,12 +75,12 @@ class _ConvFunction(Function):
     1 / 2.  pre / post: eval-mode batch norms applied inside the convolution (inference only)."""
 
     @staticmethod
-    def forward(ctx, features, weight, bias, md, kind, sizes, pre, post):
+    def forward(ctx, features, weight, bias, md, kind, sizes, pre, post, out=None):
         ctx.md, ctx.kind, ctx.sizes, ctx.fused = md, kind, sizes, pre is not None or post is not None
         ctx.has_bias = bias.numel() > 0
         ctx.save_for_backward(features, weight)
         fn = (md.submanifoldConvolution, md.convolution, md.deconvolution)[kind]
-        out, _ = fn(*sizes, features, weight, bias, pre, post, want_macs=False)
+        out, _ = fn(*sizes, features, weight, bias, pre, post, want_macs=False, out=out)
         _count(out)
         return out
 
@@ -91,7 +91,7 @@ class _ConvFunction(Function):
         features, weight = ctx.saved_tensors
         fn = (ctx.md.submanifoldConvolutionBackward, ctx.md.convolutionBackward, ctx.md.deconvolutionBackward)[ctx.kind]
         d_in, d_w, d_b = fn(*ctx.sizes, features, grad_output.contiguous(), weight, ctx.has_bias)
-        return d_in, d_w, d_b, None, None, None, None, None
+        return d_in, d_w, d_b, None, None, None, None, None, None
 
 
 class _NetworkInNetworkFunction(Function):
@@ -175,6 +175,57 @@ def join_batchnorm(parts, bn):
     output.spatial_size = parts[0].spatial_size
     output.features = _JoinBatchNormFunction.apply(bn.running_mean, bn.running_var, optionalTensor(bn, 'weight').detach(),
                                                    optionalTensor(bn, 'bias').detach(), bn.eps, bn.leakiness, *feats)
+    return output
+
+
+def _bn_slice(bn, lo, hi):
+    """The arguments _bn_args gives, for planes [lo, hi) of the batch normalisation."""
+    w, b = optionalTensor(bn, 'weight').detach(), optionalTensor(bn, 'bias').detach()
+    return (bn.running_mean[lo:hi], bn.running_var[lo:hi], w[lo:hi] if w.numel() else w, b[lo:hi] if b.numel() else b,
+            bn.eps, bn.leakiness)
+
+
+def concat_join_batchnorm(table, bn, input):
+    """ConcatTable `table`, JoinTable and the eval-mode batch normalisation `bn` run on `input` with
+    no pass over the joined matrix: when the table's last branch ends in a convolution (the
+    Deconvolution of a U-Net level), that convolution applies its planes' share of the batch norm
+    to its output and writes it straight into its columns of the joined matrix; the other
+    branches' results are normalised into theirs as join_batchnorm does.  None when this does not
+    apply (the caller then runs the three modules one after the other).  Inference only."""
+    from .containers import Sequential
+    if not _pkg.fuse_batchnorm or torch.is_grad_enabled() or not _is_bn(bn) or not isinstance(input, SparseConvNetTensor):
+        return None
+    children = list(table._modules.values())
+    if len(children) < 2 or input.features.nelement() == 0:
+        return None
+    last = children[-1]
+    if type(last) is not Sequential or last._forward_hooks or last._forward_pre_hooks:
+        return None
+    chain = last._chain()
+    if not chain or not _is_conv(chain[-1]) or chain[-1].nOut > 256:
+        return None
+    conv = chain[-1]
+    parts = [c(input) for c in children[:-1]]
+    feats = [p.features for p in parts]
+    rows = feats[0].size(0) if feats[0].dim() == 2 else -1
+    fits = all(f.dim() == 2 and f.size(0) == rows and f.nelement() for f in feats) and \
+        sum(f.size(1) for f in feats) + conv.nOut == bn.nPlanes
+    if not fits:  # as the modules by themselves would
+        parts.append(last(input))
+        from .containers import JoinTable
+        return bn(JoinTable()(parts))
+    out = feats[0].new_empty((rows, bn.nPlanes))
+    off = 0
+    for f in feats:
+        c = f.size(1)
+        mean, var, w, b, eps, leak = _bn_slice(bn, off, off + c)
+        _md.batchNormEval(f, mean, var, _opt(w), _opt(b), eps, leak, out=out[:, off:off + c])
+        off += c
+    Sequential._run(chain, input, tail=(_bn_slice(bn, off, bn.nPlanes), out[:, off:]))
+    output = SparseConvNetTensor()
+    output.metadata = parts[0].metadata
+    output.spatial_size = parts[0].spatial_size
+    output.features = out
     return output
 
 
@@ -288,8 +339,8 @@ def _count(out):
 def _bn_args(bn):
     """The tensors and constants of an eval-mode BatchNormalization module that a convolution
     applies to its input rows itself (None: nothing to apply)."""
-    if bn is None:
-        return None
+    if bn is None or isinstance(bn, tuple):
+        return bn
     return (bn.running_mean, bn.running_var, optionalTensor(bn, 'weight').detach(),
             optionalTensor(bn, 'bias').detach(), bn.eps, bn.leakiness)
 
@@ -343,7 +394,7 @@ class SubmanifoldConvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None, post_bn=None):
+    def forward(self, input, pre_bn=None, post_bn=None, out=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, self.nOut, input)
         output = SparseConvNetTensor()
         output.metadata = input.metadata
@@ -351,7 +402,7 @@ class SubmanifoldConvolution(Module):
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 0,
-                                              (input.spatial_size, self.filter_size), pre, post)
+                                              (input.spatial_size, self.filter_size), pre, post, out)
         return output
 
     def __repr__(self):
@@ -381,7 +432,7 @@ class Convolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None, post_bn=None):
+    def forward(self, input, pre_bn=None, post_bn=None, out=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
@@ -393,7 +444,7 @@ class Convolution(Module):
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 1,
-                                              a, pre, post)
+                                              a, pre, post, out)
         return output
 
     def __repr__(self):
@@ -420,7 +471,7 @@ class Deconvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None, post_bn=None):
+    def forward(self, input, pre_bn=None, post_bn=None, out=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
@@ -429,7 +480,7 @@ class Deconvolution(Module):
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 2,
-                                              a, pre, post)
+                                              a, pre, post, out)
         return output
 
     def __repr__(self):

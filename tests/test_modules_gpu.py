@@ -835,3 +835,83 @@ def test_frozen_parameters_follow_training_mode_batch_norm():
     finally:
         scn.frozen_parameters = True
     assert torch.equal(after, want)
+
+
+@pytest.mark.parametrize("n_in,n_out", [(3, 16), (16, 16), (32, 64), (64, 32), (160, 160), (20, 24)])
+def test_convolution_writes_into_columns_of_a_wider_matrix(n_in, n_out):
+    """`out=` (scn_md_next_output_stride): the convolution fills a range of columns of a wider matrix
+    and leaves the columns around it alone; the stride serves that one call."""
+    coords = synthetic.scene_batch(seed=8100 + n_in, batch=2, target=9000, spatial=64, n_boxes=8)
+    g = torch.Generator().manual_seed(n_in * 1000 + n_out)
+    feats = torch.rand(len(coords), n_in, generator=g).cuda()
+    t = scn.InputLayer(3, 64, mode=4)([torch.as_tensor(coords), feats])
+    md, size, three, two = t.metadata, t.spatial_size, torch.LongTensor([3] * 3), torch.LongTensor([2] * 3)
+    n = t.features.size(0)
+    w = (torch.randn(27, 1, n_in, n_out, generator=g) * (2.0 / (27 * n_in)) ** 0.5).cuda()
+    bias = torch.randn(n_out, generator=g).cuda()
+    bn = (torch.randn(n_out, generator=g).cuda(), torch.rand(n_out, generator=g).cuda() + 0.5,
+          torch.rand(n_out, generator=g).cuda() + 0.5, torch.randn(n_out, generator=g).cuda(), 1e-4, 0.1)
+    for post in (None, bn):
+        plain, _ = md.submanifoldConvolution(size, three, t.features, w, bias, post=post, want_macs=False)
+        wide = torch.full((n, n_out + 24), 7.0, device="cuda")
+        got, _ = md.submanifoldConvolution(size, three, t.features, w, bias, post=post, want_macs=False,
+                                           out=wide[:, 8:8 + n_out])
+        assert got.data_ptr() == wide[:, 8:].data_ptr()
+        checks.assert_close(wide[:, 8:8 + n_out].cpu().numpy(), plain.cpu().numpy(), "columns of the wide matrix")
+        assert (wide[:, :8] == 7.0).all() and (wide[:, 8 + n_out:] == 7.0).all()
+        again, _ = md.submanifoldConvolution(size, three, t.features, w, bias, post=post, want_macs=False)
+        assert again.is_contiguous() and torch.equal(again, plain), "the stride must not outlive its call"
+    # strided and transposed convolutions (8 taps): down to the coarse level and back up
+    half = (size - 2) // 2 + 1
+    w2 = (torch.randn(8, 1, n_in, n_out, generator=g) * (2.0 / (8 * n_in)) ** 0.5).cuda()
+    down, _ = md.convolution(size, half, two, two, t.features, w2, None, want_macs=False)
+    wide = torch.full((down.size(0), n_out + 16), -3.0, device="cuda")
+    md.convolution(size, half, two, two, t.features, w2, None, want_macs=False, out=wide[:, 16:])
+    checks.assert_close(wide[:, 16:].cpu().numpy(), down.cpu().numpy(), "strided convolution into columns")
+    assert (wide[:, :16] == -3.0).all()
+    w3 = (torch.randn(8, 1, n_out, n_in, generator=g) * (2.0 / (8 * n_out)) ** 0.5).cuda()
+    up, _ = md.deconvolution(half, size, two, two, down, w3, None, want_macs=False)
+    wide = torch.full((n, n_in + 8), 2.0, device="cuda")
+    md.deconvolution(half, size, two, two, down, w3, None, want_macs=False, out=wide[:, :n_in])
+    checks.assert_close(wide[:, :n_in].cpu().numpy(), up.cpu().numpy(), "transposed convolution into columns")
+    assert (wide[:, n_in:] == 2.0).all()
+
+
+def test_unet_level_joins_without_a_pass_over_the_joined_matrix():
+    """ConcatTable + JoinTable + eval-mode batch norm (every level of a U-Net): the Deconvolution
+    that ends the inner branch normalises its own planes into its columns of the joined matrix.
+    Same result as the three modules one after the other, and the path is the one taken."""
+    from sparseconvnet_amd import layers
+    torch.manual_seed(11)
+    m = 16
+    model = scn.Sequential().add(scn.SubmanifoldConvolution(3, 3, m, 3, False)).add(
+        scn.UNet(3, 2, [m, 2 * m, 3 * m], False, leakiness=0.1)).add(scn.BatchNormReLU(m)).add(
+        scn.OutputLayer(3)).cuda().eval()
+    randomise_bn(model, 11)
+    coords = synthetic.scene_batch(seed=11000, batch=2, target=8000, spatial=64, n_boxes=8, duplicate_fraction=0.2)
+    feats = torch.rand(len(coords), 3).cuda()
+    inp_layer = scn.InputLayer(3, 64, mode=4)
+    orig, taken = layers.concat_join_batchnorm, []
+
+    def counting(table, bn, input):
+        r = orig(table, bn, input)
+        taken.append(r is not None)
+        return r
+    outs = []
+    try:
+        for fn in (counting, lambda table, bn, input: None):
+            layers.concat_join_batchnorm = fn
+            with torch.no_grad():
+                outs.append(model(inp_layer([torch.as_tensor(coords), feats])).cpu().numpy())
+    finally:
+        layers.concat_join_batchnorm = orig
+    assert taken == [True, True], taken  # two levels with an inner branch
+    checks.assert_close(outs[0], outs[1], "joined by the producers vs joined by a pass")
+    # with gradients enabled the modules run one after the other
+    taken.clear()
+    layers.concat_join_batchnorm = counting
+    try:
+        model(inp_layer([torch.as_tensor(coords), feats]))
+    finally:
+        layers.concat_join_batchnorm = orig
+    assert taken == [False, False], taken
