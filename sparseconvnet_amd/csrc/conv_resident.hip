@@ -74,10 +74,19 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
   auto set_of = [&](int i) { return min(spread ? (i - set_begin) * 8 + xcd : i, n_sets - 1); };
   const int first_round = blocks_per_xcd * WAVES;
   int *ctr = queue + xcd * 32;
+  // Tables of few taps (strided and transposed convolutions: a set is one or a few items) take
+  // eight sets per visit of the counter: one same-address atomic per set costs more than the set.
+  const int chunk = K <= 8 ? 8 : 1;
+  int chunk_next = 0, chunk_left = 0;
   auto take = [&]() {
-    int v = 0;
-    if (lane == 0) v = atomicAdd(ctr, 1);
-    return set_begin + first_round + __builtin_amdgcn_readfirstlane(v);
+    if (chunk_left == 0) {
+      int v = 0;
+      if (lane == 0) v = atomicAdd(ctr, chunk);
+      chunk_next = set_begin + first_round + __builtin_amdgcn_readfirstlane(v);
+      chunk_left = chunk;
+    }
+    chunk_left--;
+    return chunk_next++;
   };
   // generator of the item stream (wave-uniform state)
   int g_set = set_begin + blk * WAVES + wave;
@@ -447,7 +456,9 @@ bool resident_fits(const Metadata &m, const Table &t, int n_in, int n_out, bool 
   // variant is faster (measured)
   if (m.bf16 && n_in >= 64 && n_in % 32 == 0) return false;
   // several parts re-read and re-write the output once per part: with few taps (strided and
-  // transposed convolutions) that costs more than the convolution itself
+  // transposed convolutions) that costs more than the convolution itself (and 64 planes as one part
+  // of four slabs, whose weights still fit LDS, measured 115 us against the row-owner kernel's 94
+  // for 64 -> 32 up to a million rows: a set of one tap is too small an item for this pipeline)
   if (n_in > 32 && t.K <= 8) return false;
   (void)with_bn;
   return n_in < 64;  // two parts and more: the row-owner kernel is 3 % (64 -> 32) to 10 % (96 -> 32) faster at 1 M sites
