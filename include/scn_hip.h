@@ -363,7 +363,9 @@ int scn_nin_bwd(scn_metadata *md, const float *in, float *d_in, const float *d_o
  * running_var updated in place as momentum * old + (1 - momentum) * batch value (unbiased
  * variance); out = leaky(x * w + b) with the batch statistics.  The reference call takes no
  * metadata; here the handle owns the scratch of the column reductions (any handle will do; the
- * caller has the tensor's at hand). */
+ * caller has the tensor's at hand).  rows == 0: save_mean and save_invstd are set to 0 and the
+ * running statistics stay as they are (the reference divides by zero).  rows == 1: the unbiased
+ * variance divides by rows - 1 = 0 and running_var becomes inf or nan, as in the reference. */
 int scn_bn_train_fwd(scn_metadata *md, const float *in, float *out, int64_t rows, int planes,
                      int64_t in_stride, int64_t out_stride, float *save_mean, float *save_invstd,
                      float *running_mean, float *running_var, const float *gamma, const float *beta,

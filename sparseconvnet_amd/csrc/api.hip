@@ -29,6 +29,7 @@ std::mutex g_pool_mutex;
 struct IdleBlock {
   void *p;
   hipStream_t last;
+  bool known;  // false: freed outside any call, by an owner that did not say where it was last used
 };
 std::multimap<std::tuple<int, int, size_t>, IdleBlock> g_pool;  // (device, cache, bytes) -> idle blocks
 std::unordered_map<void *, size_t> g_block_bytes;                // every block the cache has handed out or holds
@@ -109,7 +110,8 @@ void *pool_alloc(size_t bytes, int pool) {
       g_live_bytes += (int64_t)got;
       lock.unlock();
       const ThreadStreams &t = thread_streams();
-      if (t.known[pool] && t.s[pool] != b.last) order_streams(b.last, t.s[pool]);
+      if (!b.known) (void)hipDeviceSynchronize();
+      else if (t.known[pool] && t.s[pool] != b.last) order_streams(b.last, t.s[pool]);
       return b.p;
     }
   }
@@ -142,7 +144,7 @@ void pool_free(void *p, size_t bytes, int pool) {
   const size_t got = it != g_block_bytes.end() ? it->second : size_class(bytes ? bytes : 1);
   g_live_bytes -= (int64_t)got;
   g_idle_bytes += (int64_t)got;
-  g_pool.emplace(std::make_tuple(dev, pool, got), IdleBlock{p, thread_streams().s[pool]});
+  g_pool.emplace(std::make_tuple(dev, pool, got), IdleBlock{p, thread_streams().s[pool], thread_streams().known[pool]});
 }
 }  // namespace scn
 
@@ -923,10 +925,18 @@ scn_params *scn_params_create(void) {
     return nullptr;
   }
 }
-void scn_params_destroy(scn_params *p) { delete p; }
+// A parameter set's buffers go back to the cache tagged with the stream they were last used on.
+static void tag_params_stream(scn_params *p) {
+  if (p && p->p.last_known) pool_set_stream(POOL_COMPUTE, p->p.last);
+}
+void scn_params_destroy(scn_params *p) {
+  tag_params_stream(p);
+  delete p;
+}
 int scn_params_clear(scn_params *p) {
   return guarded([&] {
     if (!p) throw Error("null parameter set");
+    tag_params_stream(p);
     p->p.clear();
   });
 }

@@ -910,7 +910,12 @@ void bn_train_forward(Metadata *scratch, const float *in, float *out, int64_t ro
                       int64_t out_stride, float *save_mean, float *save_invstd, float *running_mean,
                       float *running_var, const float *gamma, const float *beta, float eps, float momentum,
                       float leak, hipStream_t s) {
-  if (rows <= 0 || planes <= 0) return;
+  if (planes <= 0) return;
+  if (rows <= 0) {  // no rows: defined statistics (the reference divides by zero here), running ones untouched
+    fill32(save_mean, 0, planes, s);
+    fill32(save_invstd, 0, planes, s);
+    return;
+  }
   Metadata &m = *scratch;
   const ColsumPlan p = colsum_plan(rows, planes);
   m.partial.reserve((size_t)p.blocks * 2 * planes);

@@ -294,6 +294,8 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     ~FrozenReset() {
       m.frozen = nullptr;
       m.next_out_stride = 0;
+      m.before_pack = nullptr;
+      m.wkey_ptr = 0;
     }
   } frozen_reset{m};
   if (groups < 1 || n_in < 1 || n_out < 1 || n_in % groups || n_out % groups)
@@ -316,6 +318,10 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
   m.cur_in_rows = n_in_rows;
   m.cur_in_base = in;
   FrozenParams *frozen = m.fixed_scratch ? nullptr : m.frozen;
+  if (frozen) {
+    frozen->last = s;
+    frozen->last_known = true;
+  }
   m.post_raw = CoefJob();
   if (post) {
     DevBuf<float> &buf = frozen ? frozen->post : m.postbuf;
@@ -374,13 +380,22 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     for (int c0 = 0; c0 < n_out && ok; c0 += width) {
       const int wc = std::min(width, n_out - c0);
       float *dst = m.wcols.p + rows_w * c0;
-      k_take_columns<<<dim3((unsigned)ceil_div(rows_w * wc, 256)), 256, 0, s>>>(w, rows_w, n_out, c0, wc, dst);
-      LAUNCH_CHECK();
+      // the copy runs when a kernel packs from it: not when a frozen set already holds the packed range
+      m.before_pack = [=] {
+        k_take_columns<<<dim3((unsigned)ceil_div(rows_w * wc, 256)), 256, 0, s>>>(w, rows_w, n_out, c0, wc, dst);
+        LAUNCH_CHECK();
+      };
+      m.wkey_ptr = (int64_t)(uintptr_t)(w + rows_w * c0);
+      m.wkey_from = (int64_t)(uintptr_t)dst;
+      m.wkey_c0 = c0;
+      m.wkey_wc = wc;
       Epi e = epi;
       if (e.bias) e.bias += c0;
       if (e.sc) e.sc += c0, e.sh += c0;
       e.out_stride = n_out;
       ok = conv_mfma_paths<false>(m, t, src, out + c0, dst, e, n_in, wc, PreArgs(), s);
+      m.before_pack = nullptr;
+      m.wkey_ptr = 0;
       m.last_kernel += " +";  // the next range's kernel is appended
     }
     if (ok) return;

@@ -22,15 +22,26 @@ float *scratch_partial(Metadata &m, int &n_split, int64_t split_stride_floats);
 // the handle's scratch on every call.
 template <class F>
 static float *packed_weights(Metadata &m, std::vector<int64_t> key, size_t floats, F pack) {
+  auto first = [&] {
+    if (m.before_pack) m.before_pack();
+    m.before_pack = nullptr;
+  };
   if (m.frozen && !m.fixed_scratch) {
+    if (m.wkey_ptr) {  // a column range: keyed by where it lies in the caller's weights, not by the scratch copy's address
+      key[1] += m.wkey_ptr - m.wkey_from;
+      key.push_back(m.wkey_c0);
+      key.push_back(m.wkey_wc);
+    }
     auto it = m.frozen->packed.find(key);
     if (it != m.frozen->packed.end() && it->second.cap >= floats) return it->second.p;
     DevBuf<float> &b = m.frozen->packed[key];
     b.reserve(floats);
+    first();
     pack(b.p);
     return b.p;
   }
   float *dst = scratch_wpack(m, floats);
+  first();
   pack(dst);
   return dst;
 }

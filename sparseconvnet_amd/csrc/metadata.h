@@ -1,6 +1,7 @@
 // Host-side state behind a scn_metadata handle: levels (one per spatial size), the input
 // layer's rule lists and the cached neighbour tables.
 #pragma once
+#include <functional>
 #include <map>
 #include <memory>
 
@@ -124,6 +125,8 @@ struct FrozenParams {
   std::map<std::vector<int64_t>, DevBuf<float>> packed;
   DevBuf<float> pre, post;   // scale | shift arrays, as conv_forward lays them out
   bool pre_done = false, post_done = false;
+  hipStream_t last = nullptr;  // the stream of the last convolution that used the set
+  bool last_known = false;
   void clear() {
     packed.clear();
     pre.release();
@@ -207,6 +210,10 @@ struct Metadata {
   DevBuf<float> wcols;  // column ranges of a wide layer's weights, one contiguous block per range (conv_forward)
   DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
+  std::function<void()> before_pack;  // work the packing of the running convolution's weights needs first (the column-range path's copy), run at most once
+  // while a column range of a wide layer runs: addresses in the scratch copy (from wkey_from) stand for
+  // addresses from wkey_ptr in the caller's weights in a frozen set's keys
+  int64_t wkey_ptr = 0, wkey_from = 0, wkey_c0 = 0, wkey_wc = 0;
   int64_t next_out_stride = 0;  // floats between the output rows of the next convolution call (0: its plane count); serves one call
   DevBuf<unsigned long long> ticket;  // [0]: arrival ticket of grid_count (zero between launches), [1]: the count
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order

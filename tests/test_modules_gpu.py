@@ -915,3 +915,42 @@ def test_unet_level_joins_without_a_pass_over_the_joined_matrix():
     finally:
         layers.concat_join_batchnorm = orig
     assert taken == [False, False], taken
+
+
+def test_frozen_parameters_of_a_wide_layer_do_not_grow():
+    """More than 256 output planes run as column ranges over a scratch copy of the weights.  The
+    frozen set keys those ranges by where they lie in the module's weights, not by the scratch
+    address: over a stream of scenes (a new Metadata each, scratch at changing addresses) the
+    results stay those of the uncached path and the memory the library holds stops growing."""
+    import ctypes as C
+    from sparseconvnet_amd import _lib
+    torch.manual_seed(14)
+    conv = scn.SubmanifoldConvolution(3, 16, 320, 3, True).cuda().eval()
+    with torch.no_grad():
+        conv.bias.normal_()
+    layer = scn.InputLayer(3, 64, mode=4)
+    L = _lib.lib()
+
+    def live():
+        torch.cuda.synchronize()
+        a, b = C.c_int64(0), C.c_int64(0)
+        _lib.check(L.scn_cache_stats(C.byref(a), C.byref(b), None, None))
+        return a.value
+
+    def run(seed):
+        coords = synthetic.scene_batch(seed=seed, batch=1, target=3000 + 500 * (seed % 3), spatial=64, n_boxes=6)
+        feats = torch.rand((len(coords), 16), device="cuda", generator=torch.Generator(device="cuda").manual_seed(seed))
+        with torch.no_grad():
+            return conv(layer([torch.as_tensor(coords), feats])).features.clone()
+
+    scn.frozen_parameters = False
+    try:
+        want = [run(s) for s in range(3)]
+    finally:
+        scn.frozen_parameters = True
+    sizes = []
+    for rep in range(4):
+        for s in range(3):
+            assert torch.equal(run(s), want[s]), (rep, s)
+        sizes.append(live())
+    assert sizes[1] == sizes[2] == sizes[3], sizes
