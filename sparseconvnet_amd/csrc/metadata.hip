@@ -561,20 +561,76 @@ __global__ void k_sorted_keys(const unsigned long long *keys, const int *sched, 
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t < n) skey[t] = keys[sched ? sched[t] : t];
 }
-// Distinct sites: flag the last position of every run of equal keys.
-__global__ void k_run_tails(const unsigned long long *skey, int64_t n, int *tail) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t < n) tail[t] = (t == n - 1 || skey[t + 1] != skey[t]) ? 1 : 0;
+// Levels whose keys may repeat (an input layer that does not merge points): the distinct sites are
+// the runs of equal keys in schedule order; ukey[u], urow[u] for the u-th of them, where the last
+// row of its run wins (Metadata/IOLayersRules.h:41,54: repeated `mp[p] = i`), and head[u] = 1 where a
+// block of 64 keys starts.  Two launches, with no scan between them: a workgroup
+// takes SITE_TILE consecutive positions (four per thread), k_site_tails counts the distinct
+// sites of every tile, k_site_compact adds up the tiles in front of its own, numbers its sites
+// with a prefix inside the workgroup, writes ukey / urow / head and counts the blocks
+// (grid_count); *last_site = the index of the last distinct site.
+constexpr int SITE_THREADS = 1024, SITE_TILE = 4 * SITE_THREADS;
+__global__ __launch_bounds__(SITE_THREADS) void k_site_tails(const unsigned long long *skey, int64_t n, int *tile_sites) {
+  __shared__ int total;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  const int64_t t0 = (int64_t)blockIdx.x * SITE_TILE + 4 * threadIdx.x;
+  int mine = 0;
+  for (int i = 0; i < 4; i++) {
+    const int64_t t = t0 + i;
+    mine += (t < n && (t == n - 1 || skey[t + 1] != skey[t])) ? 1 : 0;
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) mine += __shfl_xor(mine, o, 64);
+  if ((threadIdx.x & 63) == 0 && mine) atomicAdd(&total, mine);
+  __syncthreads();
+  if (threadIdx.x == 0) tile_sites[blockIdx.x] = total;
 }
-// ukey[u], urow[u] for the u-th distinct site: the last row of its run wins
-// (Metadata/IOLayersRules.h:41,54: repeated `mp[p] = i`).
-__global__ void k_compact_sites(const unsigned long long *skey, const int *sched, const int *tail,
-                                const int *tail_scan, int64_t n, unsigned long long *ukey, int *urow) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n || !tail[t]) return;
-  int u = tail_scan[t];
-  ukey[u] = skey[t];
-  urow[u] = sched ? sched[t] : (int)t;
+__global__ __launch_bounds__(SITE_THREADS) void k_site_compact(const unsigned long long *skey, const int *sched, int64_t n,
+                                                               const int *tile_sites, unsigned long long *ukey,
+                                                               int *urow, int *head, unsigned long long *ticket,
+                                                               int *last_site) {
+  __shared__ int part[SITE_THREADS / 64], wave_sites[SITE_THREADS / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int before = 0;
+  for (int i = threadIdx.x; i < (int)blockIdx.x; i += SITE_THREADS) before += tile_sites[i];
+#pragma unroll
+  for (int o = 32; o; o >>= 1) before += __shfl_xor(before, o, 64);
+  const int64_t t0 = (int64_t)blockIdx.x * SITE_TILE + 4 * threadIdx.x;
+  bool tail[4];
+  int mine = 0;
+  for (int i = 0; i < 4; i++) {
+    const int64_t t = t0 + i;
+    tail[i] = t < n && (t == n - 1 || skey[t + 1] != skey[t]);
+    mine += tail[i] ? 1 : 0;
+  }
+  int incl = mine;  // inclusive prefix over the wavefront's lanes
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  if (lane == 63) wave_sites[wave] = incl;
+  if (lane == 0) part[wave] = before;
+  __syncthreads();
+  int u = incl - mine;
+  for (int w = 0; w < SITE_THREADS / 64; w++) u += part[w] + (w < wave ? wave_sites[w] : 0);
+  int heads = 0;
+  for (int i = 0; i < 4; i++) {
+    if (!tail[i]) continue;
+    const int64_t t = t0 + i;
+    const unsigned long long k = skey[t];
+    int64_t j = t;  // first position of the site's run: the key in front of it is the previous site's
+    while (j > 0 && skey[j - 1] == k) j--;
+    const int h = (j == 0 || (skey[j - 1] >> 6) != (k >> 6)) ? 1 : 0;
+    ukey[u] = k;
+    urow[u] = sched ? sched[t] : (int)t;
+    head[u] = h;
+    heads += h;
+    u++;
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == SITE_THREADS - 1) *last_site = u - 1;
+  grid_count(heads, ticket);
 }
 // The size of a level's block table is decided on the device (no host round trip): from the
 // number of blocks, capacity = the power of two >= 2 * blocks (at least 64).
@@ -690,18 +746,17 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
     if (L.dups) {
       // distinct sites first: ukey / urow by compaction; their number stays on the device
       position_keys(L, s);
-      m.f1.reserve(n + 1);
-      m.s1.reserve(n + 1);
+      const int tiles = (int)ceil_div(n, SITE_TILE);
+      m.f1.reserve(tiles);
+      m.s1.reserve(1);
       L.urow.reserve(n);
-      k_run_tails<<<grid_for(n), TB, 0, s>>>(L.skeys.p, n, m.f1.p);
+      k_site_tails<<<dim3(tiles), SITE_THREADS, 0, s>>>(L.skeys.p, n, m.f1.p);
       LAUNCH_CHECK();
-      exclusive_scan(m, m.f1.p, m.s1.p, n, s);
-      k_compact_sites<<<grid_for(n), TB, 0, s>>>(L.skeys.p, L.sched_ptr(), m.f1.p, m.s1.p, n, m.k1.p, L.urow.p);
+      k_site_compact<<<dim3(tiles), SITE_THREADS, 0, s>>>(L.skeys.p, L.sched_ptr(), n, m.f1.p, m.k1.p, L.urow.p, m.f0.p,
+                                                         ticket, m.s1.p);
       LAUNCH_CHECK();
-      n_sites_dev = m.s1.p + (n - 1);  // index of the last distinct site (the last position ends a run)
+      n_sites_dev = m.s1.p;  // index of the last distinct site
       ukey = m.k1.p;
-      k_block_heads<<<count_grid(n), TB, 0, s>>>(ukey, n, n_sites_dev, m.f0.p, ticket);
-      LAUNCH_CHECK();
     } else if (L.skeys_ready) {  // the input layer left the positions' keys
       k_block_heads<<<count_grid(n), TB, 0, s>>>(L.skeys.p, n, nullptr, m.f0.p, ticket);
       LAUNCH_CHECK();
