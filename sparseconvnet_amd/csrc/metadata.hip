@@ -1612,7 +1612,7 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift,
                                                    int64_t n, int64_t npad_in, int64_t npad_out, const int *block_heads,
                                                    int *by_out, int *by_in, int *out_soa, unsigned long long *out_keys,
                                                    unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
-                                                   int *pidx, unsigned *pmasks) {
+                                                   int *pidx, unsigned *pmasks, bool dups) {
   const int K = 1 << gi.dim;
   __shared__ int red[HB / 64], wave_heads[HB / 64], lcount[8];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1640,16 +1640,21 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift,
   int o = 0;
   for (int w = 0; w < HB / 64; w++) o += red[w] + (w < wave ? wave_heads[w] : 0);
   o += __popcll(heads & (~0ull >> (63 - lane))) - 1;  // heads at or before this lane, less one
+  // dups (a level whose keys may repeat): only the last position of a run of equal keys is a site
+  // (see k_subm_rules); the others have no rule, but may be where an output site's run begins
+  const bool site = live && !(dups && p + 1 < n && keys[p + 1] == keys[p]);
+  if (!site) tap = -1;
   if (live) {
     const int row = sched ? sched[p] : (int)p;
     for (int k = 0; k < K; k++) by_in[(int64_t)k * npad_in + p] = k == tap ? o : -1;
-    by_out[(int64_t)tap * npad_out + o] = row;
+    if (site) by_out[(int64_t)tap * npad_out + o] = row;
     if (head) {
-      unsigned mask = 1u << tap;
-      for (int i = 1; i < K && p + i < n; i++) {
+      unsigned mask = site ? 1u << tap : 0u;
+      for (int i = 1; (dups || i < K) && p + i < n; i++) {
         int t2;
-        if (parent_key(gi, go, shift, keys[p + i], &t2) != ck) break;
-        mask |= 1u << t2;
+        const unsigned long long k2 = keys[p + i];
+        if (parent_key(gi, go, shift, k2, &t2) != ck) break;
+        if (!(dups && p + i + 1 < n && keys[p + i + 1] == k2)) mask |= 1u << t2;
       }
       int j[SCN_MAXD], b;
       site_of_key(go, ck, j, b);
@@ -1716,7 +1721,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   // Filter = stride = 2 in every dimension over exactly fitting sizes (the U-Net's and most
   // networks' downsampling): each site has one candidate, the Morton key of its coordinates
   // halved, which ascends with the site's own key, so the schedule order is already sorted.
-  bool presorted = m.dim <= 3 && f.M == 1 && !LI.dups;  // rows without a site leave holes in the order
+  bool presorted = m.dim <= 3 && f.M == 1;
   for (int d = 0; d < m.dim; d++)
     presorted = presorted && filter[d] == 2 && stride[d] == 2 && in_size[d] == 2 * out_size[d];
   // The caller has to learn the new level's size: a read-back per rulebook, except along a chain
@@ -1764,7 +1769,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     k_halve_emit<<<dim3(blocks), HB, 0, s>>>(LI.g, go, shift, keys, LI.sched_ptr(), n, LI.npad, LO.npad, m.f0.p, R.by_out.nbr.p,
                                              R.by_in.nbr.p, LO.coords.p, LO.keys.p,
                                              (unsigned long long *)R.by_out.cnt->dev.p, pk, m.k0.p, m.v0.p,
-                                             reinterpret_cast<unsigned *>(m.f1.p));
+                                             reinterpret_cast<unsigned *>(m.f1.p), LI.dups);
     LAUNCH_CHECK();
     R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
     finalize_table(m, R.by_out, nullptr, s, true);

@@ -130,6 +130,28 @@ def check_mode0_repeated_points(make, dim, seed, n=300, spatial=9, batch=2, cin=
         want_s = set((t[0], last[t[1:2 + dim]]) + t[2 + dim:] for t in bf.strided_triples(sites, dim, 3, 2, 4))
         assert got_s == want_s
         assert sum(len(r) for r in srules) == len(got_s)
+    # filter 2 / stride 2 over a size that halves exactly (the builders' path without a sort), and
+    # once more from the level that made, which has no repeated keys
+    if spatial % 4 == 0:
+        half = spatial // 2
+        srules = p.strided_rules(spatial, half, 2, 2)
+        loc_out = p.spatial_locations(half)
+        got_s = set()
+        for k, r in enumerate(srules):
+            for i, j in np.asarray(r).reshape(-1, 2).tolist():
+                got_s.add((k, int(i)) + tuple(loc_out[j].tolist()))
+        want_s = set((t[0], last[t[1:2 + dim]]) + t[2 + dim:] for t in bf.strided_triples(sites, dim, 2, 2, half))
+        assert got_s == want_s
+        assert sum(len(r) for r in srules) == len(got_s)
+        assert len(loc_out) == len(set(t[2:] for t in want_s))
+        rules2 = p.strided_rules(half, half // 2, 2, 2)
+        loc2 = p.spatial_locations(half // 2)
+        row_of = {tuple(c): i for i, c in enumerate(loc_out.tolist())}
+        got2 = set((k, int(i)) + tuple(loc2[j].tolist()) for k, r in enumerate(rules2)
+                   for i, j in np.asarray(r).reshape(-1, 2).tolist())
+        want2 = set((t[0], row_of[t[1:2 + dim]]) + t[2 + dim:]
+                    for t in bf.strided_triples(np.array(sorted(row_of), np.int64), dim, 2, 2, half // 2))
+        assert got2 == want2
 
 
 def check_bl_input_layer(make, dim, mode, seed, batch=3, length=70, spatial=9, planes=5, empties=True):

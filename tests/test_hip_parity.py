@@ -86,6 +86,7 @@ def test_input_layer_no_batch_column(make):
 @pytest.mark.parametrize("dim", [1, 2, 3])
 def test_input_layer_mode0_repeated_points(make, dim):
     checks.check_mode0_repeated_points(make, dim, seed=40 + dim)
+    checks.check_mode0_repeated_points(make, dim, seed=50 + dim, spatial=8)
     if dim == 3:  # many workgroups, MFMA convolution kernel
         checks.check_mode0_repeated_points(make, dim, seed=44, n=20000, spatial=48, cin=16, cout=16)
 

@@ -36,6 +36,7 @@ def test_input_layer_no_batch_column(make):
 @pytest.mark.parametrize("dim", [1, 2, 3])
 def test_input_layer_mode0_repeated_points(make, dim):
     checks.check_mode0_repeated_points(make, dim, seed=40 + dim)
+    checks.check_mode0_repeated_points(make, dim, seed=50 + dim, spatial=8)
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
