@@ -102,6 +102,10 @@ struct StridedRules {
   // (finish_by_in): transposed convolutions and unpooling come long after the level was built,
   // and the sort would sit on the path of the next level's construction.
   bool by_in_final = false;
+  // Filter = stride = 2 over halving sizes: every fine position has at most one rule, kept as
+  // (tap, coarse row) until finish_by_in writes the table in its sorted order (in_tap[t] < 0: no rule).
+  bool by_in_compact = false;
+  DevBuf<int> in_tap, in_row;
   SizeKey in_size, out_size;
 };
 

@@ -1604,13 +1604,13 @@ __global__ __launch_bounds__(HB) void k_halve_heads(Geom gi, Geom go, bool shift
 }
 // One thread per input position t: its output row o is the number of output sites that begin at or
 // before t, less one (workgroups before this one: block_heads; inside: ballots).  It writes its own
-// rule into both tables and -1 into the other taps of by_in; the first position of an output site
+// rule into by_out and as (tap, output row) for the fine-side table; the first position of an output site
 // looks at the up to 2^dim - 1 positions behind it for the site's tap mask, writes -1 into the
 // absent taps of by_out, the site's coordinates and key, and its pattern-sort key
 // (Metadata/ConvolutionRules.h:19-31, Metadata/RectangularRegions.h:30-38,95-105 for this filter).
 __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift, const unsigned long long *keys, const int *sched,
                                                    int64_t n, int64_t npad_in, int64_t npad_out, const int *block_heads,
-                                                   int *by_out, int *by_in, int *out_soa, unsigned long long *out_keys,
+                                                   int *by_out, int *in_tap, int *in_row, int *out_soa, unsigned long long *out_keys,
                                                    unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
                                                    int *pidx, unsigned *pmasks, bool dups) {
   const int K = 1 << gi.dim;
@@ -1646,7 +1646,8 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift,
   if (!site) tap = -1;
   if (live) {
     const int row = sched ? sched[p] : (int)p;
-    for (int k = 0; k < K; k++) by_in[(int64_t)k * npad_in + p] = k == tap ? o : -1;
+    in_tap[p] = tap;
+    in_row[p] = o;
     if (site) by_out[(int64_t)tap * npad_out + o] = row;
     if (head) {
       unsigned mask = site ? 1u << tap : 0u;
@@ -1762,12 +1763,14 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     R.by_in.n = n;
     R.by_in.npad = LI.npad;
     R.by_out.nbr.reserve((size_t)f.K * LO.npad);
-    R.by_in.nbr.reserve((size_t)f.K * LI.npad);
+    R.by_in_compact = true;
+    R.in_tap.reserve(n);
+    R.in_row.reserve(n);
     int key_bits = 0;
     const PatternKey pk = pattern_plan(n_out, f.K, key_bits);
     reserve_pattern_buffers(m, R.by_out);
     k_halve_emit<<<dim3(blocks), HB, 0, s>>>(LI.g, go, shift, keys, LI.sched_ptr(), n, LI.npad, LO.npad, m.f0.p, R.by_out.nbr.p,
-                                             R.by_in.nbr.p, LO.coords.p, LO.keys.p,
+                                             R.in_tap.p, R.in_row.p, LO.coords.p, LO.keys.p,
                                              (unsigned long long *)R.by_out.cnt->dev.p, pk, m.k0.p, m.v0.p,
                                              reinterpret_cast<unsigned *>(m.f1.p), LI.dups);
     LAUNCH_CHECK();
@@ -1813,11 +1816,63 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   return m.strided.emplace(key, std::move(R)).first->second;
 }
 
+// The fine-side table of a halving rulebook from its compact form.  Sort key of a position: its
+// range of the schedule (as finalize_table's), then its tap (positions without a rule last): the
+// order count-then-mask gives a table whose rows have one tap each, in 4 bits.
+__global__ void k_few_keys(const int *in_tap, int64_t n, int64_t window, unsigned long long *keys, int *idx) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int tap = in_tap[t];
+  keys[t] = ((unsigned long long)(t / window) << 4) | (unsigned long long)(tap < 0 ? 15 : tap);
+  idx[t] = (int)t;
+}
+// Position t of the sorted table is position perm[t] of the schedule: its one entry, -1 in the
+// other taps, its row, and the granule masks (an OR over the 16 lanes of a granule).
+__global__ void k_table_expand_few(const int *in_tap, const int *in_row, int K, int64_t n, int64_t npad, const int *perm,
+                                   const int *base, int *nbr, int *rowmap, unsigned *gmask) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned mk = 0;
+  if (t < n) {
+    const int src = perm[t];
+    const int tap = in_tap[src], row = in_row[src];
+    for (int k = 0; k < K; k++) nbr[(int64_t)k * npad + t] = k == tap ? row : -1;
+    mk = tap >= 0 ? 1u << tap : 0u;
+    rowmap[t] = base ? base[src] : src;
+  }
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) mk |= __shfl_xor(mk, o, 64);
+  if ((threadIdx.x & 15) == 0 && t < n) gmask[t >> 4] = mk;
+}
+
 void finish_by_in(Metadata &m, StridedRules &r, hipStream_t s) {
   if (r.by_in_final) return;
   auto li = m.levels.find(r.in_size);
   if (li == m.levels.end()) throw Error("strided rules: the fine level is gone");
   m.builds++;
+  Table &t = r.by_in;
+  if (r.by_in_compact && t.n > 0) {
+    int key_bits = 0;
+    const PatternKey pk = pattern_plan(t.n, t.K, key_bits);  // the ranges of the schedule, as for any table
+    int range_bits = 0;
+    while (((int64_t)1 << range_bits) < ceil_div(t.n, pk.window)) range_bits++;
+    t.spread = pk.window >= t.n;
+    reserve_pattern_buffers(m, t);
+    k_few_keys<<<grid_for(t.n), TB, 0, s>>>(r.in_tap.p, t.n, pk.window, m.k0.p, m.v0.p);
+    LAUNCH_CHECK();
+    sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, 4 + range_bits);
+    t.nbr.reserve((size_t)t.K * t.npad);
+    t.rowmap.reserve(t.npad);
+    t.gmask.reserve(ceil_div(t.n, 16));
+    k_table_expand_few<<<grid_for(t.n), TB, 0, s>>>(r.in_tap.p, r.in_row.p, t.K, t.n, t.npad, m.v1.p,
+                                                    li->second.sched_ptr(), t.nbr.p, t.rowmap.p, t.gmask.p);
+    LAUNCH_CHECK();
+    t.identity_rows = false;
+    r.in_tap.release();
+    r.in_row.release();
+    r.by_in_compact = false;
+    r.by_in_final = true;
+    return;
+  }
   finalize_table(m, r.by_in, li->second.sched_ptr(), s);
   r.by_in_final = true;
 }
