@@ -458,8 +458,19 @@ __global__ __launch_bounds__(1024) void k_active_pool_finish(const float *__rest
   const int per = (chunks + 15) / 16;
   const int q0 = min(chunks, wave * per), q1 = min(chunks, q0 + per);
   float s = 0.f;
-  if (c < planes)
-    for (int q = q0; q < q1; q++) s += partial[((size_t)b * chunks + q) * planes + c];
+  if (c < planes) {
+    // eight loads in flight (one after the other, each waits out a trip to L2); the order of the
+    // additions is fixed all the same
+    int q = q0;
+    for (; q + 8 <= q1; q += 8) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = partial[((size_t)b * chunks + q + i) * planes + c];
+#pragma unroll
+      for (int i = 0; i < 8; i++) s += v[i];
+    }
+    for (; q < q1; q++) s += partial[((size_t)b * chunks + q) * planes + c];
+  }
   part[wave][lane] = s;
   __syncthreads();
   if (wave == 0 && c < planes) {
