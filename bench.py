@@ -298,10 +298,10 @@ def unet_layer_table(torch, scn, model, x, reps=5):
     recs = []
     orig = M.Metadata._conv
 
-    def timed_conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs, out=None):
+    def timed_conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs, out=None, second=None):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        out, macs = orig(self, kind, size_args, n_rows, features, weight, bias, bn, post, True, out)
+        out, macs = orig(self, kind, size_args, n_rows, features, weight, bias, bn, post, True, out, second)
         e1.record()
         kernel = self._L.scn_md_last_conv_kernel(self._h).decode()
         recs.append((kind, features.shape[0], n_rows, weight.shape[0], weight.shape[1] * weight.shape[2],

@@ -262,6 +262,14 @@ typedef struct scn_bn_params {
   const float *gamma, *beta;               /* device, [planes], or NULL */
   float eps, leakiness;
 } scn_bn_params;
+/* No counterpart in the reference: the next convolution call on this handle also writes a second
+ * copy of its output, taken before the batch norm behind the convolution (if any) is applied and
+ * normalised with `bn` instead: out2[row * stride + col] = leaky(bn(value)).  For a producer whose
+ * plain output feeds one consumer and whose normalised output is one part of a concatenation
+ * (the skip connection of a U-Net level, sparseconvnet/networkArchitectures.py:240-253): the
+ * part lands in its columns of the joined matrix without a pass of its own.  groups = 1,
+ * nOut <= 256, stride >= nOut; serves one call; out2 = NULL switches it off. */
+int scn_md_next_second_output(scn_metadata *md, float *out2, int64_t stride, const scn_bn_params *bn);
 int scn_conv_bn_fwd(scn_metadata *md, int kind, const int64_t *a, const int64_t *b,
                     const int64_t *c, const int64_t *d, const float *in, float *out,
                     const float *weight, const float *bias, int n_in, int n_out, int groups,

@@ -60,6 +60,7 @@ SIGNATURES = {
     "scn_active_pooling_fwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_active_pooling_bwd": (C.c_int, [_vp, _i64p, _vp, _vp, C.c_int, C.c_int, _vp]),
     "scn_md_next_output_stride": (C.c_int, [_vp, C.c_int64]),
+    "scn_md_next_second_output": (C.c_int, [_vp, _vp, C.c_int64, C.POINTER(BnParams)]),
     "scn_sort_pairs": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_int64, C.c_int, _vp]),
     "scn_cache_stats": (C.c_int, [_i64p, _i64p, _i64p, _i64p]),
     "scn_conv_fwd": (C.c_int, [_vp, _i64p, _i64p, _i64p, _i64p, _vp, _vp, _vp, _vp, C.c_int, C.c_int,

@@ -30,7 +30,7 @@ class Sequential(torch.nn.Sequential):
         and a JoinTable by whatever produces each part (layers.concat_join_batchnorm).
         tail: (batch norm arguments, output columns) for the convolution that ends `mods`: it
         applies that batch norm to its output and writes it into those columns."""
-        from .layers import fuse_plan, join_batchnorm, concat_join_batchnorm
+        from .layers import fuse_plan, join_batchnorm, concat_join_batchnorm, skip_join_plan, _bn_slice, _is_conv
         i = 0
         while i < len(mods):
             if type(mods[i]) is JoinTable and i + 1 < len(mods) and isinstance(input, (list, tuple)) \
@@ -48,6 +48,22 @@ class Sequential(torch.nn.Sequential):
                     i += 3
                     continue
             plan = fuse_plan(mods[i:i + 3], input) if isinstance(input, SparseConvNetTensor) else None
+            # a convolution in front of a U-Net level's skip connection writes the skip part of the join itself
+            if isinstance(input, SparseConvNetTensor) and (plan is not None or _is_conv(mods[i])):
+                conv, pre, post, used = plan if plan is not None else (mods[i], None, None, 1)
+                skip = skip_join_plan(conv, mods[i + used:i + used + 3], input) if post is None else None
+                if skip is not None:
+                    bn, c0 = skip
+                    joined = input.features.new_empty((input.features.size(0), bn.nPlanes))
+                    x = conv(input, pre_bn=pre, second=(_bn_slice(bn, 0, c0), joined[:, :c0]))
+                    done = concat_join_batchnorm(mods[i + used], bn, x, prefilled=joined)
+                    if done is not None:
+                        input = done
+                        i += used + 3
+                    else:  # (not expected: skip_join_plan looked at the same things) as the modules by themselves
+                        input = x
+                        i += used
+                    continue
             if plan is None:
                 if tail is not None and i == len(mods) - 1:
                     input = mods[i](input, post_bn=tail[0], out=tail[1])

@@ -525,6 +525,25 @@ int scn_md_next_output_stride(scn_metadata *h, int64_t stride) {
     md(h).next_out_stride = stride;
   });
 }
+int scn_md_next_second_output(scn_metadata *h, float *out2, int64_t stride, const scn_bn_params *bn) {
+  return guarded([&] {
+    Metadata &m = md(h);
+    if (!out2) {
+      m.next_out2 = nullptr;
+      return;
+    }
+    if (!bn || !bn->running_mean || !bn->running_var) throw Error("second output: needs a batch normalisation");
+    if (stride <= 0) throw Error("second output: stride must be positive");
+    m.next_out2 = out2;
+    m.next_out2_stride = stride;
+    m.next_out2_bn[0] = bn->running_mean;
+    m.next_out2_bn[1] = bn->running_var;
+    m.next_out2_bn[2] = bn->gamma;
+    m.next_out2_bn[3] = bn->beta;
+    m.next_out2_eps = bn->eps;
+    m.next_out2_leak = bn->leakiness;
+  });
+}
 const char *scn_md_last_conv_kernel(scn_metadata *h) { return h ? h->m.last_kernel.c_str() : ""; }
 int scn_md_input_layer(scn_metadata *h, const int64_t *spatial, const int64_t *coords, int64_t n,
                        int ncols, int min_batch, int mode, void *stream, int64_t *n_active) {

@@ -109,8 +109,9 @@ __global__ void k_conv_generic(const int *nbr, const int *rowmap, int K, int64_t
     for (int c = 0; c < ip; c++) a += x[c] * wk[(int64_t)c * op];
     acc += a;
   }
-  if (epi.sc) acc = epi_act(acc, epi.sc[oc], epi.sh[oc], epi.leak);
   int64_t row = rowmap ? rowmap[t] : t;
+  if (epi.out2) epi_second(epi, row, oc, acc);
+  if (epi.sc) acc = epi_act(acc, epi.sc[oc], epi.sh[oc], epi.leak);
   out[row * (epi.out_stride ? epi.out_stride : n_out) + oc] = acc;
 }
 
@@ -218,6 +219,7 @@ __global__ void k_conv_reduce(const float *__restrict__ partial, int n_split, in
   for (int j = 0; j < 4; j++) {
     if (c0 + j >= n_out) break;
     float v = acc[j] + (epi.bias ? epi.bias[c0 + j] : 0.0f);
+    if (epi.out2) epi_second(epi, row, c0 + j, v);
     if (epi.sc) v = epi_act(v, epi.sc[c0 + j], epi.sh[c0 + j], epi.leak);
     o[j] = v;
   }
@@ -294,6 +296,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     ~FrozenReset() {
       m.frozen = nullptr;
       m.next_out_stride = 0;
+      m.next_out2 = nullptr;
       m.before_pack = nullptr;
       m.wkey_ptr = 0;
     }
@@ -322,6 +325,19 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     frozen->last = s;
     frozen->last_known = true;
   }
+  if (m.next_out2) {
+    if (n_out > 256 || m.fixed_scratch || groups != 1 || m.next_out2_stride < n_out || m.next_out2_stride > INT32_MAX)
+      throw Error("second output: groups = 1, at most 256 output planes, a stride of at least that, not with the allocation-free entry");
+    DevBuf<float> &buf = frozen ? frozen->post2 : m.post2buf;
+    buf.reserve(2 * (size_t)n_out);
+    m.jobs.post2 = CoefJob{m.next_out2_bn[0], m.next_out2_bn[1], m.next_out2_bn[2], m.next_out2_bn[3], m.next_out2_eps,
+                           n_out, n_out, buf.p, buf.p + n_out};
+    epi.out2 = m.next_out2;
+    epi.out2_stride = (int)m.next_out2_stride;
+    epi.sc2 = buf.p;
+    epi.sh2 = buf.p + n_out;
+    epi.leak2 = m.next_out2_leak;
+  }
   m.post_raw = CoefJob();
   if (post) {
     DevBuf<float> &buf = frozen ? frozen->post : m.postbuf;
@@ -348,12 +364,14 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     // side do not run when the packed weights are found)
     if (frozen->post_done) m.jobs.post = CoefJob();
     if (frozen->pre_done) m.jobs.pre = CoefJob();
-    if (m.jobs.post.n_pad || m.jobs.pre.n_pad) {
+    if (frozen->post2_done) m.jobs.post2 = CoefJob();
+    if (m.jobs.post.n_pad || m.jobs.pre.n_pad || m.jobs.post2.n_pad) {
       k_coefs<<<dim3(1), 256, 0, s>>>(take_jobs(m));
       LAUNCH_CHECK();
     }
     frozen->post_done = frozen->post_done || post != nullptr;
     frozen->pre_done = frozen->pre_done || pre_fused;
+    frozen->post2_done = frozen->post2_done || epi.out2 != nullptr;
   }
   if (pre_fused) {
     if (conv_mfma_paths<true>(m, t, in, out, w, epi, n_in, n_out, pre, s)) return;
@@ -400,7 +418,7 @@ void conv_forward(Metadata &m, const Table &t, const float *in, int64_t n_in_row
     }
     if (ok) return;
   }
-  if (m.jobs.post.n_pad) {  // no packing launch on this path: fold the coefficients by themselves
+  if (m.jobs.post.n_pad || m.jobs.post2.n_pad) {  // no packing launch on this path: fold the coefficients by themselves
     k_coefs<<<dim3(1), 256, 0, s>>>(take_jobs(m));
     LAUNCH_CHECK();
   }

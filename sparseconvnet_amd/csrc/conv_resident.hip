@@ -306,6 +306,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_conv_resident(
               const int col = 16 * cb + r16;
               if (col < n_out) {
                 float v = acc[q][cb][r] + (accumulate ? o[col] : bv[cb]);
+                if (epi.out2) epi_second(epi, row, col, v);
                 if (post) v = epi_act(v, es[cb], eh[cb], epi.leak);
                 o[col] = v;
               }
@@ -429,7 +430,7 @@ static void launch_resident_part(Metadata &m, const Table &t, const float *in, i
 template <int NCB>
 static void launch_resident_c4(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                                Epi epi, int n_in, int n_out, hipStream_t s) {
-  if (in == m.cur_in_base && !epi.out_stride && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
+  if (in == m.cur_in_base && !epi.out_stride && !epi.out2 && conv_first_serves(t, m.cur_in_rows, n_in, n_out)) {
     // epi.sc / epi.sh point at arrays nobody fills on this path: the kernel folds the batch norm itself
     take_jobs(m);
     note_kernel(m, "first", {{"nin", n_in}});
@@ -489,6 +490,11 @@ bool try_resident(Metadata &m, const Table &t, const float *in, float *out, cons
       b.sc = epi.sc;
       b.sh = epi.sh;
       b.leak = epi.leak;
+      b.out2 = epi.out2;
+      b.out2_stride = epi.out2_stride;
+      b.sc2 = epi.sc2;
+      b.sh2 = epi.sh2;
+      b.leak2 = epi.leak2;
     }
 #define SCN_RES(NCBV, SSV)                                                                                   \
   do {                                                                                                       \

@@ -361,6 +361,7 @@ __global__ __launch_bounds__(NW * 64) void k_conv_rows(
       for (int cb = 0; cb < NCB; cb++) {
         const int col = 16 * cb + r16;
         float v = acc[q][cb][r] + bv[cb];
+        if (epi.out2 && col < n_out) epi_second(epi, row, col, v);
         if (post) v = epi_act(v, es[cb], eh[cb], epi.leak);
         if (col < n_out) o[col] = v;
       }

@@ -248,6 +248,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
       for (int c = 0; c < NCBW; c++) {
         const int col = 16 * (wc * NCBW + c) + r16;
         float v = acc[q][c][r] + bv[c];
+        if (epi.out2 && col < n_out) epi_second(epi, row, col, v);
         if (post) v = epi_act(v, es[c], eh[c], epi.leak);
         if (col < n_out) o[col] = v;
       }

@@ -117,7 +117,7 @@ struct CoefJob {
   float *sc = nullptr, *sh = nullptr;
 };
 struct CoefJobs {
-  CoefJob pre, post;
+  CoefJob pre, post, post2;
 };
 
 // What a convolution derives from its parameters before it can run: the weights in MFMA operand
@@ -127,15 +127,16 @@ struct CoefJobs {
 // hands the convolution one of these objects to keep them in (scn_params_create).
 struct FrozenParams {
   std::map<std::vector<int64_t>, DevBuf<float>> packed;
-  DevBuf<float> pre, post;   // scale | shift arrays, as conv_forward lays them out
-  bool pre_done = false, post_done = false;
+  DevBuf<float> pre, post, post2;   // scale | shift arrays, as conv_forward lays them out
+  bool pre_done = false, post_done = false, post2_done = false;
   hipStream_t last = nullptr;  // the stream of the last convolution that used the set
   bool last_known = false;
   void clear() {
     packed.clear();
     pre.release();
     post.release();
-    pre_done = post_done = false;
+    post2.release();
+    pre_done = post_done = post2_done = false;
   }
 };
 
@@ -218,6 +219,12 @@ struct Metadata {
   // while a column range of a wide layer runs: addresses in the scratch copy (from wkey_from) stand for
   // addresses from wkey_ptr in the caller's weights in a frozen set's keys
   int64_t wkey_ptr = 0, wkey_from = 0, wkey_c0 = 0, wkey_wc = 0;
+  // a second output for the next convolution call (Epi::out2), with the batch norm it applies; serves one call
+  float *next_out2 = nullptr;
+  int64_t next_out2_stride = 0;
+  const float *next_out2_bn[4] = {nullptr, nullptr, nullptr, nullptr};  // mean, var, gamma, beta
+  float next_out2_eps = 0.f, next_out2_leak = 1.f;
+  DevBuf<float> post2buf;
   int64_t next_out_stride = 0;  // floats between the output rows of the next convolution call (0: its plane count); serves one call
   DevBuf<unsigned long long> ticket;  // [0]: arrival ticket of grid_count (zero between launches), [1]: the count
   DevBuf<float> wpack;    // weights of the running convolution in MFMA operand order
@@ -300,10 +307,21 @@ struct Epi {
   const float *sc = nullptr, *sh = nullptr;  // [nOut] each, or nulls
   float leak = 1.0f;
   int out_stride = 0;  // floats between output rows; 0: nOut
+  // A second copy of the output before `sc` / `sh` are applied, with a batch norm of its own
+  // (out2 == nullptr: none): out2[row * out2_stride + col] = act(value * sc2[col] + sh2[col]).
+  float *out2 = nullptr;
+  int out2_stride = 0;
+  const float *sc2 = nullptr, *sh2 = nullptr;
+  float leak2 = 1.0f;
 };
+// The second copy of one output value (raw: bias added, the convolution's own batch norm not yet).
+__device__ inline void epi_second(const Epi &epi, int64_t row, int col, float raw);
 __device__ inline float epi_act(float v, float sc, float sh, float leak) {
   const float y = v * sc + sh;
   return y > 0.f ? y : y * leak;
+}
+__device__ inline void epi_second(const Epi &epi, int64_t row, int col, float raw) {
+  epi.out2[row * epi.out2_stride + col] = epi_act(raw, epi.sc2[col], epi.sh2[col], epi.leak2);
 }
 // Folding a batch norm to scale / shift (sc[c] = gamma / sqrt(var + eps), sh[c] = beta -
 // mean * sc, zeros from n to n_pad) is a few hundred values: the weight-packing launch that
@@ -324,6 +342,7 @@ __device__ inline void coef_jobs(const CoefJobs &jobs) {
   if (blockIdx.x != 0) return;
   if (jobs.pre.n_pad) coef_job(jobs.pre);
   if (jobs.post.n_pad) coef_job(jobs.post);
+  if (jobs.post2.n_pad) coef_job(jobs.post2);
 }
 // conv_first.hip: the convolution kernel for nIn <= 4, nOut <= 32 and up to 32 taps; it reads the
 // weights as the caller holds them and folds the batch norm behind the convolution itself

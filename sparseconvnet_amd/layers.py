@@ -56,7 +56,7 @@ class _FrozenParams:
             pass
 
 
-def _use_frozen(module, md, weight, bias, pre=None, post=None):
+def _use_frozen(module, md, weight, bias, pre=None, post=None, second=None):
     """Eval mode: the module's convolution may keep what it derives from its parameters."""
     if module.training:
         return
@@ -64,7 +64,7 @@ def _use_frozen(module, md, weight, bias, pre=None, post=None):
     if f is None:
         f = module.__dict__['_frozen'] = _FrozenParams()
     tensors = [weight, bias]
-    for bn in (pre, post):
+    for bn in (pre, post, second[0] if second is not None else None):
         if bn is not None:
             tensors += list(bn[:4])
     f.use(md, tensors)
@@ -75,12 +75,12 @@ class _ConvFunction(Function):
     1 / 2.  pre / post: eval-mode batch norms applied inside the convolution (inference only)."""
 
     @staticmethod
-    def forward(ctx, features, weight, bias, md, kind, sizes, pre, post, out=None):
+    def forward(ctx, features, weight, bias, md, kind, sizes, pre, post, out=None, second=None):
         ctx.md, ctx.kind, ctx.sizes, ctx.fused = md, kind, sizes, pre is not None or post is not None
         ctx.has_bias = bias.numel() > 0
         ctx.save_for_backward(features, weight)
         fn = (md.submanifoldConvolution, md.convolution, md.deconvolution)[kind]
-        out, _ = fn(*sizes, features, weight, bias, pre, post, want_macs=False, out=out)
+        out, _ = fn(*sizes, features, weight, bias, pre, post, want_macs=False, out=out, second=second)
         _count(out)
         return out
 
@@ -91,7 +91,7 @@ class _ConvFunction(Function):
         features, weight = ctx.saved_tensors
         fn = (ctx.md.submanifoldConvolutionBackward, ctx.md.convolutionBackward, ctx.md.deconvolutionBackward)[ctx.kind]
         d_in, d_w, d_b = fn(*ctx.sizes, features, grad_output.contiguous(), weight, ctx.has_bias)
-        return d_in, d_w, d_b, None, None, None, None, None, None
+        return d_in, d_w, d_b, None, None, None, None, None, None, None
 
 
 class _NetworkInNetworkFunction(Function):
@@ -185,13 +185,43 @@ def _bn_slice(bn, lo, hi):
             bn.eps, bn.leakiness)
 
 
-def concat_join_batchnorm(table, bn, input):
+def skip_join_plan(conv, mods, input):
+    """For a SubmanifoldConvolution `conv` about to run on `input` with `mods` behind it: when those
+    begin with [ConcatTable(Identity, Sequential(... convolution)), JoinTable, eval-mode batch norm]
+    (the skip connection of a U-Net level) and concat_join_batchnorm will take them, returns
+    (batch norm, planes of the skip part): `conv` can then write the skip part of the joined matrix
+    itself, normalised, beside its plain output (the `second` output of the convolutions)."""
+    from .containers import ConcatTable, JoinTable, Sequential
+    if not _pkg.fuse_batchnorm or torch.is_grad_enabled() or len(mods) < 3 or input.features.nelement() == 0:
+        return None
+    table, join, bn = mods[0], mods[1], mods[2]
+    if type(conv) not in (SubmanifoldConvolution, ValidConvolution) or conv.groups != 1 or conv.nOut > 256:
+        return None
+    if type(table) is not ConcatTable or type(join) is not JoinTable or not _is_bn(bn):
+        return None
+    if any(m._forward_hooks or m._forward_pre_hooks for m in (table, join)):
+        return None
+    children = list(table._modules.values())
+    if len(children) != 2 or not _plain(children[0], (Identity,)):
+        return None
+    last = children[1]
+    if type(last) is not Sequential or last._forward_hooks or last._forward_pre_hooks:
+        return None
+    chain = last._chain()
+    if not chain or not _is_conv(chain[-1]) or chain[-1].nOut > 256 or conv.nOut + chain[-1].nOut != bn.nPlanes:
+        return None
+    return bn, conv.nOut
+
+
+def concat_join_batchnorm(table, bn, input, prefilled=None):
     """ConcatTable `table`, JoinTable and the eval-mode batch normalisation `bn` run on `input` with
     no pass over the joined matrix: when the table's last branch ends in a convolution (the
     Deconvolution of a U-Net level), that convolution applies its planes' share of the batch norm
     to its output and writes it straight into its columns of the joined matrix; the other
     branches' results are normalised into theirs as join_batchnorm does.  None when this does not
-    apply (the caller then runs the three modules one after the other).  Inference only."""
+    apply (the caller then runs the three modules one after the other).  Inference only.
+    prefilled: the joined matrix with the first branch's columns already written (skip_join_plan:
+    that branch is the Identity and the producer of `input` wrote them)."""
     from .containers import Sequential
     if not _pkg.fuse_batchnorm or torch.is_grad_enabled() or not _is_bn(bn) or not isinstance(input, SparseConvNetTensor):
         return None
@@ -205,7 +235,7 @@ def concat_join_batchnorm(table, bn, input):
     if not chain or not _is_conv(chain[-1]) or chain[-1].nOut > 256:
         return None
     conv = chain[-1]
-    parts = [c(input) for c in children[:-1]]
+    parts = [input] if prefilled is not None else [c(input) for c in children[:-1]]
     feats = [p.features for p in parts]
     rows = feats[0].size(0) if feats[0].dim() == 2 else -1
     fits = all(f.dim() == 2 and f.size(0) == rows and f.nelement() for f in feats) and \
@@ -214,12 +244,13 @@ def concat_join_batchnorm(table, bn, input):
         parts.append(last(input))
         from .containers import JoinTable
         return bn(JoinTable()(parts))
-    out = feats[0].new_empty((rows, bn.nPlanes))
+    out = prefilled if prefilled is not None else feats[0].new_empty((rows, bn.nPlanes))
     off = 0
     for f in feats:
         c = f.size(1)
-        mean, var, w, b, eps, leak = _bn_slice(bn, off, off + c)
-        _md.batchNormEval(f, mean, var, _opt(w), _opt(b), eps, leak, out=out[:, off:off + c])
+        if prefilled is None:
+            mean, var, w, b, eps, leak = _bn_slice(bn, off, off + c)
+            _md.batchNormEval(f, mean, var, _opt(w), _opt(b), eps, leak, out=out[:, off:off + c])
         off += c
     Sequential._run(chain, input, tail=(_bn_slice(bn, off, bn.nPlanes), out[:, off:]))
     output = SparseConvNetTensor()
@@ -394,15 +425,15 @@ class SubmanifoldConvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None, post_bn=None, out=None):
+    def forward(self, input, pre_bn=None, post_bn=None, out=None, second=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, self.nOut, input)
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
-        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post, second)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 0,
-                                              (input.spatial_size, self.filter_size), pre, post, out)
+                                              (input.spatial_size, self.filter_size), pre, post, out, second)
         return output
 
     def __repr__(self):
@@ -432,7 +463,7 @@ class Convolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None, post_bn=None, out=None):
+    def forward(self, input, pre_bn=None, post_bn=None, out=None, second=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
@@ -442,9 +473,9 @@ class Convolution(Module):
             input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
-        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post, second)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 1,
-                                              a, pre, post, out)
+                                              a, pre, post, out, second)
         return output
 
     def __repr__(self):
@@ -471,16 +502,16 @@ class Deconvolution(Module):
         if bias:
             self.bias = Parameter(torch.Tensor(nOut).zero_())
 
-    def forward(self, input, pre_bn=None, post_bn=None, out=None):
+    def forward(self, input, pre_bn=None, post_bn=None, out=None, second=None):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
         a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
-        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post)
+        _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post, second)
         output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 2,
-                                              a, pre, post, out)
+                                              a, pre, post, out, second)
         return output
 
     def __repr__(self):

@@ -203,30 +203,46 @@ class Metadata:
         _lib.check(self._L.scn_output_layer_fwd(self._h, _ptr(features), _ptr(out), features.size(1), _stream()))
         return out
 
-    def _conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs, out=None):
+    def _conv(self, kind, size_args, n_rows, features, weight, bias, bn, post, want_macs, out=None, second=None):
         """kind 0 / 1 / 2: submanifold / strided / transposed convolution.  bn, post: None, or
         (running_mean, running_var, weight, bias, eps, leakiness) of an eval-mode batch
         normalisation in front of / behind the convolution, applied inside it.  want_macs:
         return the multiply-add count (a stream synchronisation the first time a rulebook is
         used); otherwise the library adds it to this Metadata's running total (takeMacs).
         out: a [rows, planes] range of columns of a wider float32 matrix to write the result into
-        (the convolution's part of a concatenation), or None for a new tensor."""
+        (the convolution's part of a concatenation), or None for a new tensor.
+        second: None, or (batch norm arguments, columns as for `out`): the convolution also writes
+        its output there, taken before `post` and normalised with that batch norm instead."""
         features = _features(features, "features")
         weight = _features(weight, "weight")
         K, groups, ip, op = weight.shape
         bias_t = _features(bias, "bias") if bias is not None and bias.numel() else None
-        if out is None:
-            out = torch.empty((n_rows, groups * op), dtype=torch.float32, device=features.device)
-        else:
-            assert out.dtype == torch.float32 and out.device == features.device and out.dim() == 2, out
-            assert tuple(out.shape) == (n_rows, groups * op) and out.stride(1) == 1, (out.shape, out.stride())
-            if n_rows and out.stride(0) != out.size(1):
-                try:
+        resets = []  # what serves this one call is taken back, also when the call fails before it gets there
+        try:
+            if second is not None and n_rows:
+                bn2, out2 = second
+                assert out2.dtype == torch.float32 and out2.device == features.device and out2.dim() == 2, out2
+                assert tuple(out2.shape) == (n_rows, groups * op) and out2.stride(1) == 1, (out2.shape, out2.stride())
+                mean, var, g, b, eps, leak = bn2
+                t = [_features(mean, "running_mean"), _features(var, "running_var"),
+                     _features(g, "bn weight") if g is not None and g.numel() else None,
+                     _features(b, "bn bias") if b is not None and b.numel() else None]
+                resets.append(lambda: self._L.scn_md_next_second_output(self._h, None, 0, None))
+                _lib.check(self._L.scn_md_next_second_output(
+                    self._h, _ptr(out2), out2.stride(0),
+                    C.byref(_lib.BnParams(*[_ptr(x) for x in t], float(eps), float(leak)))))
+            if out is None:
+                out = torch.empty((n_rows, groups * op), dtype=torch.float32, device=features.device)
+            else:
+                assert out.dtype == torch.float32 and out.device == features.device and out.dim() == 2, out
+                assert tuple(out.shape) == (n_rows, groups * op) and out.stride(1) == 1, (out.shape, out.stride())
+                if n_rows and out.stride(0) != out.size(1):
+                    resets.append(lambda: self._L.scn_md_next_output_stride(self._h, 0))
                     _lib.check(self._L.scn_md_next_output_stride(self._h, out.stride(0)))
-                    return self._conv_into(kind, size_args, features, weight, bias_t, bn, post, want_macs, out)
-                finally:  # the stride serves one call, also one that failed before it got there
-                    self._L.scn_md_next_output_stride(self._h, 0)
-        return self._conv_into(kind, size_args, features, weight, bias_t, bn, post, want_macs, out)
+            return self._conv_into(kind, size_args, features, weight, bias_t, bn, post, want_macs, out)
+        finally:
+            for r in resets:
+                r()
 
     def _conv_into(self, kind, size_args, features, weight, bias_t, bn, post, want_macs, out):
         K, groups, ip, op = weight.shape
@@ -255,23 +271,23 @@ class Metadata:
         return out, (macs.value if want_macs else None)
 
     def submanifoldConvolution(self, spatial_size, filter_size, features, weight, bias, bn=None, post=None,
-                               want_macs=True, out=None):
+                               want_macs=True, out=None, second=None):
         sp, fs = self._s(spatial_size), self._s(filter_size)
         _lib.check(self._L.scn_md_submanifold_rules(self._h, sp, fs, _stream()))
-        return self._conv(0, (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn, post, want_macs, out)
+        return self._conv(0, (sp, fs), self.getNActive(spatial_size), features, weight, bias, bn, post, want_macs, out, second)
 
     def convolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None,
-                    want_macs=True, out=None):
+                    want_macs=True, out=None, second=None):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *a, _stream()))
-        return self._conv(1, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs, out)
+        return self._conv(1, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs, out, second)
 
     def deconvolution(self, in_size, out_size, filter_size, stride, features, weight, bias, bn=None, post=None,
-                      want_macs=True, out=None):
+                      want_macs=True, out=None, second=None):
         a = [self._s(v) for v in (in_size, out_size, filter_size, stride)]
         rb = [self._s(v) for v in (out_size, in_size, filter_size, stride)]
         _lib.check(self._L.scn_md_strided_rules(self._h, *rb, _stream()))
-        return self._conv(2, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs, out)
+        return self._conv(2, a, self.getNActive(out_size), features, weight, bias, bn, post, want_macs, out, second)
 
     def networkInNetwork(self, features, weight, bias, want_macs=True):
         """out = bias + features @ weight (weight [nIn, nOut]): a convolution with one tap."""

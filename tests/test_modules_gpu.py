@@ -861,6 +861,19 @@ def test_convolution_writes_into_columns_of_a_wider_matrix(n_in, n_out):
         assert (wide[:, :8] == 7.0).all() and (wide[:, 8 + n_out:] == 7.0).all()
         again, _ = md.submanifoldConvolution(size, three, t.features, w, bias, post=post, want_macs=False)
         assert again.is_contiguous() and torch.equal(again, plain), "the stride must not outlive its call"
+        # `second=`: the plain output as before, and beside it the raw output under another batch norm
+        raw, _ = md.submanifoldConvolution(size, three, t.features, w, bias, want_macs=False)
+        mean2, var2, g2, b2 = bn[1] - 0.7, bn[1] + 0.1, bn[3] * 0.5 + 1.0, bn[0]
+        want2 = (raw - mean2) / torch.sqrt(var2 + 1e-4) * g2 + b2
+        want2 = torch.where(want2 > 0, want2, 0.2 * want2)
+        wide2 = torch.full((n, n_out + 12), 5.0, device="cuda")
+        got, _ = md.submanifoldConvolution(size, three, t.features, w, bias, post=post, want_macs=False,
+                                           second=((mean2, var2, g2, b2, 1e-4, 0.2), wide2[:, 4:4 + n_out]))
+        checks.assert_close(got.cpu().numpy(), plain.cpu().numpy(), "plain output beside a second one")
+        checks.assert_close(wide2[:, 4:4 + n_out].cpu().numpy(), want2.cpu().numpy(), "second output")
+        assert (wide2[:, :4] == 5.0).all() and (wide2[:, 4 + n_out:] == 5.0).all()
+        again, _ = md.submanifoldConvolution(size, three, t.features, w, bias, post=post, want_macs=False)
+        assert torch.equal(again, plain), "the second output must not outlive its call"
     # strided and transposed convolutions (8 taps): down to the coarse level and back up
     half = (size - 2) // 2 + 1
     w2 = (torch.randn(8, 1, n_in, n_out, generator=g) * (2.0 / (8 * n_in)) ** 0.5).cuda()
@@ -892,21 +905,32 @@ def test_unet_level_joins_without_a_pass_over_the_joined_matrix():
     feats = torch.rand(len(coords), 3).cuda()
     inp_layer = scn.InputLayer(3, 64, mode=4)
     orig, taken = layers.concat_join_batchnorm, []
+    orig_plan, planned = layers.skip_join_plan, []
 
-    def counting(table, bn, input):
-        r = orig(table, bn, input)
-        taken.append(r is not None)
+    def counting(table, bn, input, prefilled=None):
+        r = orig(table, bn, input, prefilled)
+        taken.append((r is not None, prefilled is not None))
+        return r
+
+    def counting_plan(conv, mods, input):
+        r = orig_plan(conv, mods, input)
+        planned.append(r is not None)
         return r
     outs = []
     try:
-        for fn in (counting, lambda table, bn, input: None):
-            layers.concat_join_batchnorm = fn
+        # both halves by their producers; the transposed convolution's half only; a pass over the joined matrix
+        for fn, plan in ((counting, counting_plan), (counting, lambda conv, mods, input: None),
+                         (lambda table, bn, input, prefilled=None: None, lambda conv, mods, input: None)):
+            layers.concat_join_batchnorm, layers.skip_join_plan = fn, plan
             with torch.no_grad():
                 outs.append(model(inp_layer([torch.as_tensor(coords), feats])).cpu().numpy())
     finally:
-        layers.concat_join_batchnorm = orig
-    assert taken == [True, True], taken  # two levels with an inner branch
-    checks.assert_close(outs[0], outs[1], "joined by the producers vs joined by a pass")
+        layers.concat_join_batchnorm, layers.skip_join_plan = orig, orig_plan
+    # two levels with an inner branch, twice; the first time the skip halves were there already
+    assert taken == [(True, True)] * 2 + [(True, False)] * 2, taken
+    assert planned.count(True) == 2, planned
+    checks.assert_close(outs[0], outs[2], "joined by the producers vs joined by a pass")
+    checks.assert_close(outs[1], outs[2], "transposed convolution's half by its producer vs joined by a pass")
     # with gradients enabled the modules run one after the other
     taken.clear()
     layers.concat_join_batchnorm = counting
@@ -914,7 +938,7 @@ def test_unet_level_joins_without_a_pass_over_the_joined_matrix():
         model(inp_layer([torch.as_tensor(coords), feats]))
     finally:
         layers.concat_join_batchnorm = orig
-    assert taken == [False, False], taken
+    assert taken == [(False, False)] * 2, taken
 
 
 def test_frozen_parameters_of_a_wide_layer_do_not_grow():
