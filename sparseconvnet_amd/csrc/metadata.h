@@ -354,7 +354,7 @@ void conv_first_forward(const Table &t, const float *in, int64_t in_rows, float 
 // sort.hip: stable radix sort of (key, value) pairs by the low end_bit bits of the key; the input
 // arrays are left as they are, scratch comes from m.tmp.
 void radix_sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long long *kout, const int *vin, int *vout,
-                      int64_t n, int end_bit, hipStream_t s);
+                      int64_t n, int end_bit, hipStream_t s, const int *n_dev = nullptr);
 
 // ops.hip / conv.hip
 unsigned char *noalloc_scratch();  // the static scratch array's address on the current device

@@ -1484,14 +1484,102 @@ __global__ void k_strided_candidates(Geom gi, Geom go, Filt f, const int *soa, c
   payload[e] = (int)e;
 }
 
-// head[p] = 1 where a new output site begins in the sorted candidate keys.
-__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head) {
-  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p == n) head[p] = 0;  // one element past the end, so that a scan of n + 1 ends with the total
-  if (p < n) {
-    const unsigned long long k = skeys[p];
-    head[p] = (k != SCN_EMPTY_KEY && (p == 0 || k != skeys[p - 1])) ? 1 : 0;
+// The same candidates without the slots that hold none (filters larger than their stride: a site
+// of a 3^3 / stride-2 filter has 3.4 of its 8 on average, and the sort behind this is what a
+// strided rulebook costs).  One thread per site, CB sites per workgroup; the first launch
+// (WRITE = false) counts each workgroup's candidates, the second adds up the counts in front of
+// its own, numbers its sites' candidates with a prefix inside the workgroup and writes them in
+// (site, candidate) order; *n_valid = their number, which stays on the device (the launches
+// behind are sized for n * M and look it up).
+constexpr int CB = 256;
+template <bool WRITE>
+__global__ __launch_bounds__(CB) void k_strided_compact(Geom gi, Geom go, Filt f, const int *soa, const int *sched,
+                                                        const unsigned long long *pos_keys, int64_t n, int64_t npad,
+                                                        const unsigned long long *dup_keys, int *block_counts,
+                                                        unsigned long long *keys, int *payload, int *n_valid) {
+  __shared__ int part[CB / 64], wave_n[CB / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * CB + threadIdx.x;
+  int p[SCN_MAXD], j[SCN_MAXD], lb[SCN_MAXD], cnt[SCN_MAXD];
+  int b = 0, mine = 0;
+  const bool site = t < n && !(dup_keys && t + 1 < n && dup_keys[t + 1] == dup_keys[t]);
+  if (site) {
+    if (pos_keys) {
+      site_of_key(gi, pos_keys[t], p, b);
+    } else {
+      const int row = sched ? sched[t] : (int)t;
+      for (int d = 0; d < f.dim; d++) p[d] = soa[d * npad + row];
+      b = soa[f.dim * npad + row];
+    }
+    // candidate() per dimension, once: the first output coordinate and how many there are; a
+    // site's candidates are the product of the dimensions' ranges
+    mine = 1;
+    for (int d = 0; d < f.dim; d++) {
+      const int num = p[d] - f.size[d] + 1;
+      lb[d] = num <= 0 ? 0 : (num + f.stride[d] - 1) / f.stride[d];
+      const int ub = min(f.out_size[d] - 1, p[d] / f.stride[d]);
+      cnt[d] = max(0, min(ub - lb[d] + 1, f.m[d]));
+      mine *= cnt[d];
+    }
   }
+  int incl = mine;  // inclusive prefix over the wavefront
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  if (lane == 63) wave_n[wave] = incl;
+  if constexpr (!WRITE) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int total = 0;
+      for (int w = 0; w < CB / 64; w++) total += wave_n[w];
+      block_counts[blockIdx.x] = total;
+    }
+    return;
+  }
+  int before = 0;
+  for (int i = threadIdx.x; i < (int)blockIdx.x; i += CB) before += block_counts[i];
+#pragma unroll
+  for (int o = 32; o; o >>= 1) before += __shfl_xor(before, o, 64);
+  if (lane == 0) part[wave] = before;
+  __syncthreads();
+  int pos = incl - mine, all = 0;
+  for (int w = 0; w < CB / 64; w++) {
+    pos += part[w] + (w < wave ? wave_n[w] : 0);
+    all += part[w] + wave_n[w];
+  }
+  if (site && mine)
+    for (int m = 0; m < f.M; m++) {  // numbered as candidate() numbers them: the last dimension fastest
+      bool ok = true;
+      int rest = m;
+      for (int d = f.dim - 1; d >= 0; d--) {
+        const int md = rest % f.m[d];
+        rest /= f.m[d];
+        j[d] = lb[d] + md;
+        ok = ok && md < cnt[d];
+      }
+      if (ok) {
+        keys[pos] = site_key(go, j, b);
+        payload[pos] = (int)(t * f.M + m);
+        pos++;
+      }
+    }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *n_valid = all;
+}
+
+// head[p] = 1 where a new output site begins in the sorted candidate keys.  n_dev (optional): the
+// number of keys when only the device knows it; n is then the bound the launch is sized for.
+__global__ void k_strided_heads(const unsigned long long *skeys, int64_t n, int *head, const int *n_dev) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p > n) return;
+  const int64_t nv = n_dev ? *n_dev : n;
+  if (p >= nv) {
+    head[p] = 0;  // up to one element past the end, so that a scan of n + 1 ends with the total
+    return;
+  }
+  const unsigned long long k = skeys[p];
+  head[p] = (k != SCN_EMPTY_KEY && (p == 0 || k != skeys[p - 1])) ? 1 : 0;
 }
 
 // One thread per sorted candidate: output row = number of heads before it; the filter tap
@@ -1501,10 +1589,11 @@ __global__ void k_strided_emit(Geom gi, Filt f, const int *soa, const int *sched
                                int64_t npad_in, const unsigned long long *skeys, const int *spayload, const int *head,
                                const int *head_scan, int64_t n_cand, int64_t npad_out, int *by_out,
                                int *by_in, int *out_soa, unsigned long long *out_keys,
-                               unsigned long long *counts) {
+                               unsigned long long *counts, const int *n_dev) {
   extern __shared__ int lcount[];  // per-block rule counts, flushed with one atomic per tap
   for (int k = threadIdx.x; k < f.K; k += blockDim.x) lcount[k] = 0;
   __syncthreads();
+  if (n_dev) n_cand = *n_dev;
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   unsigned long long key = p < n_cand ? skeys[p] : SCN_EMPTY_KEY;
   if (key != SCN_EMPTY_KEY) {
@@ -1787,12 +1876,28 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   // a level with a schedule of its own (the input layer's): sites from the positions' keys
   const unsigned long long *pos_keys = (m.dim <= 3 && !LI.identity_sched) ? position_keys(LI, s) : nullptr;
   const unsigned long long *dup_keys = LI.dups ? position_keys(LI, s) : nullptr;
-  k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
-                                                   m.k0.p, m.v0.p, dup_keys);
-  LAUNCH_CHECK();
-  // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
-  sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
-  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p);
+  const int *n_cand_dev = nullptr;
+  if (f.M > 1 && nc > 32768 && nc <= ((int64_t)1 << 24)) {
+    // only the slots that hold a candidate go into the sort; their number stays on the device
+    const int blocks = (int)ceil_div(n, CB);
+    m.f1.reserve(blocks);
+    m.s1.reserve(1);
+    k_strided_compact<false><<<dim3(blocks), CB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
+                                                       dup_keys, m.f1.p, nullptr, nullptr, nullptr);
+    LAUNCH_CHECK();
+    k_strided_compact<true><<<dim3(blocks), CB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
+                                                      dup_keys, m.f1.p, m.k0.p, m.v0.p, m.s1.p);
+    LAUNCH_CHECK();
+    n_cand_dev = m.s1.p;
+    radix_sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, std::min(64, key_bits(go, batch)), s, n_cand_dev);
+  } else {
+    k_strided_candidates<<<grid_for(nc), TB, 0, s>>>(LI.g, go, f, LI.coords.p, LI.sched_ptr(), pos_keys, n, LI.npad,
+                                                     m.k0.p, m.v0.p, dup_keys);
+    LAUNCH_CHECK();
+    // one bit above the key bits keeps the EMPTY keys (all ones) behind every real key
+    sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, nc, s, std::min(64, key_bits(go, batch) + 1));
+  }
+  k_strided_heads<<<grid_for(nc + 1), TB, 0, s>>>(m.k1.p, nc, m.f0.p, n_cand_dev);
   LAUNCH_CHECK();
   exclusive_scan(m, m.f0.p, m.s0.p, nc + 1, s);
   const int64_t n_out = fetch_words(m, m.s0.p + nc, 1, s)[0];
@@ -1809,7 +1914,7 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
         R.by_out.cnt->dev.p, 0u, 2 * (int64_t)COUNT_SLOTS * std::max(f.K, 1), s);
   k_strided_emit<<<grid_for(nc), TB, f.K * sizeof(int), s>>>(LI.g, f, LI.coords.p, LI.sched_ptr(), pos_keys, LI.npad, m.k1.p, m.v1.p,
                                              m.f0.p, m.s0.p, nc, LO.npad, R.by_out.nbr.p, R.by_in.nbr.p,
-                                             LO.coords.p, LO.keys.p, (unsigned long long *)R.by_out.cnt->dev.p);
+                                             LO.coords.p, LO.keys.p, (unsigned long long *)R.by_out.cnt->dev.p, n_cand_dev);
   LAUNCH_CHECK();
   R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
   finalize_table(m, R.by_out, nullptr, s);

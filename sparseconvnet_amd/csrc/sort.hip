@@ -29,8 +29,9 @@ constexpr int RS_MAX_BITS = 10, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit
 
 template <int RS_ITEMS>
 __global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const u64 *__restrict__ keys, int64_t n, int shift, int bits,
-                                                        int tiles, int *__restrict__ hist) {
+                                                        int tiles, int *__restrict__ hist, const int *__restrict__ n_dev) {
   __shared__ int h[RS_MAX_BINS];
+  if (n_dev) n = *n_dev;  // the number of pairs when only the device knows it (n: an upper bound the grid was sized for)
   const int bins = 1 << bits;
   for (int d = threadIdx.x; d < bins; d += RS_THREADS) h[d] = 0;
   __syncthreads();
@@ -100,8 +101,9 @@ template <int RS_ITEMS>
 __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict__ kin, const int *__restrict__ vin,
                                                            u64 *__restrict__ kout, int *__restrict__ vout, int64_t n,
                                                            int shift, int bits, int tiles, const int *__restrict__ offs,
-                                                           const int *__restrict__ tot) {
+                                                           const int *__restrict__ tot, const int *__restrict__ n_dev) {
   constexpr int RS_TILE = RS_THREADS * RS_ITEMS;
+  if (n_dev) n = *n_dev;
   __shared__ int cnt[RS_WAVES][RS_MAX_BINS];
   __shared__ int base[RS_MAX_BINS];    // where the tile's first pair of each digit value goes
   __shared__ int lstart[RS_MAX_BINS];  // the same inside the tile: pairs of smaller digit values
@@ -213,8 +215,9 @@ constexpr int RS1_THREADS = 1024, RS1_WAVES = 16, RS1_ITEMS = 4, RS1_MAX = RS1_T
 constexpr int RS1_BITS = 8, RS1_BINS = 1 << RS1_BITS;
 __global__ __launch_bounds__(RS1_THREADS) void k_rs_single(const u64 *__restrict__ kin, const int *__restrict__ vin,
                                                            u64 *__restrict__ kout, int *__restrict__ vout, int n,
-                                                           int end_bit, int width) {
+                                                           int end_bit, int width, const int *__restrict__ n_dev) {
   constexpr int ITEMS = RS1_ITEMS;
+  if (n_dev) n = *n_dev;
   __shared__ int cnt[RS1_WAVES][RS1_BINS];
   __shared__ int lstart[RS1_BINS];
   __shared__ int wsum[RS1_BINS / 64];
@@ -291,8 +294,10 @@ __global__ __launch_bounds__(RS1_THREADS) void k_rs_single(const u64 *__restrict
   }
 }
 
+// n_dev (optional): the number of pairs, on the device; n is then an upper bound that sizes the
+// launches, and tiles past the real end find nothing to do.
 void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, int *vout, int64_t n, int end_bit,
-                      hipStream_t s) {
+                      hipStream_t s, const int *n_dev) {
   if (n <= 0) return;
   end_bit = std::max(1, std::min(64, end_bit));
   if (n >= ((int64_t)1 << 31)) throw Error("sort: too many pairs");
@@ -301,7 +306,7 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
   const int width = (end_bit + passes - 1) / passes;
   if (n <= RS1_MAX) {
     const int p1 = (end_bit + RS1_BITS - 1) / RS1_BITS;
-    k_rs_single<<<dim3(1), RS1_THREADS, 0, s>>>(kin, vin, kout, vout, (int)n, end_bit, (end_bit + p1 - 1) / p1);
+    k_rs_single<<<dim3(1), RS1_THREADS, 0, s>>>(kin, vin, kout, vout, (int)n, end_bit, (end_bit + p1 - 1) / p1, n_dev);
     LAUNCH_CHECK();
     return;
   }
@@ -332,13 +337,13 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
     u64 *kdst = to_out ? kout : ktmp;
     int *vdst = to_out ? vout : vtmp;
     const int shift = width * pass, bits = std::min(width, end_bit - shift);
-    if (big) k_rs_hist<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist);
-    else k_rs_hist<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist);
+    if (big) k_rs_hist<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);
+    else k_rs_hist<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);
     LAUNCH_CHECK();
     k_rs_colscan<<<dim3(1 << bits), 64, 0, s>>>(hist, tiles, tot);
     LAUNCH_CHECK();
-    if (big) k_rs_scatter<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot);
-    else k_rs_scatter<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot);
+    if (big) k_rs_scatter<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot, n_dev);
+    else k_rs_scatter<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot, n_dev);
     LAUNCH_CHECK();
     ksrc = kdst;
     vsrc = vdst;
