@@ -16,8 +16,11 @@
 // ballot per digit bit, the first of them reads and bumps the wavefront's running count of that value in LDS
 // (only this wavefront touches its counts, so no barrier), which gives every pair its rank
 // inside the wavefront's quarter; a prefix over the four wavefronts' counts then orders the
-// quarters.  (Below a few ten thousand pairs the library's merge sort is faster and the callers use it.)
+// quarters.  (Between four and thirty-two thousand pairs the library's merge sort is faster and the
+// callers use it; up to 4096 pairs k_rs_single sorts in one launch, see there.)
 // The input arrays are not written: passes alternate between the output arrays and scratch.
+// The number of pairs may live on the device only (n_dev): the launches are then sized for an
+// upper bound and tiles past the real end find nothing to do.
 #include "metadata.h"
 
 namespace scn {
