@@ -120,14 +120,15 @@ def check_mode0_repeated_points(make, dim, seed, n=300, spatial=9, batch=2, cin=
     assert_close(p.output_fwd(y), y)
     # a strided rulebook over the same level: its rules start from the winners only
     # (Metadata/ConvolutionRules.h:61-105 walks the input grids)
-    if spatial == 9:
-        srules = p.strided_rules(9, 4, 3, 2)
-        loc_out = p.spatial_locations(4)
+    if spatial % 2 == 1:
+        out3 = (spatial - 3) // 2 + 1
+        srules = p.strided_rules(spatial, out3, 3, 2)
+        loc_out = p.spatial_locations(out3)
         got_s = set()
         for k, r in enumerate(srules):
             for i, j in np.asarray(r).reshape(-1, 2).tolist():
                 got_s.add((k, int(i)) + tuple(loc_out[j].tolist()))
-        want_s = set((t[0], last[t[1:2 + dim]]) + t[2 + dim:] for t in bf.strided_triples(sites, dim, 3, 2, 4))
+        want_s = set((t[0], last[t[1:2 + dim]]) + t[2 + dim:] for t in bf.strided_triples(sites, dim, 3, 2, out3))
         assert got_s == want_s
         assert sum(len(r) for r in srules) == len(got_s)
     # filter 2 / stride 2 over a size that halves exactly (the builders' path without a sort), and

@@ -89,6 +89,8 @@ def test_input_layer_mode0_repeated_points(make, dim):
     checks.check_mode0_repeated_points(make, dim, seed=50 + dim, spatial=8)
     if dim == 3:  # many workgroups, MFMA convolution kernel
         checks.check_mode0_repeated_points(make, dim, seed=44, n=20000, spatial=48, cin=16, cout=16)
+        # an odd grid: the 3 / stride-2 rulebook with its candidates compacted (160 k slots)
+        checks.check_mode0_repeated_points(make, dim, seed=45, n=20000, spatial=49, cin=8, cout=8)
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
