@@ -36,6 +36,9 @@ struct Level {
   bool skeys_ready = false;
   bool grid_built = false;
   bool dups = false;
+  // Set when a strided rulebook makes the level: which construction of this spatial size it is
+  // (a rulebook that still has to look its sites up checks that they are the ones it made).
+  uint64_t gen = 0;
   // Active-site counts of the levels that successive filter 2 / stride 2 rulebooks make of this
   // one (size halved once, twice, ...), when somebody has computed them (metadata.hip:
   // halving_sizes): a strided build that finds its output size here needs no read-back.
@@ -106,6 +109,12 @@ struct StridedRules {
   // (tap, coarse row) until finish_by_in writes the table in its sorted order (in_tap[t] < 0: no rule).
   bool by_in_compact = false;
   DevBuf<int> in_tap, in_row;
+  // Rulebooks built by looking the fine sites up from the coarse ones (strided_rules: filters larger
+  // than their stride): by_in does not exist until finish_by_in makes it the same way, from the
+  // coarse level's site lookup; out_gen = Level::gen of the coarse level the rulebook made.
+  bool by_in_lookup = false;
+  uint64_t out_gen = 0;
+  std::vector<int64_t> filter, stride;  // kept for that
   SizeKey in_size, out_size;
 };
 
@@ -215,6 +224,8 @@ struct Metadata {
   DevBuf<float> wcols;  // column ranges of a wide layer's weights, one contiguous block per range (conv_forward)
   DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
+  DevBuf<int> ob_words, ob_list, ob_part;  // strided rulebooks by lookup: counters, the coarse level's blocks, partial ranks
+  uint64_t level_gen = 0;
   std::function<void()> before_pack;  // work the packing of the running convolution's weights needs first (the column-range path's copy), run at most once
   // while a column range of a wide layer runs: addresses in the scratch copy (from wkey_from) stand for
   // addresses from wkey_ptr in the caller's weights in a frozen set's keys

@@ -83,6 +83,7 @@ void wait_for_consumers(Metadata &m, hipStream_t s) {
   HIP_CHECK(hipEventDestroy(ev));  // released once it has completed
 }
 
+static void settle_lookups(Metadata &m, const SizeKey &size, hipStream_t s);
 static const int COUNT_SLOTS = 32;  // copies of a rulebook's per-tap counters (a power of two)
 
 __global__ void k_fill32(uint32_t *p, uint32_t v, int64_t n) {
@@ -392,6 +393,7 @@ void build_input_layer(Metadata &m, const int64_t *spatial, CoordSrc coords, int
   Geom g = make_geom(m.dim, spatial);
   SizeKey key = mk(m.dim, spatial);
   m.input_size = key;
+  if (m.levels.count(key)) settle_lookups(m, key, s);
   Level &L = m.levels[key];
   InputRules &R = m.input;
   // Metadata/IOLayersRules.h:96-107 against :180-205: the plain layer lists the first point of
@@ -633,10 +635,12 @@ __global__ __launch_bounds__(SITE_THREADS) void k_site_compact(const unsigned lo
   grid_count(heads, ticket);
 }
 // The size of a level's block table is decided on the device (no host round trip): from the
-// number of blocks, capacity = the power of two >= 2 * blocks (at least 64).
-__device__ inline unsigned long long grid_capacity(long long nblocks) {
+// number of blocks, capacity = the power of two >= 4 * blocks (at least 64), within what is
+// allocated (room for twice as many blocks as there are sites).  A wavefront of a rule kernel waits
+// for the longest of its lanes' probe sequences: a table a quarter to an eighth full keeps those short.
+__device__ inline unsigned long long grid_capacity(long long nblocks, long long cap_alloc) {
   unsigned long long cap = 64;
-  while (cap < (unsigned long long)nblocks * 2ull) cap <<= 1;
+  while (cap < (unsigned long long)nblocks * 4ull && cap < (unsigned long long)cap_alloc) cap <<= 1;
   return cap;
 }
 // skey[t] = key of the row at schedule position t; head[t] = 1 where a block of 64 keys starts;
@@ -671,7 +675,7 @@ __global__ void k_block_heads(const unsigned long long *ukey, int64_t n, const i
 __global__ void k_block_clear(BlockEntry *table, int64_t cap_alloc, const unsigned long long *ticket,
                               unsigned long long *mask_out) {
   int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const unsigned long long cap = grid_capacity((long long)ticket[1]);
+  const unsigned long long cap = grid_capacity((long long)ticket[1], cap_alloc);
   if (b == 0) *mask_out = cap - 1;
   if (b < cap_alloc && (unsigned long long)b < cap) {
     table[b].key = SCN_EMPTY_KEY;
@@ -782,11 +786,17 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
 struct Filt {
   int dim, K, M;
   int size[SCN_MAXD], stride[SCN_MAXD], out_size[SCN_MAXD], m[SCN_MAXD];
+  // tap k of the site c of a position reads c * stride + k - off: off = size / 2 for a submanifold
+  // filter (stride 1, centred), 0 for a strided one read from its coarse side
+  int off[SCN_MAXD];
 };
 
 // One thread per schedule position t: probe the filter box around the row's site
 // (Metadata/SubmanifoldConvolutionRules.h:11-45; taps enumerate the box row-major with the
 // last dimension fastest, Metadata/RectangularRegions.h:56-71).
+// The positions may also be those of the coarse level of a strided filter (soa, sched, n, npad
+// describe them) and g, table, urow the fine level its taps are looked up in
+// (Metadata/ConvolutionRules.h:19-31 read from the output side): f.stride and f.off say which.
 // dup_keys (levels whose keys may repeat, else null): the positions' keys, ascending; of a run of
 // equal keys only the last position is a site (`mp[p] = i`, Metadata/IOLayersRules.h:41,54), the
 // others are rows no rule touches.
@@ -824,7 +834,7 @@ __global__ void k_subm_rules(Geom g, Filt f, const int *soa, const int *sched, i
     for (int k = k0; k < k0 + per; k++) {
       bool inside = !shadowed;
       for (int d = 0; d < g.dim; d++) {
-        q[d] = c[d] + tap[d] - f.size[d] / 2;
+        q[d] = c[d] * f.stride[d] + tap[d] - f.off[d];
         if (q[d] < 0 || q[d] >= g.size[d]) inside = false;
       }
       int j = -1;
@@ -1113,9 +1123,13 @@ static void finalize_table(Metadata &m, Table &t, const int *base, hipStream_t s
 // is the OR of per-coordinate spread values, so each coordinate is spread three times per
 // site (for c-1, c, c+1) instead of once per tap, and the tap loop is fully unrolled.
 // One wavefront per slice of the first filter dimension, as in k_subm_rules.
+// HALF: the same filter at stride 2, looked up from the coarse side (Metadata/ConvolutionRules.h:19-31
+// read backwards): the positions are the sites of the coarse level (keys of pos_bits bits per
+// coordinate), the site c of one has the taps 2c, 2c+1, 2c+2 per dimension in level g, whose
+// table this is.
 #define S3_ROW_INTS(dim) ((dim) == 3 ? 32 : 12)  // ints per site of the site-major table: 27 or 9 taps, padded to 16 bytes
-template <int DIM>
-__global__ void k_subm_rules_s3(Geom g, const unsigned long long *skeys, int64_t n, int64_t npad,
+template <int DIM, bool HALF>
+__global__ void k_subm_rules_s3(Geom g, int pos_bits, const unsigned long long *skeys, int64_t n, int64_t npad,
                                 const BlockEntry *table, const unsigned long long *mask_p, const int *urow,
                                 int *rows, unsigned long long *counts, PatternKey pk, unsigned long long *pkeys,
                                 int *pidx, unsigned *pmasks, bool dups) {
@@ -1152,18 +1166,18 @@ __global__ void k_subm_rules_s3(Geom g, const unsigned long long *skeys, int64_t
   int cd[DIM];
 #pragma unroll
   for (int d = 0; d < DIM; d++) {
-    const int c = DIM == 3 ? (int)compact3(skey >> (DIM - 1 - d)) & ((1 << g.bits) - 1)
-                           : (int)compact2(skey >> (DIM - 1 - d)) & ((1 << g.bits) - 1);
-    cd[d] = c;
+    const int c = DIM == 3 ? (int)compact3(skey >> (DIM - 1 - d)) & ((1 << pos_bits) - 1)
+                           : (int)compact2(skey >> (DIM - 1 - d)) & ((1 << pos_bits) - 1);
+    cd[d] = HALF ? 2 * c + 1 : c;  // the middle tap's coordinate in level g
 #pragma unroll
     for (int o = 0; o < 3; o++) {
-      const int v = c + o - 1;
+      const int v = cd[d] + o - 1;
       okc[d][o] = v >= 0 && v < g.size[d];
       const unsigned long long s = DIM == 3 ? spread3((unsigned)v) : spread2((unsigned)v);
       sp[d][o] = s << (DIM - 1 - d);
     }
   }
-  const unsigned long long bpart = (skey >> (DIM * g.bits)) << (DIM * g.bits);  // the sample index, in place
+  const unsigned long long bpart = (skey >> (DIM * pos_bits)) << (DIM * g.bits);  // the sample index, in its place in level g's keys
   // The lane's taps (first-dimension offset fixed by its wavefront) lie in at most two blocks
   // along each remaining dimension: the blocks of the lowest and of the highest in-range
   // coordinate.  All of them (two, or two by two) are looked up at once, whole 32-byte entries,
@@ -1293,6 +1307,7 @@ static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const
     if (f.stride[d] < 1) throw Error("filter stride must be positive");
     f.out_size[d] = out_size ? (int)out_size[d] : 0;
     f.m[d] = (f.size[d] + f.stride[d] - 1) / f.stride[d];
+    f.off[d] = stride ? 0 : f.size[d] / 2;
     K *= size[d];
     M *= f.m[d];
     if (K > 4096) throw Error("filter volume above 4096 is not supported");
@@ -1419,11 +1434,11 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
     const int roww = S3_ROW_INTS(m.dim);
     m.rowtab.reserve((size_t)t.npad * roww);
     if (m.dim == 3)
-      k_subm_rules_s3<3><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.skeys.p, L.n, L.npad, L.table.p,
+      k_subm_rules_s3<3, false><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.g.bits, L.skeys.p, L.n, L.npad, L.table.p,
                                                            L.gridp.p, L.urow_ptr(), m.rowtab.p,
                                                            (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks, L.dups);
     else
-      k_subm_rules_s3<2><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.skeys.p, L.n, L.npad, L.table.p,
+      k_subm_rules_s3<2, false><<<dim3((unsigned)(8 * ceil_div(ceil_div(L.n, 64), 8))), 192, 0, s>>>(L.g, L.g.bits, L.skeys.p, L.n, L.npad, L.table.p,
                                                            L.gridp.p, L.urow_ptr(), m.rowtab.p,
                                                            (unsigned long long *)t.cnt->dev.p, pk, m.k0.p, m.v0.p, masks, L.dups);
     LAUNCH_CHECK();
@@ -1767,6 +1782,335 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift,
   if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&slot[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
 }
 
+// ---- filters larger than their stride, small and middle levels: rules by lookup ----
+// The sort of every (output site, input site) candidate is what such a rulebook costs on the
+// general path.  Here the output sites are found first, as occupancy bits of their blocks of 64 keys
+// in the block table that becomes the output level's site lookup (k_ob_mark); the blocks are listed
+// (k_ob_list) and put in key order by counting, for each, the sites of the blocks with smaller keys,
+// all pairs at once (k_ob_rank: a few thousand blocks at most); the sites are written in that order (k_ob_sites), which
+// is the ascending key order the general path gives them; and the rules are looked up from the
+// output side in the input level's table, as a submanifold rulebook's are.  The fine-side table is
+// made the same way from the other side, when somebody asks for it (finish_by_in).
+constexpr int OB_CAP = 65536;    // slots of the output level's block table on this path
+constexpr int OB_MAX = 16384;    // blocks it may hold: above, the build falls back to the general path
+constexpr int OB_PARTS = 32;     // k_ob_rank: pieces the blocks compared against are split into
+constexpr int OB_MAX_M = 32;     // most candidates per input site
+constexpr int OB_PROBES = 64;    // a probe sequence longer than this means a crowded table: fall back
+constexpr int64_t OB_MAX_SITES = 400000;  // input sites above which the general path is taken right away
+struct ObBlock {  // a block of the list
+  unsigned long long key;
+  int sites, slot;  // set bits of its mask; its slot in the table
+};
+// words: [0] blocks listed, [1] set when the path gives up, [2] output sites.
+__global__ void k_ob_clear(BlockEntry *table, unsigned long long *gridp, int *words, uint32_t *zero, int zero_words) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < OB_CAP) {
+    table[b].key = SCN_EMPTY_KEY;
+    table[b].mask = 0ull;
+    table[b].base = 0;
+  }
+  if (b == 0) gridp[0] = OB_CAP - 1;
+  if (b < 4) words[b] = 0;
+  for (int i = b; i < zero_words; i += gridDim.x * blockDim.x) zero[i] = 0u;
+}
+// ORs `bits` into the entry of block bkey, claiming a slot for it when it has none: one atomic
+// whose answer is waited for, one that is not.
+__device__ inline void ob_insert(BlockEntry *table, unsigned long long bkey, unsigned long long bits, int *words) {
+  unsigned long long b = hash64(bkey) & (OB_CAP - 1);
+  for (int i = 0; i < OB_PROBES; i++) {
+    const unsigned long long k = atomicCAS(&table[b].key, SCN_EMPTY_KEY, bkey);
+    if (k == SCN_EMPTY_KEY || k == bkey) {
+      atomicOr(&table[b].mask, bits);
+      return;
+    }
+    b = (b + 1) & (OB_CAP - 1);
+  }
+  words[1] = 1;
+}
+// One thread per input position: its candidate output sites (Metadata/RectangularRegions.h:109-119),
+// block by block.  The positions of a workgroup are neighbours in space and their candidates lie
+// in a handful of blocks: they meet in a small table in LDS first, and the workgroup then
+// inserts each of its blocks once (atomics on device memory are what this kernel would wait for).
+constexpr int OB_LSLOTS = 256;
+__global__ __launch_bounds__(TB) void k_ob_mark(Geom gi, Geom go, Filt f, const unsigned long long *pos_keys, int64_t n,
+                                                bool dups, BlockEntry *table, int *words) {
+  __shared__ unsigned long long lkey[OB_LSLOTS], lbits[OB_LSLOTS];
+  for (int i = threadIdx.x; i < OB_LSLOTS; i += TB) {
+    lkey[i] = SCN_EMPTY_KEY;
+    lbits[i] = 0ull;
+  }
+  __syncthreads();
+  auto put = [&](unsigned long long bkey, unsigned long long bits) {
+    unsigned h = (unsigned)((bkey * 0x9E3779B97F4A7C15ull) >> 40) & (OB_LSLOTS - 1);
+    for (int i = 0; i < OB_LSLOTS; i++) {
+      const unsigned long long k = atomicCAS(&lkey[h], SCN_EMPTY_KEY, bkey);
+      if (k == SCN_EMPTY_KEY || k == bkey) {
+        atomicOr(&lbits[h], bits);
+        return;
+      }
+      h = (h + 1) & (OB_LSLOTS - 1);
+    }
+    ob_insert(table, bkey, bits, words);  // more blocks than the small table holds (scattered points)
+  };
+  const int64_t t = (int64_t)blockIdx.x * TB + threadIdx.x;
+  const bool stop = *reinterpret_cast<volatile int *>(words + 1) != 0;
+  if (t < n && !stop && !(dups && t + 1 < n && pos_keys[t + 1] == pos_keys[t])) {
+    int p[SCN_MAXD], j[SCN_MAXD], lb[SCN_MAXD], cnt[SCN_MAXD];
+    int b;
+    site_of_key(gi, pos_keys[t], p, b);
+    // per dimension: the first output coordinate and how many there are (strides 1 and 2 without a division)
+    for (int d = 0; d < 3; d++) {
+      lb[d] = 0;
+      cnt[d] = 1;
+      if (d >= f.dim) continue;
+      const int st = f.stride[d], num = p[d] - f.size[d] + 1;
+      const int up = num <= 0 ? 0 : (st == 1 ? num : st == 2 ? (num + 1) >> 1 : (num + st - 1) / st);
+      const int down = st == 1 ? p[d] : st == 2 ? p[d] >> 1 : p[d] / st;
+      lb[d] = up;
+      cnt[d] = max(0, min(min(f.out_size[d] - 1, down) - up + 1, f.m[d]));
+    }
+    // the candidates are the product of the ranges; their order does not matter here
+    unsigned long long cur = SCN_EMPTY_KEY, bits = 0ull;
+    for (int a0 = 0; a0 < cnt[0]; a0++)
+      for (int a1 = 0; a1 < cnt[1]; a1++)
+        for (int a2 = 0; a2 < cnt[2]; a2++) {
+          j[0] = lb[0] + a0;
+          j[1] = lb[1] + a1;
+          j[2] = lb[2] + a2;
+          const unsigned long long key = site_key(go, j, b);
+          if ((key >> 6) != cur) {
+            if (cur != SCN_EMPTY_KEY) put(cur, bits);
+            cur = key >> 6;
+            bits = 0ull;
+          }
+          bits |= 1ull << (key & 63);
+        }
+    if (cur != SCN_EMPTY_KEY) put(cur, bits);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < OB_LSLOTS; i += TB)
+    if (lkey[i] != SCN_EMPTY_KEY) ob_insert(table, lkey[i], lbits[i], words);
+}
+// The blocks of the table, listed (in no order): one thread per slot, one atomic per workgroup.
+__global__ __launch_bounds__(TB) void k_ob_list(const BlockEntry *table, ObBlock *list, int *words) {
+  __shared__ int wave_n[TB / 64], wg_base;
+  const int slot = blockIdx.x * TB + threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned long long key = table[slot].key;
+  const bool live = key != SCN_EMPTY_KEY;
+  const unsigned long long ballot = __ballot(live);
+  if (lane == 0) wave_n[wave] = __popcll(ballot);
+  __syncthreads();
+  int before = 0, total = 0;
+  for (int w = 0; w < TB / 64; w++) {
+    before += w < wave ? wave_n[w] : 0;
+    total += wave_n[w];
+  }
+  if (threadIdx.x == 0 && total) {
+    wg_base = atomicAdd(&words[0], total);
+    if (wg_base + total > OB_MAX) words[1] = 1;
+  }
+  __syncthreads();
+  if (!live) return;
+  const int i = wg_base + before + __popcll(ballot & ((1ull << lane) - 1ull));
+  if (i < OB_MAX) {
+    ObBlock e;
+    e.key = key;
+    e.sites = __popcll(table[slot].mask);
+    e.slot = slot;
+    list[i] = e;
+  }
+}
+// base of every listed block = the sites of the listed blocks with smaller keys.  Workgroup
+// (x, y): blocks 256 x .. of the list against piece y of it, a tile of 256 at a time through LDS:
+// partial[y][r] = the sites of piece y's blocks in front of block r, which k_ob_sites adds up.
+// words[2] = all sites.
+__global__ __launch_bounds__(256) void k_ob_rank(const ObBlock *list, int *partial, int *words) {
+  const int nb = words[0];
+  if (words[1] || (int)blockIdx.x * 256 >= nb) return;
+  __shared__ unsigned long long tkey[256];
+  __shared__ int tpop[256];
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  const unsigned long long key = r < nb ? list[r].key : 0ull;
+  const int per = (nb + (int)gridDim.y - 1) / (int)gridDim.y;
+  const int j0 = blockIdx.y * per, j1 = min(nb, j0 + per);
+  int acc = 0, tot = 0;
+  for (int base = j0; base < j1; base += 256) {
+    const int j = base + threadIdx.x;
+    __syncthreads();
+    if (j < j1) {
+      const ObBlock e = list[j];
+      tkey[threadIdx.x] = e.key;
+      tpop[threadIdx.x] = e.sites;
+      tot += e.sites;
+    }
+    __syncthreads();
+    const int cnt = min(256, j1 - base);
+    int i = 0;
+    for (; i + 4 <= cnt; i += 4) {  // four at a time: the reads of LDS overlap
+      const unsigned long long k0 = tkey[i], k1 = tkey[i + 1], k2 = tkey[i + 2], k3 = tkey[i + 3];
+      const int p0 = tpop[i], p1 = tpop[i + 1], p2 = tpop[i + 2], p3 = tpop[i + 3];
+      acc += (k0 < key ? p0 : 0) + (k1 < key ? p1 : 0) + (k2 < key ? p2 : 0) + (k3 < key ? p3 : 0);
+    }
+    for (; i < cnt; i++) acc += tkey[i] < key ? tpop[i] : 0;
+  }
+  if (r < nb) partial[(size_t)blockIdx.y * OB_MAX + r] = acc;
+  if (blockIdx.x == 0) {
+    __shared__ int wg_tot;
+    if (threadIdx.x == 0) wg_tot = 0;
+    __syncthreads();
+#pragma unroll
+    for (int o = 32; o; o >>= 1) tot += __shfl_xor(tot, o, 64);
+    if ((threadIdx.x & 63) == 0 && tot) atomicAdd(&wg_tot, tot);
+    __syncthreads();
+    if (threadIdx.x == 0 && wg_tot) atomicAdd(&words[2], wg_tot);
+  }
+}
+// One wavefront per listed block, one lane per key of it: the block's base into the table and the
+// output level's rows, in ascending key order.
+__global__ __launch_bounds__(256) void k_ob_sites(Geom go, BlockEntry *table, const ObBlock *list, const int *partial, int nb,
+                                                  int64_t npad, int *soa, unsigned long long *keys,
+                                                  unsigned long long *skeys) {
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (r >= nb) return;
+  int base = lane < OB_PARTS ? partial[(size_t)lane * OB_MAX + r] : 0;
+#pragma unroll
+  for (int o = 32; o; o >>= 1) base += __shfl_xor(base, o, 64);
+  const ObBlock blk = list[r];
+  BlockEntry *e = table + blk.slot;
+  if (lane == 0) e->base = base;
+  const unsigned long long mask = e->mask;
+  if (!((mask >> lane) & 1ull)) return;
+  const int row = base + __popcll(mask & ((1ull << lane) - 1ull));
+  const unsigned long long key = (blk.key << 6) | (unsigned long long)lane;
+  int c[SCN_MAXD], b;
+  site_of_key(go, key, c, b);
+  for (int d = 0; d < go.dim; d++) soa[d * npad + row] = c[d];
+  soa[go.dim * npad + row] = b;
+  keys[row] = key;
+  skeys[row] = key;
+}
+// The fine-side table of such a rulebook: one thread per fine position, every tap k of its site p
+// has the output site (p - k) / stride where that is whole and inside
+// (Metadata/RectangularRegions.h:30-38,95-105), looked up in the coarse level's table.
+__global__ void k_rules_from_fine(Geom gi, Geom go, Filt f, const unsigned long long *pos_keys, int64_t n, int64_t npad,
+                                  bool dups, const BlockEntry *table, const unsigned long long *mask_p, int *nbr) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const unsigned long long mask = *mask_p;
+  int p[SCN_MAXD], j[SCN_MAXD], tap[SCN_MAXD];
+  int b;
+  site_of_key(gi, pos_keys[t], p, b);
+  const bool shadowed = dups && t + 1 < n && pos_keys[t + 1] == pos_keys[t];
+  for (int d = 0; d < f.dim; d++) tap[d] = 0;
+  unsigned long long last_bkey = SCN_EMPTY_KEY, last_bits = 0ull;
+  int last_base = 0;
+  for (int k = 0; k < f.K; k++) {
+    bool ok = !shadowed;
+    for (int d = 0; d < f.dim; d++) {
+      const int num = p[d] - tap[d];
+      j[d] = num / f.stride[d];
+      ok = ok && num >= 0 && num % f.stride[d] == 0 && j[d] < f.out_size[d];
+    }
+    int r = -1;
+    if (ok) {
+      const unsigned long long key = site_key(go, j, b);
+      if ((key >> 6) != last_bkey) {
+        last_bkey = key >> 6;
+        block_lookup(table, mask, last_bkey, last_bits, last_base);
+      }
+      const unsigned long long bit = 1ull << (key & 63);
+      if (last_bits & bit) r = last_base + __popcll(last_bits & (bit - 1ull));
+    }
+    nbr[(int64_t)k * npad + t] = r;
+    for (int d = f.dim - 1; d >= 0; d--) {  // next tap, last dimension fastest
+      if (++tap[d] < f.size[d]) break;
+      tap[d] = 0;
+    }
+  }
+}
+
+// false: more blocks than the path takes; nothing of it is left behind but LO's buffers.
+static bool rules_by_lookup(Metadata &m, StridedRules &R, const Filt &f, const Geom &go, Level &LI, Level &LO, int batch,
+                            hipStream_t s) {
+  const int64_t n = LI.n;
+  ensure_grid(m, LI, s);  // also leaves the positions' keys
+  LO.table.reserve(OB_CAP);
+  LO.gridp.reserve(2);
+  m.ob_words.reserve(4);
+  m.ob_list.reserve((size_t)OB_MAX * sizeof(ObBlock) / sizeof(int));
+  ObBlock *list = reinterpret_cast<ObBlock *>(m.ob_list.p);
+  m.ob_part.reserve((size_t)OB_PARTS * OB_MAX);
+  start_counts(R.by_out, s, false);
+  k_ob_clear<<<dim3(OB_CAP / TB), TB, 0, s>>>(LO.table.p, LO.gridp.p, m.ob_words.p, reinterpret_cast<uint32_t *>(R.by_out.cnt->dev.p),
+                                              2 * COUNT_SLOTS * std::max(f.K, 1));
+  LAUNCH_CHECK();
+  k_ob_mark<<<grid_for(n), TB, 0, s>>>(LI.g, go, f, LI.skeys.p, n, LI.dups, LO.table.p, m.ob_words.p);
+  LAUNCH_CHECK();
+  k_ob_list<<<dim3(OB_CAP / TB), TB, 0, s>>>(LO.table.p, list, m.ob_words.p);
+  LAUNCH_CHECK();
+  k_ob_rank<<<dim3(OB_MAX / 256, OB_PARTS), 256, 0, s>>>(list, m.ob_part.p, m.ob_words.p);
+  LAUNCH_CHECK();
+  const int *w = fetch_words(m, m.ob_words.p, 4, s);
+  if (w[1]) return false;
+  const int nb = w[0];
+  const int64_t n_out = w[2];
+  alloc_level(LO, go, n_out, batch);
+  LO.skeys.reserve(n_out + 1);
+  if (nb) {
+    k_ob_sites<<<dim3((unsigned)ceil_div(nb, 4)), 256, 0, s>>>(go, LO.table.p, list, m.ob_part.p, nb, LO.npad, LO.coords.p, LO.keys.p,
+                                                             LO.skeys.p);
+    LAUNCH_CHECK();
+  }
+  LO.grid_built = true;
+  LO.skeys_ready = n_out > 0;
+  LO.gen = ++m.level_gen;
+  R.out_gen = LO.gen;
+  R.by_out.n = n_out;
+  R.by_out.npad = LO.npad;
+  R.by_in.n = n;
+  R.by_in.npad = LI.npad;
+  R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
+  R.by_in_lookup = true;
+  if (n_out == 0) {
+    R.by_out.identity_rows = true;
+    return true;
+  }
+  unsigned long long *counts = reinterpret_cast<unsigned long long *>(R.by_out.cnt->dev.p);
+  bool s3 = f.dim == 2 || f.dim == 3;
+  for (int d = 0; d < f.dim; d++) s3 = s3 && f.size[d] == 3 && f.stride[d] == 2;
+  if (s3) {
+    int key_bits = 0;
+    const PatternKey pk = pattern_plan(n_out, f.K, key_bits);
+    reserve_pattern_buffers(m, R.by_out);
+    unsigned *masks = reinterpret_cast<unsigned *>(m.f1.p);
+    const int roww = S3_ROW_INTS(f.dim);
+    m.rowtab.reserve((size_t)LO.npad * roww);
+    const dim3 grid((unsigned)(8 * ceil_div(ceil_div(n_out, 64), 8)));
+    if (f.dim == 3)
+      k_subm_rules_s3<3, true><<<grid, 192, 0, s>>>(LI.g, go.bits, LO.skeys.p, n_out, LO.npad, LI.table.p, LI.gridp.p, LI.urow_ptr(),
+                                                   m.rowtab.p, counts, pk, m.k0.p, m.v0.p, masks, false);
+    else
+      k_subm_rules_s3<2, true><<<grid, 192, 0, s>>>(LI.g, go.bits, LO.skeys.p, n_out, LO.npad, LI.table.p, LI.gridp.p, LI.urow_ptr(),
+                                                   m.rowtab.p, counts, pk, m.k0.p, m.v0.p, masks, false);
+    LAUNCH_CHECK();
+    finalize_table(m, R.by_out, nullptr, s, true, m.rowtab.p, roww);
+    return true;
+  }
+  R.by_out.nbr.reserve((size_t)f.K * LO.npad);
+  const int parts = (f.dim >= 2 && f.size[0] <= 4) ? f.size[0] : 1;
+  k_subm_rules<<<grid_for(n_out, 64), 64 * parts, f.K * sizeof(int), s>>>(LI.g, f, LO.coords.p, nullptr, n_out, LO.npad, LI.table.p,
+                                                                        LI.gridp.p, LI.urow_ptr(), R.by_out.nbr.p, counts, parts,
+                                                                        nullptr);
+  LAUNCH_CHECK();
+  finalize_table(m, R.by_out, nullptr, s);
+  return true;
+}
+// A level about to be replaced: the rulebooks that would still look its sites up do it now.
+static void settle_lookups(Metadata &m, const SizeKey &size, hipStream_t s) {
+  for (auto &e : m.strided)
+    if (e.second.by_in_lookup && e.second.out_size == size) finish_by_in(m, e.second, s);
+}
+
 StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *out_size,
                             const int64_t *filter, const int64_t *stride, hipStream_t s) {
   SizeKey key = mk(m.dim, in_size, filter, stride);
@@ -1789,7 +2133,10 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   // Building a strided rulebook replaces the output level (Metadata/ConvolutionRules.h:68-70)
   // and whatever was cached for it.
   // Feature passes enqueued earlier may still be reading what is dropped here.
-  if (m.levels.count(R.out_size)) wait_for_consumers(m, s);
+  if (m.levels.count(R.out_size)) {
+    wait_for_consumers(m, s);
+    settle_lookups(m, R.out_size, s);
+  }
   for (auto i = m.subm.begin(); i != m.subm.end();)
     i = std::equal(R.out_size.begin(), R.out_size.end(), i->first.begin()) ? m.subm.erase(i) : std::next(i);
   Level &LO = m.levels[R.out_size];
@@ -1866,6 +2213,15 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
     finalize_table(m, R.by_out, nullptr, s, true);
     return m.strided.emplace(key, std::move(R)).first->second;
+  }
+  if (m.dim <= 3 && f.M > 1 && f.M <= OB_MAX_M && n <= OB_MAX_SITES) {
+    R.filter.assign(filter, filter + m.dim);
+    R.stride.assign(stride, stride + m.dim);
+    if (rules_by_lookup(m, R, f, go, LI, LO, batch, s)) return m.strided.emplace(key, std::move(R)).first->second;
+    LO = Level();  // too many blocks of output sites for that path (scattered points): the general one
+    LO.identity_sched = true;
+    zero_counts(R.by_out);
+    R.by_in.cnt = R.by_out.cnt;
   }
   m.k0.reserve(nc);
   m.k1.reserve(nc);
@@ -1977,6 +2333,21 @@ void finish_by_in(Metadata &m, StridedRules &r, hipStream_t s) {
     r.by_in_compact = false;
     r.by_in_final = true;
     return;
+  }
+  if (r.by_in_lookup) {
+    auto lo = m.levels.find(r.out_size);
+    if (lo == m.levels.end() || lo->second.gen != r.out_gen)
+      throw Error("strided rules: the coarse level was rebuilt before the fine-side table was made");
+    Level &LI = li->second, &LO = lo->second;
+    t.nbr.reserve((size_t)t.K * t.npad);
+    if (t.n > 0) {
+      ensure_grid(m, LI, s);  // the positions' keys (the table itself was needed to build the rulebook)
+      const Filt f = make_filt(m.dim, r.filter.data(), r.stride.data(), r.out_size.data());
+      k_rules_from_fine<<<grid_for(t.n), TB, 0, s>>>(LI.g, LO.g, f, LI.skeys.p, t.n, t.npad, LI.dups, LO.table.p, LO.gridp.p,
+                                                   t.nbr.p);
+      LAUNCH_CHECK();
+    }
+    r.by_in_lookup = false;
   }
   finalize_table(m, r.by_in, li->second.sched_ptr(), s);
   r.by_in_final = true;

@@ -26,7 +26,7 @@
 namespace scn {
 
 typedef unsigned long long u64;
-constexpr int RS_THREADS = 256, RS_WAVES = 4;  // a tile is RS_THREADS * ITEMS pairs: 4096 (large inputs) or 2048
+constexpr int RS_THREADS = 256, RS_WAVES = 4;  // a tile is RS_THREADS * ITEMS pairs: 4096 (large inputs) down to 512
 constexpr int RS_MAX_BITS = 10, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured on a million
 // pairs of 35 bits: four digits of 9 bits beat three of 11 and five of 7; 40 bits sort in four digits of 10)
 
@@ -315,9 +315,10 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
   }
   // Large inputs take tiles of 4096 pairs (longer runs per digit value in the scatter's stores: a
   // million pairs of 35 bits 145 -> 122 us, eight million 800 -> 490 us); below half a million pairs
-  // there are too few of those to fill the chip and 2048-pair tiles are faster.
-  const bool big = n >= 500000;
-  const int tile = RS_THREADS * (big ? 16 : 8);
+  // there are too few of those to fill the chip and smaller tiles are faster, down to 512 pairs
+  // (30 bits: 88 000 pairs 64 -> 55 us, 15 000 pairs 60 -> 44 us, 150 000 pairs 72 -> 61 us with 1024).
+  const int items = n >= 500000 ? 16 : n >= 300000 ? 8 : n >= 120000 ? 4 : 2;
+  const int tile = RS_THREADS * items;
   const int tiles = (int)ceil_div(n, tile);
   // scratch: a second pair of arrays (when there is more than one pass), the tile counts, the totals
   const size_t kbytes = round_up((size_t)n * sizeof(u64), 256), vbytes = round_up((size_t)n * sizeof(int), 256);
@@ -340,14 +341,24 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
     u64 *kdst = to_out ? kout : ktmp;
     int *vdst = to_out ? vout : vtmp;
     const int shift = width * pass, bits = std::min(width, end_bit - shift);
-    if (big) k_rs_hist<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);
-    else k_rs_hist<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);
-    LAUNCH_CHECK();
-    k_rs_colscan<<<dim3(1 << bits), 64, 0, s>>>(hist, tiles, tot);
-    LAUNCH_CHECK();
-    if (big) k_rs_scatter<16><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot, n_dev);
-    else k_rs_scatter<8><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot, n_dev);
-    LAUNCH_CHECK();
+    switch (items) {
+#define RS_PASS(I)                                                                                                  \
+  case I:                                                                                                           \
+    k_rs_hist<I><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);                      \
+    LAUNCH_CHECK();                                                                                                 \
+    k_rs_colscan<<<dim3(1 << bits), 64, 0, s>>>(hist, tiles, tot);                                                  \
+    LAUNCH_CHECK();                                                                                                 \
+    k_rs_scatter<I><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, vsrc, kdst, vdst, n, shift, bits, tiles, hist, tot, n_dev); \
+    LAUNCH_CHECK();                                                                                                 \
+    break;
+      RS_PASS(16)
+      RS_PASS(8)
+      RS_PASS(4)
+      RS_PASS(2)
+#undef RS_PASS
+    default:
+      throw Error("sort: internal tile size");
+    }
     ksrc = kdst;
     vsrc = vdst;
   }

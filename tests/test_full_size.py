@@ -131,6 +131,39 @@ def _canon(rules, loc_in, in_size, loc_out, out_size):
     return t[order], a[order], b[order]
 
 
+@pytest.mark.parametrize("n,spatial", [(60000, 2047), (60000, 255), (3000, 2047)])
+def test_rulebook_3s2_of_scattered_and_of_dense_points(n, spatial):
+    """A 3^3 / stride-2 rulebook of points scattered over a large grid (nearly every output site in a
+    64-key block of its own: more blocks than the builder that finds the output sites block by
+    block takes, so the candidate sort builds it), of the same number packed into a small grid
+    (few, full blocks) and of a small scattered set: both levels' sites and both tables bit-exact
+    against numpy, the fine-side table through the transposed rulebook's pooling."""
+    from hip_path import HipPath
+    g = HipPath(3)
+    rng = np.random.default_rng(n + spatial)
+    coords = np.unique(np.concatenate([rng.integers(0, spatial, (n, 3)), rng.integers(0, 2, (n, 1))], 1), axis=0)
+    coords = coords[rng.permutation(len(coords))].astype(np.int64)
+    assert g.input_layer(spatial, coords, 0, 4) == len(coords)
+    loc = g.spatial_locations(spatial)
+    out = (spatial - 3) // 2 + 1
+    rules = g.strided_rules(spatial, out, 3, 2)
+    lo = g.spatial_locations(out)
+    t, a, b, sites = _strided_sets(loc, spatial, 3, 2, out)
+    assert (np.sort(_lin(lo, out)) == sites).all()
+    assert (np.diff(lo[:, -1]) >= 0).all()
+    order = np.lexsort((b, a, t))
+    got = _canon(rules, loc, spatial, lo, out)
+    for u, v in zip(got, (t[order], a[order], b[order])):
+        assert u.shape == v.shape and (u == v).all()
+    # the fine-side table: unpooling adds, into every fine row, the coarse rows of its rules
+    y = rng.integers(-8, 8, (len(lo), 4)).astype(np.float32)  # small integers: sums exact in fp32
+    up = g.unpool(out, spatial, 3, 2, y)
+    want = np.zeros((len(loc), 4), np.float32)
+    for r in rules:
+        np.add.at(want, r[:, 0], y[r[:, 1]])
+    assert (up == want).all()
+
+
 def test_strided_tree_at_1m_sites():
     """Configuration 4 at its full size: 1 M sites in 4094^3, Convolution 2^3/2 32 -> 64, then
     MaxPooling(3, 2) and Deconvolution 2^3/2 64 -> 32 + BatchNormReLU from the same coarse level.
