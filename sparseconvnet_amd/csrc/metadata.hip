@@ -672,9 +672,11 @@ __global__ void k_block_heads(const unsigned long long *ukey, int64_t n, const i
 }
 // Empties the part of the table that will be used and records its mask (capacity - 1) for the
 // kernels that follow.  ticket[1]: the number of blocks, as the head kernel in front left it.
+// zero (optional): words the caller wants cleared in the same launch (a rulebook's counters).
 __global__ void k_block_clear(BlockEntry *table, int64_t cap_alloc, const unsigned long long *ticket,
-                              unsigned long long *mask_out) {
+                              unsigned long long *mask_out, uint32_t *zero, int zero_words) {
   int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (int64_t i = b; i < zero_words; i += (int64_t)gridDim.x * blockDim.x) zero[i] = 0u;
   const unsigned long long cap = grid_capacity((long long)ticket[1], cap_alloc);
   if (b == 0) *mask_out = cap - 1;
   if (b < cap_alloc && (unsigned long long)b < cap) {
@@ -730,8 +732,9 @@ static const unsigned long long *position_keys(Level &L, hipStream_t s) {
   return L.skeys.p;
 }
 
-static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
-  if (L.grid_built) return;
+// zero / zero_words: see k_block_clear; false when the table was there already and nothing was cleared.
+static bool ensure_grid(Metadata &m, Level &L, hipStream_t s, void *zero = nullptr, int zero_words = 0) {
+  if (L.grid_built) return false;
   const int64_t n = L.n;
   L.skeys.reserve(n + 1);
   m.k1.reserve(n + 1);
@@ -771,7 +774,8 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   } else {
     fill32(ticket + 1, 0, 2, s);  // no sites: no blocks
   }
-  k_block_clear<<<grid_for((int64_t)cap_alloc), TB, 0, s>>>(L.table.p, (int64_t)cap_alloc, ticket, L.gridp.p);
+  k_block_clear<<<grid_for((int64_t)cap_alloc), TB, 0, s>>>(L.table.p, (int64_t)cap_alloc, ticket, L.gridp.p,
+                                                            static_cast<uint32_t *>(zero), zero_words);
   LAUNCH_CHECK();
   if (n) {
     k_block_insert<<<grid_for(n), TB, 0, s>>>(ukey, m.f0.p, n, n_sites_dev, L.table.p, L.gridp.p);
@@ -779,6 +783,7 @@ static void ensure_grid(Metadata &m, Level &L, hipStream_t s) {
   }
   L.grid_built = true;
   L.skeys_ready = n > 0;
+  return true;
 }
 
 // ---- submanifold rules -----------------------------------------------------------------
@@ -1420,10 +1425,12 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
     return m.subm.emplace(key, std::move(t)).first->second;
   }
   Level &L = lit->second;
-  ensure_grid(m, L, s);
   t.n = L.n;
   t.npad = L.npad;
-  start_counts(t, s);
+  // the counters are cleared by the launch that clears the level's block table, when this call builds it
+  start_counts(t, s, false);
+  const int64_t count_words = 2 * (int64_t)COUNT_SLOTS * std::max(t.K, 1);
+  if (!ensure_grid(m, L, s, t.cnt->dev.p, (int)count_words)) fill32(t.cnt->dev.p, 0, count_words, s);
   bool all3 = true;
   for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
   if (all3 && (m.dim == 2 || m.dim == 3) && t.n > 0) {

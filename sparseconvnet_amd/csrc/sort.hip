@@ -30,24 +30,29 @@ constexpr int RS_THREADS = 256, RS_WAVES = 4;  // a tile is RS_THREADS * ITEMS p
 constexpr int RS_MAX_BITS = 10, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured on a million
 // pairs of 35 bits: four digits of 9 bits beat three of 11 and five of 7; 40 bits sort in four digits of 10)
 
+// The tile's digit counts.  Four times the scatter kernel's threads per tile (the same tiles): the
+// kernel is a read of the keys and a few LDS atomics per thread, and one 256-thread workgroup per
+// compute unit leaves most of the memory system idle (a million pairs: 9.3 -> 5 us per pass).
 template <int RS_ITEMS>
-__global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const u64 *__restrict__ keys, int64_t n, int shift, int bits,
-                                                        int tiles, int *__restrict__ hist, const int *__restrict__ n_dev) {
+__global__ __launch_bounds__(RS_THREADS *(RS_ITEMS >= 4 ? 4 : RS_ITEMS)) void k_rs_hist(
+    const u64 *__restrict__ keys, int64_t n, int shift, int bits, int tiles, int *__restrict__ hist,
+    const int *__restrict__ n_dev) {
+  constexpr int THREADS = RS_THREADS * (RS_ITEMS >= 4 ? 4 : RS_ITEMS), PER = RS_THREADS * RS_ITEMS / THREADS;
   __shared__ int h[RS_MAX_BINS];
   if (n_dev) n = *n_dev;  // the number of pairs when only the device knows it (n: an upper bound the grid was sized for)
   const int bins = 1 << bits;
-  for (int d = threadIdx.x; d < bins; d += RS_THREADS) h[d] = 0;
+  for (int d = threadIdx.x; d < bins; d += THREADS) h[d] = 0;
   __syncthreads();
   const unsigned mask = (unsigned)bins - 1u;
   constexpr int RS_TILE = RS_THREADS * RS_ITEMS;
   const int64_t base = (int64_t)blockIdx.x * RS_TILE;
 #pragma unroll
-  for (int r = 0; r < RS_ITEMS; r++) {
-    const int64_t i = base + r * RS_THREADS + threadIdx.x;
+  for (int r = 0; r < PER; r++) {
+    const int64_t i = base + r * THREADS + threadIdx.x;
     if (i < n) atomicAdd(&h[(unsigned)(keys[i] >> shift) & mask], 1);
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < bins; d += RS_THREADS) hist[(size_t)d * tiles + blockIdx.x] = h[d];
+  for (int d = threadIdx.x; d < bins; d += THREADS) hist[(size_t)d * tiles + blockIdx.x] = h[d];
 }
 
 // One workgroup (64 threads) per digit value: hist[d][*] becomes its exclusive prefix over tiles,
@@ -344,7 +349,7 @@ void radix_sort_pairs(Metadata &m, const u64 *kin, u64 *kout, const int *vin, in
     switch (items) {
 #define RS_PASS(I)                                                                                                  \
   case I:                                                                                                           \
-    k_rs_hist<I><<<dim3(tiles), RS_THREADS, 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);                      \
+    k_rs_hist<I><<<dim3(tiles), RS_THREADS *(I >= 4 ? 4 : I), 0, s>>>(ksrc, n, shift, bits, tiles, hist, n_dev);    \
     LAUNCH_CHECK();                                                                                                 \
     k_rs_colscan<<<dim3(1 << bits), 64, 0, s>>>(hist, tiles, tot);                                                  \
     LAUNCH_CHECK();                                                                                                 \
