@@ -14,6 +14,7 @@
 #include <cstring>
 
 #include <rocprim/rocprim.hpp>
+#include "sort_block.h"
 
 #include <algorithm>
 
@@ -930,9 +931,29 @@ __device__ inline unsigned mask_rank(unsigned mask, int K) {
     if (mask >> i & 1u) r += c_binom.v[i][__popc(mask & ((2u << i) - 1u))];
   return r;
 }
+// The same with the number of taps known to the compiler: every table read is issued before the
+// first is waited for (the loop above waits for one after the other, which a kernel with few
+// wavefronts to switch to pays in full).
+template <int K> __device__ inline unsigned mask_rank_fixed(unsigned mask) {
+  unsigned r = c_binom.above[K][__popc(mask)];
+#pragma unroll
+  for (int i = 0; i < K; i++) {
+    const unsigned term = c_binom.v[i][__popc(mask & ((2u << i) - 1u))];  // read whether the bit is set or not
+    r += (mask >> i & 1u) ? term : 0u;
+  }
+  return r;
+}
+// window_of: t / window without the 64-bit division (there are at most PATTERN_WINDOWS windows).
+__device__ inline unsigned window_of(int64_t t, int64_t window) {
+  unsigned w = 0;
+#pragma unroll
+  for (int i = 1; i < PATTERN_WINDOWS; i++) w += t >= i * window ? 1u : 0u;
+  return w;
+}
+template <int KC = 0>
 __device__ inline unsigned long long pattern_key(const PatternKey &p, int64_t t, unsigned long long mask) {
-  unsigned long long hi = (unsigned long long)(t / p.window);
-  if (p.ranked) return (hi << p.code_bits) | mask_rank((unsigned)mask, p.K);
+  unsigned long long hi = window_of(t, p.window);
+  if (p.ranked) return (hi << p.code_bits) | (KC > 0 ? mask_rank_fixed<(KC > 0 ? KC : 1)>((unsigned)mask) : mask_rank((unsigned)mask, p.K));
   if (p.pc_bits) hi = (hi << p.pc_bits) | (unsigned long long)((p.K - __popcll(mask)) >> p.pc_shift);
   const unsigned long long code = p.code_bits < p.K ? (mask * 0x9E3779B97F4A7C15ull) >> (64 - p.code_bits) : mask;
   return (hi << p.code_bits) | code;
@@ -1295,10 +1316,126 @@ __global__ void k_subm_rules_s3(Geom g, int pos_bits, const unsigned long long *
   // what the pattern sort of finalize_table starts from (k_table_masks would re-read the table for it)
   if (threadIdx.x < 64 && live) {
     const unsigned mk = lmask[threadIdx.x];
-    pkeys[t] = pattern_key(pk, t, mk);
+    pkeys[t] = pattern_key<K>(pk, t, mk);
     pidx[t] = (int)t;
     pmasks[t] = mk;
   }
+}
+
+// The same rulebook for levels of up to 1024 sites (the deep levels of a network: what their
+// rulebooks cost is launches, six of them on the path above), whole in one launch of one workgroup:
+// the sites' keys go into a hash table in LDS (no block table is built), thread t looks the 3^d
+// neighbours of position t up there, the positions are sorted by tap pattern (block_sort) and every
+// thread writes its column of the finished table: taps, output row, granule masks, counts.  The
+// table equals the one finalize_table makes of the same level (same keys, both sorts stable).
+// COUNT (up to 256 sites, 256 threads): no sort either; the place of a position in the pattern order
+// is the number of positions with a smaller key (or the same and in front of it), counted against
+// all of them in LDS, which below a few hundred is faster than the passes of a radix sort.
+constexpr int TINY_MAX = 1024, TINY_SLOTS = 4096, TINY_COUNT_MAX = 256;
+template <int DIM, bool COUNT>
+__global__ __launch_bounds__(COUNT ? TINY_COUNT_MAX : TINY_MAX) void k_subm_tiny(Geom g, const unsigned long long *skeys, const int *sched, int n,
+                                                        int64_t npad, PatternKey pk, int key_bits, int width, int *nbr,
+                                                        int *rowmap, unsigned *gmask, unsigned long long *counts,
+                                                        int count_words) {
+  constexpr int K = DIM == 3 ? 27 : 9;
+  __shared__ unsigned long long hkey[TINY_SLOTS];
+  __shared__ short hpos[TINY_SLOTS];
+  __shared__ int lcount[K];
+  __shared__ unsigned lg[TINY_MAX / 16];
+  constexpr int THREADS = COUNT ? TINY_COUNT_MAX : TINY_MAX;
+  const int t = threadIdx.x, lane = t & 63;
+  const bool live = t < n;
+  for (int i = t; i < TINY_SLOTS; i += THREADS) hkey[i] = SCN_EMPTY_KEY;
+  if (t < K) lcount[t] = 0;
+  if (t < TINY_MAX / 16) lg[t] = 0u;
+  for (int i = t; i < count_words; i += THREADS) counts[i] = 0ull;  // every copy of the counters; copy 0 gets the counts below
+  __syncthreads();
+  const unsigned long long skey = live ? skeys[t] : 0ull;
+  auto slot_of = [](unsigned long long key) { return (unsigned)((key * 0x9E3779B97F4A7C15ull) >> 40) & (TINY_SLOTS - 1); };
+  if (live) {  // the keys of a level without repeated points are distinct
+    unsigned h = slot_of(skey);
+    while (atomicCAS(&hkey[h], SCN_EMPTY_KEY, skey) != SCN_EMPTY_KEY) h = (h + 1) & (TINY_SLOTS - 1);
+    hpos[h] = (short)t;
+  }
+  __syncthreads();
+  int v[K];
+  unsigned mask = 0;
+  {
+    unsigned long long sp[DIM][3];
+    bool okc[DIM][3];
+#pragma unroll
+    for (int d = 0; d < DIM; d++) {
+      const int c = DIM == 3 ? (int)compact3(skey >> (DIM - 1 - d)) & ((1 << g.bits) - 1)
+                             : (int)compact2(skey >> (DIM - 1 - d)) & ((1 << g.bits) - 1);
+#pragma unroll
+      for (int o = 0; o < 3; o++) {
+        const int q = c + o - 1;
+        okc[d][o] = q >= 0 && q < g.size[d];
+        sp[d][o] = (DIM == 3 ? spread3((unsigned)q) : spread2((unsigned)q)) << (DIM - 1 - d);
+      }
+    }
+    const unsigned long long bpart = (skey >> (DIM * g.bits)) << (DIM * g.bits);
+#pragma unroll
+    for (int k = 0; k < K; k++) {  // taps enumerate the box with the last dimension fastest
+      const int o0 = DIM == 3 ? k / 9 : k / 3, o1 = DIM == 3 ? (k / 3) % 3 : k % 3, o2 = k % 3;
+      bool inside = live && okc[0][o0] && okc[1][o1];
+      unsigned long long key = bpart | sp[0][o0] | sp[1][o1];
+      if (DIM == 3) {
+        inside = inside && okc[DIM - 1][o2];
+        key |= sp[DIM - 1][o2];
+      }
+      int j = -1;
+      if (inside) {
+        unsigned h = slot_of(key);
+        for (;;) {
+          const unsigned long long at = hkey[h];
+          if (at == key) {
+            j = hpos[h];
+            break;
+          }
+          if (at == SCN_EMPTY_KEY) break;
+          h = (h + 1) & (TINY_SLOTS - 1);
+        }
+      }
+      v[k] = j < 0 ? -1 : (sched ? sched[j] : j);
+      if (j >= 0) mask |= 1u << k;
+      const unsigned long long hits = __ballot(j >= 0);
+      if (lane == 0 && hits) atomicAdd(&lcount[k], __popcll(hits));
+    }
+  }
+  unsigned long long key[1] = {live ? pattern_key<K>(pk, t, mask) : 0ull};
+  int P = t;  // the position of site t in the table; threads n .. npad - 1 fill the padding
+  if constexpr (COUNT) {
+    __shared__ unsigned long long ckey[TINY_COUNT_MAX];
+    ckey[t] = key[0];
+    __syncthreads();
+    int before = 0;
+    for (int j = 0; j < n; j++) {
+      const unsigned long long kj = ckey[j];
+      before += (kj < key[0] || (kj == key[0] && j < t)) ? 1 : 0;
+    }
+    if (live) P = before;
+  } else {
+    __shared__ short pos_of[TINY_MAX];
+    __shared__ BlockSort<1> sh;
+    int val[1] = {t};
+    const bool valid[1] = {live};
+    block_sort<1>(sh, key, val, valid, key_bits, width);
+    if (live) pos_of[sh.sval[t]] = (short)t;  // position t of the table holds the site sh.sval[t]
+    __syncthreads();
+    if (live) P = pos_of[t];
+  }
+  if (t < npad) {
+#pragma unroll
+    for (int k = 0; k < K; k++) nbr[(int64_t)k * npad + P] = live ? v[k] : -1;
+  }
+  if (live) {
+    rowmap[P] = sched ? sched[t] : t;
+    atomicOr(&lg[P >> 4], mask);
+  }
+  __syncthreads();
+  if (t < (n + 15) / 16) gmask[t] = lg[t];
+  if (t < K) counts[t] = (unsigned long long)lcount[t];
 }
 
 static Filt make_filt(int dim, const int64_t *size, const int64_t *stride, const int64_t *out_size) {
@@ -1427,12 +1564,37 @@ Table &submanifold_rules(Metadata &m, const int64_t *spatial, const int64_t *fil
   Level &L = lit->second;
   t.n = L.n;
   t.npad = L.npad;
+  bool all3 = true;
+  for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
+  if (all3 && (m.dim == 2 || m.dim == 3) && t.n <= TINY_MAX && !L.dups) {
+    start_counts(t, s, false);
+    int key_bits = 0;
+    const PatternKey pk = pattern_plan(t.n, t.K, key_bits);
+    const int passes = (key_bits + RS1_BITS - 1) / RS1_BITS, width = (key_bits + passes - 1) / passes;
+    t.spread = pk.window >= t.n;
+    t.nbr.reserve((size_t)t.K * t.npad);
+    t.rowmap.reserve(t.npad);
+    t.gmask.reserve(ceil_div(t.n, 16));
+    const unsigned long long *keys = L.identity_sched ? L.keys.p : position_keys(L, s);
+    unsigned long long *counts = reinterpret_cast<unsigned long long *>(t.cnt->dev.p);
+    const int count_words = COUNT_SLOTS * t.K;
+#define TINY_LAUNCH(D, C, T)                                                                                           \
+  k_subm_tiny<D, C><<<dim3(1), T, 0, s>>>(L.g, keys, L.sched_ptr(), (int)t.n, t.npad, pk, key_bits, width, t.nbr.p,     \
+                                         t.rowmap.p, t.gmask.p, counts, count_words)
+    const bool few = t.n <= TINY_COUNT_MAX;
+    if (m.dim == 3 && few) TINY_LAUNCH(3, true, TINY_COUNT_MAX);
+    else if (m.dim == 3) TINY_LAUNCH(3, false, TINY_MAX);
+    else if (few) TINY_LAUNCH(2, true, TINY_COUNT_MAX);
+    else TINY_LAUNCH(2, false, TINY_MAX);
+#undef TINY_LAUNCH
+    LAUNCH_CHECK();
+    t.identity_rows = false;
+    return m.subm.emplace(key, std::move(t)).first->second;
+  }
   // the counters are cleared by the launch that clears the level's block table, when this call builds it
   start_counts(t, s, false);
   const int64_t count_words = 2 * (int64_t)COUNT_SLOTS * std::max(t.K, 1);
   if (!ensure_grid(m, L, s, t.cnt->dev.p, (int)count_words)) fill32(t.cnt->dev.p, 0, count_words, s);
-  bool all3 = true;
-  for (int d = 0; d < m.dim; d++) all3 = all3 && f.size[d] == 3;
   if (all3 && (m.dim == 2 || m.dim == 3) && t.n > 0) {
     int key_bits = 0;
     const PatternKey pk = pattern_plan(t.n, t.K, key_bits);
@@ -1787,6 +1949,86 @@ __global__ __launch_bounds__(HB) void k_halve_emit(Geom gi, Geom go, bool shift,
   __syncthreads();
   unsigned long long *slot = counts + (size_t)(blockIdx.x & (COUNT_SLOTS - 1)) * K;
   if (threadIdx.x < K && lcount[threadIdx.x]) atomicAdd(&slot[threadIdx.x], (unsigned long long)lcount[threadIdx.x]);
+}
+
+// The same rulebook of a level of up to 1024 sites whose output size is known (a later link of a
+// chain of halvings: the deep levels of a network), whole in one launch of one workgroup instead of
+// four: k_halve_emit's work with the coarse-side table kept in LDS, the output sites' place in the
+// pattern order by counting (as k_subm_tiny does) and the finished table, output rows and granule
+// masks written from there.  zero / zero_words: every copy of the rule counters (copy 0 gets the counts).
+constexpr int HALVE_SMALL = 1024;
+__global__ __launch_bounds__(HALVE_SMALL) void k_halve_small(Geom gi, Geom go, bool shift, const unsigned long long *keys,
+                                                             const int *sched, int n, int n_out, int64_t npad_out,
+                                                             int *in_tap, int *in_row, int *out_soa,
+                                                             unsigned long long *out_keys, PatternKey pk, int *nbr,
+                                                             int *rowmap, unsigned *gmask, unsigned long long *counts,
+                                                             int count_words) {
+  const int K = 1 << gi.dim;
+  __shared__ int lb[8][HALVE_SMALL];  // the coarse-side table before the sort: [tap][output site]
+  __shared__ unsigned long long okey[HALVE_SMALL];
+  __shared__ unsigned omask[HALVE_SMALL];
+  __shared__ unsigned lg[HALVE_SMALL / 16];
+  __shared__ int wave_heads[HALVE_SMALL / 64], lcount[8];
+  const int p = threadIdx.x, lane = p & 63, wave = p >> 6;
+  for (int i = p; i < 8 * HALVE_SMALL; i += HALVE_SMALL) (&lb[0][0])[i] = -1;
+  for (int i = p; i < count_words; i += HALVE_SMALL) counts[i] = 0ull;
+  if (p < 8) lcount[p] = 0;
+  if (p < HALVE_SMALL / 16) lg[p] = 0u;
+  const bool live = p < n;
+  int tap = -1;
+  unsigned long long ck = 0;
+  bool head = false;
+  if (live) {
+    ck = parent_key(gi, go, shift, keys[p], &tap);
+    int t2;
+    head = p == 0 || ck != parent_key(gi, go, shift, keys[p - 1], &t2);
+  }
+  const unsigned long long heads = __ballot(head);
+  if (lane == 0) wave_heads[wave] = __popcll(heads);
+  __syncthreads();
+  int o = 0;
+  for (int w = 0; w < wave; w++) o += wave_heads[w];
+  o += __popcll(heads & (~0ull >> (63 - lane))) - 1;  // heads at or before this lane, less one
+  if (live) {
+    in_tap[p] = tap;
+    in_row[p] = o;
+    lb[tap][o] = sched ? sched[p] : p;
+    if (head) {
+      unsigned mask = 1u << tap;
+      for (int i = 1; i < K && p + i < n; i++) {
+        int t2;
+        if (parent_key(gi, go, shift, keys[p + i], &t2) != ck) break;
+        mask |= 1u << t2;
+      }
+      int j[SCN_MAXD], b;
+      site_of_key(go, ck, j, b);
+      for (int d = 0; d < gi.dim; d++) out_soa[d * npad_out + o] = j[d];
+      out_soa[gi.dim * npad_out + o] = b;
+      out_keys[o] = ck;
+      okey[o] = pattern_key(pk, o, mask);
+      omask[o] = mask;
+    }
+  }
+  for (int k = 0; k < K; k++) {
+    const unsigned long long bk = __ballot(tap == k);
+    if (lane == 0 && bk) atomicAdd(&lcount[k], __popcll(bk));
+  }
+  __syncthreads();
+  // thread o < n_out: output site o goes to position P of the table
+  if (p < n_out) {
+    const unsigned long long mine = okey[p];
+    int P = 0;
+    for (int j = 0; j < n_out; j++) {
+      const unsigned long long kj = okey[j];
+      P += (kj < mine || (kj == mine && j < p)) ? 1 : 0;
+    }
+    for (int k = 0; k < K; k++) nbr[(int64_t)k * npad_out + P] = lb[k][p];
+    rowmap[P] = p;
+    atomicOr(&lg[P >> 4], omask[p]);
+  }
+  __syncthreads();
+  if (p < (n_out + 15) / 16) gmask[p] = lg[p];
+  if (p < K) counts[p] = (unsigned long long)lcount[p];
 }
 
 // ---- filters larger than their stride, small and middle levels: rules by lookup ----
@@ -2180,6 +2422,34 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
     m.dflags.reserve(16 * 64);
   }
   const bool count = presorted && LI.halvings.empty();
+  if (presorted && !count && n <= HALVE_SMALL && !LI.dups) {  // a small level of known output size: one launch
+    const unsigned long long *keys = LI.identity_sched ? LI.keys.p : position_keys(LI, s);
+    const int64_t n_out = LI.halvings[0];
+    alloc_level(LO, go, n_out, batch);
+    LO.halvings.assign(LI.halvings.begin() + 1, LI.halvings.end());
+    R.by_out.n = n_out;
+    R.by_out.npad = LO.npad;
+    R.by_in.n = n;
+    R.by_in.npad = LI.npad;
+    R.by_out.nbr.reserve((size_t)f.K * LO.npad);
+    R.by_out.rowmap.reserve(LO.npad);
+    R.by_out.gmask.reserve(ceil_div(std::max<int64_t>(n_out, 1), 16));
+    R.by_in_compact = true;
+    R.in_tap.reserve(n);
+    R.in_row.reserve(n);
+    start_counts(R.by_out, s, false);
+    int key_bits = 0;
+    const PatternKey pk = pattern_plan(n_out, f.K, key_bits);
+    R.by_out.spread = pk.window >= n_out;
+    R.by_out.identity_rows = false;
+    k_halve_small<<<dim3(1), HALVE_SMALL, 0, s>>>(LI.g, go, go.bits == LI.g.bits - 1, keys, LI.sched_ptr(), (int)n, (int)n_out,
+                                                 LO.npad, R.in_tap.p, R.in_row.p, LO.coords.p, LO.keys.p, pk, R.by_out.nbr.p,
+                                                 R.by_out.rowmap.p, R.by_out.gmask.p,
+                                                 (unsigned long long *)R.by_out.cnt->dev.p, COUNT_SLOTS * f.K);
+    LAUNCH_CHECK();
+    R.by_in.cnt = R.by_out.cnt;  // both tables list the same rules
+    return m.strided.emplace(key, std::move(R)).first->second;
+  }
   if (presorted) {
     // positions' keys: the level's own when its rows are in schedule order (a level made here)
     const unsigned long long *keys = LI.identity_sched ? LI.keys.p : position_keys(LI, s);

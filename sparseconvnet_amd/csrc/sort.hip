@@ -22,10 +22,10 @@
 // The number of pairs may live on the device only (n_dev): the launches are then sized for an
 // upper bound and tiles past the real end find nothing to do.
 #include "metadata.h"
+#include "sort_block.h"
 
 namespace scn {
 
-typedef unsigned long long u64;
 constexpr int RS_THREADS = 256, RS_WAVES = 4;  // a tile is RS_THREADS * ITEMS pairs: 4096 (large inputs) down to 512
 constexpr int RS_MAX_BITS = 10, RS_MAX_BINS = 1 << RS_MAX_BITS;  // widest digit of the tiled kernels (measured on a million
 // pairs of 35 bits: four digits of 9 bits beat three of 11 and five of 7; 40 bits sort in four digits of 10)
@@ -77,32 +77,6 @@ __global__ __launch_bounds__(64) void k_rs_colscan(int *__restrict__ hist, int t
     run += c;
   }
   if (lane == 63) tot[blockIdx.x] = incl;
-}
-
-// Rank of each of a wavefront's ITEMS x 64 pairs (round r, lane) among the pairs of its quarter
-// with the same digit value, in round-major order; cnt[0 .. 2^bits) (this wavefront's, zero on entry)
-// ends as the quarter's count of every value.
-template <int ITEMS>
-__device__ inline void rank_quarter(const unsigned (&digit)[ITEMS], const bool (&valid)[ITEMS], int bits, int *cnt,
-                                    int lane, int (&rank)[ITEMS]) {
-  const u64 below = (1ull << lane) - 1ull;
-#pragma unroll
-  for (int r = 0; r < ITEMS; r++) {
-    u64 peers = __ballot(valid[r]);
-    if (!peers) {  // a round past the end of the input (the whole wavefront agrees)
-      rank[r] = 0;
-      continue;
-    }
-    for (int b = 0; b < bits; b++) {
-      const u64 has = __ballot((digit[r] >> b) & 1u);
-      peers &= ((digit[r] >> b) & 1u) ? has : ~has;
-    }
-    const int before = __popcll(peers & below);
-    int old = 0;
-    if (valid[r]) old = cnt[digit[r]];  // every lane of the group reads the count before its first lane bumps it
-    if (valid[r] && before == 0) cnt[digit[r]] = old + __popcll(peers);
-    rank[r] = old + before;
-  }
 }
 
 template <int RS_ITEMS>
@@ -213,31 +187,20 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(const u64 *__restrict
   }
 }
 
-// Up to RS1_MAX pairs: one workgroup takes them through every digit without leaving LDS, one
-// launch instead of three per digit (the deep levels of a network are a few hundred to a few
-// thousand sites, and what their rulebooks cost is launches).  Sixteen wavefronts each keep a
-// contiguous 256 pairs in registers and rank them as k_rs_scatter does, with digits of up to 8 bits
-// (the prefix over 16 wavefronts' counts of every digit value is what a pass costs here, so fewer
-// values beat fewer passes); the pairs change places through LDS between digits.
-constexpr int RS1_THREADS = 1024, RS1_WAVES = 16, RS1_ITEMS = 4, RS1_MAX = RS1_THREADS * RS1_ITEMS;
-constexpr int RS1_BITS = 8, RS1_BINS = 1 << RS1_BITS;
+// Up to RS1_MAX pairs: one workgroup takes them through every digit without leaving LDS
+// (sort_block.h), one launch instead of three per digit.
+constexpr int RS1_ITEMS = 4, RS1_MAX = RS1_THREADS * RS1_ITEMS;
 __global__ __launch_bounds__(RS1_THREADS) void k_rs_single(const u64 *__restrict__ kin, const int *__restrict__ vin,
                                                            u64 *__restrict__ kout, int *__restrict__ vout, int n,
                                                            int end_bit, int width, const int *__restrict__ n_dev) {
   constexpr int ITEMS = RS1_ITEMS;
   if (n_dev) n = *n_dev;
-  __shared__ int cnt[RS1_WAVES][RS1_BINS];
-  __shared__ int lstart[RS1_BINS];
-  __shared__ int wsum[RS1_BINS / 64];
-  __shared__ u64 skey[RS1_MAX];
-  __shared__ int sval[RS1_MAX];
+  __shared__ BlockSort<ITEMS> sh;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int q0 = wave * (ITEMS * 64);
   u64 key[ITEMS];
   int val[ITEMS];
-  unsigned digit[ITEMS];
   bool valid[ITEMS];
-  int rank[ITEMS];
 #pragma unroll
   for (int r = 0; r < ITEMS; r++) {
     const int i = q0 + r * 64 + lane;
@@ -245,60 +208,10 @@ __global__ __launch_bounds__(RS1_THREADS) void k_rs_single(const u64 *__restrict
     key[r] = valid[r] ? kin[i] : 0ull;
     val[r] = valid[r] ? vin[i] : 0;
   }
-  for (int shift = 0; shift < end_bit; shift += width) {
-    const int bits = min(width, end_bit - shift), bins = 1 << bits;
-    const unsigned mask = (unsigned)bins - 1u;
-    for (int e = threadIdx.x; e < RS1_WAVES * bins; e += RS1_THREADS) cnt[e / bins][e % bins] = 0;
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < ITEMS; r++) digit[r] = (unsigned)(key[r] >> shift) & mask;
-    rank_quarter<ITEMS>(digit, valid, bits, cnt[wave], lane, rank);
-    __syncthreads();
-    // thread d < bins: the counts of value d become their exclusive prefix over the wavefronts;
-    // then an exclusive scan of the totals over d (the first bins / 64 wavefronts)
-    int total = 0;
-    if (threadIdx.x < bins) {
-      for (int w = 0; w < RS1_WAVES; w++) {
-        const int c = cnt[w][threadIdx.x];
-        cnt[w][threadIdx.x] = total;
-        total += c;
-      }
-    }
-    int incl = total;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int up = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += up;
-    }
-    if (lane == 63 && wave < RS1_BINS / 64) wsum[wave] = incl;
-    __syncthreads();
-    if (threadIdx.x < bins) {
-      int run = incl - total;
-      for (int w = 0; w < wave; w++) run += wsum[w];
-      lstart[threadIdx.x] = run;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < ITEMS; r++) {
-      if (!valid[r]) continue;
-      const int at = lstart[digit[r]] + cnt[wave][digit[r]] + rank[r];
-      skey[at] = key[r];
-      sval[at] = val[r];
-    }
-    __syncthreads();
-    if (shift + width < end_bit) {  // the pairs of this wavefront's range for the next digit
-#pragma unroll
-      for (int r = 0; r < ITEMS; r++) {
-        const int i = q0 + r * 64 + lane;
-        key[r] = valid[r] ? skey[i] : 0ull;
-        val[r] = valid[r] ? sval[i] : 0;
-      }
-      __syncthreads();
-    }
-  }
+  block_sort<ITEMS>(sh, key, val, valid, end_bit, width);
   for (int i = threadIdx.x; i < n; i += RS1_THREADS) {
-    kout[i] = skey[i];
-    vout[i] = sval[i];
+    kout[i] = sh.skey[i];
+    vout[i] = sh.sval[i];
   }
 }
 
