@@ -224,6 +224,7 @@ struct Metadata {
   DevBuf<float> wcols;  // column ranges of a wide layer's weights, one contiguous block per range (conv_forward)
   DevBuf<int> rowtab;  // site-major neighbour table on its way from the rule kernel to the pattern sort's permutation
   DevBuf<int> dflags;
+  DevBuf<int> scan_tiles;  // exclusive_scan: the tiles' sums
   DevBuf<int> ob_words, ob_list, ob_part;  // strided rulebooks by lookup: counters, the coarse level's blocks, partial ranks
   uint64_t level_gen = 0;
   std::function<void()> before_pack;  // work the packing of the running convolution's weights needs first (the column-range path's copy), run at most once

@@ -179,11 +179,92 @@ static void sort_pairs(Metadata &m, const unsigned long long *kin, unsigned long
   HIP_CHECK(rocprim::radix_sort_pairs<RadixAlways>(m.tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u,
                                                    (unsigned)end_bit, s));
 }
-static void exclusive_scan(Metadata &m, const int *in, int *out, int64_t n, hipStream_t s) {
-  size_t bytes = 0;
-  HIP_CHECK(rocprim::exclusive_scan(nullptr, bytes, in, out, 0, (size_t)n, rocprim::plus<int>(), s));
-  m.tmp.reserve(bytes + 16);
-  HIP_CHECK(rocprim::exclusive_scan(m.tmp.p, bytes, in, out, 0, (size_t)n, rocprim::plus<int>(), s));
+// Exclusive prefix sums of one or two int arrays in two launches that wait for nothing (no
+// look-back between workgroups): k_scan_tiles sums every tile of SCAN_TILE elements, k_scan_write
+// adds up the tile sums in front of its tile (a few hundred at most per million elements) and scans
+// the tile's own elements inside the workgroup.  gridDim.y picks the array.
+constexpr int SCAN_THREADS = 1024, SCAN_TILE = 4 * SCAN_THREADS;
+struct ScanJobs {
+  const int *in[2];
+  int *out[2];
+  int64_t n[2];
+  int *tile_sums[2];
+};
+__device__ inline void scan_load(const int *in, int64_t n, int64_t i0, int (&v)[4]) {
+  if (i0 + 4 <= n) {
+    const int4 q = *reinterpret_cast<const int4 *>(in + i0);
+    v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+  } else {
+    for (int i = 0; i < 4; i++) v[i] = i0 + i < n ? in[i0 + i] : 0;
+  }
+}
+__global__ __launch_bounds__(SCAN_THREADS) void k_scan_tiles(ScanJobs j) {
+  const int a = blockIdx.y;
+  const int64_t n = j.n[a], i0 = (int64_t)blockIdx.x * SCAN_TILE + 4 * threadIdx.x;
+  if ((int64_t)blockIdx.x * SCAN_TILE >= n) return;
+  __shared__ int total;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  int v[4];
+  scan_load(j.in[a], n, i0, v);
+  int sum = v[0] + v[1] + v[2] + v[3];
+#pragma unroll
+  for (int o = 32; o; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  if ((threadIdx.x & 63) == 0 && sum) atomicAdd(&total, sum);
+  __syncthreads();
+  if (threadIdx.x == 0) j.tile_sums[a][blockIdx.x] = total;
+}
+__global__ __launch_bounds__(SCAN_THREADS) void k_scan_write(ScanJobs j) {
+  const int a = blockIdx.y;
+  const int64_t n = j.n[a], i0 = (int64_t)blockIdx.x * SCAN_TILE + 4 * threadIdx.x;
+  if ((int64_t)blockIdx.x * SCAN_TILE >= n) return;
+  __shared__ int part[SCAN_THREADS / 64], wave_sum[SCAN_THREADS / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int before = 0;
+  for (int i = threadIdx.x; i < (int)blockIdx.x; i += SCAN_THREADS) before += j.tile_sums[a][i];
+#pragma unroll
+  for (int o = 32; o; o >>= 1) before += __shfl_xor(before, o, 64);
+  int v[4];
+  scan_load(j.in[a], n, i0, v);
+  const int mine = v[0] + v[1] + v[2] + v[3];
+  int incl = mine;  // inclusive prefix over the wavefront's lanes
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  if (lane == 63) wave_sum[wave] = incl;
+  if (lane == 0) part[wave] = before;
+  __syncthreads();
+  int run = incl - mine;
+  for (int w = 0; w < SCAN_THREADS / 64; w++) run += part[w] + (w < wave ? wave_sum[w] : 0);
+  int *out = j.out[a];
+  if (i0 + 4 <= n) {
+    int4 q;
+    q.x = run, q.y = run + v[0], q.z = run + v[0] + v[1], q.w = run + v[0] + v[1] + v[2];
+    *reinterpret_cast<int4 *>(out + i0) = q;
+  } else {
+    for (int i = 0; i < 4 && i0 + i < n; i++) {
+      out[i0 + i] = run;
+      run += v[i];
+    }
+  }
+}
+// in_b == nullptr: one array.  The arrays start at 16-byte boundaries (whole buffers of the pool).
+static void exclusive_scan(Metadata &m, const int *in_a, int *out_a, int64_t n_a, hipStream_t s, const int *in_b = nullptr,
+                           int *out_b = nullptr, int64_t n_b = 0) {
+  const int64_t most = std::max(n_a, n_b);
+  if (most <= 0) return;
+  const int tiles = (int)ceil_div(most, SCAN_TILE);
+  m.scan_tiles.reserve(2 * (size_t)tiles);
+  ScanJobs j;
+  j.in[0] = in_a, j.out[0] = out_a, j.n[0] = n_a, j.tile_sums[0] = m.scan_tiles.p;
+  j.in[1] = in_b, j.out[1] = out_b, j.n[1] = in_b ? n_b : 0, j.tile_sums[1] = m.scan_tiles.p + tiles;
+  const dim3 grid((unsigned)tiles, in_b ? 2 : 1);
+  k_scan_tiles<<<grid, SCAN_THREADS, 0, s>>>(j);
+  LAUNCH_CHECK();
+  k_scan_write<<<grid, SCAN_THREADS, 0, s>>>(j);
+  LAUNCH_CHECK();
 }
 // Copies `words` ints from the device into the handle's pinned words and waits for them: the
 // one host round trip of a construction step.
@@ -463,8 +544,8 @@ void build_input_layer(Metadata &m, const int64_t *spatial, CoordSrc coords, int
   m.s1.reserve(n + 1);  // first_scan
   k_group_heads<<<grid_for(n + 1), TB, 0, s>>>(m.k1.p, m.v1.p, n, nv, m.f0.p, m.f1.p);
   LAUNCH_CHECK();
-  exclusive_scan(m, m.f0.p, m.s0.p, n + 1, s);  // head[n] = 0: the scan's last element is the number of groups
-  exclusive_scan(m, m.f1.p, m.s1.p, n, s);
+  // head[n] = 0: the last element of its scan is the number of groups; both scans in one pair of launches
+  exclusive_scan(m, m.f0.p, m.s0.p, n + 1, s, m.f1.p, m.s1.p, n);
   const int64_t N = fetch_words(m, m.s0.p + n, 1, s)[0];
   alloc_level(L, g, N, batch);
   L.sched.reserve(N);
