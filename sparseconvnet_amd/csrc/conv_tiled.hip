@@ -289,7 +289,8 @@ static bool launch_mfma(Metadata &m, const Table &t, const float *in, float *out
   const int tiles_per_xcd = t.spread ? 0 : (int)ceil_div(n_tiles, 8);  // 0: tile = workgroup index
   // Few tiles: deal the taps of every tile over several workgroups (about two per CU in all).
   int n_split = 1;
-  if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(512, n_tiles));
+  // (three per CU of the 32-row tiles: 768, 1024 and 1536 workgroups measured alike, 512 slower)
+  if (n_tiles < 256) n_split = (int)std::min<int64_t>(t.K, ceil_div(G == 2 ? 768 : 512, n_tiles));
   const int64_t split_stride = (int64_t)n_tiles * G * 16 * NCB * 16;
   float *partial = scratch_partial(m, n_split, split_stride);
   note_kernel(m, BF16 ? "tiled-bf16" : "tiled", {{"ncbw", NCBW}, {"wc", WC}, {"gw", GW}, {"ss", SS}, {"pre", PRE}, {"split", n_split}});
@@ -316,6 +317,18 @@ static bool dispatch_ncb(int ncb, Metadata &m, const Table &t, const float *in, 
   // workgroups to spread (measured: 12-23 % faster at 16 k sites, 10 % at 1 k, 30 % at 250,
   // equal at 4 k, where the tap split halves in exchange).
   if (!narrow && t.n < 30000 && ncb > 8) {
+    // Below 8192 sites (fewer than 256 such tiles: the taps of a tile are dealt over several
+    // workgroups) tiles of 32 rows with slabs of two steps: one workgroup's chain of MFMAs is what
+    // such a launch lasts (152 rows x 224 planes: 81 workgroups of 10 us of MFMAs each on a chip of
+    // 256 CUs), and halving the tile halves it.  Measured per convolution: 3.3 k sites x 160 planes
+    // 68 -> 56 us, 320 -> 160 118 -> 89, 768 x 192 34.5 -> 32, 152 x 224 28.6 -> 22; 12.7 k x 160
+    // (no tap split any more) 171 -> 191, hence the limit.
+    if (t.n < 8192 && n_in % 32 == 0) {
+      if (ncb <= 10) return launch_mfma<5, 2, 1, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      if (ncb <= 12) return launch_mfma<6, 2, 1, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      if (ncb <= 14) return launch_mfma<7, 2, 1, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+      if (ncb <= 16) return launch_mfma<8, 2, 1, 2, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
+    }
     if (ncb <= 10) return launch_mfma<5, 2, 2, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     if (ncb <= 12) return launch_mfma<3, 4, 4, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
     if (ncb <= 14) return launch_mfma<7, 2, 2, 1, VEC4, PRE>(m, t, in, out, w, epi, n_in, n_out, pre, s);
