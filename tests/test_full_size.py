@@ -131,12 +131,13 @@ def _canon(rules, loc_in, in_size, loc_out, out_size):
     return t[order], a[order], b[order]
 
 
-@pytest.mark.parametrize("n,spatial", [(60000, 2047), (60000, 255), (3000, 2047)])
+@pytest.mark.parametrize("n,spatial", [(60000, 2047), (60000, 255), (3000, 2047), (11200, 601), (12200, 601)])
 def test_rulebook_3s2_of_scattered_and_of_dense_points(n, spatial):
     """A 3^3 / stride-2 rulebook of points scattered over a large grid (nearly every output site in a
     64-key block of its own: more blocks than the builder that finds the output sites block by
     block takes, so the candidate sort builds it), of the same number packed into a small grid
-    (few, full blocks) and of a small scattered set: both levels' sites and both tables bit-exact
+    (few, full blocks), of a small scattered set, and of two sets whose output sites fill just under
+    and just over the 16 384 blocks that builder takes: both levels' sites and both tables bit-exact
     against numpy, the fine-side table through the transposed rulebook's pooling."""
     from hip_path import HipPath
     g = HipPath(3)
