@@ -1280,9 +1280,24 @@ __global__ void k_subm_rules_s3(Geom g, int pos_bits, const unsigned long long *
     for (int o = 0; o < 3; o++) {
       const int v = cd[d] + o - 1;
       okc[d][o] = v >= 0 && v < g.size[d];
-      const unsigned long long s = DIM == 3 ? spread3((unsigned)v) : spread2((unsigned)v);
-      sp[d][o] = s << (DIM - 1 - d);
     }
+    // The three coordinates' bits in place in a key of level g, without spreading them: the middle
+    // one's are the position's own (moved up one bit per coordinate and with the low bit set for the
+    // coarse side of a stride-2 filter: 2c + 1), and one more or less is an add or a subtract that
+    // carries across the other coordinates' bit positions (filled with ones for the add; the
+    // subtract borrows through their zeros).  A coordinate that leaves [0, 2^bits) gives a wrong
+    // pattern, and is out of range: okc is false for it.
+    constexpr unsigned long long EVERY = DIM == 3 ? 0x1249249249249249ull : 0x5555555555555555ull;
+    const int sh = DIM - 1 - d;
+    const unsigned long long md = (EVERY & ((1ull << (DIM * g.bits)) - 1ull)) << sh, one = 1ull << sh;
+    unsigned long long mid;
+    if (HALF)
+      mid = ((skey & ((EVERY & ((1ull << (DIM * pos_bits)) - 1ull)) << sh)) << DIM) | one;
+    else
+      mid = skey & md;
+    sp[d][1] = mid;
+    sp[d][0] = HALF ? mid & ~one : (mid - one) & md;
+    sp[d][2] = ((mid | ~md) + one) & md;
   }
   const unsigned long long bpart = (skey >> (DIM * pos_bits)) << (DIM * g.bits);  // the sample index, in its place in level g's keys
   // The lane's taps (first-dimension offset fixed by its wavefront) lie in at most two blocks
