@@ -54,12 +54,15 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   // tiles so that neighbouring tiles (which gather the same rows) share one L2.  Small levels
   // (tiles_per_xcd == 0, Table::spread) list their tiles most expensive first: workgroup i takes
   // tile i, so that the long tiles start first and on different CUs.
+  SCN_PHASE(0);  // start
   const int tile = tiles_per_xcd ? (blockIdx.x & 7) * tiles_per_xcd + (blockIdx.x >> 3) : blockIdx.x;
   if (tile >= n_tiles) return;  // whole workgroup leaves: no barrier is skipped
   const int64_t tbase = (int64_t)tile * TM;
 
   const int ntaps = tile_setup<256, G>(nbr, K, n, npad, tbase, n_split, (int)blockIdx.y, jtab, gmask, taplist, ntaps_p);
   const int total = ntaps * n_slab;
+  SCN_PHASE(1);  // tile set up
+  SCN_PHASE_VALUE(7, total);
   v4f acc[GW][NCBW];
 #pragma unroll
   for (int q = 0; q < GW; q++)
@@ -210,10 +213,13 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
   };
 
   if (total > 0) issue(0, std::integral_constant<int, 0>{});
+  SCN_PHASE(2);  // first loads issued
   for (int it = 0; it < total; it += 2) {
     iterate(it, std::integral_constant<int, 0>{});
+    if (it == 0) SCN_PHASE(3);  // first iteration done
     if (it + 1 < total) iterate(it + 1, std::integral_constant<int, 1>{});
   }
+  SCN_PHASE(4);  // tap loop done
 
   // acc[q][c][r] = result for position tbase + 16*(wr*GW+q) + 4*g + r, column 16*(wc*NCBW+c) + r16
   if (partial != nullptr) {  // [n_split][n_tiles * TM][NCB * 16]
@@ -225,6 +231,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_mfma(
 #pragma unroll
         for (int c = 0; c < NCBW; c++)
           pt[(int64_t)((wr * GW + q) * 16 + 4 * g + r) * (NCB * 16) + 16 * (wc * NCBW + c) + r16] = acc[q][c][r];
+    SCN_PHASE(5);  // partial tile stored
     return;
   }
   float bv[NCBW], es[NCBW], eh[NCBW];
@@ -357,5 +364,7 @@ bool conv_tiled_dispatch(bool vec4, bool pre_fused, Metadata &m, const Table &t,
   return vec4 ? dispatch_ncb<true, false>(ncb, m, t, in, out, w, epi, n_in, n_out, pre, s)
               : dispatch_ncb<false, false>(ncb, m, t, in, out, w, epi, n_in, n_out, pre, s);
 }
+
+SCN_PHASE_EXPORT(scn_dbg_phases_tiled)
 
 }  // namespace scn
