@@ -268,6 +268,7 @@ void launch_conv_reduce(const float *partial, int n_split, int64_t split_stride,
 template <bool PRE>
 static bool conv_mfma_paths(Metadata &m, const Table &t, const float *in, float *out, const float *w,
                             Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s) {
+  if (!PRE && try_few(m, t, in, out, w, epi, n_in, n_out, s)) return true;
   if (!PRE && try_resident(m, t, in, out, w, epi, n_in, n_out, s)) return true;
   const bool vec4 = n_in % 4 == 0 && ((uintptr_t)in % 16 == 0);
   if (n_out <= 128 && t.K <= 1024 && conv_rows_dispatch(vec4, PRE, m, t, in, out, w, epi, n_in, n_out, pre, s)) return true;

@@ -191,6 +191,9 @@ bool conv_tiled_dispatch(bool vec4, bool pre_fused, Metadata &m, const Table &t,
                          const float *w, Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s);
 bool conv_rows_dispatch(bool vec4, bool pre_fused, Metadata &m, const Table &t, const float *in, float *out,
                         const float *w, Epi epi, int n_in, int n_out, PreArgs pre, hipStream_t s);
+// conv_few.hip: transposed convolutions of filter = stride = 2 rulebooks whose weights fit LDS.
+bool try_few(Metadata &m, const Table &t, const float *in, float *out, const float *w, Epi epi, int n_in, int n_out,
+             hipStream_t s);
 bool resident_fits(const Metadata &m, const Table &t, int n_in, int n_out, bool with_bn);
 bool try_resident(Metadata &m, const Table &t, const float *in, float *out, const float *w, Epi epi, int n_in,
                   int n_out, hipStream_t s);

@@ -79,6 +79,10 @@ struct Table {
   DevBuf<int> rowmap;
   DevBuf<unsigned> gmask;  // K <= 32 and pattern-sorted: bit k of gmask[i] = some position of granule i (16 positions) has tap k
   bool identity_rows = false;  // rowmap[t] == t: kernels skip the indirection
+  // Tables with one rule per position (the fine side of a filter = stride = 2 rulebook): that rule
+  // as (tap, row) of every position, in the table's order (few_tap[t] = 255: no rule); null elsewhere.
+  DevBuf<unsigned char> few_tap;
+  DevBuf<int> few_row;
   // The pattern sort ran over all positions at once (small levels): consecutive tiles descend in
   // cost from the first to the last, so kernels deal tiles to workgroups in turn instead of giving
   // each XCD a contiguous range.

@@ -2650,25 +2650,48 @@ StridedRules &strided_rules(Metadata &m, const int64_t *in_size, const int64_t *
   return m.strided.emplace(key, std::move(R)).first->second;
 }
 
-// The fine-side table of a halving rulebook from its compact form.  Sort key of a position: its
-// range of the schedule (as finalize_table's), then its tap (positions without a rule last): the
-// order count-then-mask gives a table whose rows have one tap each, in 4 bits.
-__global__ void k_few_keys(const int *in_tap, int64_t n, int64_t window, unsigned long long *keys, int *idx) {
-  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  const int tap = in_tap[t];
-  keys[t] = ((unsigned long long)(t / window) << 4) | (unsigned long long)(tap < 0 ? 15 : tap);
-  idx[t] = (int)t;
+// The fine-side table of a halving rulebook from its compact form: the positions in tap order
+// (positions without a rule last), which gives a table whose rows have one tap each,
+// inside windows of 1024 ITEMS consecutive schedule positions instead of a few
+// ranges of the level, by one workgroup per window (block_sort, one 5-bit digit: no sort launches).
+// A window's positions share their coarse rows (the 2^dim children of a site are neighbours in
+// the schedule), so the taps' runs of a window, which one XCD works through at about the same
+// time, find a coarse row that one of them fetched still in that XCD's L2; with an eighth of a
+// million-site level per range every tap's run fetched its 4 MB of coarse rows again (counters:
+// 268 MB read for 95 MB of operands).
+template <int ITEMS>
+__global__ __launch_bounds__(RS1_THREADS) void k_few_order(const int *in_tap, int64_t n, int *perm) {
+  __shared__ BlockSort<ITEMS> sh;
+  constexpr int WINDOW = RS1_THREADS * ITEMS;
+  const int64_t base = (int64_t)blockIdx.x * WINDOW;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned long long key[ITEMS];
+  int val[ITEMS];
+  bool valid[ITEMS];
+#pragma unroll
+  for (int r = 0; r < ITEMS; r++) {
+    const int i = wave * (ITEMS * 64) + r * 64 + lane;
+    valid[r] = base + i < n;
+    const int tap = valid[r] ? in_tap[base + i] : 0;
+    key[r] = tap < 0 ? 16ull : (unsigned long long)tap;
+    val[r] = i;
+  }
+  block_sort<ITEMS>(sh, key, val, valid, 5, 5);
+  const int here = (int)min<int64_t>(WINDOW, n - base);
+  for (int i = threadIdx.x; i < here; i += RS1_THREADS) perm[base + i] = (int)(base + sh.sval[i]);
 }
 // Position t of the sorted table is position perm[t] of the schedule: its one entry, -1 in the
 // other taps, its row, and the granule masks (an OR over the 16 lanes of a granule).
 __global__ void k_table_expand_few(const int *in_tap, const int *in_row, int K, int64_t n, int64_t npad, const int *perm,
-                                   const int *base, int *nbr, int *rowmap, unsigned *gmask) {
+                                   const int *base, int *nbr, int *rowmap, unsigned *gmask, unsigned char *few_tap,
+                                   int *few_row) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   unsigned mk = 0;
   if (t < n) {
     const int src = perm[t];
     const int tap = in_tap[src], row = in_row[src];
+    few_tap[t] = tap >= 0 ? (unsigned char)tap : (unsigned char)255;
+    few_row[t] = tap >= 0 ? row : 0;
     for (int k = 0; k < K; k++) nbr[(int64_t)k * npad + t] = k == tap ? row : -1;
     mk = tap >= 0 ? 1u << tap : 0u;
     rowmap[t] = base ? base[src] : src;
@@ -2685,20 +2708,20 @@ void finish_by_in(Metadata &m, StridedRules &r, hipStream_t s) {
   m.builds++;
   Table &t = r.by_in;
   if (r.by_in_compact && t.n > 0) {
-    int key_bits = 0;
-    const PatternKey pk = pattern_plan(t.n, t.K, key_bits);  // the ranges of the schedule, as for any table
-    int range_bits = 0;
-    while (((int64_t)1 << range_bits) < ceil_div(t.n, pk.window)) range_bits++;
-    t.spread = pk.window >= t.n;
-    reserve_pattern_buffers(m, t);
-    k_few_keys<<<grid_for(t.n), TB, 0, s>>>(r.in_tap.p, t.n, pk.window, m.k0.p, m.v0.p);
+    m.v1.reserve(t.n);  // the order: position t of the table is position v1[t] of the schedule
+    constexpr int FEW_ITEMS = 4;  // windows of 4096 positions (1024, 2048 and 8192 measured alike)
+    const int window = RS1_THREADS * FEW_ITEMS;
+    t.spread = window >= t.n;
+    k_few_order<FEW_ITEMS><<<dim3((unsigned)ceil_div(t.n, window)), RS1_THREADS, 0, s>>>(r.in_tap.p, t.n, m.v1.p);
     LAUNCH_CHECK();
-    sort_pairs(m, m.k0.p, m.k1.p, m.v0.p, m.v1.p, t.n, s, 4 + range_bits);
     t.nbr.reserve((size_t)t.K * t.npad);
     t.rowmap.reserve(t.npad);
     t.gmask.reserve(ceil_div(t.n, 16));
+    t.few_tap.reserve(t.n);
+    t.few_row.reserve(t.n);
     k_table_expand_few<<<grid_for(t.n), TB, 0, s>>>(r.in_tap.p, r.in_row.p, t.K, t.n, t.npad, m.v1.p,
-                                                    li->second.sched_ptr(), t.nbr.p, t.rowmap.p, t.gmask.p);
+                                                    li->second.sched_ptr(), t.nbr.p, t.rowmap.p, t.gmask.p, t.few_tap.p,
+                                                    t.few_row.p);
     LAUNCH_CHECK();
     t.identity_rows = false;
     r.in_tap.release();

@@ -138,6 +138,40 @@ def test_strided(make, dim, size, stride):
     checks.check_strided(make, dim, size, stride, seed=3 + dim, bias=(dim == 2))
 
 
+@pytest.mark.parametrize("cin,cout", [(64, 32), (64, 24), (64, 16), (32, 32), (32, 16), (32, 9)])
+def test_deconvolution_with_all_taps_resident(make, cin, cout):
+    """Transposed convolution of a 2^3 / stride-2 rulebook at the plane counts whose weights of all
+    eight taps fit LDS (the kernel that reads the one rule of every fine position instead of the
+    table's columns): against the rules applied by hand, with a bias, and with a batch norm + leaky
+    ReLU behind it."""
+    rng = np.random.default_rng(cin + cout)
+    n, spatial = 3000, 40
+    pts = np.unique(np.concatenate([rng.integers(0, spatial, (n, 3)), rng.integers(0, 3, (n, 1))], 1), axis=0)
+    pts = pts[rng.permutation(len(pts))].astype(np.int64)
+    p = make(3)
+    p.input_layer(spatial, pts, 0, 4)
+    rules = p.strided_rules(spatial, spatial // 2, 2, 2)
+    n_coarse = p.nactive(spatial // 2)
+    y = rng.normal(size=(n_coarse, cin)).astype(np.float32)
+    w = (rng.normal(size=(8, 1, cin, cout)) * 0.2).astype(np.float32)
+    b = rng.normal(size=cout).astype(np.float32)
+    want = np.zeros((len(pts), cout), np.float64)
+    for k, r in enumerate(rules):  # the rulebook of the convolution, read backwards
+        want[r[:, 0]] += y[r[:, 1]].astype(np.float64) @ w[k, 0].astype(np.float64)
+    z, macs = p.deconv(spatial // 2, spatial, 2, 2, y, w)
+    assert macs == len(pts) * cin * cout
+    checks.assert_close(z, want, "transposed convolution")
+    zb, _ = p.deconv(spatial // 2, spatial, 2, 2, y, w, b)
+    checks.assert_close(zb, want + b, "transposed convolution with bias")
+    bn = dict(mean=rng.normal(size=cout).astype(np.float32), var=rng.uniform(0.5, 1.5, cout).astype(np.float32),
+              weight=rng.uniform(0.5, 1.5, cout).astype(np.float32), bias=rng.normal(size=cout).astype(np.float32),
+              eps=1e-4, leakiness=0.25)
+    zp, _ = p.deconv(spatial // 2, spatial, 2, 2, y, w, b, post=bn)
+    sc = bn["weight"] / np.sqrt(bn["var"] + np.float32(1e-4))
+    v = (want + b) * sc + (bn["bias"] - bn["mean"] * sc)
+    checks.assert_close(zp, np.where(v > 0, v, 0.25 * v), "transposed convolution + batch norm + leaky ReLU")
+
+
 def test_bn(make):
     checks.check_bn(make, seed=1)
     checks.check_bn(make, seed=2, n=1000, C=32)
