@@ -138,28 +138,34 @@ def test_strided(make, dim, size, stride):
     checks.check_strided(make, dim, size, stride, seed=3 + dim, bias=(dim == 2))
 
 
-@pytest.mark.parametrize("cin,cout", [(64, 32), (64, 24), (64, 16), (32, 32), (32, 16), (32, 9)])
-def test_deconvolution_with_all_taps_resident(make, cin, cout):
+@pytest.mark.parametrize("dim,mode,cin,cout", [(3, 4, 64, 32), (3, 4, 64, 24), (3, 4, 64, 16), (3, 4, 32, 32), (3, 4, 32, 16),
+                                               (3, 4, 32, 9), (2, 4, 64, 32), (1, 4, 32, 16), (3, 0, 64, 32), (2, 0, 32, 20)])
+def test_deconvolution_with_all_taps_resident(make, dim, mode, cin, cout):
     """Transposed convolution of a 2^3 / stride-2 rulebook at the plane counts whose weights of all
     eight taps fit LDS (the kernel that reads the one rule of every fine position instead of the
     table's columns): against the rules applied by hand, with a bias, and with a batch norm + leaky
-    ReLU behind it."""
-    rng = np.random.default_rng(cin + cout)
-    n, spatial = 3000, 40
-    pts = np.unique(np.concatenate([rng.integers(0, spatial, (n, 3)), rng.integers(0, 3, (n, 1))], 1), axis=0)
+    ReLU behind it; in one to three dimensions (2, 4, 8 taps), and on a level with repeated points
+    (input-layer mode 0: the rows a later point of their site shadows have no rule and get the bias)."""
+    rng = np.random.default_rng(cin + cout + dim)
+    n, spatial = 3000, {1: 4000, 2: 120, 3: 40}[dim]
+    pts = np.concatenate([rng.integers(0, spatial, (n, dim)), rng.integers(0, 3, (n, 1))], 1)
+    if mode == 0:
+        pts = np.concatenate([pts, pts[rng.integers(0, n, n // 4)]], 0)  # a quarter of the points once more
+    else:
+        pts = np.unique(pts, axis=0)
     pts = pts[rng.permutation(len(pts))].astype(np.int64)
-    p = make(3)
-    p.input_layer(spatial, pts, 0, 4)
+    p = make(dim)
+    assert p.input_layer(spatial, pts, 0, mode) == len(pts)
     rules = p.strided_rules(spatial, spatial // 2, 2, 2)
     n_coarse = p.nactive(spatial // 2)
     y = rng.normal(size=(n_coarse, cin)).astype(np.float32)
-    w = (rng.normal(size=(8, 1, cin, cout)) * 0.2).astype(np.float32)
+    w = (rng.normal(size=(2 ** dim, 1, cin, cout)) * 0.2).astype(np.float32)
     b = rng.normal(size=cout).astype(np.float32)
     want = np.zeros((len(pts), cout), np.float64)
     for k, r in enumerate(rules):  # the rulebook of the convolution, read backwards
         want[r[:, 0]] += y[r[:, 1]].astype(np.float64) @ w[k, 0].astype(np.float64)
     z, macs = p.deconv(spatial // 2, spatial, 2, 2, y, w)
-    assert macs == len(pts) * cin * cout
+    assert macs == sum(len(r) for r in rules) * cin * cout
     checks.assert_close(z, want, "transposed convolution")
     zb, _ = p.deconv(spatial // 2, spatial, 2, 2, y, w, b)
     checks.assert_close(zb, want + b, "transposed convolution with bias")
