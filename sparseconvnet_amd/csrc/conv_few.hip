@@ -25,7 +25,7 @@ namespace scn {
 
 constexpr int FEW_THREADS = 512, FEW_WAVES = FEW_THREADS / 64;
 
-template <int S, int NCB>
+template <int S, int NCB, bool IDENT>
 __global__ __launch_bounds__(FEW_THREADS) void k_deconv_few(
     const unsigned char *__restrict__ ptap, const int *__restrict__ prow, const int *__restrict__ rowmap, int K,
     int64_t n, const float *__restrict__ in, float *__restrict__ out, const float *__restrict__ wp, Epi epi, int n_out,
@@ -76,7 +76,8 @@ __global__ __launch_bounds__(FEW_THREADS) void k_deconv_few(
     const int64_t pos = Q * 64 + lane;
     const bool ok = Q < q1 && pos < n;
     const int64_t at = min(pos, n - 1);
-    const int tap = (int)ptap[at], row = prow[at], orow = rowmap ? rowmap[at] : (int)at;
+    // IDENT (a 1x1 convolution's table): the rule of position t is (tap 0, row t), nothing to read
+    const int tap = IDENT ? 0 : (int)ptap[at], row = IDENT ? (int)at : prow[at], orow = (!IDENT && rowmap) ? rowmap[at] : (int)at;
     x.tap = ok ? tap : 255;
     x.row = ok ? row : 0;
     x.orow = ok ? orow : -1;
@@ -162,7 +163,7 @@ __global__ __launch_bounds__(FEW_THREADS) void k_deconv_few(
   }
 }
 
-template <int S, int NCB>
+template <int S, int NCB, bool IDENT>
 static bool launch_few(Metadata &m, const Table &t, const float *in, float *out, const float *w, Epi epi, int n_in,
                        int n_out, hipStream_t s) {
   constexpr int SLAB_STRIDE = packed_slab_floats(S, NCB);
@@ -172,7 +173,7 @@ static bool launch_few(Metadata &m, const Table &t, const float *in, float *out,
   float *wpack = packed_weights(m, {4, (int64_t)(uintptr_t)w, t.K, n_in, n_out, S, NCB, 0}, packed, [&](float *dst) {
     launch_pack_weights(w, dst, t.K, n_in, n_out, 1, S, NCB, SLAB_STRIDE, take_jobs(m), false, s);
   });
-  auto kern = k_deconv_few<S, NCB>;
+  auto kern = k_deconv_few<S, NCB, IDENT>;
   static bool attr_set = false;
   if (!attr_set) {
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
@@ -187,7 +188,7 @@ static bool launch_few(Metadata &m, const Table &t, const float *in, float *out,
   const int gran_per_wave = (int)round_up(std::max<int64_t>(1, ceil_div(n_granules, 4096)), 4);
   const int64_t waves = ceil_div(n_granules, gran_per_wave);
   const unsigned grid = (unsigned)round_up(ceil_div(waves, FEW_WAVES), 8);
-  note_kernel(m, "few", {{"s", S}, {"ncb", NCB}, {"granules_per_wave", gran_per_wave}});
+  note_kernel(m, "few", {{"s", S}, {"ncb", NCB}, {"identity", IDENT}, {"granules_per_wave", gran_per_wave}});
   kern<<<dim3(grid), FEW_THREADS, lds_bytes, s>>>(t.few_tap.p, t.few_row.p, t.rowmap_ptr(), t.K, t.n, in, out, wpack, epi, n_out,
                                                   n_granules, gran_per_wave, (unsigned)out_bytes, (unsigned)out2_bytes);
   LAUNCH_CHECK();
@@ -195,15 +196,21 @@ static bool launch_few(Metadata &m, const Table &t, const float *in, float *out,
 }
 
 // Tables that carry their one rule per position (the fine side of a filter = stride = 2 rulebook,
-// finish_by_in) and shapes whose weights fit LDS; false: not for this kernel.
+// finish_by_in; the identity table of a 1x1 convolution, CPU/NetworkInNetwork.cpp:7-23) and shapes
+// whose weights fit LDS; false: not for this kernel.
 bool try_few(Metadata &m, const Table &t, const float *in, float *out, const float *w, Epi epi, int n_in, int n_out,
              hipStream_t s) {
-  if (!t.few_tap.p || t.K > 8 || t.n <= 0 || m.bf16 || m.fixed_scratch) return false;
+  const bool ident = t.identity_few && t.identity_rows && t.K == 1;
+  if ((!t.few_tap.p && !ident) || t.K > 8 || t.n <= 0 || m.bf16 || m.fixed_scratch) return false;
   if ((uintptr_t)in % 16 != 0) return false;
-  if (n_in == 64 && n_out <= 32 && n_out > 16) return launch_few<4, 2>(m, t, in, out, w, epi, n_in, n_out, s);
-  if (n_in == 64 && n_out <= 16) return launch_few<4, 1>(m, t, in, out, w, epi, n_in, n_out, s);
-  if (n_in == 32 && n_out <= 32 && n_out > 16) return launch_few<2, 2>(m, t, in, out, w, epi, n_in, n_out, s);
-  if (n_in == 32 && n_out <= 16) return launch_few<2, 1>(m, t, in, out, w, epi, n_in, n_out, s);
+#define FEW_CASE(S, NCB)                                                                         \
+  return ident ? launch_few<S, NCB, true>(m, t, in, out, w, epi, n_in, n_out, s)                 \
+               : launch_few<S, NCB, false>(m, t, in, out, w, epi, n_in, n_out, s)
+  if (n_in == 64 && n_out <= 32 && n_out > 16) FEW_CASE(4, 2);
+  if (n_in == 64 && n_out <= 16) FEW_CASE(4, 1);
+  if (n_in == 32 && n_out <= 32 && n_out > 16) FEW_CASE(2, 2);
+  if (n_in == 32 && n_out <= 16) FEW_CASE(2, 1);
+#undef FEW_CASE
   return false;
 }
 

@@ -83,6 +83,7 @@ struct Table {
   // as (tap, row) of every position, in the table's order (few_tap[t] = 255: no rule); null elsewhere.
   DevBuf<unsigned char> few_tap;
   DevBuf<int> few_row;
+  bool identity_few = false;  // the identity table: position t has the one rule (tap 0, row t); no arrays
   // The pattern sort ran over all positions at once (small levels): consecutive tiles descend in
   // cost from the first to the last, so kernels deal tiles to workgroups in turn instead of giving
   // each XCD a contiguous range.

@@ -2768,6 +2768,7 @@ Table &identity_table(Metadata &m, int64_t rows, hipStream_t s) {
   t.n = rows;
   t.npad = round_up(std::max<int64_t>(rows, 1), 64);
   t.identity_rows = true;
+  t.identity_few = true;
   t.cnt = std::make_shared<Counts>();
   t.cnt->K = 1;
   t.cnt->host.assign(1, rows);

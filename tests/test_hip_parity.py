@@ -188,6 +188,9 @@ def test_nin(make):
     # every convolution kernel family: few / many output planes, wide inputs, odd plane counts
     checks.check_nin(make, seed=5, shapes=((5000, 64, 32), (5000, 32, 64), (3000, 96, 160), (2000, 256, 256),
                                            (70000, 64, 32), (777, 33, 17), (4000, 3, 32), (1500, 448, 224)))
+    # the shapes whose whole weight matrix stays in LDS, at ragged row counts
+    checks.check_nin(make, seed=6, shapes=((1, 64, 32), (63, 64, 16), (4097, 32, 32), (33333, 32, 16), (9000, 64, 24),
+                                           (300001, 64, 32), (5000, 32, 8)))
 
 
 @pytest.mark.parametrize("dim", [1, 2, 3])
