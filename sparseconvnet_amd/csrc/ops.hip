@@ -78,13 +78,18 @@ void bn_eval_forward(const float *in, float *out, int64_t rows, int planes, int6
 enum { POOL_MAX = 0, POOL_AVERAGE = 1, POOL_UNPOOL = 2 };
 template <int V, int MODE>
 __global__ void k_pool(const int *nbr, const int *rowmap, const unsigned *gmask, int K, int64_t n_out, int64_t npad,
-                       const float *in, int in_stride, float *out, int planes) {
+                       const float *in, int in_stride, float *out, int planes, int64_t per_wg) {
   const int groups = planes / V;
   const float volume = (float)K;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t total = n_out * groups;
-  const int64_t step = (int64_t)gridDim.x * blockDim.x;
-  for (; i < total; i += step) {
+  // Workgroups b, b + 8, ... run on one XCD: together they take one contiguous eighth of the
+  // positions (the grid is a multiple of eight), each workgroup a contiguous piece of it, so
+  // that the rows neighbouring positions share (the coarse row above the 2^dim sites of an
+  // unpooling) are fetched into one L2 instead of eight.
+  const int64_t wg = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  int64_t i = wg * per_wg + threadIdx.x;
+  const int64_t end = min(total, (wg + 1) * per_wg);
+  for (; i < end; i += blockDim.x) {
     const int64_t o = i / groups;
     const int p = (int)(i - o * groups) * V;
     float acc[V];
@@ -128,14 +133,15 @@ static void pool_launch(const Table &t, const float *in, int in_stride, float *o
   const bool vec = planes % 4 == 0 && in_stride % 4 == 0 && drop % 4 == 0 && ((uintptr_t)in % 16 == 0) &&
                    ((uintptr_t)out % 16 == 0);
   int64_t total = t.n * (vec ? planes / 4 : planes);
-  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
+  const int64_t blocks = round_up(std::min<int64_t>(ceil_div(total, TB), 256 * 64), 8);
+  const int64_t per_wg = round_up(ceil_div(total, blocks), TB);  // elements a workgroup takes, in turns of TB
   const unsigned *gm = t.K <= 32 ? t.gmask.p : nullptr;  // null when the table kept no granule masks
   if (vec)
     k_pool<4, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in + drop,
-                                                          in_stride, out, planes);
+                                                          in_stride, out, planes, per_wg);
   else
     k_pool<1, MODE><<<dim3((unsigned)blocks), TB, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, in + drop,
-                                                          in_stride, out, planes);
+                                                          in_stride, out, planes, per_wg);
   LAUNCH_CHECK();
 }
 void maxpool_forward(const Table &t, const float *in, int in_stride, float *out, int planes, int drop,
@@ -359,28 +365,30 @@ void input_backward(const InputRules &r, float *d_in, const float *d_out, int pl
 // ---- sparse to dense --------------------------------------------------------------------
 // CPU/SparseToDense.cpp:7-19,35-64: out[sample][plane][offset(site)] = in[row][plane] on a
 // zero-filled [batch, planes, spatial...] tensor.
-__global__ void k_s2d(Geom g, const int *soa, int64_t n, int64_t npad, const float *in, float *out,
-                      int planes, int64_t vol) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = n * planes;
-  int64_t step = (int64_t)gridDim.x * blockDim.x;
-  for (; i < total; i += step) {
-    int64_t r = i / planes;
-    int p = (int)(i - r * planes);
-    int64_t off = 0;
-    for (int d = 0; d < g.dim; d++) off = off * g.size[d] + soa[d * npad + r];
-    int b = soa[g.dim * npad + r];
-    out[((int64_t)b * planes + p) * vol + off] = in[i];
-  }
+// One thread per (site, group of `pchunk` planes), sites taken in the level's schedule (ascending
+// site key): the lanes of a wavefront hold sites that are neighbours in space, so the 4-byte
+// stores of one plane that fall into the same 32-byte sector leave as one write.
+__global__ void k_s2d(Geom g, const int *__restrict__ soa, const int *__restrict__ sched, int64_t n, int64_t npad,
+                      const float *__restrict__ in, float *__restrict__ out, int planes, int64_t vol, int pchunk) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int64_t r = sched ? sched[t] : t;
+  int64_t off = 0;
+  for (int d = 0; d < g.dim; d++) off = off * g.size[d] + soa[d * npad + r];
+  const int b = soa[g.dim * npad + r];
+  const int p0 = blockIdx.y * pchunk, p1 = min(planes, p0 + pchunk);
+  const float *src = in + r * planes;
+  float *dst = out + (int64_t)b * planes * vol + off;
+  for (int p = p0; p < p1; p++) dst[(int64_t)p * vol] = src[p];
 }
 void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStream_t s) {
   int64_t vol = 1;
   for (int d = 0; d < l.g.dim; d++) vol *= l.g.size[d];
   fill32(out, 0, (int64_t)l.batch * planes * vol, s);
   if (l.n == 0 || planes <= 0) return;
-  int64_t total = l.n * planes;
-  int64_t blocks = std::min<int64_t>(ceil_div(total, TB), 256 * 64);
-  k_s2d<<<dim3((unsigned)blocks), TB, 0, s>>>(l.g, l.coords.p, l.n, l.npad, in, out, planes, vol);
+  const int pchunk = 4;
+  const dim3 grid((unsigned)ceil_div(l.n, TB), (unsigned)ceil_div(planes, pchunk));
+  k_s2d<<<grid, TB, 0, s>>>(l.g, l.coords.p, l.sched_ptr(), l.n, l.npad, in, out, planes, vol, pchunk);
   LAUNCH_CHECK();
 }
 
@@ -404,15 +412,16 @@ __global__ void k_sample_starts(const int *soa, const int *sched, int dim, int64
 // grid (sample * chunks + chunk, column tile of CW): partial[(sample * chunks + chunk) * planes + c]
 template <int V>
 __global__ __launch_bounds__(256) void k_active_pool_partial(const int *__restrict__ sched, const int *__restrict__ start,
-                                                             int chunks, const float *__restrict__ in, int planes, int CW,
-                                                             float *__restrict__ partial) {
+                                                             int n_one, int chunks, const float *__restrict__ in, int planes,
+                                                             int CW, float *__restrict__ partial) {
   // A thread owns V consecutive planes (V = 4: 16-byte loads) and has four rows in flight.
   __shared__ float red[256 * V];
   const int b = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
   const int TPR = CW / V;
   const int tx = threadIdx.x % TPR, ty = threadIdx.x / TPR, RW = 256 / TPR;
   const int c = blockIdx.y * CW + tx * V;
-  const int lo = start[b], hi = start[b + 1];
+  // n_one >= 0: a level of one sample, all n_one rows are its rows (start is not read)
+  const int lo = n_one >= 0 ? 0 : start[b], hi = n_one >= 0 ? n_one : start[b + 1];
   const int per = (hi - lo + chunks - 1) / chunks;
   const int t0 = min(hi, lo + chunk * per), t1 = min(hi, t0 + per);
   float acc[V];
@@ -450,7 +459,7 @@ __global__ __launch_bounds__(256) void k_active_pool_partial(const int *__restri
 // grid (sample, tile of 64 planes), 1024 threads: wavefront w adds up its contiguous share of the
 // sample's chunks in order, wavefront 0 then the 16 shares in order (a fixed order).
 __global__ __launch_bounds__(1024) void k_active_pool_finish(const float *__restrict__ partial, const int *__restrict__ start,
-                                                             int chunks, int batch, int planes, int average,
+                                                             int n_one, int chunks, int batch, int planes, int average,
                                                              float *__restrict__ out) {
   __shared__ float part[16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -477,7 +486,7 @@ __global__ __launch_bounds__(1024) void k_active_pool_finish(const float *__rest
     float tot = 0.f;
 #pragma unroll
     for (int w = 0; w < 16; w++) tot += part[w][lane];
-    const int count = start[b + 1] - start[b];
+    const int count = n_one >= 0 ? n_one : start[b + 1] - start[b];
     out[(size_t)b * planes + c] = (average && count > 0) ? tot * (1.0f / (float)count) : tot;
   }
 }
@@ -509,18 +518,24 @@ void active_pool_forward(Metadata &m, const Level &l, const float *in, float *ou
     fill32(out, 0, (int64_t)l.batch * planes, s);
     return;
   }
-  const int *start = sample_starts(m, l, s);
+  // One sample: every row is its row, and the rows are added up as they lie in memory (any fixed
+  // order gives the same bits on every run); several: by the schedule, where a sample's rows
+  // are one range.
+  const bool one = l.batch == 1;
+  const int *start = one ? nullptr : sample_starts(m, l, s);
+  const int *sched = one ? nullptr : l.sched_ptr();
+  const int n_one = one ? (int)l.n : -1;
   // about a thousand workgroups over the batch, at least 256 rows each on average
   int chunks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(1024, l.batch), ceil_div(l.n, (int64_t)256 * l.batch)));
   const int CW = planes <= 16 ? 16 : planes <= 32 ? 32 : 64;
   m.partial.reserve((size_t)l.batch * chunks * planes);
   const dim3 grid((unsigned)(l.batch * chunks), (unsigned)ceil_div(planes, CW));
   if (planes % 4 == 0 && (uintptr_t)in % 16 == 0)
-    k_active_pool_partial<4><<<grid, 256, 0, s>>>(l.sched_ptr(), start, chunks, in, planes, CW, m.partial.p);
+    k_active_pool_partial<4><<<grid, 256, 0, s>>>(sched, start, n_one, chunks, in, planes, CW, m.partial.p);
   else
-    k_active_pool_partial<1><<<grid, 256, 0, s>>>(l.sched_ptr(), start, chunks, in, planes, CW, m.partial.p);
+    k_active_pool_partial<1><<<grid, 256, 0, s>>>(sched, start, n_one, chunks, in, planes, CW, m.partial.p);
   LAUNCH_CHECK();
-  k_active_pool_finish<<<dim3((unsigned)l.batch, (unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, start, chunks,
+  k_active_pool_finish<<<dim3((unsigned)l.batch, (unsigned)ceil_div(planes, 64)), 1024, 0, s>>>(m.partial.p, start, n_one, chunks,
                                                                                               l.batch, planes, average, out);
   LAUNCH_CHECK();
 }
