@@ -20,6 +20,7 @@ namespace scn {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v3f __attribute__((ext_vector_type(3)));
 static const int TB = 256;
 static inline dim3 grid_for(int64_t n, int tb = TB) { return dim3((unsigned)std::max<int64_t>(1, ceil_div(n, tb))); }
 
@@ -458,15 +459,42 @@ __global__ __launch_bounds__(DT_NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4
 // 4 * (MFMA row) + i and columns 4 * (MFMA column) + j of the tile.
 // Granules without the tap are skipped by the granule masks (when the table has them).  A tap
 // with few rules gets few shares (tap_shares, from the table's rule counts) so that every
-// wavefront carries about the same number of rules; blocks of DT_BLOCK granules are dealt
+// wavefront carries about the same number of rules, and only those shares' partial results are
+// written and summed (k_sum_shares); blocks of DT_BLOCK granules are dealt
 // round-robin over a tap's shares.  The loop runs two granules ahead: while the MFMAs of one
 // granule issue, the rows of the next are on their way and the indices of the one after.
 constexpr int DWV_T = 64;
 struct TapShares {
-  unsigned short n[32];  // K <= 32: shares of tap k that have work; the rest only write zeros
+  unsigned short n[32];  // K <= 32: shares of tap k that have work; the rest neither run nor are summed
 };
-// NA, NB: channels per lane on the a- and the b-side (4, or 2 for a side of at most 32 channels: a
-// tile is 16 NA x 16 NB channels, so that a narrow side does not fill half its MFMAs with zeros).
+// k_sum_blocks over the partial results of k_conv_dw_wave: output i belongs to tap i / per_tap,
+// whose first tap_shares.n[tap] blocks hold sums (all `blocks` of them when K > 32).  Same fixed order.
+__global__ __launch_bounds__(1024) void k_sum_shares(const float *__restrict__ partial, int blocks, int64_t stride,
+                                                     int64_t count, int per_tap, int K, TapShares tap_shares,
+                                                     float *__restrict__ out) {
+  __shared__ float part[16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + lane;
+  const int waves = blockDim.x >> 6;
+  float s = 0;
+  if (i < count) {
+    const int mine = K <= 32 ? min(blocks, (int)tap_shares.n[i / per_tap]) : blocks;
+    const int per = (mine + waves - 1) / waves;
+    const int b0 = min(mine, wave * per), b1 = min(mine, b0 + per);
+#pragma unroll 4
+    for (int b = b0; b < b1; b++) s += partial[(size_t)b * stride + i];
+  }
+  part[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && i < count) {
+    float tot = 0;
+    for (int w = 0; w < waves; w++) tot += part[w][lane];
+    out[i] = tot;
+  }
+}
+// NA, NB: channels per lane on the a- and the b-side (4; 2 for a side of at most 32 channels; 3 where
+// tiles of 48 channels leave fewer empty columns than tiles of 64, e.g. 96 = 2 x 48: a tile is
+// 16 NA x 16 NB channels, and the MFMAs of a tile's empty part multiply zeros).
 // VEC: a lane's channels come as one 16- or 8-byte load (plane counts multiples of NA / NB, arrays aligned).
 template <bool VEC, int NA, int NB>
 __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nbr, const int *__restrict__ rowmap,
@@ -509,6 +537,10 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
       const unsigned off = (j < 0 || c0 >= width) ? nowhere : row + (unsigned)c0 * 4u;
       const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
       e[0] = v.x, e[1] = v.y, e[2] = v.z, e[3] = v.w;
+    } else if constexpr (VEC && N == 3) {
+      const unsigned off = (j < 0 || c0 >= width) ? nowhere : row + (unsigned)c0 * 4u;
+      const v3f v = __builtin_bit_cast(v3f, __builtin_amdgcn_raw_buffer_load_b96(rsrc, off, 0, 0));
+      e[0] = v.x, e[1] = v.y, e[2] = v.z;
     } else if constexpr (VEC && N == 2) {
       const unsigned off = (j < 0 || c0 >= width) ? nowhere : row + (unsigned)c0 * 4u;
       const v2f v = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0));
@@ -529,6 +561,7 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
   const int n_granules = (int)((n + 15) >> 4), n32 = (int)n;
   const bool idle = ct * TA >= n_a || ot * TB_ >= n_b;  // a tile past the last channel: only keeps the barrier count
   const int mine = K <= 32 ? (int)tap_shares.n[k] : shares;    // shares of this tap that have work
+  if (share >= mine) return;  // uniform over the workgroup (over the wavefront when single); k_sum_shares does not read its part
   // This share's granules: blocks share, share + mine, ... of DT_BLOCK granules, those with the tap.
   auto next_granule = [&](int gi) {  // the one after gi (n_granules: none)
     for (;;) {
@@ -567,7 +600,7 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
         for (int jx = 0; jx < NB; jx++)
           acc[i][jx] = __builtin_amdgcn_mfma_f32_16x16x4f32(q.a[kk][i], q.b[kk][jx], acc[i][jx], 0, 0, 0);
   };
-  if (share < mine) {  // uniform over the workgroup (over the wavefront when single)
+  {
     Quads X, Y;
     int g0 = share * DT_BLOCK;
     if (g0 >= n_granules) g0 = n_granules;
@@ -612,6 +645,132 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
     }
 }
 
+// Inputs of one to four channels (the first layer of a network: colour, occupancy): a tile of 16 a-side
+// channels would be three quarters empty, so the 16 rows of the MFMA hold G = 16 / NA TAPS of NA
+// channels each instead - lane (r, g) supplies channel r % NA of the row that tap m G + r / NA
+// reads at position 4 g + kk - and NG such groups cover the filter (3 channels, 27 taps: 6 groups
+// of 5 taps, 48 MFMAs per 16 positions where one tile per tap would issue 216).  A wavefront takes
+// granules w, w + W, ... of the table for ALL taps (every wavefront sees every part of the
+// pattern-sorted table; the rows of b are read once per granule), skips the groups none of whose
+// taps the granule has, and runs two granules ahead like k_conv_dw_wave.  partial[w][K][NA][n_b].
+template <int NA, int NG>
+__global__ __launch_bounds__(256) void k_conv_dw_thin(const int *__restrict__ nbr, const int *__restrict__ rowmap,
+                                                      const unsigned *__restrict__ gmask, int K, int64_t n, int64_t npad,
+                                                      const float *__restrict__ a, unsigned a_bytes,
+                                                      const float *__restrict__ b, int n_b, unsigned b_bytes,
+                                                      float *__restrict__ partial) {
+  constexpr int G = 16 / NA;
+  const int lane = threadIdx.x & 63;
+  const int w = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), W = gridDim.x * 4;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int tsub = r16 / NA, chan = r16 % NA;
+  const unsigned nowhere = 0x80000000u;  // offsets from here on read zeros
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a), 0, (int)a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(b), 0, (int)b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t nbr_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(nbr), 0, (int)((unsigned)K * (unsigned)npad * 4u), 0x00020000);
+  const __amdgpu_buffer_rsrc_t map_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(rowmap ? rowmap : nbr), 0, (int)((unsigned)npad * 4u), 0x00020000);
+  // the lane's tap in group m, as the byte offset of its row of the table (nowhere: the lane holds
+  // no tap there), and the taps of each group as a mask
+  unsigned tap_off[NG], group_taps[NG];
+#pragma unroll
+  for (int m = 0; m < NG; m++) {
+    const int tap = m * G + tsub;
+    tap_off[m] = (tsub < G && tap < K) ? (unsigned)tap * (unsigned)npad * 4u : nowhere;
+    group_taps[m] = (G >= 32 ? 0xFFFFFFFFu : ((1u << G) - 1u)) << (m * G);
+  }
+  const unsigned cb_off[2] = {r16 < n_b ? (unsigned)r16 * 4u : nowhere, 16 + r16 < n_b ? (unsigned)(16 + r16) * 4u : nowhere};
+  const unsigned b_row_bytes = (unsigned)n_b * 4u;
+  v4f acc[NG][2];
+#pragma unroll
+  for (int m = 0; m < NG; m++) acc[m][0] = acc[m][1] = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int n_granules = (int)((n + 15) >> 4), n32 = (int)n;
+  struct Rows {
+    float a[NG][4], b[4][2];
+  };
+  int4 jq[NG], rq;  // of the granule whose rows are requested next
+  auto load_indices = [&](int gi) {
+    const unsigned toff = gi < n_granules ? (unsigned)(gi * 16 + 4 * g) * 4u : nowhere;
+#pragma unroll
+    for (int m = 0; m < NG; m++)
+      jq[m] = __builtin_bit_cast(int4, __builtin_amdgcn_raw_buffer_load_b128(
+                                           nbr_rsrc, (toff | tap_off[m]) & nowhere ? nowhere : toff + tap_off[m], 0, 0));
+    const int t = gi * 16 + 4 * g;
+    rq = make_int4(t, t + 1, t + 2, t + 3);
+    if (rowmap) rq = __builtin_bit_cast(int4, __builtin_amdgcn_raw_buffer_load_b128(map_rsrc, toff, 0, 0));
+  };
+  auto load_rows = [&](int gi, Rows &q) {
+    const int r[4] = {rq.x, rq.y, rq.z, rq.w};
+    bool live[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) live[kk] = gi < n_granules && gi * 16 + 4 * g + kk < n32;
+#pragma unroll
+    for (int m = 0; m < NG; m++) {
+      const int j[4] = {jq[m].x, jq[m].y, jq[m].z, jq[m].w};
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++) {
+        // a lane without a tap read zeros for its indices: row 0, which it must not gather
+        const bool take = live[kk] && tap_off[m] != nowhere && j[kk] >= 0;
+        q.a[m][kk] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                   a_rsrc, take ? (unsigned)j[kk] * (unsigned)(NA * 4) + (unsigned)chan * 4u : nowhere, 0, 0));
+      }
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++)
+        q.b[kk][nt] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                    b_rsrc, (live[kk] && cb_off[nt] != nowhere) ? (unsigned)r[kk] * b_row_bytes + cb_off[nt] : nowhere, 0, 0));
+  };
+  auto taps_of = [&](int gi) {  // the taps granule gi has (wavefront-uniform)
+    return (gmask && gi < n_granules) ? (unsigned)__builtin_amdgcn_readfirstlane((int)gmask[gi]) : 0xFFFFFFFFu;
+  };
+  auto multiply = [&](const Rows &q, unsigned present) {
+#pragma unroll
+    for (int m = 0; m < NG; m++) {
+      if (!(present & group_taps[m])) continue;  // uniform over the wavefront
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++)
+          acc[m][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(q.a[m][kk], q.b[kk][nt], acc[m][nt], 0, 0, 0);
+    }
+  };
+  {
+    Rows X, Y;
+    int g0 = min(w, n_granules), g1 = min(g0 + W, n_granules);
+    unsigned p0 = taps_of(g0), p1 = taps_of(g1);
+    load_indices(g0);
+    load_rows(g0, X);
+    load_indices(g1);
+    while (g0 < n_granules) {
+      // X: rows of g0 (requested), jq / rq: indices of g1 (requested)
+      const int g2 = min(g1 + W, n_granules), g3 = min(g2 + W, n_granules);
+      const unsigned p2 = taps_of(g2), p3 = taps_of(g3);
+      load_rows(g1, Y);
+      load_indices(g2);
+      multiply(X, p0);
+      load_rows(g2, X);
+      load_indices(g3);
+      if (g1 < n_granules) multiply(Y, p1);
+      g0 = g2, g1 = g3, p0 = p2, p1 = p3;
+    }
+  }
+  // acc[m][nt][r] = row 4 g + r of group m = (tap m G + (4 g + r) / NA, channel (4 g + r) % NA), column 16 nt + r16
+  float *pw = partial + (size_t)w * K * NA * n_b;
+#pragma unroll
+  for (int m = 0; m < NG; m++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int row = 4 * g + r, tap = m * G + row / NA, c = row % NA;
+      if (row >= G * NA || tap >= K) continue;
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++)
+        if (16 * nt + r16 < n_b) pw[((size_t)tap * NA + c) * n_b + 16 * nt + r16] = acc[m][nt][r];
+    }
+}
+
 // Any groups, any shapes: one thread per weight, positions in order.  The correctness path for
 // grouped convolutions, which the MFMA kernel does not cover.
 __global__ void k_conv_dw_generic(const int *nbr, const int *rowmap, int K, int64_t n, int64_t npad, const float *a,
@@ -646,6 +805,33 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
     return;
   }
   const bool vec4 = n_a % 4 == 0 && n_b % 4 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0;
+  // one to four input channels: several taps share an MFMA's rows
+  if (n_a <= 4 && n_b <= 32 && t.K <= 32 && t.npad % 4 == 0 && a_rows * n_a * 4 < ((int64_t)1 << 31) &&
+      b_rows * n_b * 4 < ((int64_t)1 << 31) && (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31)) {
+    const int groups_of_taps = (int)ceil_div(t.K, 16 / n_a);
+    const int64_t n_granules = ceil_div(t.n, 16);
+    const int64_t waves = round_up(std::min<int64_t>(n_granules, 2048), 4);
+    const unsigned *gm = t.gmask.p;  // null when the table kept no granule masks
+    bool done = true;
+#define SCN_THIN(A, NGR)                                                                                            \
+  k_conv_dw_thin<A, NGR><<<dim3((unsigned)(waves / 4)), 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, \
+                                                                     (unsigned)(a_rows * n_a * 4), b, n_b,           \
+                                                                     (unsigned)(b_rows * n_b * 4), m.partial.p)
+    m.partial.reserve((size_t)waves * per_chunk);
+    if (n_a == 3 && groups_of_taps <= 2) SCN_THIN(3, 2);
+    else if (n_a == 3 && groups_of_taps <= 6) SCN_THIN(3, 6);
+    else if (n_a == 1 && groups_of_taps <= 2) SCN_THIN(1, 2);
+    else if (n_a == 4 && groups_of_taps <= 2) SCN_THIN(4, 2);
+    else if (n_a == 4 && groups_of_taps <= 7) SCN_THIN(4, 7);
+    else done = false;  // other shapes: the kernels below
+#undef SCN_THIN
+    if (done) {
+      LAUNCH_CHECK();
+      k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), sum_threads(waves), 0, s>>>(m.partial.p, (int)waves, per_chunk, per_chunk, dw);
+      LAUNCH_CHECK();
+      return;
+    }
+  }
   // up to 32 channels on both sides; from there on the per-wavefront kernel below is faster
   // (64 -> 64 at 1 M sites: 1.97 against 1.3 ms)
   if (t.K <= DT_NW * DT_SLOTS && t.gmask.p && n_a <= DT_T && n_b <= DT_T && t.npad % 4 == 0 &&
@@ -675,7 +861,23 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
       (int64_t)t.K * t.npad * 4 < ((int64_t)1 << 31) && t.K <= 65535) {
     // wider layers: a wavefront per (tap, 64 x 64 tile, share of the positions)
     // a side of at most 32 channels gives a lane two channels of it instead of four: tiles of 32 there
-    const int na = n_a <= 32 ? 2 : 4, nb = n_b <= 32 ? 2 : 4;
+    // (a lane's three channels come as one 12-byte load: only with plane counts that are multiples of three)
+    auto lane_channels = [](int planes) {
+      if (planes <= 32) return 2;
+      const int64_t pad4 = round_up(planes, 64), pad3 = round_up(planes, 48);
+      return (planes % 3 == 0 && pad3 * 8 <= pad4 * 7) ? 3 : 4;
+    };
+    int na = lane_channels(n_a), nb = lane_channels(n_b);
+    if (na == 3 && nb == 2) na = 4;  // the pairs of 3 and 2 are not built
+    if (nb == 3 && na == 2) nb = 4;
+    // one load per lane and side when the plane counts are multiples of the lane's channels and the
+    // arrays aligned (16- and 8-byte loads to their size, 12-byte loads to a word)
+    auto one_load = [&](int ka, int kb) {
+      return n_a % ka == 0 && n_b % kb == 0 && (uintptr_t)a % (ka == 3 ? 4 : 4 * ka) == 0 &&
+             (uintptr_t)b % (kb == 3 ? 4 : 4 * kb) == 0;
+    };
+    if (!one_load(na, nb)) na = na == 3 ? 4 : na, nb = nb == 3 ? 4 : nb;  // three channels per lane: as one load only
+    const bool vec = one_load(na, nb);
     const int tile_a = 16 * na, tile_b = 16 * nb;
     const int tiles64 = (int)(ceil_div(n_a, tile_a) * ceil_div(n_b, tile_b));
     const bool single = tiles64 < 4;  // fewer than four tiles: a workgroup's wavefronts are (share, tile) pairs
@@ -704,14 +906,15 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
       m.partial.reserve((size_t)shares * per_chunk);
       const dim3 grid((unsigned)t.K, (unsigned)(single ? ceil_div(shares * tiles64, 4) : shares), (unsigned)tiles);
       const unsigned *gm = (t.K <= 32 && t.gmask.p) ? t.gmask.p : nullptr;
-      // one load per lane and side when the plane counts are multiples of the lane's channels and the arrays aligned
-      const bool vec = n_a % na == 0 && n_b % nb == 0 && (uintptr_t)a % (4 * na) == 0 && (uintptr_t)b % (4 * nb) == 0;
 #define SCN_DWV(V, A, B)                                                                                              \
   k_conv_dw_wave<V, A, B><<<grid, 256, 0, s>>>(t.nbr.p, t.rowmap_ptr(), gm, t.K, t.n, t.npad, a, n_a,                 \
                                                (unsigned)(a_rows * n_a * 4), b, n_b, (unsigned)(b_rows * n_b * 4),    \
                                                (int)shares, ts, m.partial.p)
       if (vec) {
         if (na == 4 && nb == 4) SCN_DWV(true, 4, 4);
+        else if (na == 3 && nb == 3) SCN_DWV(true, 3, 3);
+        else if (na == 3) SCN_DWV(true, 3, 4);
+        else if (nb == 3) SCN_DWV(true, 4, 3);
         else if (na == 4) SCN_DWV(true, 4, 2);
         else if (nb == 4) SCN_DWV(true, 2, 4);
         else SCN_DWV(true, 2, 2);
@@ -723,8 +926,8 @@ static void weight_gradient(Metadata &m, const Table &t, const float *a, int64_t
       }
 #undef SCN_DWV
       LAUNCH_CHECK();
-      k_sum_blocks<float, float><<<dim3((unsigned)ceil_div(per_chunk, 64)), sum_threads(shares), 0, s>>>(m.partial.p, (int)shares, per_chunk,
-                                                                                      per_chunk, dw);
+      k_sum_shares<<<dim3((unsigned)ceil_div(per_chunk, 64)), sum_threads(shares), 0, s>>>(m.partial.p, (int)shares, per_chunk, per_chunk,
+                                                                                           n_a * n_b, t.K, ts, dw);
       LAUNCH_CHECK();
       return;
     }

@@ -53,7 +53,8 @@ def test_misc_backward(make):
 
 @pytest.mark.parametrize("cin,cout,groups", [(3, 32, 1), (32, 32, 1), (16, 16, 1), (64, 64, 1), (96, 128, 1),
                                              (128, 160, 1), (256, 256, 1), (30, 50, 1), (8, 12, 2), (64, 32, 1),
-                                             (320, 160, 1), (40, 288, 1)])
+                                             (320, 160, 1), (40, 288, 1), (96, 96, 1), (144, 48, 1), (192, 96, 1),
+                                             (1, 16, 1), (4, 32, 1), (3, 20, 1)])
 def test_conv_gradients_vs_oracle(oracle_built, cin, cout, groups):
     """Submanifold, strided and transposed convolution gradients on a 20,000-site room scene
     against the oracle, over the channel ranges of every forward kernel family (the input
