@@ -235,7 +235,8 @@ def test_pooling_and_nin_gradients_vs_oracle(oracle_built):
         res[-1]["d_un"] = p.unpool_bwd(63, 127, 3, 2, 32, up_d)[r1]
     for k in res[0]:
         checks.assert_close(res[0][k], res[1][k], k)
-    for rows, cin, cout in ((70000, 64, 32), (5000, 256, 256), (777, 33, 17)):
+    for rows, cin, cout in ((70000, 64, 32), (5000, 256, 256), (777, 33, 17), (9001, 3, 32), (1, 4, 16), (500, 1, 20),
+                            (4000, 96, 48)):
         a = rng.normal(size=(rows, cin)).astype(np.float32)
         w = (rng.normal(size=(cin, cout)) * 0.1).astype(np.float32)
         d = rng.normal(size=(rows, cout)).astype(np.float32)
