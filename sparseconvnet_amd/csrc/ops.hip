@@ -490,18 +490,30 @@ __global__ __launch_bounds__(1024) void k_active_pool_finish(const float *__rest
     out[(size_t)b * planes + c] = (average && count > 0) ? tot * (1.0f / (float)count) : tot;
   }
 }
-// CPU/ActivePooling.cpp:26-44,65-83: every row receives its sample's gradient.
-__global__ void k_active_pool_bwd(const int *soa, int dim, int64_t n, int64_t npad, const int *start, int planes,
-                                  int average, const float *d_out, float *d_in) {
+// CPU/ActivePooling.cpp:26-44,65-83: every row receives its sample's gradient.  A thread writes V
+// consecutive planes of a row (V = 4: 16-byte accesses); n_one >= 0: a level of one sample with
+// n_one rows (neither the sample column nor start is read).
+template <int V>
+__global__ void k_active_pool_bwd(const int *__restrict__ soa, int dim, int64_t n, int64_t npad,
+                                  const int *__restrict__ start, int n_one, int planes, int average,
+                                  const float *__restrict__ d_out, float *__restrict__ d_in) {
+  const int groups = planes / V;
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t total = n * planes, step = (int64_t)gridDim.x * blockDim.x;
+  const int64_t total = n * groups, step = (int64_t)gridDim.x * blockDim.x;
   for (; i < total; i += step) {
-    const int64_t r = i / planes;
-    const int c = (int)(i - r * planes);
-    const int b = soa[(int64_t)dim * npad + r];
-    const int count = start[b + 1] - start[b];
+    const int64_t r = i / groups;
+    const int c = (int)(i - r * groups) * V;
+    const int b = n_one >= 0 ? 0 : soa[(int64_t)dim * npad + r];
+    const int count = n_one >= 0 ? n_one : start[b + 1] - start[b];
     const float mult = (average && count > 0) ? 1.0f / (float)count : 1.0f;
-    d_in[i] = d_out[(int64_t)b * planes + c] * mult;
+    const float *src = d_out + (int64_t)b * planes + c;
+    float *dst = d_in + r * planes + c;
+    if constexpr (V == 4) {
+      const float4 x = *reinterpret_cast<const float4 *>(src);
+      *reinterpret_cast<float4 *>(dst) = make_float4(x.x * mult, x.y * mult, x.z * mult, x.w * mult);
+    } else {
+      dst[0] = src[0] * mult;
+    }
   }
 }
 static const int *sample_starts(Metadata &m, const Level &l, hipStream_t s) {
@@ -542,10 +554,17 @@ void active_pool_forward(Metadata &m, const Level &l, const float *in, float *ou
 void active_pool_backward(Metadata &m, const Level &l, float *d_in, const float *d_out, int planes, int average,
                           hipStream_t s) {
   if (l.n == 0 || planes <= 0) return;
-  const int *start = sample_starts(m, l, s);
-  const int64_t blocks = std::min<int64_t>(ceil_div(l.n * planes, TB), 256 * 64);
-  k_active_pool_bwd<<<dim3((unsigned)blocks), TB, 0, s>>>(l.coords.p, l.g.dim, l.n, l.npad, start, planes, average, d_out,
-                                                          d_in);
+  const bool one = l.batch == 1;
+  const int *start = one ? nullptr : sample_starts(m, l, s);
+  const int n_one = one ? (int)l.n : -1;
+  const bool vec = planes % 4 == 0 && (uintptr_t)d_in % 16 == 0 && (uintptr_t)d_out % 16 == 0;
+  const int64_t blocks = std::min<int64_t>(ceil_div(l.n * (vec ? planes / 4 : planes), TB), 256 * 64);
+  if (vec)
+    k_active_pool_bwd<4><<<dim3((unsigned)blocks), TB, 0, s>>>(l.coords.p, l.g.dim, l.n, l.npad, start, n_one, planes, average,
+                                                               d_out, d_in);
+  else
+    k_active_pool_bwd<1><<<dim3((unsigned)blocks), TB, 0, s>>>(l.coords.p, l.g.dim, l.n, l.npad, start, n_one, planes, average,
+                                                               d_out, d_in);
   LAUNCH_CHECK();
 }
 
