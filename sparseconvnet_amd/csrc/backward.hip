@@ -563,13 +563,38 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
   const int mine = K <= 32 ? (int)tap_shares.n[k] : shares;    // shares of this tap that have work
   if (share >= mine) return;  // uniform over the workgroup (over the wavefront when single); k_sum_shares does not read its part
   // This share's granules: blocks share, share + mine, ... of DT_BLOCK granules, those with the tap.
-  auto next_granule = [&](int gi) {  // the one after gi (n_granules: none)
+  // The masks of a block come as one pair of 16-byte loads (past the last granule they read zeros:
+  // no tap) and are kept as a bit per granule, so that the search for the next granule with the
+  // tap waits for memory once per block, not once per granule (the fine side of a filter = stride
+  // rulebook has the tap in one granule of 2^dim).
+  static_assert(DT_BLOCK == 8, "a block's granule masks are two 16-byte loads");
+  const __amdgpu_buffer_rsrc_t gm_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<unsigned *>(gmask ? gmask : reinterpret_cast<const unsigned *>(nbr)), 0, (int)((unsigned)n_granules * 4u), 0x00020000);
+  int cur_base = -DT_BLOCK;
+  unsigned cur_bits = 0u;
+  auto block_bits = [&](int base) {
+    if (!gmask) return n_granules - base >= DT_BLOCK ? 0xFFu : (1u << (n_granules - base)) - 1u;
+    const uint4 lo = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(gm_rsrc, (unsigned)base * 4u, 0, 0));
+    const uint4 hi = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(gm_rsrc, (unsigned)base * 4u + 16u, 0, 0));
+    const unsigned w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    unsigned bits = 0u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) bits |= ((w[i] >> k) & 1u) << i;
+    return bits;
+  };
+  auto seek = [&](int gi) {  // the first granule from gi on (a granule of one of the share's blocks) that has the tap
     for (;;) {
-      gi++;
-      if (gi % DT_BLOCK == 0) gi += (mine - 1) * DT_BLOCK;
       if (gi >= n_granules) return n_granules;
-      if (!gmask || ((gmask[gi] >> k) & 1u)) return gi;
+      const int base = gi & ~(DT_BLOCK - 1);
+      if (base != cur_base) cur_base = base, cur_bits = block_bits(base);
+      const unsigned rem = cur_bits >> (gi & (DT_BLOCK - 1));
+      if (rem) return gi + __builtin_ctz(rem);
+      gi = base + mine * DT_BLOCK;
     }
+  };
+  auto next_granule = [&](int gi) {  // the one after gi (n_granules: none)
+    if (gi >= n_granules) return n_granules;
+    return seek((gi & (DT_BLOCK - 1)) == DT_BLOCK - 1 ? (gi & ~(DT_BLOCK - 1)) + mine * DT_BLOCK : gi + 1);
   };
   struct Quads {
     float a[4][NA], b[4][NB];
@@ -602,9 +627,7 @@ __global__ __launch_bounds__(256) void k_conv_dw_wave(const int *__restrict__ nb
   };
   {
     Quads X, Y;
-    int g0 = share * DT_BLOCK;
-    if (g0 >= n_granules) g0 = n_granules;
-    else if (gmask && !((gmask[g0] >> k) & 1u)) g0 = next_granule(g0);
+    int g0 = seek(share * DT_BLOCK);
     int g1 = next_granule(g0);
     if (!idle) {
       load_indices(g0);
