@@ -30,6 +30,19 @@ def test_strided_backward(make, dim, size, stride):
     checks.check_strided_backward(make, dim, size, stride, seed=40 + dim)
 
 
+@pytest.mark.parametrize("dim", [1, 2, 3])
+@pytest.mark.parametrize("thin", [1, 3, 4])
+def test_thin_input_weight_gradient(make, dim, thin):
+    """One to four channels on the gathered side: the weight-gradient kernel that packs several taps
+    into an MFMA's rows, for filters of 3, 9 and 27 taps (submanifold), 2^dim taps from either
+    side (strided: the input has the thin side; transposed: the coarse level has it) and ragged
+    site counts, against torch.autograd through the dense convolutions."""
+    checks.check_conv_backward(make, dim, 3, seed=130 + 10 * dim + thin, spatial=9, n=333, cin=thin, cout=20)
+    checks.check_conv_backward(make, dim, 3, seed=230 + 10 * dim + thin, spatial=9, n=17, cin=thin, cout=32, bias=False)
+    checks.check_strided_backward(make, dim, 2, 2, seed=330 + 10 * dim + thin, n=210, cin=thin, cout=9, pools=False)
+    checks.check_strided_backward(make, dim, 2, 2, seed=430 + 10 * dim + thin, n=210, cin=24, cout=thin, pools=False)
+
+
 def test_bn_train(make):
     checks.check_bn_train(make, seed=50)
     checks.check_bn_train(make, seed=51, n=5000, C=96)
