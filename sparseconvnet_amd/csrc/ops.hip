@@ -82,14 +82,17 @@ __global__ void k_pool(const int *nbr, const int *rowmap, const unsigned *gmask,
   const int groups = planes / V;
   const float volume = (float)K;
   const int64_t total = n_out * groups;
-  // Workgroups b, b + 8, ... run on one XCD: together they take one contiguous eighth of the
-  // positions (the grid is a multiple of eight), each workgroup a contiguous piece of it, so
-  // that the rows neighbouring positions share (the coarse row above the 2^dim sites of an
-  // unpooling) are fetched into one L2 instead of eight.
-  const int64_t wg = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  int64_t i = wg * per_wg + threadIdx.x;
-  const int64_t end = min(total, (wg + 1) * per_wg);
-  for (; i < end; i += blockDim.x) {
+  // Unpooling: workgroups b, b + 8, ... run on one XCD and together take one contiguous eighth of
+  // the positions (the grid is a multiple of eight), each workgroup a contiguous piece of it, so
+  // that the coarse row above a site's 2^dim children is fetched into one L2 instead of eight
+  // (102 -> 40 MB read at a million sites).  Pooling: workgroups take turns over the table, whose
+  // positions are sorted by cost - contiguous ranges would give one XCD the expensive end.
+  const bool ranges = MODE == POOL_UNPOOL;
+  const int64_t wg = ranges ? (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3) : (int64_t)blockIdx.x;
+  int64_t i = (ranges ? wg * per_wg : wg * blockDim.x) + threadIdx.x;
+  const int64_t end = ranges ? min(total, (wg + 1) * per_wg) : total;
+  const int64_t step = ranges ? (int64_t)blockDim.x : (int64_t)gridDim.x * blockDim.x;
+  for (; i < end; i += step) {
     const int64_t o = i / groups;
     const int p = (int)(i - o * groups) * V;
     float acc[V];
