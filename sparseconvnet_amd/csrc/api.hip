@@ -299,6 +299,17 @@ void pinned_release(void *p, size_t bytes) {
 // instead the counts are copied to pinned memory behind the work already enqueued, an event
 // marks the copy, and scn_take_released_macs folds whatever has been left behind.
 namespace {
+// The rule counts of up to 48 tables copied into one staging array by one launch: block b copies
+// table b's words.  dst is pinned host memory (hipHostMalloc: device-accessible), so that a
+// handle with forty tables costs the stream one short kernel instead of forty copies.
+struct CountJobs {
+  const long long *src[48];
+  int off[48], words[48];
+};
+__global__ void k_gather_counts(CountJobs j, long long *dst) {
+  const int b = blockIdx.x;
+  for (int i = threadIdx.x; i < j.words[b]; i += blockDim.x) dst[j.off[b] + i] = j.src[b][i];
+}
 struct ReleasedMacs {
   hipEvent_t ev = nullptr;
   long long *stage = nullptr;
@@ -334,14 +345,24 @@ void release_macs(Metadata &m) {
       r.stage_bytes = round_up((int64_t)(words * sizeof(long long)), 1 << 16);
       r.stage = static_cast<long long *>(pinned_acquire(r.stage_bytes));
       size_t off = 0;
+      CountJobs jobs{};
+      int n_jobs = 0;
+      auto flush = [&] {
+        if (!n_jobs) return;
+        k_gather_counts<<<dim3((unsigned)n_jobs), 64, 0, s>>>(jobs, r.stage);
+        LAUNCH_CHECK();
+        n_jobs = 0;
+      };
       for (auto &pm : m.pending_macs) {
         Counts &c = *pm.first;
         if (c.ready || !c.K || !c.dev.p) continue;
         const size_t w = (size_t)c.K * c.slots;
-        HIP_CHECK(hipMemcpyAsync(r.stage + off, c.dev.p, w * sizeof(long long), hipMemcpyDeviceToHost, s));
+        jobs.src[n_jobs] = c.dev.p, jobs.off[n_jobs] = (int)off, jobs.words[n_jobs] = (int)w;
+        if (++n_jobs == 48) flush();
         r.items.push_back({off, c.K, c.slots, pm.second});
         off += w;
       }
+      flush();
       HIP_CHECK(hipEventCreateWithFlags(&r.ev, hipEventDisableTiming));
       HIP_CHECK(hipEventRecord(r.ev, s));
     } catch (...) {  // a lost device: the counts are not worth an error in a destructor
