@@ -368,11 +368,11 @@ void input_backward(const InputRules &r, float *d_in, const float *d_out, int pl
 // ---- sparse to dense --------------------------------------------------------------------
 // CPU/SparseToDense.cpp:7-19,35-64: out[sample][plane][offset(site)] = in[row][plane] on a
 // zero-filled [batch, planes, spatial...] tensor.
-// One thread per (site, group of `pchunk` planes), sites taken in the level's schedule (ascending
+// One thread per (site, group of `pchunk` planes; 8 with 16-byte loads of the row), sites taken in the level's schedule (ascending
 // site key): the lanes of a wavefront hold sites that are neighbours in space, so the 4-byte
 // stores of one plane that fall into the same 32-byte sector leave as one write.
 __global__ void k_s2d(Geom g, const int *__restrict__ soa, const int *__restrict__ sched, int64_t n, int64_t npad,
-                      const float *__restrict__ in, float *__restrict__ out, int planes, int64_t vol, int pchunk) {
+                      const float *__restrict__ in, float *__restrict__ out, int planes, int64_t vol, int pchunk, bool vec4) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n) return;
   const int64_t r = sched ? sched[t] : t;
@@ -382,6 +382,15 @@ __global__ void k_s2d(Geom g, const int *__restrict__ soa, const int *__restrict
   const int p0 = blockIdx.y * pchunk, p1 = min(planes, p0 + pchunk);
   const float *src = in + r * planes;
   float *dst = out + (int64_t)b * planes * vol + off;
+  if (vec4) {  // pchunk = 8 on 16-byte aligned rows: two loads, then the stores
+    const float4 x0 = *reinterpret_cast<const float4 *>(src + p0);
+    const float4 x1 = p0 + 4 < p1 ? *reinterpret_cast<const float4 *>(src + p0 + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    const float v[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      if (p0 + i < p1) dst[(int64_t)(p0 + i) * vol] = v[i];
+    return;
+  }
   for (int p = p0; p < p1; p++) dst[(int64_t)p * vol] = src[p];
 }
 void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStream_t s) {
@@ -389,9 +398,10 @@ void s2d_forward(const Level &l, const float *in, float *out, int planes, hipStr
   for (int d = 0; d < l.g.dim; d++) vol *= l.g.size[d];
   fill32(out, 0, (int64_t)l.batch * planes * vol, s);
   if (l.n == 0 || planes <= 0) return;
-  const int pchunk = 4;
+  const bool vec4 = planes % 4 == 0 && (uintptr_t)in % 16 == 0;
+  const int pchunk = vec4 ? 8 : 4;
   const dim3 grid((unsigned)ceil_div(l.n, TB), (unsigned)ceil_div(planes, pchunk));
-  k_s2d<<<grid, TB, 0, s>>>(l.g, l.coords.p, l.sched_ptr(), l.n, l.npad, in, out, planes, vol, pchunk);
+  k_s2d<<<grid, TB, 0, s>>>(l.g, l.coords.p, l.sched_ptr(), l.n, l.npad, in, out, planes, vol, pchunk, vec4);
   LAUNCH_CHECK();
 }
 
