@@ -126,13 +126,23 @@ def check(status):
         raise ScnError(lib().scn_last_error().decode())
 
 
+_sizes_made = {}
+
+
 def sizes(dim, x):
-    """A host int64[dim] ctypes array from an int, a sequence or a LongTensor."""
+    """A host int64[dim] ctypes array from an int, a sequence or a LongTensor.  The library only
+    reads these arrays, and a network asks for the same few sizes in every pass: they are kept."""
     if hasattr(x, "tolist"):
         x = x.tolist()
     if isinstance(x, (int,)):
-        x = [x] * dim
-    x = [int(v) for v in x]
-    if len(x) != dim:
-        raise ValueError("expected %d sizes, got %r" % (dim, x))
-    return (C.c_int64 * dim)(*x)
+        x = (x,) * dim
+    key = (dim, tuple(x))
+    made = _sizes_made.get(key)
+    if made is None:
+        vals = [int(v) for v in key[1]]
+        if len(vals) != dim:
+            raise ValueError("expected %d sizes, got %r" % (dim, x))
+        if len(_sizes_made) > 4096:
+            _sizes_made.clear()
+        made = _sizes_made[key] = (C.c_int64 * dim)(*vals)
+    return made

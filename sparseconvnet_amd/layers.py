@@ -70,6 +70,23 @@ def _use_frozen(module, md, weight, bias, pre=None, post=None, second=None):
     f.use(md, tensors)
 
 
+class _NoGrad:
+    """What a Function's forward is handed in place of its context when nothing will be
+    differentiated: attributes can be set on it, saved tensors are dropped."""
+
+    def save_for_backward(self, *tensors):
+        pass
+
+
+def _call(fn, *args):
+    """fn.apply(*args); with gradients disabled (inference under torch.no_grad()) the forward is
+    called directly: Function.apply costs several microseconds per module call there, for an
+    output that would carry no history either way."""
+    if torch.is_grad_enabled():
+        return fn.apply(*args)
+    return fn.forward(_NoGrad(), *args)
+
+
 class _ConvFunction(Function):
     """submanifoldConvolution.py:63-113, convolution.py:72-130, deconvolution.py:49-128: kind 0 /
     1 / 2.  pre / post: eval-mode batch norms applied inside the convolution (inference only)."""
@@ -173,7 +190,7 @@ def join_batchnorm(parts, bn):
     output = SparseConvNetTensor()
     output.metadata = parts[0].metadata
     output.spatial_size = parts[0].spatial_size
-    output.features = _JoinBatchNormFunction.apply(bn.running_mean, bn.running_var, optionalTensor(bn, 'weight').detach(),
+    output.features = _call(_JoinBatchNormFunction, bn.running_mean, bn.running_var, optionalTensor(bn, 'weight').detach(),
                                                    optionalTensor(bn, 'bias').detach(), bn.eps, bn.leakiness, *feats)
     return output
 
@@ -432,7 +449,7 @@ class SubmanifoldConvolution(Module):
         output.spatial_size = input.spatial_size
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post, second)
-        output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 0,
+        output.features = _call(_ConvFunction, input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 0,
                                               (input.spatial_size, self.filter_size), pre, post, out, second)
         return output
 
@@ -474,7 +491,7 @@ class Convolution(Module):
         a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post, second)
-        output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 1,
+        output.features = _call(_ConvFunction, input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 1,
                                               a, pre, post, out, second)
         return output
 
@@ -510,7 +527,7 @@ class Deconvolution(Module):
         a = (input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
         pre, post = _bn_args(pre_bn), _bn_args(post_bn)
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'), pre, post, second)
-        output.features = _ConvFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 2,
+        output.features = _call(_ConvFunction, input.features, self.weight, optionalTensor(self, 'bias'), input.metadata, 2,
                                               a, pre, post, out, second)
         return output
 
@@ -543,7 +560,7 @@ class NetworkInNetwork(Module):
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
         _use_frozen(self, input.metadata, self.weight, optionalTensor(self, 'bias'))
-        output.features = _NetworkInNetworkFunction.apply(input.features, self.weight, optionalTensor(self, 'bias'),
+        output.features = _call(_NetworkInNetworkFunction, input.features, self.weight, optionalTensor(self, 'bias'),
                                                           input.metadata)
         return output
 
@@ -579,7 +596,7 @@ class BatchNormalization(Module):
         output = SparseConvNetTensor()
         output.metadata = input.metadata
         output.spatial_size = input.spatial_size
-        output.features = _BatchNormalizationFunction.apply(
+        output.features = _call(_BatchNormalizationFunction,
             input.features, optionalTensor(self, 'weight'), optionalTensor(self, 'bias'), self.running_mean,
             self.running_var, self.eps, self.momentum, self.training, self.leakiness, input.metadata)
         return output
@@ -634,7 +651,7 @@ class MaxPooling(Module):
             self.pool_stride, rounding_mode='trunc') + 1
         assert ((output.spatial_size - 1) * self.pool_stride + self.pool_size == input.spatial_size).all()
         a = (input.spatial_size, output.spatial_size, self.pool_size, self.pool_stride)
-        output.features = _PoolingFunction.apply(input.features, input.metadata, "max", a, self.nFeaturesToDrop)
+        output.features = _call(_PoolingFunction, input.features, input.metadata, "max", a, self.nFeaturesToDrop)
         return output
 
     def input_spatial_size(self, out_size):
@@ -657,7 +674,7 @@ class AveragePooling(MaxPooling):
             self.pool_stride, rounding_mode='trunc') + 1
         assert ((output.spatial_size - 1) * self.pool_stride + self.pool_size == input.spatial_size).all()
         a = (input.spatial_size, output.spatial_size, self.pool_size, self.pool_stride)
-        output.features = _PoolingFunction.apply(input.features, input.metadata, "average", a, self.nFeaturesToDrop)
+        output.features = _call(_PoolingFunction, input.features, input.metadata, "average", a, self.nFeaturesToDrop)
         return output
 
     def __repr__(self):
@@ -680,7 +697,7 @@ class UnPooling(Module):
         output.metadata = input.metadata
         output.spatial_size = (input.spatial_size - 1) * self.pool_stride + self.pool_size
         a = (input.spatial_size, output.spatial_size, self.pool_size, self.pool_stride)
-        output.features = _PoolingFunction.apply(input.features, input.metadata, "un", a, self.nFeaturesToDrop)
+        output.features = _call(_PoolingFunction, input.features, input.metadata, "un", a, self.nFeaturesToDrop)
         return output
 
     def input_spatial_size(self, out_size):
@@ -717,7 +734,7 @@ class InputLayer(Module):
         if not feats.is_cuda:
             feats = feats.cuda()
         batch_size = 0 if len(input) == 2 else input[2]
-        output.features = _InputLayerFunction.apply(feats.float(), output.metadata, self.spatial_size, input[0], batch_size,
+        output.features = _call(_InputLayerFunction, feats.float(), output.metadata, self.spatial_size, input[0], batch_size,
                                                     self.mode, False)
         return output
 
@@ -730,7 +747,7 @@ class OutputLayer(Module):
         self.dimension = dimension
 
     def forward(self, input):
-        return _OutputLayerFunction.apply(input.features, input.metadata, False)
+        return _call(_OutputLayerFunction, input.features, input.metadata, False)
 
 
 class BLInputLayer(Module):
@@ -755,7 +772,7 @@ class BLInputLayer(Module):
         feats = input[1].to(self.device) if self.device else input[1]
         if not feats.is_cuda:
             feats = feats.cuda()
-        output.features = _InputLayerFunction.apply(feats.float(), output.metadata, self.spatial_size, input[0], 0,
+        output.features = _call(_InputLayerFunction, feats.float(), output.metadata, self.spatial_size, input[0], 0,
                                                     self.mode, True)
         return output
 
@@ -768,7 +785,7 @@ class BLOutputLayer(Module):
         self.dimension = dimension
 
     def forward(self, input):
-        return _OutputLayerFunction.apply(input.features, input.metadata, True)
+        return _call(_OutputLayerFunction, input.features, input.metadata, True)
 
 
 class ActivePooling(Module):
@@ -783,7 +800,7 @@ class ActivePooling(Module):
         self.average = average
 
     def forward(self, input):
-        return _ActivePoolingFunction.apply(input.features, input.metadata, input.spatial_size, self.average)
+        return _call(_ActivePoolingFunction, input.features, input.metadata, input.spatial_size, self.average)
 
     def input_spatial_size(self, out_size):
         return out_size
@@ -801,7 +818,7 @@ class SparseToDense(Module):
         self.nPlanes = nPlanes
 
     def forward(self, input):
-        return _SparseToDenseFunction.apply(input.features, input.metadata, input.spatial_size, self.nPlanes)
+        return _call(_SparseToDenseFunction, input.features, input.metadata, input.spatial_size, self.nPlanes)
 
     def input_spatial_size(self, out_size):
         return out_size

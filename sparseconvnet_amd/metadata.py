@@ -12,7 +12,14 @@ import torch
 from . import _lib
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The caller's current stream as the library takes it.  Asked several times per module call:
+    the raw handle costs a tenth of building a torch.cuda.Stream object around it."""
+    if _raw_stream is not None:
+        return C.c_void_p(_raw_stream(torch.cuda.current_device()))
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 

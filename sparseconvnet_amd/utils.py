@@ -19,9 +19,26 @@ def toLongTensor(dimension, x):
     return torch.full((dimension,), int(x), dtype=torch.int64)
 
 
+_EMPTY = torch.Tensor()
+_REGISTRIES = ('_parameters', '_buffers', '_modules')
+
+
 def optionalTensor(module, name):
-    """module.<name> if it exists, else an empty tensor (how the reference passes 'no bias')."""
-    return getattr(module, name) if hasattr(module, name) else torch.Tensor()
+    """module.<name> if it exists, else an empty tensor (how the reference passes 'no bias').
+    Called for every bias and batch-norm weight of every module call: a Module's registries are
+    looked at directly (hasattr on a Module without the attribute goes through an exception), and
+    the empty tensor is one shared object, which nobody writes to."""
+    d = getattr(module, '__dict__', None)
+    if d is not None:
+        if name in d:
+            return d[name]
+        for reg in _REGISTRIES:
+            r = d.get(reg)
+            if r is not None and name in r:
+                return r[name]
+        if not hasattr(type(module), name):
+            return _EMPTY
+    return getattr(module, name) if hasattr(module, name) else _EMPTY
 
 
 def optionalTensorReturn(a):
